@@ -1,0 +1,109 @@
+"""ctypes binding of ``csrc/libgptq_hip.so`` (the C ABI declared in include/gptq_hip.h).
+
+The library is the only compute path: if it is missing this module raises, it never
+falls back to a CPU or eager implementation.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "csrc", "libgptq_hip.so")
+
+OK = 0
+ERR_BAD_ARG = -1
+ERR_UNSUPPORTED = -2
+ERR_WORKSPACE = -3
+ERR_LAUNCH = -4
+
+KERNEL_GATHER = 1
+KERNEL_GROUPED = 2
+KERNEL_BLOCKED = 3
+
+ABI_SYMBOLS = (
+    "gptq_hip_select",
+    "gptq_hip_workspace_bytes",
+    "gptq_hip_workspace_init",
+    "gptq_hip_gemm",
+    "gptq_hip_gemm_plan",
+    "gptq_hip_dequant",
+    "gptq_hip_strerror",
+    "gptq_hip_abi_version",
+)
+
+
+class Plan(ctypes.Structure):
+    """Mirror of ``gptq_hip_plan``."""
+
+    _fields_ = [
+        ("kernel", ctypes.c_int),
+        ("row_tiles", ctypes.c_int),
+        ("m_blocks", ctypes.c_int),
+        ("waves_n", ctypes.c_int),
+        ("waves_k", ctypes.c_int),
+        ("split_k", ctypes.c_int),
+        ("k_chunk", ctypes.c_int),
+        ("grid_x", ctypes.c_int),
+        ("grid_y", ctypes.c_int),
+        ("grid_z", ctypes.c_int),
+        ("block", ctypes.c_int),
+        ("lds_bytes", ctypes.c_int),
+        ("workspace_bytes", ctypes.c_size_t),
+    ]
+
+    def as_dict(self) -> dict:
+        return {name: getattr(self, name) for name, _ in self._fields_}
+
+
+class GptqHipError(RuntimeError):
+    def __init__(self, status: int, where: str):
+        self.status = status
+        super().__init__(f"{where}: {strerror(status)} (status {status})")
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """Loads the shared library once; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m autogptq.tvm_amd.build` "
+            "(there is no fallback path)"
+        )
+    l = ctypes.CDLL(LIB_PATH)
+    vp, i, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    l.gptq_hip_select.restype = i
+    l.gptq_hip_select.argtypes = [i, i, i, i, i, i, ctypes.POINTER(Plan)]
+    l.gptq_hip_workspace_bytes.restype = sz
+    l.gptq_hip_workspace_bytes.argtypes = [i, i, i, i, i, i]
+    l.gptq_hip_workspace_init.restype = i
+    l.gptq_hip_workspace_init.argtypes = [vp, sz, vp]
+    l.gptq_hip_gemm.restype = i
+    l.gptq_hip_gemm.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, vp]
+    l.gptq_hip_gemm_plan.restype = i
+    l.gptq_hip_gemm_plan.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
+    l.gptq_hip_dequant.restype = i
+    l.gptq_hip_dequant.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
+    l.gptq_hip_strerror.restype = ctypes.c_char_p
+    l.gptq_hip_strerror.argtypes = [i]
+    l.gptq_hip_abi_version.restype = i
+    l.gptq_hip_abi_version.argtypes = []
+    _lib = l
+    return l
+
+
+def strerror(status: int) -> str:
+    return lib().gptq_hip_strerror(int(status)).decode()
+
+
+def select(M: int, K: int, N: int, bits: int, group_size: int, act_order: bool) -> Plan:
+    plan = Plan()
+    rc = lib().gptq_hip_select(M, K, N, bits, group_size, int(bool(act_order)), ctypes.byref(plan))
+    if rc != OK:
+        raise GptqHipError(rc, f"gptq_hip_select(M={M}, K={K}, N={N}, bits={bits}, group_size={group_size})")
+    return plan

@@ -1,0 +1,137 @@
+// extern "C" entry points: argument checks, plan lookup, launch.  Nothing here
+// allocates, synchronises or throws; see include/gptq_hip.h for the contract.
+#include <stdint.h>
+
+#include "gptq_internal.h"
+
+namespace {
+
+bool aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+int check_common(const int32_t *qweight, const int32_t *qzeros, const void *scales, int K, int N, int bits,
+                 int group_size)
+{
+    if (!qweight || !qzeros || !scales) return GPTQ_HIP_ERR_BAD_ARG;
+    if (bits != 3 && bits != 4) return GPTQ_HIP_ERR_BAD_ARG;
+    if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;
+    if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
+    if (!aligned(qweight, 16) || !aligned(qzeros, 4) || !aligned(scales, 8)) return GPTQ_HIP_ERR_BAD_ARG;
+    return GPTQ_HIP_OK;
+}
+
+int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G)
+{
+    const int kstep = gptq::kstep_of(bits);
+    if (pl.kernel != GPTQ_HIP_KERNEL_GATHER) return GPTQ_HIP_ERR_UNSUPPORTED;
+    if (pl.row_tiles != 1 && pl.row_tiles != 2 && pl.row_tiles != 4 && pl.row_tiles != 8)
+        return GPTQ_HIP_ERR_UNSUPPORTED;
+    if (pl.waves_n != 1 && pl.waves_n != 2 && pl.waves_n != 4) return GPTQ_HIP_ERR_UNSUPPORTED;
+    if (pl.block != 64 * pl.waves_n) return GPTQ_HIP_ERR_BAD_ARG;
+    if (pl.k_chunk < kstep || pl.k_chunk % kstep != 0) return GPTQ_HIP_ERR_BAD_ARG;
+    const int steps_total = (K + kstep - 1) / kstep;
+    if (pl.split_k < 1 || pl.split_k > steps_total) return GPTQ_HIP_ERR_BAD_ARG;
+    if (pl.m_blocks * 16 * pl.row_tiles < M) return GPTQ_HIP_ERR_BAD_ARG;
+    if (pl.grid_x * 64 * pl.waves_n < N || pl.grid_y != pl.split_k || pl.grid_z != pl.m_blocks)
+        return GPTQ_HIP_ERR_BAD_ARG;
+    const int xs_rows = M < 16 * pl.row_tiles ? M : 16 * pl.row_tiles;
+    const long long need = (long long)G * 64 * pl.waves_n * 4 + (long long)pl.k_chunk * 4 +
+                           (long long)xs_rows * (pl.k_chunk + 8) * 2;
+    if (pl.lds_bytes < need || pl.lds_bytes > 160 * 1024) return GPTQ_HIP_ERR_BAD_ARG;
+    if (pl.split_k > 1 && (size_t)pl.grid_x * pl.grid_z * sizeof(int) > gptq::kCounterBytes)
+        return GPTQ_HIP_ERR_UNSUPPORTED;
+    return GPTQ_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                                  const int32_t *g_idx, const void *bias, void *y, void *workspace,
+                                  size_t workspace_bytes, int M, int K, int N, int bits, int group_size,
+                                  const gptq_hip_plan *plan, void *stream)
+{
+    if (!x || !y || !plan || M < 1) return GPTQ_HIP_ERR_BAD_ARG;
+    int rc = check_common(qweight, qzeros, scales, K, N, bits, group_size);
+    if (rc != GPTQ_HIP_OK) return rc;
+    if (!aligned(x, 16) || !aligned(y, 8) || (bias && !aligned(bias, 8)) || (g_idx && !aligned(g_idx, 4)))
+        return GPTQ_HIP_ERR_BAD_ARG;
+    const int gs = group_size == -1 ? K : group_size;
+    const int G = (K + gs - 1) / gs;
+    rc = validate_plan(*plan, M, K, N, bits, G);
+    if (rc != GPTQ_HIP_OK) return rc;
+
+    gptq::Params p;
+    p.x = x;
+    p.qweight = (const uint32_t *)qweight;
+    p.qzeros = (const uint32_t *)qzeros;
+    p.scales = scales;
+    p.g_idx = g_idx;
+    p.bias = bias;
+    p.y = y;
+    p.partial = nullptr;
+    p.counters = nullptr;
+    p.M = M;
+    p.K = K;
+    p.N = N;
+    p.G = G;
+    p.group_size = gs;
+    const int kstep = gptq::kstep_of(bits);
+    p.steps_total = (K + kstep - 1) / kstep;
+    p.split_k = plan->split_k;
+    p.chunk_steps = plan->k_chunk / kstep;
+    p.xs_rows = M < 16 * plan->row_tiles ? M : 16 * plan->row_tiles;
+    p.row_tiles = plan->row_tiles;
+    if (plan->split_k > 1) {
+        const size_t need = gptq::kCounterBytes + (size_t)plan->split_k * M * N * sizeof(float);
+        if (!workspace || workspace_bytes < need || !aligned(workspace, 16)) return GPTQ_HIP_ERR_WORKSPACE;
+        p.counters = (int *)workspace;
+        p.partial = (float *)((char *)workspace + gptq::kCounterBytes);
+    }
+    return gptq::launch_matmul(p, bits, *plan, stream);
+}
+
+extern "C" int gptq_hip_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                             const int32_t *g_idx, const void *bias, void *y, void *workspace,
+                             size_t workspace_bytes, int M, int K, int N, int bits, int group_size, void *stream)
+{
+    gptq_hip_plan plan;
+    const int rc = gptq_hip_select(M, K, N, bits, group_size, g_idx != nullptr, &plan);
+    if (rc != GPTQ_HIP_OK) return rc;
+    return gptq_hip_gemm_plan(x, qweight, qzeros, scales, g_idx, bias, y, workspace, workspace_bytes, M, K, N,
+                              bits, group_size, &plan, stream);
+}
+
+extern "C" int gptq_hip_dequant(const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                                const int32_t *g_idx, void *w, int K, int N, int bits, int group_size,
+                                void *stream)
+{
+    if (!w) return GPTQ_HIP_ERR_BAD_ARG;
+    const int rc = check_common(qweight, qzeros, scales, K, N, bits, group_size);
+    if (rc != GPTQ_HIP_OK) return rc;
+    const int gs = group_size == -1 ? K : group_size;
+    const int G = (K + gs - 1) / gs;
+    return gptq::launch_dequant((const uint32_t *)qweight, (const uint32_t *)qzeros, scales, g_idx, w, K, N, G, bits,
+                                gs, stream);
+}
+
+extern "C" int gptq_hip_workspace_init(void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (workspace_bytes == 0) return GPTQ_HIP_OK;
+    if (!workspace || workspace_bytes % 4 != 0 || !aligned(workspace, 4)) return GPTQ_HIP_ERR_BAD_ARG;
+    // only the counters at the head need to start at zero
+    const size_t n = workspace_bytes < gptq::kCounterBytes ? workspace_bytes : gptq::kCounterBytes;
+    return gptq::launch_fill_zero(workspace, n, stream);
+}
+
+extern "C" const char *gptq_hip_strerror(int status)
+{
+    switch (status) {
+        case GPTQ_HIP_OK: return "ok";
+        case GPTQ_HIP_ERR_BAD_ARG: return "bad argument (null or misaligned pointer, size, bits or group_size)";
+        case GPTQ_HIP_ERR_UNSUPPORTED: return "shape or plan not covered by the kernels";
+        case GPTQ_HIP_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+        case GPTQ_HIP_ERR_LAUNCH: return "HIP launch failed";
+        default: return "unknown status";
+    }
+}
+
+extern "C" int gptq_hip_abi_version(void) { return 1; }

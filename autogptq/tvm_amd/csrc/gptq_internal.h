@@ -1,0 +1,40 @@
+// Internal declarations shared by the dispatcher, the launchers and the C ABI.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../../include/gptq_hip.h"
+
+namespace gptq {
+
+// Arguments common to all matmul kernels (device pointers are borrowed for the launch).
+struct Params {
+    const void *x;           // fp16 [M, K]
+    const uint32_t *qweight; // [K/32*bits, N]
+    const uint32_t *qzeros;  // [G, N/32*bits]
+    const void *scales;      // fp16 [G, N]
+    const int32_t *g_idx;    // [K] or nullptr (k / group_size)
+    const void *bias;        // fp16 [N] or nullptr
+    void *y;                 // fp16 [M, N]
+    float *partial;          // [split_k, M, N] when split_k > 1
+    int *counters;           // one per (m block, column tile) when split_k > 1; zero between calls
+    int M, K, N, G, group_size;
+    int steps_total;   // ceil(K / KSTEP): KSTEP = 32 (int4) or 128 (int3)
+    int split_k;       // workgroups per column tile
+    int chunk_steps;   // steps staged in LDS at a time
+    int xs_rows;       // rows of x kept in LDS per workgroup
+    int row_tiles;     // 16-row tiles per wave
+};
+
+// k handled by one wave step: 4 lane groups x (8 | 32) codes
+inline int kstep_of(int bits) { return bits == 4 ? 32 : 128; }
+
+// byte size of the head of the workspace that holds the split-K counters
+static const size_t kCounterBytes = 16384;
+
+int launch_matmul(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
+int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
+                   void *w, int K, int N, int G, int bits, int group_size, void *stream);
+int launch_fill_zero(void *ptr, size_t bytes, void *stream);
+
+}  // namespace gptq

@@ -1,0 +1,132 @@
+// Bit-exact unpack helpers for the AutoGPTQ int4 / int3 packed formats.
+//
+// Everything here is plain integer and fp16 arithmetic written with clang
+// vector types, so the same functions build for gfx950 and for the host
+// (the host build is what the CPU-side tests check against the oracle).
+//
+// Format (reference: auto_gptq/nn_modules/qlinear.py:105-139 pack,
+// :211-236 unpack): along the packed axis, every `bits` consecutive int32
+// words form one little-endian bit stream holding 32 codes; code j sits at
+// bit bits*j.  For 3 bits, codes 10 and 21 straddle word boundaries.
+#pragma once
+#include <stdint.h>
+
+#if defined(__HIP__) || defined(__HIPCC__)
+#define GPTQ_HD __host__ __device__ __forceinline__
+#else
+#define GPTQ_HD inline
+#endif
+
+namespace gptq {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+
+GPTQ_HD h2 as_h2(uint32_t u) { return __builtin_bit_cast(h2, u); }
+GPTQ_HD uint32_t as_u32(h2 v) { return __builtin_bit_cast(uint32_t, v); }
+
+// 32 bits of the 64-bit value hi:lo starting at bit `sh` (0 < sh < 32)
+GPTQ_HD uint32_t funnel(uint32_t hi, uint32_t lo, int sh)
+{
+    return (uint32_t)((((uint64_t)hi << 32) | (uint64_t)lo) >> sh);
+}
+
+// ---- plain integer extraction (the definition everything else must equal) ----
+GPTQ_HD int code4(uint32_t w, int j) { return (int)((w >> (4 * j)) & 0xfu); }
+
+GPTQ_HD int code3(uint32_t w0, uint32_t w1, uint32_t w2, int j)
+{
+    const int bit = 3 * j;
+    const int word = bit >> 5;
+    const int sh = bit & 31;
+    const uint32_t lo = word == 0 ? w0 : (word == 1 ? w1 : w2);
+    const uint32_t hi = word == 0 ? w1 : (word == 1 ? w2 : 0u);
+    const uint64_t v = (((uint64_t)hi << 32) | (uint64_t)lo) >> sh;
+    return (int)(v & 0x7u);
+}
+
+// Zero point (already +1) of column n from a packed qzeros row
+// (reference: qlinear.py:202-209, :217-227).
+GPTQ_HD int zero4(const uint32_t *zrow, int n) { return code4(zrow[n >> 3], n & 7) + 1; }
+
+GPTQ_HD int zero3(const uint32_t *zrow, int n)
+{
+    const uint32_t *b = zrow + 3 * (n >> 5);
+    return code3(b[0], b[1], b[2], n & 31) + 1;
+}
+
+// ---- "magic number" unpack: codes land in fp16 mantissas ----------------------
+// OR-ing a code into the mantissa of 0x6400 (= 1024.0) yields 1024 + code * 2^p
+// where p is the code's bit position inside its 16-bit half.  The halves of one
+// 32-bit register therefore carry two codes that sit 16 (+-) bits apart in the
+// stream; SLOT4 / SLOT3 give, for every (register, half), which code that is.
+//
+// int4: four registers per word.  Register r, half h holds code SLOT4[2r + h].
+//   r = 0: p = 0 ;  r = 1: p = 4 ;  r = 2: p = 0 ;  r = 3: p = 4
+static constexpr int SLOT4[8] = {0, 4, 1, 5, 2, 6, 3, 7};
+
+GPTQ_HD void magic4(uint32_t w, uint32_t out[4])
+{
+    const uint32_t w8 = w >> 8;
+    out[0] = (w & 0x000f000fu) | 0x64006400u;
+    out[1] = (w & 0x00f000f0u) | 0x64006400u;
+    out[2] = (w8 & 0x000f000fu) | 0x64006400u;
+    out[3] = (w8 & 0x00f000f0u) | 0x64006400u;
+}
+
+// magic -> exact code value as fp16 (no rounding happens: all values are small integers)
+GPTQ_HD h2 code_from_magic4(uint32_t m, int r)
+{
+    const h2 v = as_h2(m);
+    if ((r & 1) == 0) {
+        return v - (h2){(_Float16)1024.0f, (_Float16)1024.0f};
+    }
+    return v * (h2){(_Float16)0.0625f, (_Float16)0.0625f} - (h2){(_Float16)64.0f, (_Float16)64.0f};
+}
+
+// int3: sixteen registers per 3-word block.  Register r, half h holds code SLOT3[2r + h].
+// Even registers: low half p = 0, high half p = 2.  Odd registers: low p = 3, high p = 5.
+static constexpr int SLOT3[32] = {0,  6,  1,  7,  2,  8,  3,  9,  4,  10, 5,  11, 12, 18, 13, 19,
+                                  14, 20, 15, 21, 16, 22, 17, 23, 24, 30, 25, 31, 26, 28, 27, 29};
+
+GPTQ_HD void magic3(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t out[16])
+{
+    uint32_t win[8];
+    win[0] = w0;                    // stream bit 0
+    win[1] = w0 >> 6;               // 6
+    win[2] = funnel(w1, w0, 12);    // 12
+    win[3] = funnel(w2, w1, 4);     // 36
+    win[4] = funnel(w2, w1, 10);    // 42
+    win[5] = funnel(w2, w1, 16);    // 48
+    win[6] = w2 >> 8;               // 72
+    const uint32_t t = w2 >> 14;    // 78: codes 26..29 all in the low half
+    win[7] = (t << 12) | t;         // move codes 28, 29 up into the high half
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        out[2 * i] = (win[i] & 0x001c0007u) | 0x64006400u;
+        out[2 * i + 1] = (win[i] & 0x00e00038u) | 0x64006400u;
+    }
+}
+
+GPTQ_HD h2 code_from_magic3(uint32_t m, int r)
+{
+    const h2 v = as_h2(m);
+    if ((r & 1) == 0) {
+        return v * (h2){(_Float16)1.0f, (_Float16)0.25f} - (h2){(_Float16)1024.0f, (_Float16)256.0f};
+    }
+    return v * (h2){(_Float16)0.125f, (_Float16)0.03125f} - (h2){(_Float16)128.0f, (_Float16)32.0f};
+}
+
+// The dequantised weight of the reference (qlinear.py:242): fp16 scale times the
+// integer (q - zero), rounded once.  The product of an 11-bit significand and an
+// integer of magnitude <= 16 is exact in fp32, so one conversion gives that rounding.
+GPTQ_HD _Float16 dequant_one(_Float16 scale, int q, int zero)
+{
+    return (_Float16)((float)scale * (float)(q - zero));
+}
+
+}  // namespace gptq

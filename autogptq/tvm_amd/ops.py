@@ -1,0 +1,125 @@
+"""Torch-tensor front end of the C ABI: pointer plumbing and argument checks only."""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _need_gpu(name: str, t: torch.Tensor, dtype: torch.dtype):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.device.type != "cuda":
+        raise RuntimeError(
+            f"{name} is on {t.device}: the GPTQ kernels run on a ROCm GPU only and there is no CPU fallback"
+        )
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+def _stream(device: torch.device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def check_shapes(qweight, qzeros, scales, g_idx, bias, bits: int, group_size: int):
+    if bits not in (3, 4):
+        raise NotImplementedError("Only 3 and 4 bits are supported.")
+    rows, N = qweight.shape
+    if rows * 32 % bits != 0:
+        raise ValueError(f"qweight has {rows} rows, not a multiple of bits={bits} words per 32 channels")
+    K = rows * 32 // bits
+    gs = K if group_size == -1 else group_size
+    if gs <= 0:
+        raise ValueError(f"group_size must be -1 or positive, got {group_size}")
+    G = (K + gs - 1) // gs
+    if K % 32 != 0 or N % 32 != 0:
+        raise ValueError(f"infeatures ({K}) and outfeatures ({N}) must be multiples of 32")
+    if tuple(scales.shape) != (G, N):
+        raise ValueError(f"scales must be [{G}, {N}], got {tuple(scales.shape)}")
+    if tuple(qzeros.shape) != (G, N // 32 * bits):
+        raise ValueError(f"qzeros must be [{G}, {N // 32 * bits}], got {tuple(qzeros.shape)}")
+    if g_idx is not None and tuple(g_idx.shape) != (K,):
+        raise ValueError(f"g_idx must be [{K}], got {tuple(g_idx.shape)}")
+    if bias is not None and tuple(bias.shape) != (N,):
+        raise ValueError(f"bias must be [{N}], got {tuple(bias.shape)}")
+    return K, N, G
+
+
+_workspaces = {}
+
+
+def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    """A zero-initialised workspace per (device, stream), grown on demand.  The kernels leave
+    its counters at zero, so it is cleared only when it is (re)allocated."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def gemm(x: torch.Tensor, qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
+         g_idx: Optional[torch.Tensor], bias: Optional[torch.Tensor], bits: int, group_size: int,
+         plan: Optional[_lib.Plan] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y[M, N] fp16 = x[M, K] @ W (+ bias); ``g_idx=None`` means contiguous groups (k // group_size)."""
+    _need_gpu("x", x, torch.float16)
+    _need_gpu("qweight", qweight, torch.int32)
+    _need_gpu("qzeros", qzeros, torch.int32)
+    _need_gpu("scales", scales, torch.float16)
+    if g_idx is not None:
+        _need_gpu("g_idx", g_idx, torch.int32)
+    if bias is not None:
+        _need_gpu("bias", bias, torch.float16)
+    K, N, _ = check_shapes(qweight, qzeros, scales, g_idx, bias, bits, group_size)
+    if x.dim() != 2 or x.shape[1] != K:
+        raise ValueError(f"x must be [M, {K}], got {tuple(x.shape)}")
+    M = x.shape[0]
+    dev = x.device
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    else:
+        _need_gpu("out", out, torch.float16)
+        if tuple(out.shape) != (M, N):
+            raise ValueError(f"out must be [{M}, {N}]")
+    if M == 0:
+        return out
+    if plan is None:
+        plan = _lib.select(M, K, N, bits, group_size, g_idx is not None)
+    ws = _workspace(dev, plan.workspace_bytes) if plan.workspace_bytes else None
+    with torch.cuda.device(dev):
+        rc = _lib.lib().gptq_hip_gemm_plan(
+            _ptr(x), _ptr(qweight), _ptr(qzeros), _ptr(scales), _ptr(g_idx), _ptr(bias), _ptr(out),
+            _ptr(ws), ws.numel() if ws is not None else 0, M, K, N, bits, group_size,
+            ctypes.byref(plan), _stream(dev))
+    if rc != _lib.OK:
+        raise _lib.GptqHipError(rc, f"gptq_hip_gemm(M={M}, K={K}, N={N}, bits={bits}, group_size={group_size})")
+    return out
+
+
+def dequant(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
+            g_idx: Optional[torch.Tensor], bits: int, group_size: int) -> torch.Tensor:
+    """The materialised fp16 weight [K, N], bit-exact with the reference's dequantisation."""
+    _need_gpu("qweight", qweight, torch.int32)
+    _need_gpu("qzeros", qzeros, torch.int32)
+    _need_gpu("scales", scales, torch.float16)
+    if g_idx is not None:
+        _need_gpu("g_idx", g_idx, torch.int32)
+    K, N, _ = check_shapes(qweight, qzeros, scales, g_idx, None, bits, group_size)
+    dev = qweight.device
+    w = torch.empty((K, N), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().gptq_hip_dequant(_ptr(qweight), _ptr(qzeros), _ptr(scales), _ptr(g_idx), _ptr(w),
+                                         K, N, bits, group_size, _stream(dev))
+    if rc != _lib.OK:
+        raise _lib.GptqHipError(rc, f"gptq_hip_dequant(K={K}, N={N}, bits={bits})")
+    return w

@@ -1,0 +1,85 @@
+"""Vectorised packers for the AutoGPTQ int3/int4 tensor format, and seeded synthetic layers.
+
+Format (reference: auto_gptq/nn_modules/qlinear.py:105-175): along the packed axis, every
+``bits`` consecutive int32 words are one little-endian bit stream of 32 codes, code ``j`` at
+bit ``bits*j``.  ``qweight`` packs the codes along K, ``qzeros`` packs ``zero - 1`` along N.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+
+
+def pack_along_axis0(codes: np.ndarray, bits: int) -> np.ndarray:
+    """codes [R, C] with values in [0, 2**bits) -> int32 [R//32*bits, C]; R must divide by 32."""
+    codes = np.ascontiguousarray(codes)
+    rows, cols = codes.shape
+    if rows % 32 != 0:
+        raise ValueError(f"packed axis length {rows} is not a multiple of 32")
+    if bits not in (3, 4):
+        raise NotImplementedError("Only 3 and 4 bits are supported.")
+    blocks = codes.reshape(rows // 32, 32, cols).astype(np.uint64)
+    if bits == 4:
+        # 32 codes -> one 128-bit stream = four words of 8 codes
+        b = blocks.reshape(rows // 32, 4, 8, cols)
+        shifts = (4 * np.arange(8, dtype=np.uint64)).reshape(1, 1, 8, 1)
+        words = np.bitwise_or.reduce(b << shifts, axis=2)
+        return words.reshape(rows // 8, cols).astype(np.uint32).view(np.int32)
+    # 3 bits: a 96-bit stream; build it in two 64-bit halves that overlap nowhere
+    out = np.zeros((rows // 32, 3, cols), dtype=np.uint64)
+    for j in range(32):
+        bit = 3 * j
+        w, sh = divmod(bit, 32)
+        v = blocks[:, j, :] << np.uint64(sh)
+        out[:, w, :] |= v & np.uint64(0xFFFFFFFF)
+        if sh + 3 > 32:
+            out[:, w + 1, :] |= v >> np.uint64(32)
+    return out.reshape(rows // 32 * 3, cols).astype(np.uint32).view(np.int32)
+
+
+def pack_qweight(codes: np.ndarray, bits: int) -> np.ndarray:
+    """codes [K, N] -> qweight int32 [K//32*bits, N]."""
+    return pack_along_axis0(codes, bits)
+
+
+def pack_qzeros(zeros: np.ndarray, bits: int) -> np.ndarray:
+    """zero points [G, N] in [1, 2**bits] -> qzeros int32 [G, N//32*bits] (stores zero - 1)."""
+    z = np.asarray(zeros).astype(np.int64) - 1
+    if z.min() < 0 or z.max() >= (1 << bits):
+        raise ValueError("zero points must lie in [1, 2**bits]")
+    return np.ascontiguousarray(pack_along_axis0(np.ascontiguousarray(z.T), bits).T)
+
+
+def num_groups(k: int, group_size: int) -> int:
+    gs = k if group_size == -1 else group_size
+    return math.ceil(k / gs)
+
+
+def make_g_idx(k: int, group_size: int, desc_act: bool, gen: torch.Generator) -> torch.Tensor:
+    gs = k if group_size == -1 else group_size
+    if desc_act:
+        return (torch.randperm(k, generator=gen) // gs).to(torch.int32)
+    return (torch.arange(k) // gs).to(torch.int32)
+
+
+def synth_layer(seed: int, K: int, N: int, bits: int, group_size: int, desc_act: bool, M: int = 1,
+                bias: bool = False) -> dict:
+    """Seeded synthetic QuantLinear tensors (CPU): uniform codes and zero codes, scales in
+    [1e-3, 1e-2], x ~ N(0, 1).  The dict also keeps the unpacked ``codes`` and ``zeros``."""
+    gen = torch.Generator().manual_seed(seed)
+    G = num_groups(K, group_size)
+    codes = torch.randint(0, 1 << bits, (K, N), generator=gen, dtype=torch.int32)
+    zeros = torch.randint(0, 1 << bits, (G, N), generator=gen, dtype=torch.int32) + 1
+    scales = (torch.rand((G, N), generator=gen) * (1e-2 - 1e-3) + 1e-3).to(torch.float16)
+    g_idx = make_g_idx(K, group_size, desc_act, gen)
+    x = torch.randn((M, K), generator=gen).to(torch.float16)
+    b = torch.randn((N,), generator=gen).to(torch.float16) if bias else None
+    return {
+        "bits": bits, "group_size": group_size, "K": K, "N": N, "G": G, "desc_act": desc_act,
+        "codes": codes, "zeros": zeros,
+        "qweight": torch.from_numpy(pack_qweight(codes.numpy(), bits)),
+        "qzeros": torch.from_numpy(pack_qzeros(zeros.numpy(), bits)),
+        "scales": scales, "g_idx": g_idx, "x": x, "bias": b,
+    }

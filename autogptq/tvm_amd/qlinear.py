@@ -1,0 +1,112 @@
+"""``QuantLinear`` with the reference's constructor, buffers and ``forward`` contract
+(auto_gptq/nn_modules/qlinear.py:20-75,177-247; selected by ``make_quant(..., use_tvm=True)`` in
+auto_gptq/modeling/_utils.py:59-89), computing on hand-written HIP kernels.
+
+Differences from the reference's TVM-backed module (auto_gptq/nn_modules/qlinear_tvm.py), on
+purpose: the buffers are the standard AutoGPTQ ones (int32 ``qweight``/``qzeros``, ``g_idx``), the
+constructor compiles nothing and touches no GPU (so it works under ``init_empty_weights``), and
+``forward`` neither pads M nor allocates a padded output.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+import torch.nn as nn
+
+from . import ops
+from .pack import pack_qweight, pack_qzeros
+
+
+class QuantLinear(nn.Module):
+    SUPPORTED_BITS = (3, 4)
+
+    def __init__(self, bits, groupsize, infeatures, outfeatures, bias, kernel_switch_threshold=128):
+        super().__init__()
+        if bits not in self.SUPPORTED_BITS:
+            # the reference accepts 2, 3, 4, 8 (qlinear.py:31-32); this path implements 3 and 4
+            raise NotImplementedError("Only 3,4 bits are supported.")
+        if infeatures % 32 != 0 or outfeatures % 32 != 0:
+            raise ValueError("infeatures and outfeatures must be multiples of 32")
+        self.infeatures = infeatures
+        self.outfeatures = outfeatures
+        self.bits = bits
+        self.groupsize = groupsize if groupsize != -1 else infeatures
+        self.maxq = 2 ** self.bits - 1
+        self.kernel_switch_threshold = kernel_switch_threshold  # kept for signature parity; unused
+
+        groups = math.ceil(infeatures / self.groupsize)
+        self.register_buffer("qweight", torch.zeros((infeatures // 32 * bits, outfeatures), dtype=torch.int32))
+        self.register_buffer("qzeros", torch.zeros((groups, outfeatures // 32 * bits), dtype=torch.int32))
+        self.register_buffer("scales", torch.zeros((groups, outfeatures), dtype=torch.float16))
+        self.register_buffer("g_idx", (torch.arange(infeatures, dtype=torch.int64) // self.groupsize).to(torch.int32))
+        if bias:
+            self.register_buffer("bias", torch.zeros((outfeatures,), dtype=torch.float16))
+        else:
+            self.bias = None
+        self._g_state = None  # (g_idx identity, contiguous?) cached by _kernel_g_idx
+
+    # ------------------------------------------------------------------ packing
+    def pack(self, linear, scales, zeros, g_idx=None):
+        """Quantises ``linear.weight`` with the given per-group ``scales``/``zeros`` ([N, G], as the
+        reference passes them) and fills the packed buffers.  Follows qlinear.py:77-175:
+        ``q = round((W + s*z) / s)`` per input channel, codes packed along K, ``z - 1`` along N."""
+        W = linear.weight.data.clone()
+        if isinstance(linear, nn.Conv2d):
+            W = W.flatten(1)
+        elif type(linear).__name__ == "Conv1D":  # transformers.pytorch_utils.Conv1D keeps [in, out]
+            W = W.t()
+        if g_idx is not None:
+            self.g_idx = g_idx.clone().to(torch.int32)
+        scales = scales.t().contiguous()
+        zeros = zeros.t().contiguous()
+        scale_zeros = zeros * scales
+        self.scales = scales.clone().half()
+        if linear.bias is not None:
+            self.bias = linear.bias.clone().half()
+        g = self.g_idx.long().cpu()
+        # same arithmetic as the reference's per-column loop: (W[:, k] + (s*z)[g]) / half(s)[g]
+        num = W.t().cpu() + scale_zeros[g].cpu()
+        intweight = torch.round(num / self.scales[g].cpu()).to(torch.int32)
+        self.qweight = torch.from_numpy(pack_qweight(intweight.numpy().astype(np.uint32), self.bits))
+        self.qzeros = torch.from_numpy(pack_qzeros(zeros.cpu().numpy().astype(np.int64), self.bits))
+        self._g_state = None
+
+    # ------------------------------------------------------------------ forward
+    def _kernel_g_idx(self):
+        """``None`` when ``g_idx`` is the contiguous ``k // groupsize`` (lets the kernels skip the
+        gather), else the tensor.  Checked once per distinct g_idx storage."""
+        g = self.g_idx
+        key = (g.data_ptr(), g._version, g.device)
+        if self._g_state is None or self._g_state[0] != key:
+            ref = torch.arange(self.infeatures, device=g.device, dtype=torch.int64) // self.groupsize
+            contiguous = bool(torch.equal(g.to(torch.int64), ref))
+            if not contiguous:
+                lo, hi = int(g.min()), int(g.max())
+                if lo < 0 or hi >= self.scales.shape[0]:
+                    raise ValueError(f"g_idx values must lie in [0, {self.scales.shape[0]}), found [{lo}, {hi}]")
+            self._g_state = (key, contiguous)
+        return None if self._g_state[1] else g
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        out_shape = x.shape[:-1] + (self.outfeatures,)
+        x2 = x.reshape(-1, x.shape[-1])
+        if x2.dtype != torch.float16:
+            x2 = x2.half()
+        if not x2.is_contiguous():
+            x2 = x2.contiguous()
+        out = ops.gemm(x2, self.qweight, self.qzeros, self.scales, self._kernel_g_idx(), self.bias,
+                       self.bits, self.groupsize)
+        return out.reshape(out_shape)
+
+    def dequantize(self) -> torch.Tensor:
+        """fp16 [infeatures, outfeatures], the weight the reference materialises on every call."""
+        return ops.dequant(self.qweight, self.qzeros, self.scales, self._kernel_g_idx(), self.bits, self.groupsize)
+
+    def extra_repr(self) -> str:
+        return (f"bits={self.bits}, groupsize={self.groupsize}, infeatures={self.infeatures}, "
+                f"outfeatures={self.outfeatures}, bias={self.bias is not None}")
+
+
+__all__ = ["QuantLinear"]

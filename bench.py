@@ -1,0 +1,286 @@
+#!/usr/bin/env python3
+"""Benchmark of the GPTQ QuantLinear hot path on one MI355X.
+
+Default workload: BASELINE.json configs[1] -- 3-bit GEMV, M=1, K=4096, N=11008, group_size=128,
+desc_act=True (g_idx from a random permutation), synthetic seeded tensors.  One "step" is one
+call of the C-ABI entry point ``gptq_hip_gemm`` on tensors already resident in HBM.  Steps rotate
+over enough distinct weight copies to exceed twice the 256 MB Infinity Cache, so every step
+streams its packed weights from HBM (cache-cold).
+
+Prints ONE JSON line (see the keys below).  ``roofline.achieved`` is algorithmic bytes (packed
+qweight only, K*N*bits/8) or flops (2*M*K*N) per launch divided by the average launch duration
+measured here with HIP events on the launch stream.  ``cpu_baseline`` times the CPU oracle (the
+restatement of the reference's torch path) on this box's host cores.
+
+Other workloads: ``--workload NAME`` (see WORKLOADS), ``--sweep`` adds a table of all of them
+under "sweep" in the same JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
+INFINITY_CACHE_BYTES = 256 << 20
+
+# name -> (bits, K, N, group_size, desc_act, M)
+WORKLOADS = {
+    "c1-int4-4096x4096-m1": (4, 4096, 4096, 128, False, 1),
+    "c2-int3-4096x11008-act-m1": (3, 4096, 11008, 128, True, 1),
+    "int4-4096x11008-act-m1": (4, 4096, 11008, 128, True, 1),
+    "c3-int4-4096x4096-m1": (4, 4096, 4096, 128, False, 1),
+    "c3-int4-4096x11008-m1": (4, 4096, 11008, 128, False, 1),
+    "c3-int4-4096x11008-m2": (4, 4096, 11008, 128, False, 2),
+    "c3-int4-4096x11008-m4": (4, 4096, 11008, 128, False, 4),
+    "c3-int4-4096x11008-m8": (4, 4096, 11008, 128, False, 8),
+    "c3-int4-11008x4096-m1": (4, 11008, 4096, 128, False, 1),
+    "c3-int4-11008x4096-m8": (4, 11008, 4096, 128, False, 8),
+    "c4-int4-4096x11008-act-m16": (4, 4096, 11008, 128, True, 16),
+    "c4-int4-4096x11008-act-m64": (4, 4096, 11008, 128, True, 64),
+    "c4-int4-4096x11008-act-m128": (4, 4096, 11008, 128, True, 128),
+    "c4-int4-4096x11008-act-m256": (4, 4096, 11008, 128, True, 256),
+    "c4-int3-4096x11008-act-m128": (3, 4096, 11008, 128, True, 128),
+    "c4-int4-11008x4096-act-m128": (4, 11008, 4096, 128, True, 128),
+    "c4-int3-11008x4096-act-m128": (3, 11008, 4096, 128, True, 128),
+    "c5-int3-9216x9216-g1-m1": (3, 9216, 9216, -1, True, 1),
+    "c5-int3-9216x36864-g1-m1": (3, 9216, 36864, -1, True, 1),
+    "c5-int3-36864x9216-g1-m1": (3, 36864, 9216, -1, True, 1),
+    "c5-int3-9216x36864-g1-m32": (3, 9216, 36864, -1, True, 32),
+}
+DEFAULT_WORKLOAD = "c2-int3-4096x11008-act-m1"
+
+
+def build_case(name: str, dev):
+    from autogptq.tvm_amd import _lib
+    from autogptq.tvm_amd.pack import synth_layer
+
+    bits, K, N, gs, desc_act, M = WORKLOADS[name]
+    L = synth_layer(2000 + sorted(WORKLOADS).index(name), K, N, bits, gs, desc_act, M=M)
+    wbytes = K * N * bits // 8
+    copies = max(2, -(-2 * INFINITY_CACHE_BYTES // wbytes))
+    gen = torch.Generator().manual_seed(99)
+    qweights = [L["qweight"].to(dev)]
+    for _ in range(copies - 1):
+        # distinct random packed words: every int32 pattern is a valid block of codes
+        qweights.append(torch.randint(-(1 << 31), (1 << 31) - 1, L["qweight"].shape, generator=gen,
+                                      dtype=torch.int64).to(torch.int32).to(dev))
+    case = {
+        "name": name, "bits": bits, "K": K, "N": N, "gs": gs, "desc_act": desc_act, "M": M, "L": L,
+        "qweights": qweights,
+        "qzeros": L["qzeros"].to(dev), "scales": L["scales"].to(dev),
+        "g_idx": L["g_idx"].to(dev) if desc_act else None,
+        "x": L["x"].to(dev), "y": torch.empty((M, N), dtype=torch.float16, device=dev),
+        "wbytes": wbytes, "flops": 2 * M * K * N,
+    }
+    plan = _lib.select(M, K, N, bits, gs, desc_act)
+    case["plan"] = plan
+    case["ws"] = torch.zeros(max(plan.workspace_bytes, 16), dtype=torch.uint8, device=dev)
+    return case
+
+
+def make_step(case, dev):
+    """Returns step(i): one gptq_hip_gemm_plan call on weight copy i (pre-marshalled arguments)."""
+    from autogptq.tvm_amd import _lib
+
+    lib = _lib.lib()
+    fn = lib.gptq_hip_gemm_plan
+    vp = ctypes.c_void_p
+    common = dict(
+        x=vp(case["x"].data_ptr()), qz=vp(case["qzeros"].data_ptr()), sc=vp(case["scales"].data_ptr()),
+        g=vp(case["g_idx"].data_ptr()) if case["g_idx"] is not None else None,
+        y=vp(case["y"].data_ptr()), ws=vp(case["ws"].data_ptr()) if case["plan"].workspace_bytes else None,
+    )
+    qws = [vp(q.data_ptr()) for q in case["qweights"]]
+    wsb = case["plan"].workspace_bytes
+    M, K, N, bits, gs = case["M"], case["K"], case["N"], case["bits"], case["gs"]
+    planp = ctypes.byref(case["plan"])
+    n = len(qws)
+
+    def step(i, stream):
+        rc = fn(common["x"], qws[i % n], common["qz"], common["sc"], common["g"], None, common["y"],
+                common["ws"], wsb, M, K, N, bits, gs, planp, stream)
+        if rc != 0:
+            raise RuntimeError(f"gptq_hip_gemm failed: {_lib.strerror(rc)}")
+
+    return step
+
+
+def time_case(case, dev, steps: int, warmup: int):
+    """Average duration of one step in microseconds: K steps captured once in a HIP graph and
+    replayed inside one event-bracketed region (no host launch cost between the kernels), plus
+    the same K steps launched eagerly for comparison."""
+    step = make_step(case, dev)
+    stream = torch.cuda.Stream(device=dev)
+    res = {}
+    with torch.cuda.stream(stream):
+        sp = ctypes.c_void_p(stream.cuda_stream)
+        for i in range(warmup):
+            step(i, sp)
+        stream.synchronize()
+        # eager
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize(dev)
+        e0.record(stream)
+        for i in range(steps):
+            step(i, sp)
+        e1.record(stream)
+        torch.cuda.synchronize(dev)
+        res["eager_us"] = e0.elapsed_time(e1) * 1e3 / steps
+    # graph replay
+    try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            spg = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+            for i in range(steps):
+                step(i, spg)
+        g.replay()
+        torch.cuda.synchronize(dev)
+        times = []
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize(dev)
+            e0.record()
+            g.replay()
+            e1.record()
+            torch.cuda.synchronize(dev)
+            times.append(e0.elapsed_time(e1) * 1e3 / steps)
+        res["graph_us"] = min(times)
+    except Exception as exc:  # graph capture unavailable: report the eager figure only
+        res["graph_error"] = repr(exc)[:200]
+    res["us"] = min(v for k, v in res.items() if k in ("eager_us", "graph_us"))
+    return res
+
+
+def check_case(case, dev):
+    """The timed path's output against the oracle, for the first weight copy."""
+    from oracle import c_oracle
+
+    step = make_step(case, dev)
+    step(0, ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+    torch.cuda.synchronize(dev)
+    L = case["L"]
+    w16 = torch.from_numpy(c_oracle.dequant(L["qweight"].numpy(), L["qzeros"].numpy(), L["scales"].numpy(),
+                                            L["g_idx"].numpy(), case["bits"]).copy())
+    want = L["x"].float() @ w16.float()
+    got = case["y"].float().cpu()
+    err = (got - want).abs()
+    ok = bool((err <= 1e-2 + 1e-2 * want.abs()).all())
+    return ok, float(err.max())
+
+
+def summarize(case, t):
+    us = t["us"]
+    out = {"workload": case["name"], "us": round(us, 3)}
+    out.update({k: (round(v, 3) if isinstance(v, float) else v) for k, v in t.items() if k != "us"})
+    out["weight_GBps"] = round(case["wbytes"] / us * 1e-3, 1)
+    out["hbm_frac"] = round(case["wbytes"] / us * 1e-3 / HBM_PEAK_GBS, 4)
+    out["TFLOPs"] = round(case["flops"] / us * 1e-6, 2)
+    out["mfma_frac"] = round(case["flops"] / us * 1e-6 / MFMA_FP16_PEAK_TFLOPS, 4)
+    out["plan"] = {k: v for k, v in case["plan"].as_dict().items()
+                   if k in ("kernel", "row_tiles", "waves_n", "waves_k", "split_k", "grid_x", "grid_y", "grid_z")}
+    return out
+
+
+def cpu_baseline(case, budget_s: float = 20.0):
+    """The reference's CPU path (oracle restatement of qlinear.py:198-245: unpack + gather + dequant
+    + fp16 matmul on every call) on this box's host cores."""
+    from oracle import gptq_oracle as orc
+
+    L = case["L"]
+    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1))
+    torch.set_num_threads(threads)
+    args = (L["x"], L["qweight"], L["qzeros"], L["scales"], L["g_idx"], None, case["bits"])
+    t0 = time.perf_counter()
+    orc.forward_ref(*args)
+    first = time.perf_counter() - t0
+    n = max(3, min(10, int(budget_s / max(first, 1e-3)) - 1))
+    ts = []
+    for _ in range(n):
+        t0 = time.perf_counter()
+        orc.forward_ref(*args)
+        ts.append(time.perf_counter() - t0)
+    med = statistics.median(ts)
+    return {
+        "value": round(med * 1e6, 1), "unit": "us", "cores": threads, "kind": "port",
+        "sample": f"median of {n} full calls after 1 warm-up of the torch CPU path on the same "
+                  f"{case['name']} tensors (unpack+gather+dequant+fp16 matmul per call)",
+        "weight_GBps": round(case["wbytes"] / med * 1e-9, 3),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
+    ap.add_argument("--sweep", action="store_true", help="also time every workload in WORKLOADS")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures the QuantLinear kernels on ONE GPU; --gpus must be 1 "
+              "(the path shards by output columns with no exchange, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the kernels have no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    case = build_case(args.workload, dev)
+    ok, max_err = check_case(case, dev)
+    torch.cuda.synchronize(dev)
+    t = time_case(case, dev, args.steps, args.warmup)
+    torch.cuda.synchronize(dev)
+    s = summarize(case, t)
+    bits, K, N, gs, desc_act, M = WORKLOADS[args.workload]
+    gemv = M <= 8
+    line = {
+        "metric": f"GEMV latency, int{bits} {K}x{N} M={M}, cache-cold" if gemv
+                  else f"GEMM latency, int{bits} {K}x{N} M={M}",
+        "value": s["us"], "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(s["us"] * 1e-3, 6), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": args.workload, "bits": bits, "K": K, "N": N, "M": M, "group_size": gs,
+                   "desc_act": desc_act, "weight_copies": len(case["qweights"]), "plan": s["plan"]},
+        "parity": {"ok": ok, "max_abs_err": round(max_err, 6), "rtol": 1e-2, "atol": 1e-2},
+        "timing": {k: s[k] for k in ("eager_us", "graph_us", "graph_error") if k in s},
+        "hbm_frac": s["hbm_frac"], "tflops": s["TFLOPs"],
+    }
+    if gemv:
+        line["roofline"] = {"bound": "hbm", "achieved": s["weight_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": s["hbm_frac"], "traffic": None}
+    else:
+        line["roofline"] = {"bound": "mfma", "achieved": s["TFLOPs"], "peak": MFMA_FP16_PEAK_TFLOPS,
+                            "unit": "TFLOP/s", "frac": s["mfma_frac"], "traffic": None}
+    if args.sweep:
+        sweep = []
+        for name in sorted(WORKLOADS):
+            c = build_case(name, dev)
+            okc, errc = check_case(c, dev)
+            r = summarize(c, time_case(c, dev, min(args.steps, 100), min(args.warmup, 10)))
+            r["parity_ok"] = okc
+            r["max_abs_err"] = round(errc, 6)
+            sweep.append(r)
+            del c
+            torch.cuda.empty_cache()
+        line["sweep"] = sweep
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(case)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,110 @@
+/*
+ * C ABI of the MI355X (gfx950) GPTQ int3/int4 QuantLinear kernels.
+ *
+ * Every pointer except `plan` outputs is a DEVICE pointer owned by the caller.
+ * Nothing here allocates, frees or synchronises; launches go to `stream`
+ * (a hipStream_t passed as void*, NULL = the default stream).  Functions
+ * return GPTQ_HIP_OK or a negative gptq_hip_status and never throw.
+ *
+ * Tensor formats are those of the reference's standard QuantLinear
+ * (auto_gptq/nn_modules/qlinear.py:40-59):
+ *   qweight int32 [K/32*bits, N]   codes packed along K, little-endian bit stream
+ *   qzeros  int32 [G, N/32*bits]   (zero point - 1) packed along N the same way
+ *   scales  fp16  [G, N]
+ *   g_idx   int32 [K]              group of input channel k; NULL means k / group_size
+ *   bias    fp16  [N] or NULL
+ *   x       fp16  [M, K] row-major, y fp16 [M, N] row-major
+ * with G = ceil(K / group_size) and group_size = -1 meaning K.
+ */
+#ifndef GPTQ_HIP_H
+#define GPTQ_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum gptq_hip_status {
+    GPTQ_HIP_OK = 0,
+    GPTQ_HIP_ERR_BAD_ARG = -1,     /* null pointer, non-positive size, bits not in {3,4}, misaligned */
+    GPTQ_HIP_ERR_UNSUPPORTED = -2, /* shape outside what the kernels cover (see gptq_hip_select) */
+    GPTQ_HIP_ERR_WORKSPACE = -3,   /* workspace missing or smaller than the plan needs */
+    GPTQ_HIP_ERR_LAUNCH = -4       /* the HIP runtime refused the launch */
+} gptq_hip_status;
+
+/* kernel families the dispatcher chooses between */
+enum {
+    GPTQ_HIP_KERNEL_GATHER = 1, /* per-weight scale/zero gather, exact fp16 weights; any g_idx, any M */
+    GPTQ_HIP_KERNEL_GROUPED = 2, /* rows expanded by group, scales applied once per group; small G*M */
+    GPTQ_HIP_KERNEL_BLOCKED = 3 /* contiguous groups (g_idx == NULL), scales applied at group ends */
+};
+
+/* What the dispatcher decided for one problem; filled by gptq_hip_select. */
+typedef struct gptq_hip_plan {
+    int kernel;             /* GPTQ_HIP_KERNEL_* */
+    int row_tiles;          /* 16-row MFMA tiles held per wave */
+    int m_blocks;           /* grid extent along M */
+    int waves_n;            /* waves of a workgroup laid along N (64 columns each) */
+    int waves_k;            /* waves of a workgroup laid along K */
+    int split_k;            /* workgroups sharing one column tile; >1 uses the workspace */
+    int k_chunk;            /* input channels staged in LDS at a time */
+    int grid_x, grid_y, grid_z;
+    int block;              /* threads per workgroup */
+    int lds_bytes;          /* dynamic LDS per workgroup */
+    size_t workspace_bytes; /* 0 when split_k == 1 */
+} gptq_hip_plan;
+
+/*
+ * Shape dispatcher: a pure host function (no GPU needed).  Takes the place of
+ * the reference's handler database and M-bucket dispatch
+ * (auto_gptq/nn_modules/tvm_untils/cache.py:11-62,
+ *  auto_gptq/nn_modules/tvm_untils/pycuda_warpper.py:77-127,138-189).
+ * act_order != 0 means a g_idx array will be passed.
+ */
+int gptq_hip_select(int M, int K, int N, int bits, int group_size, int act_order, gptq_hip_plan *plan);
+
+/* Bytes of workspace gptq_hip_gemm needs for this problem (0 if none). */
+size_t gptq_hip_workspace_bytes(int M, int K, int N, int bits, int group_size, int act_order);
+
+/*
+ * Zero-fills a workspace with a fill kernel.  A workspace must be zero before
+ * its first use; gptq_hip_gemm leaves it ready for the next call on the same
+ * stream.  Calls that share a workspace must not overlap.
+ */
+int gptq_hip_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * y = x @ dequant(qweight, qzeros, scales, g_idx) (+ bias), fp32 accumulate.
+ * Replaces the reference's handler call
+ *   handler(x, qweight, y, scales, zeros)   (pycuda_warpper.py:138, qlinear_tvm.py:123,150)
+ * and computes what qlinear.py:198-245 computes.  Unlike the reference, y is
+ * written for exactly M rows (no padded rows) and need not be pre-zeroed.
+ */
+int gptq_hip_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                  const int32_t *g_idx, const void *bias, void *y, void *workspace, size_t workspace_bytes,
+                  int M, int K, int N, int bits, int group_size, void *stream);
+
+/* Same, with the plan forced by the caller (benchmarks and tests of single kernels). */
+int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                       const int32_t *g_idx, const void *bias, void *y, void *workspace, size_t workspace_bytes,
+                       int M, int K, int N, int bits, int group_size, const gptq_hip_plan *plan, void *stream);
+
+/*
+ * W fp16 [K, N] = scales[g] * (q - (zq[g] + 1)), one rounding per element:
+ * the materialised weight of qlinear.py:198-242, for the bit-exact check.
+ */
+int gptq_hip_dequant(const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *g_idx,
+                     void *w, int K, int N, int bits, int group_size, void *stream);
+
+/* Human-readable text for a gptq_hip_status. */
+const char *gptq_hip_strerror(int status);
+
+/* ABI version of this library (bumped when a signature changes). */
+int gptq_hip_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GPTQ_HIP_H */

@@ -1,0 +1,128 @@
+"""The C-ABI library loads without a GPU, exports what include/gptq_hip.h declares, and its
+host-side logic (dispatcher, argument checks) behaves.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from autogptq.tvm_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "gptq_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gptq_hip_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.lib()
+    names = declared_functions()
+    assert set(names) == set(_lib.ABI_SYMBOLS)
+    for name in names:
+        assert getattr(lib, name) is not None
+    assert lib.gptq_hip_abi_version() == 1
+
+
+def test_plan_struct_matches_header():
+    text = open(os.path.join(ROOT, "include", "gptq_hip.h")).read()
+    body = re.search(r"typedef struct gptq_hip_plan \{(.*?)\} gptq_hip_plan;", text, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        typ, names = decl.rsplit(" ", 1)[0], decl.split(" ", 1)[1]
+        typ = "size_t" if decl.startswith("size_t") else "int"
+        for nm in names.replace("int", "").replace("size_t", "").split(","):
+            fields.append((nm.strip(), typ))
+    assert [f for f, _ in fields] == [f for f, _ in _lib.Plan._fields_]
+    for (_, typ), (_, ct) in zip(fields, _lib.Plan._fields_):
+        assert ct is (ctypes.c_size_t if typ == "size_t" else ctypes.c_int)
+
+
+def test_strerror_texts():
+    assert _lib.strerror(0) == "ok"
+    for code in (-1, -2, -3, -4):
+        assert _lib.strerror(code) not in ("ok", "unknown status")
+    assert _lib.strerror(-99) == "unknown status"
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 64, 128, 256, 1000])
+@pytest.mark.parametrize("KN", [(4096, 4096), (4096, 11008), (11008, 4096), (9216, 36864), (36864, 9216), (64, 32)])
+@pytest.mark.parametrize("gs", [128, -1])
+def test_select_plans_are_consistent(bits, M, KN, gs):
+    K, N = KN
+    if gs != -1 and K % gs != 0:
+        gs = 32
+    for act in (False, True):
+        p = _lib.select(M, K, N, bits, gs, act)
+        assert p.kernel in (_lib.KERNEL_GATHER, _lib.KERNEL_GROUPED, _lib.KERNEL_BLOCKED)
+        assert p.row_tiles in (1, 2, 4, 8)
+        assert p.m_blocks * 16 * p.row_tiles >= M
+        assert p.block == 64 * p.waves_n * p.waves_k and p.block <= 1024
+        assert p.grid_x * 64 * p.waves_n >= N
+        kstep = 32 if bits == 4 else 128
+        steps = (K + kstep - 1) // kstep
+        assert 1 <= p.split_k <= steps
+        assert p.lds_bytes <= 160 * 1024
+        assert p.grid_x >= 1 and p.grid_y >= 1 and p.grid_z >= 1
+        if p.split_k > 1:
+            assert p.workspace_bytes >= p.split_k * M * N * 4
+            # partial sums stay small next to the packed weights
+            assert p.split_k * M * N * 4 <= K * N * bits // 8
+        else:
+            assert p.workspace_bytes == 0
+        lib = _lib.lib()
+        assert lib.gptq_hip_workspace_bytes(M, K, N, bits, gs, int(act)) == p.workspace_bytes
+
+
+def test_select_fills_the_chip_at_m1():
+    # the headline shapes must give every CU work: at least 256 workgroups
+    for bits in (3, 4):
+        for (K, N) in [(4096, 4096), (4096, 11008), (11008, 4096)]:
+            p = _lib.select(1, K, N, bits, 128, True)
+            assert p.grid_x * p.grid_y * p.grid_z >= 256, (bits, K, N, p.as_dict())
+
+
+@pytest.mark.parametrize("args", [
+    (1, 4096, 4096, 2, 128),   # bits
+    (1, 4096, 4096, 8, 128),
+    (0, 4096, 4096, 4, 128),   # M
+    (1, 4100, 4096, 4, 128),   # K % 32
+    (1, 4096, 4100, 4, 128),   # N % 32
+    (1, 4096, 4096, 4, 0),     # group_size
+    (1, 4096, 4096, 4, -5),
+])
+def test_select_rejects_bad_arguments(args):
+    M, K, N, bits, gs = args
+    with pytest.raises(_lib.GptqHipError) as e:
+        _lib.select(M, K, N, bits, gs, False)
+    assert e.value.status == _lib.ERR_BAD_ARG
+
+
+def test_entry_points_reject_null_and_bad_sizes_before_touching_the_gpu():
+    lib = _lib.lib()
+    null = ctypes.c_void_p(None)
+    fake = ctypes.c_void_p(0x1000)  # aligned, never dereferenced: the checks fail first
+    # null pointers
+    assert lib.gptq_hip_gemm(null, fake, fake, fake, null, null, fake, null, 0, 1, 64, 64, 4, 32, null) == _lib.ERR_BAD_ARG
+    assert lib.gptq_hip_gemm(fake, null, fake, fake, null, null, fake, null, 0, 1, 64, 64, 4, 32, null) == _lib.ERR_BAD_ARG
+    # bits outside {3, 4}
+    assert lib.gptq_hip_gemm(fake, fake, fake, fake, null, null, fake, null, 0, 1, 64, 64, 8, 32, null) == _lib.ERR_BAD_ARG
+    # K not a multiple of 32
+    assert lib.gptq_hip_gemm(fake, fake, fake, fake, null, null, fake, null, 0, 1, 72, 64, 4, 8, null) == _lib.ERR_BAD_ARG
+    # misaligned qweight
+    assert lib.gptq_hip_gemm(fake, ctypes.c_void_p(0x1004), fake, fake, null, null, fake, null, 0, 1, 64, 64, 4, 32,
+                             null) == _lib.ERR_BAD_ARG
+    # a split-K plan without a workspace
+    assert lib.gptq_hip_gemm(fake, fake, fake, fake, null, null, fake, null, 0, 1, 4096, 4096, 4, 128,
+                             null) == _lib.ERR_WORKSPACE
+    assert lib.gptq_hip_dequant(fake, fake, fake, null, null, 64, 64, 4, 32, null) == _lib.ERR_BAD_ARG
+    assert lib.gptq_hip_dequant(fake, fake, fake, null, fake, 64, 64, 5, 32, null) == _lib.ERR_BAD_ARG
+    assert lib.gptq_hip_workspace_init(null, 64, null) == _lib.ERR_BAD_ARG
+    assert lib.gptq_hip_workspace_init(null, 0, null) == _lib.OK

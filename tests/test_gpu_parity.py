@@ -1,0 +1,220 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI (ctypes -> libgptq_hip.so),
+against the CPU oracle on the same seeded inputs.
+
+Bars: dequantised weights bit-exact; outputs within rtol = atol = 1e-2 of x @ W (W the oracle's
+fp16 weight, fp32-or-wider accumulation).  Tighter internal bounds are also asserted so that an
+indexing slip cannot hide inside the contract's tolerance.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from autogptq.tvm_amd import QuantLinear, _lib, ops
+from tests.parity_util import ATOL, RTOL, assert_close, expected_output, expected_weight, layer, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+def run_gemm(D, g_idx="auto", plan=None, x=None):
+    g = D["g_idx"] if (g_idx == "auto" and D["desc_act"]) else (None if g_idx == "auto" else g_idx)
+    return ops.gemm(D["x"] if x is None else x, D["qweight"], D["qzeros"], D["scales"], g, D.get("bias"),
+                    D["bits"], D["group_size"], plan=plan)
+
+
+# ------------------------------------------------------------------ dequant: bit-exact
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("desc_act", [False, True])
+@pytest.mark.parametrize("shape", [(64, 32, 32), (256, 96, 64), (4096, 256, 128), (1024, 160, -1)])
+def test_dequant_bit_exact_small(dev, bits, desc_act, shape):
+    K, N, gs = shape
+    L = layer(100 + bits, K, N, bits, gs, desc_act)
+    D = to_dev(L, dev)
+    for g in (D["g_idx"], None if not desc_act else D["g_idx"]):
+        w = ops.dequant(D["qweight"], D["qzeros"], D["scales"], g, bits, gs).cpu()
+        want = expected_weight(L)
+        assert torch.equal(w.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("bits,K,N,gs,desc_act", [
+    (4, 4096, 4096, 128, False),      # config 1
+    (3, 4096, 11008, 128, True),      # config 2
+    (4, 11008, 4096, 128, True),      # config 3/4 down projection
+    (3, 9216, 9216, -1, True),        # config 5 attention
+])
+def test_dequant_bit_exact_full_size(dev, bits, K, N, gs, desc_act):
+    L = layer(200 + bits, K, N, bits, gs, desc_act)
+    D = to_dev(L, dev)
+    w = ops.dequant(D["qweight"], D["qzeros"], D["scales"], D["g_idx"], bits, gs).cpu()
+    want = expected_weight(L)
+    assert torch.equal(w.view(torch.int16), want.view(torch.int16))
+
+
+def test_dequant_extreme_scales_bit_exact(dev):
+    # subnormal, tiny, large and negative fp16 scales: the single rounding must still match
+    L = layer(7, 128, 64, 4, 32, True)
+    pats = torch.tensor([0x0001, 0x03FF, 0x0400, 0x1234, 0x7BFF, 0x8001, 0xB555, 0xFBFF, 0x0000, 0x3C00],
+                        dtype=torch.int32).to(torch.int16)
+    flat = L["scales"].view(torch.int16).flatten()
+    flat[: 10 * (flat.numel() // 10)] = pats.repeat(flat.numel() // 10)
+    D = to_dev(L, dev)
+    w = ops.dequant(D["qweight"], D["qzeros"], D["scales"], D["g_idx"], 4, 32).cpu()
+    assert torch.equal(w.view(torch.int16), expected_weight(L).view(torch.int16))
+
+
+# ------------------------------------------------------------------ matmul: small shapes, all the edges
+M_EDGES = [1, 2, 3, 5, 8, 15, 16, 17, 31, 33, 64, 65, 127, 129, 257]
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("desc_act", [False, True])
+@pytest.mark.parametrize("M", M_EDGES)
+def test_gemm_ragged_m(dev, bits, desc_act, M):
+    L = layer(300 + M, 512, 192, bits, 128, desc_act, M=M, bias=(M % 2 == 1))
+    D = to_dev(L, dev)
+    y = run_gemm(D)
+    assert y.shape == (M, 192) and y.dtype == torch.float16
+    err = assert_close(y, expected_output(L), f"bits={bits} act={desc_act} M={M}")
+    assert err < 4e-3, err  # fp32 accumulation + one fp16 rounding of |y| < 8
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("K,N,gs", [(32, 32, 32), (96, 32, 32), (160, 96, -1), (384, 64, 64), (1024, 416, 32),
+                                    (2048, 1056, 256)])
+@pytest.mark.parametrize("M", [1, 7, 40])
+def test_gemm_odd_shapes(dev, bits, K, N, gs, M):
+    for desc_act in (False, True):
+        L = layer(400 + K + N, K, N, bits, gs, desc_act, M=M)
+        D = to_dev(L, dev)
+        err = assert_close(run_gemm(D), expected_output(L), f"bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
+        assert err < 4e-3, err
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_gemm_explicit_contiguous_g_idx_equals_null(dev, bits):
+    L = layer(55, 512, 128, bits, 64, False, M=4)
+    D = to_dev(L, dev)
+    a = run_gemm(D, g_idx=None)
+    b = run_gemm(D, g_idx=D["g_idx"])
+    assert_close(a, expected_output(L), "null g_idx")
+    assert_close(b, expected_output(L), "explicit g_idx")
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_gemm_integer_exact(dev, bits):
+    # x = 1, scales = 1, one group: y[n] = sum_k (q - z), exactly representable -> must be exact
+    L = layer(66, 256, 64, bits, -1, False, M=2)
+    L["scales"] = torch.ones_like(L["scales"])
+    L["x"] = torch.ones_like(L["x"])
+    D = to_dev(L, dev)
+    y = run_gemm(D).float().cpu()
+    want = (L["codes"].numpy() - L["zeros"].numpy()[0][None, :]).sum(axis=0).astype(np.float32)
+    assert np.array_equal(y[0].numpy(), want) and np.array_equal(y[1].numpy(), want)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("split", [1, 2, 3, 7])
+@pytest.mark.parametrize("M", [1, 20])
+def test_gemm_forced_split_k(dev, bits, split, M):
+    K, N = 2048, 320
+    L = layer(500 + split, K, N, bits, 128, True, M=M, bias=True)
+    D = to_dev(L, dev)
+    plan = _lib.select(M, K, N, bits, 128, True)
+    plan.split_k = split
+    plan.grid_y = split
+    plan.workspace_bytes = 16384 + split * M * N * 4 if split > 1 else 0
+    y1 = run_gemm(D, plan=plan)
+    y2 = run_gemm(D, plan=plan)  # same workspace again: counters must have been left at zero
+    assert_close(y1, expected_output(L), f"split={split}")
+    assert torch.equal(y1, y2), "split-K result changed between two identical calls"
+
+
+def test_gemm_does_not_write_outside_y(dev):
+    M, K, N = 5, 512, 96
+    L = layer(77, K, N, 4, 128, True, M=M)
+    D = to_dev(L, dev)
+    guard = 4096
+    buf = torch.full((guard + M * N + guard,), 1234.0, dtype=torch.float16, device=dev)
+    out = buf[guard: guard + M * N].view(M, N)
+    ops.gemm(D["x"], D["qweight"], D["qzeros"], D["scales"], D["g_idx"], None, 4, 128, out=out)
+    assert_close(out, expected_output(L), "guarded out")
+    assert bool((buf[:guard] == 1234.0).all()) and bool((buf[guard + M * N:] == 1234.0).all())
+
+
+# ------------------------------------------------------------------ the benchmark configurations
+FULL = [
+    # (name, bits, K, N, gs, desc_act, Ms)
+    ("c1-int4-4096x4096", 4, 4096, 4096, 128, False, [1]),
+    ("c2-int3-4096x11008-act", 3, 4096, 11008, 128, True, [1]),
+    ("c3-int4-4096x11008", 4, 4096, 11008, 128, False, [1, 2, 4, 8]),
+    ("c3-int4-11008x4096", 4, 11008, 4096, 128, False, [1, 8]),
+    ("c4-int4-4096x11008-act", 4, 4096, 11008, 128, True, [16, 128]),
+    ("c4-int3-11008x4096-act", 3, 11008, 4096, 128, True, [64, 256]),
+    ("c5-int3-9216x9216-act-g1", 3, 9216, 9216, -1, True, [1, 32]),
+]
+
+
+@pytest.mark.parametrize("name,bits,K,N,gs,desc_act,Ms", FULL, ids=[f[0] for f in FULL])
+def test_gemm_full_size(dev, name, bits, K, N, gs, desc_act, Ms):
+    L = layer(7000 + [f[0] for f in FULL].index(name), K, N, bits, gs, desc_act, M=max(Ms))
+    D = to_dev(L, dev)
+    w16 = expected_weight(L)
+    for M in Ms:
+        x = L["x"][:M].contiguous()
+        y = run_gemm(D, x=x.to(dev))
+        err = assert_close(y, expected_output(L, x=x, w16=w16), f"{name} M={M}")
+        assert err < 8e-3, (name, M, err)
+        y2 = run_gemm(D, x=x.to(dev))
+        assert torch.equal(y, y2), f"{name} M={M}: two identical calls differ"
+
+
+def test_gemm_linearity_at_full_size(dev):
+    # size-independent property: f(a + b) = f(a) + f(b) up to rounding, f(2x) = 2 f(x) exactly
+    L = layer(900, 4096, 11008, 3, 128, True, M=2)
+    D = to_dev(L, dev)
+    x = D["x"]
+    y = run_gemm(D)
+    y2 = run_gemm(D, x=(x * 2).contiguous())
+    assert torch.equal(y2.float(), y.float() * 2)  # scaling by 2 is exact in fp16 and fp32
+    ysum = run_gemm(D, x=(x[0:1] + x[1:2]).contiguous())
+    assert_close(ysum, (y[0:1].float() + y[1:2].float()), "additivity", rtol=2e-2, atol=2e-2)
+
+
+# ------------------------------------------------------------------ the module
+@pytest.mark.parametrize("bits", [3, 4])
+def test_quantlinear_forward(dev, bits):
+    K, N, gs = 512, 256, 128
+    L = layer(42, K, N, bits, gs, True, M=6, bias=True)
+    q = QuantLinear(bits, gs, K, N, True)
+    q.load_state_dict({k: L[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})
+    q = q.to(dev)
+    x = L["x"].reshape(2, 3, K).to(dev)
+    y = q(x)
+    assert y.shape == (2, 3, N) and y.dtype == torch.float16
+    assert_close(y.reshape(6, N), expected_output(L), "module forward")
+    y32 = q(x.float())  # any float dtype is accepted and cast to fp16, as the reference does
+    assert torch.equal(y32, y)
+    w = q.dequantize().cpu()
+    assert torch.equal(w.view(torch.int16), expected_weight(L).view(torch.int16))
+    # contiguous g_idx is detected and handled by the no-gather path
+    q2 = QuantLinear(bits, gs, K, N, False)
+    L2 = layer(43, K, N, bits, gs, False, M=1)
+    q2.load_state_dict({k: L2[k] for k in ("qweight", "qzeros", "scales", "g_idx")})
+    q2 = q2.to(dev)
+    assert q2._kernel_g_idx() is None
+    assert_close(q2(L2["x"].to(dev)), expected_output(L2), "module forward, contiguous groups")
+
+
+def test_bad_g_idx_is_rejected_by_the_module(dev):
+    q = QuantLinear(4, 32, 64, 32, False).to(dev)
+    q.g_idx[3] = 99
+    with pytest.raises(ValueError, match="g_idx"):
+        q(torch.zeros(1, 64, device=dev))

@@ -1,0 +1,62 @@
+"""Host-side behaviour of QuantLinear that needs no GPU: constructor contract, buffer names,
+meta-device construction, and loud failure when asked to compute off the GPU."""
+import pytest
+import torch
+
+from autogptq.tvm_amd import QuantLinear, ops
+
+
+def test_buffers_follow_the_reference_layout():
+    q = QuantLinear(3, 128, 4096, 11008, True)
+    sd = q.state_dict()
+    assert set(sd) == {"qweight", "qzeros", "scales", "g_idx", "bias"}
+    assert sd["qweight"].shape == (384, 11008) and sd["qweight"].dtype == torch.int32
+    assert sd["qzeros"].shape == (32, 1032) and sd["qzeros"].dtype == torch.int32
+    assert sd["scales"].shape == (32, 11008) and sd["scales"].dtype == torch.float16
+    assert sd["g_idx"].shape == (4096,) and sd["g_idx"].dtype == torch.int32
+    assert sd["g_idx"][127] == 0 and sd["g_idx"][128] == 1
+    assert q.maxq == 7 and q.groupsize == 128 and q.infeatures == 4096 and q.outfeatures == 11008
+    q = QuantLinear(4, -1, 9216, 9216, False)
+    assert q.groupsize == 9216 and q.bias is None
+    assert q.scales.shape == (1, 9216) and q.qzeros.shape == (1, 1152)
+    assert set(q.state_dict()) == {"qweight", "qzeros", "scales", "g_idx"}
+
+
+@pytest.mark.parametrize("bits", [2, 5, 8, 16])
+def test_unsupported_bits_raise(bits):
+    with pytest.raises(NotImplementedError):
+        QuantLinear(bits, 128, 256, 256, False)
+
+
+def test_constructs_on_meta_device_without_touching_a_gpu():
+    with torch.device("meta"):
+        q = QuantLinear(4, 128, 4096, 4096, True)
+    assert q.qweight.is_meta and q.scales.is_meta and q.g_idx.is_meta
+
+
+def test_state_dict_round_trip():
+    a = QuantLinear(4, 32, 64, 32, True)
+    a.qweight.random_(0, 1000)
+    a.scales.fill_(0.5)
+    b = QuantLinear(4, 32, 64, 32, True)
+    b.load_state_dict(a.state_dict())
+    assert torch.equal(b.qweight, a.qweight) and torch.equal(b.scales, a.scales)
+
+
+def test_forward_on_cpu_fails_loudly():
+    q = QuantLinear(4, 32, 64, 32, False)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        q(torch.zeros(1, 64))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.dequant(q.qweight, q.qzeros, q.scales, None, 4, 32)
+
+
+def test_shape_checks():
+    q = QuantLinear(4, 32, 64, 32, False)
+    with pytest.raises(ValueError):
+        ops.check_shapes(q.qweight, q.qzeros, q.scales[:, :16], None, None, 4, 32)
+    with pytest.raises(ValueError):
+        ops.check_shapes(q.qweight, q.qzeros, q.scales, q.g_idx[:10], None, 4, 32)
+    with pytest.raises(NotImplementedError):
+        ops.check_shapes(q.qweight, q.qzeros, q.scales, None, None, 2, 32)
+    assert ops.check_shapes(q.qweight, q.qzeros, q.scales, q.g_idx, None, 4, 32) == (64, 32, 2)
