@@ -122,11 +122,13 @@ GPTQ_HD h2 code_from_magic3(uint32_t m, int r)
 }
 
 // The dequantised weight of the reference (qlinear.py:242): fp16 scale times the
-// integer (q - zero), rounded once.  The product of an 11-bit significand and an
-// integer of magnitude <= 16 is exact in fp32, so one conversion gives that rounding.
+// integer (q - zero), rounded once.  (q - zero) is exact in fp16, so one fp16 multiply
+// is that rounding, signed zeros and subnormals included.  (Going through an fp32
+// product and a conversion is equal in value, but the compiler fuses it into a
+// mixed-precision fma with a +0 addend, which turns -0 results into +0.)
 GPTQ_HD _Float16 dequant_one(_Float16 scale, int q, int zero)
 {
-    return (_Float16)((float)scale * (float)(q - zero));
+    return scale * (_Float16)(float)(q - zero);
 }
 
 }  // namespace gptq

@@ -62,8 +62,8 @@ int main()
         const _Float16 s = (_Float16)(0.001f + (float)(rnd() & 0xffff) / 65536.0f * 0.009f);
         const int q = (int)(rnd() & 15), z = 1 + (int)(rnd() & 15);
         const _Float16 d = dequant_one(s, q, z);
-        const _Float16 e = (_Float16)(s * (_Float16)(float)(q - z));  // fp16 multiply
-        if ((float)d != (float)e) {
+        const _Float16 e = (_Float16)((float)s * (float)(q - z));  // exact fp32 product, one rounding
+        if (__builtin_bit_cast(uint16_t, d) != __builtin_bit_cast(uint16_t, e)) {
             printf("dequant mismatch s=%f q=%d z=%d\n", (float)s, q, z);
             return 1;
         }
