@@ -23,6 +23,7 @@ KERNEL_BLOCKED = 3
 
 ABI_SYMBOLS = (
     "gptq_hip_select",
+    "gptq_hip_plan_for",
     "gptq_hip_workspace_bytes",
     "gptq_hip_workspace_init",
     "gptq_hip_gemm",
@@ -79,6 +80,8 @@ def lib() -> ctypes.CDLL:
     vp, i, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
     l.gptq_hip_select.restype = i
     l.gptq_hip_select.argtypes = [i, i, i, i, i, i, ctypes.POINTER(Plan)]
+    l.gptq_hip_plan_for.restype = i
+    l.gptq_hip_plan_for.argtypes = [i, i, i, i, i, i, i, i, i, ctypes.POINTER(Plan)]
     l.gptq_hip_workspace_bytes.restype = sz
     l.gptq_hip_workspace_bytes.argtypes = [i, i, i, i, i, i]
     l.gptq_hip_workspace_init.restype = i
@@ -106,4 +109,16 @@ def select(M: int, K: int, N: int, bits: int, group_size: int, act_order: bool) 
     rc = lib().gptq_hip_select(M, K, N, bits, group_size, int(bool(act_order)), ctypes.byref(plan))
     if rc != OK:
         raise GptqHipError(rc, f"gptq_hip_select(M={M}, K={K}, N={N}, bits={bits}, group_size={group_size})")
+    return plan
+
+
+def plan_for(kernel: int, M: int, K: int, N: int, bits: int, group_size: int, act_order: bool,
+             split_k: int = 0, waves_n: int = 0) -> Plan:
+    """Plan of one kernel family with ``split_k`` / ``waves_n`` forced (0 = dispatcher's choice)."""
+    plan = Plan()
+    rc = lib().gptq_hip_plan_for(kernel, M, K, N, bits, group_size, int(bool(act_order)), split_k, waves_n,
+                                 ctypes.byref(plan))
+    if rc != OK:
+        raise GptqHipError(rc, f"gptq_hip_plan_for(kernel={kernel}, M={M}, K={K}, N={N}, bits={bits}, "
+                               f"group_size={group_size}, split_k={split_k}, waves_n={waves_n})")
     return plan

@@ -19,27 +19,39 @@ int check_common(const int32_t *qweight, const int32_t *qzeros, const void *scal
     return GPTQ_HIP_OK;
 }
 
-int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G)
+int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G, int gs, int act_order)
 {
     const int kstep = gptq::kstep_of(bits);
-    if (pl.kernel != GPTQ_HIP_KERNEL_GATHER) return GPTQ_HIP_ERR_UNSUPPORTED;
-    if (pl.row_tiles != 1 && pl.row_tiles != 2 && pl.row_tiles != 4 && pl.row_tiles != 8)
-        return GPTQ_HIP_ERR_UNSUPPORTED;
+    const int steps_total = (K + kstep - 1) / kstep;
     if (pl.waves_n != 1 && pl.waves_n != 2 && pl.waves_n != 4) return GPTQ_HIP_ERR_UNSUPPORTED;
     if (pl.block != 64 * pl.waves_n) return GPTQ_HIP_ERR_BAD_ARG;
-    if (pl.k_chunk < kstep || pl.k_chunk % kstep != 0) return GPTQ_HIP_ERR_BAD_ARG;
-    const int steps_total = (K + kstep - 1) / kstep;
     if (pl.split_k < 1 || pl.split_k > steps_total) return GPTQ_HIP_ERR_BAD_ARG;
-    if (pl.m_blocks * 16 * pl.row_tiles < M) return GPTQ_HIP_ERR_BAD_ARG;
-    if (pl.grid_x * 64 * pl.waves_n < N || pl.grid_y != pl.split_k || pl.grid_z != pl.m_blocks)
-        return GPTQ_HIP_ERR_BAD_ARG;
-    const int xs_rows = M < 16 * pl.row_tiles ? M : 16 * pl.row_tiles;
-    const long long need = (long long)G * 64 * pl.waves_n * 4 + (long long)pl.k_chunk * 4 +
-                           (long long)xs_rows * (pl.k_chunk + 8) * 2;
-    if (pl.lds_bytes < need || pl.lds_bytes > 160 * 1024) return GPTQ_HIP_ERR_BAD_ARG;
-    if (pl.split_k > 1 && (size_t)pl.grid_x * pl.grid_z * sizeof(int) > gptq::kCounterBytes)
+    if (pl.grid_x * 64 * pl.waves_n < N || pl.grid_y != pl.split_k) return GPTQ_HIP_ERR_BAD_ARG;
+    if (pl.lds_bytes > 160 * 1024) return GPTQ_HIP_ERR_BAD_ARG;
+    if (pl.split_k > 1 && (size_t)pl.grid_x * (pl.grid_z > 0 ? pl.grid_z : 1) * sizeof(int) > gptq::kCounterBytes)
         return GPTQ_HIP_ERR_UNSUPPORTED;
-    return GPTQ_HIP_OK;
+    if (pl.kernel == GPTQ_HIP_KERNEL_GATHER) {
+        if (pl.row_tiles != 1 && pl.row_tiles != 2 && pl.row_tiles != 4 && pl.row_tiles != 8)
+            return GPTQ_HIP_ERR_UNSUPPORTED;
+        if (pl.k_chunk < kstep || pl.k_chunk % kstep != 0) return GPTQ_HIP_ERR_BAD_ARG;
+        if (pl.m_blocks * 16 * pl.row_tiles < M || pl.grid_z != pl.m_blocks) return GPTQ_HIP_ERR_BAD_ARG;
+        const int xs_rows = M < 16 * pl.row_tiles ? M : 16 * pl.row_tiles;
+        const long long need = (long long)G * 64 * pl.waves_n * 4 + (long long)pl.k_chunk * 4 +
+                               (long long)xs_rows * (pl.k_chunk + 8) * 2;
+        if (pl.lds_bytes < need) return GPTQ_HIP_ERR_BAD_ARG;
+        return GPTQ_HIP_OK;
+    }
+    if (pl.kernel == GPTQ_HIP_KERNEL_GROUPED) {
+        if (M > 2 || pl.grid_z != 1 || pl.row_tiles % M != 0) return GPTQ_HIP_ERR_UNSUPPORTED;
+        const int steps = (steps_total + pl.split_k - 1) / pl.split_k;
+        const int kr = steps * kstep;
+        const int tpm = pl.row_tiles / M;
+        const int need_tpm = gptq::grouped_tpm(gptq::grouped_groups(kr, gs, G, act_order), M);
+        if (need_tpm == 0 || tpm != need_tpm) return GPTQ_HIP_ERR_UNSUPPORTED;
+        if (pl.lds_bytes < (long long)kr * pl.row_tiles * 32) return GPTQ_HIP_ERR_BAD_ARG;
+        return GPTQ_HIP_OK;
+    }
+    return GPTQ_HIP_ERR_UNSUPPORTED;
 }
 
 }  // namespace
@@ -56,7 +68,9 @@ extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const i
         return GPTQ_HIP_ERR_BAD_ARG;
     const int gs = group_size == -1 ? K : group_size;
     const int G = (K + gs - 1) / gs;
-    rc = validate_plan(*plan, M, K, N, bits, G);
+    const int act_order = (g_idx != nullptr && G > 1) ? 1 : 0;
+    if (G == 1) g_idx = nullptr;  // a single group: the gather has nothing to choose
+    rc = validate_plan(*plan, M, K, N, bits, G, gs, act_order);
     if (rc != GPTQ_HIP_OK) return rc;
 
     gptq::Params p;
@@ -80,13 +94,15 @@ extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const i
     p.chunk_steps = plan->k_chunk / kstep;
     p.xs_rows = M < 16 * plan->row_tiles ? M : 16 * plan->row_tiles;
     p.row_tiles = plan->row_tiles;
+    p.gpad = plan->kernel == GPTQ_HIP_KERNEL_GROUPED ? 16 * (plan->row_tiles / M) : 0;
     if (plan->split_k > 1) {
         const size_t need = gptq::kCounterBytes + (size_t)plan->split_k * M * N * sizeof(float);
         if (!workspace || workspace_bytes < need || !aligned(workspace, 16)) return GPTQ_HIP_ERR_WORKSPACE;
         p.counters = (int *)workspace;
         p.partial = (float *)((char *)workspace + gptq::kCounterBytes);
     }
-    return gptq::launch_matmul(p, bits, *plan, stream);
+    if (plan->kernel == GPTQ_HIP_KERNEL_GROUPED) return gptq::launch_grouped(p, bits, *plan, stream);
+    return gptq::launch_gather(p, bits, *plan, stream);
 }
 
 extern "C" int gptq_hip_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,

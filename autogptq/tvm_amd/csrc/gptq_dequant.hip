@@ -1,0 +1,77 @@
+// Dequantisation (bit-exact fp16 weight) and workspace fill kernels.
+#include "gptq_device.h"
+
+namespace gptq {
+
+// ---------------------------------------------------------------------------------
+// DEQUANT kernel: the materialised fp16 weight, bit for bit what the reference
+// computes (qlinear.py:198-242).  One thread per (32 input channels, column).
+// ---------------------------------------------------------------------------------
+template <int BITS>
+__global__ __launch_bounds__(256) void dequant_kernel(const uint32_t *__restrict__ qweight,
+                                                      const uint32_t *__restrict__ qzeros,
+                                                      const _Float16 *__restrict__ scales,
+                                                      const int32_t *__restrict__ g_idx, _Float16 *__restrict__ W,
+                                                      int K, int N, int G, int group_size)
+{
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    const int kb = blockIdx.y;  // block of 32 input channels
+    if (n >= N) return;
+    const int zwords = N / 32 * BITS;
+    uint32_t w[BITS];
+#pragma unroll
+    for (int i = 0; i < BITS; i++) w[i] = qweight[(size_t)(kb * BITS + i) * N + n];
+    int g_prev = -1;
+    _Float16 s = (_Float16)0.0f;
+    int z = 0;
+    for (int j = 0; j < 32; j++) {
+        const int k = kb * 32 + j;
+        int g = g_idx ? g_idx[k] : k / group_size;
+        g = min(max(g, 0), G - 1);
+        if (g != g_prev) {
+            s = scales[(size_t)g * N + n];
+            z = zero_of<BITS>(qzeros + (size_t)g * zwords, n);
+            g_prev = g;
+        }
+        int q;
+        if constexpr (BITS == 4) {
+            q = code4(w[j >> 3], j & 7);
+        } else {
+            q = code3(w[0], w[1], w[2], j);
+        }
+        W[(size_t)k * N + n] = dequant_one(s, q, z);
+    }
+}
+
+__global__ void fill_zero_kernel(uint32_t *ptr, size_t words)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < words) ptr[i] = 0u;
+}
+
+int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
+                   void *w, int K, int N, int G, int bits, int group_size, void *stream_v)
+{
+    hipStream_t stream = (hipStream_t)stream_v;
+    const dim3 grid((N + 255) / 256, K / 32);
+    if (bits == 4) {
+        hipLaunchKernelGGL(dequant_kernel<4>, grid, dim3(256), 0, stream, qweight, qzeros,
+                           (const _Float16 *)scales, g_idx, (_Float16 *)w, K, N, G, group_size);
+    } else {
+        hipLaunchKernelGGL(dequant_kernel<3>, grid, dim3(256), 0, stream, qweight, qzeros,
+                           (const _Float16 *)scales, g_idx, (_Float16 *)w, K, N, G, group_size);
+    }
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+}
+
+int launch_fill_zero(void *ptr, size_t bytes, void *stream_v)
+{
+    hipStream_t stream = (hipStream_t)stream_v;
+    const size_t words = bytes / 4;
+    if (words == 0) return GPTQ_HIP_OK;
+    const unsigned blocks = (unsigned)((words + 255) / 256);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, stream, (uint32_t *)ptr, words);
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+}
+
+}  // namespace gptq

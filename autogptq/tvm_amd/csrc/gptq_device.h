@@ -1,0 +1,112 @@
+// Device-side pieces shared by the GPTQ int3/int4 matmul kernels on gfx950 (CDNA4, wave64).
+//
+// Common geometry of the matmul kernels
+// -------------------------------------
+// The product runs on v_mfma_f32_16x16x32_f16.  A wave owns 64 output columns:
+// lane (i = lane % 16, q = lane / 16) loads one 128-bit vector of qweight per packed
+// row, i.e. the four adjacent columns n0 + 4i .. n0 + 4i + 3, so a wave load is four
+// 256-byte runs.  Column set c (0..3) of a wave is {n0 + 4i + c : i = 0..15}; it is the
+// N dimension of one MFMA.  The K dimension of an MFMA is 4 lane groups x 8 codes:
+// lane group q supplies 8 codes of ITS packed row (int4: one word row = 8 codes;
+// int3: one 3-word block = 32 codes = four MFMAs), and the activation operand
+// supplies x for the same input channels in the same order.  That order is the
+// "slot" order of gptq_unpack.h (codes come out of the magic-number unpack in pairs
+// that are not adjacent in k); x is written to LDS already permuted into slot order.
+//
+// One "step" of a wave is 4 packed rows (int4: 32 input channels, int3: 128).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "gptq_internal.h"
+#include "gptq_unpack.h"
+
+namespace gptq {
+
+template <int BITS>
+struct Fmt;
+template <>
+struct Fmt<4> {
+    static constexpr int KLANE = 8;    // codes per lane per step
+    static constexpr int NB = 1;       // MFMAs along K per column set per step
+    static constexpr int WORDS = 1;    // 128-bit loads per lane per step
+    static constexpr int KSTEP = 32;   // input channels per wave step
+};
+template <>
+struct Fmt<3> {
+    static constexpr int KLANE = 32;
+    static constexpr int NB = 4;
+    static constexpr int WORDS = 3;
+    static constexpr int KSTEP = 128;
+};
+
+struct InvTables {
+    unsigned char inv4[8];
+    unsigned char inv3[32];
+    constexpr InvTables() : inv4(), inv3()
+    {
+        for (int s = 0; s < 8; s++) inv4[SLOT4[s]] = (unsigned char)s;
+        for (int s = 0; s < 32; s++) inv3[SLOT3[s]] = (unsigned char)s;
+    }
+};
+static __constant__ InvTables kInv = InvTables();
+
+// slot (position in the MFMA operand order) of code j of a lane block
+template <int BITS>
+__device__ __forceinline__ int slot_of_code(int j)
+{
+    return BITS == 4 ? (int)kInv.inv4[j] : (int)kInv.inv3[j];
+}
+
+template <int BITS>
+__device__ __forceinline__ int zero_of(const uint32_t *zrow, int n)
+{
+    return BITS == 4 ? zero4(zrow, n) : zero3(zrow, n);
+}
+
+extern __shared__ __align__(16) unsigned char smem[];
+
+// ---------------------------------------------------------------------------------
+// Split-K tail: every workgroup of a column tile writes its fp32 partial tile, the one
+// that arrives last adds them in split order (so the sum does not depend on arrival
+// order) and writes y.
+//
+// The partials travel through device-coherent accesses only (relaxed agent-scope
+// atomic stores and loads: write-through stores and L2-bypassing loads), so no cache
+// writeback or invalidate is needed around the counter: an agent-scope release fence
+// here costs a whole-L2 writeback per wave, which serialises the workgroups of an XCD
+// and dominated the run time of the first version of these kernels.  Waiting for the
+// stores to be acknowledged before the counter is bumped is all the ordering required.
+// ---------------------------------------------------------------------------------
+__device__ __forceinline__ void store_partial(float *dst, f4 v)
+{
+#pragma unroll
+    for (int c = 0; c < 4; c++) __hip_atomic_store(dst + c, v[c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ f4 load_partial(const float *src)
+{
+    f4 v;
+#pragma unroll
+    for (int c = 0; c < 4; c++) v[c] = __hip_atomic_load(src + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return v;
+}
+
+// Returns true in the workgroup that must do the final sum.  Every thread calls it.
+__device__ __forceinline__ bool arrive_last(int *counter, int split_k, int *lds_flag)
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partial stores are acknowledged
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int last = (old == split_k - 1);
+        if (last) {
+            // leave the counter at zero for the next launch that uses this workspace
+            __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        *lds_flag = last;
+    }
+    __syncthreads();
+    return *lds_flag != 0;
+}
+
+}  // namespace gptq

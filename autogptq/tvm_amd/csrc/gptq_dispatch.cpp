@@ -14,22 +14,11 @@ const int kTargetWorkgroups = 512;  // two per CU keeps every XCD fed at M = 1
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-}  // namespace
-
-extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, int act_order, gptq_hip_plan *plan)
+// GATHER: exact weights, any g_idx, any M.
+int plan_gather(int M, int K, int N, int bits, int G, int force_split, int force_waves, gptq_hip_plan *plan)
 {
-    if (!plan) return GPTQ_HIP_ERR_BAD_ARG;
-    memset(plan, 0, sizeof(*plan));
-    if (bits != 3 && bits != 4) return GPTQ_HIP_ERR_BAD_ARG;
-    if (M < 1 || K < 32 || N < 32) return GPTQ_HIP_ERR_BAD_ARG;
-    if (K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;  // the packed format needs both
-    if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
-    (void)act_order;
-    const int gs = group_size == -1 ? K : group_size;
-    const int G = ceil_div(K, gs);
     const int kstep = gptq::kstep_of(bits);
     const int steps_total = ceil_div(K, kstep);
-
     plan->kernel = GPTQ_HIP_KERNEL_GATHER;
     plan->row_tiles = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8));
     plan->m_blocks = ceil_div(M, 16 * plan->row_tiles);
@@ -37,9 +26,8 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     int kc = xs_rows <= 16 ? 512 : (xs_rows <= 32 ? 256 : 128);
     if (kc > steps_total * kstep) kc = steps_total * kstep;
     plan->k_chunk = kc;
-    const int chunk_steps = kc / kstep;
 
-    int waves = 4;
+    int waves = force_waves > 0 ? force_waves : 4;
     int lds = 0;
     for (; waves >= 1; waves >>= 1) {
         const int bn = 64 * waves;
@@ -58,10 +46,10 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     int cap = (int)(((long long)K * bits) / (128LL * M));
     if (cap < 1) cap = 1;
     if (split > cap) split = cap;
-    const int max_split = steps_total / (chunk_steps > 0 ? 1 : 1);
-    if (split > max_split) split = max_split;
+    if (split > steps_total) split = steps_total;
     if (split > 64) split = 64;
     if (split < 1) split = 1;
+    if (force_split > 0) split = force_split > steps_total ? steps_total : force_split;
     if ((size_t)col_tiles * plan->m_blocks * sizeof(int) > gptq::kCounterBytes) split = 1;
     plan->split_k = split;
     plan->grid_x = col_tiles;
@@ -69,6 +57,114 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     plan->grid_z = plan->m_blocks;
     plan->workspace_bytes = split > 1 ? gptq::kCounterBytes + (size_t)split * M * N * sizeof(float) : 0;
     return GPTQ_HIP_OK;
+}
+
+}  // namespace
+
+namespace gptq {
+
+// Row tiles (of 16 groups) per activation row that the GROUPED kernel is built for.
+int grouped_tpm(int groups, int M)
+{
+    int tpm = ceil_div(groups, 16);
+    if (tpm == 5) tpm = 6;
+    const int max_tpm = M == 1 ? 6 : 2;
+    return tpm <= max_tpm ? tpm : 0;
+}
+
+// Upper bound of the number of distinct groups one K range of `kr` channels can touch.
+int grouped_groups(int kr, int gs, int G, int act_order)
+{
+    int groups = act_order ? G : (kr - 1) / gs + 2;
+    return groups > G ? G : groups;
+}
+
+}  // namespace gptq
+
+namespace {
+
+// GROUPED: rows expanded by group, M of 1 or 2.  Returns false when the shape does not fit
+// (too many groups for the row tiles, or an LDS operand that no split makes small enough).
+bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, int force_split, int force_waves,
+                  gptq_hip_plan *plan)
+{
+    const int kstep = gptq::kstep_of(bits);
+    const int steps_total = ceil_div(K, kstep);
+    const int waves = force_waves > 0 ? force_waves : 4;
+    const int col_tiles = ceil_div(N, 64 * waves);
+    if ((size_t)col_tiles * sizeof(int) > gptq::kCounterBytes) return false;
+    const int lds_cap = 64 * 1024;
+    int want = force_split > 0 ? force_split : ceil_div(kTargetWorkgroups, col_tiles);
+    if (want > steps_total) want = steps_total;
+    if (want < 1) want = 1;
+    for (int split = want; split <= steps_total && split <= 256; split++) {
+        if (force_split > 0 && split != want) return false;
+        const int steps = ceil_div(steps_total, split);  // the longest K range, in steps
+        const int kr = steps * kstep;
+        const int tpm = gptq::grouped_tpm(gptq::grouped_groups(kr, gs, G, act_order), M);
+        if (tpm == 0) {
+            if (act_order) return false;  // the group count does not shrink with the K range
+            continue;
+        }
+        const int rt = M * tpm;
+        const int lds = kr * rt * 32;
+        if (lds > lds_cap) continue;
+        plan->kernel = GPTQ_HIP_KERNEL_GROUPED;
+        plan->row_tiles = rt;
+        plan->m_blocks = 1;
+        plan->waves_n = waves;
+        plan->waves_k = 1;
+        plan->split_k = split;
+        plan->k_chunk = kr;
+        plan->grid_x = col_tiles;
+        plan->grid_y = split;
+        plan->grid_z = 1;
+        plan->block = 64 * waves;
+        plan->lds_bytes = lds;
+        plan->workspace_bytes = split > 1 ? gptq::kCounterBytes + (size_t)split * M * N * sizeof(float) : 0;
+        return true;
+    }
+    return false;
+}
+
+}  // namespace
+
+extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, int act_order, gptq_hip_plan *plan)
+{
+    if (!plan) return GPTQ_HIP_ERR_BAD_ARG;
+    memset(plan, 0, sizeof(*plan));
+    if (bits != 3 && bits != 4) return GPTQ_HIP_ERR_BAD_ARG;
+    if (M < 1 || K < 32 || N < 32) return GPTQ_HIP_ERR_BAD_ARG;
+    if (K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;  // the packed format needs both
+    if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
+    const int gs = group_size == -1 ? K : group_size;
+    const int G = ceil_div(K, gs);
+    // one group for the whole matrix: g_idx carries no information
+    if (G == 1) act_order = 0;
+    if (M <= 2 && plan_grouped(M, K, N, bits, gs, G, act_order, 0, 0, plan)) return GPTQ_HIP_OK;
+    memset(plan, 0, sizeof(*plan));
+    return plan_gather(M, K, N, bits, G, 0, 0, plan);
+}
+
+extern "C" int gptq_hip_plan_for(int kernel, int M, int K, int N, int bits, int group_size, int act_order,
+                                 int split_k, int waves_n, gptq_hip_plan *plan)
+{
+    gptq_hip_plan tmp;
+    const int rc = gptq_hip_select(M, K, N, bits, group_size, act_order, &tmp);  // argument checks
+    if (rc != GPTQ_HIP_OK) return rc;
+    if (!plan || split_k < 0 || (waves_n != 0 && waves_n != 1 && waves_n != 2 && waves_n != 4))
+        return GPTQ_HIP_ERR_BAD_ARG;
+    memset(plan, 0, sizeof(*plan));
+    const int gs = group_size == -1 ? K : group_size;
+    const int G = ceil_div(K, gs);
+    if (G == 1) act_order = 0;
+    if (kernel == GPTQ_HIP_KERNEL_GATHER) return plan_gather(M, K, N, bits, G, split_k, waves_n, plan);
+    if (kernel == GPTQ_HIP_KERNEL_GROUPED) {
+        if (M <= 2 && plan_grouped(M, K, N, bits, gs, G, act_order, split_k, waves_n, plan)) return GPTQ_HIP_OK;
+        memset(plan, 0, sizeof(*plan));
+        return GPTQ_HIP_ERR_UNSUPPORTED;
+    }
+    return GPTQ_HIP_ERR_UNSUPPORTED;
 }
 
 extern "C" size_t gptq_hip_workspace_bytes(int M, int K, int N, int bits, int group_size, int act_order)

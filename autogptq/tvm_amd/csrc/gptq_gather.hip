@@ -1,94 +1,7 @@
-// HIP kernels for the GPTQ int3/int4 QuantLinear product on gfx950 (CDNA4, wave64).
-//
-// Common geometry of the matmul kernels
-// -------------------------------------
-// The product runs on v_mfma_f32_16x16x32_f16.  A wave owns 64 output columns:
-// lane (i = lane % 16, q = lane / 16) loads one 128-bit vector of qweight per packed
-// row, i.e. the four adjacent columns n0 + 4i .. n0 + 4i + 3, so a wave load is four
-// 256-byte runs.  Column set c (0..3) of a wave is {n0 + 4i + c : i = 0..15}; it is the
-// N dimension of one MFMA.  The K dimension of an MFMA is 4 lane groups x 8 codes:
-// lane group q supplies 8 codes of ITS packed row (int4: one word row = 8 codes;
-// int3: one 3-word block = 32 codes = four MFMAs), and the activation operand
-// supplies x for the same input channels in the same order.  That order is the
-// "slot" order of gptq_unpack.h (codes come out of the magic-number unpack in pairs
-// that are not adjacent in k); x is written to LDS already permuted into slot order.
-//
-// One "step" of a wave is 4 packed rows (int4: 32 input channels, int3: 128).
-#include <hip/hip_runtime.h>
-
-#include "gptq_internal.h"
-#include "gptq_unpack.h"
+// GATHER kernel family: see the geometry notes in gptq_device.h.
+#include "gptq_device.h"
 
 namespace gptq {
-
-template <int BITS>
-struct Fmt;
-template <>
-struct Fmt<4> {
-    static constexpr int KLANE = 8;    // codes per lane per step
-    static constexpr int NB = 1;       // MFMAs along K per column set per step
-    static constexpr int WORDS = 1;    // 128-bit loads per lane per step
-    static constexpr int KSTEP = 32;   // input channels per wave step
-};
-template <>
-struct Fmt<3> {
-    static constexpr int KLANE = 32;
-    static constexpr int NB = 4;
-    static constexpr int WORDS = 3;
-    static constexpr int KSTEP = 128;
-};
-
-struct InvTables {
-    unsigned char inv4[8];
-    unsigned char inv3[32];
-    constexpr InvTables() : inv4(), inv3()
-    {
-        for (int s = 0; s < 8; s++) inv4[SLOT4[s]] = (unsigned char)s;
-        for (int s = 0; s < 32; s++) inv3[SLOT3[s]] = (unsigned char)s;
-    }
-};
-__constant__ InvTables kInv = InvTables();
-
-// slot (position in the MFMA operand order) of code j of a lane block
-template <int BITS>
-__device__ __forceinline__ int slot_of_code(int j)
-{
-    return BITS == 4 ? (int)kInv.inv4[j] : (int)kInv.inv3[j];
-}
-
-template <int BITS>
-__device__ __forceinline__ int zero_of(const uint32_t *zrow, int n)
-{
-    return BITS == 4 ? zero4(zrow, n) : zero3(zrow, n);
-}
-
-extern __shared__ __align__(16) unsigned char smem[];
-
-// ---------------------------------------------------------------------------------
-// Split-K tail: every workgroup of a column tile writes its fp32 partial tile, the one
-// that arrives last adds them in split order (so the sum does not depend on arrival
-// order) and writes y.  Returns true in the workgroup that must do the final sum.
-// ---------------------------------------------------------------------------------
-__device__ __forceinline__ bool arrive_last(int *counter, int split_k, int *lds_flag)
-{
-    __threadfence();  // publish this thread's partials device-wide
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        const int last = (old == split_k - 1);
-        if (last) {
-            // leave the counter at zero for the next launch that uses this workspace
-            __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        *lds_flag = last;
-    }
-    __syncthreads();
-    const bool last = *lds_flag != 0;
-    if (last) {
-        __threadfence();  // see the other workgroups' partials
-    }
-    return last;
-}
 
 // ---------------------------------------------------------------------------------
 // GATHER kernel: exact fp16 weights, scale/zero looked up per weight through g_idx.
@@ -275,7 +188,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
                 const int row = 16 * rt + 4 * lq + v;
                 if (row < rows_here) {
                     const f4 o = {acc[rt][0][v], acc[rt][1][v], acc[rt][2][v], acc[rt][3][v]};
-                    *(f4 *)(p.partial + ((size_t)split * p.M + (m0 + row)) * p.N + n0) = o;
+                    store_partial(p.partial + ((size_t)split * p.M + (m0 + row)) * p.N + n0, o);
                 }
             }
         }
@@ -291,9 +204,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
                 if (row < rows_here) {
                     f4 sum = bv;
                     for (int s = 0; s < p.split_k; s++) {
-                        const f4 t = __builtin_nontemporal_load(
-                            (const f4 *)(p.partial + ((size_t)s * p.M + (m0 + row)) * p.N + n0));
-                        sum += t;
+                        sum += load_partial(p.partial + ((size_t)s * p.M + (m0 + row)) * p.N + n0);
                     }
                     h4 o;
 #pragma unroll
@@ -305,57 +216,8 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
     }
 }
 
-// ---------------------------------------------------------------------------------
-// DEQUANT kernel: the materialised fp16 weight, bit for bit what the reference
-// computes (qlinear.py:198-242).  One thread per (32 input channels, column).
-// ---------------------------------------------------------------------------------
-template <int BITS>
-__global__ __launch_bounds__(256) void dequant_kernel(const uint32_t *__restrict__ qweight,
-                                                      const uint32_t *__restrict__ qzeros,
-                                                      const _Float16 *__restrict__ scales,
-                                                      const int32_t *__restrict__ g_idx, _Float16 *__restrict__ W,
-                                                      int K, int N, int G, int group_size)
-{
-    const int n = blockIdx.x * blockDim.x + threadIdx.x;
-    const int kb = blockIdx.y;  // block of 32 input channels
-    if (n >= N) return;
-    const int zwords = N / 32 * BITS;
-    uint32_t w[BITS];
-#pragma unroll
-    for (int i = 0; i < BITS; i++) w[i] = qweight[(size_t)(kb * BITS + i) * N + n];
-    int g_prev = -1;
-    _Float16 s = (_Float16)0.0f;
-    int z = 0;
-    for (int j = 0; j < 32; j++) {
-        const int k = kb * 32 + j;
-        int g = g_idx ? g_idx[k] : k / group_size;
-        g = min(max(g, 0), G - 1);
-        if (g != g_prev) {
-            s = scales[(size_t)g * N + n];
-            z = zero_of<BITS>(qzeros + (size_t)g * zwords, n);
-            g_prev = g;
-        }
-        int q;
-        if constexpr (BITS == 4) {
-            q = code4(w[j >> 3], j & 7);
-        } else {
-            q = code3(w[0], w[1], w[2], j);
-        }
-        W[(size_t)k * N + n] = dequant_one(s, q, z);
-    }
-}
-
-__global__ void fill_zero_kernel(uint32_t *ptr, size_t words)
-{
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < words) ptr[i] = 0u;
-}
-
-// ---------------------------------------------------------------------------------
-// Launchers
-// ---------------------------------------------------------------------------------
 template <int BITS, int RT>
-static int launch_gather(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
+static int launch_gather_one(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
     auto kern = gather_kernel<BITS, RT>;
     if (plan.lds_bytes > 65536) {
@@ -374,48 +236,18 @@ template <int BITS>
 static int launch_gather_rt(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
     switch (plan.row_tiles) {
-        case 1: return launch_gather<BITS, 1>(p, plan, stream);
-        case 2: return launch_gather<BITS, 2>(p, plan, stream);
-        case 4: return launch_gather<BITS, 4>(p, plan, stream);
-        case 8: return launch_gather<BITS, 8>(p, plan, stream);
+        case 1: return launch_gather_one<BITS, 1>(p, plan, stream);
+        case 2: return launch_gather_one<BITS, 2>(p, plan, stream);
+        case 4: return launch_gather_one<BITS, 4>(p, plan, stream);
+        case 8: return launch_gather_one<BITS, 8>(p, plan, stream);
         default: return GPTQ_HIP_ERR_UNSUPPORTED;
     }
 }
 
-int launch_matmul(const Params &p, int bits, const gptq_hip_plan &plan, void *stream_v)
+int launch_gather(const Params &p, int bits, const gptq_hip_plan &plan, void *stream)
 {
-    hipStream_t stream = (hipStream_t)stream_v;
-    switch (plan.kernel) {
-        case GPTQ_HIP_KERNEL_GATHER:
-            return bits == 4 ? launch_gather_rt<4>(p, plan, stream) : launch_gather_rt<3>(p, plan, stream);
-        default:
-            return GPTQ_HIP_ERR_UNSUPPORTED;
-    }
-}
-
-int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
-                   void *w, int K, int N, int G, int bits, int group_size, void *stream_v)
-{
-    hipStream_t stream = (hipStream_t)stream_v;
-    const dim3 grid((N + 255) / 256, K / 32);
-    if (bits == 4) {
-        hipLaunchKernelGGL(dequant_kernel<4>, grid, dim3(256), 0, stream, qweight, qzeros,
-                           (const _Float16 *)scales, g_idx, (_Float16 *)w, K, N, G, group_size);
-    } else {
-        hipLaunchKernelGGL(dequant_kernel<3>, grid, dim3(256), 0, stream, qweight, qzeros,
-                           (const _Float16 *)scales, g_idx, (_Float16 *)w, K, N, G, group_size);
-    }
-    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
-}
-
-int launch_fill_zero(void *ptr, size_t bytes, void *stream_v)
-{
-    hipStream_t stream = (hipStream_t)stream_v;
-    const size_t words = bytes / 4;
-    if (words == 0) return GPTQ_HIP_OK;
-    const unsigned blocks = (unsigned)((words + 255) / 256);
-    hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, stream, (uint32_t *)ptr, words);
-    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+    return bits == 4 ? launch_gather_rt<4>(p, plan, (hipStream_t)stream)
+                     : launch_gather_rt<3>(p, plan, (hipStream_t)stream);
 }
 
 }  // namespace gptq

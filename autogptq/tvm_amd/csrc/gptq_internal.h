@@ -24,6 +24,7 @@ struct Params {
     int chunk_steps;   // steps staged in LDS at a time
     int xs_rows;       // rows of x kept in LDS per workgroup
     int row_tiles;     // 16-row tiles per wave
+    int gpad;          // GROUPED kernel: rows per activation row = groups rounded up to 16
 };
 
 // k handled by one wave step: 4 lane groups x (8 | 32) codes
@@ -32,7 +33,12 @@ inline int kstep_of(int bits) { return bits == 4 ? 32 : 128; }
 // byte size of the head of the workspace that holds the split-K counters
 static const size_t kCounterBytes = 16384;
 
-int launch_matmul(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
+// GROUPED kernel sizing, shared by the dispatcher and the plan check
+int grouped_tpm(int groups, int M);
+int grouped_groups(int kr, int gs, int G, int act_order);
+
+int launch_gather(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
+int launch_grouped(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
 int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
                    void *w, int K, int N, int G, int bits, int group_size, void *stream);
 int launch_fill_zero(void *ptr, size_t bytes, void *stream);

@@ -62,7 +62,7 @@ WORKLOADS = {
 DEFAULT_WORKLOAD = "c2-int3-4096x11008-act-m1"
 
 
-def build_case(name: str, dev):
+def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int = 0):
     from autogptq.tvm_amd import _lib
     from autogptq.tvm_amd.pack import synth_layer
 
@@ -84,7 +84,12 @@ def build_case(name: str, dev):
         "x": L["x"].to(dev), "y": torch.empty((M, N), dtype=torch.float16, device=dev),
         "wbytes": wbytes, "flops": 2 * M * K * N,
     }
-    plan = _lib.select(M, K, N, bits, gs, desc_act)
+    if kernel or split_k or waves_n:
+        if not kernel:
+            kernel = _lib.select(M, K, N, bits, gs, desc_act).kernel
+        plan = _lib.plan_for(kernel, M, K, N, bits, gs, desc_act, split_k, waves_n)
+    else:
+        plan = _lib.select(M, K, N, bits, gs, desc_act)
     case["plan"] = plan
     case["ws"] = torch.zeros(max(plan.workspace_bytes, 16), dtype=torch.uint8, device=dev)
     return case
@@ -228,6 +233,9 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument("--sweep", action="store_true", help="also time every workload in WORKLOADS")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernel", type=int, default=0, help="force a kernel family (1 gather, 2 grouped, 3 blocked)")
+    ap.add_argument("--split-k", type=int, default=0, help="force the split-K factor")
+    ap.add_argument("--waves-n", type=int, default=0, help="force the waves per workgroup along N")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures the QuantLinear kernels on ONE GPU; --gpus must be 1 "
@@ -239,7 +247,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    case = build_case(args.workload, dev)
+    case = build_case(args.workload, dev, args.kernel, args.split_k, args.waves_n)
     ok, max_err = check_case(case, dev)
     torch.cuda.synchronize(dev)
     t = time_case(case, dev, args.steps, args.warmup)

@@ -65,6 +65,15 @@ typedef struct gptq_hip_plan {
  */
 int gptq_hip_select(int M, int K, int N, int bits, int group_size, int act_order, gptq_hip_plan *plan);
 
+/*
+ * The plan of one kernel family with split_k and waves_n forced (0 = let the dispatcher
+ * choose); GPTQ_HIP_ERR_UNSUPPORTED when that family does not cover the problem.  For
+ * benchmarks and tests of single kernels; the reference's counterpart is editing the tile
+ * parameters of one handler-database entry (pycuda_warpper.py:77-127).
+ */
+int gptq_hip_plan_for(int kernel, int M, int K, int N, int bits, int group_size, int act_order, int split_k,
+                      int waves_n, gptq_hip_plan *plan);
+
 /* Bytes of workspace gptq_hip_gemm needs for this problem (0 if none). */
 size_t gptq_hip_workspace_bytes(int M, int K, int N, int bits, int group_size, int act_order);
 

@@ -51,3 +51,10 @@ def assert_close(got: torch.Tensor, want: torch.Tensor, what: str, rtol=RTOL, at
 
 def layer(seed, K, N, bits, gs, desc_act, M=1, bias=False):
     return synth_layer(seed, K, N, bits, gs, desc_act, M=M, bias=bias)
+
+
+def assert_tight(got: torch.Tensor, want: torch.Tensor, what: str):
+    """A bound much tighter than the contract's, so that an indexing slip cannot hide inside
+    the tolerance: one fp16 rounding of y (relative 2^-11) plus fp32 accumulation noise and, for
+    the kernels that apply scales per group, the reference's own weight-rounding noise."""
+    return assert_close(got, want, what + " (tight)", rtol=1.5e-3, atol=1.5e-3)

@@ -62,8 +62,11 @@ def test_select_plans_are_consistent(bits, M, KN, gs):
     for act in (False, True):
         p = _lib.select(M, K, N, bits, gs, act)
         assert p.kernel in (_lib.KERNEL_GATHER, _lib.KERNEL_GROUPED, _lib.KERNEL_BLOCKED)
-        assert p.row_tiles in (1, 2, 4, 8)
-        assert p.m_blocks * 16 * p.row_tiles >= M
+        if p.kernel == _lib.KERNEL_GROUPED:
+            assert M <= 2 and 1 <= p.row_tiles <= 6 and p.m_blocks == 1
+        else:
+            assert p.row_tiles in (1, 2, 4, 8)
+            assert p.m_blocks * 16 * p.row_tiles >= M
         assert p.block == 64 * p.waves_n * p.waves_k and p.block <= 1024
         assert p.grid_x * 64 * p.waves_n >= N
         kstep = 32 if bits == 4 else 128
@@ -126,3 +129,27 @@ def test_entry_points_reject_null_and_bad_sizes_before_touching_the_gpu():
     assert lib.gptq_hip_dequant(fake, fake, fake, null, fake, 64, 64, 5, 32, null) == _lib.ERR_BAD_ARG
     assert lib.gptq_hip_workspace_init(null, 64, null) == _lib.ERR_BAD_ARG
     assert lib.gptq_hip_workspace_init(null, 0, null) == _lib.OK
+
+
+def test_plan_for_forces_family_split_and_waves():
+    p = _lib.plan_for(_lib.KERNEL_GATHER, 1, 4096, 11008, 3, 128, True, split_k=5, waves_n=2)
+    assert p.kernel == _lib.KERNEL_GATHER and p.split_k == 5 and p.grid_y == 5 and p.waves_n == 2
+    assert p.grid_x == 11008 // 128 and p.block == 128
+    p = _lib.plan_for(_lib.KERNEL_GROUPED, 1, 4096, 11008, 3, 128, True, split_k=8)
+    assert p.kernel == _lib.KERNEL_GROUPED and p.split_k == 8 and p.row_tiles == 2
+    assert p.lds_bytes == (4096 // 8) * 2 * 32
+    # M = 3 is outside the GROUPED family; so are 128 groups under activation order
+    with pytest.raises(_lib.GptqHipError) as e:
+        _lib.plan_for(_lib.KERNEL_GROUPED, 3, 4096, 4096, 4, 128, True)
+    assert e.value.status == _lib.ERR_UNSUPPORTED
+    with pytest.raises(_lib.GptqHipError):
+        _lib.plan_for(_lib.KERNEL_GROUPED, 1, 4096, 4096, 4, 32, True)
+    with pytest.raises(_lib.GptqHipError) as e:
+        _lib.plan_for(_lib.KERNEL_GATHER, 1, 4096, 4096, 4, 128, True, waves_n=3)
+    assert e.value.status == _lib.ERR_BAD_ARG
+
+
+def test_single_group_ignores_act_order():
+    a = _lib.select(1, 9216, 9216, 3, -1, True).as_dict()
+    b = _lib.select(1, 9216, 9216, 3, -1, False).as_dict()
+    assert a == b
