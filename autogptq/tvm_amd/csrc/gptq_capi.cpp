@@ -14,6 +14,7 @@ int check_common(const int32_t *qweight, const int32_t *qzeros, const void *scal
     if (!qweight || !qzeros || !scales) return GPTQ_HIP_ERR_BAD_ARG;
     if (bits != 3 && bits != 4) return GPTQ_HIP_ERR_BAD_ARG;
     if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;
+    if ((long long)K * N * bits / 8 >= (1LL << 31)) return GPTQ_HIP_ERR_UNSUPPORTED;  // kernels use 32-bit byte offsets
     if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
     if (!aligned(qweight, 16) || !aligned(qzeros, 4) || !aligned(scales, 8)) return GPTQ_HIP_ERR_BAD_ARG;
     return GPTQ_HIP_OK;
@@ -24,13 +25,15 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
     const int kstep = gptq::kstep_of(bits);
     const int steps_total = (K + kstep - 1) / kstep;
     if (pl.waves_n != 1 && pl.waves_n != 2 && pl.waves_n != 4) return GPTQ_HIP_ERR_UNSUPPORTED;
-    if (pl.block != 64 * pl.waves_n) return GPTQ_HIP_ERR_BAD_ARG;
+    if (pl.waves_k < 1 || pl.waves_n * pl.waves_k > 8) return GPTQ_HIP_ERR_UNSUPPORTED;
+    if (pl.block != 64 * pl.waves_n * pl.waves_k) return GPTQ_HIP_ERR_BAD_ARG;
     if (pl.split_k < 1 || pl.split_k > steps_total) return GPTQ_HIP_ERR_BAD_ARG;
     if (pl.grid_x * 64 * pl.waves_n < N || pl.grid_y != pl.split_k) return GPTQ_HIP_ERR_BAD_ARG;
     if (pl.lds_bytes > 160 * 1024) return GPTQ_HIP_ERR_BAD_ARG;
     if (pl.split_k > 1 && (size_t)pl.grid_x * (pl.grid_z > 0 ? pl.grid_z : 1) * sizeof(int) > gptq::kCounterBytes)
         return GPTQ_HIP_ERR_UNSUPPORTED;
     if (pl.kernel == GPTQ_HIP_KERNEL_GATHER) {
+        if (pl.waves_k != 1) return GPTQ_HIP_ERR_UNSUPPORTED;
         if (pl.row_tiles != 1 && pl.row_tiles != 2 && pl.row_tiles != 4 && pl.row_tiles != 8)
             return GPTQ_HIP_ERR_UNSUPPORTED;
         if (pl.k_chunk < kstep || pl.k_chunk % kstep != 0) return GPTQ_HIP_ERR_BAD_ARG;
@@ -43,12 +46,14 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
     }
     if (pl.kernel == GPTQ_HIP_KERNEL_GROUPED) {
         if (M > 2 || pl.grid_z != 1 || pl.row_tiles % M != 0) return GPTQ_HIP_ERR_UNSUPPORTED;
-        const int steps = (steps_total + pl.split_k - 1) / pl.split_k;
-        const int kr = steps * kstep;
+        // k_chunk is the K range of one workgroup: waves_k * wave_steps whole steps
+        if (pl.k_chunk < kstep * pl.waves_k || pl.k_chunk % (kstep * pl.waves_k) != 0) return GPTQ_HIP_ERR_BAD_ARG;
+        const int kr = pl.k_chunk;
+        if ((long long)kr * pl.split_k < (long long)steps_total * kstep) return GPTQ_HIP_ERR_BAD_ARG;
         const int tpm = pl.row_tiles / M;
         const int need_tpm = gptq::grouped_tpm(gptq::grouped_groups(kr, gs, G, act_order), M);
         if (need_tpm == 0 || tpm != need_tpm) return GPTQ_HIP_ERR_UNSUPPORTED;
-        if (pl.lds_bytes < (long long)kr * pl.row_tiles * 32) return GPTQ_HIP_ERR_BAD_ARG;
+        if (pl.lds_bytes < gptq::grouped_lds_bytes(kr, M, tpm, pl.waves_n, pl.waves_k)) return GPTQ_HIP_ERR_BAD_ARG;
         return GPTQ_HIP_OK;
     }
     return GPTQ_HIP_ERR_UNSUPPORTED;
@@ -94,6 +99,9 @@ extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const i
     p.chunk_steps = plan->k_chunk / kstep;
     p.xs_rows = M < 16 * plan->row_tiles ? M : 16 * plan->row_tiles;
     p.row_tiles = plan->row_tiles;
+    p.waves_n = plan->waves_n;
+    p.waves_k = plan->waves_k;
+    p.wave_steps = plan->kernel == GPTQ_HIP_KERNEL_GROUPED ? plan->k_chunk / kstep / plan->waves_k : 0;
     p.gpad = plan->kernel == GPTQ_HIP_KERNEL_GROUPED ? 16 * (plan->row_tiles / M) : 0;
     if (plan->split_k > 1) {
         const size_t need = gptq::kCounterBytes + (size_t)plan->split_k * M * N * sizeof(float);

@@ -79,6 +79,16 @@ int grouped_groups(int kr, int gs, int G, int act_order)
     return groups > G ? G : groups;
 }
 
+// LDS of the GROUPED kernel for a K range of kr channels: operand tiles (+ slot masks in the
+// compact two-tile layout) + the reduction buffer of the waves along K.
+int grouped_lds_bytes(int kr, int M, int tpm, int waves_n, int waves_k)
+{
+    const int nblk8 = kr / 8;
+    const bool compact = tpm == 2;
+    const int stored = compact ? M : M * tpm;
+    return nblk8 * stored * 256 + (compact ? nblk8 * 16 : 0) + waves_k * waves_n * M * 64 * 4;
+}
+
 }  // namespace gptq
 
 namespace {
@@ -90,36 +100,42 @@ bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, i
 {
     const int kstep = gptq::kstep_of(bits);
     const int steps_total = ceil_div(K, kstep);
-    const int waves = force_waves > 0 ? force_waves : 4;
-    const int col_tiles = ceil_div(N, 64 * waves);
+    const int waves_n = force_waves > 0 ? force_waves : 1;
+    const int col_tiles = ceil_div(N, 64 * waves_n);
     if ((size_t)col_tiles * sizeof(int) > gptq::kCounterBytes) return false;
-    const int lds_cap = 64 * 1024;
-    int want = force_split > 0 ? force_split : ceil_div(kTargetWorkgroups, col_tiles);
+    const int lds_cap = 144 * 1024;
+    // a column tile per workgroup and no split is best (nothing crosses workgroups) unless
+    // that leaves most of the 256 CUs idle
+    int want = force_split > 0 ? force_split : (col_tiles >= 128 ? 1 : ceil_div(192, col_tiles));
     if (want > steps_total) want = steps_total;
-    if (want < 1) want = 1;
-    for (int split = want; split <= steps_total && split <= 256; split++) {
-        if (force_split > 0 && split != want) return false;
-        const int steps = ceil_div(steps_total, split);  // the longest K range, in steps
-        const int kr = steps * kstep;
+    for (int want_split = want; want_split <= steps_total && want_split <= 256; want_split++) {
+        if (force_split > 0 && want_split != want) return false;
+        // uniform partition: every wave gets wave_steps steps, every workgroup waves_k of those
+        int waves_k = 8 / waves_n;
+        if (waves_k * want_split > steps_total) waves_k = steps_total / want_split;
+        if (waves_k < 1) waves_k = 1;
+        const int wave_steps = ceil_div(steps_total, want_split * waves_k);
+        const int wg_steps = wave_steps * waves_k;
+        const int split = ceil_div(steps_total, wg_steps);
+        const int kr = wg_steps * kstep;
         const int tpm = gptq::grouped_tpm(gptq::grouped_groups(kr, gs, G, act_order), M);
         if (tpm == 0) {
             if (act_order) return false;  // the group count does not shrink with the K range
             continue;
         }
-        const int rt = M * tpm;
-        const int lds = kr * rt * 32;
+        const int lds = gptq::grouped_lds_bytes(kr, M, tpm, waves_n, waves_k);
         if (lds > lds_cap) continue;
         plan->kernel = GPTQ_HIP_KERNEL_GROUPED;
-        plan->row_tiles = rt;
+        plan->row_tiles = M * tpm;
         plan->m_blocks = 1;
-        plan->waves_n = waves;
-        plan->waves_k = 1;
+        plan->waves_n = waves_n;
+        plan->waves_k = waves_k;
         plan->split_k = split;
         plan->k_chunk = kr;
         plan->grid_x = col_tiles;
         plan->grid_y = split;
         plan->grid_z = 1;
-        plan->block = 64 * waves;
+        plan->block = 64 * waves_n * waves_k;
         plan->lds_bytes = lds;
         plan->workspace_bytes = split > 1 ? gptq::kCounterBytes + (size_t)split * M * N * sizeof(float) : 0;
         return true;

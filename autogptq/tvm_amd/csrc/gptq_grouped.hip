@@ -12,15 +12,30 @@
 // performs is not reproduced here (products are exact, sums are fp32), so y differs
 // from the reference by its rounding noise, far inside the 1e-2 tolerance.
 //
-// LDS holds the expanded activation operand of the workgroup's K range, laid out as
-// the MFMA wants it: tile (block b, sub-block nb, row tile rt) is 16 rows x 8 slots of
-// fp16 = 256 bytes, lane i reads its 16 bytes at i*16.  It is zero-filled and then
-// scattered into: one 2-byte store per (m, k).
+// Work split: a workgroup owns 64 * waves_n columns and one K range (all of K when
+// split_k == 1); its waves_k waves along K each take a share of that range, issue all
+// their weight loads up front, and meet in LDS for the reduction.  With split_k == 1
+// nothing crosses workgroups.
 //
-// grid = (column tiles, split_k), block = 64 * waves, every wave owns 64 columns.
+// LDS holds the expanded activation operand of the workgroup's K range, laid out as
+// the MFMA wants it: a tile is 16 rows x 8 slots of fp16 = 256 bytes, lane i reads its
+// 16 bytes at i*16.  It is zero-filled and then scattered into, one 2-byte store per
+// (m, k).  Two layouts:
+//   dense   : one tile per 16 groups (row = g - g_base), M * TPM tiles per 8 slots;
+//   compact : for 17..32 groups, ONE tile per m with row = g % 16, plus a 16-byte mask
+//             per 8 slots saying which slots belong to groups < 16.  The two row tiles
+//             are that tile AND mask / AND NOT mask: half the LDS, so K = 4096 with 32
+//             groups fits one workgroup.
 #include "gptq_device.h"
 
 namespace gptq {
+
+#ifdef GPTQ_PHASE_TIMES
+__device__ long long g_phase[16 * 8192];
+#define PHASE(i) do { if (lane == 0) g_phase[((size_t)blockIdx.x * 8 + wave) * 16 + (i)] = clock64(); } while (0)
+#else
+#define PHASE(i) do { } while (0)
+#endif
 
 // The four zero points (already +1) of columns n .. n+3 (n % 4 == 0) of one qzeros row.
 template <int BITS>
@@ -53,26 +68,43 @@ __device__ __forceinline__ void zeros_from_words(uint32_t wa, uint32_t wb, int n
     }
 }
 
-// RT = row tiles = M * TPM, TPM = tiles (of 16 groups) per activation row.
-template <int BITS, int M, int TPM, int NSTEP>
-__global__ __launch_bounds__(256) void grouped_kernel(const Params p)
+__device__ __forceinline__ h8 and_h8(h8 a, u4 m)
+{
+    u4 v = __builtin_bit_cast(u4, a);
+    v &= m;
+    return __builtin_bit_cast(h8, v);
+}
+
+// TPM = row tiles (of 16 groups) per activation row; COMPACT needs TPM == 2.
+template <int BITS, int M, int TPM, bool COMPACT, int NSTEP>
+__global__ __launch_bounds__(512) void grouped_kernel(const Params p)
 {
     using F = Fmt<BITS>;
-    constexpr int RT = M * TPM;
+    constexpr int ST = COMPACT ? M : M * TPM;    // tiles stored in LDS per 8 slots
+    static_assert(!COMPACT || TPM == 2, "compact layout is for two row tiles");
     const int tid = threadIdx.x;
+    const int nthreads = (int)blockDim.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+    const int WN = p.waves_n;
+    const int WK = p.waves_k;
+    const int wn = wave % WN;
+    const int wk = wave / WN;
     const int li = lane & 15;
     const int lq = lane >> 4;
-    const int BN = (int)blockDim.x;
-    const int n0 = blockIdx.x * BN + wave * 64 + 4 * li;
+    const int BN = 64 * WN;
+    const int n0 = blockIdx.x * BN + wn * 64 + 4 * li;
     const bool n_ok = n0 < p.N;
     const int split = blockIdx.y;
-    const int s_begin = (int)((long long)p.steps_total * split / p.split_k);
-    const int s_end = (int)((long long)p.steps_total * (split + 1) / p.split_k);
-    const int nsteps = s_end - s_begin;
+    // every wave owns wave_steps consecutive steps (the host made the partition uniform, so no
+    // division happens here); ranges past the end of K are cut by s_end
+    const int wg_steps = p.wave_steps * WK;
+    const int s_begin = split * wg_steps;
+    const int s_end = min(s_begin + wg_steps, p.steps_total);
+    const int ws = s_begin + wk * p.wave_steps;  // this wave's steps
+    const int we = min(ws + p.wave_steps, s_end);
     const int k_base = s_begin * F::KSTEP;
-    const int kspan = nsteps * F::KSTEP;
+    const int kspan = wg_steps * F::KSTEP;
     const int prows = p.K / (BITS == 4 ? 8 : 32);  // packed rows (int4) or 3-word blocks (int3)
     // contiguous groups: only those inside this K range need rows, counted from the first one
     const int g_base = p.g_idx ? 0 : k_base / p.group_size;
@@ -82,140 +114,267 @@ __global__ __launch_bounds__(256) void grouped_kernel(const Params p)
     const _Float16 *scales = (const _Float16 *)p.scales;
     const int zwords = p.N / 32 * BITS;
 
-    // ---- 1. first batch of weight loads goes out before anything else -----------------
+    const int nblk8 = kspan / 8;  // 8-slot blocks in the K range
+    unsigned char *tiles = smem;
+    unsigned char *masks = smem + (size_t)nblk8 * ST * 256;
+    float *red = (float *)(masks + (COMPACT ? (size_t)nblk8 * 16 : 0));
+
+    PHASE(0);
+    int qslot[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) qslot[e] = slot_of_code<BITS>((4 * tid) % F::KLANE + e);
+    // ---- 1. x and g_idx of the K range: four channels per thread per pass ---------------
+    constexpr int QP = 2;  // passes kept in registers so that their loads are the first to return
+    const int qpr = kspan / 4;  // quads per activation row
+    const int nquads = qpr * M;
+    int gq[QP][4];
+    h4 xq[QP];
+#pragma unroll
+    for (int ps = 0; ps < QP; ps++) {
+        const int idx = tid + ps * nthreads;
+        xq[ps] = (h4){0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < 4; e++) gq[ps][e] = 0;
+        if (idx < nquads) {
+            const int m = M == 1 ? 0 : idx / qpr;
+            const int k = k_base + 4 * (idx - m * qpr);
+            if (k < p.K) {  // K % 4 == 0: a quad is inside or outside as a whole
+                xq[ps] = *(const h4 *)(x + (size_t)m * p.K + k);
+                if (p.g_idx) {
+                    const int4 gv = *(const int4 *)(p.g_idx + k);
+                    gq[ps][0] = gv.x;
+                    gq[ps][1] = gv.y;
+                    gq[ps][2] = gv.z;
+                    gq[ps][3] = gv.w;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) gq[ps][e] = (k + e) / p.group_size;
+                }
+            }
+        }
+    }
+
+    // ---- 2. zero the expanded activation operand in LDS while those loads fly ---------
+    {
+        u4 *z = (u4 *)tiles;
+        const int n16 = nblk8 * ST * 16;
+        for (int i = tid; i < n16; i += nthreads) z[i] = (u4){0u, 0u, 0u, 0u};
+    }
+    // ---- 3. weight loads, software-pipelined: a wave blocks while it issues loads into a full
+    //         memory pipeline, so only the first PF steps go out now (they cover the LDS work
+    //         below); step s + PF is issued right before step s is consumed ---------------
+    constexpr int PF = BITS == 4 ? 6 : 2;
     u4 w[NSTEP][F::WORDS];
-    auto load_batch = [&](int st0) {
+    auto load_step = [&](int s, int st) {  // register slot s <- step st
+        const int prow = 4 * st + lq;
+        const bool ok = n_ok && st < we && prow < prows;
 #pragma unroll
-        for (int s = 0; s < NSTEP; s++) {
-            const int prow = 4 * (st0 + s) + lq;
-            const bool ok = n_ok && (st0 + s) < s_end && prow < prows;
+        for (int wd = 0; wd < F::WORDS; wd++) {
+            w[s][wd] = (u4){0u, 0u, 0u, 0u};
+            if (ok) {
+                // 32-bit byte offset from a uniform base: one VALU op per load instead of 64-bit math
+                const uint32_t off = ((uint32_t)(prow * F::WORDS + wd) * (uint32_t)p.N + (uint32_t)n0) * 4u;
+                w[s][wd] = __builtin_nontemporal_load((const u4 *)((const char *)p.qweight + off));
+            }
+        }
+    };
 #pragma unroll
-            for (int wd = 0; wd < F::WORDS; wd++) {
-                w[s][wd] = (u4){0u, 0u, 0u, 0u};
-                if (ok) {
-                    w[s][wd] = __builtin_nontemporal_load(
-                        (const u4 *)(p.qweight + (size_t)(prow * F::WORDS + wd) * p.N + n0));
+    for (int s = 0; s < PF && s < NSTEP; s++) load_step(s, ws + s);
+    __builtin_amdgcn_sched_barrier(0);
+    PHASE(1);
+
+    // ---- 4. scales / zero words this lane needs in the epilogue (rows g = 16 t + 4 q + v);
+    //         loaded once the last weight loads are out ---------------------------------
+    h4 sc[TPM][4];
+    uint32_t zwa[TPM][4], zwb[TPM][4];
+    auto load_epilogue_operands = [&]() {
+#pragma unroll
+        for (int t = 0; t < TPM; t++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int g = g_base + 16 * t + 4 * lq + v;
+                sc[t][v] = (h4){0, 0, 0, 0};
+                zwa[t][v] = 0u;
+                zwb[t][v] = 0u;
+                if (n_ok && g < p.G) {
+                    const uint32_t soff = ((uint32_t)g * (uint32_t)p.N + (uint32_t)n0) * 2u;
+                    sc[t][v] = *(const h4 *)((const char *)scales + soff);
+                    load_zero_words<BITS>(p.qzeros + (uint32_t)g * (uint32_t)zwords, n0, zwa[t][v], zwb[t][v]);
                 }
             }
         }
     };
-    load_batch(s_begin);
 
-    // ---- 2. scales / zero words this lane needs in the epilogue: rows g = 16 t + 4 q + v -
-    h4 sc[TPM][4];
-    uint32_t zwa[TPM][4], zwb[TPM][4];
+    __syncthreads();
+    PHASE(2);
+    // ---- 5. scatter x into the operand tiles (waits for x / g_idx only) -------------------
+    // A thread always owns quads with the same position inside a lane block (kc % KLANE is
+    // 4 * (tid % (KLANE / 4)) in every pass because the block size is a multiple of 8), so the
+    // four slots of its quad are fixed: qslot[e], looked up once at the top of the kernel.
+    auto scatter = [&](int m, int kc, int slot, int g, _Float16 xv) {
+        const int r = min(max(g, 0), p.G - 1) - g_base;  // row of this group
+        const int rr = min(max(r, 0), 16 * TPM - 1);
+        const int b8 = (kc / F::KLANE) * F::NB + (slot >> 3);
+        if constexpr (COMPACT) {
+            ((_Float16 *)tiles)[((b8 * ST + m) * 16 + (rr & 15)) * 8 + (slot & 7)] = xv;
+            if (m == 0) ((unsigned short *)masks)[b8 * 8 + (slot & 7)] = rr < 16 ? 0xffffu : 0u;
+        } else {
+            ((_Float16 *)tiles)[((b8 * ST + m * TPM + (rr >> 4)) * 16 + (rr & 15)) * 8 + (slot & 7)] = xv;
+        }
+    };
 #pragma unroll
-    for (int t = 0; t < TPM; t++) {
+    for (int ps = 0; ps < QP; ps++) {
+        const int idx = tid + ps * nthreads;
+        if (idx < nquads) {
+            const int m = M == 1 ? 0 : idx / qpr;
+            const int kc = 4 * (idx - m * qpr);
+            if (k_base + kc < p.K) {
 #pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const int g = g_base + 16 * t + 4 * lq + v;
-            sc[t][v] = (h4){0, 0, 0, 0};
-            zwa[t][v] = 0u;
-            zwb[t][v] = 0u;
-            if (n_ok && g < p.G) {
-                sc[t][v] = *(const h4 *)(scales + (size_t)g * p.N + n0);
-                load_zero_words<BITS>(p.qzeros + (size_t)g * zwords, n0, zwa[t][v], zwb[t][v]);
+                for (int e = 0; e < 4; e++) scatter(m, kc + e, qslot[e], gq[ps][e], xq[ps][e]);
             }
         }
     }
-
-    // ---- 3. expanded activation operand in LDS -----------------------------------------
-    const int nblk8 = kspan / 8;  // 8-slot blocks in the K range
-    {
-        u4 *z = (u4 *)smem;
-        const int n16 = nblk8 * RT * 16;
-        for (int i = tid; i < n16; i += (int)blockDim.x) z[i] = (u4){0u, 0u, 0u, 0u};
-    }
-    __syncthreads();
-    for (int idx = tid; idx < kspan * M; idx += (int)blockDim.x) {
-        const int m = idx / kspan;
-        const int kc = idx - m * kspan;
+    for (int idx = tid + QP * nthreads; idx < nquads; idx += nthreads) {  // long K ranges
+        const int m = M == 1 ? 0 : idx / qpr;
+        const int kc = 4 * (idx - m * qpr);
         const int k = k_base + kc;
         if (k < p.K) {
-            int g = p.g_idx ? p.g_idx[k] : k / p.group_size;
-            g = min(max(g, 0), p.G - 1);
-            const _Float16 xv = x[(size_t)m * p.K + k];
-            const int r = m * (16 * TPM) + min(g - g_base, 16 * TPM - 1);
-            const int b = kc / F::KLANE;
-            const int slot = slot_of_code<BITS>(kc % F::KLANE);
-            const int tile = ((b * F::NB + (slot >> 3)) * RT + (r >> 4));
-            ((_Float16 *)smem)[(tile * 16 + (r & 15)) * 8 + (slot & 7)] = xv;
+            const h4 xv = *(const h4 *)(x + (size_t)m * p.K + k);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int g = p.g_idx ? p.g_idx[k + e] : (k + e) / p.group_size;
+                scatter(m, kc + e, qslot[e], g, xv[e]);
+            }
         }
     }
     __syncthreads();
+    PHASE(3);
+    load_epilogue_operands();
 
-    // ---- 4. main loop -----------------------------------------------------------------
-    f4 acc[RT][4];
-    f4 accx[RT];
+    // ---- 6. main loop -----------------------------------------------------------------
+    // acc[m][t][c] collects sum x * (base + code); accx[m][t] is the same operand against the
+    // constant columns "all ones" (column 0 -> X) and "the slot bases" (column 1 -> the base
+    // part to subtract).  In the compact layout t = 0 is the masked tile (groups < 16) and
+    // t = 1 the unmasked one (all groups): groups >= 16 are their difference.
+    f4 acc[M][TPM][4];
+    f4 accx[M][TPM];
 #pragma unroll
-    for (int rt = 0; rt < RT; rt++) {
-        accx[rt] = (f4){0.f, 0.f, 0.f, 0.f};
+    for (int m = 0; m < M; m++)
 #pragma unroll
-        for (int c = 0; c < 4; c++) acc[rt][c] = (f4){0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < TPM; t++) {
+            accx[m][t] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc[m][t][c] = (f4){0.f, 0.f, 0.f, 0.f};
+        }
+    h8 cb;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const float base = BITS == 4 ? BASE4[e] : BASE3[e];
+        cb[e] = (_Float16)(li == 0 ? 1.0f : (li == 1 ? base : 0.0f));
     }
-    const h8 ones = {1, 1, 1, 1, 1, 1, 1, 1};
+    const uint32_t magic_a = opaque_vgpr(BITS == 4 ? MAGIC4_LO : MAGIC3_EVEN);
+    const uint32_t magic_b = opaque_vgpr(BITS == 4 ? MAGIC4_HI : MAGIC3_ODD);
 
-    for (int st0 = s_begin; st0 < s_end; st0 += NSTEP) {
-        if (st0 != s_begin) load_batch(st0);
+    for (int st0 = ws; st0 < we; st0 += NSTEP) {
+        if (st0 != ws) {
+#pragma unroll
+            for (int s = 0; s < PF && s < NSTEP; s++) load_step(s, st0 + s);
+        }
 #pragma unroll
         for (int s = 0; s < NSTEP; s++) {
-            if (st0 + s < s_end) {
+            if (s + PF < NSTEP) {
+                if (st0 + s + PF < we) load_step(s + PF, st0 + s + PF);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (st0 + s < we) {
                 const int b = (st0 + s - s_begin) * 4 + lq;
-                uint32_t mg[4][4 * F::NB];
+                uint32_t bq[4][4 * F::NB];
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
                     if constexpr (BITS == 4) {
-                        magic4(w[s][0][c], mg[c]);
+                        biased4(w[s][0][c], bq[c], magic_a, magic_b);
                     } else {
-                        magic3(w[s][0][c], w[s][1][c], w[s][2][c], mg[c]);
+                        biased3(w[s][0][c], w[s][1][c], w[s][2][c], bq[c], magic_a, magic_b);
                     }
                 }
 #pragma unroll
                 for (int nb = 0; nb < F::NB; nb++) {
-                    h8 bop[4];
+                    const int b8 = b * F::NB + nb;
+                    h8 a[M][TPM];
+                    if constexpr (COMPACT) {
+                        const u4 mk = *(const u4 *)(masks + (size_t)b8 * 16);
+#pragma unroll
+                        for (int m = 0; m < M; m++) {
+                            a[m][1] = *(const h8 *)(tiles + ((size_t)(b8 * ST + m) * 16 + li) * 16);
+                            a[m][0] = and_h8(a[m][1], mk);
+                        }
+                    } else {
+#pragma unroll
+                        for (int m = 0; m < M; m++)
+#pragma unroll
+                            for (int t = 0; t < TPM; t++) {
+                                a[m][t] = *(const h8 *)(tiles + ((size_t)(b8 * ST + m * TPM + t) * 16 + li) * 16);
+                            }
+                    }
 #pragma unroll
                     for (int c = 0; c < 4; c++) {
+                        const u4 bw = {bq[c][nb * 4 + 0], bq[c][nb * 4 + 1], bq[c][nb * 4 + 2], bq[c][nb * 4 + 3]};
+                        const h8 bop = __builtin_bit_cast(h8, bw);
 #pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            const h2 q2 = BITS == 4 ? code_from_magic4(mg[c][nb * 4 + r], nb * 4 + r)
-                                                    : code_from_magic3(mg[c][nb * 4 + r], nb * 4 + r);
-                            bop[c][2 * r] = q2.x;
-                            bop[c][2 * r + 1] = q2.y;
-                        }
+                        for (int m = 0; m < M; m++)
+#pragma unroll
+                            for (int t = 0; t < TPM; t++) {
+                                acc[m][t][c] =
+                                    __builtin_amdgcn_mfma_f32_16x16x32_f16(a[m][t], bop, acc[m][t][c], 0, 0, 0);
+                            }
                     }
 #pragma unroll
-                    for (int rt = 0; rt < RT; rt++) {
-                        const h8 a = *(const h8 *)(smem + ((size_t)((b * F::NB + nb) * RT + rt) * 16 + li) * 16);
+                    for (int m = 0; m < M; m++)
 #pragma unroll
-                        for (int c = 0; c < 4; c++) {
-                            acc[rt][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bop[c], acc[rt][c], 0, 0, 0);
+                        for (int t = 0; t < TPM; t++) {
+                            accx[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[m][t], cb, accx[m][t], 0, 0, 0);
                         }
-                        accx[rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, ones, accx[rt], 0, 0, 0);
-                    }
                 }
             }
         }
     }
 
-    // ---- 5. epilogue: scales and zero points once per group, then sum over groups -------
-    // acc[m*TPM + t][c][v] = P[m][g = g_base + 16 t + 4 q + v][n0 + c];  accx[m*TPM + t][v] = X[m][g]
+    PHASE(4);
+    // ---- 7. scales and zero points once per group, then sum over groups ------------------
+    // row v of tile t in lane group q is group g_base + 16 t + 4 q + v
     float tot[M][4];
 #pragma unroll
     for (int m = 0; m < M; m++)
 #pragma unroll
         for (int c = 0; c < 4; c++) tot[m][c] = 0.f;
 #pragma unroll
-    for (int t = 0; t < TPM; t++) {
+    for (int m = 0; m < M; m++) {
+        float xs_prev[4] = {0.f, 0.f, 0.f, 0.f}, bs_prev[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int v = 0; v < 4; v++) {
-            float z[4];
-            zeros_from_words<BITS>(zwa[t][v], zwb[t][v], n0, z);
+        for (int t = 0; t < TPM; t++) {
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const float s = (float)sc[t][v][c];
+            for (int v = 0; v < 4; v++) {
+                float xsum = __shfl(accx[m][t][v], lane & 48);        // column 0: sum of x
+                float bsum = __shfl(accx[m][t][v], (lane & 48) | 1);  // column 1: sum of x * base
+                float pv[4];
 #pragma unroll
-                for (int m = 0; m < M; m++) {
-                    tot[m][c] += s * (acc[m * TPM + t][c][v] - z[c] * accx[m * TPM + t][v]);
+                for (int c = 0; c < 4; c++) pv[c] = acc[m][t][c][v];
+                if constexpr (COMPACT) {
+                    if (t == 0) {
+                        xs_prev[v] = xsum;
+                        bs_prev[v] = bsum;
+                    } else {
+                        xsum -= xs_prev[v];
+                        bsum -= bs_prev[v];
+#pragma unroll
+                        for (int c = 0; c < 4; c++) pv[c] -= acc[m][0][c][v];
+                    }
+                }
+                float z[4];
+                zeros_from_words<BITS>(zwa[t][v], zwb[t][v], n0, z);
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    tot[m][c] += (float)sc[t][v][c] * ((pv[c] - bsum) - z[c] * xsum);
                 }
             }
         }
@@ -229,54 +388,62 @@ __global__ __launch_bounds__(256) void grouped_kernel(const Params p)
         }
     }
 
+    PHASE(5);
+    // ---- 8. waves along K meet in LDS; one thread per four output columns finishes --------
+    if (lq == 0) {
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            *(f4 *)(red + (((size_t)wk * WN + wn) * M + m) * 64 + 4 * li) =
+                (f4){tot[m][0], tot[m][1], tot[m][2], tot[m][3]};
+        }
+    }
+    __syncthreads();
+    PHASE(6);
+    const bool fin = tid < WN * M * 16;
+    const int f_wn = tid / (M * 16);
+    const int f_m = (tid >> 4) % M;
+    const int f_n = blockIdx.x * BN + f_wn * 64 + 4 * (tid & 15);
+    const bool writer = fin && f_n < p.N;
+    f4 sum = {0.f, 0.f, 0.f, 0.f};
+    if (writer) {
+        for (int k = 0; k < WK; k++) {
+            sum += *(const f4 *)(red + (((size_t)k * WN + f_wn) * M + f_m) * 64 + 4 * (tid & 15));
+        }
+    }
     const _Float16 *bias = (const _Float16 *)p.bias;
     f4 bv = {0.f, 0.f, 0.f, 0.f};
-    if (bias && n_ok) {
-        const h4 b4 = *(const h4 *)(bias + n0);
+    if (bias && writer) {
+        const h4 b4 = *(const h4 *)(bias + f_n);
         bv = (f4){(float)b4[0], (float)b4[1], (float)b4[2], (float)b4[3]};
     }
     _Float16 *y = (_Float16 *)p.y;
-    const bool writer = n_ok && lq == 0;
     if (p.split_k == 1) {
         if (writer) {
-#pragma unroll
-            for (int m = 0; m < M; m++) {
-                h4 o;
-#pragma unroll
-                for (int c = 0; c < 4; c++) o[c] = (_Float16)(tot[m][c] + bv[c]);
-                *(h4 *)(y + (size_t)m * p.N + n0) = o;
-            }
-        }
-        return;
-    }
-    if (writer) {
-#pragma unroll
-        for (int m = 0; m < M; m++) {
-            const f4 o = {tot[m][0], tot[m][1], tot[m][2], tot[m][3]};
-            store_partial(p.partial + ((size_t)split * M + m) * p.N + n0, o);
-        }
-    }
-    if (!arrive_last(p.counters + blockIdx.x, p.split_k, &last_flag)) return;
-    if (writer) {
-#pragma unroll
-        for (int m = 0; m < M; m++) {
-            f4 sum = bv;
-            for (int s = 0; s < p.split_k; s++) {
-                sum += load_partial(p.partial + ((size_t)s * M + m) * p.N + n0);
-            }
             h4 o;
 #pragma unroll
-            for (int c = 0; c < 4; c++) o[c] = (_Float16)sum[c];
-            *(h4 *)(y + (size_t)m * p.N + n0) = o;
+            for (int c = 0; c < 4; c++) o[c] = (_Float16)(sum[c] + bv[c]);
+            *(h4 *)(y + (size_t)f_m * p.N + f_n) = o;
         }
+        PHASE(7);
+        return;
+    }
+    if (writer) store_partial(p.partial + ((size_t)split * M + f_m) * p.N + f_n, sum);
+    if (!arrive_last(p.counters + blockIdx.x, p.split_k, &last_flag)) return;
+    if (writer) {
+        f4 total = bv;
+        for (int s = 0; s < p.split_k; s++) total += load_partial(p.partial + ((size_t)s * M + f_m) * p.N + f_n);
+        h4 o;
+#pragma unroll
+        for (int c = 0; c < 4; c++) o[c] = (_Float16)total[c];
+        *(h4 *)(y + (size_t)f_m * p.N + f_n) = o;
     }
 }
 
-template <int BITS, int M, int TPM>
+template <int BITS, int M, int TPM, bool COMPACT>
 static int launch_grouped_one(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
-    constexpr int NSTEP = BITS == 4 ? 8 : 4;
-    auto kern = grouped_kernel<BITS, M, TPM, NSTEP>;
+    constexpr int NSTEP = BITS == 4 ? 16 : 4;
+    auto kern = grouped_kernel<BITS, M, TPM, COMPACT, NSTEP>;
     if (plan.lds_bytes > 65536) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, plan.lds_bytes) !=
             hipSuccess) {
@@ -294,23 +461,30 @@ static int launch_grouped_bits(const Params &p, const gptq_hip_plan &plan, hipSt
     const int tpm = p.gpad / 16;
     if (p.M == 1) {
         switch (tpm) {
-            case 1: return launch_grouped_one<BITS, 1, 1>(p, plan, stream);
-            case 2: return launch_grouped_one<BITS, 1, 2>(p, plan, stream);
-            case 3: return launch_grouped_one<BITS, 1, 3>(p, plan, stream);
-            case 4: return launch_grouped_one<BITS, 1, 4>(p, plan, stream);
-            case 6: return launch_grouped_one<BITS, 1, 6>(p, plan, stream);
+            case 1: return launch_grouped_one<BITS, 1, 1, false>(p, plan, stream);
+            case 2: return launch_grouped_one<BITS, 1, 2, true>(p, plan, stream);
+            case 3: return launch_grouped_one<BITS, 1, 3, false>(p, plan, stream);
+            case 4: return launch_grouped_one<BITS, 1, 4, false>(p, plan, stream);
+            case 6: return launch_grouped_one<BITS, 1, 6, false>(p, plan, stream);
             default: return GPTQ_HIP_ERR_UNSUPPORTED;
         }
     }
     if (p.M == 2) {
         switch (tpm) {
-            case 1: return launch_grouped_one<BITS, 2, 1>(p, plan, stream);
-            case 2: return launch_grouped_one<BITS, 2, 2>(p, plan, stream);
+            case 1: return launch_grouped_one<BITS, 2, 1, false>(p, plan, stream);
+            case 2: return launch_grouped_one<BITS, 2, 2, true>(p, plan, stream);
             default: return GPTQ_HIP_ERR_UNSUPPORTED;
         }
     }
     return GPTQ_HIP_ERR_UNSUPPORTED;
 }
+
+#ifdef GPTQ_PHASE_TIMES
+extern "C" int gptq_hip_debug_read(void *host, size_t bytes)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_phase), bytes, 0, hipMemcpyDeviceToHost);
+}
+#endif
 
 int launch_grouped(const Params &p, int bits, const gptq_hip_plan &plan, void *stream)
 {

@@ -25,6 +25,9 @@ struct Params {
     int xs_rows;       // rows of x kept in LDS per workgroup
     int row_tiles;     // 16-row tiles per wave
     int gpad;          // GROUPED kernel: rows per activation row = groups rounded up to 16
+    int waves_n;       // waves of the workgroup along N
+    int waves_k;       // waves of the workgroup along K
+    int wave_steps;    // GROUPED kernel: steps per wave (uniform partition of K)
 };
 
 // k handled by one wave step: 4 lane groups x (8 | 32) codes
@@ -36,6 +39,7 @@ static const size_t kCounterBytes = 16384;
 // GROUPED kernel sizing, shared by the dispatcher and the plan check
 int grouped_tpm(int groups, int M);
 int grouped_groups(int kr, int gs, int G, int act_order);
+int grouped_lds_bytes(int kr, int M, int tpm, int waves_n, int waves_k);
 
 int launch_gather(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
 int launch_grouped(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);

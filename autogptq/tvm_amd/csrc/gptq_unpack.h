@@ -121,6 +121,66 @@ GPTQ_HD h2 code_from_magic3(uint32_t m, int r)
     return v * (h2){(_Float16)0.125f, (_Float16)0.03125f} - (h2){(_Float16)128.0f, (_Float16)32.0f};
 }
 
+
+// ---- "biased" unpack: every code with unit weight, no arithmetic after the OR -----------
+// Choosing the fp16 exponent per half so that the code's lowest bit has weight one makes the
+// register read (base + code) directly: a code at mantissa bit p wants exponent 2^(10 - p),
+// i.e. base = 1024 >> p.  The bases differ per slot but not per weight, so a product against
+// x picks up sum_k x[k] * base(slot(k)), which one extra MFMA against the constant vector
+// BASE4 / BASE3 measures and the epilogue subtracts.
+//
+// v_and_or_b32 takes one scalar constant at most, so the magic constant must sit in a vector
+// register for the compiler to fuse the AND and the OR: opaque_vgpr() hides its value.
+GPTQ_HD uint32_t opaque_vgpr(uint32_t v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("" : "+v"(v));
+#endif
+    return v;
+}
+
+GPTQ_HD uint32_t and_or(uint32_t x, uint32_t mask, uint32_t magic) { return (x & mask) | magic; }
+
+// int4: register r, half h holds BASE4[2r + h] + code SLOT4[2r + h]
+static constexpr float BASE4[8] = {1024.f, 1024.f, 64.f, 64.f, 1024.f, 1024.f, 64.f, 64.f};
+
+GPTQ_HD void biased4(uint32_t w, uint32_t out[4], uint32_t magic_lo, uint32_t magic_hi)
+{
+    const uint32_t w8 = w >> 8;
+    out[0] = and_or(w, 0x000f000fu, magic_lo);   // 0x64006400: 1024 + code
+    out[1] = and_or(w, 0x00f000f0u, magic_hi);   // 0x54005400: 64 + code
+    out[2] = and_or(w8, 0x000f000fu, magic_lo);
+    out[3] = and_or(w8, 0x00f000f0u, magic_hi);
+}
+static constexpr uint32_t MAGIC4_LO = 0x64006400u;
+static constexpr uint32_t MAGIC4_HI = 0x54005400u;
+
+// int3: register r, half h holds BASE3[2r + h] + code SLOT3[2r + h]; even registers carry
+// (p = 0, p = 2) -> bases (1024, 256); odd registers (p = 3, p = 5) -> bases (128, 32).
+static constexpr float BASE3[8] = {1024.f, 256.f, 128.f, 32.f, 1024.f, 256.f, 128.f, 32.f};
+static constexpr uint32_t MAGIC3_EVEN = 0x5c006400u;
+static constexpr uint32_t MAGIC3_ODD = 0x50005800u;
+
+GPTQ_HD void biased3(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t out[16], uint32_t magic_even,
+                     uint32_t magic_odd)
+{
+    uint32_t win[8];
+    win[0] = w0;
+    win[1] = w0 >> 6;
+    win[2] = funnel(w1, w0, 12);
+    win[3] = funnel(w2, w1, 4);
+    win[4] = funnel(w2, w1, 10);
+    win[5] = funnel(w2, w1, 16);
+    win[6] = w2 >> 8;
+    const uint32_t t = w2 >> 14;
+    win[7] = (t << 12) | t;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        out[2 * i] = and_or(win[i], 0x001c0007u, magic_even);
+        out[2 * i + 1] = and_or(win[i], 0x00e00038u, magic_odd);
+    }
+}
+
 // The dequantised weight of the reference (qlinear.py:242): fp16 scale times the
 // integer (q - zero), rounded once.  (q - zero) is exact in fp16, so one fp16 multiply
 // is that rounding, signed zeros and subnormals included.  (Going through an fp32

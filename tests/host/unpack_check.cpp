@@ -51,6 +51,32 @@ int main()
                 checked++;
             }
         }
+        // biased unpack: register value minus its slot's base is the code
+        uint32_t b4[4];
+        biased4(w0, b4, MAGIC4_LO, MAGIC4_HI);
+        for (int r = 0; r < 4; r++) {
+            const h2 v = as_h2(b4[r]);
+            for (int h = 0; h < 2; h++) {
+                if ((float)v[h] - BASE4[2 * r + h] != (float)code4(w0, SLOT4[2 * r + h])) {
+                    printf("biased4 mismatch w=%08x reg %d half %d got %f\n", w0, r, h, (float)v[h]);
+                    return 1;
+                }
+                checked++;
+            }
+        }
+        uint32_t b3[16];
+        biased3(w0, w1, w2, b3, MAGIC3_EVEN, MAGIC3_ODD);
+        for (int r = 0; r < 16; r++) {
+            const h2 v = as_h2(b3[r]);
+            for (int h = 0; h < 2; h++) {
+                if ((float)v[h] - BASE3[(2 * r + h) & 7] != (float)code3(w0, w1, w2, SLOT3[2 * r + h])) {
+                    printf("biased3 mismatch w=%08x %08x %08x reg %d half %d got %f\n", w0, w1, w2, r, h,
+                           (float)v[h]);
+                    return 1;
+                }
+                checked++;
+            }
+        }
         // code3 itself against the reference's straddle formulas (qlinear.py:233-234)
         const int c10 = (int)(((w0 >> 30) & 0x3u) | ((w1 << 2) & 0x4u));
         const int c21 = (int)(((w1 >> 31) & 0x1u) | ((w2 << 1) & 0x6u));

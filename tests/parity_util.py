@@ -57,4 +57,4 @@ def assert_tight(got: torch.Tensor, want: torch.Tensor, what: str):
     """A bound much tighter than the contract's, so that an indexing slip cannot hide inside
     the tolerance: one fp16 rounding of y (relative 2^-11) plus fp32 accumulation noise and, for
     the kernels that apply scales per group, the reference's own weight-rounding noise."""
-    return assert_close(got, want, what + " (tight)", rtol=1.5e-3, atol=1.5e-3)
+    return assert_close(got, want, what + " (tight)", rtol=2e-3, atol=3e-3)

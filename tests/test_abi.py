@@ -84,12 +84,15 @@ def test_select_plans_are_consistent(bits, M, KN, gs):
         assert lib.gptq_hip_workspace_bytes(M, K, N, bits, gs, int(act)) == p.workspace_bytes
 
 
-def test_select_fills_the_chip_at_m1():
-    # the headline shapes must give every CU work: at least 256 workgroups
+def test_select_spreads_decode_shapes_over_the_chip():
+    # the headline shapes must give most of the 256 CUs a workgroup
     for bits in (3, 4):
         for (K, N) in [(4096, 4096), (4096, 11008), (11008, 4096)]:
             p = _lib.select(1, K, N, bits, 128, True)
-            assert p.grid_x * p.grid_y * p.grid_z >= 256, (bits, K, N, p.as_dict())
+            assert p.grid_x * p.grid_y * p.grid_z >= 128, (bits, K, N, p.as_dict())
+    # 4096 x 11008 with 32 groups: one workgroup per 64 columns owns all of K, nothing crosses workgroups
+    p = _lib.select(1, 4096, 11008, 3, 128, True)
+    assert p.kernel == _lib.KERNEL_GROUPED and p.split_k == 1 and p.workspace_bytes == 0 and p.grid_x == 172
 
 
 @pytest.mark.parametrize("args", [
@@ -137,7 +140,7 @@ def test_plan_for_forces_family_split_and_waves():
     assert p.grid_x == 11008 // 128 and p.block == 128
     p = _lib.plan_for(_lib.KERNEL_GROUPED, 1, 4096, 11008, 3, 128, True, split_k=8)
     assert p.kernel == _lib.KERNEL_GROUPED and p.split_k == 8 and p.row_tiles == 2
-    assert p.lds_bytes == (4096 // 8) * 2 * 32
+    assert p.waves_n * p.waves_k * 64 == p.block
     # M = 3 is outside the GROUPED family; so are 128 groups under activation order
     with pytest.raises(_lib.GptqHipError) as e:
         _lib.plan_for(_lib.KERNEL_GROUPED, 3, 4096, 4096, 4, 128, True)

@@ -223,11 +223,14 @@ def test_gemm_full_size(dev, name, bits, K, N, gs, desc_act, Ms):
 def test_gemm_linearity_at_full_size(dev):
     # size-independent property: f(a + b) = f(a) + f(b) up to rounding, f(2x) = 2 f(x) exactly
     L = layer(900, 4096, 11008, 3, 128, True, M=2)
+    # keep fp16 subnormals out of x: doubling must stay exact on every path, matrix cores included
+    L["x"] = torch.where(L["x"].abs() < 1e-3, torch.zeros_like(L["x"]), L["x"])
     D = to_dev(L, dev)
     x = D["x"]
     y = run_gemm(D)
     y2 = run_gemm(D, x=(x * 2).contiguous())
-    assert torch.equal(y2.float(), y.float() * 2)  # scaling by 2 is exact in fp16 and fp32
+    normal = y.float().abs() >= 2.0 ** -13  # an fp16-subnormal output rounds on a fixed grid, not a relative one
+    assert torch.equal(y2.float()[normal], (y.float() * 2)[normal])  # scaling by 2 is exact in fp16 and fp32
     ysum = run_gemm(D, x=(x[0:1] + x[1:2]).contiguous())
     assert_close(ysum, (y[0:1].float() + y[1:2].float()), "additivity", rtol=2e-2, atol=2e-2)
 
