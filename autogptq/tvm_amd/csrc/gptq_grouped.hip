@@ -37,19 +37,20 @@ __device__ long long g_phase[16 * 8192];
 #define PHASE(i) do { } while (0)
 #endif
 
-// The four zero points (already +1) of columns n .. n+3 (n % 4 == 0) of one qzeros row.
+// The words holding the four zero points of columns n .. n+3 (n % 4 == 0) of the qzeros row
+// that starts zrow_off words into qzeros.  32-bit offsets from the uniform base pointer.
 template <int BITS>
-__device__ __forceinline__ void load_zero_words(const uint32_t *zrow, int n, uint32_t &wa, uint32_t &wb)
+__device__ __forceinline__ void load_zero_words(const uint32_t *qzeros, uint32_t zrow_off, int n, uint32_t &wa,
+                                                uint32_t &wb)
 {
     if constexpr (BITS == 4) {
-        wa = zrow[n >> 3];
+        wa = *(const uint32_t *)((const char *)qzeros + (zrow_off + (uint32_t)(n >> 3)) * 4u);
         wb = 0u;
     } else {
-        const uint32_t *blk = zrow + 3 * (n >> 5);
-        const int o = 3 * (n & 31);  // bit offset inside the 96-bit block: a multiple of 12
-        const int w = o >> 5;
-        wa = blk[w];
-        wb = blk[w < 2 ? w + 1 : 2];
+        const uint32_t blk = zrow_off + 3u * (uint32_t)(n >> 5);
+        const uint32_t w = (3u * (uint32_t)(n & 31)) >> 5;  // word of the 12-bit field inside the 96-bit block
+        wa = *(const uint32_t *)((const char *)qzeros + (blk + w) * 4u);
+        wb = *(const uint32_t *)((const char *)qzeros + (blk + (w < 2u ? w + 1u : 2u)) * 4u);
     }
 }
 
@@ -187,20 +188,18 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     //         loaded once the last weight loads are out ---------------------------------
     h4 sc[TPM][4];
     uint32_t zwa[TPM][4], zwb[TPM][4];
+    // Rows past the last group and lanes past the last column load clamped addresses: their
+    // products are zero (no x was scattered there) or never stored, so no branch is needed.
+    const int n_ld = min(n0, p.N - 4);
     auto load_epilogue_operands = [&]() {
 #pragma unroll
         for (int t = 0; t < TPM; t++) {
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const int g = g_base + 16 * t + 4 * lq + v;
-                sc[t][v] = (h4){0, 0, 0, 0};
-                zwa[t][v] = 0u;
-                zwb[t][v] = 0u;
-                if (n_ok && g < p.G) {
-                    const uint32_t soff = ((uint32_t)g * (uint32_t)p.N + (uint32_t)n0) * 2u;
-                    sc[t][v] = *(const h4 *)((const char *)scales + soff);
-                    load_zero_words<BITS>(p.qzeros + (uint32_t)g * (uint32_t)zwords, n0, zwa[t][v], zwb[t][v]);
-                }
+                const uint32_t g = (uint32_t)min(g_base + 16 * t + 4 * lq + v, p.G - 1);
+                const uint32_t soff = (g * (uint32_t)p.N + (uint32_t)n_ld) * 2u;
+                sc[t][v] = *(const h4 *)((const char *)scales + soff);
+                load_zero_words<BITS>(p.qzeros, g * (uint32_t)zwords, n_ld, zwa[t][v], zwb[t][v]);
             }
         }
     };
@@ -288,7 +287,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
             __builtin_amdgcn_sched_barrier(0);
             if (st0 + s < we) {
                 const int b = (st0 + s - s_begin) * 4 + lq;
-                uint32_t bq[4][4 * F::NB];
+                u4 bq[4][F::NB];
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
                     if constexpr (BITS == 4) {
@@ -318,8 +317,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
                     }
 #pragma unroll
                     for (int c = 0; c < 4; c++) {
-                        const u4 bw = {bq[c][nb * 4 + 0], bq[c][nb * 4 + 1], bq[c][nb * 4 + 2], bq[c][nb * 4 + 3]};
-                        const h8 bop = __builtin_bit_cast(h8, bw);
+                        const h8 bop = __builtin_bit_cast(h8, bq[c][nb]);
 #pragma unroll
                         for (int m = 0; m < M; m++)
 #pragma unroll
@@ -371,7 +369,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
                     }
                 }
                 float z[4];
-                zeros_from_words<BITS>(zwa[t][v], zwb[t][v], n0, z);
+                zeros_from_words<BITS>(zwa[t][v], zwb[t][v], n_ld, z);
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
                     tot[m][c] += (float)sc[t][v][c] * ((pv[c] - bsum) - z[c] * xsum);

@@ -144,13 +144,15 @@ GPTQ_HD uint32_t and_or(uint32_t x, uint32_t mask, uint32_t magic) { return (x &
 // int4: register r, half h holds BASE4[2r + h] + code SLOT4[2r + h]
 static constexpr float BASE4[8] = {1024.f, 1024.f, 64.f, 64.f, 1024.f, 1024.f, 64.f, 64.f};
 
-GPTQ_HD void biased4(uint32_t w, uint32_t out[4], uint32_t magic_lo, uint32_t magic_hi)
+// The outputs are whole MFMA operands (four consecutive registers each) so that the register
+// allocator can build them in place.
+GPTQ_HD void biased4(uint32_t w, u4 out[1], uint32_t magic_lo, uint32_t magic_hi)
 {
     const uint32_t w8 = w >> 8;
-    out[0] = and_or(w, 0x000f000fu, magic_lo);   // 0x64006400: 1024 + code
-    out[1] = and_or(w, 0x00f000f0u, magic_hi);   // 0x54005400: 64 + code
-    out[2] = and_or(w8, 0x000f000fu, magic_lo);
-    out[3] = and_or(w8, 0x00f000f0u, magic_hi);
+    out[0][0] = and_or(w, 0x000f000fu, magic_lo);   // 0x64006400: 1024 + code
+    out[0][1] = and_or(w, 0x00f000f0u, magic_hi);   // 0x54005400: 64 + code
+    out[0][2] = and_or(w8, 0x000f000fu, magic_lo);
+    out[0][3] = and_or(w8, 0x00f000f0u, magic_hi);
 }
 static constexpr uint32_t MAGIC4_LO = 0x64006400u;
 static constexpr uint32_t MAGIC4_HI = 0x54005400u;
@@ -161,7 +163,7 @@ static constexpr float BASE3[8] = {1024.f, 256.f, 128.f, 32.f, 1024.f, 256.f, 12
 static constexpr uint32_t MAGIC3_EVEN = 0x5c006400u;
 static constexpr uint32_t MAGIC3_ODD = 0x50005800u;
 
-GPTQ_HD void biased3(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t out[16], uint32_t magic_even,
+GPTQ_HD void biased3(uint32_t w0, uint32_t w1, uint32_t w2, u4 out[4], uint32_t magic_even,
                      uint32_t magic_odd)
 {
     uint32_t win[8];
@@ -176,8 +178,8 @@ GPTQ_HD void biased3(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t out[16], ui
     win[7] = (t << 12) | t;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        out[2 * i] = and_or(win[i], 0x001c0007u, magic_even);
-        out[2 * i + 1] = and_or(win[i], 0x00e00038u, magic_odd);
+        out[i >> 1][2 * (i & 1)] = and_or(win[i], 0x001c0007u, magic_even);
+        out[i >> 1][2 * (i & 1) + 1] = and_or(win[i], 0x00e00038u, magic_odd);
     }
 }
 

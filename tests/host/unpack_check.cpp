@@ -52,10 +52,10 @@ int main()
             }
         }
         // biased unpack: register value minus its slot's base is the code
-        uint32_t b4[4];
+        u4 b4[1];
         biased4(w0, b4, MAGIC4_LO, MAGIC4_HI);
         for (int r = 0; r < 4; r++) {
-            const h2 v = as_h2(b4[r]);
+            const h2 v = as_h2(b4[0][r]);
             for (int h = 0; h < 2; h++) {
                 if ((float)v[h] - BASE4[2 * r + h] != (float)code4(w0, SLOT4[2 * r + h])) {
                     printf("biased4 mismatch w=%08x reg %d half %d got %f\n", w0, r, h, (float)v[h]);
@@ -64,10 +64,10 @@ int main()
                 checked++;
             }
         }
-        uint32_t b3[16];
+        u4 b3[4];
         biased3(w0, w1, w2, b3, MAGIC3_EVEN, MAGIC3_ODD);
         for (int r = 0; r < 16; r++) {
-            const h2 v = as_h2(b3[r]);
+            const h2 v = as_h2(b3[r >> 2][r & 3]);
             for (int h = 0; h < 2; h++) {
                 if ((float)v[h] - BASE3[(2 * r + h) & 7] != (float)code3(w0, w1, w2, SLOT3[2 * r + h])) {
                     printf("biased3 mismatch w=%08x %08x %08x reg %d half %d got %f\n", w0, w1, w2, r, h,
