@@ -61,6 +61,13 @@ WORKLOADS = {
 }
 DEFAULT_WORKLOAD = "c2-int3-4096x11008-act-m1"
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the
+# same counter reads for a plain 256 MiB device copy); a profiler run is needed to refresh them, so
+# they are recorded here per workload.  None = not measured.
+MEASURED_TRAFFIC_BYTES = {
+    "c2-int3-4096x11008-act-m1": 18_403 * 1024 + 22_016,
+}
+
 
 def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int = 0):
     from autogptq.tvm_amd import _lib
@@ -236,6 +243,9 @@ def main():
     ap.add_argument("--kernel", type=int, default=0, help="force a kernel family (1 gather, 2 grouped, 3 blocked)")
     ap.add_argument("--split-k", type=int, default=0, help="force the split-K factor")
     ap.add_argument("--waves-n", type=int, default=0, help="force the waves per workgroup along N")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain 256 MiB device copy a few times (known traffic, for scaling the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a profiler run) and exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures the QuantLinear kernels on ONE GPU; --gpus must be 1 "
@@ -247,6 +257,16 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.copy_calibration:
+        nbytes = 256 << 20
+        src = torch.arange(nbytes // 4, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize(dev)
+        print(json.dumps({"copy_calibration": {"bytes_read": nbytes, "bytes_written": nbytes, "launches": 5,
+                                               "kernel": "torch elementwise copy (int32)"}}))
+        return
     case = build_case(args.workload, dev, args.kernel, args.split_k, args.waves_n)
     ok, max_err = check_case(case, dev)
     torch.cuda.synchronize(dev)
@@ -269,10 +289,11 @@ def main():
     }
     if gemv:
         line["roofline"] = {"bound": "hbm", "achieved": s["weight_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                            "frac": s["hbm_frac"], "traffic": None}
+                            "frac": s["hbm_frac"], "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
     else:
         line["roofline"] = {"bound": "mfma", "achieved": s["TFLOPs"], "peak": MFMA_FP16_PEAK_TFLOPS,
-                            "unit": "TFLOP/s", "frac": s["mfma_frac"], "traffic": None}
+                            "unit": "TFLOP/s", "frac": s["mfma_frac"],
+                            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
     if args.sweep:
         sweep = []
         for name in sorted(WORKLOADS):
