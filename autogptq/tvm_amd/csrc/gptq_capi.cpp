@@ -33,15 +33,19 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
     if (pl.split_k > 1 && (size_t)pl.grid_x * (pl.grid_z > 0 ? pl.grid_z : 1) * sizeof(int) > gptq::kCounterBytes)
         return GPTQ_HIP_ERR_UNSUPPORTED;
     if (pl.kernel == GPTQ_HIP_KERNEL_GATHER) {
-        if (pl.waves_k != 1) return GPTQ_HIP_ERR_UNSUPPORTED;
+        if (pl.waves_n * pl.waves_k > 4) return GPTQ_HIP_ERR_UNSUPPORTED;
         if (pl.row_tiles != 1 && pl.row_tiles != 2 && pl.row_tiles != 4 && pl.row_tiles != 8)
             return GPTQ_HIP_ERR_UNSUPPORTED;
         if (pl.k_chunk < kstep || pl.k_chunk % kstep != 0) return GPTQ_HIP_ERR_BAD_ARG;
         if (pl.m_blocks * 16 * pl.row_tiles < M || pl.grid_z != pl.m_blocks) return GPTQ_HIP_ERR_BAD_ARG;
+        if (pl.split_k * pl.waves_k > steps_total && pl.split_k * pl.waves_k > 1) return GPTQ_HIP_ERR_BAD_ARG;
         const int xs_rows = M < 16 * pl.row_tiles ? M : 16 * pl.row_tiles;
-        const long long need = (long long)G * 64 * pl.waves_n * 4 + (long long)pl.k_chunk * 4 +
-                               (long long)xs_rows * (pl.k_chunk + 8) * 2;
-        if (pl.lds_bytes < need) return GPTQ_HIP_ERR_BAD_ARG;
+        // staging registers: at most 8 vectors of x and 4 group indices per thread and chunk
+        if (xs_rows * pl.k_chunk / 8 > gptq::gather_xv(bits, pl.row_tiles) * 64 * pl.waves_n ||
+            pl.k_chunk > 4 * 64 * pl.waves_n)
+            return GPTQ_HIP_ERR_UNSUPPORTED;
+        if (pl.lds_bytes < gptq::gather_lds_bytes(G, pl.k_chunk, xs_rows, pl.row_tiles, pl.waves_n, pl.waves_k))
+            return GPTQ_HIP_ERR_BAD_ARG;
         return GPTQ_HIP_OK;
     }
     if (pl.kernel == GPTQ_HIP_KERNEL_GROUPED) {
@@ -101,7 +105,9 @@ extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const i
     p.row_tiles = plan->row_tiles;
     p.waves_n = plan->waves_n;
     p.waves_k = plan->waves_k;
-    p.wave_steps = plan->kernel == GPTQ_HIP_KERNEL_GROUPED ? plan->k_chunk / kstep / plan->waves_k : 0;
+    p.wave_steps = plan->kernel == GPTQ_HIP_KERNEL_GROUPED
+                       ? plan->k_chunk / kstep / plan->waves_k
+                       : (p.steps_total + plan->split_k * plan->waves_k - 1) / (plan->split_k * plan->waves_k);
     p.gpad = plan->kernel == GPTQ_HIP_KERNEL_GROUPED ? 16 * (plan->row_tiles / M) : 0;
     if (plan->split_k > 1) {
         const size_t need = gptq::kCounterBytes + (size_t)plan->split_k * M * N * sizeof(float);

@@ -15,42 +15,83 @@ const int kTargetWorkgroups = 512;  // two per CU keeps every XCD fed at M = 1
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // GATHER: exact weights, any g_idx, any M.
+int plan_gather_rt(int row_tiles, int M, int K, int N, int bits, int G, int force_split, int force_waves,
+                   gptq_hip_plan *plan);
+
 int plan_gather(int M, int K, int N, int bits, int G, int force_split, int force_waves, gptq_hip_plan *plan)
+{
+    // the tallest tile that fits; shorter tiles (more M blocks) when LDS or staging registers
+    // cannot hold it, e.g. with hundreds of groups in the (scale, zero) table
+    int rt = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8));
+    for (; rt >= 1; rt >>= 1) {
+        memset(plan, 0, sizeof(*plan));
+        const int rc = plan_gather_rt(rt, M, K, N, bits, G, force_split, force_waves, plan);
+        if (rc != GPTQ_HIP_ERR_UNSUPPORTED) return rc;
+    }
+    return GPTQ_HIP_ERR_UNSUPPORTED;
+}
+
+int plan_gather_rt(int row_tiles, int M, int K, int N, int bits, int G, int force_split, int force_waves,
+                   gptq_hip_plan *plan)
 {
     const int kstep = gptq::kstep_of(bits);
     const int steps_total = ceil_div(K, kstep);
     plan->kernel = GPTQ_HIP_KERNEL_GATHER;
-    plan->row_tiles = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8));
+    plan->row_tiles = row_tiles;
     plan->m_blocks = ceil_div(M, 16 * plan->row_tiles);
     const int xs_rows = M < 16 * plan->row_tiles ? M : 16 * plan->row_tiles;
-    int kc = xs_rows <= 16 ? 512 : (xs_rows <= 32 ? 256 : 128);
+    // channels of x staged per K wave at a time: less for taller tiles
+    int kc = xs_rows <= 16 ? 512 : (xs_rows <= 32 ? 256 : (xs_rows <= 64 ? 128 : 64));
+    if (kc < kstep) kc = kstep;
     if (kc > steps_total * kstep) kc = steps_total * kstep;
-    plan->k_chunk = kc;
 
-    int waves = force_waves > 0 ? force_waves : 4;
-    int lds = 0;
-    for (; waves >= 1; waves >>= 1) {
-        const int bn = 64 * waves;
-        lds = G * bn * 4 + kc * 4 + xs_rows * (kc + 8) * 2;
-        if (lds <= kLdsBudget) break;
+    // decode-like shapes stream: four waves side by side; taller tiles are MFMA-bound: two
+    // waves along N share the x tile and two along K halve the depth each one walks
+    // candidate workgroup shapes, best first
+    static const int tall[][2] = {{2, 2}, {2, 1}, {1, 2}, {1, 1}};
+    static const int skinny[][2] = {{4, 1}, {2, 1}, {1, 1}};
+    const int (*cand)[2] = row_tiles == 1 ? skinny : tall;
+    const int ncand = row_tiles == 1 ? 3 : 4;
+    const int xv = gptq::gather_xv(bits, plan->row_tiles);
+    int waves_n = 0, waves_k = 0, lds = 0;
+    const int kc0 = kc;
+    for (int i = 0; i < ncand; i++) {
+        const int wn = cand[i][0];
+        int wk = cand[i][1];
+        if (force_waves > 0 && wn != force_waves) continue;
+        if (wk > steps_total) wk = 1;
+        kc = kc0;
+        // a thread stages at most xv vectors of x and 4 group indices per chunk
+        while (kc > kstep && (xs_rows * kc / 8 > xv * 64 * wn || kc > 4 * 64 * wn)) kc -= kstep;
+        if (xs_rows * kc / 8 > xv * 64 * wn || kc > 4 * 64 * wn) continue;
+        const int need = gptq::gather_lds_bytes(G, kc, xs_rows, plan->row_tiles, wn, wk);
+        if (need > kLdsBudget) continue;
+        waves_n = wn;
+        waves_k = wk;
+        lds = need;
+        break;
     }
-    if (waves < 1) return GPTQ_HIP_ERR_UNSUPPORTED;  // more groups than the LDS table holds
-    plan->waves_n = waves;
-    plan->waves_k = 1;
+    if (waves_n == 0) return GPTQ_HIP_ERR_UNSUPPORTED;  // e.g. more groups than the LDS table holds
+    plan->k_chunk = kc;
+    plan->waves_n = waves_n;
+    plan->waves_k = waves_k;
     plan->lds_bytes = lds;
-    plan->block = 64 * waves;
-    const int col_tiles = ceil_div(N, 64 * waves);
+    plan->block = 64 * waves_n * waves_k;
+    const int col_tiles = ceil_div(N, 64 * waves_n);
 
-    int split = ceil_div(kTargetWorkgroups, col_tiles * plan->m_blocks);
-    // partial sums cost split*M*N*4 bytes each way; keep them well under the packed weights
-    int cap = (int)(((long long)K * bits) / (128LL * M));
+    int split = ceil_div(M <= 16 ? kTargetWorkgroups : 256, col_tiles * plan->m_blocks);
+    // partial sums cost split*M*N*4 bytes each way; keep them in proportion to the packed weights
+    int cap = (int)((3LL * K * bits) / (128LL * M));
     if (cap < 1) cap = 1;
     if (split > cap) split = cap;
-    if (split > steps_total) split = steps_total;
     if (split > 64) split = 64;
+    if (force_split > 0) split = force_split;
+    if (split * waves_k > steps_total) split = steps_total / waves_k;
     if (split < 1) split = 1;
-    if (force_split > 0) split = force_split > steps_total ? steps_total : force_split;
     if ((size_t)col_tiles * plan->m_blocks * sizeof(int) > gptq::kCounterBytes) split = 1;
+    // uniform partition: the split actually needed once every K wave takes whole steps
+    const int wave_steps = ceil_div(steps_total, split * waves_k);
+    split = ceil_div(steps_total, wave_steps * waves_k);
     plan->split_k = split;
     plan->grid_x = col_tiles;
     plan->grid_y = split;
@@ -77,6 +118,17 @@ int grouped_groups(int kr, int gs, int G, int act_order)
 {
     int groups = act_order ? G : (kr - 1) / gs + 2;
     return groups > G ? G : groups;
+}
+
+// LDS of the GATHER kernel: (scale, zero) table + per K wave the staged chunk (group offsets and
+// x rows), or the reduction buffer of the waves along K, which reuses the same bytes.
+int gather_lds_bytes(int G, int kc, int xs_rows, int row_tiles, int waves_n, int waves_k)
+{
+    const long long stage =
+        (long long)G * 64 * waves_n * 4 + 2LL * waves_k * (kc * 4 + xs_rows * (kc + 8) * 2);  // double-buffered
+    const long long red = (long long)(waves_k - 1) * waves_n * row_tiles * 16 * 64 * 4;
+    const long long need = stage > red ? stage : red;
+    return need > (1 << 30) ? (1 << 30) : (int)need;
 }
 
 // LDS of the GROUPED kernel for a K range of kr channels: operand tiles (+ slot masks in the

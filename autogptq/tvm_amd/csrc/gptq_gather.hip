@@ -1,55 +1,166 @@
 // GATHER kernel family: see the geometry notes in gptq_device.h.
+//
+// The weights are dequantised exactly as the reference does (fp16(scale * (q - zero)), one
+// rounding) in registers, straight into the B operand of the MFMA; x goes through LDS.
+// It covers every g_idx (activation order included) and every M; the dispatcher uses it
+// for M >= 3 and as the fallback of the GROUPED family.
+//
+// Workgroup = waves_n x waves_k waves.  A wave owns 64 columns and all 16 * RT rows of its
+// M block, so a weight is unpacked once per workgroup column tile; the waves along K split
+// the workgroup's K range and meet in LDS at the end.  split_k > 1 adds workgroups along K
+// whose partial tiles meet through the workspace.
+//
+// LDS: (scale, zero) of every group x the tile's columns [G][BN]; per K wave, double-buffered,
+// the group offsets of a chunk of input channels and the x rows of that chunk, both in slot
+// order.  The global loads of chunk i+1 are issued before chunk i is multiplied and written
+// to the other buffer afterwards: one barrier per chunk, no exposed load latency.
+// ACT = false (contiguous groups no narrower than a lane's packed row) reads one table entry
+// per packed row instead of one per weight.
+// grid = (column tiles, split_k, m blocks).
 #include "gptq_device.h"
 
 namespace gptq {
 
-// ---------------------------------------------------------------------------------
-// GATHER kernel: exact fp16 weights, scale/zero looked up per weight through g_idx.
-// Covers every g_idx (activation order included) and every M.
-// LDS: table of (scale, zero) for all groups x the tile's columns; per chunk of input
-// channels the group offsets (slot order) and the x rows (slot order).
-// grid = (column tiles, split_k, m blocks), block = 64 * waves (all waves along N).
-// ---------------------------------------------------------------------------------
-template <int BITS, int RT>
+template <int BITS, int RT, bool ACT>
 __global__ __launch_bounds__(256) void gather_kernel(const Params p)
 {
     using F = Fmt<BITS>;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+    const int WN = p.waves_n;
+    const int WK = p.waves_k;
+    const int wn = wave % WN;
+    const int wk = wave / WN;
     const int li = lane & 15;
     const int lq = lane >> 4;
-    const int BN = (int)blockDim.x;  // 64 columns per wave
+    const int BN = 64 * WN;
+    const int GT = 64 * WN;  // threads of one K wave group
+    const int gtid = wn * 64 + lane;
     const int n_blk = blockIdx.x * BN;
-    const int col_l = wave * 64 + 4 * li;
+    const int col_l = wn * 64 + 4 * li;
     const int n0 = n_blk + col_l;
     const bool n_ok = n0 < p.N;
     const int m0 = blockIdx.z * (16 * RT);
     const int rows_here = min(16 * RT, p.M - m0);
     const int split = blockIdx.y;
-    const int s_begin = (int)((long long)p.steps_total * split / p.split_k);
-    const int s_end = (int)((long long)p.steps_total * (split + 1) / p.split_k);
+    // uniform partition made by the host: wave_steps steps per K wave
+    const int wg_steps = p.wave_steps * WK;
+    const int s_begin = split * wg_steps;
+    const int s_end = min(s_begin + wg_steps, p.steps_total);
+    const int ws = s_begin + wk * p.wave_steps;
+    const int we = min(ws + p.wave_steps, s_end);
 
-    const int KC = p.chunk_steps * F::KSTEP;
+    const int CS = p.chunk_steps;
+    const int KC = CS * F::KSTEP;
     const int XS = KC + 8;
-    unsigned char *tab_b = smem;                            // h2 [G][BN] = (scale, zero)
-    int *gl = (int *)(smem + (size_t)p.G * BN * 4);         // [KC] byte offset of the group's table row
-    _Float16 *xs = (_Float16 *)(gl + KC);                   // [xs_rows][XS]
+    // per K wave group: two buffers (double buffering) of [KC] group offsets + [xs_rows][XS] x
+    const size_t buf_bytes = (size_t)KC * 4 + (size_t)p.xs_rows * XS * 2;
+    unsigned char *tab_b = smem;  // h2 [G][BN] = (scale, zero)
+    unsigned char *stage = smem + (size_t)p.G * BN * 4 + (size_t)wk * 2 * buf_bytes;
     __shared__ int last_flag;
 
     const _Float16 *x = (const _Float16 *)p.x;
     const _Float16 *scales = (const _Float16 *)p.scales;
     const int zwords = p.N / 32 * BITS;
+    const int prows = p.K / (BITS == 4 ? 8 : 32);
 
-    for (int idx = tid; idx < p.G * BN; idx += (int)blockDim.x) {
-        const int g = idx / BN;
-        const int n = n_blk + idx % BN;
-        h2 e = {(_Float16)0.0f, (_Float16)0.0f};
-        if (n < p.N) {
-            e.x = scales[(size_t)g * p.N + n];
-            e.y = (_Float16)(float)zero_of<BITS>(p.qzeros + (size_t)g * zwords, n);
+    auto load_w = [&](int st, u4 (&w)[F::WORDS]) {
+        const int prow = 4 * st + lq;  // packed row (int4) or 3-word block (int3)
+        const bool ok = n_ok && st < we && prow < prows;
+#pragma unroll
+        for (int wd = 0; wd < F::WORDS; wd++) {
+            w[wd] = (u4){0u, 0u, 0u, 0u};
+            if (ok) {
+                const uint32_t off = ((uint32_t)(prow * F::WORDS + wd) * (uint32_t)p.N + (uint32_t)n0) * 4u;
+                w[wd] = __builtin_nontemporal_load((const u4 *)((const char *)p.qweight + off));
+            }
         }
-        ((h2 *)tab_b)[idx] = e;
+    };
+    u4 wcur[F::WORDS], wnext[F::WORDS];
+    load_w(ws, wcur);
+
+    // ---- staging of one chunk, split into "global -> registers" and "registers -> LDS" so that
+    //      the loads of chunk i+1 fly while chunk i is being multiplied ---------------------
+    constexpr int XV = (BITS == 3 && RT >= 4) ? 16 : 8;  // 16-byte vectors of x per thread per chunk (see gather_xv)
+    constexpr int GV = 4;  // group indices per thread per chunk
+    h8 xreg[XV];
+    int greg[GV];
+    auto fetch_chunk = [&](int ch) {
+        const int c0 = ws + ch * CS;
+        const int c1 = min(c0 + CS, we);
+        const int k0 = c0 * F::KSTEP;
+        const int kspan = max(c1 - c0, 0) * F::KSTEP;
+        const int vec_per_row = KC / 8;
+#pragma unroll
+        for (int i = 0; i < XV; i++) {
+            const int v = gtid + i * GT;
+            const int r = v / vec_per_row;
+            const int kc = 8 * (v - r * vec_per_row);
+            xreg[i] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+            if (r < rows_here && kc < kspan && k0 + kc < p.K) {
+                xreg[i] = *(const h8 *)(x + (size_t)(m0 + r) * p.K + k0 + kc);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < GV; i++) {
+            const int kc = gtid + i * GT;
+            const int k = k0 + kc;
+            greg[i] = 0;
+            if (kc < kspan && k < p.K) greg[i] = p.g_idx ? p.g_idx[k] : k / p.group_size;
+        }
+    };
+    auto store_chunk = [&](int buf) {
+        int *gl = (int *)(stage + (size_t)buf * buf_bytes);
+        _Float16 *xs = (_Float16 *)(gl + KC);
+        const int vec_per_row = KC / 8;
+#pragma unroll
+        for (int i = 0; i < XV; i++) {
+            const int v = gtid + i * GT;
+            const int r = v / vec_per_row;
+            const int kc = 8 * (v - r * vec_per_row);
+            if (r < p.xs_rows) {
+                _Float16 *dst = xs + r * XS + (kc / F::KLANE) * F::KLANE;
+                if constexpr (BITS == 4) {
+                    h8 o;  // all eight land in one lane block: one 16-byte store in slot order
+#pragma unroll
+                    for (int s = 0; s < 8; s++) o[s] = xreg[i][SLOT4[s]];
+                    *(h8 *)dst = o;
+                } else {
+                    const int jb = kc % F::KLANE;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) dst[slot_of_code<BITS>(jb + e)] = xreg[i][e];
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < GV; i++) {
+            const int kc = gtid + i * GT;
+            if (kc < KC) {
+                const int g = min(max(greg[i], 0), p.G - 1);
+                gl[(kc / F::KLANE) * F::KLANE + slot_of_code<BITS>(kc % F::KLANE)] = g * BN * 4;
+            }
+        }
+    };
+
+    const int nchunks = (p.wave_steps + CS - 1) / CS;
+    fetch_chunk(0);
+
+    // (scale, zero) table: four columns of one group per thread and pass
+    for (int idx = tid; idx < p.G * (BN / 4); idx += (int)blockDim.x) {
+        const int g = idx / (BN / 4);
+        const int c4 = 4 * (idx - g * (BN / 4));
+        const int n = n_blk + c4;
+        u4 e = {0u, 0u, 0u, 0u};
+        if (n < p.N) {
+            const h4 s4 = *(const h4 *)(scales + (size_t)g * p.N + n);
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const h2 sz = {s4[c], (_Float16)(float)zero_of<BITS>(p.qzeros + (size_t)g * zwords, n + c)};
+                e[c] = as_u32(sz);
+            }
+        }
+        *(u4 *)(tab_b + ((size_t)g * BN + c4) * 4) = e;
     }
 
     f4 acc[RT][4];
@@ -58,84 +169,79 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
 #pragma unroll
         for (int c = 0; c < 4; c++) acc[rt][c] = (f4){0.f, 0.f, 0.f, 0.f};
 
-    const int rows3 = p.K / 32;  // 3-word blocks (int3) ...
-    const int rows4 = p.K / 8;   // ... or word rows (int4) along K
+    const uint32_t magic_a = opaque_vgpr(BITS == 4 ? MAGIC4_LO : MAGIC3_EVEN);
+    const uint32_t magic_b = opaque_vgpr(BITS == 4 ? MAGIC4_HI : MAGIC3_ODD);
 
-    for (int c0 = s_begin; c0 < s_end; c0 += p.chunk_steps) {
-        const int c1 = min(c0 + p.chunk_steps, s_end);
-        const int k0 = c0 * F::KSTEP;
-        const int kspan = (c1 - c0) * F::KSTEP;
-        __syncthreads();  // the previous chunk has been consumed by every wave
-        for (int kc = tid; kc < kspan; kc += (int)blockDim.x) {
-            const int k = k0 + kc;
-            int g = 0;
-            if (k < p.K) {
-                g = p.g_idx ? p.g_idx[k] : k / p.group_size;
-                g = min(max(g, 0), p.G - 1);
-            }
-            const int b = kc / F::KLANE;
-            gl[b * F::KLANE + slot_of_code<BITS>(kc % F::KLANE)] = g * BN * 4;
-        }
-        const int vec_per_row = kspan / 8;
-        for (int v = tid; v < rows_here * vec_per_row; v += (int)blockDim.x) {
-            const int r = v / vec_per_row;
-            const int kc = 8 * (v % vec_per_row);
-            const int k = k0 + kc;
-            h8 val = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (k < p.K) val = *(const h8 *)(x + (size_t)(m0 + r) * p.K + k);
-            _Float16 *dst = xs + r * XS + (kc / F::KLANE) * F::KLANE;
-            const int jb = kc % F::KLANE;
-#pragma unroll
-            for (int e = 0; e < 8; e++) dst[slot_of_code<BITS>(jb + e)] = val[e];
-        }
-        __syncthreads();
+    store_chunk(0);
+    __syncthreads();
+    for (int ch = 0; ch < nchunks; ch++) {
+        const int c0 = ws + ch * CS;
+        const int c1 = min(c0 + CS, we);
+        if (ch + 1 < nchunks) fetch_chunk(ch + 1);
+        const int *gl = (const int *)(stage + (size_t)(ch & 1) * buf_bytes);
+        const _Float16 *xs = (const _Float16 *)(gl + KC);
 
         for (int st = c0; st < c1; ++st) {
+            load_w(st + 1, wnext);  // next step's weights fly while this one is consumed
             const int b = (st - c0) * 4 + lq;  // this lane's block inside the chunk
-            u4 w[F::WORDS];
-            {
-                const int prow = 4 * st + lq;  // packed row (int4) or 3-word block (int3)
-                const bool ok = n_ok && prow < (BITS == 4 ? rows4 : rows3);
-#pragma unroll
-                for (int wd = 0; wd < F::WORDS; wd++) {
-                    w[wd] = (u4){0u, 0u, 0u, 0u};
-                    if (ok) w[wd] = *(const u4 *)(p.qweight + (size_t)(prow * F::WORDS + wd) * p.N + n0);
-                }
-            }
-            uint32_t mg[4][4 * F::NB];
+            u4 bq[4][F::NB];
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 if constexpr (BITS == 4) {
-                    magic4(w[0][c], mg[c]);
+                    biased4(wcur[0][c], bq[c], magic_a, magic_b);
                 } else {
-                    magic3(w[0][c], w[1][c], w[2][c], mg[c]);
+                    biased3(wcur[0][c], wcur[1][c], wcur[2][c], bq[c], magic_a, magic_b);
                 }
+            }
+            // contiguous groups: the (scale, zero) of this lane's packed row, four columns
+            u4 erow = {0u, 0u, 0u, 0u};
+            if constexpr (!ACT) {
+                erow = *(const u4 *)(tab_b + (uint32_t)gl[b * F::KLANE] + (uint32_t)col_l * 4u);
             }
 #pragma unroll
             for (int nb = 0; nb < F::NB; nb++) {
-                // (scale, zero) of the 8 slots x 4 columns
-                const u4 go0 = *(const u4 *)(gl + b * F::KLANE + nb * 8);
-                const u4 go1 = *(const u4 *)(gl + b * F::KLANE + nb * 8 + 4);
-                u4 ent[8];
-#pragma unroll
-                for (int s = 0; s < 8; s++) {
-                    const uint32_t off = (s < 4 ? go0[s & 3] : go1[s & 3]) + (uint32_t)col_l * 4u;
-                    ent[s] = *(const u4 *)(tab_b + off);
-                }
                 h8 bop[4];
+                if constexpr (ACT) {
+                    // (scale, zero) of the 8 slots x 4 columns
+                    const u4 go0 = *(const u4 *)(gl + b * F::KLANE + nb * 8);
+                    const u4 go1 = *(const u4 *)(gl + b * F::KLANE + nb * 8 + 4);
+                    u4 ent[8];
 #pragma unroll
-                for (int c = 0; c < 4; c++) {
+                    for (int s = 0; s < 8; s++) {
+                        const uint32_t off = (s < 4 ? go0[s & 3] : go1[s & 3]) + (uint32_t)col_l * 4u;
+                        ent[s] = *(const u4 *)(tab_b + off);
+                    }
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        const uint32_t ea = ent[2 * r][c];
-                        const uint32_t eb = ent[2 * r + 1][c];
-                        const h2 s2 = as_h2((ea & 0xffffu) | (eb << 16));
-                        const h2 z2 = as_h2((ea >> 16) | (eb & 0xffff0000u));
-                        const h2 q2 = BITS == 4 ? code_from_magic4(mg[c][nb * 4 + r], nb * 4 + r)
-                                                : code_from_magic3(mg[c][nb * 4 + r], nb * 4 + r);
-                        const h2 w2 = (q2 - z2) * s2;
-                        bop[c][2 * r] = w2.x;
-                        bop[c][2 * r + 1] = w2.y;
+                    for (int c = 0; c < 4; c++) {
+                        u4 wv;
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            const uint32_t ea = ent[2 * r][c];
+                            const uint32_t eb = ent[2 * r + 1][c];
+                            const h2 s2 = as_h2((ea & 0xffffu) | (eb << 16));
+                            const h2 z2 = as_h2((ea >> 16) | (eb & 0xffff0000u));
+                            const float ba = BITS == 4 ? BASE4[2 * r] : BASE3[2 * r];
+                            const float bb = BITS == 4 ? BASE4[2 * r + 1] : BASE3[2 * r + 1];
+                            const h2 zb = z2 + (h2){(_Float16)ba, (_Float16)bb};     // exact: small integers
+                            wv[r] = as_u32((as_h2(bq[c][nb][r]) - zb) * s2);         // exact difference, one rounding
+                        }
+                        bop[c] = __builtin_bit_cast(h8, wv);
+                    }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        const uint32_t e = erow[c];
+                        const h2 s2 = as_h2((e & 0xffffu) | (e << 16));
+                        const h2 z2 = as_h2((e >> 16) | (e & 0xffff0000u));
+                        u4 wv;
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            const float ba = BITS == 4 ? BASE4[2 * r] : BASE3[2 * r];
+                            const float bb = BITS == 4 ? BASE4[2 * r + 1] : BASE3[2 * r + 1];
+                            const h2 zb = z2 + (h2){(_Float16)ba, (_Float16)bb};
+                            wv[r] = as_u32((as_h2(bq[c][nb][r]) - zb) * s2);
+                        }
+                        bop[c] = __builtin_bit_cast(h8, wv);
                     }
                 }
 #pragma unroll
@@ -150,19 +256,51 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
                     }
                 }
             }
+#pragma unroll
+            for (int wd = 0; wd < F::WORDS; wd++) wcur[wd] = wnext[wd];
+        }
+        if (ch + 1 < nchunks) store_chunk((ch + 1) & 1);
+        __syncthreads();  // chunk ch+1 is in LDS, and chunk ch's buffer may be overwritten next time
+    }
+
+    // ---- waves along K meet in LDS: wave (wn, 0) adds the others' tiles in order ------------
+    if (WK > 1) {
+        float *red = (float *)smem;  // [WK - 1][WN][RT * 16][64], reuses the staging area
+        __syncthreads();
+        if (wk > 0) {
+            float *dst = red + ((size_t)((wk - 1) * WN + wn) * (RT * 16)) * 64 + lane;
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) dst[((rt * 4 + c) * 4 + v) * 64] = acc[rt][c][v];
+        }
+        __syncthreads();
+        if (wk == 0) {
+            for (int k = 1; k < WK; k++) {
+                const float *src = red + ((size_t)((k - 1) * WN + wn) * (RT * 16)) * 64 + lane;
+#pragma unroll
+                for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+                    for (int c = 0; c < 4; c++)
+#pragma unroll
+                        for (int v = 0; v < 4; v++) acc[rt][c][v] += src[((rt * 4 + c) * 4 + v) * 64];
+            }
         }
     }
+    const bool owner = wk == 0 && n_ok;
 
     // ---- epilogue: acc[rt][c][v] is y[m0 + 16 rt + 4 q + v][n0 + c] ----
     const _Float16 *bias = (const _Float16 *)p.bias;
     f4 bv = {0.f, 0.f, 0.f, 0.f};
-    if (bias && n_ok) {
+    if (bias && owner) {
         const h4 b4 = *(const h4 *)(bias + n0);
         bv = (f4){(float)b4[0], (float)b4[1], (float)b4[2], (float)b4[3]};
     }
     _Float16 *y = (_Float16 *)p.y;
     if (p.split_k == 1) {
-        if (n_ok) {
+        if (owner) {
 #pragma unroll
             for (int rt = 0; rt < RT; rt++) {
 #pragma unroll
@@ -180,7 +318,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
         return;
     }
 
-    if (n_ok) {
+    if (owner) {
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
 #pragma unroll
@@ -195,7 +333,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
     }
     int *counter = p.counters + blockIdx.z * gridDim.x + blockIdx.x;
     if (!arrive_last(counter, p.split_k, &last_flag)) return;
-    if (n_ok) {
+    if (owner) {
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
 #pragma unroll
@@ -216,10 +354,10 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
     }
 }
 
-template <int BITS, int RT>
+template <int BITS, int RT, bool ACT>
 static int launch_gather_one(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
-    auto kern = gather_kernel<BITS, RT>;
+    auto kern = gather_kernel<BITS, RT, ACT>;
     if (plan.lds_bytes > 65536) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, plan.lds_bytes) !=
             hipSuccess) {
@@ -232,22 +370,28 @@ static int launch_gather_one(const Params &p, const gptq_hip_plan &plan, hipStre
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 
-template <int BITS>
+template <int BITS, bool ACT>
 static int launch_gather_rt(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
     switch (plan.row_tiles) {
-        case 1: return launch_gather_one<BITS, 1>(p, plan, stream);
-        case 2: return launch_gather_one<BITS, 2>(p, plan, stream);
-        case 4: return launch_gather_one<BITS, 4>(p, plan, stream);
-        case 8: return launch_gather_one<BITS, 8>(p, plan, stream);
+        case 1: return launch_gather_one<BITS, 1, ACT>(p, plan, stream);
+        case 2: return launch_gather_one<BITS, 2, ACT>(p, plan, stream);
+        case 4: return launch_gather_one<BITS, 4, ACT>(p, plan, stream);
+        case 8: return launch_gather_one<BITS, 8, ACT>(p, plan, stream);
         default: return GPTQ_HIP_ERR_UNSUPPORTED;
     }
 }
 
-int launch_gather(const Params &p, int bits, const gptq_hip_plan &plan, void *stream)
+int launch_gather(const Params &p, int bits, const gptq_hip_plan &plan, void *stream_v)
 {
-    return bits == 4 ? launch_gather_rt<4>(p, plan, (hipStream_t)stream)
-                     : launch_gather_rt<3>(p, plan, (hipStream_t)stream);
+    hipStream_t stream = (hipStream_t)stream_v;
+    // the per-row table read needs every code of a lane's packed row in one group
+    const int klane = bits == 4 ? 8 : 32;
+    const bool act = p.g_idx != nullptr || (p.group_size % klane) != 0;
+    if (bits == 4) {
+        return act ? launch_gather_rt<4, true>(p, plan, stream) : launch_gather_rt<4, false>(p, plan, stream);
+    }
+    return act ? launch_gather_rt<3, true>(p, plan, stream) : launch_gather_rt<3, false>(p, plan, stream);
 }
 
 }  // namespace gptq

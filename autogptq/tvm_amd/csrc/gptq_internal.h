@@ -27,7 +27,7 @@ struct Params {
     int gpad;          // GROUPED kernel: rows per activation row = groups rounded up to 16
     int waves_n;       // waves of the workgroup along N
     int waves_k;       // waves of the workgroup along K
-    int wave_steps;    // GROUPED kernel: steps per wave (uniform partition of K)
+    int wave_steps;    // steps per wave along K (uniform partition of K made by the host)
 };
 
 // k handled by one wave step: 4 lane groups x (8 | 32) codes
@@ -40,6 +40,9 @@ static const size_t kCounterBytes = 16384;
 int grouped_tpm(int groups, int M);
 int grouped_groups(int kr, int gs, int G, int act_order);
 int grouped_lds_bytes(int kr, int M, int tpm, int waves_n, int waves_k);
+// 16-byte vectors of x one thread of the GATHER kernel can stage per chunk
+inline int gather_xv(int bits, int row_tiles) { return (bits == 3 && row_tiles >= 4) ? 16 : 8; }
+int gather_lds_bytes(int G, int kc, int xs_rows, int row_tiles, int waves_n, int waves_k);
 
 int launch_gather(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
 int launch_grouped(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
