@@ -70,25 +70,37 @@ extern __shared__ __align__(16) unsigned char smem[];
 // that arrives last adds them in split order (so the sum does not depend on arrival
 // order) and writes y.
 //
-// The partials travel through device-coherent accesses only (relaxed agent-scope
-// atomic stores and loads: write-through stores and L2-bypassing loads), so no cache
+// The partials travel through device-coherent accesses only (write-through stores and
+// L2-bypassing loads, the instructions an agent-scope atomic store/load compiles to), so no cache
 // writeback or invalidate is needed around the counter: an agent-scope release fence
 // here costs a whole-L2 writeback per wave, which serialises the workgroups of an XCD
 // and dominated the run time of the first version of these kernels.  Waiting for the
 // stores to be acknowledged before the counter is bumped is all the ordering required.
 // ---------------------------------------------------------------------------------
+// Device-coherent store / load of four floats as two 64-bit relaxed agent-scope atomics
+// (global_store_dwordx2 sc1 / global_load_dwordx2 sc1): the widest such access the language
+// offers.  (A hand-written 128-bit "sc0 sc1" instruction in inline assembly halves the count
+// again, but next to the matrix instructions of the tallest tiles it read one accumulator
+// register too early in a few lanes; the compiler does not track hazards into inline assembly.)
 __device__ __forceinline__ void store_partial(float *dst, f4 v)
 {
-#pragma unroll
-    for (int c = 0; c < 4; c++) __hip_atomic_store(dst + c, v[c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const f2 lo = {v[0], v[1]}, hi = {v[2], v[3]};
+    __hip_atomic_store((unsigned long long *)dst, __builtin_bit_cast(unsigned long long, lo), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store((unsigned long long *)dst + 1, __builtin_bit_cast(unsigned long long, hi), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ f4 load_partial(const float *src)
 {
-    f4 v;
-#pragma unroll
-    for (int c = 0; c < 4; c++) v[c] = __hip_atomic_load(src + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return v;
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const unsigned long long a =
+        __hip_atomic_load((const unsigned long long *)src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long b =
+        __hip_atomic_load((const unsigned long long *)src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const f2 lo = __builtin_bit_cast(f2, a), hi = __builtin_bit_cast(f2, b);
+    return (f4){lo[0], lo[1], hi[0], hi[1]};
 }
 
 // Returns true in the workgroup that must do the final sum.  Every thread calls it.

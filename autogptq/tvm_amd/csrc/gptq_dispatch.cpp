@@ -125,7 +125,7 @@ int grouped_groups(int kr, int gs, int G, int act_order)
 int gather_lds_bytes(int G, int kc, int xs_rows, int row_tiles, int waves_n, int waves_k)
 {
     const long long stage =
-        (long long)G * 64 * waves_n * 4 + 2LL * waves_k * (kc * 4 + xs_rows * (kc + 8) * 2);  // double-buffered
+        (long long)G * (64 * waves_n * 4 + 16) + 2LL * waves_k * (kc * 4 + xs_rows * (kc + 8) * 2);  // double-buffered
     const long long red = (long long)(waves_k - 1) * waves_n * row_tiles * 16 * 64 * 4;
     const long long need = stage > red ? stage : red;
     return need > (1 << 30) ? (1 << 30) : (int)need;

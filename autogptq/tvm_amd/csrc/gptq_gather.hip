@@ -56,8 +56,11 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
     const int XS = KC + 8;
     // per K wave group: two buffers (double buffering) of [KC] group offsets + [xs_rows][XS] x
     const size_t buf_bytes = (size_t)KC * 4 + (size_t)p.xs_rows * XS * 2;
-    unsigned char *tab_b = smem;  // h2 [G][BN] = (scale, zero)
-    unsigned char *stage = smem + (size_t)p.G * BN * 4 + (size_t)wk * 2 * buf_bytes;
+    // (scale, zero) table: h2 [G][BN], rows padded by 16 bytes so that the four lane groups, which
+    // read rows of different groups, do not all land on the same LDS banks
+    const int TROW = BN * 4 + 16;
+    unsigned char *tab_b = smem;
+    unsigned char *stage = smem + (size_t)p.G * TROW + (size_t)wk * 2 * buf_bytes;
     __shared__ int last_flag;
 
     const _Float16 *x = (const _Float16 *)p.x;
@@ -138,7 +141,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
             const int kc = gtid + i * GT;
             if (kc < KC) {
                 const int g = min(max(greg[i], 0), p.G - 1);
-                gl[(kc / F::KLANE) * F::KLANE + slot_of_code<BITS>(kc % F::KLANE)] = g * BN * 4;
+                gl[(kc / F::KLANE) * F::KLANE + slot_of_code<BITS>(kc % F::KLANE)] = g * TROW;
             }
         }
     };
@@ -160,7 +163,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
                 e[c] = as_u32(sz);
             }
         }
-        *(u4 *)(tab_b + ((size_t)g * BN + c4) * 4) = e;
+        *(u4 *)(tab_b + (size_t)g * TROW + c4 * 4) = e;
     }
 
     f4 acc[RT][4];
