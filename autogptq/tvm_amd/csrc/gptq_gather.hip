@@ -50,6 +50,10 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
     const int s_end = min(s_begin + wg_steps, p.steps_total);
     const int ws = s_begin + wk * p.wave_steps;
     const int we = min(ws + p.wave_steps, s_end);
+    // groups whose (scale, zero) this workgroup can meet: all of them under a g_idx, else those of
+    // its K range
+    const int g_lo = p.g_idx ? 0 : (s_begin * F::KSTEP) / p.group_size;
+    const int g_hi = p.g_idx ? p.G - 1 : min(p.G - 1, (min(s_end * F::KSTEP, p.K) - 1) / p.group_size);
 
     const int CS = p.chunk_steps;
     const int KC = CS * F::KSTEP;
@@ -140,7 +144,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
         for (int i = 0; i < GV; i++) {
             const int kc = gtid + i * GT;
             if (kc < KC) {
-                const int g = min(max(greg[i], 0), p.G - 1);
+                const int g = min(max(greg[i], g_lo), g_hi) - g_lo;
                 gl[(kc / F::KLANE) * F::KLANE + slot_of_code<BITS>(kc % F::KLANE)] = g * TROW;
             }
         }
@@ -149,21 +153,42 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
     const int nchunks = (p.wave_steps + CS - 1) / CS;
     fetch_chunk(0);
 
-    // (scale, zero) table: four columns of one group per thread and pass
-    for (int idx = tid; idx < p.G * (BN / 4); idx += (int)blockDim.x) {
-        const int g = idx / (BN / 4);
-        const int c4 = 4 * (idx - g * (BN / 4));
-        const int n = n_blk + c4;
-        u4 e = {0u, 0u, 0u, 0u};
-        if (n < p.N) {
-            const h4 s4 = *(const h4 *)(scales + (size_t)g * p.N + n);
+    // (scale, zero) table: four columns of one group per thread and item.  With contiguous groups
+    // only the groups of this workgroup's K range are staged (row 0 = the first of them).  Items
+    // go four at a time so that their global loads overlap.
+    const int tab_rows = g_hi - g_lo + 1;
+    const int tab_items = tab_rows * (BN / 4);
+    for (int base = tid; base < tab_items; base += 4 * (int)blockDim.x) {
+        h4 s4[4];
+        uint32_t za[4], zb[4];
+        int nn[4];
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const h2 sz = {s4[c], (_Float16)(float)zero_of<BITS>(p.qzeros + (size_t)g * zwords, n + c)};
-                e[c] = as_u32(sz);
+        for (int u = 0; u < 4; u++) {
+            const int idx = base + u * (int)blockDim.x;
+            const int gr = min(idx, tab_items - 1) / (BN / 4);
+            const int c4 = 4 * (min(idx, tab_items - 1) - gr * (BN / 4));
+            nn[u] = min(n_blk + c4, p.N - 4);
+            const uint32_t g = (uint32_t)(g_lo + gr);
+            s4[u] = *(const h4 *)((const char *)scales + (g * (uint32_t)p.N + (uint32_t)nn[u]) * 2u);
+            load_zero_words<BITS>(p.qzeros, g * (uint32_t)zwords, nn[u], za[u], zb[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int idx = base + u * (int)blockDim.x;
+            if (idx < tab_items) {
+                const int gr = idx / (BN / 4);
+                const int c4 = 4 * (idx - gr * (BN / 4));
+                float z[4];
+                zeros_from_words<BITS>(za[u], zb[u], nn[u], z);
+                u4 e;
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const h2 sz = {s4[u][c], (_Float16)z[c]};
+                    e[c] = as_u32(sz);
+                }
+                *(u4 *)(tab_b + (size_t)gr * TROW + c4 * 4) = e;
             }
         }
-        *(u4 *)(tab_b + (size_t)g * TROW + c4 * 4) = e;
     }
 
     f4 acc[RT][4];

@@ -37,38 +37,6 @@ __device__ long long g_phase[16 * 8192];
 #define PHASE(i) do { } while (0)
 #endif
 
-// The words holding the four zero points of columns n .. n+3 (n % 4 == 0) of the qzeros row
-// that starts zrow_off words into qzeros.  32-bit offsets from the uniform base pointer.
-template <int BITS>
-__device__ __forceinline__ void load_zero_words(const uint32_t *qzeros, uint32_t zrow_off, int n, uint32_t &wa,
-                                                uint32_t &wb)
-{
-    if constexpr (BITS == 4) {
-        wa = *(const uint32_t *)((const char *)qzeros + (zrow_off + (uint32_t)(n >> 3)) * 4u);
-        wb = 0u;
-    } else {
-        const uint32_t blk = zrow_off + 3u * (uint32_t)(n >> 5);
-        const uint32_t w = (3u * (uint32_t)(n & 31)) >> 5;  // word of the 12-bit field inside the 96-bit block
-        wa = *(const uint32_t *)((const char *)qzeros + (blk + w) * 4u);
-        wb = *(const uint32_t *)((const char *)qzeros + (blk + (w < 2u ? w + 1u : 2u)) * 4u);
-    }
-}
-
-template <int BITS>
-__device__ __forceinline__ void zeros_from_words(uint32_t wa, uint32_t wb, int n, float z[4])
-{
-    if constexpr (BITS == 4) {
-        const uint32_t f = wa >> (16 * ((n >> 2) & 1));
-#pragma unroll
-        for (int c = 0; c < 4; c++) z[c] = (float)(int)(((f >> (4 * c)) & 0xfu) + 1u);
-    } else {
-        const int sh = (3 * (n & 31)) & 31;
-        const uint32_t f = (uint32_t)((((uint64_t)wb << 32) | (uint64_t)wa) >> sh);
-#pragma unroll
-        for (int c = 0; c < 4; c++) z[c] = (float)(int)(((f >> (3 * c)) & 0x7u) + 1u);
-    }
-}
-
 __device__ __forceinline__ h8 and_h8(h8 a, u4 m)
 {
     u4 v = __builtin_bit_cast(u4, a);
