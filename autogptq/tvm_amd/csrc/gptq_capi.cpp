@@ -39,10 +39,13 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
         if (pl.k_chunk < kstep || pl.k_chunk % kstep != 0) return GPTQ_HIP_ERR_BAD_ARG;
         if (pl.m_blocks * 16 * pl.row_tiles < M || pl.grid_z != pl.m_blocks) return GPTQ_HIP_ERR_BAD_ARG;
         if (pl.split_k * pl.waves_k > steps_total && pl.split_k * pl.waves_k > 1) return GPTQ_HIP_ERR_BAD_ARG;
-        const int xs_rows = M < 16 * pl.row_tiles ? M : 16 * pl.row_tiles;
-        // staging registers: at most 8 vectors of x and 4 group indices per thread and chunk
-        if (xs_rows * pl.k_chunk / 8 > gptq::gather_xv(bits, pl.row_tiles) * 64 * pl.waves_n ||
-            pl.k_chunk > 4 * 64 * pl.waves_n)
+        const int xs_rows = 16 * pl.row_tiles;
+        // chunk: a power of two; every thread stages a whole number (1 .. xv) of x vectors and
+        // at most 4 group indices
+        if (pl.k_chunk != gptq::gather_kc(bits, pl.row_tiles)) return GPTQ_HIP_ERR_BAD_ARG;
+        const int vectors = xs_rows * pl.k_chunk / 8, threads = 64 * pl.waves_n;
+        if (vectors % threads != 0 || vectors / threads > gptq::gather_xv(bits, pl.row_tiles) ||
+            pl.k_chunk > gptq::gather_gv() * threads)
             return GPTQ_HIP_ERR_UNSUPPORTED;
         if (pl.lds_bytes < gptq::gather_lds_bytes(G, pl.k_chunk, xs_rows, pl.row_tiles, pl.waves_n, pl.waves_k))
             return GPTQ_HIP_ERR_BAD_ARG;
@@ -101,7 +104,7 @@ extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const i
     p.steps_total = (K + kstep - 1) / kstep;
     p.split_k = plan->split_k;
     p.chunk_steps = plan->k_chunk / kstep;
-    p.xs_rows = M < 16 * plan->row_tiles ? M : 16 * plan->row_tiles;
+    p.xs_rows = 16 * plan->row_tiles;
     p.row_tiles = plan->row_tiles;
     p.waves_n = plan->waves_n;
     p.waves_k = plan->waves_k;

@@ -97,6 +97,16 @@ __device__ __forceinline__ void zeros_from_words(uint32_t wa, uint32_t wb, int n
 
 extern __shared__ __align__(16) unsigned char smem[];
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also carries a memory fence
+// that waits for every outstanding global load (s_waitcnt vmcnt(0)), which drains the weight
+// prefetch at every barrier and exposes the full HBM latency each time; these kernels only
+// exchange data through LDS at their barriers, so waiting for the LDS counter is enough.
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0) only (gfx9 encoding: vmcnt and expcnt left at max)
+    __builtin_amdgcn_s_barrier();
+}
+
 // ---------------------------------------------------------------------------------
 // Split-K tail: every workgroup of a column tile writes its fp32 partial tile, the one
 // that arrives last adds them in split order (so the sum does not depend on arrival

@@ -39,37 +39,37 @@ int plan_gather_rt(int row_tiles, int M, int K, int N, int bits, int G, int forc
     plan->kernel = GPTQ_HIP_KERNEL_GATHER;
     plan->row_tiles = row_tiles;
     plan->m_blocks = ceil_div(M, 16 * plan->row_tiles);
-    const int xs_rows = M < 16 * plan->row_tiles ? M : 16 * plan->row_tiles;
-    // channels of x staged per K wave at a time: less for taller tiles
-    int kc = xs_rows <= 16 ? 512 : (xs_rows <= 32 ? 256 : (xs_rows <= 64 ? 128 : 64));
-    if (kc < kstep) kc = kstep;
-    if (kc > steps_total * kstep) kc = steps_total * kstep;
+    // x is staged for all 16 * row_tiles rows of the tile (rows past M hold zeros)
+    const int xs_rows = 16 * plan->row_tiles;
+    // channels of x staged per K wave at a time: fixed per (bits, row tiles), see gather_kc
+    const int kc_fixed = gptq::gather_kc(bits, plan->row_tiles);
 
-    // decode-like shapes stream: four waves side by side; taller tiles are MFMA-bound: two
-    // waves along N share the x tile and two along K halve the depth each one walks
     // candidate workgroup shapes, best first
     static const int tall[][2] = {{2, 2}, {2, 1}, {1, 2}, {1, 1}};
     static const int skinny[][2] = {{4, 1}, {2, 1}, {1, 1}};
     const int (*cand)[2] = row_tiles == 1 ? skinny : tall;
     const int ncand = row_tiles == 1 ? 3 : 4;
     const int xv = gptq::gather_xv(bits, plan->row_tiles);
-    int waves_n = 0, waves_k = 0, lds = 0;
-    const int kc0 = kc;
-    for (int i = 0; i < ncand; i++) {
+    int waves_n = 0, waves_k = 0, lds = 0, kc = 0;
+    for (int i = 0; i < ncand && waves_n == 0; i++) {
         const int wn = cand[i][0];
         int wk = cand[i][1];
         if (force_waves > 0 && wn != force_waves) continue;
         if (wk > steps_total) wk = 1;
-        kc = kc0;
-        // a thread stages at most xv vectors of x and 4 group indices per chunk
-        while (kc > kstep && (xs_rows * kc / 8 > xv * 64 * wn || kc > 4 * 64 * wn)) kc -= kstep;
-        if (xs_rows * kc / 8 > xv * 64 * wn || kc > 4 * 64 * wn) continue;
-        const int need = gptq::gather_lds_bytes(G, kc, xs_rows, plan->row_tiles, wn, wk);
-        if (need > kLdsBudget) continue;
-        waves_n = wn;
-        waves_k = wk;
-        lds = need;
-        break;
+        // every thread of a K wave group stages the same whole number of 16-byte vectors of x
+        // (1 .. xv) and at most 4 group indices per chunk
+        for (int k = kc_fixed; k == kc_fixed; k = 0) {
+            const int vectors = xs_rows * k / 8;
+            const int threads = 64 * wn;
+            if (vectors % threads != 0 || vectors / threads > xv || k > gptq::gather_gv() * threads) continue;
+            const int need = gptq::gather_lds_bytes(G, k, xs_rows, plan->row_tiles, wn, wk);
+            if (need > kLdsBudget) continue;
+            waves_n = wn;
+            waves_k = wk;
+            lds = need;
+            kc = k;
+            break;
+        }
     }
     if (waves_n == 0) return GPTQ_HIP_ERR_UNSUPPORTED;  // e.g. more groups than the LDS table holds
     plan->k_chunk = kc;

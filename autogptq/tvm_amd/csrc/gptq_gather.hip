@@ -21,6 +21,22 @@
 
 namespace gptq {
 
+#ifdef GPTQ_PHASE_TIMES
+__device__ long long g_phase_gather[16 * 8192];
+#define PHASE(i)                                                                                                   \
+    do {                                                                                                           \
+        if (lane == 0)                                                                                             \
+            g_phase_gather[((size_t)((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 4 + wave) * 16 + \
+                           (i)] = clock64();                                                                       \
+    } while (0)
+extern "C" int gptq_hip_debug_read_gather(void *host, size_t bytes)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_phase_gather), bytes, 0, hipMemcpyDeviceToHost);
+}
+#else
+#define PHASE(i) do { } while (0)
+#endif
+
 template <int BITS, int RT, bool ACT>
 __global__ __launch_bounds__(256) void gather_kernel(const Params p)
 {
@@ -41,6 +57,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
     const int col_l = wn * 64 + 4 * li;
     const int n0 = n_blk + col_l;
     const bool n_ok = n0 < p.N;
+    PHASE(0);
     const int m0 = blockIdx.z * (16 * RT);
     const int rows_here = min(16 * RT, p.M - m0);
     const int split = blockIdx.y;
@@ -55,11 +72,11 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
     const int g_lo = p.g_idx ? 0 : (s_begin * F::KSTEP) / p.group_size;
     const int g_hi = p.g_idx ? p.G - 1 : min(p.G - 1, (min(s_end * F::KSTEP, p.K) - 1) / p.group_size);
 
-    const int CS = p.chunk_steps;
-    const int KC = CS * F::KSTEP;
+    constexpr int KC = gather_kc(BITS, RT);  // channels staged per chunk (a power of two)
+    constexpr int CS = KC / F::KSTEP;        // steps per chunk; divides PF
     const int XS = KC + 8;
-    // per K wave group: two buffers (double buffering) of [KC] group offsets + [xs_rows][XS] x
-    const size_t buf_bytes = (size_t)KC * 4 + (size_t)p.xs_rows * XS * 2;
+    // per K wave group: two buffers (double buffering) of [KC] group offsets + [16 RT][XS] x
+    const size_t buf_bytes = (size_t)KC * 4 + (size_t)(16 * RT) * XS * 2;
     // (scale, zero) table: h2 [G][BN], rows padded by 16 bytes so that the four lane groups, which
     // read rows of different groups, do not all land on the same LDS banks
     const int TROW = BN * 4 + 16;
@@ -72,25 +89,33 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
     const int zwords = p.N / 32 * BITS;
     const int prows = p.K / (BITS == 4 ? 8 : 32);
 
+    // Everything in the main loop is branch-free per lane: addresses are clamped into bounds and
+    // what must not count is multiplied by a zero x (rows past M, channels past K) or never
+    // stored (columns past N).  Per-lane branches here cost more than the matrix work.
+    const uint32_t n_ld = (uint32_t)min(n0, p.N - 4);
     auto load_w = [&](int st, u4 (&w)[F::WORDS]) {
-        const int prow = 4 * st + lq;  // packed row (int4) or 3-word block (int3)
-        const bool ok = n_ok && st < we && prow < prows;
+        const uint32_t prow = (uint32_t)min(4 * st + lq, prows - 1);  // packed row (int4) / 3-word block (int3)
 #pragma unroll
         for (int wd = 0; wd < F::WORDS; wd++) {
-            w[wd] = (u4){0u, 0u, 0u, 0u};
-            if (ok) {
-                const uint32_t off = ((uint32_t)(prow * F::WORDS + wd) * (uint32_t)p.N + (uint32_t)n0) * 4u;
-                w[wd] = __builtin_nontemporal_load((const u4 *)((const char *)p.qweight + off));
-            }
+            const uint32_t off = ((prow * F::WORDS + wd) * (uint32_t)p.N + n_ld) * 4u;
+            w[wd] = __builtin_nontemporal_load((const u4 *)((const char *)p.qweight + off));
         }
     };
-    u4 wcur[F::WORDS], wnext[F::WORDS];
-    load_w(ws, wcur);
+    // Weight loads run PF steps ahead of their use in a ring of registers: with one wave per
+    // SIMD the cache-cold HBM latency must be covered by loads in flight, not by other waves.
+    constexpr int PF = BITS == 4 ? 8 : 4;
+    static_assert(PF % CS == 0, "a chunk must divide the prefetch ring");
+    u4 w[PF][F::WORDS];
+#pragma unroll
+    for (int u = 0; u < PF; u++) load_w(ws + u, w[u]);
 
     // ---- staging of one chunk, split into "global -> registers" and "registers -> LDS" so that
     //      the loads of chunk i+1 fly while chunk i is being multiplied ---------------------
-    constexpr int XV = (BITS == 3 && RT >= 4) ? 16 : 8;  // 16-byte vectors of x per thread per chunk (see gather_xv)
-    constexpr int GV = 4;  // group indices per thread per chunk
+    constexpr int XV = gather_xv(BITS, RT);  // 16-byte vectors of x per thread per chunk, at most
+    constexpr int GV = gather_gv();          // group indices per thread per chunk, at most
+    const int vshift = __builtin_ctz(KC / 8);          // log2(vectors per row)
+    const int xve = ((16 * RT) << vshift) / GT;        // vectors this thread stages (uniform)
+    const int gve = (KC + GT - 1) / GT;
     h8 xreg[XV];
     int greg[GV];
     auto fetch_chunk = [&](int ch) {
@@ -98,35 +123,38 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
         const int c1 = min(c0 + CS, we);
         const int k0 = c0 * F::KSTEP;
         const int kspan = max(c1 - c0, 0) * F::KSTEP;
-        const int vec_per_row = KC / 8;
 #pragma unroll
         for (int i = 0; i < XV; i++) {
-            const int v = gtid + i * GT;
-            const int r = v / vec_per_row;
-            const int kc = 8 * (v - r * vec_per_row);
-            xreg[i] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
-            if (r < rows_here && kc < kspan && k0 + kc < p.K) {
-                xreg[i] = *(const h8 *)(x + (size_t)(m0 + r) * p.K + k0 + kc);
+            if (i < xve) {
+                const int v = gtid + i * GT;
+                const int r = v >> vshift;
+                const int kc = 8 * (v & ((1 << vshift) - 1));
+                const bool ok = r < rows_here && kc < kspan && k0 + kc < p.K;
+                const uint32_t off =
+                    ((uint32_t)(m0 + min(r, rows_here - 1)) * (uint32_t)p.K + (uint32_t)min(k0 + kc, p.K - 8)) * 2u;
+                const u4 raw = *(const u4 *)((const char *)x + off);
+                const u4 zero = {0u, 0u, 0u, 0u};
+                xreg[i] = __builtin_bit_cast(h8, ok ? raw : zero);
             }
         }
 #pragma unroll
         for (int i = 0; i < GV; i++) {
-            const int kc = gtid + i * GT;
-            const int k = k0 + kc;
-            greg[i] = 0;
-            if (kc < kspan && k < p.K) greg[i] = p.g_idx ? p.g_idx[k] : k / p.group_size;
+            if (i < gve) {
+                const int kc = min(gtid + i * GT, KC - 1);  // threads past the chunk repeat its last entry
+                const int k = min(k0 + kc, p.K - 1);
+                greg[i] = p.g_idx ? p.g_idx[k] : k / p.group_size;
+            }
         }
     };
     auto store_chunk = [&](int buf) {
         int *gl = (int *)(stage + (size_t)buf * buf_bytes);
         _Float16 *xs = (_Float16 *)(gl + KC);
-        const int vec_per_row = KC / 8;
 #pragma unroll
         for (int i = 0; i < XV; i++) {
-            const int v = gtid + i * GT;
-            const int r = v / vec_per_row;
-            const int kc = 8 * (v - r * vec_per_row);
-            if (r < p.xs_rows) {
+            if (i < xve) {
+                const int v = gtid + i * GT;
+                const int r = v >> vshift;
+                const int kc = 8 * (v & ((1 << vshift) - 1));
                 _Float16 *dst = xs + r * XS + (kc / F::KLANE) * F::KLANE;
                 if constexpr (BITS == 4) {
                     h8 o;  // all eight land in one lane block: one 16-byte store in slot order
@@ -142,8 +170,8 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
         }
 #pragma unroll
         for (int i = 0; i < GV; i++) {
-            const int kc = gtid + i * GT;
-            if (kc < KC) {
+            if (i < gve) {
+                const int kc = min(gtid + i * GT, KC - 1);
                 const int g = min(max(greg[i], g_lo), g_hi) - g_lo;
                 gl[(kc / F::KLANE) * F::KLANE + slot_of_code<BITS>(kc % F::KLANE)] = g * TROW;
             }
@@ -152,6 +180,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
 
     const int nchunks = (p.wave_steps + CS - 1) / CS;
     fetch_chunk(0);
+    PHASE(1);
 
     // (scale, zero) table: four columns of one group per thread and item.  With contiguous groups
     // only the groups of this workgroup's K range are staged (row 0 = the first of them).  Items
@@ -191,6 +220,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
         }
     }
 
+    PHASE(2);
     f4 acc[RT][4];
 #pragma unroll
     for (int rt = 0; rt < RT; rt++)
@@ -201,100 +231,112 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
     const uint32_t magic_b = opaque_vgpr(BITS == 4 ? MAGIC4_HI : MAGIC3_ODD);
 
     store_chunk(0);
-    __syncthreads();
-    for (int ch = 0; ch < nchunks; ch++) {
-        const int c0 = ws + ch * CS;
-        const int c1 = min(c0 + CS, we);
-        if (ch + 1 < nchunks) fetch_chunk(ch + 1);
-        const int *gl = (const int *)(stage + (size_t)(ch & 1) * buf_bytes);
-        const _Float16 *xs = (const _Float16 *)(gl + KC);
-
-        for (int st = c0; st < c1; ++st) {
-            load_w(st + 1, wnext);  // next step's weights fly while this one is consumed
-            const int b = (st - c0) * 4 + lq;  // this lane's block inside the chunk
-            u4 bq[4][F::NB];
+    lds_barrier();
+    PHASE(3);
+    // steps every wave of the workgroup walks: whole chunks, rounded up to the prefetch ring
+    const int total = (nchunks * CS + PF - 1) / PF * PF;
+    const int walk_chunks = (total + CS - 1) / CS;  // chunks past the wave's range are staged as zeros
+    int ch = 0;  // chunk being multiplied
+    for (int i0 = 0; i0 < total; i0 += PF) {
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-                if constexpr (BITS == 4) {
-                    biased4(wcur[0][c], bq[c], magic_a, magic_b);
-                } else {
-                    biased3(wcur[0][c], wcur[1][c], wcur[2][c], bq[c], magic_a, magic_b);
-                }
-            }
-            // contiguous groups: the (scale, zero) of this lane's packed row, four columns
-            u4 erow = {0u, 0u, 0u, 0u};
-            if constexpr (!ACT) {
-                erow = *(const u4 *)(tab_b + (uint32_t)gl[b * F::KLANE] + (uint32_t)col_l * 4u);
-            }
-#pragma unroll
-            for (int nb = 0; nb < F::NB; nb++) {
-                h8 bop[4];
-                if constexpr (ACT) {
-                    // (scale, zero) of the 8 slots x 4 columns
-                    const u4 go0 = *(const u4 *)(gl + b * F::KLANE + nb * 8);
-                    const u4 go1 = *(const u4 *)(gl + b * F::KLANE + nb * 8 + 4);
-                    u4 ent[8];
-#pragma unroll
-                    for (int s = 0; s < 8; s++) {
-                        const uint32_t off = (s < 4 ? go0[s & 3] : go1[s & 3]) + (uint32_t)col_l * 4u;
-                        ent[s] = *(const u4 *)(tab_b + off);
-                    }
+        for (int u = 0; u < PF; u++) {
+            // No condition guards the matrix work: steps past the wave's range (the host rounds the
+            // walk up to whole chunks and to a multiple of PF) multiply x rows that were staged
+            // as zeros.  Guarding them makes the compiler shuttle all accumulators between
+            // register files at every merge point.
+            {
+                const int st = ws + i0 + u;
+                const int ci = u % CS;  // step inside the chunk: known at compile time
+                if ((u % CS) == 0 && ch + 1 < walk_chunks) fetch_chunk(ch + 1);
+                const int *gl = (const int *)(stage + (size_t)(ch & 1) * buf_bytes);
+                const _Float16 *xs = (const _Float16 *)(gl + KC);
+                {
+                    const int b = ci * 4 + lq;  // this lane's block inside the chunk
+                    u4 bq[4][F::NB];
 #pragma unroll
                     for (int c = 0; c < 4; c++) {
-                        u4 wv;
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            const uint32_t ea = ent[2 * r][c];
-                            const uint32_t eb = ent[2 * r + 1][c];
-                            const h2 s2 = as_h2((ea & 0xffffu) | (eb << 16));
-                            const h2 z2 = as_h2((ea >> 16) | (eb & 0xffff0000u));
-                            const float ba = BITS == 4 ? BASE4[2 * r] : BASE3[2 * r];
-                            const float bb = BITS == 4 ? BASE4[2 * r + 1] : BASE3[2 * r + 1];
-                            const h2 zb = z2 + (h2){(_Float16)ba, (_Float16)bb};     // exact: small integers
-                            wv[r] = as_u32((as_h2(bq[c][nb][r]) - zb) * s2);         // exact difference, one rounding
+                        if constexpr (BITS == 4) {
+                            biased4(w[u][0][c], bq[c], magic_a, magic_b);
+                        } else {
+                            biased3(w[u][0][c], w[u][1][c], w[u][2][c], bq[c], magic_a, magic_b);
                         }
-                        bop[c] = __builtin_bit_cast(h8, wv);
                     }
-                } else {
+                    // contiguous groups: the (scale, zero) of this lane's packed row, four columns
+                    u4 erow = {0u, 0u, 0u, 0u};
+                    if constexpr (!ACT) {
+                        erow = *(const u4 *)(tab_b + (uint32_t)gl[b * F::KLANE] + (uint32_t)col_l * 4u);
+                    }
 #pragma unroll
-                    for (int c = 0; c < 4; c++) {
-                        const uint32_t e = erow[c];
-                        const h2 s2 = as_h2((e & 0xffffu) | (e << 16));
-                        const h2 z2 = as_h2((e >> 16) | (e & 0xffff0000u));
-                        u4 wv;
+                    for (int nb = 0; nb < F::NB; nb++) {
+                        h8 bop[4];
+                        if constexpr (ACT) {
+                            // (scale, zero) of the 8 slots x 4 columns
+                            const u4 go0 = *(const u4 *)(gl + b * F::KLANE + nb * 8);
+                            const u4 go1 = *(const u4 *)(gl + b * F::KLANE + nb * 8 + 4);
+                            u4 ent[8];
 #pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            const float ba = BITS == 4 ? BASE4[2 * r] : BASE3[2 * r];
-                            const float bb = BITS == 4 ? BASE4[2 * r + 1] : BASE3[2 * r + 1];
-                            const h2 zb = z2 + (h2){(_Float16)ba, (_Float16)bb};
-                            wv[r] = as_u32((as_h2(bq[c][nb][r]) - zb) * s2);
+                            for (int s = 0; s < 8; s++) {
+                                const uint32_t off = (s < 4 ? go0[s & 3] : go1[s & 3]) + (uint32_t)col_l * 4u;
+                                ent[s] = *(const u4 *)(tab_b + off);
+                            }
+#pragma unroll
+                            for (int c = 0; c < 4; c++) {
+                                u4 wv;
+#pragma unroll
+                                for (int r = 0; r < 4; r++) {
+                                    const uint32_t ea = ent[2 * r][c];
+                                    const uint32_t eb = ent[2 * r + 1][c];
+                                    const h2 s2 = as_h2((ea & 0xffffu) | (eb << 16));
+                                    const h2 z2 = as_h2((ea >> 16) | (eb & 0xffff0000u));
+                                    const float ba = BITS == 4 ? BASE4[2 * r] : BASE3[2 * r];
+                                    const float bb = BITS == 4 ? BASE4[2 * r + 1] : BASE3[2 * r + 1];
+                                    const h2 zb = z2 + (h2){(_Float16)ba, (_Float16)bb};  // exact: small integers
+                                    wv[r] = as_u32((as_h2(bq[c][nb][r]) - zb) * s2);      // exact difference, one rounding
+                                }
+                                bop[c] = __builtin_bit_cast(h8, wv);
+                            }
+                        } else {
+#pragma unroll
+                            for (int c = 0; c < 4; c++) {
+                                const uint32_t e = erow[c];
+                                const h2 s2 = as_h2((e & 0xffffu) | (e << 16));
+                                const h2 z2 = as_h2((e >> 16) | (e & 0xffff0000u));
+                                u4 wv;
+#pragma unroll
+                                for (int r = 0; r < 4; r++) {
+                                    const float ba = BITS == 4 ? BASE4[2 * r] : BASE3[2 * r];
+                                    const float bb = BITS == 4 ? BASE4[2 * r + 1] : BASE3[2 * r + 1];
+                                    const h2 zb = z2 + (h2){(_Float16)ba, (_Float16)bb};
+                                    wv[r] = as_u32((as_h2(bq[c][nb][r]) - zb) * s2);
+                                }
+                                bop[c] = __builtin_bit_cast(h8, wv);
+                            }
                         }
-                        bop[c] = __builtin_bit_cast(h8, wv);
+#pragma unroll
+                        for (int rt = 0; rt < RT; rt++) {
+                            const h8 a = *(const h8 *)(xs + (16 * rt + li) * XS + b * F::KLANE + nb * 8);
+#pragma unroll
+                            for (int c = 0; c < 4; c++) {
+                                acc[rt][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bop[c], acc[rt][c], 0, 0, 0);
+                            }
+                        }
                     }
                 }
-#pragma unroll
-                for (int rt = 0; rt < RT; rt++) {
-                    h8 a = {0, 0, 0, 0, 0, 0, 0, 0};
-                    if (16 * rt + li < rows_here) {
-                        a = *(const h8 *)(xs + (16 * rt + li) * XS + b * F::KLANE + nb * 8);
-                    }
-#pragma unroll
-                    for (int c = 0; c < 4; c++) {
-                        acc[rt][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bop[c], acc[rt][c], 0, 0, 0);
-                    }
+                load_w(st + PF, w[u]);  // refill this ring slot
+                if ((u % CS) == CS - 1) {
+                    if (ch + 1 < walk_chunks) store_chunk((ch + 1) & 1);
+                    lds_barrier();  // chunk ch+1 is in LDS, and chunk ch's buffer may be overwritten next time
+                    ch++;
                 }
             }
-#pragma unroll
-            for (int wd = 0; wd < F::WORDS; wd++) wcur[wd] = wnext[wd];
         }
-        if (ch + 1 < nchunks) store_chunk((ch + 1) & 1);
-        __syncthreads();  // chunk ch+1 is in LDS, and chunk ch's buffer may be overwritten next time
     }
 
+    PHASE(4);
     // ---- waves along K meet in LDS: wave (wn, 0) adds the others' tiles in order ------------
     if (WK > 1) {
         float *red = (float *)smem;  // [WK - 1][WN][RT * 16][64], reuses the staging area
-        __syncthreads();
+        lds_barrier();
         if (wk > 0) {
             float *dst = red + ((size_t)((wk - 1) * WN + wn) * (RT * 16)) * 64 + lane;
 #pragma unroll
@@ -304,7 +346,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
 #pragma unroll
                     for (int v = 0; v < 4; v++) dst[((rt * 4 + c) * 4 + v) * 64] = acc[rt][c][v];
         }
-        __syncthreads();
+        lds_barrier();
         if (wk == 0) {
             for (int k = 1; k < WK; k++) {
                 const float *src = red + ((size_t)((k - 1) * WN + wn) * (RT * 16)) * 64 + lane;
@@ -318,6 +360,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
         }
     }
     const bool owner = wk == 0 && n_ok;
+    PHASE(5);
 
     // ---- epilogue: acc[rt][c][v] is y[m0 + 16 rt + 4 q + v][n0 + c] ----
     const _Float16 *bias = (const _Float16 *)p.bias;
@@ -343,6 +386,8 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
                 }
             }
         }
+        PHASE(6);
+        PHASE(7);
         return;
     }
 
@@ -359,8 +404,12 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
             }
         }
     }
+    PHASE(6);
     int *counter = p.counters + blockIdx.z * gridDim.x + blockIdx.x;
-    if (!arrive_last(counter, p.split_k, &last_flag)) return;
+    if (!arrive_last(counter, p.split_k, &last_flag)) {
+        PHASE(7);
+        return;
+    }
     if (owner) {
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
@@ -380,6 +429,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
             }
         }
     }
+    PHASE(7);
 }
 
 template <int BITS, int RT, bool ACT>

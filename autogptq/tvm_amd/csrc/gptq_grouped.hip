@@ -172,7 +172,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         }
     };
 
-    __syncthreads();
+    lds_barrier();
     PHASE(2);
     // ---- 5. scatter x into the operand tiles (waits for x / g_idx only) -------------------
     // A thread always owns quads with the same position inside a lane block (kc % KLANE is
@@ -214,7 +214,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
             }
         }
     }
-    __syncthreads();
+    lds_barrier();
     PHASE(3);
     load_epilogue_operands();
 
@@ -363,7 +363,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
                 (f4){tot[m][0], tot[m][1], tot[m][2], tot[m][3]};
         }
     }
-    __syncthreads();
+    lds_barrier();
     PHASE(6);
     const bool fin = tid < WN * M * 16;
     const int f_wn = tid / (M * 16);

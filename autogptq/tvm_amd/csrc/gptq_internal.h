@@ -40,8 +40,18 @@ static const size_t kCounterBytes = 16384;
 int grouped_tpm(int groups, int M);
 int grouped_groups(int kr, int gs, int G, int act_order);
 int grouped_lds_bytes(int kr, int M, int tpm, int waves_n, int waves_k);
+// Input channels of x the GATHER kernel stages per K wave at a time: fixed per (bits, row tiles) so
+// that the kernel's unrolled step loop knows its chunk boundaries at compile time.  The chunk is a
+// whole number of steps that divides the weight prefetch depth (8 steps int4, 4 steps int3).
+constexpr int gather_kc(int bits, int row_tiles)
+{
+    return bits == 4 ? (row_tiles >= 8 ? 64 : (row_tiles == 4 ? 128 : 256))
+                     : (row_tiles >= 4 ? 128 : (row_tiles == 2 ? 256 : 512));
+}
 // 16-byte vectors of x one thread of the GATHER kernel can stage per chunk
-inline int gather_xv(int bits, int row_tiles) { return (bits == 3 && row_tiles >= 4) ? 16 : 8; }
+constexpr int gather_xv(int bits, int row_tiles) { return (bits == 3 && row_tiles != 2) ? 16 : 8; }
+// group indices one thread can stage per chunk
+constexpr int gather_gv() { return 8; }
 int gather_lds_bytes(int G, int kc, int xs_rows, int row_tiles, int waves_n, int waves_k);
 
 int launch_gather(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);

@@ -52,6 +52,8 @@ WORKLOADS = {
     "c4-int4-4096x11008-act-m128": (4, 4096, 11008, 128, True, 128),
     "c4-int4-4096x11008-act-m256": (4, 4096, 11008, 128, True, 256),
     "c4-int3-4096x11008-act-m128": (3, 4096, 11008, 128, True, 128),
+    "int4-4096x11008-m128": (4, 4096, 11008, 128, False, 128),
+    "int4-4096x11008-m256": (4, 4096, 11008, 128, False, 256),
     "c4-int4-11008x4096-act-m128": (4, 11008, 4096, 128, True, 128),
     "c4-int3-11008x4096-act-m128": (3, 11008, 4096, 128, True, 128),
     "c5-int3-9216x9216-g1-m1": (3, 9216, 9216, -1, True, 1),
