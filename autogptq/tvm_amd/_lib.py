@@ -19,7 +19,7 @@ ERR_LAUNCH = -4
 
 KERNEL_GATHER = 1
 KERNEL_GROUPED = 2
-KERNEL_BLOCKED = 3
+KERNEL_STREAM = 3
 
 ABI_SYMBOLS = (
     "gptq_hip_select",

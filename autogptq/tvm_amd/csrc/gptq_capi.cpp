@@ -24,6 +24,24 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
 {
     const int kstep = gptq::kstep_of(bits);
     const int steps_total = (K + kstep - 1) / kstep;
+    if (pl.kernel == GPTQ_HIP_KERNEL_STREAM) {
+        if (pl.waves_n != 1 || (pl.waves_k != 1 && pl.waves_k != 2 && pl.waves_k != 4 && pl.waves_k != 8))
+            return GPTQ_HIP_ERR_UNSUPPORTED;
+        if (pl.row_tiles != 1 && pl.row_tiles != 2 && pl.row_tiles != 4) return GPTQ_HIP_ERR_UNSUPPORTED;
+        if (pl.block != 64 * pl.waves_k || pl.split_k < 1 || pl.grid_y != pl.split_k) return GPTQ_HIP_ERR_BAD_ARG;
+        if ((long long)pl.grid_x * 64 < N || pl.m_blocks < 1 || pl.grid_z != pl.m_blocks ||
+            (long long)pl.m_blocks * 16 * pl.row_tiles < M)
+            return GPTQ_HIP_ERR_BAD_ARG;
+        if ((size_t)pl.grid_x * pl.grid_z * sizeof(int) > gptq::kCounterBytes) return GPTQ_HIP_ERR_UNSUPPORTED;
+        const int wave_steps = gptq::stream_wave_steps(bits, steps_total, pl.split_k, pl.waves_k);
+        // every workgroup along K must start inside K
+        if ((long long)(pl.split_k - 1) * pl.waves_k * wave_steps >= steps_total) return GPTQ_HIP_ERR_BAD_ARG;
+        const int act_table = gptq::stream_act_table(bits, gs, act_order);
+        if (pl.lds_bytes > 160 * 1024 ||
+            pl.lds_bytes < gptq::stream_lds_bytes(bits, K, G, gs, act_table, pl.row_tiles, pl.waves_k, wave_steps))
+            return GPTQ_HIP_ERR_BAD_ARG;
+        return GPTQ_HIP_OK;
+    }
     if (pl.waves_n != 1 && pl.waves_n != 2 && pl.waves_n != 4) return GPTQ_HIP_ERR_UNSUPPORTED;
     if (pl.waves_k < 1 || pl.waves_n * pl.waves_k > 8) return GPTQ_HIP_ERR_UNSUPPORTED;
     if (pl.block != 64 * pl.waves_n * pl.waves_k) return GPTQ_HIP_ERR_BAD_ARG;
@@ -112,6 +130,30 @@ extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const i
                        ? plan->k_chunk / kstep / plan->waves_k
                        : (p.steps_total + plan->split_k * plan->waves_k - 1) / (plan->split_k * plan->waves_k);
     p.gpad = plan->kernel == GPTQ_HIP_KERNEL_GROUPED ? 16 * (plan->row_tiles / M) : 0;
+    p.xpack = nullptr;
+    p.gpack = nullptr;
+    p.rt_total = 0;
+    p.steps_pad = 0;
+    p.act_table = 0;
+    if (plan->kernel == GPTQ_HIP_KERNEL_STREAM) {
+        // workspace: counters | partial tiles (split_k > 1) | packed x | packed table offsets
+        p.wave_steps = gptq::stream_wave_steps(bits, p.steps_total, plan->split_k, plan->waves_k);
+        p.steps_pad = plan->split_k * plan->waves_k * p.wave_steps;
+        p.rt_total = plan->row_tiles * plan->m_blocks;
+        p.act_table = gptq::stream_act_table(bits, gs, act_order);
+        const size_t part =
+            plan->split_k > 1 ? ((size_t)plan->split_k * M * N * sizeof(float) + 255) / 256 * 256 : 0;
+        const size_t xb = gptq::stream_xpack_bytes(bits, p.steps_pad, p.rt_total);
+        const size_t gb = gptq::stream_gpack_bytes(bits, p.steps_pad, p.act_table);
+        if (xb >= (1ull << 32)) return GPTQ_HIP_ERR_UNSUPPORTED;  // the kernel uses 32-bit byte offsets
+        const size_t need = gptq::kCounterBytes + part + xb + gb;
+        if (!workspace || workspace_bytes < need || !aligned(workspace, 16)) return GPTQ_HIP_ERR_WORKSPACE;
+        p.counters = (int *)workspace;
+        p.partial = (float *)((char *)workspace + gptq::kCounterBytes);
+        p.xpack = (char *)workspace + gptq::kCounterBytes + part;
+        p.gpack = (int32_t *)((char *)p.xpack + xb);
+        return gptq::launch_stream(p, bits, *plan, stream);
+    }
     if (plan->split_k > 1) {
         const size_t need = gptq::kCounterBytes + (size_t)plan->split_k * M * N * sizeof(float);
         if (!workspace || workspace_bytes < need || !aligned(workspace, 16)) return GPTQ_HIP_ERR_WORKSPACE;

@@ -131,6 +131,39 @@ int gather_lds_bytes(int G, int kc, int xs_rows, int row_tiles, int waves_n, int
     return need > (1 << 30) ? (1 << 30) : (int)need;
 }
 
+// LDS of the STREAM kernel: the (scale, zero) table of 64 columns, or the reduction buffer of the
+// waves along K (half of them write at a time), which reuses the same bytes.
+int stream_lds_bytes(int bits, int K, int G, int group_size, int act_table, int row_tiles, int waves_k,
+                     int wave_steps)
+{
+    (void)K;
+    long long rows = G;
+    if (!act_table) {
+        const long long span = (long long)waves_k * wave_steps * kstep_of(bits);
+        rows = (span - 1) / group_size + 2;
+        if (rows > G) rows = G;
+    }
+    const long long table = rows * kStreamTableRow;
+    const long long red = (long long)(waves_k / 2) * row_tiles * 16 * 64 * 4;
+    const long long need = table > red ? table : red;
+    return need > (1 << 30) ? (1 << 30) : (int)need;
+}
+
+size_t stream_xpack_bytes(int bits, int steps_pad, int rt_total)
+{
+    // + the depth of the kernel's A ring: its refills run past the end unclamped
+    const size_t blocks = (size_t)steps_pad * (bits == 4 ? 1 : 4) + kStreamRingBlocks;
+    return blocks * (size_t)rt_total * 1024;
+}
+
+size_t stream_gpack_bytes(int bits, int steps_pad, int act_table)
+{
+    const size_t blocks = (size_t)steps_pad * (bits == 4 ? 1 : 4) + kStreamRingBlocks;
+    const size_t bytes = act_table ? blocks * 4 * 8 * sizeof(int32_t)
+                                   : (size_t)(steps_pad + stream_pf(bits)) * 4 * sizeof(int32_t);
+    return (bytes + 255) / 256 * 256;
+}
+
 // LDS of the GROUPED kernel for a K range of kr channels: operand tiles (+ slot masks in the
 // compact two-tile layout) + the reduction buffer of the waves along K.
 int grouped_lds_bytes(int kr, int M, int tpm, int waves_n, int waves_k)
@@ -195,6 +228,63 @@ bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, i
     return false;
 }
 
+// STREAM: exact weights, any g_idx, any M; x pre-packed, waves independent.
+// force_waves is the number of waves along K (1, 2, 4 or 8), 0 = choose.
+int plan_stream(int M, int K, int N, int bits, int gs, int G, int act_order, int force_split, int force_waves,
+                gptq_hip_plan *plan)
+{
+    const int kstep = gptq::kstep_of(bits);
+    const int steps_total = ceil_div(K, kstep);
+    const int pf = gptq::stream_pf(bits);
+    const int rt = M <= 16 ? 1 : (M <= 32 ? 2 : gptq::stream_max_row_tiles());
+    const int m_blocks = ceil_div(M, 16 * rt);
+    const int col_tiles = ceil_div(N, 64);
+    const long long tiles = (long long)col_tiles * m_blocks;
+    const int act_table = gptq::stream_act_table(bits, gs, act_order);
+    if (tiles * (long long)sizeof(int) > (long long)gptq::kCounterBytes) return GPTQ_HIP_ERR_UNSUPPORTED;
+
+    // Waves come from column tiles x M blocks x waves along K inside a workgroup (free: their
+    // tiles meet in LDS) x workgroups along K (dear: the partial tiles cross HBM twice and the
+    // last workgroup of a tile adds them alone).  Eight waves per workgroup while all workgroups
+    // still fit the chip at two waves per SIMD (2048 wave slots), else four; workgroups along K
+    // only when the tiles alone leave most CUs idle.
+    int waves_k = force_waves > 0 ? force_waves : (tiles * 8 <= 2048 ? 8 : 4);
+    while (waves_k > 1 && waves_k * pf > steps_total) waves_k >>= 1;
+    int split = tiles >= 128 ? 1 : ceil_div(256, (int)tiles);
+    int cap = (int)((3LL * K * bits) / (128LL * M));
+    if (cap < 1) cap = 1;
+    if (split > cap) split = cap;
+    if (split > 64) split = 64;
+    if (force_split > 0) split = force_split;
+    if (split * waves_k * pf > steps_total) split = steps_total / (waves_k * pf);
+    if (split < 1) split = 1;
+    int wave_steps = gptq::stream_wave_steps(bits, steps_total, split, waves_k);
+    split = ceil_div(steps_total, wave_steps * waves_k);  // the split actually needed
+    wave_steps = gptq::stream_wave_steps(bits, steps_total, split, waves_k);
+    const int lds = gptq::stream_lds_bytes(bits, K, G, gs, act_table, rt, waves_k, wave_steps);
+    if (lds > 150 * 1024) return GPTQ_HIP_ERR_UNSUPPORTED;  // more groups than the LDS table holds
+
+    plan->kernel = GPTQ_HIP_KERNEL_STREAM;
+    plan->row_tiles = rt;
+    plan->m_blocks = m_blocks;
+    plan->waves_n = 1;
+    plan->waves_k = waves_k;
+    plan->split_k = split;
+    plan->k_chunk = kstep;
+    plan->grid_x = col_tiles;
+    plan->grid_y = split;
+    plan->grid_z = m_blocks;
+    plan->block = 64 * waves_k;
+    plan->lds_bytes = lds;
+    const int steps_pad = split * waves_k * wave_steps;
+    size_t ws = gptq::kCounterBytes;
+    if (split > 1) ws += ((size_t)split * M * N * sizeof(float) + 255) / 256 * 256;
+    ws += gptq::stream_xpack_bytes(bits, steps_pad, rt * m_blocks);
+    ws += gptq::stream_gpack_bytes(bits, steps_pad, act_table);
+    plan->workspace_bytes = ws;
+    return GPTQ_HIP_OK;
+}
+
 }  // namespace
 
 extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, int act_order, gptq_hip_plan *plan)
@@ -211,6 +301,8 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     if (G == 1) act_order = 0;
     if (M <= 2 && plan_grouped(M, K, N, bits, gs, G, act_order, 0, 0, plan)) return GPTQ_HIP_OK;
     memset(plan, 0, sizeof(*plan));
+    if (plan_stream(M, K, N, bits, gs, G, act_order, 0, 0, plan) == GPTQ_HIP_OK) return GPTQ_HIP_OK;
+    memset(plan, 0, sizeof(*plan));
     return plan_gather(M, K, N, bits, G, 0, 0, plan);
 }
 
@@ -220,13 +312,19 @@ extern "C" int gptq_hip_plan_for(int kernel, int M, int K, int N, int bits, int 
     gptq_hip_plan tmp;
     const int rc = gptq_hip_select(M, K, N, bits, group_size, act_order, &tmp);  // argument checks
     if (rc != GPTQ_HIP_OK) return rc;
-    if (!plan || split_k < 0 || (waves_n != 0 && waves_n != 1 && waves_n != 2 && waves_n != 4))
+    if (!plan || split_k < 0 || (waves_n != 0 && waves_n != 1 && waves_n != 2 && waves_n != 4 && waves_n != 8))
         return GPTQ_HIP_ERR_BAD_ARG;
+    if (waves_n == 8 && kernel != GPTQ_HIP_KERNEL_STREAM) return GPTQ_HIP_ERR_BAD_ARG;
     memset(plan, 0, sizeof(*plan));
     const int gs = group_size == -1 ? K : group_size;
     const int G = ceil_div(K, gs);
     if (G == 1) act_order = 0;
     if (kernel == GPTQ_HIP_KERNEL_GATHER) return plan_gather(M, K, N, bits, G, split_k, waves_n, plan);
+    if (kernel == GPTQ_HIP_KERNEL_STREAM) {
+        const int rc2 = plan_stream(M, K, N, bits, gs, G, act_order, split_k, waves_n, plan);
+        if (rc2 != GPTQ_HIP_OK) memset(plan, 0, sizeof(*plan));
+        return rc2;
+    }
     if (kernel == GPTQ_HIP_KERNEL_GROUPED) {
         if (M <= 2 && plan_grouped(M, K, N, bits, gs, G, act_order, split_k, waves_n, plan)) return GPTQ_HIP_OK;
         memset(plan, 0, sizeof(*plan));

@@ -28,6 +28,12 @@ struct Params {
     int waves_n;       // waves of the workgroup along N
     int waves_k;       // waves of the workgroup along K
     int wave_steps;    // steps per wave along K (uniform partition of K made by the host)
+    // STREAM kernel: x re-laid into matrix-instruction fragment order by its pack pass
+    void *xpack;       // [steps_pad * NB][rt_total][64 lanes][8] fp16
+    int32_t *gpack;    // table row byte offsets: per weight [steps_pad * NB][4][8], or per lane block [steps_pad][4]
+    int rt_total;      // 16-row tiles over all M blocks
+    int steps_pad;     // steps walked by all waves of a column tile together (>= steps_total)
+    int act_table;     // 1: one (scale, zero) lookup per weight; 0: one per lane block
 };
 
 // k handled by one wave step: 4 lane groups x (8 | 32) codes
@@ -54,6 +60,34 @@ constexpr int gather_xv(int bits, int row_tiles) { return (bits == 3 && row_tile
 constexpr int gather_gv() { return 8; }
 int gather_lds_bytes(int G, int kc, int xs_rows, int row_tiles, int waves_n, int waves_k);
 
+// STREAM kernel sizing.  A row of its (scale, zero) table: 64 columns x (fp16 scale, fp16 zero),
+// padded by 16 bytes so that lane groups reading rows of different groups spread over the banks.
+static const int kStreamTableRow = 64 * 4 + 16;
+// blocks of 32 channels the A fragments and table offsets run ahead
+static const int kStreamRingBlocks = 4;
+// steps the weight loads run ahead; every wave walks a multiple of it
+constexpr int stream_pf(int bits) { return bits == 4 ? 4 : 2; }
+inline int stream_wave_steps(int bits, int steps_total, int split_k, int waves_k)
+{
+    const int pf = stream_pf(bits);
+    const int per_wave = (steps_total + split_k * waves_k - 1) / (split_k * waves_k);
+    return (per_wave + pf - 1) / pf * pf;
+}
+// tallest tile of a STREAM wave in 16-row tiles: 64 rows keep a wave under 256 registers, so two
+// waves share a SIMD; taller problems take more M blocks
+constexpr int stream_max_row_tiles() { return 4; }
+// one lookup per weight unless groups are contiguous and no narrower than a lane block
+inline int stream_act_table(int bits, int group_size, int act_order)
+{
+    return (act_order || group_size % (bits == 4 ? 8 : 32) != 0) ? 1 : 0;
+}
+int stream_lds_bytes(int bits, int K, int G, int group_size, int act_table, int row_tiles, int waves_k,
+                     int wave_steps);
+// bytes of the packed x and of the packed table offsets, each rounded up to 256
+size_t stream_xpack_bytes(int bits, int steps_pad, int rt_total);
+size_t stream_gpack_bytes(int bits, int steps_pad, int act_table);
+
+int launch_stream(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
 int launch_gather(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
 int launch_grouped(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
 int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,

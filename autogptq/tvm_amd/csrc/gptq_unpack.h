@@ -183,6 +183,31 @@ GPTQ_HD void biased3(uint32_t w0, uint32_t w1, uint32_t w2, u4 out[4], uint32_t 
     }
 }
 
+// One quarter of biased3: the four registers (8 codes) of MFMA block nb of the 3-word block.
+GPTQ_HD void biased3_block(uint32_t w0, uint32_t w1, uint32_t w2, int nb, u4 &out, uint32_t magic_even,
+                           uint32_t magic_odd)
+{
+    uint32_t lo, hi;
+    if (nb == 0) {
+        lo = w0;
+        hi = w0 >> 6;
+    } else if (nb == 1) {
+        lo = funnel(w1, w0, 12);
+        hi = funnel(w2, w1, 4);
+    } else if (nb == 2) {
+        lo = funnel(w2, w1, 10);
+        hi = funnel(w2, w1, 16);
+    } else {
+        lo = w2 >> 8;
+        const uint32_t t = w2 >> 14;
+        hi = (t << 12) | t;
+    }
+    out[0] = and_or(lo, 0x001c0007u, magic_even);
+    out[1] = and_or(lo, 0x00e00038u, magic_odd);
+    out[2] = and_or(hi, 0x001c0007u, magic_even);
+    out[3] = and_or(hi, 0x00e00038u, magic_odd);
+}
+
 // The dequantised weight of the reference (qlinear.py:242): fp16 scale times the
 // integer (q - zero), rounded once.  (q - zero) is exact in fp16, so one fp16 multiply
 // is that rounding, signed zeros and subnormals included.  (Going through an fp32

@@ -36,9 +36,10 @@ typedef enum gptq_hip_status {
 
 /* kernel families the dispatcher chooses between */
 enum {
-    GPTQ_HIP_KERNEL_GATHER = 1, /* per-weight scale/zero gather, exact fp16 weights; any g_idx, any M */
-    GPTQ_HIP_KERNEL_GROUPED = 2, /* rows expanded by group, scales applied once per group; small G*M */
-    GPTQ_HIP_KERNEL_BLOCKED = 3 /* contiguous groups (g_idx == NULL), scales applied at group ends */
+    GPTQ_HIP_KERNEL_GATHER = 1, /* exact fp16 weights, x staged through LDS by the workgroup; any g_idx, any M */
+    GPTQ_HIP_KERNEL_GROUPED = 2, /* rows expanded by group, scales applied once per group; M <= 2, few groups */
+    GPTQ_HIP_KERNEL_STREAM = 3  /* exact fp16 weights, x pre-packed into fragment order (always needs the
+                                   workspace), independent waves; any g_idx, any M */
 };
 
 /* What the dispatcher decided for one problem; filled by gptq_hip_select. */
@@ -49,11 +50,11 @@ typedef struct gptq_hip_plan {
     int waves_n;            /* waves of a workgroup laid along N (64 columns each) */
     int waves_k;            /* waves of a workgroup laid along K */
     int split_k;            /* workgroups sharing one column tile; >1 uses the workspace */
-    int k_chunk;            /* input channels staged in LDS at a time */
+    int k_chunk;            /* input channels staged in LDS at a time (STREAM: per wave step) */
     int grid_x, grid_y, grid_z;
     int block;              /* threads per workgroup */
     int lds_bytes;          /* dynamic LDS per workgroup */
-    size_t workspace_bytes; /* 0 when split_k == 1 */
+    size_t workspace_bytes; /* 0 when the plan needs none (GATHER / GROUPED with split_k == 1) */
 } gptq_hip_plan;
 
 /*

@@ -61,7 +61,7 @@ def test_select_plans_are_consistent(bits, M, KN, gs):
         gs = 32
     for act in (False, True):
         p = _lib.select(M, K, N, bits, gs, act)
-        assert p.kernel in (_lib.KERNEL_GATHER, _lib.KERNEL_GROUPED, _lib.KERNEL_BLOCKED)
+        assert p.kernel in (_lib.KERNEL_GATHER, _lib.KERNEL_GROUPED, _lib.KERNEL_STREAM)
         if p.kernel == _lib.KERNEL_GROUPED:
             assert M <= 2 and 1 <= p.row_tiles <= 6 and p.m_blocks == 1
         else:
@@ -78,6 +78,9 @@ def test_select_plans_are_consistent(bits, M, KN, gs):
             assert p.workspace_bytes >= p.split_k * M * N * 4
             # partial sums stay in proportion to the packed weights (or there is a single split)
             assert p.split_k * M * N * 4 <= 3 * K * N * bits // 8 or p.split_k == 2
+        elif p.kernel == _lib.KERNEL_STREAM:
+            # always holds the packed x: at least one 16-row tile over all of K
+            assert p.workspace_bytes >= 16 * K * 2
         else:
             assert p.workspace_bytes == 0
         lib = _lib.lib()

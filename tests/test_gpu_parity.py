@@ -139,6 +139,40 @@ def test_gather_forced_split_k(dev, bits, split, M, waves):
 
 @pytest.mark.parametrize("bits", [3, 4])
 @pytest.mark.parametrize("desc_act", [False, True])
+@pytest.mark.parametrize("waves,split", [(1, 1), (2, 1), (4, 1), (8, 1), (1, 3), (4, 2), (8, 2)])
+@pytest.mark.parametrize("M", [3, 20, 40, 130])
+def test_stream_forced_waves_and_split_k(dev, bits, desc_act, waves, split, M):
+    # K = 4096 gives every (waves, split) at least one whole ring of steps per wave; N = 352 ends
+    # in a partly filled column tile; M covers every tile height and ragged last M blocks
+    K, N = 4096, 352
+    L = layer(700 + waves * 10 + split, K, N, bits, 128, desc_act, M=M, bias=True)
+    D = to_dev(L, dev)
+    plan = _lib.plan_for(_lib.KERNEL_STREAM, M, K, N, bits, 128, desc_act, split_k=split, waves_n=waves)
+    assert plan.kernel == _lib.KERNEL_STREAM and plan.waves_k == waves and plan.split_k == split
+    y1 = run_gemm(D, plan=plan)
+    y2 = run_gemm(D, plan=plan)  # same workspace again: counters left at zero, packed x rewritten
+    assert_close(y1, expected_output(L), f"waves={waves} split={split}")
+    assert_tight(y1, expected_output(L), f"waves={waves} split={split}")
+    assert torch.equal(y1, y2), "result changed between two identical calls"
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("K,N,gs", [(32, 32, 32), (160, 96, -1), (1024, 416, 32), (2048, 1056, 256), (1056, 64, 16)])
+@pytest.mark.parametrize("M", [3, 33])
+def test_stream_matches_gather(dev, bits, K, N, gs, M):
+    # two independent kernels, same exact fp16 weights: they may differ only in summation order
+    for desc_act in (False, True):
+        L = layer(800 + M, K, N, bits, gs, desc_act, M=M)
+        D = to_dev(L, dev)
+        a = run_gemm(D, plan=_lib.plan_for(_lib.KERNEL_STREAM, M, K, N, bits, gs, desc_act))
+        b = run_gemm(D, plan=_lib.plan_for(_lib.KERNEL_GATHER, M, K, N, bits, gs, desc_act))
+        assert_close(a, expected_output(L), "stream")
+        assert_close(b, expected_output(L), "gather")
+        assert_close(a, b.float().cpu(), "stream vs gather")
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("desc_act", [False, True])
 @pytest.mark.parametrize("M", [1, 2])
 @pytest.mark.parametrize("split", [1, 2, 5, 16])
 def test_grouped_forced_split_k(dev, bits, desc_act, M, split):
