@@ -70,3 +70,63 @@ def test_quantlinear_pack_round_trips_through_the_oracle(bits):
     w16 = orc.dequant_ref(q.qweight, q.qzeros, q.scales, q.g_idx, bits)
     assert torch.equal(w16, W.t().half())
     assert torch.equal(q.bias, lin.bias.half())
+
+
+# ---------------------------------------------------------------------------------------------
+# Golden vectors written by the reference's own QuantLinear.pack (tests/golden/make_pack_vectors.py):
+# real-valued weights, so the rounding of (W + scale * zero) / scale is what is being pinned.
+def _golden_cases():
+    import os
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "pack_vectors.npz")
+    data = np.load(path, allow_pickle=False)
+    names = sorted({k.rsplit(".", 1)[0] for k in data.files})
+    return data, names
+
+
+_GOLD, _GOLD_NAMES = _golden_cases()
+
+
+@pytest.mark.parametrize("name", _GOLD_NAMES)
+def test_quantlinear_pack_matches_reference_vectors(name):
+    from autogptq.tvm_amd import QuantLinear
+
+    bits, K, N, gs, act, has_bias = (int(v) for v in _GOLD[name + ".meta"])
+    linear = torch.nn.Linear(K, N, bias=bool(has_bias))
+    with torch.no_grad():
+        linear.weight.copy_(torch.from_numpy(_GOLD[name + ".weight"]))
+        if has_bias:
+            linear.bias.copy_(torch.from_numpy(_GOLD[name + ".bias_in"]))
+    q = QuantLinear(bits, gs, K, N, bool(has_bias))
+    q.pack(linear, torch.from_numpy(_GOLD[name + ".scales_in"]).clone(),
+           torch.from_numpy(_GOLD[name + ".zeros_in"]).clone(), torch.from_numpy(_GOLD[name + ".g_idx"]).clone())
+    assert np.array_equal(q.qweight.numpy(), _GOLD[name + ".qweight"])
+    assert np.array_equal(q.qzeros.numpy(), _GOLD[name + ".qzeros"])
+    assert np.array_equal(q.scales.numpy().view(np.uint16), _GOLD[name + ".scales"])
+    assert np.array_equal(q.g_idx.numpy(), _GOLD[name + ".g_idx"])
+    if has_bias:
+        assert np.array_equal(q.bias.detach().numpy().view(np.uint16), _GOLD[name + ".bias"])
+
+
+@pytest.mark.parametrize("name", _GOLD_NAMES)
+def test_oracle_unpacks_reference_packed_tensors(name):
+    """The oracle's unpack and dequant applied to tensors the reference packed: the codes must be
+    round((W + s z) / s) and the dequantised weight within half a quantisation step of W wherever
+    the code did not saturate."""
+    bits, K, N, gs, act, has_bias = (int(v) for v in _GOLD[name + ".meta"])
+    qweight, qzeros = _GOLD[name + ".qweight"], _GOLD[name + ".qzeros"]
+    scales16 = _GOLD[name + ".scales"].view(np.float16)
+    g_idx = _GOLD[name + ".g_idx"]
+    codes = orc.unpack_bitstream(qweight, bits, axis=0)            # [K, N]
+    zeros = orc.unpack_bitstream(qzeros, bits, axis=1) + 1         # [G, N]
+    assert np.array_equal(zeros, _GOLD[name + ".zeros_in"].T.astype(np.int64))
+    W = _GOLD[name + ".weight"].T.astype(np.float32)               # [K, N]
+    s = scales16.astype(np.float32)[g_idx]                          # [K, N]
+    z = zeros[g_idx].astype(np.float32)
+    s_in = _GOLD[name + ".scales_in"].T.astype(np.float32)[g_idx]
+    want = np.rint((W + z * s_in) / s).astype(np.int64)             # the reference's expression
+    assert want.min() >= 0 and want.max() < (1 << bits)             # the fixture keeps codes in range
+    assert np.array_equal(codes, want)
+    deq = orc.dequant_ref(torch.from_numpy(qweight), torch.from_numpy(qzeros),
+                          torch.from_numpy(scales16.copy()), torch.from_numpy(g_idx), bits).float().numpy()
+    assert np.all(np.abs(deq - W) <= 0.5 * s * 1.01 + 1e-3)         # within half a quantisation step
