@@ -76,7 +76,7 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
         const int kr = pl.k_chunk;
         if ((long long)kr * pl.split_k < (long long)steps_total * kstep) return GPTQ_HIP_ERR_BAD_ARG;
         const int tpm = pl.row_tiles / M;
-        const int need_tpm = gptq::grouped_tpm(gptq::grouped_groups(kr, gs, G, act_order), M);
+        const int need_tpm = gptq::grouped_tpm(gptq::grouped_groups(kr / pl.waves_k, gs, G, act_order), M);
         if (need_tpm == 0 || tpm != need_tpm) return GPTQ_HIP_ERR_UNSUPPORTED;
         if (pl.lds_bytes < gptq::grouped_lds_bytes(kr, M, tpm, pl.waves_n, pl.waves_k)) return GPTQ_HIP_ERR_BAD_ARG;
         return GPTQ_HIP_OK;

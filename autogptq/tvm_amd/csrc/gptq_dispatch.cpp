@@ -203,7 +203,8 @@ bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, i
         const int wg_steps = wave_steps * waves_k;
         const int split = ceil_div(steps_total, wg_steps);
         const int kr = wg_steps * kstep;
-        const int tpm = gptq::grouped_tpm(gptq::grouped_groups(kr, gs, G, act_order), M);
+        // rows are counted per wave: the groups one wave's K range can touch
+        const int tpm = gptq::grouped_tpm(gptq::grouped_groups(wave_steps * kstep, gs, G, act_order), M);
         if (tpm == 0) {
             if (act_order) return false;  // the group count does not shrink with the K range
             continue;

@@ -21,7 +21,7 @@
 // the MFMA wants it: a tile is 16 rows x 8 slots of fp16 = 256 bytes, lane i reads its
 // 16 bytes at i*16.  It is zero-filled and then scattered into, one 2-byte store per
 // (m, k).  Two layouts:
-//   dense   : one tile per 16 groups (row = g - g_base), M * TPM tiles per 8 slots;
+//   dense   : one tile per 16 groups (row = g - first group of the consuming wave), M * TPM tiles per 8 slots;
 //   compact : for 17..32 groups, ONE tile per m with row = g % 16, plus a 16-byte mask
 //             per 8 slots saying which slots belong to groups < 16.  The two row tiles
 //             are that tile AND mask / AND NOT mask: half the LDS, so K = 4096 with 32
@@ -76,7 +76,9 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     const int kspan = wg_steps * F::KSTEP;
     const int prows = p.K / (BITS == 4 ? 8 : 32);  // packed rows (int4) or 3-word blocks (int3)
     // contiguous groups: only those inside this K range need rows, counted from the first one
-    const int g_base = p.g_idx ? 0 : k_base / p.group_size;
+    // (rows are counted per wave: a wave's K range meets few groups, so one row tile usually holds them)
+    const int wave_k = p.wave_steps * F::KSTEP;  // channels per wave
+    const int g_base = p.g_idx ? 0 : (ws * F::KSTEP) / p.group_size;
     __shared__ int last_flag;
 
     const _Float16 *x = (const _Float16 *)p.x;
@@ -178,8 +180,9 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     // A thread always owns quads with the same position inside a lane block (kc % KLANE is
     // 4 * (tid % (KLANE / 4)) in every pass because the block size is a multiple of 8), so the
     // four slots of its quad are fixed: qslot[e], looked up once at the top of the kernel.
-    auto scatter = [&](int m, int kc, int slot, int g, _Float16 xv) {
-        const int r = min(max(g, 0), p.G - 1) - g_base;  // row of this group
+    // gb: first group of the wave that will consume channel kc (0 under a g_idx)
+    auto scatter = [&](int m, int kc, int slot, int g, int gb, _Float16 xv) {
+        const int r = min(max(g, 0), p.G - 1) - gb;  // row of this group
         const int rr = min(max(r, 0), 16 * TPM - 1);
         const int b8 = (kc / F::KLANE) * F::NB + (slot >> 3);
         if constexpr (COMPACT) {
@@ -196,8 +199,9 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
             const int m = M == 1 ? 0 : idx / qpr;
             const int kc = 4 * (idx - m * qpr);
             if (k_base + kc < p.K) {
+                const int gb = p.g_idx ? 0 : (k_base + (kc / wave_k) * wave_k) / p.group_size;
 #pragma unroll
-                for (int e = 0; e < 4; e++) scatter(m, kc + e, qslot[e], gq[ps][e], xq[ps][e]);
+                for (int e = 0; e < 4; e++) scatter(m, kc + e, qslot[e], gq[ps][e], gb, xq[ps][e]);
             }
         }
     }
@@ -207,10 +211,11 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         const int k = k_base + kc;
         if (k < p.K) {
             const h4 xv = *(const h4 *)(x + (size_t)m * p.K + k);
+            const int gb = p.g_idx ? 0 : (k_base + (kc / wave_k) * wave_k) / p.group_size;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int g = p.g_idx ? p.g_idx[k + e] : (k + e) / p.group_size;
-                scatter(m, kc + e, qslot[e], g, xv[e]);
+                scatter(m, kc + e, qslot[e], g, gb, xv[e]);
             }
         }
     }
