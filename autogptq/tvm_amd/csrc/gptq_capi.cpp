@@ -94,7 +94,7 @@ extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const i
     if (!x || !y || !plan || M < 1) return GPTQ_HIP_ERR_BAD_ARG;
     int rc = check_common(qweight, qzeros, scales, K, N, bits, group_size);
     if (rc != GPTQ_HIP_OK) return rc;
-    if (!aligned(x, 16) || !aligned(y, 8) || (bias && !aligned(bias, 8)) || (g_idx && !aligned(g_idx, 4)))
+    if (!aligned(x, 16) || !aligned(y, 8) || (bias && !aligned(bias, 8)) || (g_idx && !aligned(g_idx, 16)))
         return GPTQ_HIP_ERR_BAD_ARG;
     const int gs = group_size == -1 ? K : group_size;
     const int G = (K + gs - 1) / gs;
@@ -135,6 +135,9 @@ extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const i
     p.rt_total = 0;
     p.steps_pad = 0;
     p.act_table = 0;
+    p.direct = 0;
+    p.gdiv_magic = 0;
+    p.gdiv_add = 0;
     if (plan->kernel == GPTQ_HIP_KERNEL_STREAM) {
         // workspace: counters | partial tiles (split_k > 1) | packed x | packed table offsets
         p.wave_steps = gptq::stream_wave_steps(bits, p.steps_total, plan->split_k, plan->waves_k);
@@ -143,6 +146,27 @@ extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const i
         p.act_table = gptq::stream_act_table(bits, gs, act_order);
         const size_t part =
             plan->split_k > 1 ? ((size_t)plan->split_k * M * N * sizeof(float) + 255) / 256 * 256 : 0;
+        p.direct = gptq::stream_direct(bits, K, plan->row_tiles, p.act_table, g_idx != nullptr);
+        p.gdiv_magic = 0;
+        p.gdiv_add = 0;
+        if (p.direct) {
+            if (!p.act_table) {
+                // group of lane block r = r / d, d = lane blocks per group, as a multiply-high
+                const uint32_t d = (uint32_t)(gs / (bits == 4 ? 8 : 32));
+                if (d == 1) {
+                    p.gdiv_add = 1;
+                } else {
+                    p.gdiv_magic = (uint32_t)((1ull << 32) / d) + 1u;
+                }
+            }
+            if (plan->split_k > 1) {
+                const size_t need = gptq::kCounterBytes + part;
+                if (!workspace || workspace_bytes < need || !aligned(workspace, 16)) return GPTQ_HIP_ERR_WORKSPACE;
+                p.counters = (int *)workspace;
+                p.partial = (float *)((char *)workspace + gptq::kCounterBytes);
+            }
+            return gptq::launch_stream(p, bits, *plan, stream);
+        }
         const size_t xb = gptq::stream_xpack_bytes(bits, p.steps_pad, p.rt_total);
         const size_t gb = gptq::stream_gpack_bytes(bits, p.steps_pad, p.act_table);
         if (xb >= (1ull << 32)) return GPTQ_HIP_ERR_UNSUPPORTED;  // the kernel uses 32-bit byte offsets

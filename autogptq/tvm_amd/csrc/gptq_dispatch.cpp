@@ -191,7 +191,7 @@ bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, i
     const int lds_cap = 144 * 1024;
     // a column tile per workgroup and no split is best (nothing crosses workgroups) unless
     // that leaves most of the 256 CUs idle
-    int want = force_split > 0 ? force_split : (col_tiles >= 128 ? 1 : ceil_div(192, col_tiles));
+    int want = force_split > 0 ? force_split : (col_tiles >= 128 ? 1 : ceil_div(256, col_tiles));
     if (want > steps_total) want = steps_total;
     for (int want_split = want; want_split <= steps_total && want_split <= 256; want_split++) {
         if (force_split > 0 && want_split != want) return false;
@@ -280,8 +280,12 @@ int plan_stream(int M, int K, int N, int bits, int gs, int G, int act_order, int
     const int steps_pad = split * waves_k * wave_steps;
     size_t ws = gptq::kCounterBytes;
     if (split > 1) ws += ((size_t)split * M * N * sizeof(float) + 255) / 256 * 256;
-    ws += gptq::stream_xpack_bytes(bits, steps_pad, rt * m_blocks);
-    ws += gptq::stream_gpack_bytes(bits, steps_pad, act_table);
+    if (gptq::stream_direct(bits, K, rt, act_table, act_order)) {
+        if (split == 1) ws = 0;  // no pack pass, no partial tiles: nothing to hold
+    } else {
+        ws += gptq::stream_xpack_bytes(bits, steps_pad, rt * m_blocks);
+        ws += gptq::stream_gpack_bytes(bits, steps_pad, act_table);
+    }
     plan->workspace_bytes = ws;
     return GPTQ_HIP_OK;
 }
@@ -300,7 +304,10 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     const int G = ceil_div(K, gs);
     // one group for the whole matrix: g_idx carries no information
     if (G == 1) act_order = 0;
-    if (M <= 2 && plan_grouped(M, K, N, bits, gs, G, act_order, 0, 0, plan)) return GPTQ_HIP_OK;
+    // GROUPED for decoding (M = 1); for M = 2 only where a workgroup holds all of K, since its
+    // operand in LDS doubles with M and the cross-workgroup sum costs more than STREAM's pack pass
+    if (M <= 2 && plan_grouped(M, K, N, bits, gs, G, act_order, 0, 0, plan) && (M == 1 || plan->split_k == 1))
+        return GPTQ_HIP_OK;
     memset(plan, 0, sizeof(*plan));
     if (plan_stream(M, K, N, bits, gs, G, act_order, 0, 0, plan) == GPTQ_HIP_OK) return GPTQ_HIP_OK;
     memset(plan, 0, sizeof(*plan));

@@ -32,7 +32,7 @@ namespace gptq {
 
 #ifdef GPTQ_PHASE_TIMES
 __device__ long long g_phase[16 * 8192];
-#define PHASE(i) do { if (lane == 0) g_phase[((size_t)blockIdx.x * 8 + wave) * 16 + (i)] = clock64(); } while (0)
+#define PHASE(i) do { if (lane == 0) g_phase[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 8 + wave) * 16 + (i)] = clock64(); } while (0)
 #else
 #define PHASE(i) do { } while (0)
 #endif
@@ -399,7 +399,11 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         return;
     }
     if (writer) store_partial(p.partial + ((size_t)split * M + f_m) * p.N + f_n, sum);
-    if (!arrive_last(p.counters + blockIdx.x, p.split_k, &last_flag)) return;
+    if (!arrive_last(p.counters + blockIdx.x, p.split_k, &last_flag)) {
+        PHASE(7);
+        return;
+    }
+    PHASE(11);
     if (writer) {
         f4 total = bv;
         for (int s = 0; s < p.split_k; s++) total += load_partial(p.partial + ((size_t)s * M + f_m) * p.N + f_n);
@@ -408,6 +412,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         for (int c = 0; c < 4; c++) o[c] = (_Float16)total[c];
         *(h4 *)(y + (size_t)f_m * p.N + f_n) = o;
     }
+    PHASE(7);
 }
 
 template <int BITS, int M, int TPM, bool COMPACT>

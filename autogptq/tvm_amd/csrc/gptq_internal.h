@@ -34,6 +34,9 @@ struct Params {
     int rt_total;      // 16-row tiles over all M blocks
     int steps_pad;     // steps walked by all waves of a column tile together (>= steps_total)
     int act_table;     // 1: one (scale, zero) lookup per weight; 0: one per lane block
+    int direct;        // 1: no pack pass, the kernel reads x and g_idx itself (M <= 16)
+    uint32_t gdiv_magic;  // direct, contiguous groups: group of lane block r = umulhi(r, magic) + (add ? r : 0)
+    int gdiv_add;
 };
 
 // k handled by one wave step: 4 lane groups x (8 | 32) codes
@@ -80,6 +83,13 @@ constexpr int stream_max_row_tiles() { return 4; }
 inline int stream_act_table(int bits, int group_size, int act_order)
 {
     return (act_order || group_size % (bits == 4 ? 8 : 32) != 0) ? 1 : 0;
+}
+// The pack pass can be skipped for one row tile (M <= 16): the kernel then reads x rows and g_idx
+// itself.  Needs a g_idx whenever the lookup is per weight, and lane-block numbers below 2^16
+// (exactness of its multiply-high division).
+inline int stream_direct(int bits, int K, int row_tiles, int act_table, int has_g_idx)
+{
+    return row_tiles == 1 && (!act_table || has_g_idx) && K / (bits == 4 ? 8 : 32) < 65536;
 }
 int stream_lds_bytes(int bits, int K, int G, int group_size, int act_table, int row_tiles, int waves_k,
                      int wave_steps);

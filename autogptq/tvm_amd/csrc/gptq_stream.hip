@@ -113,6 +113,166 @@ __global__ __launch_bounds__(256) void pack_kernel(const Params p)
     }
 }
 
+
+// ---- pieces shared by the two matmul kernels of this file ---------------------------------------
+
+// Stages (scale, zero) of groups g_lo .. g_hi x the 64 columns from n_blk on into LDS rows of
+// kStreamTableRow bytes (row 0 = g_lo).  Four items per thread at a time so their loads overlap.
+template <int BITS>
+__device__ __forceinline__ void stage_table(const Params &p, int g_lo, int g_hi, int n_blk, int tid)
+{
+    constexpr int TROW = kStreamTableRow;
+    const _Float16 *scales = (const _Float16 *)p.scales;
+    const int zwords = p.N / 32 * BITS;
+    const int tab_items = (g_hi - g_lo + 1) * 16;  // four columns of one group each
+    for (int base = tid; base < tab_items; base += 4 * (int)blockDim.x) {
+        h4 s4[4];
+        uint32_t za[4], zb[4];
+        int nn[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int idx = min(base + u * (int)blockDim.x, tab_items - 1);
+            const int gr = idx >> 4;
+            nn[u] = min(n_blk + 4 * (idx & 15), p.N - 4);
+            const uint32_t g = (uint32_t)(g_lo + gr);
+            s4[u] = *(const h4 *)((const char *)scales + (g * (uint32_t)p.N + (uint32_t)nn[u]) * 2u);
+            load_zero_words<BITS>(p.qzeros, g * (uint32_t)zwords, nn[u], za[u], zb[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int idx = base + u * (int)blockDim.x;
+            if (idx < tab_items) {
+                float z[4];
+                zeros_from_words<BITS>(za[u], zb[u], nn[u], z);
+                u4 e;
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const h2 sz = {s4[u][c], (_Float16)z[c]};
+                    e[c] = as_u32(sz);
+                }
+                *(u4 *)(smem + (size_t)(idx >> 4) * TROW + (idx & 15) * 16) = e;
+            }
+        }
+    }
+}
+
+// B operands of one block: the reference's weights fp16(scale * (q - zero)) of 8 slots x 4 column
+// sets from the biased codes bq[c] (base + q).  (base + q) - (base + zero) is exact, so the one
+// rounding is the product's.  ent[s][c]: (scale, zero) of slot s (ACT) / erow[c]: of all slots.
+template <int BITS, bool ACT>
+__device__ __forceinline__ void dequant_block(const u4 (&bqn)[4], const u4 (&ent)[8], const u4 &erow, h8 (&bop)[4])
+{
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        u4 wv;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            // (scale, zero) of the two slots of register r: low halves / high halves
+            const uint32_t ea = ACT ? ent[2 * r][c] : erow[c];
+            const uint32_t eb = ACT ? ent[2 * r + 1][c] : erow[c];
+            const h2 s2 = as_h2(__builtin_amdgcn_perm(eb, ea, 0x05040100u));
+            const h2 z2 = as_h2(__builtin_amdgcn_perm(eb, ea, 0x07060302u));
+            const float ba = BITS == 4 ? BASE4[2 * r] : BASE3[2 * r];
+            const float bb = BITS == 4 ? BASE4[2 * r + 1] : BASE3[2 * r + 1];
+            const h2 zb = z2 + (h2){(_Float16)ba, (_Float16)bb};  // exact: small integers
+            wv[r] = as_u32((as_h2(bqn[c][r]) - zb) * s2);
+        }
+        bop[c] = __builtin_bit_cast(h8, wv);
+    }
+}
+
+// The waves of the workgroup add their tiles through LDS in a fixed tree; wave 0 ends up with the sum.
+template <int RT>
+__device__ __forceinline__ void reduce_waves(f4 (&acc)[RT][4], int wave, int WK, int lane)
+{
+    f4 *red = (f4 *)smem;  // [WK / 2][RT * 4 tiles][64 lanes] of f4, reuses the table's bytes
+    for (int stride = WK >> 1; stride >= 1; stride >>= 1) {
+        lds_barrier();  // the table, or the previous round, is no longer read
+        if (wave >= stride && wave < 2 * stride) {
+            f4 *dst = red + (size_t)(wave - stride) * (RT * 4) * 64 + lane;
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) dst[(rt * 4 + c) * 64] = acc[rt][c];
+        }
+        lds_barrier();
+        if (wave < stride) {
+            const f4 *src = red + (size_t)wave * (RT * 4) * 64 + lane;
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) acc[rt][c] += src[(rt * 4 + c) * 64];
+        }
+    }
+}
+
+// Epilogue of wave 0: acc[rt][c][v] is y[m0 + 16 rt + 4 q + v][n0 + c]; bias, fp16, or the
+// split-K exchange through the workspace.  Every thread of the workgroup calls it.
+template <int RT>
+__device__ __forceinline__ void write_out(const Params &p, f4 (&acc)[RT][4], bool owner, int m0, int rows_here,
+                                          int n0, int lq, int split, int *last_flag)
+{
+    const _Float16 *bias = (const _Float16 *)p.bias;
+    f4 bv = {0.f, 0.f, 0.f, 0.f};
+    if (bias && owner) {
+        const h4 b4 = *(const h4 *)(bias + n0);
+        bv = (f4){(float)b4[0], (float)b4[1], (float)b4[2], (float)b4[3]};
+    }
+    _Float16 *y = (_Float16 *)p.y;
+    if (p.split_k == 1) {
+        if (owner) {
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int row = 16 * rt + 4 * lq + v;
+                    if (row < rows_here) {
+                        h4 o;
+#pragma unroll
+                        for (int c = 0; c < 4; c++) o[c] = (_Float16)(acc[rt][c][v] + bv[c]);
+                        *(h4 *)(y + (size_t)(m0 + row) * p.N + n0) = o;
+                    }
+                }
+            }
+        }
+        return;
+    }
+    if (owner) {
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int row = 16 * rt + 4 * lq + v;
+                if (row < rows_here) {
+                    const f4 o = {acc[rt][0][v], acc[rt][1][v], acc[rt][2][v], acc[rt][3][v]};
+                    store_partial(p.partial + ((size_t)split * p.M + (m0 + row)) * p.N + n0, o);
+                }
+            }
+        }
+    }
+    int *counter = p.counters + blockIdx.z * gridDim.x + blockIdx.x;
+    if (!arrive_last(counter, p.split_k, last_flag)) return;
+    if (owner) {
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int row = 16 * rt + 4 * lq + v;
+                if (row < rows_here) {
+                    f4 sum = bv;
+                    for (int s = 0; s < p.split_k; s++) {
+                        sum += load_partial(p.partial + ((size_t)s * p.M + (m0 + row)) * p.N + n0);
+                    }
+                    h4 o;
+#pragma unroll
+                    for (int c = 0; c < 4; c++) o[c] = (_Float16)sum[c];
+                    *(h4 *)(y + (size_t)(m0 + row) * p.N + n0) = o;
+                }
+            }
+        }
+    }
+}
+
 // Global loads return in order (one counter), so a wait for any load also waits for every older
 // one.  The main loop therefore issues its loads in the order it consumes them and keeps all of
 // them the same distance ahead: in step s the weights of step s + PF are requested first, then,
@@ -210,42 +370,11 @@ __global__ __launch_bounds__(512) void stream_kernel(const Params p)
 
     // ---- (scale, zero) table of the 64 columns: all groups under a g_idx, else those of the
     //      workgroup's K range (row 0 = the first of them) ---------------------------------
-    const _Float16 *scales = (const _Float16 *)p.scales;
-    const int zwords = p.N / 32 * BITS;
     const int k_lo = min(s_begin * F::KSTEP, p.K - 1);
     const int k_hi = min((s_begin + WK * p.wave_steps) * F::KSTEP, p.K) - 1;
     const int g_lo = ACT ? 0 : k_lo / p.group_size;
     const int g_hi = ACT ? p.G - 1 : min(p.G - 1, max(k_hi, k_lo) / p.group_size);
-    const int tab_items = (g_hi - g_lo + 1) * 16;  // four columns of one group each
-    for (int base = tid; base < tab_items; base += 4 * (int)blockDim.x) {
-        h4 s4[4];
-        uint32_t za[4], zb[4];
-        int nn[4];
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int idx = min(base + u * (int)blockDim.x, tab_items - 1);
-            const int gr = idx >> 4;
-            nn[u] = min(n_blk + 4 * (idx & 15), p.N - 4);
-            const uint32_t g = (uint32_t)(g_lo + gr);
-            s4[u] = *(const h4 *)((const char *)scales + (g * (uint32_t)p.N + (uint32_t)nn[u]) * 2u);
-            load_zero_words<BITS>(p.qzeros, g * (uint32_t)zwords, nn[u], za[u], zb[u]);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int idx = base + u * (int)blockDim.x;
-            if (idx < tab_items) {
-                float z[4];
-                zeros_from_words<BITS>(za[u], zb[u], nn[u], z);
-                u4 e;
-#pragma unroll
-                for (int c = 0; c < 4; c++) {
-                    const h2 sz = {s4[u][c], (_Float16)z[c]};
-                    e[c] = as_u32(sz);
-                }
-                *(u4 *)(smem + (size_t)(idx >> 4) * TROW + (idx & 15) * 16) = e;
-            }
-        }
-    }
+    stage_table<BITS>(p, g_lo, g_hi, n_blk, tid);
     const int tab_bias = col_l * 4 - g_lo * TROW;  // this lane's four columns, rows counted from g_lo
 
     f4 acc[RT][4];
@@ -288,45 +417,20 @@ __global__ __launch_bounds__(512) void stream_kernel(const Params p)
                         biased3_block(w[u][0][c], w[u][1][c], w[u][2][c], nb, bq[c][nb], magic_a, magic_b);
                 }
                 h8 bop[4];
+                u4 ent[8];
                 if constexpr (ACT) {
-                    u4 ent[8];
 #pragma unroll
                     for (int s = 0; s < 8; s++) {
                         const uint32_t off = s < 4 ? go[slot][0][s & 3] : go[slot][1][s & 3];
                         ent[s] = *(const u4 *)(smem + (off + (uint32_t)tab_bias));
                     }
                     load_go(b + AD, go[slot]);
+                }
+                {
+                    u4 bqn[4];
 #pragma unroll
-                    for (int c = 0; c < 4; c++) {
-                        u4 wv;
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            // (scale, zero) of the two slots of register r: low halves / high halves
-                            const h2 s2 = as_h2(__builtin_amdgcn_perm(ent[2 * r + 1][c], ent[2 * r][c], 0x05040100u));
-                            const h2 z2 = as_h2(__builtin_amdgcn_perm(ent[2 * r + 1][c], ent[2 * r][c], 0x07060302u));
-                            const float ba = BITS == 4 ? BASE4[2 * r] : BASE3[2 * r];
-                            const float bb = BITS == 4 ? BASE4[2 * r + 1] : BASE3[2 * r + 1];
-                            const h2 zb = z2 + (h2){(_Float16)ba, (_Float16)bb};  // exact: small integers
-                            wv[r] = as_u32((as_h2(bq[c][nb][r]) - zb) * s2);      // exact difference, one rounding
-                        }
-                        bop[c] = __builtin_bit_cast(h8, wv);
-                    }
-                } else {
-#pragma unroll
-                    for (int c = 0; c < 4; c++) {
-                        const uint32_t e = erow[c];
-                        const h2 s2 = as_h2(__builtin_amdgcn_perm(e, e, 0x05040100u));
-                        const h2 z2 = as_h2(__builtin_amdgcn_perm(e, e, 0x07060302u));
-                        u4 wv;
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            const float ba = BITS == 4 ? BASE4[2 * r] : BASE3[2 * r];
-                            const float bb = BITS == 4 ? BASE4[2 * r + 1] : BASE3[2 * r + 1];
-                            const h2 zb = z2 + (h2){(_Float16)ba, (_Float16)bb};
-                            wv[r] = as_u32((as_h2(bq[c][nb][r]) - zb) * s2);
-                        }
-                        bop[c] = __builtin_bit_cast(h8, wv);
-                    }
+                    for (int c = 0; c < 4; c++) bqn[c] = bq[c][nb];
+                    dequant_block<BITS, ACT>(bqn, ent, erow, bop);
                 }
 #pragma unroll
                 for (int rt = 0; rt < RT; rt++) {
@@ -346,91 +450,161 @@ __global__ __launch_bounds__(512) void stream_kernel(const Params p)
     }
 
     PHASE(3);
-    // ---- the waves of the workgroup add their tiles through LDS in a fixed tree ----------------
-    f4 *red = (f4 *)smem;  // [WK / 2][RT * 4 tiles][64 lanes] of f4, reuses the table's bytes
-    for (int stride = WK >> 1; stride >= 1; stride >>= 1) {
-        lds_barrier();  // the table, or the previous round, is no longer read
-        if (wave >= stride && wave < 2 * stride) {
-            f4 *dst = red + (size_t)(wave - stride) * (RT * 4) * 64 + lane;
-#pragma unroll
-            for (int rt = 0; rt < RT; rt++)
-#pragma unroll
-                for (int c = 0; c < 4; c++) dst[(rt * 4 + c) * 64] = acc[rt][c];
-        }
-        lds_barrier();
-        if (wave < stride) {
-            const f4 *src = red + (size_t)wave * (RT * 4) * 64 + lane;
-#pragma unroll
-            for (int rt = 0; rt < RT; rt++)
-#pragma unroll
-                for (int c = 0; c < 4; c++) acc[rt][c] += src[(rt * 4 + c) * 64];
-        }
-    }
-    const bool owner = wave == 0 && n_ok;
+    reduce_waves<RT>(acc, wave, WK, lane);
     PHASE(4);
+    write_out<RT>(p, acc, wave == 0 && n_ok, m0, rows_here, n0, lq, split, &last_flag);
+    PHASE(5);
+}
 
-    // ---- epilogue: acc[rt][c][v] is y[m0 + 16 rt + 4 q + v][n0 + c] ----
-    const _Float16 *bias = (const _Float16 *)p.bias;
-    f4 bv = {0.f, 0.f, 0.f, 0.f};
-    if (bias && owner) {
-        const h4 b4 = *(const h4 *)(bias + n0);
-        bv = (f4){(float)b4[0], (float)b4[1], (float)b4[2], (float)b4[3]};
-    }
-    _Float16 *y = (_Float16 *)p.y;
-    if (p.split_k == 1) {
-        if (owner) {
-#pragma unroll
-            for (int rt = 0; rt < RT; rt++) {
-#pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    const int row = 16 * rt + 4 * lq + v;
-                    if (row < rows_here) {
-                        h4 o;
-#pragma unroll
-                        for (int c = 0; c < 4; c++) o[c] = (_Float16)(acc[rt][c][v] + bv[c]);
-                        *(h4 *)(y + (size_t)(m0 + row) * p.N + n0) = o;
-                    }
-                }
-            }
-        }
-        PHASE(5);
-        return;
-    }
 
-    if (owner) {
+// ---- M <= 16 without the pack pass ------------------------------------------------------------
+// One row tile: lane (i, q) reads the 8 (int4) / 32 (int3) channels of ITS lane block straight
+// from row min(i, M - 1) of x, and the g_idx entries of the same channels, in natural order, and
+// sorts them into slot order in registers (byte permutes for x, plain renaming for the 32-bit
+// group numbers).  Both ride in rings of the same depth as the weights, requested right after
+// them, so the in-order rule of the loads above holds.  Rows past M compute values nobody
+// stores; lane blocks past K are zeroed.
+template <int N>
+__device__ __forceinline__ uint32_t pick_halves(const uint32_t (&r)[N], int ha, int hb)
+{
+    const uint32_t sel = ((ha & 1) ? 0x0302u : 0x0100u) | (((hb & 1) ? 0x0706u : 0x0504u) << 16);
+    return __builtin_amdgcn_perm(r[hb >> 1], r[ha >> 1], sel);
+}
+
+template <int BITS, bool ACT>
+__global__ __launch_bounds__(512) void stream_direct_kernel(const Params p)
+{
+    using F = Fmt<BITS>;
+    constexpr int PF = stream_pf(BITS);
+    constexpr int TROW = kStreamTableRow;
+    constexpr int XV = F::KLANE / 8;  // 16-byte vectors of x per lane block
+    constexpr int GV = F::KLANE / 4;  // 16-byte vectors of g_idx per lane block
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int WK = p.waves_k;
+    const int li = lane & 15;
+    const int lq = lane >> 4;
+    const int n_blk = blockIdx.x * 64;
+    const int col_l = 4 * li;
+    const int n0 = n_blk + col_l;
+    const bool n_ok = n0 < p.N;
+    const int split = blockIdx.y;
+    const int s_begin = split * WK * p.wave_steps;
+    const int ws = s_begin + wave * p.wave_steps;
+    const int prows = p.K / F::KLANE;  // lane blocks along K
+    const int last_step = p.steps_total - 1;
+    __shared__ int last_flag;
+
+    const uint32_t n_ld = (uint32_t)min(n0, p.N - 4);
+    const uint32_t x_row = (uint32_t)min(li, p.M - 1) * (uint32_t)p.K * 2u;
+    u4 w[PF][F::WORDS];
+    u4 xr[PF][XV];
+    u4 gr[ACT ? PF : 1][ACT ? GV : 1];
+    auto load_step = [&](int st, u4 (&wr)[F::WORDS], u4 (&xv)[XV], u4 (&gv)[ACT ? GV : 1]) {
+        const int st_c = min(st, last_step);
+        const int lq_c = min(lq, prows - 1 - 4 * st_c);  // lane blocks past K repeat the last one
+        const uint32_t blk = (uint32_t)(4 * st_c + lq_c);
+        const char *wbase = (const char *)p.qweight + (size_t)st_c * (4u * F::WORDS * (uint32_t)p.N * 4u);
+        const uint32_t woff = ((uint32_t)lq_c * F::WORDS * (uint32_t)p.N + n_ld) * 4u;
 #pragma unroll
-        for (int rt = 0; rt < RT; rt++) {
+        for (int wd = 0; wd < F::WORDS; wd++) {
+            wr[wd] = __builtin_nontemporal_load((const u4 *)(wbase + (woff + (uint32_t)wd * (uint32_t)p.N * 4u)));
+        }
+        const uint32_t k0 = blk * F::KLANE;
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const int row = 16 * rt + 4 * lq + v;
-                if (row < rows_here) {
-                    const f4 o = {acc[rt][0][v], acc[rt][1][v], acc[rt][2][v], acc[rt][3][v]};
-                    store_partial(p.partial + ((size_t)split * p.M + (m0 + row)) * p.N + n0, o);
+        for (int v = 0; v < XV; v++) xv[v] = *(const u4 *)((const char *)p.x + (x_row + (k0 + 8u * v) * 2u));
+        if constexpr (ACT) {
+#pragma unroll
+            for (int v = 0; v < GV; v++) gv[v] = *(const u4 *)((const char *)p.g_idx + (k0 + 4u * v) * 4u);
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < PF; u++) load_step(ws + u, w[u], xr[u], gr[ACT ? u : 0]);
+    STREAM_PIN_LOADS();
+
+    const int k_lo = min(s_begin * F::KSTEP, p.K - 1);
+    const int k_hi = min((s_begin + WK * p.wave_steps) * F::KSTEP, p.K) - 1;
+    const int g_lo = ACT ? 0 : k_lo / p.group_size;
+    const int g_hi = ACT ? p.G - 1 : min(p.G - 1, max(k_hi, k_lo) / p.group_size);
+    stage_table<BITS>(p, g_lo, g_hi, n_blk, tid);
+    const int tab_bias = col_l * 4 - g_lo * TROW;
+
+    f4 acc[1][4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) acc[0][c] = (f4){0.f, 0.f, 0.f, 0.f};
+    const uint32_t magic_a = opaque_vgpr(BITS == 4 ? MAGIC4_LO : MAGIC3_EVEN);
+    const uint32_t magic_b = opaque_vgpr(BITS == 4 ? MAGIC4_HI : MAGIC3_ODD);
+    lds_barrier();  // the table is complete
+
+    for (int i0 = 0; i0 < p.wave_steps; i0 += PF) {
+#pragma unroll
+        for (int u = 0; u < PF; u++) {
+            const int st = ws + i0 + u;
+            const bool live = 4 * st + lq < prows;  // this lane's block lies inside K
+            // everything that reads the ring slot comes first, then the slot is refilled
+            u4 bq[4][F::NB];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                if constexpr (BITS == 4) {
+                    biased4(w[u][0][c], bq[c], magic_a, magic_b);
+                } else {
+                    biased3(w[u][0][c], w[u][1][c], w[u][2][c], bq[c], magic_a, magic_b);
+                }
+            }
+            uint32_t xs[F::KLANE / 2];  // natural order, two channels per register
+#pragma unroll
+            for (int v = 0; v < XV; v++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) xs[4 * v + e] = live ? xr[u][v][e] : 0u;
+            h8 a[F::NB];
+#pragma unroll
+            for (int nb = 0; nb < F::NB; nb++) {
+                u4 f;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    f[r] = pick_halves(xs, code_of_slot<BITS>(8 * nb + 2 * r), code_of_slot<BITS>(8 * nb + 2 * r + 1));
+                }
+                a[nb] = __builtin_bit_cast(h8, f);
+            }
+            uint32_t go[ACT ? F::KLANE : 1];  // table row offsets in slot order
+            u4 erow = {0u, 0u, 0u, 0u};
+            if constexpr (ACT) {
+#pragma unroll
+                for (int s = 0; s < F::KLANE; s++) {
+                    const int cd = code_of_slot<BITS>(s);
+                    const int g = (int)gr[u][cd >> 2][cd & 3];
+                    go[s] = (uint32_t)(min(max(g, 0), p.G - 1) * TROW + tab_bias);
+                }
+            } else {
+                const uint32_t r = (uint32_t)min(4 * st + lq, prows - 1);
+                const uint32_t g = __umulhi(r, p.gdiv_magic) + (p.gdiv_add ? r : 0u);
+                erow = *(const u4 *)(smem + (g * TROW + (uint32_t)tab_bias));
+            }
+            STREAM_PIN_LOADS();
+            load_step(st + PF, w[u], xr[u], gr[ACT ? u : 0]);
+            STREAM_PIN_LOADS();
+#pragma unroll
+            for (int nb = 0; nb < F::NB; nb++) {
+                u4 ent[8];
+                if constexpr (ACT) {
+#pragma unroll
+                    for (int s = 0; s < 8; s++) ent[s] = *(const u4 *)(smem + go[8 * nb + s]);
+                }
+                u4 bqn[4];
+#pragma unroll
+                for (int c = 0; c < 4; c++) bqn[c] = bq[c][nb];
+                h8 bop[4];
+                dequant_block<BITS, ACT>(bqn, ent, erow, bop);
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    acc[0][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[nb], bop[c], acc[0][c], 0, 0, 0);
                 }
             }
         }
     }
-    int *counter = p.counters + blockIdx.z * gridDim.x + blockIdx.x;
-    if (!arrive_last(counter, p.split_k, &last_flag)) return;
-    if (owner) {
-#pragma unroll
-        for (int rt = 0; rt < RT; rt++) {
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const int row = 16 * rt + 4 * lq + v;
-                if (row < rows_here) {
-                    f4 sum = bv;
-                    for (int s = 0; s < p.split_k; s++) {
-                        sum += load_partial(p.partial + ((size_t)s * p.M + (m0 + row)) * p.N + n0);
-                    }
-                    h4 o;
-#pragma unroll
-                    for (int c = 0; c < 4; c++) o[c] = (_Float16)sum[c];
-                    *(h4 *)(y + (size_t)(m0 + row) * p.N + n0) = o;
-                }
-            }
-        }
-    }
+    reduce_waves<1>(acc, wave, WK, lane);
+    write_out<1>(p, acc, wave == 0 && n_ok, 0, min(16, p.M), n0, lq, split, &last_flag);
 }
 
 template <int BITS, int RT, bool ACT>
@@ -442,6 +616,16 @@ static int launch_stream_one(const Params &p, const gptq_hip_plan &plan, hipStre
             hipSuccess) {
             (void)hipGetLastError();
             return GPTQ_HIP_ERR_LAUNCH;
+        }
+    }
+    const dim3 grid_d(plan.grid_x, plan.grid_y, plan.grid_z);
+    if (p.direct) {
+        if constexpr (RT == 1) {
+            auto kd = stream_direct_kernel<BITS, ACT>;
+            hipLaunchKernelGGL(kd, grid_d, dim3(plan.block), plan.lds_bytes, stream, p);
+            return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+        } else {
+            return GPTQ_HIP_ERR_BAD_ARG;
         }
     }
     const uint32_t pack_threads = (uint32_t)p.steps_pad * (uint32_t)p.rt_total * 64u;

@@ -11,7 +11,7 @@
  *   qweight int32 [K/32*bits, N]   codes packed along K, little-endian bit stream
  *   qzeros  int32 [G, N/32*bits]   (zero point - 1) packed along N the same way
  *   scales  fp16  [G, N]
- *   g_idx   int32 [K]              group of input channel k; NULL means k / group_size
+ *   g_idx   int32 [K]              group of input channel k; NULL means k / group_size (16-byte aligned)
  *   bias    fp16  [N] or NULL
  *   x       fp16  [M, K] row-major, y fp16 [M, N] row-major
  * with G = ceil(K / group_size) and group_size = -1 meaning K.
