@@ -252,6 +252,8 @@ int plan_stream(int M, int K, int N, int bits, int gs, int G, int act_order, int
     int waves_k = force_waves > 0 ? force_waves : (tiles * 8 <= 2048 ? 8 : 4);
     while (waves_k > 1 && waves_k * pf > steps_total) waves_k >>= 1;
     int split = tiles >= 128 ? 1 : ceil_div(256, (int)tiles);
+    // a long K per wave pays for the cross-workgroup sum when the tiles alone leave CUs idle
+    if (tiles >= 128 && tiles < 256 && K / waves_k >= 2048) split = ceil_div(384, (int)tiles);
     int cap = (int)((3LL * K * bits) / (128LL * M));
     if (cap < 1) cap = 1;
     if (split > cap) split = cap;
@@ -306,7 +308,11 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     if (G == 1) act_order = 0;
     // GROUPED for decoding (M = 1); for M = 2 only where a workgroup holds all of K, since its
     // operand in LDS doubles with M and the cross-workgroup sum costs more than STREAM's pack pass
-    if (M <= 2 && plan_grouped(M, K, N, bits, gs, G, act_order, 0, 0, plan) && (M == 1 || plan->split_k == 1))
+    // A single group over a large matrix gains nothing from GROUPED's expansion by group: STREAM's
+    // one table entry per lane block is cheaper there.
+    const bool one_big_group = G == 1 && (long long)K * N >= (1LL << 27);
+    if (M <= 2 && !one_big_group && plan_grouped(M, K, N, bits, gs, G, act_order, 0, 0, plan) &&
+        (M == 1 || plan->split_k == 1))
         return GPTQ_HIP_OK;
     memset(plan, 0, sizeof(*plan));
     if (plan_stream(M, K, N, bits, gs, G, act_order, 0, 0, plan) == GPTQ_HIP_OK) return GPTQ_HIP_OK;
