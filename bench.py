@@ -245,14 +245,14 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernel", type=int, default=0, help="force a kernel family (1 gather, 2 grouped, 3 blocked)")
     ap.add_argument("--split-k", type=int, default=0, help="force the split-K factor")
-    ap.add_argument("--waves-n", type=int, default=0, help="force the waves per workgroup along N")
+    ap.add_argument("--waves-n", type=int, default=0, help="force the waves per workgroup along N (STREAM kernel: along K)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 256 MiB device copy a few times (known traffic, for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters of a profiler run) and exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures the QuantLinear kernels on ONE GPU; --gpus must be 1 "
-              "(the path shards by output columns with no exchange, see DESIGN.md)", file=sys.stderr)
+              "(the path shards by output columns with no exchange between GPUs)", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the kernels have no CPU fallback", file=sys.stderr)
