@@ -1,0 +1,176 @@
+"""Loading a standard AutoGPTQ checkpoint onto the MI355X ``QuantLinear``.
+
+Mirrors the three pieces of the reference's loading path that touch the quantised layers:
+
+* ``find_layers``   auto_gptq/modeling/_utils.py:38-49
+* ``make_quant``    auto_gptq/modeling/_utils.py:59-90 (the ``use_tvm=True`` branch picks this
+                    package's ``QuantLinear`` instead of ``qlinear_tvm.QuantLinear``)
+* ``from_quantized`` auto_gptq/modeling/_base.py:478-569: read ``quantize_config.json``, build the
+  model from its config with empty weights, swap the linear layers, load the checkpoint tensors
+  by name onto the device.
+
+The checkpoint is read with ``safetensors`` or ``torch.load(weights_only=True)``: nothing from the
+file is executed.  Unlike the reference's TVM module, ``QuantLinear`` here can be built on the
+``meta`` device (its constructor compiles and allocates nothing on the GPU).
+"""
+import json
+import os
+from typing import Dict, Iterable, Optional
+
+import torch
+import torch.nn as nn
+
+from .qlinear import QuantLinear
+
+
+def _conv1d_type():
+    try:
+        from transformers.pytorch_utils import Conv1D
+
+        return Conv1D
+    except Exception:  # transformers missing or too old: no Conv1D layers to find
+        return None
+
+
+def find_layers(module: nn.Module, layer_types=None, name: str = "", found: Optional[dict] = None) -> Dict[str, nn.Module]:
+    """``{qualified name: layer}`` of every Linear / Conv2d / Conv1D below ``module``."""
+    if found is None:
+        found = {}
+    if not layer_types:
+        layer_types = [t for t in (_conv1d_type(), nn.Conv2d, nn.Linear) if t is not None]
+    for child_name, child in module.named_children():
+        full = name + "." + child_name if name else child_name
+        if isinstance(child, tuple(layer_types)):
+            found[full] = child
+        find_layers(child, layer_types, full, found)
+    return found
+
+
+def make_quant(module: nn.Module, names: Iterable[str], bits: int, groupsize: int, name: str = "") -> None:
+    """Replaces, in place, every child whose qualified name is in ``names`` by a ``QuantLinear`` of the
+    same shape on the same device (``meta`` included)."""
+    if isinstance(module, QuantLinear):
+        return
+    conv1d = _conv1d_type()
+    for child_name, child in list(module.named_children()):
+        full = name + "." + child_name if name else child_name
+        if full in names and not isinstance(child, QuantLinear):
+            if isinstance(child, nn.Linear):
+                in_features, out_features = child.in_features, child.out_features
+            elif isinstance(child, nn.Conv2d):
+                in_features, out_features = child.in_channels, child.out_channels
+            elif conv1d is not None and isinstance(child, conv1d):
+                in_features, out_features = child.weight.shape[0], child.weight.shape[1]
+            else:
+                raise TypeError(f"{full}: cannot quantise a {type(child).__name__}")
+            device = child.weight.device
+            new_layer = QuantLinear(bits, groupsize, in_features, out_features, child.bias is not None)
+            setattr(module, child_name, new_layer.to(device))
+    for child_name, child in module.named_children():
+        make_quant(child, names, bits, groupsize, name + "." + child_name if name else child_name)
+
+
+def read_quantize_config(save_dir: str) -> dict:
+    """``quantize_config.json`` as the reference writes it (auto_gptq/modeling/_base.py:66-77)."""
+    with open(os.path.join(save_dir, "quantize_config.json"), "r", encoding="utf-8") as f:
+        cfg = json.load(f)
+    for key in ("bits", "group_size"):
+        if key not in cfg:
+            raise ValueError(f"quantize_config.json has no '{key}'")
+    cfg.setdefault("desc_act", True)
+    return cfg
+
+
+def load_state_dict_file(path: str) -> Dict[str, torch.Tensor]:
+    """Tensors of a checkpoint file, read with a loader that executes nothing from the file."""
+    if path.endswith(".safetensors"):
+        from safetensors.torch import load_file
+
+        return load_file(path, device="cpu")
+    return torch.load(path, map_location="cpu", weights_only=True)
+
+
+def load_quantized_state(model: nn.Module, state: Dict[str, torch.Tensor], device) -> None:
+    """Materialises ``model`` (possibly on ``meta``) on ``device`` from ``state``, by name.  Every
+    parameter and persistent buffer must be present; the packed tensors keep their integer dtype."""
+    device = torch.device(device)
+    missing = []
+    own = dict(model.named_parameters())
+    own.update({k: v for k, v in model.named_buffers()})
+    non_persistent = set()
+    for mod_name, mod in model.named_modules():
+        for b in getattr(mod, "_non_persistent_buffers_set", ()):
+            non_persistent.add(mod_name + "." + b if mod_name else b)
+    for name, old in own.items():
+        if name in non_persistent:
+            # not in any checkpoint (e.g. rotary tables): keep the value the constructor computed
+            if old.device.type == "meta":
+                raise ValueError(f"non-persistent buffer {name} is on the meta device; build the model without "
+                                 f"empty buffers")
+            owner, _, leaf = name.rpartition(".")
+            (model.get_submodule(owner) if owner else model)._buffers[leaf] = old.to(device)
+            continue
+        if name not in state:
+            missing.append(name)
+            continue
+        new = state[name]
+        if tuple(new.shape) != tuple(old.shape):
+            raise ValueError(f"{name}: checkpoint shape {tuple(new.shape)} != model shape {tuple(old.shape)}")
+        dtype = new.dtype if not old.dtype.is_floating_point else old.dtype
+        value = new.to(device=device, dtype=dtype)
+        owner, _, leaf = name.rpartition(".")
+        mod = model.get_submodule(owner) if owner else model
+        if leaf in mod._parameters:
+            mod._parameters[leaf] = nn.Parameter(value, requires_grad=False)
+        else:
+            mod._buffers[leaf] = value
+    if missing:
+        raise KeyError(f"checkpoint lacks {len(missing)} tensors, e.g. {missing[:4]}")
+
+
+def from_quantized(save_dir: str, device="cuda:0", model_basename: Optional[str] = None,
+                   use_safetensors: bool = True, ignore_layers: Iterable[str] = ("lm_head",),
+                   trust_remote_code: bool = False):
+    """Builds the ``transformers`` causal LM described by ``save_dir/config.json`` with every linear
+    layer (except ``ignore_layers`` prefixes: the reference skips ``lm_head`` and the modules outside
+    the decoder stack) replaced by ``QuantLinear``, and fills it from
+    ``save_dir/gptq_model-{bits}bit-{group_size}g.{safetensors|bin}``.  Returns ``(model, quantize_config)``."""
+    import accelerate
+    from transformers import AutoConfig, AutoModelForCausalLM
+
+    qcfg = read_quantize_config(save_dir)
+    bits, group_size = int(qcfg["bits"]), int(qcfg["group_size"])
+    if model_basename is None:
+        model_basename = f"gptq_model-{bits}bit-{group_size}g"
+    path = os.path.join(save_dir, model_basename + (".safetensors" if use_safetensors else ".bin"))
+    if not os.path.isfile(path):
+        raise FileNotFoundError(f"Could not find model at {path}")
+    config = AutoConfig.from_pretrained(save_dir, trust_remote_code=trust_remote_code)
+    with accelerate.init_empty_weights(include_buffers=False):
+        model = AutoModelForCausalLM.from_config(config, trust_remote_code=trust_remote_code, torch_dtype=torch.float16)
+    layers = find_layers(model)
+    for lname in list(layers):
+        if any(lname.startswith(prefix) for prefix in ignore_layers):
+            del layers[lname]
+    with accelerate.init_empty_weights(include_buffers=True):  # the packed buffers too: nothing is allocated
+        make_quant(model, layers, bits, group_size)
+    state = load_state_dict_file(path)
+    # tied output embeddings are stored once
+    if hasattr(model, "tie_weights"):
+        for tied in ("lm_head.weight",):
+            if tied not in state and getattr(config, "tie_word_embeddings", False):
+                emb = model.get_input_embeddings()
+                for k, v in model.named_parameters():
+                    if v is emb.weight and k in state:
+                        state[tied] = state[k]
+    load_quantized_state(model, state, device)
+    if hasattr(model, "tie_weights"):
+        model.tie_weights()
+    seqlen = 4096
+    for key in ("max_position_embeddings", "seq_length", "n_positions"):
+        if key in model.config.to_dict():
+            seqlen = model.config.to_dict()[key]
+            break
+    model.seqlen = seqlen
+    model.eval()
+    return model, qcfg

@@ -1,0 +1,99 @@
+"""The checkpoint loader (reference: auto_gptq/modeling/_utils.py:38-90, _base.py:478-569)."""
+import numpy as np
+import pytest
+import torch
+
+from autogptq.tvm_amd import QuantLinear
+from autogptq.tvm_amd.loader import find_layers, from_quantized, make_quant
+from tests.loader_util import build_checkpoint
+
+
+def test_find_layers_and_make_quant_on_a_plain_module():
+    net = torch.nn.Sequential()
+    net.add_module("a", torch.nn.Linear(64, 32, bias=True))
+    net.add_module("act", torch.nn.ReLU())
+    inner = torch.nn.Module()
+    inner.proj = torch.nn.Linear(32, 64, bias=False)
+    net.add_module("inner", inner)
+    layers = find_layers(net)
+    assert sorted(layers) == ["a", "inner.proj"]
+    make_quant(net, ["inner.proj"], 3, 32)
+    assert isinstance(net.a, torch.nn.Linear)
+    q = net.inner.proj
+    assert isinstance(q, QuantLinear) and (q.infeatures, q.outfeatures, q.bits, q.groupsize) == (32, 64, 3, 32)
+    assert q.bias is None and q.qweight.shape == (3, 64)
+    make_quant(net, ["inner.proj"], 3, 32)  # already quantised: left alone
+    assert net.inner.proj is q
+
+
+def test_make_quant_on_meta_allocates_nothing():
+    import accelerate
+
+    with accelerate.init_empty_weights(include_buffers=True):
+        net = torch.nn.Sequential(torch.nn.Linear(4096, 11008, bias=False))
+        make_quant(net, ["0"], 4, 128)
+    assert net[0].qweight.device.type == "meta" and net[0].qweight.shape == (512, 11008)
+
+
+@pytest.mark.parametrize("bits,act_order", [(4, True), (3, False)])
+def test_from_quantized_restores_every_tensor(tmp_path, bits, act_order):
+    cfg, state, dense = build_checkpoint(str(tmp_path), bits=bits, gs=32, act_order=act_order)
+    model, qcfg = from_quantized(str(tmp_path), device="cpu")
+    assert qcfg["bits"] == bits and qcfg["group_size"] == 32
+    quantised = {n: m for n, m in model.named_modules() if isinstance(m, QuantLinear)}
+    assert len(quantised) == 2 * 7 and "lm_head" not in quantised           # q k v o gate up down per layer
+    assert isinstance(model.lm_head, torch.nn.Linear)
+    got = model.state_dict()
+    for name, want in state.items():
+        assert name in got, name
+        assert got[name].dtype == want.dtype and got[name].device.type == "cpu", name
+        assert torch.equal(got[name], want), name
+    assert model.seqlen == 64 and not model.training
+    with pytest.raises(RuntimeError):  # no CPU path: the kernels must not be silently replaced
+        model(torch.zeros((1, 4), dtype=torch.long))
+
+
+def test_from_quantized_reports_missing_files_and_tensors(tmp_path):
+    with pytest.raises(FileNotFoundError):
+        from_quantized(str(tmp_path))
+    cfg, state, dense = build_checkpoint(str(tmp_path), bits=4, gs=32, act_order=False)
+    from safetensors.torch import save_file
+
+    broken = {k: v for k, v in state.items() if not k.endswith("q_proj.qzeros")}
+    save_file(broken, str(tmp_path / "gptq_model-4bit-32g.safetensors"))
+    with pytest.raises(KeyError):
+        from_quantized(str(tmp_path), device="cpu")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits,act_order", [(4, True), (3, True), (4, False)])
+def test_loaded_model_matches_the_dequantised_float_model(tmp_path, bits, act_order):
+    """End to end: logits of the loaded quantised model on the GPU against the same architecture
+    with every quantised layer replaced by a float Linear holding the oracle's dequantised weight."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from transformers import AutoModelForCausalLM
+
+    from oracle import gptq_oracle as orc
+
+    cfg, state, dense = build_checkpoint(str(tmp_path), bits=bits, gs=32, act_order=act_order, seed=3)
+    model, _ = from_quantized(str(tmp_path), device="cuda:0")
+    ref = AutoModelForCausalLM.from_config(cfg).float()
+    ref_state = {}
+    for k, v in state.items():
+        if k.endswith((".qweight", ".qzeros", ".scales", ".g_idx")):
+            continue
+        ref_state[k] = v.float()
+    for name, q in dense.items():
+        w = orc.dequant_ref(q.qweight, q.qzeros, q.scales, q.g_idx, bits)   # [K, N] fp16
+        ref_state[name + ".weight"] = w.t().float().contiguous()
+    ref.load_state_dict(ref_state, strict=True)
+    ref.eval()
+    ids = torch.randint(0, cfg.vocab_size, (2, 9), generator=torch.Generator().manual_seed(5))
+    with torch.no_grad():
+        want = ref(ids).logits
+        got = model(ids.to("cuda:0")).logits.float().cpu()
+    assert got.shape == want.shape
+    # fp16 activations through two decoder layers against an fp32 model
+    assert float((got - want).abs().max()) <= 2e-2 + 2e-2 * float(want.abs().max())
+    assert np.isfinite(got.numpy()).all()
