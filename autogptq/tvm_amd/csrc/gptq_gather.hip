@@ -21,22 +21,6 @@
 
 namespace gptq {
 
-#ifdef GPTQ_PHASE_TIMES
-__device__ long long g_phase_gather[16 * 8192];
-#define PHASE(i)                                                                                                   \
-    do {                                                                                                           \
-        if (lane == 0)                                                                                             \
-            g_phase_gather[((size_t)((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 4 + wave) * 16 + \
-                           (i)] = clock64();                                                                       \
-    } while (0)
-extern "C" int gptq_hip_debug_read_gather(void *host, size_t bytes)
-{
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_phase_gather), bytes, 0, hipMemcpyDeviceToHost);
-}
-#else
-#define PHASE(i) do { } while (0)
-#endif
-
 template <int BITS, int RT, bool ACT>
 __global__ __launch_bounds__(256) void gather_kernel(const Params p)
 {
@@ -57,7 +41,6 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
     const int col_l = wn * 64 + 4 * li;
     const int n0 = n_blk + col_l;
     const bool n_ok = n0 < p.N;
-    PHASE(0);
     const int m0 = blockIdx.z * (16 * RT);
     const int rows_here = min(16 * RT, p.M - m0);
     const int split = blockIdx.y;
@@ -180,7 +163,6 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
 
     const int nchunks = (p.wave_steps + CS - 1) / CS;
     fetch_chunk(0);
-    PHASE(1);
 
     // (scale, zero) table: four columns of one group per thread and item.  With contiguous groups
     // only the groups of this workgroup's K range are staged (row 0 = the first of them).  Items
@@ -220,7 +202,6 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
         }
     }
 
-    PHASE(2);
     f4 acc[RT][4];
 #pragma unroll
     for (int rt = 0; rt < RT; rt++)
@@ -232,7 +213,6 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
 
     store_chunk(0);
     lds_barrier();
-    PHASE(3);
     // steps every wave of the workgroup walks: whole chunks, rounded up to the prefetch ring
     const int total = (nchunks * CS + PF - 1) / PF * PF;
     const int walk_chunks = (total + CS - 1) / CS;  // chunks past the wave's range are staged as zeros
@@ -332,7 +312,6 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
         }
     }
 
-    PHASE(4);
     // ---- waves along K meet in LDS: wave (wn, 0) adds the others' tiles in order ------------
     if (WK > 1) {
         float *red = (float *)smem;  // [WK - 1][WN][RT * 16][64], reuses the staging area
@@ -360,7 +339,6 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
         }
     }
     const bool owner = wk == 0 && n_ok;
-    PHASE(5);
 
     // ---- epilogue: acc[rt][c][v] is y[m0 + 16 rt + 4 q + v][n0 + c] ----
     const _Float16 *bias = (const _Float16 *)p.bias;
@@ -386,8 +364,6 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
                 }
             }
         }
-        PHASE(6);
-        PHASE(7);
         return;
     }
 
@@ -404,10 +380,8 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
             }
         }
     }
-    PHASE(6);
     int *counter = p.counters + blockIdx.z * gridDim.x + blockIdx.x;
     if (!arrive_last(counter, p.split_k, &last_flag)) {
-        PHASE(7);
         return;
     }
     if (owner) {
@@ -429,7 +403,6 @@ __global__ __launch_bounds__(256) void gather_kernel(const Params p)
             }
         }
     }
-    PHASE(7);
 }
 
 template <int BITS, int RT, bool ACT>

@@ -30,13 +30,6 @@
 
 namespace gptq {
 
-#ifdef GPTQ_PHASE_TIMES
-__device__ long long g_phase[16 * 8192];
-#define PHASE(i) do { if (lane == 0) g_phase[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 8 + wave) * 16 + (i)] = clock64(); } while (0)
-#else
-#define PHASE(i) do { } while (0)
-#endif
-
 __device__ __forceinline__ h8 and_h8(h8 a, u4 m)
 {
     u4 v = __builtin_bit_cast(u4, a);
@@ -90,7 +83,6 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     unsigned char *masks = smem + (size_t)nblk8 * ST * 256;
     float *red = (float *)(masks + (COMPACT ? (size_t)nblk8 * 16 : 0));
 
-    PHASE(0);
     int qslot[4];
 #pragma unroll
     for (int e = 0; e < 4; e++) qslot[e] = slot_of_code<BITS>((4 * tid) % F::KLANE + e);
@@ -152,7 +144,6 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
 #pragma unroll
     for (int s = 0; s < PF && s < NSTEP; s++) load_step(s, ws + s);
     __builtin_amdgcn_sched_barrier(0);
-    PHASE(1);
 
     // ---- 4. scales / zero words this lane needs in the epilogue (rows g = 16 t + 4 q + v);
     //         loaded once the last weight loads are out ---------------------------------
@@ -175,7 +166,6 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     };
 
     lds_barrier();
-    PHASE(2);
     // ---- 5. scatter x into the operand tiles (waits for x / g_idx only) -------------------
     // A thread always owns quads with the same position inside a lane block (kc % KLANE is
     // 4 * (tid % (KLANE / 4)) in every pass because the block size is a multiple of 8), so the
@@ -220,7 +210,6 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         }
     }
     lds_barrier();
-    PHASE(3);
     load_epilogue_operands();
 
     // ---- 6. main loop -----------------------------------------------------------------
@@ -310,7 +299,6 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         }
     }
 
-    PHASE(4);
     // ---- 7. scales and zero points once per group, then sum over groups ------------------
     // row v of tile t in lane group q is group g_base + 16 t + 4 q + v
     float tot[M][4];
@@ -359,7 +347,6 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         }
     }
 
-    PHASE(5);
     // ---- 8. waves along K meet in LDS; one thread per four output columns finishes --------
     if (lq == 0) {
 #pragma unroll
@@ -369,7 +356,6 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         }
     }
     lds_barrier();
-    PHASE(6);
     const bool fin = tid < WN * M * 16;
     const int f_wn = tid / (M * 16);
     const int f_m = (tid >> 4) % M;
@@ -395,15 +381,10 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
             for (int c = 0; c < 4; c++) o[c] = (_Float16)(sum[c] + bv[c]);
             *(h4 *)(y + (size_t)f_m * p.N + f_n) = o;
         }
-        PHASE(7);
         return;
     }
     if (writer) store_partial(p.partial + ((size_t)split * M + f_m) * p.N + f_n, sum);
-    if (!arrive_last(p.counters + blockIdx.x, p.split_k, &last_flag)) {
-        PHASE(7);
-        return;
-    }
-    PHASE(11);
+    if (!arrive_last(p.counters + blockIdx.x, p.split_k, &last_flag)) return;
     if (writer) {
         f4 total = bv;
         for (int s = 0; s < p.split_k; s++) total += load_partial(p.partial + ((size_t)s * M + f_m) * p.N + f_n);
@@ -412,7 +393,6 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         for (int c = 0; c < 4; c++) o[c] = (_Float16)total[c];
         *(h4 *)(y + (size_t)f_m * p.N + f_n) = o;
     }
-    PHASE(7);
 }
 
 template <int BITS, int M, int TPM, bool COMPACT>
@@ -454,13 +434,6 @@ static int launch_grouped_bits(const Params &p, const gptq_hip_plan &plan, hipSt
     }
     return GPTQ_HIP_ERR_UNSUPPORTED;
 }
-
-#ifdef GPTQ_PHASE_TIMES
-extern "C" int gptq_hip_debug_read(void *host, size_t bytes)
-{
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_phase), bytes, 0, hipMemcpyDeviceToHost);
-}
-#endif
 
 int launch_grouped(const Params &p, int bits, const gptq_hip_plan &plan, void *stream)
 {

@@ -28,22 +28,6 @@
 
 namespace gptq {
 
-#ifdef GPTQ_PHASE_TIMES
-__device__ long long g_phase_stream[16 * 8192];
-#define PHASE(i)                                                                                                   \
-    do {                                                                                                           \
-        if (lane == 0)                                                                                             \
-            g_phase_stream[((size_t)((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 8 + wave) * 16 + \
-                           (i)] = clock64();                                                                       \
-    } while (0)
-extern "C" int gptq_hip_debug_read_stream(void *host, size_t bytes)
-{
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_phase_stream), bytes, 0, hipMemcpyDeviceToHost);
-}
-#else
-#define PHASE(i) do { } while (0)
-#endif
-
 namespace {
 
 // code of slot s of a lane block, as compile-time tables (SLOT4 / SLOT3 of gptq_unpack.h)
@@ -296,7 +280,6 @@ __global__ __launch_bounds__(512) void stream_kernel(const Params p)
     const int WK = p.waves_k;
     const int li = lane & 15;
     const int lq = lane >> 4;
-    PHASE(0);
     const int n_blk = blockIdx.x * 64;
     const int col_l = 4 * li;
     const int n0 = n_blk + col_l;
@@ -366,7 +349,6 @@ __global__ __launch_bounds__(512) void stream_kernel(const Params p)
         }
     }
     STREAM_PIN_LOADS();
-    PHASE(1);
 
     // ---- (scale, zero) table of the 64 columns: all groups under a g_idx, else those of the
     //      workgroup's K range (row 0 = the first of them) ---------------------------------
@@ -387,7 +369,6 @@ __global__ __launch_bounds__(512) void stream_kernel(const Params p)
     const uint32_t magic_b = opaque_vgpr(BITS == 4 ? MAGIC4_HI : MAGIC3_ODD);
 
     lds_barrier();  // the table is complete
-    PHASE(2);
 
     // ---- main loop: nothing in it is conditional -------------------------------------------
     for (int i0 = 0; i0 < p.wave_steps; i0 += PF) {
@@ -449,11 +430,8 @@ __global__ __launch_bounds__(512) void stream_kernel(const Params p)
         }
     }
 
-    PHASE(3);
     reduce_waves<RT>(acc, wave, WK, lane);
-    PHASE(4);
     write_out<RT>(p, acc, wave == 0 && n_ok, m0, rows_here, n0, lq, split, &last_flag);
-    PHASE(5);
 }
 
 

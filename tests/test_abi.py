@@ -129,6 +129,12 @@ def test_entry_points_reject_null_and_bad_sizes_before_touching_the_gpu():
     # misaligned qweight
     assert lib.gptq_hip_gemm(fake, ctypes.c_void_p(0x1004), fake, fake, null, null, fake, null, 0, 1, 64, 64, 4, 32,
                              null) == _lib.ERR_BAD_ARG
+    # g_idx that is not 16-byte aligned (the kernels read it four entries at a time)
+    assert lib.gptq_hip_gemm(fake, fake, fake, fake, ctypes.c_void_p(0x1004), null, fake, null, 0, 1, 64, 64, 4, 32,
+                             null) == _lib.ERR_BAD_ARG
+    # a STREAM plan for M > 16 always needs the workspace (packed activations)
+    assert lib.gptq_hip_gemm(fake, fake, fake, fake, null, null, fake, null, 0, 64, 4096, 11008, 4, 128,
+                             null) == _lib.ERR_WORKSPACE
     # a split-K plan without a workspace
     assert lib.gptq_hip_gemm(fake, fake, fake, fake, null, null, fake, null, 0, 1, 4096, 4096, 4, 128,
                              null) == _lib.ERR_WORKSPACE
@@ -154,6 +160,28 @@ def test_plan_for_forces_family_split_and_waves():
     with pytest.raises(_lib.GptqHipError) as e:
         _lib.plan_for(_lib.KERNEL_GATHER, 1, 4096, 4096, 4, 128, True, waves_n=3)
     assert e.value.status == _lib.ERR_BAD_ARG
+
+
+def test_dispatcher_families_by_m():
+    # decode: GROUPED; M = 2 only while one workgroup holds all of K; batches: STREAM, direct up to 16 rows
+    assert _lib.select(1, 4096, 11008, 4, 128, True).kernel == _lib.KERNEL_GROUPED
+    assert _lib.select(2, 4096, 11008, 4, 128, False).kernel == _lib.KERNEL_STREAM
+    p = _lib.select(8, 4096, 11008, 4, 128, True)
+    assert p.kernel == _lib.KERNEL_STREAM and p.row_tiles == 1 and p.workspace_bytes == 0 and p.split_k == 1
+    p = _lib.select(128, 4096, 11008, 3, 128, True)
+    assert p.kernel == _lib.KERNEL_STREAM and p.row_tiles == 4 and p.m_blocks == 2 and p.split_k == 1
+    assert p.workspace_bytes >= 128 * 4096 * 2
+    # one group over a large matrix streams better without the expansion by group
+    assert _lib.select(1, 9216, 36864, 3, -1, False).kernel == _lib.KERNEL_STREAM
+    # forcing the STREAM family with waves along K and a split
+    p = _lib.plan_for(_lib.KERNEL_STREAM, 40, 4096, 352, 3, 128, True, split_k=2, waves_n=8)
+    assert p.kernel == _lib.KERNEL_STREAM and p.waves_k == 8 and p.waves_n == 1 and p.split_k == 2 and p.block == 512
+    # more groups than the LDS table of STREAM holds: the GATHER fallback, or unsupported
+    try:
+        p = _lib.select(4, 36864, 9216, 4, 32, True)
+        assert p.kernel == _lib.KERNEL_GATHER
+    except _lib.GptqHipError as e:
+        assert e.status == _lib.ERR_UNSUPPORTED
 
 
 def test_single_group_ignores_act_order():
