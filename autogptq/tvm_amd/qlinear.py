@@ -15,7 +15,7 @@ import numpy as np
 import torch
 import torch.nn as nn
 
-from . import ops
+from . import _lib, ops
 from .pack import pack_qweight, pack_qzeros
 
 
@@ -87,7 +87,14 @@ class QuantLinear(nn.Module):
                 if lo < 0 or hi >= self.scales.shape[0]:
                     raise ValueError(f"g_idx values must lie in [0, {self.scales.shape[0]}), found [{lo}, {hi}]")
             self._g_state = (key, contiguous)
-        return None if self._g_state[1] else g
+        if self._g_state[1]:
+            return None
+        if not g.is_contiguous() or g.data_ptr() % 16 != 0 or g.dtype != torch.int32:
+            # the kernels read g_idx four entries at a time
+            self.g_idx = g.to(torch.int32).contiguous().clone()
+            self._g_state = None
+            return self._kernel_g_idx()
+        return g
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         out_shape = x.shape[:-1] + (self.outfeatures,)
@@ -96,8 +103,19 @@ class QuantLinear(nn.Module):
             x2 = x2.half()
         if not x2.is_contiguous():
             x2 = x2.contiguous()
-        out = ops.gemm(x2, self.qweight, self.qzeros, self.scales, self._kernel_g_idx(), self.bias,
-                       self.bits, self.groupsize)
+        try:
+            out = ops.gemm(x2, self.qweight, self.qzeros, self.scales, self._kernel_g_idx(), self.bias,
+                           self.bits, self.groupsize)
+        except _lib.GptqHipError as e:
+            if e.status != _lib.ERR_UNSUPPORTED:
+                raise
+            # A shape the fused kernels do not cover (activation order with more groups than their
+            # LDS table holds): materialise W with the HIP dequant kernel and multiply with the
+            # library GEMM, which is what the reference does above its kernel_switch_threshold
+            # (auto_gptq/nn_modules/qlinear.py:198-245).  Still GPU only.
+            out = torch.matmul(x2, self.dequantize())
+            if self.bias is not None:
+                out = out + self.bias
         return out.reshape(out_shape)
 
     def dequantize(self) -> torch.Tensor:

@@ -294,6 +294,19 @@ def test_quantlinear_forward(dev, bits):
     assert_close(q2(L2["x"].to(dev)), expected_output(L2), "module forward, contiguous groups")
 
 
+def test_module_falls_back_to_dequant_plus_library_gemm_for_uncovered_shapes(dev):
+    # activation order with more groups than any fused kernel's LDS table holds
+    K, N, gs, M = 36864, 64, 32, 4
+    L = layer(77, K, N, 4, gs, True, M=M, bias=True)
+    with pytest.raises(_lib.GptqHipError):
+        _lib.select(M, K, N, 4, gs, True)
+    q = QuantLinear(4, gs, K, N, True)
+    q.qweight, q.qzeros, q.scales, q.g_idx, q.bias = L["qweight"], L["qzeros"], L["scales"], L["g_idx"], L["bias"]
+    q = q.to(dev)
+    y = q(L["x"].to(dev))
+    assert_close(y, expected_output(L), "fallback")
+
+
 def test_bad_g_idx_is_rejected_by_the_module(dev):
     q = QuantLinear(4, 32, 64, 32, False).to(dev)
     q.g_idx[3] = 99
