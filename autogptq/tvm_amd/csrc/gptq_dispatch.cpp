@@ -242,7 +242,7 @@ int plan_stream(int M, int K, int N, int bits, int gs, int G, int act_order, int
     const int col_tiles = ceil_div(N, 64);
     const long long tiles = (long long)col_tiles * m_blocks;
     const int act_table = gptq::stream_act_table(bits, gs, act_order);
-    if (tiles * (long long)sizeof(int) > (long long)gptq::kCounterBytes) return GPTQ_HIP_ERR_UNSUPPORTED;
+    const bool can_split = tiles * (long long)sizeof(int) <= (long long)gptq::kCounterBytes;  // one counter per tile
 
     // Waves come from column tiles x M blocks x waves along K inside a workgroup (free: their
     // tiles meet in LDS) x workgroups along K (dear: the partial tiles cross HBM twice and the
@@ -259,6 +259,10 @@ int plan_stream(int M, int K, int N, int bits, int gs, int G, int act_order, int
     if (split > cap) split = cap;
     if (split > 64) split = 64;
     if (force_split > 0) split = force_split;
+    if (!can_split) {
+        if (force_split > 1) return GPTQ_HIP_ERR_UNSUPPORTED;
+        split = 1;
+    }
     if (split * waves_k * pf > steps_total) split = steps_total / (waves_k * pf);
     if (split < 1) split = 1;
     int wave_steps = gptq::stream_wave_steps(bits, steps_total, split, waves_k);

@@ -22,7 +22,7 @@ from .pack import pack_qweight, pack_qzeros
 class QuantLinear(nn.Module):
     SUPPORTED_BITS = (3, 4)
 
-    def __init__(self, bits, groupsize, infeatures, outfeatures, bias, kernel_switch_threshold=128):
+    def __init__(self, bits, groupsize, infeatures, outfeatures, bias, kernel_switch_threshold=1024):
         super().__init__()
         if bits not in self.SUPPORTED_BITS:
             # the reference accepts 2, 3, 4, 8 (qlinear.py:31-32); this path implements 3 and 4
@@ -34,7 +34,11 @@ class QuantLinear(nn.Module):
         self.bits = bits
         self.groupsize = groupsize if groupsize != -1 else infeatures
         self.maxq = 2 ** self.bits - 1
-        self.kernel_switch_threshold = kernel_switch_threshold  # kept for signature parity; unused
+        # Rows of x from which forward() materialises W (HIP dequant kernel) and calls the library
+        # GEMM instead of the fused kernels, as the reference does (qlinear.py:25,198: default 128
+        # there).  Measured on MI355X at 4096x11008 int4: fused 95 us vs 116 us at 512 rows, 172 us
+        # vs 143 us at 1024 rows, hence 1024.  0 or None disables the switch.
+        self.kernel_switch_threshold = kernel_switch_threshold
 
         groups = math.ceil(infeatures / self.groupsize)
         self.register_buffer("qweight", torch.zeros((infeatures // 32 * bits, outfeatures), dtype=torch.int32))
@@ -104,15 +108,17 @@ class QuantLinear(nn.Module):
         if not x2.is_contiguous():
             x2 = x2.contiguous()
         try:
+            if self.kernel_switch_threshold and x2.shape[0] >= self.kernel_switch_threshold:
+                raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, "above kernel_switch_threshold")
             out = ops.gemm(x2, self.qweight, self.qzeros, self.scales, self._kernel_g_idx(), self.bias,
                            self.bits, self.groupsize)
         except _lib.GptqHipError as e:
             if e.status != _lib.ERR_UNSUPPORTED:
                 raise
-            # A shape the fused kernels do not cover (activation order with more groups than their
-            # LDS table holds): materialise W with the HIP dequant kernel and multiply with the
-            # library GEMM, which is what the reference does above its kernel_switch_threshold
-            # (auto_gptq/nn_modules/qlinear.py:198-245).  Still GPU only.
+            # Long prompts (kernel_switch_threshold), or a shape the fused kernels do not cover
+            # (activation order with more groups than their LDS table holds): materialise W with
+            # the HIP dequant kernel and multiply with the library GEMM, which is what the reference
+            # does above its threshold (auto_gptq/nn_modules/qlinear.py:198-245).  Still GPU only.
             out = torch.matmul(x2, self.dequantize())
             if self.bias is not None:
                 out = out + self.bias

@@ -294,6 +294,19 @@ def test_quantlinear_forward(dev, bits):
     assert_close(q2(L2["x"].to(dev)), expected_output(L2), "module forward, contiguous groups")
 
 
+def test_module_switches_to_dequant_plus_library_gemm_for_long_prompts(dev):
+    K, N, gs = 256, 96, 64
+    L = layer(78, K, N, 3, gs, True, M=40, bias=True)
+    q = QuantLinear(3, gs, K, N, True, kernel_switch_threshold=32)
+    q.qweight, q.qzeros, q.scales, q.g_idx, q.bias = L["qweight"], L["qzeros"], L["scales"], L["g_idx"], L["bias"]
+    q = q.to(dev)
+    y_lib = q(L["x"].to(dev))                 # 40 rows >= 32: library GEMM on the materialised weight
+    q.kernel_switch_threshold = None
+    y_fused = q(L["x"].to(dev))               # fused kernel
+    assert_close(y_lib, expected_output(L), "library path")
+    assert_close(y_fused, expected_output(L), "fused path")
+
+
 def test_module_falls_back_to_dequant_plus_library_gemm_for_uncovered_shapes(dev):
     # activation order with more groups than any fused kernel's LDS table holds
     K, N, gs, M = 36864, 64, 32, 4
