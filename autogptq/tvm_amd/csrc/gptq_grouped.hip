@@ -126,7 +126,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     // ---- 3. weight loads, software-pipelined: a wave blocks while it issues loads into a full
     //         memory pipeline, so only the first PF steps go out now (they cover the LDS work
     //         below); step s + PF is issued right before step s is consumed ---------------
-    constexpr int PF = BITS == 4 ? 6 : 2;
+    constexpr int PF = BITS == 4 ? 8 : 1;
     u4 w[NSTEP][F::WORDS];
     auto load_step = [&](int s, int st) {  // register slot s <- step st
         const int prow = 4 * st + lq;
