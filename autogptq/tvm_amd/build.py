@@ -5,6 +5,7 @@
 """
 from __future__ import annotations
 
+import json
 import os
 import shutil
 import subprocess
@@ -44,14 +45,54 @@ def is_stale() -> bool:
     return any(os.path.getmtime(d) > t for d in deps)
 
 
+REPORT = os.path.join(CSRC, "kernel_resources.json")
+
+
+def parse_resource_remarks(text: str) -> dict:
+    """{kernel symbol: {"vgprs", "agprs", "scratch", "vgpr_spill", "sgpr_spill", "occupancy"}} from the
+    compiler's -Rpass-analysis=kernel-resource-usage remarks."""
+    keys = {"VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch", "VGPRs Spill": "vgpr_spill",
+            "SGPRs Spill": "sgpr_spill", "Occupancy [waves/SIMD]": "occupancy"}
+    res, cur = {}, None
+    for line in text.splitlines():
+        if "remark:" not in line:
+            continue
+        body = line.split("remark:", 1)[1].split("[-Rpass", 1)[0].strip()
+        if body.startswith("Function Name:"):
+            cur = res.setdefault(body.split(":", 1)[1].strip(), {})
+        elif cur is not None and ":" in body:
+            k, v = body.rsplit(":", 1)
+            if k.strip() in keys:
+                cur[keys[k.strip()]] = int(v)
+    return res
+
+
 def build(verbose: bool = False) -> str:
-    cmd = [hipcc()] + flags() + ["-o", LIB] + [os.path.join(CSRC, s) for s in SOURCES]
+    cmd = ([hipcc()] + flags() + ["-Rpass-analysis=kernel-resource-usage", "-o", LIB] +
+           [os.path.join(CSRC, s) for s in SOURCES])
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in proc.stdout.splitlines() if "is not a recognized feature" not in l)
+    report = parse_resource_remarks(proc.stdout)
+    noise = ("is not a recognized feature", "remark:", "-Rpass-analysis")
+    lines, skip = [], 0
+    for l in proc.stdout.splitlines():
+        if skip:          # the two source-echo lines that follow every remark
+            skip -= 1
+            continue
+        if "remark: Function Name" in l:
+            skip = 2
+        if not any(n in l for n in noise):
+            lines.append(l)
+    out = "\n".join(lines)
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + out)
-    if verbose and out.strip():
-        print(out)
+    with open(REPORT, "w", encoding="utf-8") as f:   # registers, scratch and spills per kernel
+        json.dump(report, f, indent=1, sort_keys=True)
+    spilled = sorted(k for k, v in report.items() if v.get("vgpr_spill", 0) or v.get("scratch", 0))
+    if verbose:
+        if out.strip():
+            print(out)
+        for k in spilled:
+            print(f"note: {k} spills {report[k].get('vgpr_spill', 0)} VGPRs ({report[k].get('scratch', 0)} B scratch/lane)")
     return LIB
 
 

@@ -32,8 +32,7 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
         if ((long long)pl.grid_x * 64 < N || pl.m_blocks < 1 || pl.grid_z != pl.m_blocks ||
             (long long)pl.m_blocks * 16 * pl.row_tiles < M)
             return GPTQ_HIP_ERR_BAD_ARG;
-        if (pl.split_k > 1 && (size_t)pl.grid_x * pl.grid_z * sizeof(int) > gptq::kCounterBytes)
-            return GPTQ_HIP_ERR_UNSUPPORTED;
+        if (pl.split_k > 1 && (long long)M * N >= (1LL << 32)) return GPTQ_HIP_ERR_UNSUPPORTED;  // reduce pass indexing
         const int wave_steps = gptq::stream_wave_steps(bits, steps_total, pl.split_k, pl.waves_k);
         // every workgroup along K must start inside K
         if ((long long)(pl.split_k - 1) * pl.waves_k * wave_steps >= steps_total) return GPTQ_HIP_ERR_BAD_ARG;

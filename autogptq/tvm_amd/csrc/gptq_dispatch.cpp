@@ -242,18 +242,18 @@ int plan_stream(int M, int K, int N, int bits, int gs, int G, int act_order, int
     const int col_tiles = ceil_div(N, 64);
     const long long tiles = (long long)col_tiles * m_blocks;
     const int act_table = gptq::stream_act_table(bits, gs, act_order);
-    const bool can_split = tiles * (long long)sizeof(int) <= (long long)gptq::kCounterBytes;  // one counter per tile
+    const bool can_split = (long long)M * N < (1LL << 32);  // indexing of the pass that adds the partial tiles
 
-    // Waves come from column tiles x M blocks x waves along K inside a workgroup (free: their
-    // tiles meet in LDS) x workgroups along K (dear: the partial tiles cross HBM twice and the
-    // last workgroup of a tile adds them alone).  Eight waves per workgroup while all workgroups
-    // still fit the chip at two waves per SIMD (2048 wave slots), else four; workgroups along K
-    // only when the tiles alone leave most CUs idle.
-    int waves_k = force_waves > 0 ? force_waves : (tiles * 8 <= 2048 ? 8 : 4);
+    // Waves come from column tiles x M blocks x waves along K inside a workgroup (their tiles meet in
+    // LDS) x workgroups along K (their fp32 tiles cross the workspace and a reduce pass adds them:
+    // ~3-4 us).  64-row tiles run four waves per workgroup (two workgroups share a CU); shorter
+    // tiles eight while all workgroups still fit the chip (2048 wave slots at two per SIMD).
+    // Workgroups along K bring the count to about one per CU (256); a long K per wave affords more.
+    int waves_k = force_waves > 0 ? force_waves : (rt == 4 ? 4 : (tiles * 8 <= 2048 ? 8 : 4));
     while (waves_k > 1 && waves_k * pf > steps_total) waves_k >>= 1;
-    int split = tiles >= 128 ? 1 : ceil_div(256, (int)tiles);
-    // a long K per wave pays for the cross-workgroup sum when the tiles alone leave CUs idle
-    if (tiles >= 128 && tiles < 256 && K / waves_k >= 2048) split = ceil_div(384, (int)tiles);
+    int split = (int)((256 + tiles / 2) / tiles);
+    if (split < 1) split = 1;
+    if (rt == 1 && tiles >= 128 && tiles < 256 && K / waves_k >= 2048) split = ceil_div(384, (int)tiles);
     int cap = (int)((3LL * K * bits) / (128LL * M));
     if (cap < 1) cap = 1;
     if (split > cap) split = cap;

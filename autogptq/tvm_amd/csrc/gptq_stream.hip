@@ -141,28 +141,45 @@ __device__ __forceinline__ void stage_table(const Params &p, int g_lo, int g_hi,
 }
 
 // B operands of one block: the reference's weights fp16(scale * (q - zero)) of 8 slots x 4 column
-// sets from the biased codes bq[c] (base + q).  (base + q) - (base + zero) is exact, so the one
-// rounding is the product's.  ent[s][c]: (scale, zero) of slot s (ACT) / erow[c]: of all slots.
+// sets from the biased codes bqn[c] (base + q).  (base + q) - (base + zero) is exact, so the one
+// rounding is the product's.  eoff[s]: LDS byte offset of the (scale, zero) entries of slot s
+// (ACT); erow[c]: the entry shared by all slots.
 template <int BITS, bool ACT>
-__device__ __forceinline__ void dequant_block(const u4 (&bqn)[4], const u4 (&ent)[8], const u4 &erow, h8 (&bop)[4])
+__device__ __forceinline__ void dequant_block(const u4 (&bqn)[4], const uint32_t (&eoff)[8], const u4 &erow,
+                                              h8 (&bop)[4])
 {
+    // int3 tiles are the ones short of registers: they take the table in two rounds of four slots
+    constexpr int ROUNDS = BITS == 3 ? 2 : 1;
+    constexpr int SPR = 8 / ROUNDS;  // slots per round
+    u4 wv[4];
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
-        u4 wv;
+    for (int round = 0; round < ROUNDS; round++) {
+        u4 ent[SPR];
+        if constexpr (ACT) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            // (scale, zero) of the two slots of register r: low halves / high halves
-            const uint32_t ea = ACT ? ent[2 * r][c] : erow[c];
-            const uint32_t eb = ACT ? ent[2 * r + 1][c] : erow[c];
-            const h2 s2 = as_h2(__builtin_amdgcn_perm(eb, ea, 0x05040100u));
-            const h2 z2 = as_h2(__builtin_amdgcn_perm(eb, ea, 0x07060302u));
-            const float ba = BITS == 4 ? BASE4[2 * r] : BASE3[2 * r];
-            const float bb = BITS == 4 ? BASE4[2 * r + 1] : BASE3[2 * r + 1];
-            const h2 zb = z2 + (h2){(_Float16)ba, (_Float16)bb};  // exact: small integers
-            wv[r] = as_u32((as_h2(bqn[c][r]) - zb) * s2);
+            for (int s = 0; s < SPR; s++) ent[s] = *(const u4 *)(smem + eoff[SPR * round + s]);
         }
-        bop[c] = __builtin_bit_cast(h8, wv);
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+#pragma unroll
+            for (int rr = 0; rr < SPR / 2; rr++) {
+                const int r = (SPR / 2) * round + rr;
+                // (scale, zero) of the two slots of register r: low halves / high halves
+                const uint32_t ea = ACT ? ent[2 * rr][c] : erow[c];
+                const uint32_t eb = ACT ? ent[2 * rr + 1][c] : erow[c];
+                const h2 s2 = as_h2(__builtin_amdgcn_perm(eb, ea, 0x05040100u));
+                const h2 z2 = as_h2(__builtin_amdgcn_perm(eb, ea, 0x07060302u));
+                const float ba = BITS == 4 ? BASE4[2 * r] : BASE3[2 * r];
+                const float bb = BITS == 4 ? BASE4[2 * r + 1] : BASE3[2 * r + 1];
+                const h2 zb = z2 + (h2){(_Float16)ba, (_Float16)bb};  // exact: small integers
+                wv[c][r] = as_u32((as_h2(bqn[c][r]) - zb) * s2);
+            }
+        }
+        // keeps the next round's table reads below this point (everything else may cross)
+        if constexpr (ACT && ROUNDS > 1) __builtin_amdgcn_sched_barrier(0x067f);
     }
+#pragma unroll
+    for (int c = 0; c < 4; c++) bop[c] = __builtin_bit_cast(h8, wv[c]);
 }
 
 // The waves of the workgroup add their tiles through LDS in a fixed tree; wave 0 ends up with the sum.
@@ -190,11 +207,11 @@ __device__ __forceinline__ void reduce_waves(f4 (&acc)[RT][4], int wave, int WK,
     }
 }
 
-// Epilogue of wave 0: acc[rt][c][v] is y[m0 + 16 rt + 4 q + v][n0 + c]; bias, fp16, or the
-// split-K exchange through the workspace.  Every thread of the workgroup calls it.
+// Epilogue of wave 0: acc[rt][c][v] is y[m0 + 16 rt + 4 q + v][n0 + c]; bias and fp16, or, when K
+// is split over workgroups, the fp32 tile into the workspace.
 template <int RT>
 __device__ __forceinline__ void write_out(const Params &p, f4 (&acc)[RT][4], bool owner, int m0, int rows_here,
-                                          int n0, int lq, int split, int *last_flag)
+                                          int n0, int lq, int split)
 {
     const _Float16 *bias = (const _Float16 *)p.bias;
     f4 bv = {0.f, 0.f, 0.f, 0.f};
@@ -221,6 +238,10 @@ __device__ __forceinline__ void write_out(const Params &p, f4 (&acc)[RT][4], boo
         }
         return;
     }
+    // split_k > 1: the fp32 tile goes to the workspace with plain stores; reduce_kernel, launched
+    // right behind this kernel on the same stream, adds the split_k tiles in order and writes y.
+    // (The in-kernel alternative, a counter and the last workgroup summing, costs three dependent
+    // round trips to device-coherent memory and slow 64-bit coherent stores for tall tiles.)
     if (owner) {
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
@@ -229,32 +250,31 @@ __device__ __forceinline__ void write_out(const Params &p, f4 (&acc)[RT][4], boo
                 const int row = 16 * rt + 4 * lq + v;
                 if (row < rows_here) {
                     const f4 o = {acc[rt][0][v], acc[rt][1][v], acc[rt][2][v], acc[rt][3][v]};
-                    store_partial(p.partial + ((size_t)split * p.M + (m0 + row)) * p.N + n0, o);
+                    *(f4 *)(p.partial + ((size_t)split * p.M + (m0 + row)) * p.N + n0) = o;
                 }
             }
         }
     }
-    int *counter = p.counters + blockIdx.z * gridDim.x + blockIdx.x;
-    if (!arrive_last(counter, p.split_k, last_flag)) return;
-    if (owner) {
-#pragma unroll
-        for (int rt = 0; rt < RT; rt++) {
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const int row = 16 * rt + 4 * lq + v;
-                if (row < rows_here) {
-                    f4 sum = bv;
-                    for (int s = 0; s < p.split_k; s++) {
-                        sum += load_partial(p.partial + ((size_t)s * p.M + (m0 + row)) * p.N + n0);
-                    }
-                    h4 o;
-#pragma unroll
-                    for (int c = 0; c < 4; c++) o[c] = (_Float16)sum[c];
-                    *(h4 *)(y + (size_t)(m0 + row) * p.N + n0) = o;
-                }
-            }
-        }
+}
+
+// y = fp16(sum over split of partial[split] (+ bias)), four columns per thread, in split order.
+__global__ __launch_bounds__(256) void reduce_kernel(const Params p)
+{
+    const uint32_t q = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t nq = (uint32_t)p.N / 4u;
+    if (q >= (uint32_t)p.M * nq) return;
+    const uint32_t row = q / nq;
+    const uint32_t col = 4u * (q - row * nq);
+    f4 sum = {0.f, 0.f, 0.f, 0.f};
+    if (p.bias) {
+        const h4 b4 = *(const h4 *)((const _Float16 *)p.bias + col);
+        sum = (f4){(float)b4[0], (float)b4[1], (float)b4[2], (float)b4[3]};
     }
+    for (int s = 0; s < p.split_k; s++) sum += *(const f4 *)(p.partial + ((size_t)s * p.M + row) * p.N + col);
+    h4 o;
+#pragma unroll
+    for (int c = 0; c < 4; c++) o[c] = (_Float16)sum[c];
+    *(h4 *)((_Float16 *)p.y + (size_t)row * p.N + col) = o;
 }
 
 // Global loads return in order (one counter), so a wait for any load also waits for every older
@@ -292,7 +312,6 @@ __global__ __launch_bounds__(512) void stream_kernel(const Params p)
     const int s_begin = split * WK * p.wave_steps;
     const int ws = s_begin + wave * p.wave_steps;
     const int prows = p.K / (BITS == 4 ? 8 : 32);
-    __shared__ int last_flag;
 
     // ---- register rings --------------------------------------------------------------------
     // Addresses are a wave-uniform base (step or block number, in scalar registers) plus a
@@ -398,20 +417,22 @@ __global__ __launch_bounds__(512) void stream_kernel(const Params p)
                         biased3_block(w[u][0][c], w[u][1][c], w[u][2][c], nb, bq[c][nb], magic_a, magic_b);
                 }
                 h8 bop[4];
-                u4 ent[8];
-                if constexpr (ACT) {
-#pragma unroll
-                    for (int s = 0; s < 8; s++) {
-                        const uint32_t off = s < 4 ? go[slot][0][s & 3] : go[slot][1][s & 3];
-                        ent[s] = *(const u4 *)(smem + (off + (uint32_t)tab_bias));
-                    }
-                    load_go(b + AD, go[slot]);
-                }
                 {
+                    uint32_t eoff[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+                    if constexpr (ACT) {
+#pragma unroll
+                        for (int s = 0; s < 8; s++) {
+                            eoff[s] = (s < 4 ? go[slot][0][s & 3] : go[slot][1][s & 3]) + (uint32_t)tab_bias;
+                        }
+                    }
+                    // refill with the offsets of the block AD ahead; where the request is issued
+                    // relative to the table reads is measured per width (int3 before, int4 after)
+                    if constexpr (ACT && BITS == 3) load_go(b + AD, go[slot]);
                     u4 bqn[4];
 #pragma unroll
                     for (int c = 0; c < 4; c++) bqn[c] = bq[c][nb];
-                    dequant_block<BITS, ACT>(bqn, ent, erow, bop);
+                    dequant_block<BITS, ACT>(bqn, eoff, erow, bop);
+                    if constexpr (ACT && BITS == 4) load_go(b + AD, go[slot]);
                 }
 #pragma unroll
                 for (int rt = 0; rt < RT; rt++) {
@@ -431,7 +452,7 @@ __global__ __launch_bounds__(512) void stream_kernel(const Params p)
     }
 
     reduce_waves<RT>(acc, wave, WK, lane);
-    write_out<RT>(p, acc, wave == 0 && n_ok, m0, rows_here, n0, lq, split, &last_flag);
+    write_out<RT>(p, acc, wave == 0 && n_ok, m0, rows_here, n0, lq, split);
 }
 
 
@@ -472,7 +493,6 @@ __global__ __launch_bounds__(512) void stream_direct_kernel(const Params p)
     const int ws = s_begin + wave * p.wave_steps;
     const int prows = p.K / F::KLANE;  // lane blocks along K
     const int last_step = p.steps_total - 1;
-    __shared__ int last_flag;
 
     const uint32_t n_ld = (uint32_t)min(n0, p.N - 4);
     const uint32_t x_row = (uint32_t)min(li, p.M - 1) * (uint32_t)p.K * 2u;
@@ -564,16 +584,16 @@ __global__ __launch_bounds__(512) void stream_direct_kernel(const Params p)
             STREAM_PIN_LOADS();
 #pragma unroll
             for (int nb = 0; nb < F::NB; nb++) {
-                u4 ent[8];
+                uint32_t eoff[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
                 if constexpr (ACT) {
 #pragma unroll
-                    for (int s = 0; s < 8; s++) ent[s] = *(const u4 *)(smem + go[8 * nb + s]);
+                    for (int s = 0; s < 8; s++) eoff[s] = go[8 * nb + s];
                 }
                 u4 bqn[4];
 #pragma unroll
                 for (int c = 0; c < 4; c++) bqn[c] = bq[c][nb];
                 h8 bop[4];
-                dequant_block<BITS, ACT>(bqn, ent, erow, bop);
+                dequant_block<BITS, ACT>(bqn, eoff, erow, bop);
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
                     acc[0][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[nb], bop[c], acc[0][c], 0, 0, 0);
@@ -582,7 +602,15 @@ __global__ __launch_bounds__(512) void stream_direct_kernel(const Params p)
         }
     }
     reduce_waves<1>(acc, wave, WK, lane);
-    write_out<1>(p, acc, wave == 0 && n_ok, 0, min(16, p.M), n0, lq, split, &last_flag);
+    write_out<1>(p, acc, wave == 0 && n_ok, 0, min(16, p.M), n0, lq, split);
+}
+
+static int launch_reduce(const Params &p, hipStream_t stream)
+{
+    if (p.split_k == 1) return GPTQ_HIP_OK;
+    const uint32_t quads = (uint32_t)p.M * ((uint32_t)p.N / 4u);
+    hipLaunchKernelGGL(reduce_kernel, dim3((quads + 255u) / 256u), dim3(256), 0, stream, p);
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 
 template <int BITS, int RT, bool ACT>
@@ -601,7 +629,8 @@ static int launch_stream_one(const Params &p, const gptq_hip_plan &plan, hipStre
         if constexpr (RT == 1) {
             auto kd = stream_direct_kernel<BITS, ACT>;
             hipLaunchKernelGGL(kd, grid_d, dim3(plan.block), plan.lds_bytes, stream, p);
-            return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+            if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ERR_LAUNCH;
+            return launch_reduce(p, stream);
         } else {
             return GPTQ_HIP_ERR_BAD_ARG;
         }
@@ -611,7 +640,8 @@ static int launch_stream_one(const Params &p, const gptq_hip_plan &plan, hipStre
     if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ERR_LAUNCH;
     const dim3 grid(plan.grid_x, plan.grid_y, plan.grid_z);
     hipLaunchKernelGGL(kern, grid, dim3(plan.block), plan.lds_bytes, stream, p);
-    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+    if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ERR_LAUNCH;
+    return launch_reduce(p, stream);
 }
 
 template <int BITS, bool ACT>
