@@ -321,6 +321,7 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     memset(plan, 0, sizeof(*plan));
     if (plan_stream(M, K, N, bits, gs, G, act_order, 0, 0, plan) == GPTQ_HIP_OK) return GPTQ_HIP_OK;
     memset(plan, 0, sizeof(*plan));
+    // last resort (its table limit is tighter than STREAM's, so this rarely finds a plan either)
     return plan_gather(M, K, N, bits, G, 0, 0, plan);
 }
 
