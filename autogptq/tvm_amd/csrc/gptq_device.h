@@ -11,7 +11,8 @@
 // int3: one 3-word block = 32 codes = four MFMAs), and the activation operand
 // supplies x for the same input channels in the same order.  That order is the
 // "slot" order of gptq_unpack.h (codes come out of the magic-number unpack in pairs
-// that are not adjacent in k); x is written to LDS already permuted into slot order.
+// that are not adjacent in k); x reaches the matrix instruction already permuted into slot order
+// (in LDS for GROUPED and GATHER, by the pack pass or register permutes for STREAM).
 //
 // One "step" of a wave is 4 packed rows (int4: 32 input channels, int3: 128).
 #pragma once

@@ -1,10 +1,10 @@
-// STREAM kernel family: the matmul for M >= 3 (prompt processing and batched decoding).
+// STREAM kernel family: the matmul for M >= 2 (batched decoding and prompt processing).
 //
-// Two launches per call.
+// Up to three launches per call.
 //
-// 1. pack_kernel rewrites x [M, K] into the order the matrix instruction wants it: for every
-//    block of 32 input channels and every 16-row tile, the 64 x 16 bytes that the 64 lanes of a
-//    wave hand to v_mfma_f32_16x16x32_f16 as its A operand, lane after lane (1 KiB per
+// 1. pack_kernel (M > 16) rewrites x [M, K] into the order the matrix instruction wants it: for
+//    every block of 32 input channels and every 16-row tile, the 64 x 16 bytes that the 64 lanes
+//    of a wave hand to v_mfma_f32_16x16x32_f16 as its A operand, lane after lane (1 KiB per
 //    fragment), with the 8 values of a lane already in the slot order in which the weight
 //    codes leave the unpack.  Rows past M and channels past K are written as zeros, and the
 //    channel range is padded to what the matmul waves walk.  It also writes, per block and
@@ -22,8 +22,12 @@
 //    Weights, group offsets and A fragments arrive through register rings that are refilled
 //    right after use; two waves per SIMD cover what latency is left.
 //    The (scale, zero) pairs of the 64 columns live in LDS, [groups][64] + padding.
-//    split_k > 1 adds workgroups along K whose partial tiles meet through the workspace.
-// grid = (column tiles, split_k, m blocks), block = 64 * waves_k.
+//    stream_direct_kernel is the same walk for one row tile (M <= 16) without the pack pass:
+//    its lanes read x and g_idx themselves.
+//
+// 3. reduce_kernel (split_k > 1): the workgroups along K leave fp32 tiles in the workspace; this
+//    pass adds them in split order, adds the bias and writes y.
+// grid of the matmul = (column tiles, split_k, m blocks), block = 64 * waves_k.
 #include "gptq_device.h"
 
 namespace gptq {
