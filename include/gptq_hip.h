@@ -38,8 +38,9 @@ typedef enum gptq_hip_status {
 enum {
     GPTQ_HIP_KERNEL_GATHER = 1, /* exact fp16 weights, x staged through LDS by the workgroup; any g_idx, any M */
     GPTQ_HIP_KERNEL_GROUPED = 2, /* rows expanded by group, scales applied once per group; M <= 2, few groups */
-    GPTQ_HIP_KERNEL_STREAM = 3  /* exact fp16 weights, x pre-packed into fragment order (always needs the
-                                   workspace), independent waves; any g_idx, any M */
+    GPTQ_HIP_KERNEL_STREAM = 3  /* exact fp16 weights, independent waves along K; any g_idx, any M.  M > 16: x is
+                                   pre-packed into matrix-instruction fragment order (needs the workspace);
+                                   M <= 16: the kernel reads x itself.  split_k > 1 adds a reduce launch. */
 };
 
 /* What the dispatcher decided for one problem; filled by gptq_hip_select. */
@@ -68,14 +69,16 @@ int gptq_hip_select(int M, int K, int N, int bits, int group_size, int act_order
 
 /*
  * The plan of one kernel family with split_k and waves_n forced (0 = let the dispatcher
- * choose); GPTQ_HIP_ERR_UNSUPPORTED when that family does not cover the problem.  For
- * benchmarks and tests of single kernels; the reference's counterpart is editing the tile
- * parameters of one handler-database entry (pycuda_warpper.py:77-127).
+ * choose; for GPTQ_HIP_KERNEL_STREAM waves_n is the number of waves along K: 1, 2, 4 or 8);
+ * GPTQ_HIP_ERR_UNSUPPORTED when that family does not cover the problem.  For benchmarks and
+ * tests of single kernels; the reference's counterpart is editing the tile parameters of one
+ * handler-database entry (pycuda_warpper.py:77-127).
  */
 int gptq_hip_plan_for(int kernel, int M, int K, int N, int bits, int group_size, int act_order, int split_k,
                       int waves_n, gptq_hip_plan *plan);
 
-/* Bytes of workspace gptq_hip_gemm needs for this problem (0 if none). */
+/* Bytes of workspace gptq_hip_gemm needs for this problem (0 if none): split-K counters and
+ * partial tiles, and for M > 16 the pre-packed activations. */
 size_t gptq_hip_workspace_bytes(int M, int K, int N, int bits, int group_size, int act_order);
 
 /*
@@ -90,7 +93,8 @@ int gptq_hip_workspace_init(void *workspace, size_t workspace_bytes, void *strea
  * Replaces the reference's handler call
  *   handler(x, qweight, y, scales, zeros)   (pycuda_warpper.py:138, qlinear_tvm.py:123,150)
  * and computes what qlinear.py:198-245 computes.  Unlike the reference, y is
- * written for exactly M rows (no padded rows) and need not be pre-zeroed.
+ * written for exactly M rows (no padded rows) and need not be pre-zeroed.  One to three kernel
+ * launches on `stream` (pack pass for M > 16, matmul, reduce pass when the plan splits K).
  */
 int gptq_hip_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                   const int32_t *g_idx, const void *bias, void *y, void *workspace, size_t workspace_bytes,
