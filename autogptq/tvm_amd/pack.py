@@ -52,6 +52,63 @@ def pack_qzeros(zeros: np.ndarray, bits: int) -> np.ndarray:
     return np.ascontiguousarray(pack_along_axis0(np.ascontiguousarray(z.T), bits).T)
 
 
+def unpack_along_axis0(words: np.ndarray, bits: int) -> np.ndarray:
+    """Inverse of pack_along_axis0: int32 [R//32*bits, C] -> codes uint8 [R, C]."""
+    if bits not in (3, 4):
+        raise NotImplementedError("Only 3 and 4 bits are supported.")
+    w = np.ascontiguousarray(words).view(np.uint32)
+    rows, cols = w.shape
+    if rows % bits != 0:
+        raise ValueError(f"{rows} packed rows are not a multiple of bits={bits}")
+    if bits == 4:
+        shifts = (4 * np.arange(8, dtype=np.uint32)).reshape(1, 8, 1)
+        return ((w[:, None, :] >> shifts) & np.uint32(15)).astype(np.uint8).reshape(rows * 8, cols)
+    b = w.reshape(rows // 3, 3, cols).astype(np.uint64)
+    lo = b[:, 0, :] | (b[:, 1, :] << np.uint64(32))       # stream bits 0..63
+    hi = (b[:, 1, :] >> np.uint64(31)) | (b[:, 2, :] << np.uint64(1))  # stream bits 63..95 at bit 0
+    out = np.empty((rows // 3, 32, cols), dtype=np.uint8)
+    for j in range(32):
+        bit = 3 * j
+        if bit + 3 <= 64:
+            out[:, j, :] = ((lo >> np.uint64(bit)) & np.uint64(7)).astype(np.uint8)
+        else:
+            out[:, j, :] = ((hi >> np.uint64(bit - 63)) & np.uint64(7)).astype(np.uint8)
+    return out.reshape(rows // 3 * 32, cols)
+
+
+def sort_channels_by_group(qweight: torch.Tensor, g_idx: torch.Tensor, bits: int, group_size: int):
+    """Load-time preparation for activation-order checkpoints: reorders the input channels so that
+    every group is contiguous, which lets the decode kernel treat the layer like one without
+    ``g_idx``.  Returns ``(qweight_sorted int32 [K//32*bits, N], kmap int32 [K])`` on the CPU, or
+    ``None`` when the layer does not qualify.
+
+    Sorted position j holds original channel perm[j] (stable sort by group).  ``kmap[k]`` tells the
+    kernel where original channel k goes: low 16 bits = its position inside the sorted K range with
+    the codes of each lane block (8 channels for int4, 32 for int3) already in the order the
+    kernels' register unpack produces them, high 16 bits = its group.  Requires K < 65536, every
+    group (but the last) to hold exactly ``group_size`` channels, and ``group_size`` to be a
+    multiple of the lane block."""
+    from . import _slots
+
+    K = int(g_idx.numel())
+    gs = K if group_size == -1 else group_size
+    klane = 8 if bits == 4 else 32
+    if K >= 65536 or gs % klane != 0 or K % 32 != 0:
+        return None
+    g = g_idx.detach().cpu().to(torch.int64)
+    perm = torch.argsort(g, stable=True)
+    if not torch.equal(g[perm], torch.arange(K, dtype=torch.int64) // gs):
+        return None
+    codes = unpack_along_axis0(qweight.detach().cpu().numpy(), bits)
+    qweight_sorted = torch.from_numpy(pack_along_axis0(codes[perm.numpy()], bits))
+    inv = torch.empty(K, dtype=torch.int64)
+    inv[perm] = torch.arange(K, dtype=torch.int64)          # original k -> sorted position
+    slot_of_code = torch.tensor(_slots.slot_of_code(bits), dtype=torch.int64)
+    pos = (inv // klane) * klane + slot_of_code[inv % klane]
+    kmap = (pos | ((inv // gs) << 16)).to(torch.int32)
+    return qweight_sorted, kmap
+
+
 def num_groups(k: int, group_size: int) -> int:
     gs = k if group_size == -1 else group_size
     return math.ceil(k / gs)

@@ -104,5 +104,10 @@ int main()
         return 1;
     }
     printf("ok %ld\n", checked);
+    printf("slot4");
+    for (int i = 0; i < 8; i++) printf(" %d", SLOT4[i]);
+    printf("\nslot3");
+    for (int i = 0; i < 32; i++) printf(" %d", SLOT3[i]);
+    printf("\n");
     return 0;
 }

@@ -130,3 +130,48 @@ def test_oracle_unpacks_reference_packed_tensors(name):
     deq = orc.dequant_ref(torch.from_numpy(qweight), torch.from_numpy(qzeros),
                           torch.from_numpy(scales16.copy()), torch.from_numpy(g_idx), bits).float().numpy()
     assert np.all(np.abs(deq - W) <= 0.5 * s * 1.01 + 1e-3)         # within half a quantisation step
+
+
+# ---------------------------------------------------------------------------------------------
+# Load-time preparation of activation-order layers: channels sorted by group.
+@pytest.mark.parametrize("bits", [3, 4])
+def test_unpack_is_the_inverse_of_pack(bits):
+    rng = np.random.default_rng(bits + 40)
+    codes = rng.integers(0, 1 << bits, size=(224, 7)).astype(np.uint8)
+    assert np.array_equal(pack.unpack_along_axis0(pack.pack_along_axis0(codes, bits), bits), codes)
+    words = rng.integers(-(1 << 31), 1 << 31, size=(12, 5)).astype(np.int32)
+    assert np.array_equal(pack.unpack_along_axis0(words, bits), orc.unpack_bitstream(words, bits, axis=0))
+
+
+@pytest.mark.parametrize("bits,K,gs", [(4, 256, 32), (3, 256, 64), (3, 128, -1), (4, 96, 8)])
+def test_sort_channels_by_group_preserves_the_layer(bits, K, gs):
+    from autogptq.tvm_amd import _slots
+
+    N = 32
+    L = pack.synth_layer(90 + bits, K, N, bits, gs, True)
+    res = pack.sort_channels_by_group(L["qweight"], L["g_idx"], bits, gs)
+    assert res is not None
+    qs, kmap = res
+    assert qs.shape == L["qweight"].shape and qs.dtype == torch.int32 and kmap.shape == (K,)
+    g = K if gs == -1 else gs
+    klane = 8 if bits == 4 else 32
+    pos, grp = (kmap & 0xFFFF).long(), (kmap >> 16).long()
+    assert torch.equal(grp, L["g_idx"].long())
+    # undo the slot order to get the sorted position of every original channel
+    code_of_slot = torch.tensor(_slots.code_of_slot(bits))
+    sorted_pos = (pos // klane) * klane + code_of_slot[pos % klane]
+    assert sorted(sorted_pos.tolist()) == list(range(K))            # a permutation
+    assert torch.equal(sorted_pos // g, L["g_idx"].long())           # groups became contiguous
+    # the sorted layer with contiguous groups dequantises to the original weight rows, permuted
+    w_orig = orc.dequant_ref(L["qweight"], L["qzeros"], L["scales"], L["g_idx"], bits)
+    contiguous = (torch.arange(K) // g).to(torch.int32)
+    w_sorted = orc.dequant_ref(qs, L["qzeros"], L["scales"], contiguous, bits)
+    assert torch.equal(w_sorted[sorted_pos], w_orig)
+
+
+def test_sort_channels_declines_what_it_cannot_sort():
+    L = pack.synth_layer(7, 128, 32, 4, 32, True)
+    g = L["g_idx"].clone()
+    g[g == 3] = 2                                   # uneven groups
+    assert pack.sort_channels_by_group(L["qweight"], g, 4, 32) is None
+    assert pack.sort_channels_by_group(L["qweight"], L["g_idx"], 3, 16) is None   # group narrower than a lane block

@@ -27,3 +27,9 @@ def test_magic_unpack_matches_bit_extraction(tmp_path):
     out = subprocess.run([str(exe)], stdout=subprocess.PIPE, text=True)
     assert out.returncode == 0, out.stdout
     assert out.stdout.startswith("ok ")
+    # the Python mirror of the slot tables (used by the load-time channel sort) matches the header
+    from autogptq.tvm_amd import _slots
+
+    lines = {l.split()[0]: [int(v) for v in l.split()[1:]] for l in out.stdout.splitlines()[1:]}
+    assert lines["slot4"] == _slots.CODE_OF_SLOT4
+    assert lines["slot3"] == _slots.CODE_OF_SLOT3
