@@ -86,10 +86,10 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
 
 }  // namespace
 
-extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
-                                  const int32_t *g_idx, const void *bias, void *y, void *workspace,
-                                  size_t workspace_bytes, int M, int K, int N, int bits, int group_size,
-                                  const gptq_hip_plan *plan, void *stream)
+// kmap != nullptr: qweight holds the channels sorted by group (g_idx must then be nullptr)
+static int run_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *g_idx,
+             const int32_t *kmap, const void *bias, void *y, void *workspace, size_t workspace_bytes, int M, int K,
+             int N, int bits, int group_size, const gptq_hip_plan *plan, void *stream)
 {
     if (!x || !y || !plan || M < 1) return GPTQ_HIP_ERR_BAD_ARG;
     int rc = check_common(qweight, qzeros, scales, K, N, bits, group_size);
@@ -138,6 +138,14 @@ extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const i
     p.direct = 0;
     p.gdiv_magic = 0;
     p.gdiv_add = 0;
+    p.kmap = nullptr;
+    p.wave_div_magic = 0;
+    if (kmap) {
+        // positions are below 65536 and a wave holds at least one step: the multiply-high is exact
+        if (plan->kernel != GPTQ_HIP_KERNEL_GROUPED) return GPTQ_HIP_ERR_UNSUPPORTED;
+        p.kmap = kmap;
+        p.wave_div_magic = (uint32_t)((1ull << 32) / (uint32_t)(p.wave_steps * kstep)) + 1u;
+    }
     if (plan->kernel == GPTQ_HIP_KERNEL_STREAM) {
         // workspace: counters | partial tiles (split_k > 1) | packed x | packed table offsets
         p.wave_steps = gptq::stream_wave_steps(bits, p.steps_total, plan->split_k, plan->waves_k);
@@ -186,6 +194,36 @@ extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const i
     }
     if (plan->kernel == GPTQ_HIP_KERNEL_GROUPED) return gptq::launch_grouped(p, bits, *plan, stream);
     return gptq::launch_gather(p, bits, *plan, stream);
+}
+
+extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                                  const int32_t *g_idx, const void *bias, void *y, void *workspace,
+                                  size_t workspace_bytes, int M, int K, int N, int bits, int group_size,
+                                  const gptq_hip_plan *plan, void *stream)
+{
+    return run_gemm(x, qweight, qzeros, scales, g_idx, nullptr, bias, y, workspace, workspace_bytes, M, K, N, bits,
+                    group_size, plan, stream);
+}
+
+extern "C" int gptq_hip_gemm_sorted(const void *x, const int32_t *qweight_sorted, const int32_t *qzeros,
+                                    const void *scales, const int32_t *kmap, const void *bias, void *y,
+                                    void *workspace, size_t workspace_bytes, int M, int K, int N, int bits,
+                                    int group_size, const gptq_hip_plan *plan, void *stream)
+{
+    if (!kmap || !aligned(kmap, 16)) return GPTQ_HIP_ERR_BAD_ARG;
+    if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
+    const int gs = group_size == -1 ? K : group_size;
+    // the map holds 16-bit positions; a group is a whole number of unpack blocks
+    if (K >= 65536 || K % gs != 0 || gs % (bits == 4 ? 8 : 32) != 0) return GPTQ_HIP_ERR_UNSUPPORTED;
+    gptq_hip_plan chosen;
+    if (!plan) {
+        const int rc = gptq_hip_select(M, K, N, bits, group_size, 0, &chosen);
+        if (rc != GPTQ_HIP_OK) return rc;
+        plan = &chosen;
+    }
+    if (plan->kernel != GPTQ_HIP_KERNEL_GROUPED) return GPTQ_HIP_ERR_UNSUPPORTED;
+    return run_gemm(x, qweight_sorted, qzeros, scales, nullptr, kmap, bias, y, workspace, workspace_bytes, M, K, N,
+                    bits, group_size, plan, stream);
 }
 
 extern "C" int gptq_hip_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,

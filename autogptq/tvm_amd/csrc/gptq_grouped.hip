@@ -26,6 +26,11 @@
 //             per 8 slots saying which slots belong to groups < 16.  The two row tiles
 //             are that tile AND mask / AND NOT mask: half the LDS, so K = 4096 with 32
 //             groups fits one workgroup.
+//
+// Sorted layers: when the loader has sorted the channels of an activation-order layer by
+// group (qweight rows permuted, p.kmap saying where each original channel went), the groups
+// are contiguous for the weight stream and only the scatter of x follows the map: every
+// workgroup walks all of x and keeps the channels whose sorted position falls in its K range.
 #include "gptq_device.h"
 
 namespace gptq {
@@ -73,6 +78,9 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     const int wave_k = p.wave_steps * F::KSTEP;  // channels per wave
     const int g_base = p.g_idx ? 0 : (ws * F::KSTEP) / p.group_size;
     __shared__ int last_flag;
+    __shared__ int wave_gb[8];  // sorted layers: first group of each wave along K
+    const int32_t *kmap = p.kmap;
+    if (kmap && tid < WK) wave_gb[tid] = (k_base + tid * wave_k) / p.group_size;
 
     const _Float16 *x = (const _Float16 *)p.x;
     const _Float16 *scales = (const _Float16 *)p.scales;
@@ -88,7 +96,8 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     for (int e = 0; e < 4; e++) qslot[e] = slot_of_code<BITS>((4 * tid) % F::KLANE + e);
     // ---- 1. x and g_idx of the K range: four channels per thread per pass ---------------
     constexpr int QP = 2;  // passes kept in registers so that their loads are the first to return
-    const int qpr = kspan / 4;  // quads per activation row
+    const int scan_base = kmap ? 0 : k_base;     // a sorted layer's channels may sit anywhere in x
+    const int qpr = (kmap ? p.K : kspan) / 4;    // quads per activation row
     const int nquads = qpr * M;
     int gq[QP][4];
     h4 xq[QP];
@@ -100,11 +109,11 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         for (int e = 0; e < 4; e++) gq[ps][e] = 0;
         if (idx < nquads) {
             const int m = M == 1 ? 0 : idx / qpr;
-            const int k = k_base + 4 * (idx - m * qpr);
+            const int k = scan_base + 4 * (idx - m * qpr);
             if (k < p.K) {  // K % 4 == 0: a quad is inside or outside as a whole
                 xq[ps] = *(const h4 *)(x + (size_t)m * p.K + k);
-                if (p.g_idx) {
-                    const int4 gv = *(const int4 *)(p.g_idx + k);
+                if (p.g_idx || kmap) {
+                    const int4 gv = *(const int4 *)((kmap ? kmap : p.g_idx) + k);
                     gq[ps][0] = gv.x;
                     gq[ps][1] = gv.y;
                     gq[ps][2] = gv.z;
@@ -182,13 +191,27 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
             ((_Float16 *)tiles)[((b8 * ST + m * TPM + (rr >> 4)) * 16 + (rr & 15)) * 8 + (slot & 7)] = xv;
         }
     };
+    // sorted layer: the map gives position (already in unpack order) and group; channels of other
+    // K ranges are dropped
+    auto scatter_mapped = [&](int m, int entry, _Float16 xv) {
+        const int kc = (entry & 0xffff) - k_base;
+        if ((unsigned)kc < (unsigned)kspan) {
+            const int gb = wave_gb[__umulhi((uint32_t)kc, p.wave_div_magic)];
+            scatter(m, kc, kc % F::KLANE, entry >> 16, gb, xv);
+        }
+    };
 #pragma unroll
     for (int ps = 0; ps < QP; ps++) {
         const int idx = tid + ps * nthreads;
         if (idx < nquads) {
             const int m = M == 1 ? 0 : idx / qpr;
             const int kc = 4 * (idx - m * qpr);
-            if (k_base + kc < p.K) {
+            if (kmap) {
+                if (kc < p.K) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) scatter_mapped(m, gq[ps][e], xq[ps][e]);
+                }
+            } else if (k_base + kc < p.K) {
                 const int gb = p.g_idx ? 0 : (k_base + (kc / wave_k) * wave_k) / p.group_size;
 #pragma unroll
                 for (int e = 0; e < 4; e++) scatter(m, kc + e, qslot[e], gq[ps][e], gb, xq[ps][e]);
@@ -198,8 +221,17 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     for (int idx = tid + QP * nthreads; idx < nquads; idx += nthreads) {  // long K ranges
         const int m = M == 1 ? 0 : idx / qpr;
         const int kc = 4 * (idx - m * qpr);
-        const int k = k_base + kc;
-        if (k < p.K) {
+        const int k = scan_base + kc;
+        if (kmap) {
+            if (k < p.K) {
+                const h4 xv = *(const h4 *)(x + (size_t)m * p.K + k);
+                const int4 mv = *(const int4 *)(kmap + k);
+                scatter_mapped(m, mv.x, xv[0]);
+                scatter_mapped(m, mv.y, xv[1]);
+                scatter_mapped(m, mv.z, xv[2]);
+                scatter_mapped(m, mv.w, xv[3]);
+            }
+        } else if (k < p.K) {
             const h4 xv = *(const h4 *)(x + (size_t)m * p.K + k);
             const int gb = p.g_idx ? 0 : (k_base + (kc / wave_k) * wave_k) / p.group_size;
 #pragma unroll

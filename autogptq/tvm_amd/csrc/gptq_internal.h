@@ -37,6 +37,10 @@ struct Params {
     int direct;        // 1: no pack pass, the kernel reads x and g_idx itself (M <= 16)
     uint32_t gdiv_magic;  // direct, contiguous groups: group of lane block r = umulhi(r, magic) + (add ? r : 0)
     int gdiv_add;
+    // GROUPED kernel on a layer whose channels were sorted by group when it was loaded
+    const int32_t *kmap;  // [K] or nullptr: channel k sits at position (kmap[k] & 0xffff) of the sorted
+                          // qweight, counted in the order the unpack yields codes; kmap[k] >> 16 = its group
+    uint32_t wave_div_magic;  // position / channels per wave = umulhi(position, magic), positions < 65536
 };
 
 // k handled by one wave step: 4 lane groups x (8 | 32) codes

@@ -106,6 +106,55 @@ def gemm(x: torch.Tensor, qweight: torch.Tensor, qzeros: torch.Tensor, scales: t
     return out
 
 
+def sorted_plan(M: int, K: int, N: int, bits: int, group_size: int) -> Optional[_lib.Plan]:
+    """The plan ``gemm_sorted`` would run, or None when the sorted path does not cover the problem
+    (it is for decode sizes: the GROUPED family)."""
+    gs = K if group_size == -1 else group_size
+    if K >= 65536 or K % gs != 0 or gs % (8 if bits == 4 else 32) != 0:
+        return None
+    try:
+        plan = _lib.select(M, K, N, bits, group_size, False)
+    except _lib.GptqHipError:
+        return None
+    return plan if plan.kernel == _lib.KERNEL_GROUPED else None
+
+
+def gemm_sorted(x: torch.Tensor, qweight_sorted: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
+                kmap: torch.Tensor, bias: Optional[torch.Tensor], bits: int, group_size: int,
+                plan: Optional[_lib.Plan] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``gemm`` for an activation-order layer whose channels ``pack.sort_channels_by_group`` sorted by
+    group; ``x`` and the result are in the layer's original channel order.  M <= 2."""
+    _need_gpu("x", x, torch.float16)
+    _need_gpu("qweight_sorted", qweight_sorted, torch.int32)
+    _need_gpu("qzeros", qzeros, torch.int32)
+    _need_gpu("scales", scales, torch.float16)
+    _need_gpu("kmap", kmap, torch.int32)
+    if bias is not None:
+        _need_gpu("bias", bias, torch.float16)
+    K, N, _ = check_shapes(qweight_sorted, qzeros, scales, kmap, bias, bits, group_size)
+    if x.dim() != 2 or x.shape[1] != K:
+        raise ValueError(f"x must be [M, {K}], got {tuple(x.shape)}")
+    M = x.shape[0]
+    dev = x.device
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    if M == 0:
+        return out
+    if plan is None:
+        plan = sorted_plan(M, K, N, bits, group_size)
+        if plan is None:
+            raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, f"gptq_hip_gemm_sorted(M={M}, K={K}, N={N}, bits={bits})")
+    ws = _workspace(dev, plan.workspace_bytes) if plan.workspace_bytes else None
+    with torch.cuda.device(dev):
+        rc = _lib.lib().gptq_hip_gemm_sorted(
+            _ptr(x), _ptr(qweight_sorted), _ptr(qzeros), _ptr(scales), _ptr(kmap), _ptr(bias), _ptr(out),
+            _ptr(ws), ws.numel() if ws is not None else 0, M, K, N, bits, group_size,
+            ctypes.byref(plan), _stream(dev))
+    if rc != _lib.OK:
+        raise _lib.GptqHipError(rc, f"gptq_hip_gemm_sorted(M={M}, K={K}, N={N}, bits={bits}, group_size={group_size})")
+    return out
+
+
 def dequant(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
             g_idx: Optional[torch.Tensor], bits: int, group_size: int) -> torch.Tensor:
     """The materialised fp16 weight [K, N], bit-exact with the reference's dequantisation."""

@@ -76,37 +76,72 @@ def unpack_along_axis0(words: np.ndarray, bits: int) -> np.ndarray:
     return out.reshape(rows // 3 * 32, cols)
 
 
+def unpack_rows_torch(words: torch.Tensor, bits: int) -> torch.Tensor:
+    """``unpack_along_axis0`` with torch ops, on whatever device ``words`` is: int32
+    [R//32*bits, C] -> codes int64 [R, C]."""
+    rows, cols = words.shape
+    w = words.to(torch.int64) & 0xFFFFFFFF
+    if bits == 4:
+        shifts = (4 * torch.arange(8, device=words.device)).view(1, 8, 1)
+        return ((w.unsqueeze(1) >> shifts) & 15).reshape(rows * 8, cols)
+    b = w.view(rows // 3, 3, cols)
+    out = torch.empty((rows // 3, 32, cols), dtype=torch.int64, device=words.device)
+    for j in range(32):
+        wi, sh = divmod(3 * j, 32)
+        v = b[:, wi, :] >> sh
+        if sh > 29:  # the code continues in the next word
+            v = v | (b[:, wi + 1, :] << (32 - sh))
+        out[:, j, :] = v & 7
+    return out.reshape(rows // 3 * 32, cols)
+
+
+def pack_rows_torch(codes: torch.Tensor, bits: int) -> torch.Tensor:
+    """``pack_along_axis0`` with torch ops: codes [R, C] (any integer dtype, values < 2**bits) ->
+    int32 [R//32*bits, C]."""
+    R, cols = codes.shape
+    c = codes.to(torch.int64).view(R // 32, 32, cols)
+    words = torch.zeros((R // 32, bits, cols), dtype=torch.int64, device=codes.device)
+    for j in range(32):
+        wi, sh = divmod(bits * j, 32)
+        words[:, wi, :] |= (c[:, j, :] << sh) & 0xFFFFFFFF
+        if sh + bits > 32:
+            words[:, wi + 1, :] |= c[:, j, :] >> (32 - sh)
+    words = torch.where(words >= (1 << 31), words - (1 << 32), words)
+    return words.to(torch.int32).view(R // 32 * bits, cols)
+
+
 def sort_channels_by_group(qweight: torch.Tensor, g_idx: torch.Tensor, bits: int, group_size: int):
     """Load-time preparation for activation-order checkpoints: reorders the input channels so that
     every group is contiguous, which lets the decode kernel treat the layer like one without
-    ``g_idx``.  Returns ``(qweight_sorted int32 [K//32*bits, N], kmap int32 [K])`` on the CPU, or
-    ``None`` when the layer does not qualify.
+    ``g_idx``.  Returns ``(qweight_sorted int32 [K//32*bits, N], kmap int32 [K])`` on the device of
+    ``qweight``, or ``None`` when the layer does not qualify.
 
     Sorted position j holds original channel perm[j] (stable sort by group).  ``kmap[k]`` tells the
     kernel where original channel k goes: low 16 bits = its position inside the sorted K range with
     the codes of each lane block (8 channels for int4, 32 for int3) already in the order the
     kernels' register unpack produces them, high 16 bits = its group.  Requires K < 65536, every
-    group (but the last) to hold exactly ``group_size`` channels, and ``group_size`` to be a
-    multiple of the lane block."""
+    group to hold exactly ``group_size`` channels, and ``group_size`` to be a multiple of the lane
+    block."""
     from . import _slots
 
     K = int(g_idx.numel())
     gs = K if group_size == -1 else group_size
     klane = 8 if bits == 4 else 32
-    if K >= 65536 or gs % klane != 0 or K % 32 != 0:
+    if K >= 65536 or gs % klane != 0 or K % 32 != 0 or K % gs != 0:
         return None
-    g = g_idx.detach().cpu().to(torch.int64)
+    dev = qweight.device
+    g = g_idx.detach().to(device=dev, dtype=torch.int64)
     perm = torch.argsort(g, stable=True)
-    if not torch.equal(g[perm], torch.arange(K, dtype=torch.int64) // gs):
+    ar = torch.arange(K, dtype=torch.int64, device=dev)
+    if not torch.equal(g[perm], ar // gs):
         return None
-    codes = unpack_along_axis0(qweight.detach().cpu().numpy(), bits)
-    qweight_sorted = torch.from_numpy(pack_along_axis0(codes[perm.numpy()], bits))
-    inv = torch.empty(K, dtype=torch.int64)
-    inv[perm] = torch.arange(K, dtype=torch.int64)          # original k -> sorted position
-    slot_of_code = torch.tensor(_slots.slot_of_code(bits), dtype=torch.int64)
+    qweight_sorted = pack_rows_torch(unpack_rows_torch(qweight.detach(), bits)[perm], bits)
+    inv = torch.empty(K, dtype=torch.int64, device=dev)
+    inv[perm] = ar                                          # original k -> sorted position
+    slot_of_code = torch.tensor(_slots.slot_of_code(bits), dtype=torch.int64, device=dev)
     pos = (inv // klane) * klane + slot_of_code[inv % klane]
     kmap = (pos | ((inv // gs) << 16)).to(torch.int32)
-    return qweight_sorted, kmap
+    return qweight_sorted.contiguous(), kmap.contiguous()
 
 
 def num_groups(k: int, group_size: int) -> int:

@@ -16,13 +16,14 @@ import torch
 import torch.nn as nn
 
 from . import _lib, ops
-from .pack import pack_qweight, pack_qzeros
+from .pack import pack_qweight, pack_qzeros, sort_channels_by_group
 
 
 class QuantLinear(nn.Module):
     SUPPORTED_BITS = (3, 4)
 
-    def __init__(self, bits, groupsize, infeatures, outfeatures, bias, kernel_switch_threshold=1024):
+    def __init__(self, bits, groupsize, infeatures, outfeatures, bias, kernel_switch_threshold=1024,
+                 sort_for_decode=True):
         super().__init__()
         if bits not in self.SUPPORTED_BITS:
             # the reference accepts 2, 3, 4, 8 (qlinear.py:31-32); this path implements 3 and 4
@@ -50,6 +51,13 @@ class QuantLinear(nn.Module):
         else:
             self.bias = None
         self._g_state = None  # (g_idx identity, contiguous?) cached by _kernel_g_idx
+        # Activation-order layers: on the first decode-size call (one or two rows of x), keep a second
+        # copy of qweight with the input channels sorted by group (plus a [K] int32 map), which the
+        # decode kernel reads faster than it can follow g_idx.  Costs the layer's packed size again in
+        # device memory; False keeps only the checkpoint's tensors.
+        self.sort_for_decode = sort_for_decode
+        self._sorted = None   # (key, (qweight_sorted, kmap) or None)
+        self._sorted_plans = {}  # M -> plan of the sorted path, or None where it does not apply
 
     # ------------------------------------------------------------------ packing
     def pack(self, linear, scales, zeros, g_idx=None):
@@ -100,6 +108,34 @@ class QuantLinear(nn.Module):
             return self._kernel_g_idx()
         return g
 
+    def prepare_decode(self):
+        """Builds (once per distinct qweight / g_idx storage) the sorted copy used by decode-size
+        calls; returns ``(qweight_sorted, kmap)`` or None when the layer has no activation order or
+        does not qualify.  ``forward`` calls this lazily; loaders may call it up front."""
+        g = self._kernel_g_idx()
+        q = self.qweight
+        key = (q.data_ptr(), q._version, None if g is None else (g.data_ptr(), g._version))
+        if self._sorted is None or self._sorted[0] != key:
+            tensors = None
+            if g is not None and q.device.type == "cuda":
+                tensors = sort_channels_by_group(q, g, self.bits, self.groupsize)
+            self._sorted = (key, tensors)
+        return self._sorted[1]
+
+    def _decode_sorted(self, x2):
+        """The decode product through the sorted copy, or None when that path does not apply."""
+        plans = self._sorted_plans
+        M = x2.shape[0]
+        if M not in plans:
+            plans[M] = ops.sorted_plan(M, self.infeatures, self.outfeatures, self.bits, self.groupsize)
+        if plans[M] is None:
+            return None
+        tensors = self.prepare_decode()
+        if tensors is None:
+            return None
+        return ops.gemm_sorted(x2, tensors[0], self.qzeros, self.scales, tensors[1], self.bias, self.bits,
+                               self.groupsize, plan=plans[M])
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         out_shape = x.shape[:-1] + (self.outfeatures,)
         x2 = x.reshape(-1, x.shape[-1])
@@ -110,8 +146,10 @@ class QuantLinear(nn.Module):
         try:
             if self.kernel_switch_threshold and x2.shape[0] >= self.kernel_switch_threshold:
                 raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, "above kernel_switch_threshold")
-            out = ops.gemm(x2, self.qweight, self.qzeros, self.scales, self._kernel_g_idx(), self.bias,
-                           self.bits, self.groupsize)
+            out = self._decode_sorted(x2) if (self.sort_for_decode and 0 < x2.shape[0] <= 2) else None
+            if out is None:
+                out = ops.gemm(x2, self.qweight, self.qzeros, self.scales, self._kernel_g_idx(), self.bias,
+                               self.bits, self.groupsize)
         except _lib.GptqHipError as e:
             if e.status != _lib.ERR_UNSUPPORTED:
                 raise

@@ -72,9 +72,12 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
-def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int = 0):
+def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int = 0, prepared: bool = False):
+    """prepared: the layer as QuantLinear holds it for decode-size calls after its one-time
+    preparation (channels of an activation-order layer sorted by group), run through
+    gptq_hip_gemm_sorted; only for workloads that path covers (see prepared_applies)."""
     from autogptq.tvm_amd import _lib
-    from autogptq.tvm_amd.pack import synth_layer
+    from autogptq.tvm_amd.pack import sort_channels_by_group, synth_layer
 
     bits, K, N, gs, desc_act, M = WORKLOADS[name]
     L = synth_layer(2000 + sorted(WORKLOADS).index(name), K, N, bits, gs, desc_act, M=M)
@@ -92,8 +95,13 @@ def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int =
         "qzeros": L["qzeros"].to(dev), "scales": L["scales"].to(dev),
         "g_idx": L["g_idx"].to(dev) if desc_act else None,
         "x": L["x"].to(dev), "y": torch.empty((M, N), dtype=torch.float16, device=dev),
-        "wbytes": wbytes, "flops": 2 * M * K * N,
+        "wbytes": wbytes, "flops": 2 * M * K * N, "kmap": None,
     }
+    if prepared:
+        case["qweights"][0], case["kmap"] = sort_channels_by_group(qweights[0], case["g_idx"], bits, gs)
+        case["g_idx"] = None
+        desc_act = False  # the plan is that of contiguous groups
+        kernel = kernel or _lib.KERNEL_GROUPED
     if kernel or split_k or waves_n:
         if not kernel:
             kernel = _lib.select(M, K, N, bits, gs, desc_act).kernel
@@ -105,16 +113,26 @@ def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int =
     return case
 
 
+def prepared_applies(name: str) -> bool:
+    from autogptq.tvm_amd import ops
+
+    bits, K, N, gs, desc_act, M = WORKLOADS[name]
+    G = 1 if gs == -1 else -(-K // gs)
+    return bool(desc_act and G > 1 and M <= 2 and ops.sorted_plan(M, K, N, bits, gs) is not None)
+
+
 def make_step(case, dev):
-    """Returns step(i): one gptq_hip_gemm_plan call on weight copy i (pre-marshalled arguments)."""
+    """Returns step(i): one gptq_hip_gemm_plan (or gptq_hip_gemm_sorted) call on weight copy i
+    (pre-marshalled arguments)."""
     from autogptq.tvm_amd import _lib
 
     lib = _lib.lib()
-    fn = lib.gptq_hip_gemm_plan
+    fn = lib.gptq_hip_gemm_sorted if case["kmap"] is not None else lib.gptq_hip_gemm_plan
     vp = ctypes.c_void_p
+    gmap = case["kmap"] if case["kmap"] is not None else case["g_idx"]
     common = dict(
         x=vp(case["x"].data_ptr()), qz=vp(case["qzeros"].data_ptr()), sc=vp(case["scales"].data_ptr()),
-        g=vp(case["g_idx"].data_ptr()) if case["g_idx"] is not None else None,
+        g=vp(gmap.data_ptr()) if gmap is not None else None,
         y=vp(case["y"].data_ptr()), ws=vp(case["ws"].data_ptr()) if case["plan"].workspace_bytes else None,
     )
     qws = [vp(q.data_ptr()) for q in case["qweights"]]

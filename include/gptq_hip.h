@@ -106,6 +106,23 @@ int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const int32_t *qze
                        int M, int K, int N, int bits, int group_size, const gptq_hip_plan *plan, void *stream);
 
 /*
+ * The decode product (M <= 2) for a layer prepared when it was loaded: an activation-order g_idx makes
+ * every weight look its group up (qlinear.py:200-242 gathers scales and zeros by g_idx), so the
+ * loader sorts the input channels by group once; qweight_sorted holds the same codes with groups
+ * contiguous along K and
+ *   kmap int32 [K] (16-byte aligned): kmap[k] & 0xffff = where channel k went, as a position in the
+ *                                     order the kernels unpack codes; kmap[k] >> 16 = g_idx[k]
+ * tells the kernel where each x[m, k] belongs.  x and y are in the layer's original channel order.
+ * qzeros and scales are unchanged.  plan: NULL lets the dispatcher choose, else a GROUPED plan for
+ * (M, K, N, bits, group_size, act_order = 0); workspace as that plan asks.  Needs K < 65536, equal
+ * groups and group_size a multiple of 8 (int4) or 32 (int3); GPTQ_HIP_ERR_UNSUPPORTED otherwise, or
+ * when the problem is not one for the GROUPED family.  One launch.
+ */
+int gptq_hip_gemm_sorted(const void *x, const int32_t *qweight_sorted, const int32_t *qzeros, const void *scales,
+                         const int32_t *kmap, const void *bias, void *y, void *workspace, size_t workspace_bytes,
+                         int M, int K, int N, int bits, int group_size, const gptq_hip_plan *plan, void *stream);
+
+/*
  * W fp16 [K, N] = scales[g] * (q - (zq[g] + 1)), one rounding per element:
  * the materialised weight of qlinear.py:198-242, for the bit-exact check.
  */

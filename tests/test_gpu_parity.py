@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from autogptq.tvm_amd import QuantLinear, _lib, ops
+from autogptq.tvm_amd import QuantLinear, _lib, ops, pack
 from tests.parity_util import (ATOL, RTOL, assert_close, assert_tight, expected_output, expected_weight, layer,
                                to_dev)
 
@@ -270,6 +270,96 @@ def test_gemm_linearity_at_full_size(dev):
 
 
 # ------------------------------------------------------------------ the module
+# ------------------------------------------------------------------ activation order, channels sorted at load time
+def run_sorted(D, plan=None):
+    qs, kmap = pack.sort_channels_by_group(D["qweight"], D["g_idx"], D["bits"], D["group_size"])
+    return ops.gemm_sorted(D["x"], qs, D["qzeros"], D["scales"], kmap, D.get("bias"), D["bits"], D["group_size"],
+                           plan=plan)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("K,N,gs", [(96, 32, 32), (1024, 416, 32), (2048, 1056, 256), (11008, 256, 128),
+                                    (4096, 64, 64), (4096, 352, 128), (1024, 160, -1)])
+@pytest.mark.parametrize("M", [1, 2])
+def test_sorted_decode_matches_oracle_and_unsorted_kernel(dev, bits, K, N, gs, M):
+    L = layer(900 + K + M, K, N, bits, gs, True, M=M, bias=True)
+    D = to_dev(L, dev)
+    plan = ops.sorted_plan(M, K, N, bits, gs)
+    if plan is None:
+        pytest.skip("not a GROUPED problem")
+    want = expected_output(L)
+    y = run_sorted(D)
+    assert_close(y, want, "sorted decode")
+    assert_tight(y, want, "sorted decode")
+    assert torch.equal(y, run_sorted(D))
+    assert_tight(y, run_gemm(D).cpu(), "sorted vs unsorted kernel")
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("split", [1, 2, 5, 16])
+def test_sorted_decode_forced_split_k(dev, bits, M, split):
+    # with K split over workgroups each one keeps only the channels whose sorted position is its own
+    K, N, gs = 2048, 320, 128
+    L = layer(950 + split, K, N, bits, gs, True, M=M, bias=True)
+    D = to_dev(L, dev)
+    try:
+        plan = _lib.plan_for(_lib.KERNEL_GROUPED, M, K, N, bits, gs, False, split_k=split)
+    except _lib.GptqHipError as e:
+        assert e.status == _lib.ERR_UNSUPPORTED
+        pytest.skip("this split is outside the GROUPED family for the shape")
+    y = run_sorted(D, plan=plan)
+    assert_close(y, expected_output(L), f"sorted split={split}")
+    assert_tight(y, expected_output(L), f"sorted split={split}")
+
+
+def test_sorted_decode_integer_exact_and_rejections(dev):
+    # unit scales, zero points 1 (stored 0), integer x: every product and sum is exact in fp32
+    K, N, gs, bits = 4096, 352, 128, 3
+    L = layer(960, K, N, bits, gs, True, M=1)
+    L["scales"] = torch.ones_like(L["scales"])
+    L["qzeros"] = torch.zeros_like(L["qzeros"])
+    L["x"] = torch.randint(-2, 3, (1, K), generator=torch.Generator().manual_seed(5)).half()
+    D = to_dev(L, dev)
+    codes = torch.from_numpy(pack.unpack_along_axis0(L["qweight"].numpy(), bits).astype(np.float64))
+    want = (L["x"].double() @ (codes - 1.0))
+    assert torch.equal(run_sorted(D).cpu().double(), want.half().double())
+    # a plan of another family, a map that is not 16-byte aligned, 3-bit groups narrower than 32
+    qs, kmap = pack.sort_channels_by_group(D["qweight"], D["g_idx"], bits, gs)
+    with pytest.raises(_lib.GptqHipError) as e:
+        ops.gemm_sorted(D["x"], qs, D["qzeros"], D["scales"], kmap, None, bits, gs,
+                        plan=_lib.plan_for(_lib.KERNEL_GATHER, 1, K, N, bits, gs, False))
+    assert e.value.status == _lib.ERR_UNSUPPORTED
+    shifted = torch.zeros(K + 1, dtype=torch.int32, device=dev)[1:]
+    shifted.copy_(kmap)
+    with pytest.raises(_lib.GptqHipError) as e:
+        ops.gemm_sorted(D["x"], qs, D["qzeros"], D["scales"], shifted, None, bits, gs)
+    assert e.value.status == _lib.ERR_BAD_ARG
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_quantlinear_decode_uses_the_sorted_copy(dev, bits):
+    K, N, gs = 2048, 8192, 128   # wide enough for the decode family to take two rows as well
+    L = layer(44, K, N, bits, gs, True, M=2, bias=True)
+    q = QuantLinear(bits, gs, K, N, True)
+    q.load_state_dict({k: L[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})
+    q = q.to(dev)
+    assert q._sorted is None
+    y = q(L["x"].to(dev))
+    assert q._sorted is not None and q._sorted[1] is not None     # built by the first decode-size call
+    assert_close(y, expected_output(L), "module decode, sorted")
+    assert_close(q(L["x"][:1].to(dev)), expected_output(L)[:1], "module decode, sorted, one row")
+    # switching the preparation off gives the same numbers from the checkpoint's own tensors
+    q.sort_for_decode = False
+    assert_tight(q(L["x"].to(dev)), y.cpu(), "module decode, unsorted")
+    # new weights invalidate the copy
+    q.sort_for_decode = True
+    L2 = layer(45, K, N, bits, gs, True, M=2, bias=True)
+    q.load_state_dict({k: L2[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})
+    L2["x"] = L["x"]
+    assert_close(q(L["x"].to(dev)), expected_output(L2), "module decode after reload")
+
+
 @pytest.mark.parametrize("bits", [3, 4])
 def test_quantlinear_forward(dev, bits):
     K, N, gs = 512, 256, 128

@@ -141,6 +141,11 @@ def test_unpack_is_the_inverse_of_pack(bits):
     assert np.array_equal(pack.unpack_along_axis0(pack.pack_along_axis0(codes, bits), bits), codes)
     words = rng.integers(-(1 << 31), 1 << 31, size=(12, 5)).astype(np.int32)
     assert np.array_equal(pack.unpack_along_axis0(words, bits), orc.unpack_bitstream(words, bits, axis=0))
+    # the torch versions (they run on the GPU when a layer is prepared) agree with the numpy ones
+    assert np.array_equal(pack.unpack_rows_torch(torch.from_numpy(words), bits).numpy(),
+                          pack.unpack_along_axis0(words, bits))
+    assert np.array_equal(pack.pack_rows_torch(torch.from_numpy(codes.astype(np.int64)), bits).numpy(),
+                          pack.pack_along_axis0(codes, bits))
 
 
 @pytest.mark.parametrize("bits,K,gs", [(4, 256, 32), (3, 256, 64), (3, 128, -1), (4, 96, 8)])
