@@ -139,11 +139,25 @@ static int run_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros
     p.gdiv_magic = 0;
     p.gdiv_add = 0;
     p.kmap = nullptr;
+    p.xsrc = nullptr;
     p.wave_div_magic = 0;
+    if (plan->kernel == GPTQ_HIP_KERNEL_GROUPED && !g_idx && gs % (bits == 4 ? 8 : 32) == 0) {
+        // group of lane block r = r / d, d = lane blocks per group, as a multiply-high (r < 65536)
+        const uint32_t d = (uint32_t)(gs / (bits == 4 ? 8 : 32));
+        if (d == 1) {
+            p.gdiv_add = 1;
+        } else {
+            p.gdiv_magic = (uint32_t)((1ull << 32) / d) + 1u;
+        }
+    }
     if (kmap) {
         // positions are below 65536 and a wave holds at least one step: the multiply-high is exact
         if (plan->kernel != GPTQ_HIP_KERNEL_GROUPED) return GPTQ_HIP_ERR_UNSUPPORTED;
-        p.kmap = kmap;
+        if (plan->split_k == 1) {
+            p.kmap = kmap;
+        } else {
+            p.xsrc = kmap + K;
+        }
         p.wave_div_magic = (uint32_t)((1ull << 32) / (uint32_t)(p.wave_steps * kstep)) + 1u;
     }
     if (plan->kernel == GPTQ_HIP_KERNEL_STREAM) {

@@ -27,10 +27,19 @@
 //             are that tile AND mask / AND NOT mask: half the LDS, so K = 4096 with 32
 //             groups fits one workgroup.
 //
+// LITE: with contiguous groups that are whole lane blocks (8 channels int4, 32 int3) all 8 slots
+// of an operand tile belong to one group, so the tile is "x in row r, zeros elsewhere".  LDS then
+// holds just x in unpack order (2 bytes per channel instead of 32) plus 16 zero bytes: a lane reads
+// x when its row is the block's group and the zeros otherwise.  No zero fill, and the scatter is
+// one 2-byte store per channel to spread addresses instead of one bank.
+//
 // Sorted layers: when the loader has sorted the channels of an activation-order layer by
 // group (qweight rows permuted, p.kmap saying where each original channel went), the groups
 // are contiguous for the weight stream and only the scatter of x follows the map: every
-// workgroup walks all of x and keeps the channels whose sorted position falls in its K range.
+// workgroup walks all of x and keeps the channels whose sorted position falls in its K range
+// (p.kmap, when one workgroup holds all of K), or looks up where the x of each of its positions
+// comes from (p.xsrc, when K is split: a walk over all of x would cost every workgroup the whole
+// scatter for a fraction of the channels).
 #include "gptq_device.h"
 
 namespace gptq {
@@ -43,12 +52,13 @@ __device__ __forceinline__ h8 and_h8(h8 a, u4 m)
 }
 
 // TPM = row tiles (of 16 groups) per activation row; COMPACT needs TPM == 2.
-template <int BITS, int M, int TPM, bool COMPACT, int NSTEP>
+template <int BITS, int M, int TPM, bool COMPACT, int NSTEP, bool LITE>
 __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
 {
     using F = Fmt<BITS>;
     constexpr int ST = COMPACT ? M : M * TPM;    // tiles stored in LDS per 8 slots
     static_assert(!COMPACT || TPM == 2, "compact layout is for two row tiles");
+    static_assert(!LITE || (TPM == 1 && !COMPACT), "the lite operand is one row tile of contiguous groups");
     const int tid = threadIdx.x;
     const int nthreads = (int)blockDim.x;
     const int lane = tid & 63;
@@ -80,6 +90,8 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     __shared__ int last_flag;
     __shared__ int wave_gb[8];  // sorted layers: first group of each wave along K
     const int32_t *kmap = p.kmap;
+    const int32_t *xsrc = p.xsrc;
+    auto src_ok = [&](int c) { return (int)min((uint32_t)c, (uint32_t)p.K - 1u); };  // a bad map must not fault
     if (kmap && tid < WK) wave_gb[tid] = (k_base + tid * wave_k) / p.group_size;
 
     const _Float16 *x = (const _Float16 *)p.x;
@@ -90,6 +102,13 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     unsigned char *tiles = smem;
     unsigned char *masks = smem + (size_t)nblk8 * ST * 256;
     float *red = (float *)(masks + (COMPACT ? (size_t)nblk8 * 16 : 0));
+    // LITE: x of the K range in unpack order, [M][kspan] fp16, then 16 zero bytes
+    _Float16 *xlds = (_Float16 *)smem;
+    const uint32_t zero_off = (uint32_t)M * (uint32_t)kspan * 2u;
+    if constexpr (LITE) {
+        red = (float *)(smem + zero_off + 16);
+        if (tid < 4) ((uint32_t *)(smem + zero_off))[tid] = 0u;
+    }
 
     int qslot[4];
 #pragma unroll
@@ -101,16 +120,24 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     const int nquads = qpr * M;
     int gq[QP][4];
     h4 xq[QP];
+    int4 sq[QP];  // xsrc: the channels of x this thread's positions take
 #pragma unroll
     for (int ps = 0; ps < QP; ps++) {
         const int idx = tid + ps * nthreads;
         xq[ps] = (h4){0, 0, 0, 0};
+        sq[ps] = make_int4(0, 0, 0, 0);
 #pragma unroll
         for (int e = 0; e < 4; e++) gq[ps][e] = 0;
         if (idx < nquads) {
             const int m = M == 1 ? 0 : idx / qpr;
             const int k = scan_base + 4 * (idx - m * qpr);
             if (k < p.K) {  // K % 4 == 0: a quad is inside or outside as a whole
+                if (xsrc) {
+                    sq[ps] = *(const int4 *)(xsrc + k);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) gq[ps][e] = (k + e) / p.group_size;
+                    continue;
+                }
                 xq[ps] = *(const h4 *)(x + (size_t)m * p.K + k);
                 if (p.g_idx || kmap) {
                     const int4 gv = *(const int4 *)((kmap ? kmap : p.g_idx) + k);
@@ -128,8 +155,9 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
 
     // ---- 2. zero the expanded activation operand in LDS while those loads fly ---------
     {
+        // LITE: only x itself (channels past the end of K must read as zero)
         u4 *z = (u4 *)tiles;
-        const int n16 = nblk8 * ST * 16;
+        const int n16 = LITE ? M * kspan / 8 : nblk8 * ST * 16;
         for (int i = tid; i < n16; i += nthreads) z[i] = (u4){0u, 0u, 0u, 0u};
     }
     // ---- 3. weight loads, software-pipelined: a wave blocks while it issues loads into a full
@@ -153,6 +181,18 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
 #pragma unroll
     for (int s = 0; s < PF && s < NSTEP; s++) load_step(s, ws + s);
     __builtin_amdgcn_sched_barrier(0);
+    if (xsrc) {  // the x values of this thread's positions, now that their source channels are known
+#pragma unroll
+        for (int ps = 0; ps < QP; ps++) {
+            const int idx = tid + ps * nthreads;
+            const int m = M == 1 ? 0 : idx / qpr;
+            if (idx < nquads && k_base + 4 * (idx - m * qpr) < p.K) {
+                const _Float16 *xr = x + (size_t)m * p.K;
+                xq[ps] = (h4){xr[src_ok(sq[ps].x)], xr[src_ok(sq[ps].y)], xr[src_ok(sq[ps].z)], xr[src_ok(sq[ps].w)]};
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
 
     // ---- 4. scales / zero words this lane needs in the epilogue (rows g = 16 t + 4 q + v);
     //         loaded once the last weight loads are out ---------------------------------
@@ -181,6 +221,10 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     // four slots of its quad are fixed: qslot[e], looked up once at the top of the kernel.
     // gb: first group of the wave that will consume channel kc (0 under a g_idx)
     auto scatter = [&](int m, int kc, int slot, int g, int gb, _Float16 xv) {
+        if constexpr (LITE) {
+            xlds[m * kspan + (kc / F::KLANE) * F::KLANE + slot] = xv;
+            return;
+        }
         const int r = min(max(g, 0), p.G - 1) - gb;  // row of this group
         const int rr = min(max(r, 0), 16 * TPM - 1);
         const int b8 = (kc / F::KLANE) * F::NB + (slot >> 3);
@@ -196,8 +240,12 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     auto scatter_mapped = [&](int m, int entry, _Float16 xv) {
         const int kc = (entry & 0xffff) - k_base;
         if ((unsigned)kc < (unsigned)kspan) {
-            const int gb = wave_gb[__umulhi((uint32_t)kc, p.wave_div_magic)];
-            scatter(m, kc, kc % F::KLANE, entry >> 16, gb, xv);
+            if constexpr (LITE) {
+                xlds[m * kspan + kc] = xv;
+            } else {
+                const int gb = wave_gb[__umulhi((uint32_t)kc, p.wave_div_magic)];
+                scatter(m, kc, kc % F::KLANE, entry >> 16, gb, xv);
+            }
         }
     };
 #pragma unroll
@@ -218,26 +266,58 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
             }
         }
     }
-    for (int idx = tid + QP * nthreads; idx < nquads; idx += nthreads) {  // long K ranges
-        const int m = M == 1 ? 0 : idx / qpr;
-        const int kc = 4 * (idx - m * qpr);
-        const int k = scan_base + kc;
-        if (kmap) {
-            if (k < p.K) {
-                const h4 xv = *(const h4 *)(x + (size_t)m * p.K + k);
-                const int4 mv = *(const int4 *)(kmap + k);
-                scatter_mapped(m, mv.x, xv[0]);
-                scatter_mapped(m, mv.y, xv[1]);
-                scatter_mapped(m, mv.z, xv[2]);
-                scatter_mapped(m, mv.w, xv[3]);
-            }
-        } else if (k < p.K) {
-            const h4 xv = *(const h4 *)(x + (size_t)m * p.K + k);
-            const int gb = p.g_idx ? 0 : (k_base + (kc / wave_k) * wave_k) / p.group_size;
+    // long K ranges (and sorted layers, whose workgroups walk all of x): LP passes per trip, all
+    // loads of a trip issued before its first scatter
+    constexpr int LP = 4;
+    for (int base = tid + QP * nthreads; base < nquads; base += LP * nthreads) {
+        h4 xl[LP];
+        int4 gl[LP];
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int g = p.g_idx ? p.g_idx[k + e] : (k + e) / p.group_size;
-                scatter(m, kc + e, qslot[e], g, gb, xv[e]);
+        for (int u = 0; u < LP; u++) {
+            const int idx = base + u * nthreads;
+            xl[u] = (h4){0, 0, 0, 0};
+            gl[u] = make_int4(0, 0, 0, 0);
+            if (idx < nquads) {
+                const int m = M == 1 ? 0 : idx / qpr;
+                const int k = scan_base + 4 * (idx - m * qpr);
+                if (k < p.K) {
+                    if (xsrc) {
+                        gl[u] = *(const int4 *)(xsrc + k);
+                    } else {
+                        xl[u] = *(const h4 *)(x + (size_t)m * p.K + k);
+                        if (p.g_idx || kmap) gl[u] = *(const int4 *)((kmap ? kmap : p.g_idx) + k);
+                    }
+                }
+            }
+        }
+        if (xsrc) {
+#pragma unroll
+            for (int u = 0; u < LP; u++) {
+                const int idx = base + u * nthreads;
+                const int m = M == 1 ? 0 : min(idx, nquads - 1) / qpr;
+                const _Float16 *xr = x + (size_t)m * p.K;  // sources of skipped quads are 0: a valid channel
+                xl[u] = (h4){xr[src_ok(gl[u].x)], xr[src_ok(gl[u].y)], xr[src_ok(gl[u].z)], xr[src_ok(gl[u].w)]};
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < LP; u++) {
+            const int idx = base + u * nthreads;
+            if (idx >= nquads) continue;
+            const int m = M == 1 ? 0 : idx / qpr;
+            const int kc = 4 * (idx - m * qpr);
+            const int k = scan_base + kc;
+            if (k >= p.K) continue;
+            const int gv[4] = {gl[u].x, gl[u].y, gl[u].z, gl[u].w};
+            if (kmap) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) scatter_mapped(m, gv[e], xl[u][e]);
+            } else {
+                const int gb = p.g_idx ? 0 : (k_base + (kc / wave_k) * wave_k) / p.group_size;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int g = p.g_idx ? gv[e] : (k + e) / p.group_size;
+                    scatter(m, kc + e, qslot[e], g, gb, xl[u][e]);
+                }
             }
         }
     }
@@ -294,7 +374,16 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
                 for (int nb = 0; nb < F::NB; nb++) {
                     const int b8 = b * F::NB + nb;
                     h8 a[M][TPM];
-                    if constexpr (COMPACT) {
+                    if constexpr (LITE) {
+                        // the group of this lane block, as a row of the wave's tile
+                        const uint32_t lb = (uint32_t)((st0 + s) * 4 + lq);
+                        const int row = (int)(__umulhi(lb, p.gdiv_magic) + (p.gdiv_add ? lb : 0u)) - g_base;
+#pragma unroll
+                        for (int m = 0; m < M; m++) {
+                            const uint32_t off = row == li ? (uint32_t)(m * kspan + b8 * 8) * 2u : zero_off;
+                            a[m][0] = *(const h8 *)(smem + off);
+                        }
+                    } else if constexpr (COMPACT) {
                         const u4 mk = *(const u4 *)(masks + (size_t)b8 * 16);
 #pragma unroll
                         for (int m = 0; m < M; m++) {
@@ -427,19 +516,30 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     }
 }
 
-template <int BITS, int M, int TPM, bool COMPACT>
+template <int BITS, int M, int TPM, bool COMPACT, bool LITE = false>
 static int launch_grouped_one(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
     constexpr int NSTEP = BITS == 4 ? 16 : 4;
-    auto kern = grouped_kernel<BITS, M, TPM, COMPACT, NSTEP>;
-    if (plan.lds_bytes > 65536) {
-        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, plan.lds_bytes) !=
+    if constexpr (BITS == 3 && TPM == 1 && !COMPACT && !LITE) {
+        // contiguous groups made of whole lane blocks: the lean operand.  Not for int4: its steps are
+        // a quarter as long, and choosing the row per step costs what the lean prologue saves
+        // (measured: 4096 x 4096 8.3 -> 8.7 us, 11008 x 4096 10.8 -> 11.7 us).
+        if (!p.g_idx && p.group_size % Fmt<BITS>::KLANE == 0 && p.K / Fmt<BITS>::KLANE < 65536)
+            return launch_grouped_one<BITS, M, TPM, COMPACT, true>(p, plan, stream);
+    }
+    auto kern = grouped_kernel<BITS, M, TPM, COMPACT, NSTEP, LITE>;
+    // LITE keeps x itself (2 bytes per channel and row), 16 zero bytes and the waves' partial sums
+    const int lds_bytes =
+        LITE ? p.M * p.wave_steps * p.waves_k * Fmt<BITS>::KSTEP * 2 + 16 + p.waves_k * p.waves_n * p.M * 256
+             : plan.lds_bytes;
+    if (lds_bytes > 65536) {
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) !=
             hipSuccess) {
             (void)hipGetLastError();
             return GPTQ_HIP_ERR_LAUNCH;
         }
     }
-    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, 1), dim3(plan.block), plan.lds_bytes, stream, p);
+    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, 1), dim3(plan.block), lds_bytes, stream, p);
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 

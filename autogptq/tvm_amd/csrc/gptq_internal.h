@@ -40,6 +40,8 @@ struct Params {
     // GROUPED kernel on a layer whose channels were sorted by group when it was loaded
     const int32_t *kmap;  // [K] or nullptr: channel k sits at position (kmap[k] & 0xffff) of the sorted
                           // qweight, counted in the order the unpack yields codes; kmap[k] >> 16 = its group
+    const int32_t *xsrc;  // [K] or nullptr: xsrc[j] = the channel of x whose codes are j-th along K in the sorted qweight; the
+                          // kernel follows kmap when a workgroup holds all of K and xsrc when K is split
     uint32_t wave_div_magic;  // position / channels per wave = umulhi(position, magic), positions < 65536
 };
 

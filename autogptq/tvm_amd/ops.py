@@ -131,7 +131,9 @@ def gemm_sorted(x: torch.Tensor, qweight_sorted: torch.Tensor, qzeros: torch.Ten
     _need_gpu("kmap", kmap, torch.int32)
     if bias is not None:
         _need_gpu("bias", bias, torch.float16)
-    K, N, _ = check_shapes(qweight_sorted, qzeros, scales, kmap, bias, bits, group_size)
+    K, N, _ = check_shapes(qweight_sorted, qzeros, scales, None, bias, bits, group_size)
+    if tuple(kmap.shape) != (2 * K,):
+        raise ValueError(f"kmap must be [{2 * K}], got {tuple(kmap.shape)}")
     if x.dim() != 2 or x.shape[1] != K:
         raise ValueError(f"x must be [M, {K}], got {tuple(x.shape)}")
     M = x.shape[0]

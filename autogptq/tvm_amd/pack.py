@@ -113,13 +113,14 @@ def pack_rows_torch(codes: torch.Tensor, bits: int) -> torch.Tensor:
 def sort_channels_by_group(qweight: torch.Tensor, g_idx: torch.Tensor, bits: int, group_size: int):
     """Load-time preparation for activation-order checkpoints: reorders the input channels so that
     every group is contiguous, which lets the decode kernel treat the layer like one without
-    ``g_idx``.  Returns ``(qweight_sorted int32 [K//32*bits, N], kmap int32 [K])`` on the device of
+    ``g_idx``.  Returns ``(qweight_sorted int32 [K//32*bits, N], kmap int32 [2K])`` on the device of
     ``qweight``, or ``None`` when the layer does not qualify.
 
     Sorted position j holds original channel perm[j] (stable sort by group).  ``kmap[k]`` tells the
     kernel where original channel k goes: low 16 bits = its position inside the sorted K range with
     the codes of each lane block (8 channels for int4, 32 for int3) already in the order the
-    kernels' register unpack produces them, high 16 bits = its group.  Requires K < 65536, every
+    kernels' register unpack produces them, high 16 bits = its group.  ``kmap[K + j]`` is
+    perm[j], the original channel whose codes are j-th along K in ``qweight_sorted``.  Requires K < 65536, every
     group to hold exactly ``group_size`` channels, and ``group_size`` to be a multiple of the lane
     block."""
     from . import _slots
@@ -140,7 +141,7 @@ def sort_channels_by_group(qweight: torch.Tensor, g_idx: torch.Tensor, bits: int
     inv[perm] = ar                                          # original k -> sorted position
     slot_of_code = torch.tensor(_slots.slot_of_code(bits), dtype=torch.int64, device=dev)
     pos = (inv // klane) * klane + slot_of_code[inv % klane]
-    kmap = (pos | ((inv // gs) << 16)).to(torch.int32)
+    kmap = torch.cat([pos | ((inv // gs) << 16), perm]).to(torch.int32)
     return qweight_sorted.contiguous(), kmap.contiguous()
 
 

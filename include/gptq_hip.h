@@ -110,8 +110,9 @@ int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const int32_t *qze
  * every weight look its group up (qlinear.py:200-242 gathers scales and zeros by g_idx), so the
  * loader sorts the input channels by group once; qweight_sorted holds the same codes with groups
  * contiguous along K and
- *   kmap int32 [K] (16-byte aligned): kmap[k] & 0xffff = where channel k went, as a position in the
- *                                     order the kernels unpack codes; kmap[k] >> 16 = g_idx[k]
+ *   kmap int32 [2K] (16-byte aligned): kmap[k] & 0xffff = where channel k went, as a position in the
+ *                                      order the kernels unpack codes; kmap[k] >> 16 = g_idx[k];
+ *                                      kmap[K + j] = the channel whose codes are j-th along K in qweight_sorted
  * tells the kernel where each x[m, k] belongs.  x and y are in the layer's original channel order.
  * qzeros and scales are unchanged.  plan: NULL lets the dispatcher choose, else a GROUPED plan for
  * (M, K, N, bits, group_size, act_order = 0); workspace as that plan asks.  Needs K < 65536, equal

@@ -330,7 +330,7 @@ def test_sorted_decode_integer_exact_and_rejections(dev):
         ops.gemm_sorted(D["x"], qs, D["qzeros"], D["scales"], kmap, None, bits, gs,
                         plan=_lib.plan_for(_lib.KERNEL_GATHER, 1, K, N, bits, gs, False))
     assert e.value.status == _lib.ERR_UNSUPPORTED
-    shifted = torch.zeros(K + 1, dtype=torch.int32, device=dev)[1:]
+    shifted = torch.zeros(2 * K + 1, dtype=torch.int32, device=dev)[1:]
     shifted.copy_(kmap)
     with pytest.raises(_lib.GptqHipError) as e:
         ops.gemm_sorted(D["x"], qs, D["qzeros"], D["scales"], shifted, None, bits, gs)

@@ -157,7 +157,8 @@ def test_sort_channels_by_group_preserves_the_layer(bits, K, gs):
     res = pack.sort_channels_by_group(L["qweight"], L["g_idx"], bits, gs)
     assert res is not None
     qs, kmap = res
-    assert qs.shape == L["qweight"].shape and qs.dtype == torch.int32 and kmap.shape == (K,)
+    assert qs.shape == L["qweight"].shape and qs.dtype == torch.int32 and kmap.shape == (2 * K,)
+    kmap, src = kmap[:K], kmap[K:].long()
     g = K if gs == -1 else gs
     klane = 8 if bits == 4 else 32
     pos, grp = (kmap & 0xFFFF).long(), (kmap >> 16).long()
@@ -166,6 +167,7 @@ def test_sort_channels_by_group_preserves_the_layer(bits, K, gs):
     code_of_slot = torch.tensor(_slots.code_of_slot(bits))
     sorted_pos = (pos // klane) * klane + code_of_slot[pos % klane]
     assert sorted(sorted_pos.tolist()) == list(range(K))            # a permutation
+    assert torch.equal(sorted_pos[src], torch.arange(K))            # second half: channel at each sorted index
     assert torch.equal(sorted_pos // g, L["g_idx"].long())           # groups became contiguous
     # the sorted layer with contiguous groups dequantises to the original weight rows, permuted
     w_orig = orc.dequant_ref(L["qweight"], L["qzeros"], L["scales"], L["g_idx"], bits)
