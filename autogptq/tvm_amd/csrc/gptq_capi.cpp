@@ -153,7 +153,9 @@ static int run_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros
     if (kmap) {
         // positions are below 65536 and a wave holds at least one step: the multiply-high is exact
         if (plan->kernel != GPTQ_HIP_KERNEL_GROUPED) return GPTQ_HIP_ERR_UNSUPPORTED;
-        if (plan->split_k == 1) {
+        // a workgroup that holds all of K, or a short x, walks x once and keeps its channels; with K
+        // split and a long x it looks its channels up instead (measured crossover near K = 6000)
+        if (plan->split_k == 1 || K <= 6144) {
             p.kmap = kmap;
         } else {
             p.xsrc = kmap + K;

@@ -315,8 +315,12 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     // A single group over a large matrix gains nothing from GROUPED's expansion by group: STREAM's
     // one table entry per lane block is cheaper there.
     const bool one_big_group = G == 1 && (long long)K * N >= (1LL << 27);
+    // Under an activation order every group a workgroup meets needs a row: past three row tiles
+    // (48 groups) the expansion costs more than STREAM's lookup per weight (measured at N = 4096,
+    // int3 / int4: K = 5120 16.1 / 11.6 us against 19.1 / 12.8; K = 8192 19.8 / 22.1 against 15.3 / 13.7;
+    // K = 11008 79 / 93 against 20.1 / 16.8).
     if (M <= 2 && !one_big_group && plan_grouped(M, K, N, bits, gs, G, act_order, 0, 0, plan) &&
-        (M == 1 || plan->split_k == 1))
+        (M == 1 || plan->split_k == 1) && (!act_order || plan->row_tiles / M <= 3))
         return GPTQ_HIP_OK;
     memset(plan, 0, sizeof(*plan));
     if (plan_stream(M, K, N, bits, gs, G, act_order, 0, 0, plan) == GPTQ_HIP_OK) return GPTQ_HIP_OK;

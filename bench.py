@@ -3,7 +3,11 @@
 
 Default workload: BASELINE.json configs[1] -- 3-bit GEMV, M=1, K=4096, N=11008, group_size=128,
 desc_act=True (g_idx from a random permutation), synthetic seeded tensors.  One "step" is one
-call of the C-ABI entry point ``gptq_hip_gemm`` on tensors already resident in HBM.  Steps rotate
+call of the C-ABI entry point that ``QuantLinear.forward`` makes for that shape, on tensors already
+resident in HBM: ``gptq_hip_gemm_sorted`` for decode sizes on activation-order layers (the layer
+as the module holds it after its one-time load preparation, the channel sort; ``--unprepared``
+times ``gptq_hip_gemm`` on the checkpoint's own tensors instead, and the default run reports that
+figure too under ``timing.unprepared_us``), ``gptq_hip_gemm`` otherwise.  Steps rotate
 over enough distinct weight copies to exceed twice the 256 MB Infinity Cache, so every step
 streams its packed weights from HBM (cache-cold).
 
@@ -47,6 +51,10 @@ WORKLOADS = {
     "c3-int4-4096x11008-m8": (4, 4096, 11008, 128, False, 8),
     "c3-int4-11008x4096-m1": (4, 11008, 4096, 128, False, 1),
     "c3-int4-11008x4096-m8": (4, 11008, 4096, 128, False, 8),
+    "int3-11008x4096-act-m1": (3, 11008, 4096, 128, True, 1),
+    "int4-11008x4096-act-m1": (4, 11008, 4096, 128, True, 1),
+    "int3-4096x4096-act-m1": (3, 4096, 4096, 128, True, 1),
+    "int3-4096x11008-m1": (3, 4096, 11008, 128, False, 1),
     "c4-int4-4096x11008-act-m16": (4, 4096, 11008, 128, True, 16),
     "c4-int4-4096x11008-act-m64": (4, 4096, 11008, 128, True, 64),
     "c4-int4-4096x11008-act-m128": (4, 4096, 11008, 128, True, 128),
@@ -261,6 +269,9 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument("--sweep", action="store_true", help="also time every workload in WORKLOADS")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--unprepared", action="store_true",
+                    help="decode on activation-order layers: time gptq_hip_gemm on the checkpoint's tensors "
+                         "instead of gptq_hip_gemm_sorted on the load-time prepared ones")
     ap.add_argument("--kernel", type=int, default=0, help="force a kernel family (1 gather, 2 grouped, 3 blocked)")
     ap.add_argument("--split-k", type=int, default=0, help="force the split-K factor")
     ap.add_argument("--waves-n", type=int, default=0, help="force the waves per workgroup along N (STREAM kernel: along K)")
@@ -288,12 +299,21 @@ def main():
         print(json.dumps({"copy_calibration": {"bytes_read": nbytes, "bytes_written": nbytes, "launches": 5,
                                                "kernel": "torch elementwise copy (int32)"}}))
         return
-    case = build_case(args.workload, dev, args.kernel, args.split_k, args.waves_n)
+    forced = bool(args.kernel or args.split_k or args.waves_n)
+    prepared = prepared_applies(args.workload) and not args.unprepared and not forced
+    case = build_case(args.workload, dev, args.kernel, args.split_k, args.waves_n, prepared=prepared)
     ok, max_err = check_case(case, dev)
     torch.cuda.synchronize(dev)
     t = time_case(case, dev, args.steps, args.warmup)
     torch.cuda.synchronize(dev)
     s = summarize(case, t)
+    if prepared:
+        plain = build_case(args.workload, dev)
+        okp, _ = check_case(plain, dev)
+        s["unprepared_us"] = round(time_case(plain, dev, min(args.steps, 100), min(args.warmup, 10))["us"], 3)
+        ok = ok and okp
+        del plain
+        torch.cuda.empty_cache()
     bits, K, N, gs, desc_act, M = WORKLOADS[args.workload]
     gemv = M <= 8
     line = {
@@ -303,9 +323,11 @@ def main():
         "ms_per_step": round(s["us"] * 1e-3, 6), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": args.workload, "bits": bits, "K": K, "N": N, "M": M, "group_size": gs,
-                   "desc_act": desc_act, "weight_copies": len(case["qweights"]), "plan": s["plan"]},
+                   "desc_act": desc_act, "weight_copies": len(case["qweights"]), "plan": s["plan"],
+                   "entry": "gptq_hip_gemm_sorted" if prepared else "gptq_hip_gemm_plan",
+                   "prepared": "input channels sorted by group once at load" if prepared else None},
         "parity": {"ok": ok, "max_abs_err": round(max_err, 6), "rtol": 1e-2, "atol": 1e-2},
-        "timing": {k: s[k] for k in ("eager_us", "graph_us", "graph_error") if k in s},
+        "timing": {k: s[k] for k in ("eager_us", "graph_us", "graph_error", "unprepared_us") if k in s},
         "hbm_frac": s["hbm_frac"], "tflops": s["TFLOPs"],
     }
     if gemv:
@@ -317,10 +339,13 @@ def main():
                             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
     if args.sweep:
         sweep = []
-        for name in sorted(WORKLOADS):
-            c = build_case(name, dev)
+        for name, prep in [(n, pr) for n in sorted(WORKLOADS) for pr in (False, True)]:
+            if prep and not prepared_applies(name):
+                continue
+            c = build_case(name, dev, prepared=prep)
             okc, errc = check_case(c, dev)
             r = summarize(c, time_case(c, dev, min(args.steps, 100), min(args.warmup, 10)))
+            r["prepared"] = prep
             r["parity_ok"] = okc
             r["max_abs_err"] = round(errc, 6)
             sweep.append(r)

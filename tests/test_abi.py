@@ -138,6 +138,15 @@ def test_entry_points_reject_null_and_bad_sizes_before_touching_the_gpu():
     # a split-K plan without a workspace
     assert lib.gptq_hip_gemm(fake, fake, fake, fake, null, null, fake, null, 0, 1, 4096, 4096, 4, 128,
                              null) == _lib.ERR_WORKSPACE
+    # the sorted entry: no map, a misaligned map, a shape outside the decode family, K past the map's 16-bit positions,
+    # groups that are not whole lane blocks
+    srt = lib.gptq_hip_gemm_sorted
+    assert srt(fake, fake, fake, fake, null, null, fake, null, 0, 1, 4096, 11008, 3, 128, None, null) == _lib.ERR_BAD_ARG
+    assert srt(fake, fake, fake, fake, ctypes.c_void_p(0x1004), null, fake, null, 0, 1, 4096, 11008, 3, 128, None,
+               null) == _lib.ERR_BAD_ARG
+    assert srt(fake, fake, fake, fake, fake, null, fake, null, 0, 8, 4096, 11008, 3, 128, None, null) == _lib.ERR_UNSUPPORTED
+    assert srt(fake, fake, fake, fake, fake, null, fake, null, 0, 1, 65536, 64, 4, 128, None, null) == _lib.ERR_UNSUPPORTED
+    assert srt(fake, fake, fake, fake, fake, null, fake, null, 0, 1, 4096, 64, 3, 16, None, null) == _lib.ERR_UNSUPPORTED
     assert lib.gptq_hip_dequant(fake, fake, fake, null, null, 64, 64, 4, 32, null) == _lib.ERR_BAD_ARG
     assert lib.gptq_hip_dequant(fake, fake, fake, null, fake, 64, 64, 5, 32, null) == _lib.ERR_BAD_ARG
     assert lib.gptq_hip_workspace_init(null, 64, null) == _lib.ERR_BAD_ARG
@@ -171,6 +180,11 @@ def test_dispatcher_families_by_m():
     p = _lib.select(128, 4096, 11008, 3, 128, True)
     assert p.kernel == _lib.KERNEL_STREAM and p.row_tiles == 4 and p.m_blocks == 2 and p.split_k == 1
     assert p.workspace_bytes >= 128 * 4096 * 2
+    # activation order over many groups: past 48 the expansion by group loses to STREAM's lookups, while
+    # the same layer with its channels sorted at load is a plain GROUPED problem
+    assert _lib.select(1, 11008, 4096, 4, 128, True).kernel == _lib.KERNEL_STREAM
+    assert _lib.select(1, 5120, 4096, 3, 128, True).kernel == _lib.KERNEL_GROUPED
+    assert _lib.select(1, 11008, 4096, 4, 128, False).kernel == _lib.KERNEL_GROUPED
     # one group over a large matrix streams better without the expansion by group
     assert _lib.select(1, 9216, 36864, 3, -1, False).kernel == _lib.KERNEL_STREAM
     # forcing the STREAM family with waves along K and a split
