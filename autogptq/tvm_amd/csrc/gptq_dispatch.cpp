@@ -166,8 +166,10 @@ size_t stream_gpack_bytes(int bits, int steps_pad, int act_table)
 
 // LDS of the GROUPED kernel for a K range of kr channels: operand tiles (+ slot masks in the
 // compact two-tile layout) + the reduction buffer of the waves along K.
-int grouped_lds_bytes(int kr, int M, int tpm, int waves_n, int waves_k)
+int grouped_lds_bytes(int kr, int M, int tpm, int waves_n, int waves_k, bool lite)
 {
+    const int red = waves_k * waves_n * M * 64 * 4;
+    if (lite) return M * kr * 2 + 16 + red;  // x in unpack order, 16 zero bytes
     const int nblk8 = kr / 8;
     const bool compact = tpm == 2;
     const int stored = compact ? M : M * tpm;
@@ -209,7 +211,8 @@ bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, i
             if (act_order) return false;  // the group count does not shrink with the K range
             continue;
         }
-        const int lds = gptq::grouped_lds_bytes(kr, M, tpm, waves_n, waves_k);
+        const int lds = gptq::grouped_lds_bytes(kr, M, tpm, waves_n, waves_k,
+                                                gptq::grouped_lite(bits, K, gs, act_order != 0, tpm));
         if (lds > lds_cap) continue;
         plan->kernel = GPTQ_HIP_KERNEL_GROUPED;
         plan->row_tiles = M * tpm;
@@ -319,8 +322,11 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     // (48 groups) the expansion costs more than STREAM's lookup per weight (measured at N = 4096,
     // int3 / int4: K = 5120 16.1 / 11.6 us against 19.1 / 12.8; K = 8192 19.8 / 22.1 against 15.3 / 13.7;
     // K = 11008 79 / 93 against 20.1 / 16.8).
+    // With the lean operand (int3, contiguous groups) two rows also win when K is split (4096 x 4096
+    // 9.0 against 9.2 us, 11008 x 4096 12.0 against 13.1).
     if (M <= 2 && !one_big_group && plan_grouped(M, K, N, bits, gs, G, act_order, 0, 0, plan) &&
-        (M == 1 || plan->split_k == 1) && (!act_order || plan->row_tiles / M <= 3))
+        (M == 1 || plan->split_k == 1 || gptq::grouped_lite(bits, K, gs, act_order != 0, plan->row_tiles / M)) &&
+        (!act_order || plan->row_tiles / M <= 3))
         return GPTQ_HIP_OK;
     memset(plan, 0, sizeof(*plan));
     if (plan_stream(M, K, N, bits, gs, G, act_order, 0, 0, plan) == GPTQ_HIP_OK) return GPTQ_HIP_OK;

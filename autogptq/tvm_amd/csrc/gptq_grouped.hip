@@ -524,14 +524,11 @@ static int launch_grouped_one(const Params &p, const gptq_hip_plan &plan, hipStr
         // contiguous groups made of whole lane blocks: the lean operand.  Not for int4: its steps are
         // a quarter as long, and choosing the row per step costs what the lean prologue saves
         // (measured: 4096 x 4096 8.3 -> 8.7 us, 11008 x 4096 10.8 -> 11.7 us).
-        if (!p.g_idx && p.group_size % Fmt<BITS>::KLANE == 0 && p.K / Fmt<BITS>::KLANE < 65536)
+        if (grouped_lite(BITS, p.K, p.group_size, p.g_idx != nullptr, TPM))
             return launch_grouped_one<BITS, M, TPM, COMPACT, true>(p, plan, stream);
     }
     auto kern = grouped_kernel<BITS, M, TPM, COMPACT, NSTEP, LITE>;
-    // LITE keeps x itself (2 bytes per channel and row), 16 zero bytes and the waves' partial sums
-    const int lds_bytes =
-        LITE ? p.M * p.wave_steps * p.waves_k * Fmt<BITS>::KSTEP * 2 + 16 + p.waves_k * p.waves_n * p.M * 256
-             : plan.lds_bytes;
+    const int lds_bytes = plan.lds_bytes;  // sized by the dispatcher for the operand layout in use
     if (lds_bytes > 65536) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) !=
             hipSuccess) {

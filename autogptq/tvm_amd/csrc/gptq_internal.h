@@ -54,7 +54,13 @@ static const size_t kCounterBytes = 16384;
 // GROUPED kernel sizing, shared by the dispatcher and the plan check
 int grouped_tpm(int groups, int M);
 int grouped_groups(int kr, int gs, int G, int act_order);
-int grouped_lds_bytes(int kr, int M, int tpm, int waves_n, int waves_k);
+int grouped_lds_bytes(int kr, int M, int tpm, int waves_n, int waves_k, bool lite);
+// The lean operand (x itself in LDS instead of operand tiles): int3, groups that are contiguous for the
+// weight stream and made of whole 32-channel lane blocks, one row tile.
+constexpr bool grouped_lite(int bits, int K, int gs, bool has_g_idx, int tpm)
+{
+    return bits == 3 && !has_g_idx && tpm == 1 && gs % 32 == 0 && K / 32 < 65536;
+}
 // Input channels of x the GATHER kernel stages per K wave at a time: fixed per (bits, row tiles) so
 // that the kernel's unrolled step loop knows its chunk boundaries at compile time.  The chunk is a
 // whole number of steps that divides the weight prefetch depth (8 steps int4, 4 steps int3).

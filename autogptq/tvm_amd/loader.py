@@ -130,11 +130,14 @@ def load_quantized_state(model: nn.Module, state: Dict[str, torch.Tensor], devic
 
 def from_quantized(save_dir: str, device="cuda:0", model_basename: Optional[str] = None,
                    use_safetensors: bool = True, ignore_layers: Iterable[str] = ("lm_head",),
-                   trust_remote_code: bool = False):
+                   trust_remote_code: bool = False, fuse_shared_inputs: bool = False):
     """Builds the ``transformers`` causal LM described by ``save_dir/config.json`` with every linear
     layer (except ``ignore_layers`` prefixes: the reference skips ``lm_head`` and the modules outside
     the decoder stack) replaced by ``QuantLinear``, and fills it from
-    ``save_dir/gptq_model-{bits}bit-{group_size}g.{safetensors|bin}``.  Returns ``(model, quantize_config)``."""
+    ``save_dir/gptq_model-{bits}bit-{group_size}g.{safetensors|bin}``.  ``fuse_shared_inputs`` then merges
+    q/k/v and gate/up projections into one product each (``fused.fuse_shared_input_layers``; an inference
+    optimisation the reference does not have: the state-dict names of those layers change).
+    Returns ``(model, quantize_config)``."""
     import accelerate
     from transformers import AutoConfig, AutoModelForCausalLM
 
@@ -166,6 +169,10 @@ def from_quantized(save_dir: str, device="cuda:0", model_basename: Optional[str]
     load_quantized_state(model, state, device)
     if hasattr(model, "tie_weights"):
         model.tie_weights()
+    if fuse_shared_inputs:
+        from .fused import fuse_shared_input_layers
+
+        fuse_shared_input_layers(model)
     seqlen = 4096
     for key in ("max_position_embeddings", "seq_length", "n_positions"):
         if key in model.config.to_dict():

@@ -55,6 +55,11 @@ WORKLOADS = {
     "int4-11008x4096-act-m1": (4, 11008, 4096, 128, True, 1),
     "int3-4096x4096-act-m1": (3, 4096, 4096, 128, True, 1),
     "int3-4096x11008-m1": (3, 4096, 11008, 128, False, 1),
+    # q/k/v and gate/up of a 4096-wide block as one product each (fused.fuse_shared_input_layers)
+    "qkv-int4-4096x12288-act-m1": (4, 4096, 12288, 128, True, 1),
+    "qkv-int3-4096x12288-act-m1": (3, 4096, 12288, 128, True, 1),
+    "gateup-int4-4096x22016-act-m1": (4, 4096, 22016, 128, True, 1),
+    "gateup-int3-4096x22016-act-m1": (3, 4096, 22016, 128, True, 1),
     "c4-int4-4096x11008-act-m16": (4, 4096, 11008, 128, True, 16),
     "c4-int4-4096x11008-act-m64": (4, 4096, 11008, 128, True, 64),
     "c4-int4-4096x11008-act-m128": (4, 4096, 11008, 128, True, 128),

@@ -20,7 +20,10 @@ def rtn_quantize(weight: torch.Tensor, bits: int, gs: int):
     return scales, zeros
 
 
-def build_checkpoint(tmp_dir: str, bits: int = 4, gs: int = 32, act_order: bool = True, seed: int = 0):
+def build_checkpoint(tmp_dir: str, bits: int = 4, gs: int = 32, act_order: bool = True, seed: int = 0,
+                     shared_order: bool = False):
+    """shared_order: layers that read the same input (q/k/v, gate/up) get the same g_idx, as GPTQ
+    produces them (its activation order depends on the inputs only)."""
     from safetensors.torch import save_file
     from transformers import AutoModelForCausalLM, LlamaConfig
 
@@ -35,6 +38,7 @@ def build_checkpoint(tmp_dir: str, bits: int = 4, gs: int = 32, act_order: bool 
     state = {k: v.clone() for k, v in model.state_dict().items()}
     dense = {}  # name -> the fp16 weight the quantised layer represents
     gen = torch.Generator().manual_seed(seed + 1)
+    shared_g = None
     for name, layer in find_layers(model).items():
         if name.startswith("lm_head"):
             continue
@@ -42,6 +46,12 @@ def build_checkpoint(tmp_dir: str, bits: int = 4, gs: int = 32, act_order: bool 
         scales, zeros = rtn_quantize(layer.weight.data, bits, gs)
         if act_order:
             g_idx = (torch.randperm(K, generator=gen) // gs).to(torch.int32)
+            if shared_order:
+                leaf = name.rsplit(".", 1)[-1]
+                if leaf in ("k_proj", "v_proj", "up_proj"):
+                    g_idx = shared_g
+                else:
+                    shared_g = g_idx
             # quantise against the permuted grouping so that codes stay in range
             w = layer.weight.data.float()
             G = K // gs
