@@ -152,7 +152,22 @@ static int run_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros
             p.gdiv_magic = (uint32_t)((1ull << 32) / d) + 1u;
         }
     }
-    if (kmap) {
+    size_t ws_plan = workspace_bytes;  // bytes of the workspace the plan itself may use
+    if (kmap && plan->kernel == GPTQ_HIP_KERNEL_STREAM) {
+        // small batches on a sorted layer: x goes into the sorted channel order first (one small pass
+        // into the tail of the workspace), then the kernel for contiguous groups reads it directly
+        if (M > gptq::kSortedMaxRows || plan->row_tiles != 1 ||
+            !gptq::stream_direct(bits, K, 1, gptq::stream_act_table(bits, gs, 0), false))
+            return GPTQ_HIP_ERR_UNSUPPORTED;
+        const size_t head = gptq::sorted_x_offset(plan->workspace_bytes);
+        const size_t xs_bytes = (size_t)M * K * 2;
+        if (!workspace || workspace_bytes < head + xs_bytes || !aligned(workspace, 16)) return GPTQ_HIP_ERR_WORKSPACE;
+        void *xs = (char *)workspace + head;
+        rc = gptq::launch_permute_x(x, kmap + K, xs, M, K, stream);
+        if (rc != GPTQ_HIP_OK) return rc;
+        p.x = xs;
+        ws_plan = head;
+    } else if (kmap) {
         // positions are below 65536 and a wave holds at least one step: the multiply-high is exact
         if (plan->kernel != GPTQ_HIP_KERNEL_GROUPED) return GPTQ_HIP_ERR_UNSUPPORTED;
         // a workgroup that holds all of K, or a short x, walks x once and keeps its channels; with K
@@ -187,7 +202,7 @@ static int run_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros
             }
             if (plan->split_k > 1) {
                 const size_t need = gptq::kCounterBytes + part;
-                if (!workspace || workspace_bytes < need || !aligned(workspace, 16)) return GPTQ_HIP_ERR_WORKSPACE;
+                if (!workspace || ws_plan < need || !aligned(workspace, 16)) return GPTQ_HIP_ERR_WORKSPACE;
                 p.counters = (int *)workspace;
                 p.partial = (float *)((char *)workspace + gptq::kCounterBytes);
             }
@@ -239,9 +254,19 @@ extern "C" int gptq_hip_gemm_sorted(const void *x, const int32_t *qweight_sorted
         if (rc != GPTQ_HIP_OK) return rc;
         plan = &chosen;
     }
-    if (plan->kernel != GPTQ_HIP_KERNEL_GROUPED) return GPTQ_HIP_ERR_UNSUPPORTED;
+    if (plan->kernel != GPTQ_HIP_KERNEL_GROUPED && !(plan->kernel == GPTQ_HIP_KERNEL_STREAM && M <= gptq::kSortedMaxRows))
+        return GPTQ_HIP_ERR_UNSUPPORTED;
     return run_gemm(x, qweight_sorted, qzeros, scales, nullptr, kmap, bias, y, workspace, workspace_bytes, M, K, N,
                     bits, group_size, plan, stream);
+}
+
+extern "C" size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits, int group_size)
+{
+    gptq_hip_plan plan;
+    if (gptq_hip_select(M, K, N, bits, group_size, 0, &plan) != GPTQ_HIP_OK) return 0;
+    if (plan.kernel == GPTQ_HIP_KERNEL_STREAM && M <= gptq::kSortedMaxRows)
+        return gptq::sorted_x_offset(plan.workspace_bytes) + (size_t)M * K * 2;
+    return plan.workspace_bytes;
 }
 
 extern "C" int gptq_hip_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,

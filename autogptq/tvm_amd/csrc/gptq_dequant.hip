@@ -64,6 +64,36 @@ int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const void *
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 
+// xs[m][j] = x[m][src[j]]: the activations of a layer whose channels were sorted by group, in the
+// sorted order.  Eight outputs per thread: two index vectors, eight 2-byte gathers (x is small and
+// stays in L2), one 16-byte store.  K is a multiple of 32.
+__global__ __launch_bounds__(256) void permute_x_kernel(const _Float16 *x, const int32_t *src, _Float16 *xs, int M,
+                                                        int K)
+{
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t per_row = (uint32_t)K / 8u;
+    if (t >= (uint32_t)M * per_row) return;
+    const uint32_t m = t / per_row;
+    const uint32_t j = 8u * (t - m * per_row);
+    const int4 a = *(const int4 *)(src + j);
+    const int4 b = *(const int4 *)(src + j + 4);
+    const int idx[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    const _Float16 *row = x + (size_t)m * K;
+    h8 o;
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] = row[min((uint32_t)idx[e], (uint32_t)K - 1u)];  // a bad map must not fault
+    *(h8 *)(xs + (size_t)m * K + j) = o;
+}
+
+int launch_permute_x(const void *x, const int32_t *src, void *xs, int M, int K, void *stream_v)
+{
+    hipStream_t stream = (hipStream_t)stream_v;
+    const unsigned threads = (unsigned)M * (unsigned)(K / 8);
+    hipLaunchKernelGGL(permute_x_kernel, dim3((threads + 255u) / 256u), dim3(256), 0, stream, (const _Float16 *)x, src,
+                       (_Float16 *)xs, M, K);
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+}
+
 int launch_fill_zero(void *ptr, size_t bytes, void *stream_v)
 {
     hipStream_t stream = (hipStream_t)stream_v;

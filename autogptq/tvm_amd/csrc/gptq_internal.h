@@ -115,5 +115,16 @@ int launch_grouped(const Params &p, int bits, const gptq_hip_plan &plan, void *s
 int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
                    void *w, int K, int N, int G, int bits, int group_size, void *stream);
 int launch_fill_zero(void *ptr, size_t bytes, void *stream);
+int launch_permute_x(const void *x, const int32_t *src, void *xs, int M, int K, void *stream);
+// Rows of x up to which the sorted entry point covers small batches (the STREAM kernel that reads x
+// itself, behind a pass that puts x into the sorted channel order)
+static const int kSortedMaxRows = 16;
+// where that pass puts x in the workspace: behind what the plan itself uses, and never over the
+// counters at the head, which every call must leave zero
+inline size_t sorted_x_offset(size_t plan_bytes)
+{
+    const size_t head = plan_bytes > kCounterBytes ? plan_bytes : kCounterBytes;
+    return (head + 255) / 256 * 256;
+}
 
 }  // namespace gptq

@@ -106,9 +106,13 @@ def gemm(x: torch.Tensor, qweight: torch.Tensor, qzeros: torch.Tensor, scales: t
     return out
 
 
+SORTED_MAX_ROWS = 16
+
+
 def sorted_plan(M: int, K: int, N: int, bits: int, group_size: int) -> Optional[_lib.Plan]:
     """The plan ``gemm_sorted`` would run, or None when the sorted path does not cover the problem
-    (it is for decode sizes: the GROUPED family)."""
+    (it is for decode sizes: the GROUPED family, or up to ``SORTED_MAX_ROWS`` rows on the STREAM kernel
+    that reads x itself)."""
     gs = K if group_size == -1 else group_size
     if K >= 65536 or K % gs != 0 or gs % (8 if bits == 4 else 32) != 0:
         return None
@@ -116,14 +120,22 @@ def sorted_plan(M: int, K: int, N: int, bits: int, group_size: int) -> Optional[
         plan = _lib.select(M, K, N, bits, group_size, False)
     except _lib.GptqHipError:
         return None
-    return plan if plan.kernel == _lib.KERNEL_GROUPED else None
+    if plan.kernel == _lib.KERNEL_GROUPED:
+        return plan
+    if plan.kernel == _lib.KERNEL_STREAM and M <= SORTED_MAX_ROWS and plan.row_tiles == 1:
+        # the pass that reorders x costs a launch (~2 us): int3 gains 2-4 us over the per-weight lookups
+        # of the unsorted kernel at every size measured, int4 1-2 us at 4096 x 11008 and 11008 x 4096
+        # but loses 0.7 us at 4096 x 4096
+        if bits == 3 or K * N >= (1 << 25):
+            return plan
+    return None
 
 
 def gemm_sorted(x: torch.Tensor, qweight_sorted: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
                 kmap: torch.Tensor, bias: Optional[torch.Tensor], bits: int, group_size: int,
                 plan: Optional[_lib.Plan] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``gemm`` for an activation-order layer whose channels ``pack.sort_channels_by_group`` sorted by
-    group; ``x`` and the result are in the layer's original channel order.  M <= 2."""
+    group; ``x`` and the result are in the layer's original channel order.  M <= ``SORTED_MAX_ROWS``."""
     _need_gpu("x", x, torch.float16)
     _need_gpu("qweight_sorted", qweight_sorted, torch.int32)
     _need_gpu("qzeros", qzeros, torch.int32)
@@ -146,7 +158,10 @@ def gemm_sorted(x: torch.Tensor, qweight_sorted: torch.Tensor, qzeros: torch.Ten
         plan = sorted_plan(M, K, N, bits, group_size)
         if plan is None:
             raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, f"gptq_hip_gemm_sorted(M={M}, K={K}, N={N}, bits={bits})")
-    ws = _workspace(dev, plan.workspace_bytes) if plan.workspace_bytes else None
+    ws_bytes = plan.workspace_bytes
+    if plan.kernel == _lib.KERNEL_STREAM:   # x in the sorted order goes behind what the plan itself uses
+        ws_bytes = _lib.lib().gptq_hip_sorted_workspace_bytes(M, K, N, bits, group_size)
+    ws = _workspace(dev, ws_bytes) if ws_bytes else None
     with torch.cuda.device(dev):
         rc = _lib.lib().gptq_hip_gemm_sorted(
             _ptr(x), _ptr(qweight_sorted), _ptr(qzeros), _ptr(scales), _ptr(kmap), _ptr(bias), _ptr(out),

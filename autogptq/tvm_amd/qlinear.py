@@ -51,7 +51,7 @@ class QuantLinear(nn.Module):
         else:
             self.bias = None
         self._g_state = None  # (g_idx identity, contiguous?) cached by _kernel_g_idx
-        # Activation-order layers: on the first decode-size call (one or two rows of x), keep a second
+        # Activation-order layers: on the first decode-size call (up to 16 rows of x), keep a second
         # copy of qweight with the input channels sorted by group (plus a [K] int32 map), which the
         # decode kernel reads faster than it can follow g_idx.  Costs the layer's packed size again in
         # device memory; False keeps only the checkpoint's tensors.
@@ -146,7 +146,7 @@ class QuantLinear(nn.Module):
         try:
             if self.kernel_switch_threshold and x2.shape[0] >= self.kernel_switch_threshold:
                 raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, "above kernel_switch_threshold")
-            out = self._decode_sorted(x2) if (self.sort_for_decode and 0 < x2.shape[0] <= 2) else None
+            out = self._decode_sorted(x2) if (self.sort_for_decode and 0 < x2.shape[0] <= ops.SORTED_MAX_ROWS) else None
             if out is None:
                 out = ops.gemm(x2, self.qweight, self.qzeros, self.scales, self._kernel_g_idx(), self.bias,
                                self.bits, self.groupsize)

@@ -114,15 +114,22 @@ def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int =
         case["qweights"][0], case["kmap"] = sort_channels_by_group(qweights[0], case["g_idx"], bits, gs)
         case["g_idx"] = None
         desc_act = False  # the plan is that of contiguous groups
-        kernel = kernel or _lib.KERNEL_GROUPED
-    if kernel or split_k or waves_n:
+    if prepared and not (kernel or split_k or waves_n):
+        from autogptq.tvm_amd import ops
+
+        plan = ops.sorted_plan(M, K, N, bits, gs)
+    elif kernel or split_k or waves_n:
         if not kernel:
             kernel = _lib.select(M, K, N, bits, gs, desc_act).kernel
         plan = _lib.plan_for(kernel, M, K, N, bits, gs, desc_act, split_k, waves_n)
     else:
         plan = _lib.select(M, K, N, bits, gs, desc_act)
     case["plan"] = plan
-    case["ws"] = torch.zeros(max(plan.workspace_bytes, 16), dtype=torch.uint8, device=dev)
+    ws_bytes = plan.workspace_bytes
+    if prepared and plan.kernel == _lib.KERNEL_STREAM:   # x in the sorted order goes behind the plan's own bytes
+        ws_bytes = _lib.lib().gptq_hip_sorted_workspace_bytes(M, K, N, bits, gs)
+    case["ws_bytes"] = ws_bytes
+    case["ws"] = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
     return case
 
 
@@ -131,7 +138,7 @@ def prepared_applies(name: str) -> bool:
 
     bits, K, N, gs, desc_act, M = WORKLOADS[name]
     G = 1 if gs == -1 else -(-K // gs)
-    return bool(desc_act and G > 1 and M <= 2 and ops.sorted_plan(M, K, N, bits, gs) is not None)
+    return bool(desc_act and G > 1 and M <= ops.SORTED_MAX_ROWS and ops.sorted_plan(M, K, N, bits, gs) is not None)
 
 
 def make_step(case, dev):
@@ -146,10 +153,10 @@ def make_step(case, dev):
     common = dict(
         x=vp(case["x"].data_ptr()), qz=vp(case["qzeros"].data_ptr()), sc=vp(case["scales"].data_ptr()),
         g=vp(gmap.data_ptr()) if gmap is not None else None,
-        y=vp(case["y"].data_ptr()), ws=vp(case["ws"].data_ptr()) if case["plan"].workspace_bytes else None,
+        y=vp(case["y"].data_ptr()), ws=vp(case["ws"].data_ptr()) if case["ws_bytes"] else None,
     )
     qws = [vp(q.data_ptr()) for q in case["qweights"]]
-    wsb = case["plan"].workspace_bytes
+    wsb = case["ws_bytes"]
     M, K, N, bits, gs = case["M"], case["K"], case["N"], case["bits"], case["gs"]
     planp = ctypes.byref(case["plan"])
     n = len(qws)

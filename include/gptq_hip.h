@@ -106,7 +106,7 @@ int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const int32_t *qze
                        int M, int K, int N, int bits, int group_size, const gptq_hip_plan *plan, void *stream);
 
 /*
- * The decode product (M <= 2) for a layer prepared when it was loaded: an activation-order g_idx makes
+ * The decode product (one row, or a batch of up to 16) for a layer prepared when it was loaded: an activation-order g_idx makes
  * every weight look its group up (qlinear.py:200-242 gathers scales and zeros by g_idx), so the
  * loader sorts the input channels by group once; qweight_sorted holds the same codes with groups
  * contiguous along K and
@@ -114,14 +114,23 @@ int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const int32_t *qze
  *                                      order the kernels unpack codes; kmap[k] >> 16 = g_idx[k];
  *                                      kmap[K + j] = the channel whose codes are j-th along K in qweight_sorted
  * tells the kernel where each x[m, k] belongs.  x and y are in the layer's original channel order.
- * qzeros and scales are unchanged.  plan: NULL lets the dispatcher choose, else a GROUPED plan for
- * (M, K, N, bits, group_size, act_order = 0); workspace as that plan asks.  Needs K < 65536, equal
- * groups and group_size a multiple of 8 (int4) or 32 (int3); GPTQ_HIP_ERR_UNSUPPORTED otherwise, or
- * when the problem is not one for the GROUPED family.  One launch.
+ * qzeros and scales are unchanged.  plan: NULL lets the dispatcher choose, else a plan for
+ * (M, K, N, bits, group_size, act_order = 0) of the GROUPED family (one launch; the scatter of x into
+ * LDS follows the map) or, for M <= 16, of the STREAM family with one row tile (a small pass first
+ * writes x in the sorted order into the tail of the workspace, then the kernel for contiguous groups
+ * runs: two or three launches).  workspace: gptq_hip_sorted_workspace_bytes, zeroed like any other.
+ * Needs K < 65536, equal groups and group_size a multiple of 8 (int4) or 32 (int3);
+ * GPTQ_HIP_ERR_UNSUPPORTED otherwise, or for larger batches (they run on the checkpoint's own
+ * tensors through gptq_hip_gemm).
  */
 int gptq_hip_gemm_sorted(const void *x, const int32_t *qweight_sorted, const int32_t *qzeros, const void *scales,
                          const int32_t *kmap, const void *bias, void *y, void *workspace, size_t workspace_bytes,
                          int M, int K, int N, int bits, int group_size, const gptq_hip_plan *plan, void *stream);
+
+/* Bytes of workspace gptq_hip_gemm_sorted needs with plan = NULL (0 if none): what the plan for contiguous
+ * groups needs and, when that plan is a STREAM one, M*K*2 bytes for x in the sorted order behind it (at
+ * max(plan bytes, 16 KiB) rounded up to 256: the counters at the head of a workspace stay untouched). */
+size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits, int group_size);
 
 /*
  * W fp16 [K, N] = scales[g] * (q - (zq[g] + 1)), one rounding per element:

@@ -144,7 +144,13 @@ def test_entry_points_reject_null_and_bad_sizes_before_touching_the_gpu():
     assert srt(fake, fake, fake, fake, null, null, fake, null, 0, 1, 4096, 11008, 3, 128, None, null) == _lib.ERR_BAD_ARG
     assert srt(fake, fake, fake, fake, ctypes.c_void_p(0x1004), null, fake, null, 0, 1, 4096, 11008, 3, 128, None,
                null) == _lib.ERR_BAD_ARG
-    assert srt(fake, fake, fake, fake, fake, null, fake, null, 0, 8, 4096, 11008, 3, 128, None, null) == _lib.ERR_UNSUPPORTED
+    # a small batch runs behind a pass that reorders x into the workspace: none given
+    assert srt(fake, fake, fake, fake, fake, null, fake, null, 0, 8, 4096, 11008, 3, 128, None, null) == _lib.ERR_WORKSPACE
+    assert srt(fake, fake, fake, fake, fake, null, fake, null, 0, 17, 4096, 11008, 3, 128, None, null) == _lib.ERR_UNSUPPORTED
+    assert lib.gptq_hip_sorted_workspace_bytes(8, 4096, 11008, 3, 128) == 16384 + 8 * 4096 * 2   # behind the counters
+    assert lib.gptq_hip_sorted_workspace_bytes(1, 4096, 11008, 3, 128) == 0
+    p4 = _lib.select(4, 11008, 4096, 4, 128, False)
+    assert lib.gptq_hip_sorted_workspace_bytes(4, 11008, 4096, 4, 128) == (max(p4.workspace_bytes, 16384) + 255) // 256 * 256 + 4 * 11008 * 2
     assert srt(fake, fake, fake, fake, fake, null, fake, null, 0, 1, 65536, 64, 4, 128, None, null) == _lib.ERR_UNSUPPORTED
     assert srt(fake, fake, fake, fake, fake, null, fake, null, 0, 1, 4096, 64, 3, 16, None, null) == _lib.ERR_UNSUPPORTED
     assert lib.gptq_hip_dequant(fake, fake, fake, null, null, 64, 64, 4, 32, null) == _lib.ERR_BAD_ARG

@@ -296,6 +296,35 @@ def test_sorted_decode_matches_oracle_and_unsorted_kernel(dev, bits, K, N, gs, M
 
 
 @pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("K,N,gs", [(1024, 416, 32), (2048, 1056, 256), (11008, 256, 128), (4096, 352, 128), (1024, 160, -1)])
+@pytest.mark.parametrize("M", [3, 8, 16])
+def test_sorted_small_batch_matches_oracle(dev, bits, K, N, gs, M):
+    # up to 16 rows: x is put into the sorted order by a small pass, then the kernel for contiguous groups runs
+    L = layer(930 + K + M, K, N, bits, gs, True, M=M, bias=True)
+    D = to_dev(L, dev)
+    plan = ops.sorted_plan(M, K, N, bits, gs)
+    if plan is None:
+        pytest.skip("not covered by the sorted path")
+    assert plan.kernel == _lib.KERNEL_STREAM and plan.row_tiles == 1
+    want = expected_output(L)
+    y = run_sorted(D)
+    assert_close(y, want, "sorted small batch")
+    assert_tight(y, want, "sorted small batch")
+    assert torch.equal(y, run_sorted(D))
+    # x in the sorted order sits behind the counters at the head of the shared workspace: a split-K
+    # call on the same stream right after still finds them zero
+    L2 = layer(931, 512, 192, bits, 128, False, M=1)
+    assert _lib.select(1, 512, 192, bits, 128, False).split_k > 1
+    assert_close(run_gemm(to_dev(L2, dev)), expected_output(L2), "split-K call after a sorted small batch")
+    with pytest.raises(_lib.GptqHipError) as e:    # larger batches are not for this entry point
+        qs, kmap = pack.sort_channels_by_group(D["qweight"], D["g_idx"], bits, gs)
+        x17 = torch.zeros((17, K), dtype=torch.float16, device=dev)
+        ops.gemm_sorted(x17, qs, D["qzeros"], D["scales"], kmap, None, bits, gs,
+                        plan=_lib.select(17, K, N, bits, gs, False))
+    assert e.value.status == _lib.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("bits", [3, 4])
 @pytest.mark.parametrize("M", [1, 2])
 @pytest.mark.parametrize("split", [1, 2, 5, 16])
 def test_sorted_decode_forced_split_k(dev, bits, M, split):
@@ -349,6 +378,8 @@ def test_quantlinear_decode_uses_the_sorted_copy(dev, bits):
     assert q._sorted is not None and q._sorted[1] is not None     # built by the first decode-size call
     assert_close(y, expected_output(L), "module decode, sorted")
     assert_close(q(L["x"][:1].to(dev)), expected_output(L)[:1], "module decode, sorted, one row")
+    x8 = torch.randn(8, K, generator=torch.Generator().manual_seed(8)).half()
+    assert_close(q(x8.to(dev)), expected_output(L, x=x8), "module small batch, sorted")
     # switching the preparation off gives the same numbers from the checkpoint's own tensors
     q.sort_for_decode = False
     assert_tight(q(L["x"].to(dev)), y.cpu(), "module decode, unsorted")
