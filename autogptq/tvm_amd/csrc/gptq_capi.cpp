@@ -8,11 +8,12 @@ namespace {
 
 bool aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
 
+// wide: also the widths only the dequant kernel covers (2 and 8 bits)
 int check_common(const int32_t *qweight, const int32_t *qzeros, const void *scales, int K, int N, int bits,
-                 int group_size)
+                 int group_size, bool wide = false)
 {
     if (!qweight || !qzeros || !scales) return GPTQ_HIP_ERR_BAD_ARG;
-    if (bits != 3 && bits != 4) return GPTQ_HIP_ERR_BAD_ARG;
+    if (bits != 3 && bits != 4 && !(wide && (bits == 2 || bits == 8))) return GPTQ_HIP_ERR_BAD_ARG;
     if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;
     if ((long long)K * N * bits / 8 >= (1LL << 31)) return GPTQ_HIP_ERR_UNSUPPORTED;  // kernels use 32-bit byte offsets
     if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
@@ -285,7 +286,7 @@ extern "C" int gptq_hip_dequant(const int32_t *qweight, const int32_t *qzeros, c
                                 void *stream)
 {
     if (!w) return GPTQ_HIP_ERR_BAD_ARG;
-    const int rc = check_common(qweight, qzeros, scales, K, N, bits, group_size);
+    const int rc = check_common(qweight, qzeros, scales, K, N, bits, group_size, true);
     if (rc != GPTQ_HIP_OK) return rc;
     const int gs = group_size == -1 ? K : group_size;
     const int G = (K + gs - 1) / gs;

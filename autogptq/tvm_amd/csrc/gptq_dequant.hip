@@ -34,10 +34,10 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint32_t *__restrict
             g_prev = g;
         }
         int q;
-        if constexpr (BITS == 4) {
-            q = code4(w[j >> 3], j & 7);
-        } else {
+        if constexpr (BITS == 3) {
             q = code3(w[0], w[1], w[2], j);
+        } else {
+            q = code_pow2<BITS>(w, j);
         }
         W[(size_t)k * N + n] = dequant_one(s, q, z);
     }
@@ -54,13 +54,17 @@ int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const void *
 {
     hipStream_t stream = (hipStream_t)stream_v;
     const dim3 grid((N + 255) / 256, K / 32);
-    if (bits == 4) {
-        hipLaunchKernelGGL(dequant_kernel<4>, grid, dim3(256), 0, stream, qweight, qzeros,
-                           (const _Float16 *)scales, g_idx, (_Float16 *)w, K, N, G, group_size);
-    } else {
-        hipLaunchKernelGGL(dequant_kernel<3>, grid, dim3(256), 0, stream, qweight, qzeros,
-                           (const _Float16 *)scales, g_idx, (_Float16 *)w, K, N, G, group_size);
+#define GPTQ_LAUNCH_DEQUANT(B)                                                                           \
+    hipLaunchKernelGGL(dequant_kernel<B>, grid, dim3(256), 0, stream, qweight, qzeros, (const _Float16 *)scales, \
+                       g_idx, (_Float16 *)w, K, N, G, group_size)
+    switch (bits) {
+        case 2: GPTQ_LAUNCH_DEQUANT(2); break;
+        case 3: GPTQ_LAUNCH_DEQUANT(3); break;
+        case 4: GPTQ_LAUNCH_DEQUANT(4); break;
+        case 8: GPTQ_LAUNCH_DEQUANT(8); break;
+        default: return GPTQ_HIP_ERR_BAD_ARG;
     }
+#undef GPTQ_LAUNCH_DEQUANT
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 

@@ -61,7 +61,11 @@ __device__ __forceinline__ int slot_of_code(int j)
 template <int BITS>
 __device__ __forceinline__ int zero_of(const uint32_t *zrow, int n)
 {
-    return BITS == 4 ? zero4(zrow, n) : zero3(zrow, n);
+    if constexpr (BITS == 3) {
+        return zero3(zrow, n);
+    } else {
+        return code_pow2<BITS>(zrow + (n >> 5) * BITS, n & 31) + 1;
+    }
 }
 
 // The words holding the four zero points of columns n .. n+3 (n % 4 == 0) of the qzeros row

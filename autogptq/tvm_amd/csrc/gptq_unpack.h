@@ -49,6 +49,14 @@ GPTQ_HD int code3(uint32_t w0, uint32_t w1, uint32_t w2, int j)
     return (int)(v & 0x7u);
 }
 
+// Widths that divide a word (2, 4, 8 bits): code j of a block of 32 codes held in `BITS` words.
+template <int BITS>
+GPTQ_HD int code_pow2(const uint32_t *w, int j)
+{
+    static_assert(BITS == 2 || BITS == 4 || BITS == 8, "width must divide 32");
+    return (int)((w[(BITS * j) >> 5] >> ((BITS * j) & 31)) & ((1u << BITS) - 1u));
+}
+
 // Zero point (already +1) of column n from a packed qzeros row
 // (reference: qlinear.py:202-209, :217-227).
 GPTQ_HD int zero4(const uint32_t *zrow, int n) { return code4(zrow[n >> 3], n & 7) + 1; }

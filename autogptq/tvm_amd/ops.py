@@ -30,9 +30,13 @@ def _stream(device: torch.device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
-def check_shapes(qweight, qzeros, scales, g_idx, bias, bits: int, group_size: int):
-    if bits not in (3, 4):
-        raise NotImplementedError("Only 3 and 4 bits are supported.")
+FUSED_BITS = (3, 4)        # widths the matmul kernels cover
+FORMAT_BITS = (2, 3, 4, 8)  # widths of the checkpoint format; 2 and 8 run as dequant + library GEMM
+
+
+def check_shapes(qweight, qzeros, scales, g_idx, bias, bits: int, group_size: int, widths=FUSED_BITS):
+    if bits not in widths:
+        raise NotImplementedError(f"Only {', '.join(map(str, widths))} bits are supported here.")
     rows, N = qweight.shape
     if rows * 32 % bits != 0:
         raise ValueError(f"qweight has {rows} rows, not a multiple of bits={bits} words per 32 channels")
@@ -180,7 +184,7 @@ def dequant(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
     _need_gpu("scales", scales, torch.float16)
     if g_idx is not None:
         _need_gpu("g_idx", g_idx, torch.int32)
-    K, N, _ = check_shapes(qweight, qzeros, scales, g_idx, None, bits, group_size)
+    K, N, _ = check_shapes(qweight, qzeros, scales, g_idx, None, bits, group_size, widths=FORMAT_BITS)
     dev = qweight.device
     w = torch.empty((K, N), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):

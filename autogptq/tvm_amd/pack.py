@@ -18,15 +18,16 @@ def pack_along_axis0(codes: np.ndarray, bits: int) -> np.ndarray:
     rows, cols = codes.shape
     if rows % 32 != 0:
         raise ValueError(f"packed axis length {rows} is not a multiple of 32")
-    if bits not in (3, 4):
-        raise NotImplementedError("Only 3 and 4 bits are supported.")
+    if bits not in (2, 3, 4, 8):
+        raise NotImplementedError("Only 2, 3, 4 and 8 bits are supported.")
     blocks = codes.reshape(rows // 32, 32, cols).astype(np.uint64)
-    if bits == 4:
-        # 32 codes -> one 128-bit stream = four words of 8 codes
-        b = blocks.reshape(rows // 32, 4, 8, cols)
-        shifts = (4 * np.arange(8, dtype=np.uint64)).reshape(1, 1, 8, 1)
+    if bits != 3:
+        # widths that divide a word: 32 codes -> `bits` words of 32 / bits codes each
+        per = 32 // bits
+        b = blocks.reshape(rows // 32, bits, per, cols)
+        shifts = (bits * np.arange(per, dtype=np.uint64)).reshape(1, 1, per, 1)
         words = np.bitwise_or.reduce(b << shifts, axis=2)
-        return words.reshape(rows // 8, cols).astype(np.uint32).view(np.int32)
+        return words.reshape(rows // per, cols).astype(np.uint32).view(np.int32)
     # 3 bits: a 96-bit stream; build it in two 64-bit halves that overlap nowhere
     out = np.zeros((rows // 32, 3, cols), dtype=np.uint64)
     for j in range(32):
@@ -54,15 +55,17 @@ def pack_qzeros(zeros: np.ndarray, bits: int) -> np.ndarray:
 
 def unpack_along_axis0(words: np.ndarray, bits: int) -> np.ndarray:
     """Inverse of pack_along_axis0: int32 [R//32*bits, C] -> codes uint8 [R, C]."""
-    if bits not in (3, 4):
-        raise NotImplementedError("Only 3 and 4 bits are supported.")
+    if bits not in (2, 3, 4, 8):
+        raise NotImplementedError("Only 2, 3, 4 and 8 bits are supported.")
     w = np.ascontiguousarray(words).view(np.uint32)
     rows, cols = w.shape
     if rows % bits != 0:
         raise ValueError(f"{rows} packed rows are not a multiple of bits={bits}")
-    if bits == 4:
-        shifts = (4 * np.arange(8, dtype=np.uint32)).reshape(1, 8, 1)
-        return ((w[:, None, :] >> shifts) & np.uint32(15)).astype(np.uint8).reshape(rows * 8, cols)
+    if bits != 3:
+        per = 32 // bits
+        shifts = (bits * np.arange(per, dtype=np.uint32)).reshape(1, per, 1)
+        mask = np.uint32((1 << bits) - 1)
+        return ((w[:, None, :] >> shifts) & mask).astype(np.uint8).reshape(rows * per, cols)
     b = w.reshape(rows // 3, 3, cols).astype(np.uint64)
     lo = b[:, 0, :] | (b[:, 1, :] << np.uint64(32))       # stream bits 0..63
     hi = (b[:, 1, :] >> np.uint64(31)) | (b[:, 2, :] << np.uint64(1))  # stream bits 63..95 at bit 0

@@ -19,15 +19,32 @@ from . import _lib, ops
 from .pack import pack_qweight, pack_qzeros, sort_channels_by_group
 
 
+class _ProductWithInputGrad(torch.autograd.Function):
+    """The product with a gradient for x (the packed weights are constants): grad_x = grad_y @ W^T on
+    the dequantised weight, which is what the reference's Triton back end offers for training on top
+    of quantised layers (auto_gptq/nn_modules/qlinear_triton.py:195-273), here with the HIP dequant
+    kernel and the library GEMM."""
+
+    @staticmethod
+    def forward(ctx, x2, layer):
+        ctx.layer = layer
+        return layer._product(x2)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        w = ctx.layer.dequantize()                                   # [K, N] fp16
+        return torch.matmul(grad_out.to(w.dtype), w.t()), None
+
+
 class QuantLinear(nn.Module):
-    SUPPORTED_BITS = (3, 4)
+    SUPPORTED_BITS = (2, 3, 4, 8)   # the widths of the format (qlinear.py:31-32)
+    FUSED_BITS = (3, 4)             # those the fused kernels cover; 2 and 8 run as dequant + library GEMM
 
     def __init__(self, bits, groupsize, infeatures, outfeatures, bias, kernel_switch_threshold=1024,
                  sort_for_decode=True):
         super().__init__()
         if bits not in self.SUPPORTED_BITS:
-            # the reference accepts 2, 3, 4, 8 (qlinear.py:31-32); this path implements 3 and 4
-            raise NotImplementedError("Only 3,4 bits are supported.")
+            raise NotImplementedError("Only 2,3,4,8 bits are supported.")
         if infeatures % 32 != 0 or outfeatures % 32 != 0:
             raise ValueError("infeatures and outfeatures must be multiples of 32")
         self.infeatures = infeatures
@@ -143,7 +160,17 @@ class QuantLinear(nn.Module):
             x2 = x2.half()
         if not x2.is_contiguous():
             x2 = x2.contiguous()
+        if x2.requires_grad and torch.is_grad_enabled():
+            out = _ProductWithInputGrad.apply(x2, self)   # e.g. adapters trained on top of frozen layers
+        else:
+            out = self._product(x2)
+        return out.reshape(out_shape)
+
+    def _product(self, x2: torch.Tensor) -> torch.Tensor:
+        """y[M, N] = x2[M, K] @ W + bias for a contiguous fp16 x2."""
         try:
+            if self.bits not in self.FUSED_BITS:
+                raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, "width without a fused kernel")
             if self.kernel_switch_threshold and x2.shape[0] >= self.kernel_switch_threshold:
                 raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, "above kernel_switch_threshold")
             out = self._decode_sorted(x2) if (self.sort_for_decode and 0 < x2.shape[0] <= ops.SORTED_MAX_ROWS) else None
@@ -153,14 +180,14 @@ class QuantLinear(nn.Module):
         except _lib.GptqHipError as e:
             if e.status != _lib.ERR_UNSUPPORTED:
                 raise
-            # Long prompts (kernel_switch_threshold), or a shape the fused kernels do not cover
-            # (activation order with more groups than their LDS table holds): materialise W with
+            # Long prompts (kernel_switch_threshold), 2- and 8-bit layers, or a shape the fused kernels do
+            # not cover (activation order with more groups than their LDS table holds): materialise W with
             # the HIP dequant kernel and multiply with the library GEMM, which is what the reference
             # does above its threshold (auto_gptq/nn_modules/qlinear.py:198-245).  Still GPU only.
             out = torch.matmul(x2, self.dequantize())
             if self.bias is not None:
                 out = out + self.bias
-        return out.reshape(out_shape)
+        return out
 
     def dequantize(self) -> torch.Tensor:
         """fp16 [infeatures, outfeatures], the weight the reference materialises on every call."""

@@ -134,7 +134,9 @@ size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits, int group_
 
 /*
  * W fp16 [K, N] = scales[g] * (q - (zq[g] + 1)), one rounding per element:
- * the materialised weight of qlinear.py:198-242, for the bit-exact check.
+ * the materialised weight of qlinear.py:198-242, for the bit-exact check.  bits may also be 2 or 8
+ * here (the other widths of the format, qlinear.py:31-32,211-215): those layers run as this kernel
+ * followed by a library GEMM.
  */
 int gptq_hip_dequant(const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *g_idx,
                      void *w, int K, int N, int bits, int group_size, void *stream);

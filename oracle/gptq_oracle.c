@@ -114,11 +114,14 @@ static void unpack3_block(int32_t w0, int32_t w1, int32_t w2, int32_t out[32])
 /* qweight int32 [K/32*bits, N] -> codes int32 [K, N] */
 int oracle_unpack_rows(const int32_t *qweight, int K, int N, int bits, int32_t *codes)
 {
-    if (bits == 4) {
-        for (int r = 0; r < K / 8; r++) {
-            for (int j = 0; j < 8; j++) {
+    if (bits == 2 || bits == 4 || bits == 8) {
+        /* 32 / bits codes per word, code j at bit bits * j (qlinear.py:211-215) */
+        const int per = 32 / bits;
+        const int32_t mask = (1 << bits) - 1;
+        for (int r = 0; r < K / per; r++) {
+            for (int j = 0; j < per; j++) {
                 for (int n = 0; n < N; n++) {
-                    codes[(size_t)(8 * r + j) * N + n] = (qweight[(size_t)r * N + n] >> (4 * j)) & 0xf;
+                    codes[(size_t)(per * r + j) * N + n] = (qweight[(size_t)r * N + n] >> (bits * j)) & mask;
                 }
             }
         }
@@ -144,10 +147,12 @@ int oracle_unpack_rows(const int32_t *qweight, int K, int N, int bits, int32_t *
 int oracle_unpack_zeros(const int32_t *qzeros, int G, int N, int bits, int32_t *zeros)
 {
     const int words = N / 32 * bits;
-    if (bits == 4) {
+    if (bits == 2 || bits == 4 || bits == 8) {
+        const int per = 32 / bits;
+        const int32_t mask = (1 << bits) - 1;
         for (int g = 0; g < G; g++) {
             for (int n = 0; n < N; n++) {
-                zeros[(size_t)g * N + n] = ((qzeros[(size_t)g * words + n / 8] >> (4 * (n % 8))) & 0xf) + 1;
+                zeros[(size_t)g * N + n] = ((qzeros[(size_t)g * words + n / per] >> (bits * (n % per))) & mask) + 1;
             }
         }
         return 0;
@@ -189,7 +194,7 @@ int oracle_dequant(const int32_t *qweight, const int32_t *qzeros, const uint16_t
                 break;
             }
             for (int n = 0; n < N; n++) {
-                /* scale (11 significant bits) times an integer of magnitude <= 16 is exact in
+                /* scale (11 significant bits) times an integer of magnitude <= 256 is exact in
                  * float, so one rounding to half equals the reference's fp16 multiply */
                 const float s = half_to_float(scales[(size_t)g * N + n]);
                 const float d = (float)(codes[(size_t)k * N + n] - zeros[(size_t)g * N + n]);

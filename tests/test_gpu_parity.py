@@ -270,6 +270,57 @@ def test_gemm_linearity_at_full_size(dev):
 
 
 # ------------------------------------------------------------------ the module
+# ------------------------------------------------------------------ the other widths of the format: 2 and 8 bits
+@pytest.mark.parametrize("bits", [2, 8])
+@pytest.mark.parametrize("desc_act", [False, True])
+@pytest.mark.parametrize("shape", [(64, 32, 32), (256, 96, 64), (4096, 256, 128), (1024, 160, -1)])
+def test_dequant_bit_exact_two_and_eight_bits(dev, bits, desc_act, shape):
+    K, N, gs = shape
+    L = layer(120 + bits, K, N, bits, gs, desc_act)
+    D = to_dev(L, dev)
+    w = ops.dequant(D["qweight"], D["qzeros"], D["scales"], D["g_idx"] if desc_act else None, bits, gs).cpu()
+    assert torch.equal(w.view(torch.int16), expected_weight(L).view(torch.int16))
+
+
+@pytest.mark.parametrize("bits", [2, 8])
+@pytest.mark.parametrize("M", [1, 7])
+def test_module_runs_two_and_eight_bit_layers_as_dequant_plus_gemm(dev, bits, M):
+    K, N, gs = 512, 256, 128
+    L = layer(130 + bits, K, N, bits, gs, True, M=M, bias=True)
+    q = QuantLinear(bits, gs, K, N, True)
+    q.load_state_dict({k: L[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})
+    q = q.to(dev)
+    y = q(L["x"].to(dev))
+    assert y.shape == (M, N) and y.dtype == torch.float16
+    assert_close(y, expected_output(L), f"module forward, {bits} bits")
+    assert torch.equal(q.dequantize().cpu().view(torch.int16), expected_weight(L).view(torch.int16))
+    # the fused entry points do not take these widths
+    with pytest.raises(NotImplementedError):
+        run_gemm(to_dev(L, dev))
+
+
+@pytest.mark.parametrize("bits", [3, 4, 8])
+@pytest.mark.parametrize("M", [1, 9])
+def test_module_gives_a_gradient_for_its_input(dev, bits, M):
+    # grad_x = grad_y @ W^T (qlinear_triton.py:195-273), against the oracle's dequantised weight
+    K, N, gs = 512, 256, 128
+    L = layer(140 + bits, K, N, bits, gs, True, M=M, bias=True)
+    q = QuantLinear(bits, gs, K, N, True)
+    q.load_state_dict({k: L[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})
+    q = q.to(dev)
+    x = L["x"].to(dev).requires_grad_(True)
+    y = q(x)
+    assert y.requires_grad
+    assert_close(y, expected_output(L), "forward under autograd")
+    gy = torch.randn(M, N, generator=torch.Generator().manual_seed(9)).half()
+    y.backward(gy.to(dev))
+    want = gy.float() @ expected_weight(L).float().t()
+    assert x.grad is not None and x.grad.shape == (M, K)
+    assert_close(x.grad, want, "input gradient", rtol=1e-2, atol=2e-2)
+    with torch.no_grad():
+        assert not q(x).requires_grad
+
+
 # ------------------------------------------------------------------ activation order, channels sorted at load time
 def run_sorted(D, plan=None):
     qs, kmap = pack.sort_channels_by_group(D["qweight"], D["g_idx"], D["bits"], D["group_size"])

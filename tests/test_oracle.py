@@ -50,8 +50,20 @@ def test_int3_straddling_codes_known_words():
     assert packed[:, 0].tolist() == [1, 2, 4]
 
 
+def test_known_words_two_and_eight_bits():
+    # 8 bits: word 0x04030201 holds codes 1, 2, 3, 4; 2 bits: 0xE4 = 0b11100100 holds 0, 1, 2, 3
+    w8 = np.array([[0x04030201], [0x7FFFFF80 - (1 << 32) + (1 << 31)]], dtype=np.int64).astype(np.int32)
+    got = orc.unpack_bitstream(w8, 8, axis=0)[:, 0].tolist()
+    assert got[:4] == [1, 2, 3, 4] and got[4:] == [0x80, 0xFF, 0xFF, 0xFF]
+    w2 = np.array([[0xE4], [-1]], dtype=np.int32)
+    got = orc.unpack_bitstream(w2, 2, axis=0)[:, 0].tolist()
+    assert got[:4] == [0, 1, 2, 3] and got[4:16] == [0] * 12 and got[16:] == [3] * 16
+    assert np.array_equal(orc.unpack_qweight_ref(torch.from_numpy(w8), 8).numpy()[:, 0], orc.unpack_bitstream(w8, 8)[:, 0])
+    assert np.array_equal(orc.unpack_qweight_ref(torch.from_numpy(w2), 2).numpy()[:, 0], orc.unpack_bitstream(w2, 2)[:, 0])
+
+
 def test_zero_point_plus_one_known():
-    for bits in (3, 4):
+    for bits in (2, 3, 4, 8):
         n = 64
         qz = np.zeros((2, n // 32 * bits), dtype=np.int32)
         assert (orc.unpack_qzeros_ref(torch.from_numpy(qz), bits, n).numpy() == 1).all()
@@ -60,7 +72,7 @@ def test_zero_point_plus_one_known():
 
 
 # ---------------------------------------------------------------- three statements agree
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 def test_unpack_statements_agree_on_random_words(bits, c_oracle):
     rng = np.random.default_rng(10 + bits)
     qw = rand_words(rng, (bits * 6, 40))  # 6 blocks of 32 channels, arbitrary bit patterns
@@ -73,7 +85,7 @@ def test_unpack_statements_agree_on_random_words(bits, c_oracle):
     assert a.min() >= 0 and a.max() < (1 << bits)
 
 
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 def test_unpack_zeros_statements_agree(bits, c_oracle):
     rng = np.random.default_rng(20 + bits)
     n = 96
@@ -85,7 +97,7 @@ def test_unpack_zeros_statements_agree(bits, c_oracle):
     assert np.array_equal(a, c)
 
 
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 def test_pack_unpack_round_trip(bits):
     rng = np.random.default_rng(30 + bits)
     codes = rng.integers(0, 1 << bits, size=(96, 7))
@@ -116,7 +128,7 @@ def _layer(bits, K, N, gs, desc_act, seed):
     return synth_layer(seed, K, N, bits, gs, desc_act, M=3)
 
 
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 @pytest.mark.parametrize("desc_act", [False, True])
 def test_dequant_statements_agree(bits, desc_act, c_oracle):
     L = _layer(bits, 128, 64, 32, desc_act, 40 + bits)
@@ -134,7 +146,7 @@ def test_dequant_statements_agree(bits, desc_act, c_oracle):
         assert a[k, n] == want
 
 
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 def test_dequant_unit_scale_is_integer_exact(bits):
     L = _layer(bits, 64, 32, -1, False, 50 + bits)
     ones = torch.ones_like(L["scales"])
@@ -146,7 +158,7 @@ def test_fp16_multiply_equals_fp32_product_rounded_once(c_oracle):
     # the claim the kernels and the C oracle rely on, over all scale bit patterns that are finite
     s_bits = np.arange(0, 0x7C00, 7, dtype=np.uint16)
     s = torch.from_numpy(s_bits.view(np.float16).copy())
-    for d in range(-16, 16):
+    for d in list(range(-16, 16)) + [-256, -255, -129, -100, 97, 127, 200, 254]:   # 8-bit layers reach +-256
         torch_prod = (s * torch.tensor(d, dtype=torch.int32)).numpy()  # fp16 tensor * int tensor -> fp16
         restated = (s.numpy().astype(np.float32) * np.float32(d)).astype(np.float16)
         assert np.array_equal(torch_prod.view(np.uint16), restated.view(np.uint16)), d

@@ -28,7 +28,7 @@ def test_pack_rejects_bad_input():
     with pytest.raises(ValueError):
         pack.pack_qweight(np.zeros((33, 4), dtype=np.int64), 4)
     with pytest.raises(NotImplementedError):
-        pack.pack_qweight(np.zeros((32, 4), dtype=np.int64), 2)
+        pack.pack_qweight(np.zeros((32, 4), dtype=np.int64), 5)
     with pytest.raises(ValueError):
         pack.pack_qzeros(np.zeros((1, 32), dtype=np.int64), 4)  # zero point 0 is not storable
 

@@ -22,7 +22,7 @@ def test_buffers_follow_the_reference_layout():
     assert set(q.state_dict()) == {"qweight", "qzeros", "scales", "g_idx"}
 
 
-@pytest.mark.parametrize("bits", [2, 5, 8, 16])
+@pytest.mark.parametrize("bits", [1, 5, 16])
 def test_unsupported_bits_raise(bits):
     with pytest.raises(NotImplementedError):
         QuantLinear(bits, 128, 256, 256, False)
