@@ -324,7 +324,14 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     // K = 11008 79 / 93 against 20.1 / 16.8).
     // With the lean operand (int3, contiguous groups) two rows also win when K is split (4096 x 4096
     // 9.0 against 9.2 us, 11008 x 4096 12.0 against 13.1).
-    if (M <= 2 && !one_big_group && plan_grouped(M, K, N, bits, gs, G, act_order, 0, 0, plan) &&
+    // 257..512 column tiles would run as one full round of workgroups and a partial one: 128 columns
+    // per workgroup (two waves along N, four along K) keep it to one (4096 x 22016, gate and up as one
+    // product: int3 14.4 -> 12.4 us, int4 17.7 -> 13.9).
+    const int tiles64 = ceil_div(N, 64);
+    const int wide = (tiles64 > 256 && tiles64 <= 512) ? 2 : 0;
+    if (M <= 2 && !one_big_group &&
+        ((wide && plan_grouped(M, K, N, bits, gs, G, act_order, 0, wide, plan)) ||
+         plan_grouped(M, K, N, bits, gs, G, act_order, 0, 0, plan)) &&
         (M == 1 || plan->split_k == 1 || gptq::grouped_lite(bits, K, gs, act_order != 0, plan->row_tiles / M)) &&
         (!act_order || plan->row_tiles / M <= 3))
         return GPTQ_HIP_OK;

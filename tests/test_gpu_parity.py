@@ -193,6 +193,26 @@ def test_grouped_forced_split_k(dev, bits, desc_act, M, split):
 
 
 @pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("desc_act", [False, True])
+@pytest.mark.parametrize("M", [1, 2])
+def test_grouped_wide_workgroups(dev, bits, desc_act, M):
+    # 257..512 column tiles: the dispatcher gives a workgroup 128 columns (two waves along N)
+    K, N, gs = 512, 16480, 128
+    L = layer(650 + bits + M, K, N, bits, gs, desc_act, M=M, bias=True)
+    D = to_dev(L, dev)
+    plan = _lib.select(M, K, N, bits, gs, desc_act)
+    if plan.kernel == _lib.KERNEL_GROUPED:
+        assert plan.waves_n == 2 and plan.grid_x == (N + 127) // 128
+    y = run_gemm(D)
+    assert_close(y, expected_output(L), "wide workgroups")
+    assert_tight(y, expected_output(L), "wide workgroups")
+    if desc_act and ops.sorted_plan(M, K, N, bits, gs) is not None:
+        ys = run_sorted(D)
+        assert_close(ys, expected_output(L), "wide workgroups, sorted")
+        assert_tight(ys, expected_output(L), "wide workgroups, sorted")
+
+
+@pytest.mark.parametrize("bits", [3, 4])
 @pytest.mark.parametrize("K,N,gs", [(96, 32, 32), (1024, 416, 32), (2048, 1056, 256), (11008, 256, 128), (4096, 64, 64)])
 @pytest.mark.parametrize("M", [1, 2])
 def test_grouped_matches_gather(dev, bits, K, N, gs, M):
