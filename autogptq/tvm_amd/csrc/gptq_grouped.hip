@@ -118,39 +118,31 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     const int scan_base = kmap ? 0 : k_base;     // a sorted layer's channels may sit anywhere in x
     const int qpr = (kmap ? p.K : kspan) / 4;    // quads per activation row
     const int nquads = qpr * M;
+    // Every load below is unconditional (clamped addresses, results masked where they are used): a
+    // load inside a branch makes the number of loads in flight unknown at the next wait, and the
+    // compiler then waits for all of them (vmcnt(0)), which serialises x, map and weight latencies.
+    // A layer without a map still loads "map" entries (from the packed weights: any readable memory)
+    // and ignores them.
     int gq[QP][4];
     h4 xq[QP];
-    int4 sq[QP];  // xsrc: the channels of x this thread's positions take
+    int4 sq[QP];   // raw map entries (xsrc: the channels of x this thread's positions take)
+    bool qv[QP];   // the quad lies inside the rows and channels walked
+    const int32_t *mapsrc = xsrc ? xsrc : (kmap ? kmap : (p.g_idx ? p.g_idx : (const int32_t *)p.qweight));
+    const bool has_map = kmap != nullptr || p.g_idx != nullptr;
 #pragma unroll
     for (int ps = 0; ps < QP; ps++) {
         const int idx = tid + ps * nthreads;
-        xq[ps] = (h4){0, 0, 0, 0};
-        sq[ps] = make_int4(0, 0, 0, 0);
+        const int idc = min(idx, nquads - 1);
+        const int m = M == 1 ? 0 : idc / qpr;
+        const int k = scan_base + 4 * (idc - m * qpr);
+        qv[ps] = idx < nquads && k < p.K;  // K % 4 == 0: a quad is inside or outside as a whole
+        const int kl = min(k, p.K - 4);
+        xq[ps] = *(const h4 *)(x + (size_t)m * p.K + kl);
+        sq[ps] = *(const int4 *)(mapsrc + kl);
+        // groups of a layer without a map; the choice between these and the loaded entries is made
+        // where they are used, so that nothing here waits for a load
 #pragma unroll
-        for (int e = 0; e < 4; e++) gq[ps][e] = 0;
-        if (idx < nquads) {
-            const int m = M == 1 ? 0 : idx / qpr;
-            const int k = scan_base + 4 * (idx - m * qpr);
-            if (k < p.K) {  // K % 4 == 0: a quad is inside or outside as a whole
-                if (xsrc) {
-                    sq[ps] = *(const int4 *)(xsrc + k);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) gq[ps][e] = (k + e) / p.group_size;
-                    continue;
-                }
-                xq[ps] = *(const h4 *)(x + (size_t)m * p.K + k);
-                if (p.g_idx || kmap) {
-                    const int4 gv = *(const int4 *)((kmap ? kmap : p.g_idx) + k);
-                    gq[ps][0] = gv.x;
-                    gq[ps][1] = gv.y;
-                    gq[ps][2] = gv.z;
-                    gq[ps][3] = gv.w;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) gq[ps][e] = (k + e) / p.group_size;
-                }
-            }
-        }
+        for (int e = 0; e < 4; e++) gq[ps][e] = (k + e) / p.group_size;
     }
 
     // ---- 2. zero the expanded activation operand in LDS while those loads fly ---------
@@ -170,12 +162,12 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         const bool ok = n_ok && st < we && prow < prows;
 #pragma unroll
         for (int wd = 0; wd < F::WORDS; wd++) {
-            w[s][wd] = (u4){0u, 0u, 0u, 0u};
-            if (ok) {
-                // 32-bit byte offset from a uniform base: one VALU op per load instead of 64-bit math
-                const uint32_t off = ((uint32_t)(prow * F::WORDS + wd) * (uint32_t)p.N + (uint32_t)n0) * 4u;
-                w[s][wd] = __builtin_nontemporal_load((const u4 *)((const char *)p.qweight + off));
-            }
+            // 32-bit byte offset from a uniform base: one VALU op per load instead of 64-bit math.
+            // Steps past the wave's range, rows past K and columns past N read the first words of
+            // qweight instead (one hot line): whatever they yield meets zeros of x, is skipped, or is
+            // never stored.
+            const uint32_t off = ok ? ((uint32_t)(prow * F::WORDS + wd) * (uint32_t)p.N + (uint32_t)n0) * 4u : 0u;
+            w[s][wd] = __builtin_nontemporal_load((const u4 *)((const char *)p.qweight + off));
         }
     };
 #pragma unroll
@@ -184,12 +176,9 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     if (xsrc) {  // the x values of this thread's positions, now that their source channels are known
 #pragma unroll
         for (int ps = 0; ps < QP; ps++) {
-            const int idx = tid + ps * nthreads;
-            const int m = M == 1 ? 0 : idx / qpr;
-            if (idx < nquads && k_base + 4 * (idx - m * qpr) < p.K) {
-                const _Float16 *xr = x + (size_t)m * p.K;
-                xq[ps] = (h4){xr[src_ok(sq[ps].x)], xr[src_ok(sq[ps].y)], xr[src_ok(sq[ps].z)], xr[src_ok(sq[ps].w)]};
-            }
+            const int idc = min(tid + ps * nthreads, nquads - 1);
+            const _Float16 *xr = x + (size_t)(M == 1 ? 0 : idc / qpr) * p.K;
+            xq[ps] = (h4){xr[src_ok(sq[ps].x)], xr[src_ok(sq[ps].y)], xr[src_ok(sq[ps].z)], xr[src_ok(sq[ps].w)]};
         }
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -251,18 +240,17 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
 #pragma unroll
     for (int ps = 0; ps < QP; ps++) {
         const int idx = tid + ps * nthreads;
-        if (idx < nquads) {
+        if (qv[ps]) {
             const int m = M == 1 ? 0 : idx / qpr;
             const int kc = 4 * (idx - m * qpr);
+            const int gm[4] = {sq[ps].x, sq[ps].y, sq[ps].z, sq[ps].w};
             if (kmap) {
-                if (kc < p.K) {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) scatter_mapped(m, gq[ps][e], xq[ps][e]);
-                }
-            } else if (k_base + kc < p.K) {
+                for (int e = 0; e < 4; e++) scatter_mapped(m, gm[e], xq[ps][e]);
+            } else {
                 const int gb = p.g_idx ? 0 : (k_base + (kc / wave_k) * wave_k) / p.group_size;
 #pragma unroll
-                for (int e = 0; e < 4; e++) scatter(m, kc + e, qslot[e], gq[ps][e], gb, xq[ps][e]);
+                for (int e = 0; e < 4; e++) scatter(m, kc + e, qslot[e], has_map ? gm[e] : gq[ps][e], gb, xq[ps][e]);
             }
         }
     }
@@ -355,11 +343,10 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         }
 #pragma unroll
         for (int s = 0; s < NSTEP; s++) {
-            if (s + PF < NSTEP) {
-                if (st0 + s + PF < we) load_step(s + PF, st0 + s + PF);
-            }
+            if (st0 + s >= we) break;  // a short range ends the chunk early (no load sits behind this branch)
+            if (s + PF < NSTEP) load_step(s + PF, st0 + s + PF);  // past the wave's range: one hot line
             __builtin_amdgcn_sched_barrier(0);
-            if (st0 + s < we) {
+            {
                 const int b = (st0 + s - s_begin) * 4 + lq;
                 u4 bq[4][F::NB];
 #pragma unroll
