@@ -51,6 +51,21 @@ struct InvTables {
 };
 static __constant__ InvTables kInv = InvTables();
 
+// The same tables as immediates, for a thread that owns codes 4 q .. 4 q + 3 of a lane block: byte q
+// of quad_slots<BITS>(e) is the slot of code 4 q + e.  A lookup in kInv is a load from constant memory
+// that nothing else in a kernel has touched yet: it costs a full memory latency at the top of the
+// kernel and sits first in the in-order return queue of every later load.
+template <int BITS>
+__device__ __forceinline__ constexpr uint64_t quad_slots(int e)
+{
+    constexpr InvTables t = InvTables();
+    uint64_t w = 0;
+    for (int q = 0; q < Fmt<BITS>::KLANE / 4; q++) {
+        w |= (uint64_t)(BITS == 4 ? t.inv4[4 * q + e] : t.inv3[4 * q + e]) << (8 * q);
+    }
+    return w;
+}
+
 // slot (position in the MFMA operand order) of code j of a lane block
 template <int BITS>
 __device__ __forceinline__ int slot_of_code(int j)

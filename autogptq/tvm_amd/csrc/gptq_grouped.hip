@@ -112,7 +112,11 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
 
     int qslot[4];
 #pragma unroll
-    for (int e = 0; e < 4; e++) qslot[e] = slot_of_code<BITS>((4 * tid) % F::KLANE + e);
+    for (int e = 0; e < 4; e++) {
+        constexpr uint64_t words[4] = {quad_slots<BITS>(0), quad_slots<BITS>(1), quad_slots<BITS>(2),
+                                       quad_slots<BITS>(3)};
+        qslot[e] = (int)((words[e] >> (8 * (tid % (F::KLANE / 4)))) & 0xffu);
+    }
     // ---- 1. x and g_idx of the K range: four channels per thread per pass ---------------
     constexpr int QP = 2;  // passes kept in registers so that their loads are the first to return
     const int scan_base = kmap ? 0 : k_base;     // a sorted layer's channels may sit anywhere in x
