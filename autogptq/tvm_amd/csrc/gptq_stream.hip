@@ -583,9 +583,22 @@ __global__ __launch_bounds__(512) void stream_direct_kernel(const Params p)
                 const uint32_t g = __umulhi(r, p.gdiv_magic) + (p.gdiv_add ? r : 0u);
                 erow = *(const u4 *)(smem + (g * TROW + (uint32_t)tab_bias));
             }
-            STREAM_PIN_LOADS();
+            // Nothing may cross these two points: with only the loads pinned the scheduler hoists the
+            // ring reads (and with them the waits) of all PF steps above the first refill, so every
+            // group of PF steps waits for its loads, computes, and only then requests the next group.
+            // (int3 under an activation order keeps the looser pin: with the order fixed it spills 41
+            // registers and runs 18 -> 25 us at M = 8.)
+            if constexpr (BITS == 3 && ACT) {
+                STREAM_PIN_LOADS();
+            } else {
+                __builtin_amdgcn_sched_barrier(0);
+            }
             load_step(st + PF, w[u], xr[u], gr[ACT ? u : 0]);
-            STREAM_PIN_LOADS();
+            if constexpr (BITS == 3 && ACT) {
+                STREAM_PIN_LOADS();
+            } else {
+                __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
             for (int nb = 0; nb < F::NB; nb++) {
                 uint32_t eoff[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
