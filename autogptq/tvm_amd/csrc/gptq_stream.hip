@@ -406,9 +406,9 @@ __global__ __launch_bounds__(512) void stream_kernel(const Params p)
             u4 erow = {0u, 0u, 0u, 0u};
             if constexpr (!ACT) erow = *(const u4 *)(smem + (uint32_t)(grow[u] + tab_bias));
             if constexpr (BITS == 4) {
-                STREAM_PIN_LOADS();
+                __builtin_amdgcn_sched_barrier(0);
                 load_w(st + PF, w[u], grow[u]);  // refill this ring slot
-                STREAM_PIN_LOADS();
+                __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
             for (int nb = 0; nb < F::NB; nb++) {
@@ -446,7 +446,7 @@ __global__ __launch_bounds__(512) void stream_kernel(const Params p)
                     }
                     a[slot][rt] = load_a(b + AD, rt);  // refill: this tile of the block AD ahead
                 }
-                STREAM_PIN_LOADS();
+                __builtin_amdgcn_sched_barrier(0);
             }
             if constexpr (BITS == 3) {
                 load_w(st + PF, w[u], grow[u]);  // refill this ring slot (its words were needed until here)
