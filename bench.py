@@ -80,8 +80,8 @@ DEFAULT_WORKLOAD = "c2-int3-4096x11008-act-m1"
 # same counter reads for a plain 256 MiB device copy); a profiler run is needed to refresh them, so
 # they are recorded here per workload.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "c2-int3-4096x11008-act-m1": 18_393 * 1024 + 22_016,        # GROUPED kernel (prepared path): read + written
-    "c4-int4-4096x11008-act-m128": (56_370 + 2_752) * 1024,     # STREAM matmul kernel alone (pack pass: 3,154 KiB more)
+    "c2-int3-4096x11008-act-m1": 18_354 * 1024 + 22_016,        # GROUPED kernel (prepared path): read + written
+    "c4-int4-4096x11008-act-m128": (56_364 + 2_752) * 1024,     # STREAM matmul kernel alone (pack pass: 3,154 KiB more)
 }
 
 
