@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the GPTQ QuantLinear hot path on one MI355X.
 
-Default workload: BASELINE.json configs[1] -- 3-bit GEMV, M=1, K=4096, N=11008, group_size=128,
+Default workload: the headline configuration of the reference's benchmarks -- 3-bit GEMV, M=1, K=4096, N=11008, group_size=128,
 desc_act=True (g_idx from a random permutation), synthetic seeded tensors.  One "step" is one
 call of the C-ABI entry point that ``QuantLinear.forward`` makes for that shape, on tensors already
 resident in HBM: ``gptq_hip_gemm_sorted`` for decode sizes on activation-order layers (the layer

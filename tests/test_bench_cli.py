@@ -28,7 +28,7 @@ def test_workload_table_covers_the_baseline_configurations():
     names = set(bench.WORKLOADS)
     assert bench.DEFAULT_WORKLOAD in names
     bits, K, N, gs, act, M = bench.WORKLOADS[bench.DEFAULT_WORKLOAD]
-    assert (bits, K, N, gs, act, M) == (3, 4096, 11008, 128, True, 1)      # BASELINE configs[1]
+    assert (bits, K, N, gs, act, M) == (3, 4096, 11008, 128, True, 1)      # the headline configuration
     assert bench.WORKLOADS["c1-int4-4096x4096-m1"] == (4, 4096, 4096, 128, False, 1)  # configs[0]
     assert any(v[5] == 128 and v[4] for v in bench.WORKLOADS.values())     # act-order GEMM at M = 128
     assert any(v[3] == -1 and v[1] == 36864 for v in bench.WORKLOADS.values())  # OPT-66B long K
