@@ -517,3 +517,40 @@ def test_bad_g_idx_is_rejected_by_the_module(dev):
     q.g_idx[3] = 99
     with pytest.raises(ValueError, match="g_idx"):
         q(torch.zeros(1, 64, device=dev))
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_module_forward_replays_in_a_graph(dev, bits):
+    """Decoding loops replay a captured graph: the module's calls (sorted decode, small batch behind the
+    reorder pass, pack pass + matmul + reduce pass) must give the eager result on every replay, with the
+    program's own eager work between replays."""
+    K, N, gs = 2048, 4096, 128
+    L = layer(970 + bits, K, N, bits, gs, True, M=40, bias=True)
+    q = QuantLinear(bits, gs, K, N, True)
+    q.load_state_dict({k: L[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})
+    q = q.to(dev)
+    gen = torch.Generator().manual_seed(12)
+    xs = {M: torch.randn(M, K, generator=gen).half().to(dev) for M in (1, 8, 40)}
+    for M in xs:          # eager first: workspaces and the sorted copy are allocated outside the capture
+        q(xs[M])
+    torch.cuda.synchronize(dev)
+    stream = torch.cuda.Stream(device=dev)
+    graph = torch.cuda.CUDAGraph()
+    outs = {}
+    with torch.cuda.stream(stream):
+        for M in xs:
+            q(xs[M])      # the side stream gets its own workspace here, before the capture
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            for M in xs:
+                outs[M] = q(xs[M])
+    for rep in range(3):
+        for M in xs:      # new inputs in place, eager reference computed between the replays
+            xs[M].copy_(torch.randn(M, K, generator=gen).half())
+        want = {M: q(xs[M]).clone() for M in xs}
+        torch.cuda.synchronize(dev)
+        graph.replay()
+        torch.cuda.synchronize(dev)
+        for M in xs:
+            assert torch.equal(outs[M], want[M]), (rep, M)
+            assert_close(outs[M], expected_output(L, x=xs[M].cpu()), f"graph replay {rep}, M={M}")
