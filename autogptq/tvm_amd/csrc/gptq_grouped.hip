@@ -13,9 +13,9 @@
 // from the reference by its rounding noise, far inside the 1e-2 tolerance.
 //
 // Work split: a workgroup owns 64 * waves_n columns and one K range (all of K when
-// split_k == 1); its waves_k waves along K each take a share of that range, issue all
-// their weight loads up front, and meet in LDS for the reduction.  With split_k == 1
-// nothing crosses workgroups.
+// split_k == 1); its waves_k waves along K each take a share of that range, keep their
+// weight loads one (int3) or eight (int4) steps ahead of the matrix instructions, and meet
+// in LDS for the reduction.  With split_k == 1 nothing crosses workgroups.
 //
 // LDS holds the expanded activation operand of the workgroup's K range, laid out as
 // the MFMA wants it: a tile is 16 rows x 8 slots of fp16 = 256 bytes, lane i reads its
@@ -30,16 +30,17 @@
 // LITE: with contiguous groups that are whole lane blocks (8 channels int4, 32 int3) all 8 slots
 // of an operand tile belong to one group, so the tile is "x in row r, zeros elsewhere".  LDS then
 // holds just x in unpack order (2 bytes per channel instead of 32) plus 16 zero bytes: a lane reads
-// x when its row is the block's group and the zeros otherwise.  No zero fill, and the scatter is
-// one 2-byte store per channel to spread addresses instead of one bank.
+// x when its row is the block's group and the zeros otherwise.  Only x itself is zero-filled (8 KB
+// instead of 128 KB at K = 4096), and the scatter's 2-byte stores spread over the banks instead of
+// hitting the two banks of one tile row.  Used for int3 (see launch_grouped_one).
 //
 // Sorted layers: when the loader has sorted the channels of an activation-order layer by
 // group (qweight rows permuted, p.kmap saying where each original channel went), the groups
 // are contiguous for the weight stream and only the scatter of x follows the map: every
 // workgroup walks all of x and keeps the channels whose sorted position falls in its K range
-// (p.kmap, when one workgroup holds all of K), or looks up where the x of each of its positions
-// comes from (p.xsrc, when K is split: a walk over all of x would cost every workgroup the whole
-// scatter for a fraction of the channels).
+// (p.kmap: one memory round trip), or looks up where the x of each of its positions comes from
+// (p.xsrc: two dependent round trips, but no scatter work on channels of other K ranges; the
+// host picks it when K is split and long).
 #include "gptq_device.h"
 
 namespace gptq {
@@ -188,7 +189,8 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     }
 
     // ---- 4. scales / zero words this lane needs in the epilogue (rows g = 16 t + 4 q + v);
-    //         loaded once the last weight loads are out ---------------------------------
+    //         requested behind the scatter of x: ahead of it they delay x and the first weights
+    //         (measured 7.4 -> 7.7 us at int3 4096 x 11008) ---------------------------------
     h4 sc[TPM][4];
     uint32_t zwa[TPM][4], zwb[TPM][4];
     // Rows past the last group and lanes past the last column load clamped addresses: their
