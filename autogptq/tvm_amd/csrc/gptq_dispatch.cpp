@@ -314,27 +314,44 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     // one group for the whole matrix: g_idx carries no information
     if (G == 1) act_order = 0;
     // GROUPED for decoding (M = 1); for M = 2 only where a workgroup holds all of K, since its
-    // operand in LDS doubles with M and the cross-workgroup sum costs more than STREAM's pack pass
-    // A single group over a large matrix gains nothing from GROUPED's expansion by group: STREAM's
-    // one table entry per lane block is cheaper there.
-    const bool one_big_group = G == 1 && (long long)K * N >= (1LL << 27);
+    // operand in LDS doubles with M and the cross-workgroup sum costs more than STREAM's pack pass.
+    // With the lean operand (int3, contiguous groups) two rows also win when K is split (4096 x 4096
+    // 9.0 against 9.2 us, 11008 x 4096 12.0 against 13.1).
     // Under an activation order every group a workgroup meets needs a row: past three row tiles
     // (48 groups) the expansion costs more than STREAM's lookup per weight (measured at N = 4096,
     // int3 / int4: K = 5120 16.1 / 11.6 us against 19.1 / 12.8; K = 8192 19.8 / 22.1 against 15.3 / 13.7;
     // K = 11008 79 / 93 against 20.1 / 16.8).
-    // With the lean operand (int3, contiguous groups) two rows also win when K is split (4096 x 4096
-    // 9.0 against 9.2 us, 11008 x 4096 12.0 against 13.1).
-    // 257..512 column tiles would run as one full round of workgroups and a partial one: 128 columns
-    // per workgroup (two waves along N, four along K) keep it to one (4096 x 22016, gate and up as one
-    // product: int3 14.4 -> 12.4 us, int4 17.7 -> 13.9).
+    // Many column tiles: every workgroup stages x for itself, and past 256 workgroups they run in
+    // rounds, so a workgroup takes 128 columns (257..512 tiles) or 256 (more) when that does not
+    // force a finer split of K (4096 x 22016: int3 14.4 -> 12.4 us, int4 17.7 -> 13.9; 9216 x 36864:
+    // int3 35.9 -> 32.8, int4 55.4 -> 33.9; int4 8192 x 28672 35.6 -> 26.8, while int3 there keeps
+    // 64 columns: 22.7 against 26.1 with K split in two).
+    // A split into eight or more K ranges leaves the sum to a long tail of workgroups: STREAM's own
+    // pass is cheaper then (int4 36864 x 9216: 52.6 us in nine ranges against 42.1).
     const int tiles64 = ceil_div(N, 64);
-    const int wide = (tiles64 > 256 && tiles64 <= 512) ? 2 : 0;
-    if (M <= 2 && !one_big_group &&
-        ((wide && plan_grouped(M, K, N, bits, gs, G, act_order, 0, wide, plan)) ||
-         plan_grouped(M, K, N, bits, gs, G, act_order, 0, 0, plan)) &&
-        (M == 1 || plan->split_k == 1 || gptq::grouped_lite(bits, K, gs, act_order != 0, plan->row_tiles / M)) &&
-        (!act_order || plan->row_tiles / M <= 3))
+    const int wide = tiles64 > 512 ? 4 : (tiles64 > 256 ? 2 : 0);
+    bool grouped = false;
+    if (M <= 2) {
+        gptq_hip_plan narrow;
+        memset(&narrow, 0, sizeof(narrow));
+        const bool have_narrow = plan_grouped(M, K, N, bits, gs, G, act_order, 0, 0, &narrow);
+        const bool have_wide = wide && plan_grouped(M, K, N, bits, gs, G, act_order, 0, wide, plan);
+        if (have_wide && (!have_narrow || plan->split_k <= narrow.split_k)) {
+            grouped = true;
+        } else if (have_narrow) {
+            *plan = narrow;
+            grouped = true;
+        }
+    }
+    if (grouped && (M == 1 || plan->split_k == 1 || gptq::grouped_lite(bits, K, gs, act_order != 0, plan->row_tiles / M)) &&
+        (!act_order || plan->row_tiles / M <= 3)) {
+        if (plan->split_k < 8) return GPTQ_HIP_OK;
+        gptq_hip_plan alt;
+        memset(&alt, 0, sizeof(alt));
+        if (plan_stream(M, K, N, bits, gs, G, act_order, 0, 0, &alt) != GPTQ_HIP_OK) return GPTQ_HIP_OK;
+        *plan = alt;
         return GPTQ_HIP_OK;
+    }
     memset(plan, 0, sizeof(*plan));
     if (plan_stream(M, K, N, bits, gs, G, act_order, 0, 0, plan) == GPTQ_HIP_OK) return GPTQ_HIP_OK;
     memset(plan, 0, sizeof(*plan));

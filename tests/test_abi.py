@@ -191,8 +191,15 @@ def test_dispatcher_families_by_m():
     assert _lib.select(1, 11008, 4096, 4, 128, True).kernel == _lib.KERNEL_STREAM
     assert _lib.select(1, 5120, 4096, 3, 128, True).kernel == _lib.KERNEL_GROUPED
     assert _lib.select(1, 11008, 4096, 4, 128, False).kernel == _lib.KERNEL_GROUPED
-    # one group over a large matrix streams better without the expansion by group
-    assert _lib.select(1, 9216, 36864, 3, -1, False).kernel == _lib.KERNEL_STREAM
+    # very wide layers: 256 columns per workgroup (four waves along N) keep the grid to one round
+    p = _lib.select(1, 9216, 36864, 3, -1, False)
+    assert p.kernel == _lib.KERNEL_GROUPED and p.waves_n == 4 and p.grid_x == 144 and p.split_k == 1
+    # a GROUPED plan that would cut K into eight or more ranges loses to STREAM's own pass
+    assert _lib.select(1, 36864, 9216, 4, -1, False).kernel == _lib.KERNEL_STREAM
+    assert _lib.select(1, 36864, 9216, 3, -1, False).kernel == _lib.KERNEL_GROUPED
+    # wide workgroups only where they do not force a finer split of K
+    assert _lib.select(1, 8192, 28672, 4, 128, False).waves_n == 2
+    assert _lib.select(1, 8192, 28672, 3, 128, False).waves_n == 1
     # forcing the STREAM family with waves along K and a split
     p = _lib.plan_for(_lib.KERNEL_STREAM, 40, 4096, 352, 3, 128, True, split_k=2, waves_n=8)
     assert p.kernel == _lib.KERNEL_STREAM and p.waves_k == 8 and p.waves_n == 1 and p.split_k == 2 and p.block == 512
