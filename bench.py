@@ -73,6 +73,10 @@ WORKLOADS = {
     "c5-int3-9216x36864-g1-m1": (3, 9216, 36864, -1, True, 1),
     "c5-int3-36864x9216-g1-m1": (3, 36864, 9216, -1, True, 1),
     "c5-int3-9216x36864-g1-m32": (3, 9216, 36864, -1, True, 32),
+    # larger layers, where the fixed cost of a launch weighs less
+    "int4-9216x36864-g1-m1": (4, 9216, 36864, -1, True, 1),
+    "int4-8192x28672-m1": (4, 8192, 28672, 128, False, 1),
+    "int3-8192x28672-act-m1": (3, 8192, 28672, 128, True, 1),
 }
 DEFAULT_WORKLOAD = "c2-int3-4096x11008-act-m1"
 
