@@ -195,14 +195,15 @@ def test_grouped_forced_split_k(dev, bits, desc_act, M, split):
 @pytest.mark.parametrize("bits", [3, 4])
 @pytest.mark.parametrize("desc_act", [False, True])
 @pytest.mark.parametrize("M", [1, 2])
-def test_grouped_wide_workgroups(dev, bits, desc_act, M):
-    # 257..512 column tiles: the dispatcher gives a workgroup 128 columns (two waves along N)
-    K, N, gs = 512, 16480, 128
+@pytest.mark.parametrize("N,wn", [(16480, 2), (32864, 4)])
+def test_grouped_wide_workgroups(dev, bits, desc_act, M, N, wn):
+    # 257..512 column tiles: the dispatcher gives a workgroup 128 columns (two waves along N); more: 256
+    K, gs = 512, 128
     L = layer(650 + bits + M, K, N, bits, gs, desc_act, M=M, bias=True)
     D = to_dev(L, dev)
     plan = _lib.select(M, K, N, bits, gs, desc_act)
     if plan.kernel == _lib.KERNEL_GROUPED:
-        assert plan.waves_n == 2 and plan.grid_x == (N + 127) // 128
+        assert plan.waves_n == wn and plan.grid_x == (N + 64 * wn - 1) // (64 * wn)
     y = run_gemm(D)
     assert_close(y, expected_output(L), "wide workgroups")
     assert_tight(y, expected_output(L), "wide workgroups")
