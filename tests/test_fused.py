@@ -135,8 +135,9 @@ def test_fused_model_matches_the_unfused_one(tmp_path):
 
     cfg, _, _ = build_checkpoint(str(tmp_path), bits=4, gs=32, act_order=True, seed=4, shared_order=True)
     plain, _ = from_quantized(str(tmp_path), device="cuda:0")
-    merged, _ = from_quantized(str(tmp_path), device="cuda:0", fuse_shared_inputs=True)
+    merged, _ = from_quantized(str(tmp_path), device="cuda:0", fuse_shared_inputs=True, prepare_decode=True)
     assert isinstance(merged.model.layers[0].self_attn.k_proj, fused.FusedMember)
+    assert merged.model.layers[0].mlp.down_proj._sorted is not None       # prepared at load
     ids = torch.randint(0, cfg.vocab_size, (2, 9), generator=torch.Generator().manual_seed(5)).to("cuda:0")
     with torch.no_grad():
         a = plain(ids).logits.float().cpu()
