@@ -85,6 +85,7 @@ DEFAULT_WORKLOAD = "c2-int3-4096x11008-act-m1"
 # they are recorded here per workload.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
     "c2-int3-4096x11008-act-m1": 18_354 * 1024 + 22_016,        # GROUPED kernel (prepared path): read + written
+    "int4-9216x36864-g1-m1": (167_123 + 954) * 1024,             # GROUPED kernel, 256-column workgroups
     "c4-int4-4096x11008-act-m128": (56_383 + 2_752) * 1024,     # STREAM matmul kernel alone (pack pass: 3,154 KiB more)
 }
 
