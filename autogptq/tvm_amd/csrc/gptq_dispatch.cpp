@@ -326,8 +326,10 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     // force a finer split of K (4096 x 22016: int3 14.4 -> 12.4 us, int4 17.7 -> 13.9; 9216 x 36864:
     // int3 35.9 -> 32.8, int4 55.4 -> 33.9; int4 8192 x 28672 35.6 -> 26.8, while int3 there keeps
     // 64 columns: 22.7 against 26.1 with K split in two).
-    // A split into eight or more K ranges leaves the sum to a long tail of workgroups: STREAM's own
-    // pass is cheaper then (int4 36864 x 9216: 52.6 us in nine ranges against 42.1).
+    // A split into many K ranges leaves the sum to a long tail of workgroups: from eight ranges on
+    // (int3: past eight) STREAM's own pass is cheaper (int4 36864 x 9216: 52.6 us in nine ranges
+    // against 42.1; 4096 x 512: 14.6 / 15.0 us in 32 ranges against 8.3 / 7.1; 4096 x 2048 in eight
+    // ranges: int3 8.0 against 8.5, int4 8.7 against 7.7).
     const int tiles64 = ceil_div(N, 64);
     const int wide = tiles64 > 512 ? 4 : (tiles64 > 256 ? 2 : 0);
     bool grouped = false;
@@ -345,7 +347,7 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     }
     if (grouped && (M == 1 || plan->split_k == 1 || gptq::grouped_lite(bits, K, gs, act_order != 0, plan->row_tiles / M)) &&
         (!act_order || plan->row_tiles / M <= 3)) {
-        if (plan->split_k < 8) return GPTQ_HIP_OK;
+        if (plan->split_k < (bits == 3 ? 9 : 8)) return GPTQ_HIP_OK;
         gptq_hip_plan alt;
         memset(&alt, 0, sizeof(alt));
         if (plan_stream(M, K, N, bits, gs, G, act_order, 0, 0, &alt) != GPTQ_HIP_OK) return GPTQ_HIP_OK;
