@@ -54,9 +54,12 @@ class QuantLinear(nn.Module):
         self.maxq = 2 ** self.bits - 1
         # Rows of x from which forward() materialises W (HIP dequant kernel) and calls the library
         # GEMM instead of the fused kernels, as the reference does (qlinear.py:25,198: default 128
-        # there).  Measured on MI355X at 4096x11008 int4: fused 95 us vs 116 us at 512 rows, 172 us
-        # vs 143 us at 1024 rows, hence 1024.  0 or None disables the switch.
+        # there).  Measured on MI355X at 4096x11008, fused against dequant + library GEMM: contiguous
+        # groups 124 vs 139 us at 768 rows, 152 vs 146 at 1024 (int4; int3 136 vs 146); activation
+        # order 126 vs 130 at 640 rows, 139 vs 133 at 768, 169 vs 142 at 1024.  Hence 1024, and 640 for
+        # layers with an activation order.  0 or None disables the switch.
         self.kernel_switch_threshold = kernel_switch_threshold
+        self.act_order_switch_threshold = 640
 
         groups = math.ceil(infeatures / self.groupsize)
         self.register_buffer("qweight", torch.zeros((infeatures // 32 * bits, outfeatures), dtype=torch.int32))
@@ -171,7 +174,10 @@ class QuantLinear(nn.Module):
         try:
             if self.bits not in self.FUSED_BITS:
                 raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, "width without a fused kernel")
-            if self.kernel_switch_threshold and x2.shape[0] >= self.kernel_switch_threshold:
+            threshold = self.kernel_switch_threshold
+            if threshold and self.act_order_switch_threshold and self._kernel_g_idx() is not None:
+                threshold = min(threshold, self.act_order_switch_threshold)
+            if threshold and x2.shape[0] >= threshold:
                 raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, "above kernel_switch_threshold")
             out = self._decode_sorted(x2) if (self.sort_for_decode and 0 < x2.shape[0] <= ops.SORTED_MAX_ROWS) else None
             if out is None:
