@@ -30,6 +30,7 @@ ABI_SYMBOLS = (
     "gptq_hip_gemm_plan",
     "gptq_hip_gemm_sorted",
     "gptq_hip_sorted_workspace_bytes",
+    "gptq_hip_sort_channels",
     "gptq_hip_dequant",
     "gptq_hip_strerror",
     "gptq_hip_abi_version",
@@ -96,6 +97,8 @@ def lib() -> ctypes.CDLL:
     l.gptq_hip_gemm_sorted.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
     l.gptq_hip_sorted_workspace_bytes.restype = sz
     l.gptq_hip_sorted_workspace_bytes.argtypes = [i, i, i, i, i]
+    l.gptq_hip_sort_channels.restype = i
+    l.gptq_hip_sort_channels.argtypes = [vp, vp, vp, vp, i, i, i, i, vp]
     l.gptq_hip_dequant.restype = i
     l.gptq_hip_dequant.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
     l.gptq_hip_strerror.restype = ctypes.c_char_p

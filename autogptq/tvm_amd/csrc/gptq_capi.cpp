@@ -261,6 +261,21 @@ extern "C" int gptq_hip_gemm_sorted(const void *x, const int32_t *qweight_sorted
                     bits, group_size, plan, stream);
 }
 
+extern "C" int gptq_hip_sort_channels(const int32_t *qweight, const int32_t *g_idx, int32_t *qweight_sorted,
+                                      int32_t *kmap, int K, int N, int bits, int group_size, void *stream)
+{
+    if (!qweight || !g_idx || !qweight_sorted || !kmap || qweight == qweight_sorted) return GPTQ_HIP_ERR_BAD_ARG;
+    if (bits != 3 && bits != 4) return GPTQ_HIP_ERR_BAD_ARG;
+    if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;
+    if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
+    if (!aligned(qweight, 16) || !aligned(qweight_sorted, 16) || !aligned(kmap, 16) || !aligned(g_idx, 4))
+        return GPTQ_HIP_ERR_BAD_ARG;
+    const int gs = group_size == -1 ? K : group_size;
+    if (K >= 65536 || K % gs != 0 || gs % (bits == 4 ? 8 : 32) != 0) return GPTQ_HIP_ERR_UNSUPPORTED;
+    return gptq::launch_sort_channels((const uint32_t *)qweight, g_idx, (uint32_t *)qweight_sorted, kmap, K, N, K / gs,
+                                      bits, gs, stream);
+}
+
 extern "C" size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits, int group_size)
 {
     gptq_hip_plan plan;

@@ -68,6 +68,84 @@ int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const void *
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 
+// ---------------------------------------------------------------------------------
+// Load-time channel sort of an activation-order layer (see gptq_hip_sort_channels).
+// Pass 1: channel k goes to sorted index g * group_size + (number of earlier channels of its
+// group): a stable sort by group without a sort.  Every thread counts over the g_idx entries
+// before its own, a tile at a time through LDS (K * K / 2 compares: a one-time cost of tens of
+// microseconds at K = 4096).  It writes both halves of the channel map.
+// ---------------------------------------------------------------------------------
+template <int BITS>
+__global__ __launch_bounds__(256) void sort_map_kernel(const int32_t *__restrict__ g_idx, int32_t *__restrict__ kmap,
+                                                       int K, int G, int group_size)
+{
+    __shared__ int tile[256];
+    constexpr int KLANE = Fmt<BITS>::KLANE;
+    const int k = blockIdx.x * 256 + threadIdx.x;
+    const int g = k < K ? min(max(g_idx[k], 0), G - 1) : -1;
+    int rank = 0;
+    for (int t0 = 0; t0 <= (int)blockIdx.x * 256; t0 += 256) {
+        const int j = t0 + threadIdx.x;
+        __syncthreads();
+        tile[threadIdx.x] = j < K ? min(max(g_idx[j], 0), G - 1) : -2;
+        __syncthreads();
+        const int upto = min(256, k - t0);  // entries of this tile that lie before k
+        for (int i = 0; i < upto; i++) rank += tile[i] == g ? 1 : 0;
+    }
+    if (k >= K) return;
+    // a group with more than group_size members would leave its range: keep every index in bounds
+    const int inv = g * group_size + min(rank, group_size - 1);
+    const int code = inv % KLANE;
+    const int slot = BITS == 4 ? (int)kInv.inv4[code] : (int)kInv.inv3[code];
+    kmap[k] = ((inv - code) + slot) | (g << 16);
+    kmap[K + inv] = k;
+}
+
+// Pass 2: qweight_sorted row j = qweight row kmap[K + j], 32 rows (one packed block) and one column per thread.
+template <int BITS>
+__global__ __launch_bounds__(256) void sort_repack_kernel(const uint32_t *__restrict__ qweight,
+                                                          const int32_t *__restrict__ kmap,
+                                                          uint32_t *__restrict__ out, int K, int N)
+{
+    const int n = blockIdx.x * 256 + threadIdx.x;
+    const int jb = blockIdx.y;
+    if (n >= N) return;
+    uint32_t words[BITS];
+#pragma unroll
+    for (int i = 0; i < BITS; i++) words[i] = 0u;
+    for (int i = 0; i < 32; i++) {
+        const int src = min(max(kmap[K + 32 * jb + i], 0), K - 1);
+        const uint32_t *blk = qweight + (size_t)(src >> 5) * BITS * N + n;  // the packed block of 32 channels
+        uint32_t q;
+        const int bit = BITS * (src & 31);
+        const int wd = bit >> 5, sh = bit & 31;
+        q = blk[(size_t)wd * N] >> sh;
+        if (sh + BITS > 32) q |= blk[(size_t)(wd + 1) * N] << (32 - sh);
+        q &= (1u << BITS) - 1u;
+        const int obit = BITS * i;
+        const int owd = obit >> 5, osh = obit & 31;
+        words[owd] |= q << osh;
+        if (osh + BITS > 32) words[owd + 1] |= q >> (32 - osh);
+    }
+#pragma unroll
+    for (int i = 0; i < BITS; i++) out[(size_t)(jb * BITS + i) * N + n] = words[i];
+}
+
+int launch_sort_channels(const uint32_t *qweight, const int32_t *g_idx, uint32_t *qweight_sorted, int32_t *kmap, int K,
+                         int N, int G, int bits, int group_size, void *stream_v)
+{
+    hipStream_t stream = (hipStream_t)stream_v;
+    const dim3 g1((K + 255) / 256), g2((N + 255) / 256, K / 32);
+    if (bits == 4) {
+        hipLaunchKernelGGL(sort_map_kernel<4>, g1, dim3(256), 0, stream, g_idx, kmap, K, G, group_size);
+        hipLaunchKernelGGL(sort_repack_kernel<4>, g2, dim3(256), 0, stream, qweight, kmap, qweight_sorted, K, N);
+    } else {
+        hipLaunchKernelGGL(sort_map_kernel<3>, g1, dim3(256), 0, stream, g_idx, kmap, K, G, group_size);
+        hipLaunchKernelGGL(sort_repack_kernel<3>, g2, dim3(256), 0, stream, qweight, kmap, qweight_sorted, K, N);
+    }
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+}
+
 // xs[m][j] = x[m][src[j]]: the activations of a layer whose channels were sorted by group, in the
 // sorted order.  Eight outputs per thread: two index vectors, eight 2-byte gathers (x is small and
 // stays in L2), one 16-byte store.  K is a multiple of 32.

@@ -115,6 +115,8 @@ int launch_grouped(const Params &p, int bits, const gptq_hip_plan &plan, void *s
 int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
                    void *w, int K, int N, int G, int bits, int group_size, void *stream);
 int launch_fill_zero(void *ptr, size_t bytes, void *stream);
+int launch_sort_channels(const uint32_t *qweight, const int32_t *g_idx, uint32_t *qweight_sorted, int32_t *kmap, int K,
+                         int N, int G, int bits, int group_size, void *stream);
 int launch_permute_x(const void *x, const int32_t *src, void *xs, int M, int K, void *stream);
 // Rows of x up to which the sorted entry point covers small batches (the STREAM kernel that reads x
 // itself, behind a pass that puts x into the sorted channel order)

@@ -176,6 +176,26 @@ def gemm_sorted(x: torch.Tensor, qweight_sorted: torch.Tensor, qzeros: torch.Ten
     return out
 
 
+def sort_channels(qweight: torch.Tensor, g_idx: torch.Tensor, bits: int, group_size: int):
+    """``pack.sort_channels_by_group`` on the library's own kernels: ``(qweight_sorted, kmap)`` on the GPU.
+    The caller vouches that every group has exactly ``group_size`` channels."""
+    _need_gpu("qweight", qweight, torch.int32)
+    _need_gpu("g_idx", g_idx, torch.int32)
+    rows, N = qweight.shape
+    K = rows * 32 // bits
+    if tuple(g_idx.shape) != (K,):
+        raise ValueError(f"g_idx must be [{K}], got {tuple(g_idx.shape)}")
+    dev = qweight.device
+    out = torch.empty_like(qweight)
+    kmap = torch.empty(2 * K, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().gptq_hip_sort_channels(_ptr(qweight), _ptr(g_idx), _ptr(out), _ptr(kmap), K, N, bits,
+                                               group_size, _stream(dev))
+    if rc != _lib.OK:
+        raise _lib.GptqHipError(rc, f"gptq_hip_sort_channels(K={K}, N={N}, bits={bits}, group_size={group_size})")
+    return out, kmap
+
+
 def dequant(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
             g_idx: Optional[torch.Tensor], bits: int, group_size: int) -> torch.Tensor:
     """The materialised fp16 weight [K, N], bit-exact with the reference's dequantisation."""

@@ -16,7 +16,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib, ops
-from .pack import pack_qweight, pack_qzeros, sort_channels_by_group
+from .pack import pack_qweight, pack_qzeros
 
 
 class _ProductWithInputGrad(torch.autograd.Function):
@@ -138,9 +138,21 @@ class QuantLinear(nn.Module):
         if self._sorted is None or self._sorted[0] != key:
             tensors = None
             if g is not None and q.device.type == "cuda":
-                tensors = sort_channels_by_group(q, g, self.bits, self.groupsize)
+                tensors = self._sort_on_gpu(q, g)
             self._sorted = (key, tensors)
         return self._sorted[1]
+
+    def _sort_on_gpu(self, q, g):
+        """``pack.sort_channels_by_group`` through the library's own kernels (gptq_hip_sort_channels), after
+        the one check they cannot make: that every group holds exactly ``groupsize`` channels."""
+        K, gs = self.infeatures, self.groupsize
+        klane = 8 if self.bits == 4 else 32
+        if K >= 65536 or K % gs != 0 or gs % klane != 0:
+            return None
+        counts = torch.bincount(g.to(torch.int64), minlength=K // gs)
+        if counts.numel() != K // gs or not bool((counts == gs).all()):
+            return None
+        return ops.sort_channels(q, g, self.bits, self.groupsize)
 
     def _decode_sorted(self, x2):
         """The decode product through the sorted copy, or None when that path does not apply."""

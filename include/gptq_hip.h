@@ -127,6 +127,19 @@ int gptq_hip_gemm_sorted(const void *x, const int32_t *qweight_sorted, const int
                          const int32_t *kmap, const void *bias, void *y, void *workspace, size_t workspace_bytes,
                          int M, int K, int N, int bits, int group_size, const gptq_hip_plan *plan, void *stream);
 
+/*
+ * The one-time preparation gptq_hip_gemm_sorted asks for, on the GPU: from a layer's qweight and g_idx
+ * writes qweight_sorted int32 [K/32*bits, N] (a separate buffer) and kmap int32 [2K], both 16-byte
+ * aligned.  The sort is stable (channels of a group keep their order).  g_idx must give every group
+ * exactly group_size channels (what GPTQ's activation order produces); other contents give a map
+ * that stays in bounds but does not describe the layer.  Same limits as gptq_hip_gemm_sorted
+ * (GPTQ_HIP_ERR_UNSUPPORTED beyond them).  Two launches on `stream`; K*K/2 compares, so tens of
+ * microseconds at K = 4096 and milliseconds at K = 65535.  The reference's counterpart is the weight
+ * re-layout of its TVM module's constructor (qlinear_tvm.py:25-40).
+ */
+int gptq_hip_sort_channels(const int32_t *qweight, const int32_t *g_idx, int32_t *qweight_sorted, int32_t *kmap,
+                           int K, int N, int bits, int group_size, void *stream);
+
 /* Bytes of workspace gptq_hip_gemm_sorted needs with plan = NULL (0 if none): what the plan for contiguous
  * groups needs and, when that plan is a STREAM one, M*K*2 bytes for x in the sorted order behind it (at
  * max(plan bytes, 16 KiB) rounded up to 256: the counters at the head of a workspace stay untouched). */

@@ -153,6 +153,13 @@ def test_entry_points_reject_null_and_bad_sizes_before_touching_the_gpu():
     assert lib.gptq_hip_sorted_workspace_bytes(4, 11008, 4096, 4, 128) == (max(p4.workspace_bytes, 16384) + 255) // 256 * 256 + 4 * 11008 * 2
     assert srt(fake, fake, fake, fake, fake, null, fake, null, 0, 1, 65536, 64, 4, 128, None, null) == _lib.ERR_UNSUPPORTED
     assert srt(fake, fake, fake, fake, fake, null, fake, null, 0, 1, 4096, 64, 3, 16, None, null) == _lib.ERR_UNSUPPORTED
+    # the load-time sort: in place, missing buffers, limits of the map
+    assert lib.gptq_hip_sort_channels(fake, fake, fake, fake, 4096, 64, 4, 128, null) == _lib.ERR_BAD_ARG
+    assert lib.gptq_hip_sort_channels(fake, fake, null, fake, 4096, 64, 4, 128, null) == _lib.ERR_BAD_ARG
+    other = ctypes.c_void_p(0x2000)
+    assert lib.gptq_hip_sort_channels(fake, fake, other, fake, 65536, 64, 4, 128, null) == _lib.ERR_UNSUPPORTED
+    assert lib.gptq_hip_sort_channels(fake, fake, other, fake, 4096, 64, 3, 16, null) == _lib.ERR_UNSUPPORTED
+    assert lib.gptq_hip_sort_channels(fake, fake, other, fake, 4096, 64, 2, 128, null) == _lib.ERR_BAD_ARG
     assert lib.gptq_hip_dequant(fake, fake, fake, null, null, 64, 64, 4, 32, null) == _lib.ERR_BAD_ARG
     assert lib.gptq_hip_dequant(fake, fake, fake, null, fake, 64, 64, 5, 32, null) == _lib.ERR_BAD_ARG
     assert lib.gptq_hip_workspace_init(null, 64, null) == _lib.ERR_BAD_ARG

@@ -397,6 +397,28 @@ def test_sorted_small_batch_matches_oracle(dev, bits, K, N, gs, M):
 
 
 @pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("K,N,gs", [(96, 32, 32), (1024, 416, 32), (2048, 1056, 256), (11008, 256, 128), (1024, 160, -1),
+                                    (4096, 352, 128)])
+def test_library_sort_equals_the_torch_preparation(dev, bits, K, N, gs):
+    # gptq_hip_sort_channels against pack.sort_channels_by_group: both tensors bit for bit
+    L = layer(980 + K, K, N, bits, gs, True)
+    D = to_dev(L, dev)
+    want = pack.sort_channels_by_group(D["qweight"], D["g_idx"], bits, gs)
+    if want is None:
+        with pytest.raises(_lib.GptqHipError) as e:
+            ops.sort_channels(D["qweight"], D["g_idx"], bits, gs)
+        assert e.value.status == _lib.ERR_UNSUPPORTED
+        return
+    got = ops.sort_channels(D["qweight"], D["g_idx"], bits, gs)
+    assert torch.equal(got[1], want[1])
+    assert torch.equal(got[0], want[0])
+    # a contiguous g_idx is its own sorted order
+    contiguous = (torch.arange(K, device=dev) // (K if gs == -1 else gs)).to(torch.int32)
+    same, kmap = ops.sort_channels(D["qweight"], contiguous, bits, gs)
+    assert torch.equal(same, D["qweight"]) and torch.equal(kmap[K:].long(), torch.arange(K, device=dev))
+
+
+@pytest.mark.parametrize("bits", [3, 4])
 @pytest.mark.parametrize("M", [1, 2])
 @pytest.mark.parametrize("split", [1, 2, 5, 16])
 def test_sorted_decode_forced_split_k(dev, bits, M, split):
