@@ -213,3 +213,31 @@ def dequant(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
     if rc != _lib.OK:
         raise _lib.GptqHipError(rc, f"gptq_hip_dequant(K={K}, N={N}, bits={bits})")
     return w
+
+
+# ---------------------------------------------------------------------------------------------
+# torch.ops.gptq_hip.{gemm, dequant}: the same two calls as dispatcher-visible operators (GPU kernels
+# and shape-only "meta" versions; no CPU kernel is registered, so a CPU tensor fails in the dispatcher
+# instead of falling back).
+def _meta_gemm(x, qweight, qzeros, scales, g_idx, bias, bits, group_size):
+    return x.new_empty((x.shape[0], qweight.shape[1]), dtype=torch.float16)
+
+
+def _meta_dequant(qweight, qzeros, scales, g_idx, bits, group_size):
+    return scales.new_empty((qweight.shape[0] * 32 // bits, qweight.shape[1]), dtype=torch.float16)
+
+
+def _register_torch_ops():
+    lib = torch.library.Library("gptq_hip", "DEF")
+    lib.define("gemm(Tensor x, Tensor qweight, Tensor qzeros, Tensor scales, Tensor? g_idx, Tensor? bias, "
+               "int bits, int group_size) -> Tensor")
+    lib.define("dequant(Tensor qweight, Tensor qzeros, Tensor scales, Tensor? g_idx, int bits, int group_size) "
+               "-> Tensor")
+    lib.impl("gemm", lambda x, qw, qz, sc, g, b, bits, gs: gemm(x, qw, qz, sc, g, b, bits, gs), "CUDA")
+    lib.impl("dequant", lambda qw, qz, sc, g, bits, gs: dequant(qw, qz, sc, g, bits, gs), "CUDA")
+    lib.impl("gemm", _meta_gemm, "Meta")
+    lib.impl("dequant", _meta_dequant, "Meta")
+    return lib
+
+
+_TORCH_OPS = _register_torch_ops()  # kept alive for the life of the module

@@ -577,3 +577,12 @@ def test_module_forward_replays_in_a_graph(dev, bits):
         for M in xs:
             assert torch.equal(outs[M], want[M]), (rep, M)
             assert_close(outs[M], expected_output(L, x=xs[M].cpu()), f"graph replay {rep}, M={M}")
+
+
+def test_torch_operator_equals_the_python_front_end(dev):
+    L = layer(990, 512, 256, 3, 128, True, M=5, bias=True)
+    D = to_dev(L, dev)
+    a = torch.ops.gptq_hip.gemm(D["x"], D["qweight"], D["qzeros"], D["scales"], D["g_idx"], D["bias"], 3, 128)
+    assert torch.equal(a, run_gemm(D))
+    w = torch.ops.gptq_hip.dequant(D["qweight"], D["qzeros"], D["scales"], D["g_idx"], 3, 128)
+    assert torch.equal(w.cpu().view(torch.int16), expected_weight(L).view(torch.int16))

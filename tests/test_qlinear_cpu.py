@@ -60,3 +60,17 @@ def test_shape_checks():
     with pytest.raises(NotImplementedError):
         ops.check_shapes(q.qweight, q.qzeros, q.scales, None, None, 2, 32)
     assert ops.check_shapes(q.qweight, q.qzeros, q.scales, q.g_idx, None, 4, 32) == (64, 32, 2)
+
+
+def test_torch_ops_are_registered_without_a_cpu_kernel():
+    from autogptq.tvm_amd import ops  # noqa: F401  (registers the operators)
+
+    q = QuantLinear(4, 32, 64, 96, False)
+    x = torch.zeros((3, 64), dtype=torch.float16)
+    meta = [t.to("meta") for t in (x, q.qweight, q.qzeros, q.scales)]
+    y = torch.ops.gptq_hip.gemm(meta[0], meta[1], meta[2], meta[3], None, None, 4, 32)
+    assert y.device.type == "meta" and tuple(y.shape) == (3, 96) and y.dtype == torch.float16
+    w = torch.ops.gptq_hip.dequant(meta[1], meta[2], meta[3], None, 4, 32)
+    assert tuple(w.shape) == (64, 96) and w.dtype == torch.float16
+    with pytest.raises((NotImplementedError, RuntimeError)):   # no CPU fallback, not even in the dispatcher
+        torch.ops.gptq_hip.gemm(x, q.qweight, q.qzeros, q.scales, None, None, 4, 32)
