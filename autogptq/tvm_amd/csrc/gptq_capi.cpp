@@ -80,7 +80,8 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
         const int need_tpm = gptq::grouped_tpm(gptq::grouped_groups(kr / pl.waves_k, gs, G, act_order), M);
         if (need_tpm == 0 || tpm != need_tpm) return GPTQ_HIP_ERR_UNSUPPORTED;
         if (pl.lds_bytes < gptq::grouped_lds_bytes(kr, M, tpm, pl.waves_n, pl.waves_k,
-                                                   gptq::grouped_lite(bits, K, gs, act_order != 0, tpm)))
+                                                   gptq::grouped_lite(bits, K, gs, act_order != 0, tpm, M, kr,
+                                                                      pl.waves_n, pl.waves_k, pl.split_k)))
             return GPTQ_HIP_ERR_BAD_ARG;
         return GPTQ_HIP_OK;
     }

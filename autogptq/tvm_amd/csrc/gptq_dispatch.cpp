@@ -190,7 +190,7 @@ bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, i
     const int waves_n = force_waves > 0 ? force_waves : 1;
     const int col_tiles = ceil_div(N, 64 * waves_n);
     if ((size_t)col_tiles * sizeof(int) > gptq::kCounterBytes) return false;
-    const int lds_cap = 144 * 1024;
+    const int lds_cap = gptq::kGroupedLdsCap;
     // a column tile per workgroup and no split is best (nothing crosses workgroups) unless
     // that leaves most of the 256 CUs idle
     int want = force_split > 0 ? force_split : (col_tiles >= 128 ? 1 : ceil_div(256, col_tiles));
@@ -211,8 +211,10 @@ bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, i
             if (act_order) return false;  // the group count does not shrink with the K range
             continue;
         }
-        const int lds = gptq::grouped_lds_bytes(kr, M, tpm, waves_n, waves_k,
-                                                gptq::grouped_lite(bits, K, gs, act_order != 0, tpm));
+        // int4 plans are sized for the tile layout and switch to the lean operand only afterwards
+        const bool lite = gptq::grouped_lite(bits, K, gs, act_order != 0, tpm, M, kr, waves_n, waves_k, split);
+        if (bits == 4 && gptq::grouped_lds_bytes(kr, M, tpm, waves_n, waves_k, false) > lds_cap) continue;
+        const int lds = gptq::grouped_lds_bytes(kr, M, tpm, waves_n, waves_k, lite);
         if (lds > lds_cap) continue;
         plan->kernel = GPTQ_HIP_KERNEL_GROUPED;
         plan->row_tiles = M * tpm;
@@ -345,7 +347,10 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
             grouped = true;
         }
     }
-    if (grouped && (M == 1 || plan->split_k == 1 || gptq::grouped_lite(bits, K, gs, act_order != 0, plan->row_tiles / M)) &&
+    if (grouped &&
+        (M == 1 || plan->split_k == 1 ||
+         gptq::grouped_lite(bits, K, gs, act_order != 0, plan->row_tiles / M, M, plan->k_chunk, plan->waves_n,
+                            plan->waves_k, plan->split_k)) &&
         (!act_order || plan->row_tiles / M <= 3)) {
         if (plan->split_k < (bits == 3 ? 9 : 8)) return GPTQ_HIP_OK;
         gptq_hip_plan alt;

@@ -32,7 +32,8 @@
 // holds just x in unpack order (2 bytes per channel instead of 32) plus 16 zero bytes: a lane reads
 // x when its row is the block's group and the zeros otherwise.  Only x itself is zero-filled (8 KB
 // instead of 128 KB at K = 4096), and the scatter's 2-byte stores spread over the banks instead of
-// hitting the two banks of one tile row.  Used for int3 (see launch_grouped_one).
+// hitting the two banks of one tile row.  Used for int3, and for int4 where one workgroup holds all
+// of K (grouped_lite in gptq_internal.h).
 //
 // Sorted layers: when the loader has sorted the channels of an activation-order layer by
 // group (qweight rows permuted, p.kmap saying where each original channel went), the groups
@@ -513,11 +514,10 @@ template <int BITS, int M, int TPM, bool COMPACT, bool LITE = false>
 static int launch_grouped_one(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
     constexpr int NSTEP = BITS == 4 ? 16 : 4;
-    if constexpr (BITS == 3 && TPM == 1 && !COMPACT && !LITE) {
-        // contiguous groups made of whole lane blocks: the lean operand.  Not for int4: its steps are
-        // a quarter as long, and choosing the row per step costs what the lean prologue saves
-        // (measured: 4096 x 4096 8.3 -> 8.7 us, 11008 x 4096 10.8 -> 11.7 us).
-        if (grouped_lite(BITS, p.K, p.group_size, p.g_idx != nullptr, TPM))
+    if constexpr (TPM == 1 && !COMPACT && !LITE) {
+        // contiguous groups made of whole lane blocks: the lean operand (the same rule sized the plan's LDS)
+        if (grouped_lite(BITS, p.K, p.group_size, p.g_idx != nullptr, TPM, M, plan.k_chunk, plan.waves_n, plan.waves_k,
+                         plan.split_k))
             return launch_grouped_one<BITS, M, TPM, COMPACT, true>(p, plan, stream);
     }
     auto kern = grouped_kernel<BITS, M, TPM, COMPACT, NSTEP, LITE>;

@@ -55,11 +55,21 @@ static const size_t kCounterBytes = 16384;
 int grouped_tpm(int groups, int M);
 int grouped_groups(int kr, int gs, int G, int act_order);
 int grouped_lds_bytes(int kr, int M, int tpm, int waves_n, int waves_k, bool lite);
-// The lean operand (x itself in LDS instead of operand tiles): int3, groups that are contiguous for the
-// weight stream and made of whole 32-channel lane blocks, one row tile.
-constexpr bool grouped_lite(int bits, int K, int gs, bool has_g_idx, int tpm)
+// LDS the GROUPED plans may use
+static const int kGroupedLdsCap = 144 * 1024;
+// The lean operand (x itself in LDS instead of operand tiles) needs groups that are contiguous for the
+// weight stream and made of whole lane blocks, and one row tile.  int3 always takes it.  int4 takes it
+// only where the tile layout would also hold all of K in one workgroup: there it saves the zero fill
+// and the bank conflicts of the scatter (4096 x 11008 9.1 -> 8.3 us); with K split over workgroups
+// it is a little slower than the tiles (4096 x 4096 8.4 -> 8.6 us), and a plan that no longer needs to
+// split K for LDS loses the workgroups that filled the chip (9216 x 36864 33.9 -> 37.5 us).
+inline bool grouped_lite(int bits, int K, int gs, bool has_g_idx, int tpm, int M, int kr, int waves_n, int waves_k,
+                         int split_k)
 {
-    return bits == 3 && !has_g_idx && tpm == 1 && gs % 32 == 0 && K / 32 < 65536;
+    const int klane = bits == 4 ? 8 : 32;
+    if (has_g_idx || tpm != 1 || gs % klane != 0 || K / klane >= 65536) return false;
+    if (bits == 3) return true;
+    return split_k == 1 && grouped_lds_bytes(kr, M, tpm, waves_n, waves_k, false) <= kGroupedLdsCap;
 }
 // Input channels of x the GATHER kernel stages per K wave at a time: fixed per (bits, row tiles) so
 // that the kernel's unrolled step loop knows its chunk boundaries at compile time.  The chunk is a
