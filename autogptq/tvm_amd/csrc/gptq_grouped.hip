@@ -54,13 +54,16 @@ __device__ __forceinline__ h8 and_h8(h8 a, u4 m)
 }
 
 // TPM = row tiles (of 16 groups) per activation row; COMPACT needs TPM == 2.
-template <int BITS, int M, int TPM, bool COMPACT, int NSTEP, bool LITE>
+// WAVEX (lean operand without a channel map, a wave's K range of at most 512 channels): every wave
+// stages the x of its own K range itself, so nothing crosses waves before the reduction.
+template <int BITS, int M, int TPM, bool COMPACT, int NSTEP, bool LITE, bool WAVEX = false>
 __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
 {
     using F = Fmt<BITS>;
     constexpr int ST = COMPACT ? M : M * TPM;    // tiles stored in LDS per 8 slots
     static_assert(!COMPACT || TPM == 2, "compact layout is for two row tiles");
     static_assert(!LITE || (TPM == 1 && !COMPACT), "the lite operand is one row tile of contiguous groups");
+    static_assert(!WAVEX || LITE, "wave-private staging is for the lean operand");
     const int tid = threadIdx.x;
     const int nthreads = (int)blockDim.x;
     const int lane = tid & 63;
@@ -109,7 +112,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     const uint32_t zero_off = (uint32_t)M * (uint32_t)kspan * 2u;
     if constexpr (LITE) {
         red = (float *)(smem + zero_off + 16);
-        if (tid < 4) ((uint32_t *)(smem + zero_off))[tid] = 0u;
+        if (WAVEX ? lane < 4 : tid < 4) ((uint32_t *)(smem + zero_off))[lane & 3] = 0u;  // WAVEX: every wave writes them
     }
 
     int qslot[4];
@@ -136,7 +139,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     const int32_t *mapsrc = xsrc ? xsrc : (kmap ? kmap : (p.g_idx ? p.g_idx : (const int32_t *)p.qweight));
     const bool has_map = kmap != nullptr || p.g_idx != nullptr;
 #pragma unroll
-    for (int ps = 0; ps < QP; ps++) {
+    for (int ps = 0; ps < (WAVEX ? 0 : QP); ps++) {
         const int idx = tid + ps * nthreads;
         const int idc = min(idx, nquads - 1);
         const int m = M == 1 ? 0 : idc / qpr;
@@ -151,12 +154,39 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         for (int e = 0; e < 4; e++) gq[ps][e] = (k + e) / p.group_size;
     }
 
+    // ---- 1w. WAVEX: the wave requests the x of its own K range: at most 512 channels per activation
+    //          row, 64 quads per pass ------------------------------------------------------------
+    constexpr int XP = 2 * M;
+    h4 wxq[XP];
+    bool wqv[XP];  // the quad is inside the wave's range and inside K
+    int wpos[XP];  // where the quad's lane block starts in xlds
+    if constexpr (WAVEX) {
+        const int wq = wave_k / 4;  // quads per activation row in this wave's range
+#pragma unroll
+        for (int ps = 0; ps < XP; ps++) {
+            const int q = lane + 64 * ps;
+            const int m = M == 1 ? 0 : min(q / wq, M - 1);
+            const int kc = wk * wave_k + 4 * (q - m * wq);  // position inside the workgroup's K range
+            const int k = k_base + kc;
+            wqv[ps] = q < M * wq && k < p.K;
+            const int kl = min(max(k, 0), p.K - 4);
+            wpos[ps] = m * kspan + (kc / F::KLANE) * F::KLANE;
+            wxq[ps] = *(const h4 *)(x + (size_t)m * p.K + kl);
+        }
+    }
+
     // ---- 2. zero the expanded activation operand in LDS while those loads fly ---------
-    {
-        // LITE: only x itself (channels past the end of K must read as zero)
+    if constexpr (!WAVEX && !LITE) {
         u4 *z = (u4 *)tiles;
-        const int n16 = LITE ? M * kspan / 8 : nblk8 * ST * 16;
+        const int n16 = nblk8 * ST * 16;
         for (int i = tid; i < n16; i += nthreads) z[i] = (u4){0u, 0u, 0u, 0u};
+    }
+    if constexpr (!WAVEX && LITE) {
+        // only positions past the end of K must read as zero; the scatter writes every other one, so
+        // the two never touch the same bytes and no barrier is needed between them
+        const int tail0 = max(p.K - k_base, 0) / 8;  // K % 32 == 0
+        for (int m = 0; m < M; m++)
+            for (int i = tail0 + tid; i < kspan / 8; i += nthreads) ((u4 *)(xlds + m * kspan))[i] = (u4){0u, 0u, 0u, 0u};
     }
     // ---- 3. weight loads, software-pipelined: a wave blocks while it issues loads into a full
     //         memory pipeline, so only the first PF steps go out now (they cover the LDS work
@@ -177,9 +207,9 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         }
     };
 #pragma unroll
-    for (int s = 0; s < PF && s < NSTEP; s++) load_step(s, ws + s);
+    for (int s = 0; s < (WAVEX ? 0 : PF) && s < NSTEP; s++) load_step(s, ws + s);
     __builtin_amdgcn_sched_barrier(0);
-    if (xsrc) {  // the x values of this thread's positions, now that their source channels are known
+    if (!WAVEX && xsrc) {  // the x values of this thread's positions, now that their source channels are known
 #pragma unroll
         for (int ps = 0; ps < QP; ps++) {
             const int idc = min(tid + ps * nthreads, nquads - 1);
@@ -210,7 +240,29 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         }
     };
 
-    lds_barrier();
+    // ---- 4w. WAVEX: the first weight requests, the epilogue operands, and only then the wait for x ----
+    if constexpr (WAVEX) {
+#pragma unroll
+        for (int s = 0; s < PF && s < NSTEP; s++) load_step(s, ws + s);
+        __builtin_amdgcn_sched_barrier(0);
+        load_epilogue_operands();
+        __builtin_amdgcn_sched_barrier(0);
+        // x into this wave's part of LDS in unpack order, channels past the end of K as zeros
+#pragma unroll
+        for (int ps = 0; ps < XP; ps++) {
+            if (lane + 64 * ps < M * (wave_k / 4)) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) xlds[wpos[ps] + qslot[e]] = wqv[ps] ? wxq[ps][e] : (_Float16)0;
+            }
+        }
+        // LDS serves the accesses of one wave in order; the fences only keep the compiler from moving
+        // the main loop's reads above these writes
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    if constexpr (!WAVEX) {
+    if constexpr (!LITE) lds_barrier();  // the zero fill is complete
     // ---- 5. scatter x into the operand tiles (waits for x / g_idx only) -------------------
     // A thread always owns quads with the same position inside a lane block (kc % KLANE is
     // 4 * (tid % (KLANE / 4)) in every pass because the block size is a multiple of 8), so the
@@ -318,6 +370,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     }
     lds_barrier();
     load_epilogue_operands();
+    }  // !WAVEX
 
     // ---- 6. main loop -----------------------------------------------------------------
     // acc[m][t][c] collects sum x * (base + code); accx[m][t] is the same operand against the
@@ -510,7 +563,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     }
 }
 
-template <int BITS, int M, int TPM, bool COMPACT, bool LITE = false>
+template <int BITS, int M, int TPM, bool COMPACT, bool LITE = false, bool WAVEX = false>
 static int launch_grouped_one(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
     constexpr int NSTEP = BITS == 4 ? 16 : 4;
@@ -520,7 +573,12 @@ static int launch_grouped_one(const Params &p, const gptq_hip_plan &plan, hipStr
                          plan.split_k))
             return launch_grouped_one<BITS, M, TPM, COMPACT, true>(p, plan, stream);
     }
-    auto kern = grouped_kernel<BITS, M, TPM, COMPACT, NSTEP, LITE>;
+    if constexpr (LITE && !WAVEX) {
+        // short K ranges per wave and x in the order of the weights: every wave stages its own x
+        if (grouped_wavex(true, p.wave_steps * Fmt<BITS>::KSTEP) && !p.kmap && !p.xsrc)
+            return launch_grouped_one<BITS, M, TPM, COMPACT, true, true>(p, plan, stream);
+    }
+    auto kern = grouped_kernel<BITS, M, TPM, COMPACT, NSTEP, LITE, WAVEX>;
     const int lds_bytes = plan.lds_bytes;  // sized by the dispatcher for the operand layout in use
     if (lds_bytes > 65536) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) !=
