@@ -71,11 +71,20 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
         return GPTQ_HIP_OK;
     }
     if (pl.kernel == GPTQ_HIP_KERNEL_GROUPED) {
-        if (M > 2 || pl.grid_z != 1 || pl.row_tiles % M != 0) return GPTQ_HIP_ERR_UNSUPPORTED;
+        if (M > gptq::kPackedRows || pl.grid_z != 1) return GPTQ_HIP_ERR_UNSUPPORTED;
         // k_chunk is the K range of one workgroup: waves_k * wave_steps whole steps
         if (pl.k_chunk < kstep * pl.waves_k || pl.k_chunk % (kstep * pl.waves_k) != 0) return GPTQ_HIP_ERR_BAD_ARG;
         const int kr = pl.k_chunk;
         if ((long long)kr * pl.split_k < (long long)steps_total * kstep) return GPTQ_HIP_ERR_BAD_ARG;
+        if (M > 2) {
+            // packed rows: one operand tile, LDS and partial sums sized for four rows
+            if (pl.row_tiles != gptq::kPackedRows || !gptq::grouped_packable(bits, K, gs, act_order != 0, M, kr, pl.waves_k))
+                return GPTQ_HIP_ERR_UNSUPPORTED;
+            if (pl.lds_bytes < gptq::grouped_lds_bytes(kr, gptq::kPackedRows, 1, pl.waves_n, pl.waves_k, true))
+                return GPTQ_HIP_ERR_BAD_ARG;
+            return GPTQ_HIP_OK;
+        }
+        if (pl.row_tiles % M != 0) return GPTQ_HIP_ERR_UNSUPPORTED;
         const int tpm = pl.row_tiles / M;
         const int need_tpm = gptq::grouped_tpm(gptq::grouped_groups(kr / pl.waves_k, gs, G, act_order), M);
         if (need_tpm == 0 || tpm != need_tpm) return GPTQ_HIP_ERR_UNSUPPORTED;
@@ -133,7 +142,7 @@ static int run_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros
     p.wave_steps = plan->kernel == GPTQ_HIP_KERNEL_GROUPED
                        ? plan->k_chunk / kstep / plan->waves_k
                        : (p.steps_total + plan->split_k * plan->waves_k - 1) / (plan->split_k * plan->waves_k);
-    p.gpad = plan->kernel == GPTQ_HIP_KERNEL_GROUPED ? 16 * (plan->row_tiles / M) : 0;
+    p.gpad = plan->kernel == GPTQ_HIP_KERNEL_GROUPED ? (M > 2 ? 16 : 16 * (plan->row_tiles / M)) : 0;
     p.xpack = nullptr;
     p.gpack = nullptr;
     p.rt_total = 0;
@@ -155,11 +164,12 @@ static int run_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros
         }
     }
     size_t ws_plan = workspace_bytes;  // bytes of the workspace the plan itself may use
-    if (kmap && plan->kernel == GPTQ_HIP_KERNEL_STREAM) {
+    if (kmap && (plan->kernel == GPTQ_HIP_KERNEL_STREAM || (plan->kernel == GPTQ_HIP_KERNEL_GROUPED && M > 2))) {
         // small batches on a sorted layer: x goes into the sorted channel order first (one small pass
         // into the tail of the workspace), then the kernel for contiguous groups reads it directly
-        if (M > gptq::kSortedMaxRows || plan->row_tiles != 1 ||
-            !gptq::stream_direct(bits, K, 1, gptq::stream_act_table(bits, gs, 0), false))
+        if (plan->kernel == GPTQ_HIP_KERNEL_STREAM &&
+            (M > gptq::kSortedMaxRows || plan->row_tiles != 1 ||
+             !gptq::stream_direct(bits, K, 1, gptq::stream_act_table(bits, gs, 0), false)))
             return GPTQ_HIP_ERR_UNSUPPORTED;
         const size_t head = gptq::sorted_x_offset(plan->workspace_bytes);
         const size_t xs_bytes = (size_t)M * K * 2;
@@ -281,7 +291,8 @@ extern "C" size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits,
 {
     gptq_hip_plan plan;
     if (gptq_hip_select(M, K, N, bits, group_size, 0, &plan) != GPTQ_HIP_OK) return 0;
-    if (plan.kernel == GPTQ_HIP_KERNEL_STREAM && M <= gptq::kSortedMaxRows)
+    if ((plan.kernel == GPTQ_HIP_KERNEL_STREAM && M <= gptq::kSortedMaxRows) ||
+        (plan.kernel == GPTQ_HIP_KERNEL_GROUPED && M > 2))
         return gptq::sorted_x_offset(plan.workspace_bytes) + (size_t)M * K * 2;
     return plan.workspace_bytes;
 }

@@ -234,6 +234,48 @@ bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, i
     return false;
 }
 
+// GROUPED with three or four activation rows packed into the one operand tile (contiguous groups only).
+// The plan is sized for four rows whatever M is.
+bool plan_grouped_packed(int M, int K, int N, int bits, int gs, int force_split, int force_waves, gptq_hip_plan *plan)
+{
+    const int kstep = gptq::kstep_of(bits);
+    const int steps_total = ceil_div(K, kstep);
+    const int waves_n = force_waves > 0 ? force_waves : 1;
+    const int col_tiles = ceil_div(N, 64 * waves_n);
+    if ((size_t)col_tiles * sizeof(int) > gptq::kCounterBytes) return false;
+    int want = force_split > 0 ? force_split : (col_tiles >= 128 ? 1 : ceil_div(256, col_tiles));
+    if (want > steps_total) want = steps_total;
+    for (int want_split = want; want_split <= steps_total && want_split <= 256; want_split++) {
+        if (force_split > 0 && want_split != want) return false;
+        int waves_k = 8 / waves_n;
+        if (waves_k * want_split > steps_total) waves_k = steps_total / want_split;
+        if (waves_k < 1) waves_k = 1;
+        const int wave_steps = ceil_div(steps_total, want_split * waves_k);
+        const int wg_steps = wave_steps * waves_k;
+        const int split = ceil_div(steps_total, wg_steps);
+        const int kr = wg_steps * kstep;
+        if (!gptq::grouped_packable(bits, K, gs, false, M, kr, waves_k)) continue;
+        const int lds = gptq::grouped_lds_bytes(kr, gptq::kPackedRows, 1, waves_n, waves_k, true);
+        if (lds > gptq::kGroupedLdsCap) continue;
+        plan->kernel = GPTQ_HIP_KERNEL_GROUPED;
+        plan->row_tiles = gptq::kPackedRows;
+        plan->m_blocks = 1;
+        plan->waves_n = waves_n;
+        plan->waves_k = waves_k;
+        plan->split_k = split;
+        plan->k_chunk = kr;
+        plan->grid_x = col_tiles;
+        plan->grid_y = split;
+        plan->grid_z = 1;
+        plan->block = 64 * waves_n * waves_k;
+        plan->lds_bytes = lds;
+        plan->workspace_bytes =
+            split > 1 ? gptq::kCounterBytes + (size_t)split * gptq::kPackedRows * N * sizeof(float) : 0;
+        return true;
+    }
+    return false;
+}
+
 // STREAM: exact weights, any g_idx, any M; x pre-packed, waves independent.
 // force_waves is the number of waves along K (1, 2, 4 or 8), 0 = choose.
 int plan_stream(int M, int K, int N, int bits, int gs, int G, int act_order, int force_split, int force_waves,
@@ -347,8 +389,22 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
             grouped = true;
         }
     }
+    bool packed = false;
+    if ((M == 3 || M == 4) && !act_order) {
+        // three or four rows for the matrix instructions of one (contiguous groups, short K ranges per wave)
+        gptq_hip_plan narrow;
+        memset(&narrow, 0, sizeof(narrow));
+        const bool have_narrow = plan_grouped_packed(M, K, N, bits, gs, 0, 0, &narrow);
+        const bool have_wide = wide && plan_grouped_packed(M, K, N, bits, gs, 0, wide, plan);
+        if (have_wide && (!have_narrow || plan->split_k <= narrow.split_k)) {
+            grouped = packed = true;
+        } else if (have_narrow) {
+            *plan = narrow;
+            grouped = packed = true;
+        }
+    }
     if (grouped &&
-        (M == 1 || plan->split_k == 1 ||
+        (M == 1 || packed || plan->split_k == 1 ||
          gptq::grouped_lite(bits, K, gs, act_order != 0, plan->row_tiles / M, M, plan->k_chunk, plan->waves_n,
                             plan->waves_k, plan->split_k)) &&
         (!act_order || plan->row_tiles / M <= 3)) {
@@ -387,6 +443,8 @@ extern "C" int gptq_hip_plan_for(int kernel, int M, int K, int N, int bits, int 
     }
     if (kernel == GPTQ_HIP_KERNEL_GROUPED) {
         if (M <= 2 && plan_grouped(M, K, N, bits, gs, G, act_order, split_k, waves_n, plan)) return GPTQ_HIP_OK;
+        if ((M == 3 || M == 4) && !act_order && plan_grouped_packed(M, K, N, bits, gs, split_k, waves_n, plan))
+            return GPTQ_HIP_OK;
         memset(plan, 0, sizeof(*plan));
         return GPTQ_HIP_ERR_UNSUPPORTED;
     }

@@ -1,4 +1,4 @@
-// GROUPED kernel family: decode-size products (M of 1 or 2) for any g_idx.
+// GROUPED kernel family: decode-size products (M of 1 or 2 for any g_idx; 3 or 4 with contiguous groups).
 //
 // Instead of looking a scale and zero up for every weight, the rows of the MFMA are
 // expanded by group:  row (m, g) of the activation operand holds x[m, k] where
@@ -56,7 +56,10 @@ __device__ __forceinline__ h8 and_h8(h8 a, u4 m)
 // TPM = row tiles (of 16 groups) per activation row; COMPACT needs TPM == 2.
 // WAVEX (lean operand without a channel map, a wave's K range of at most 512 channels): every wave
 // stages the x of its own K range itself, so nothing crosses waves before the reduction.
-template <int BITS, int M, int TPM, bool COMPACT, int NSTEP, bool LITE, bool WAVEX = false>
+// PACK (WAVEX, at most four groups in a wave's K range, M = 4 rows of which p.M are real): row 4 m + g of
+// the ONE operand tile holds x[m] for group g of the wave, so three or four activation rows cost the
+// matrix instructions of one; lane group q of the result is activation row q, register v its group v.
+template <int BITS, int M, int TPM, bool COMPACT, int NSTEP, bool LITE, bool WAVEX = false, bool PACK = false>
 __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
 {
     using F = Fmt<BITS>;
@@ -64,14 +67,16 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     static_assert(!COMPACT || TPM == 2, "compact layout is for two row tiles");
     static_assert(!LITE || (TPM == 1 && !COMPACT), "the lite operand is one row tile of contiguous groups");
     static_assert(!WAVEX || LITE, "wave-private staging is for the lean operand");
+    static_assert(!PACK || (WAVEX && M == 4), "packed rows: four activation rows x four groups in one tile");
+    constexpr int MA = PACK ? 1 : M;  // operand tiles (and accumulator sets) per row tile
     const int tid = threadIdx.x;
-    const int nthreads = (int)blockDim.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int WN = p.waves_n;
+    const int WN = p.waves_n;  // 1, 2 or 4
     const int WK = p.waves_k;
-    const int wn = wave % WN;
-    const int wk = wave / WN;
+    const int nthreads = 64 * WN * WK;  // the block size, without a second trip to the kernel arguments
+    const int wn = wave & (WN - 1);
+    const int wk = wave >> (WN >> 1);  // log2 of 1, 2, 4
     const int li = lane & 15;
     const int lq = lane >> 4;
     const int BN = 64 * WN;
@@ -91,13 +96,18 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     // contiguous groups: only those inside this K range need rows, counted from the first one
     // (rows are counted per wave: a wave's K range meets few groups, so one row tile usually holds them)
     const int wave_k = p.wave_steps * F::KSTEP;  // channels per wave
-    const int g_base = p.g_idx ? 0 : (ws * F::KSTEP) / p.group_size;
+    // (the lean operand comes with the lane-block-to-group multiplier, which spares a division here)
+    const uint32_t lb0 = (uint32_t)(ws * (F::KSTEP / F::KLANE));  // first lane block of the wave
+    const int g_base = LITE ? (int)(__umulhi(lb0, p.gdiv_magic) + (p.gdiv_add ? lb0 : 0u))
+                            : (p.g_idx ? 0 : (ws * F::KSTEP) / p.group_size);
     __shared__ int last_flag;
     __shared__ int wave_gb[8];  // sorted layers: first group of each wave along K
     const int32_t *kmap = p.kmap;
     const int32_t *xsrc = p.xsrc;
     auto src_ok = [&](int c) { return (int)min((uint32_t)c, (uint32_t)p.K - 1u); };  // a bad map must not fault
-    if (kmap && tid < WK) wave_gb[tid] = (k_base + tid * wave_k) / p.group_size;
+    if constexpr (!LITE) {
+        if (kmap && tid < WK) wave_gb[tid] = (k_base + tid * wave_k) / p.group_size;
+    }
 
     const _Float16 *x = (const _Float16 *)p.x;
     const _Float16 *scales = (const _Float16 *)p.scales;
@@ -168,10 +178,10 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
             const int m = M == 1 ? 0 : min(q / wq, M - 1);
             const int kc = wk * wave_k + 4 * (q - m * wq);  // position inside the workgroup's K range
             const int k = k_base + kc;
-            wqv[ps] = q < M * wq && k < p.K;
+            wqv[ps] = q < M * wq && k < p.K && (!PACK || m < p.M);  // PACK: rows past p.M stay zero
             const int kl = min(max(k, 0), p.K - 4);
             wpos[ps] = m * kspan + (kc / F::KLANE) * F::KLANE;
-            wxq[ps] = *(const h4 *)(x + (size_t)m * p.K + kl);
+            wxq[ps] = *(const h4 *)(x + (size_t)(PACK ? min(m, p.M - 1) : m) * p.K + kl);
         }
     }
 
@@ -232,12 +242,26 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
         for (int t = 0; t < TPM; t++) {
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const uint32_t g = (uint32_t)min(g_base + 16 * t + 4 * lq + v, p.G - 1);
+                const uint32_t g = (uint32_t)min(g_base + (PACK ? v : 16 * t + 4 * lq + v), p.G - 1);
                 const uint32_t soff = (g * (uint32_t)p.N + (uint32_t)n_ld) * 2u;
                 sc[t][v] = *(const h4 *)((const char *)scales + soff);
                 load_zero_words<BITS>(p.qzeros, g * (uint32_t)zwords, n_ld, zwa[t][v], zwb[t][v]);
             }
         }
+    };
+
+    // The epilogue's scales and zero points as floats.  The lean-operand kernels convert them after the
+    // first step of the main loop, while the wave waits for weights anyway, instead of after the last.
+    float zf[TPM][4][4], sf[TPM][4][4];
+    auto prep_epilogue = [&]() {
+#pragma unroll
+        for (int t = 0; t < TPM; t++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                zeros_from_words<BITS>(zwa[t][v], zwb[t][v], n_ld, zf[t][v]);
+#pragma unroll
+                for (int c = 0; c < 4; c++) sf[t][v][c] = (float)sc[t][v][c];
+            }
     };
 
     // ---- 4w. WAVEX: the first weight requests, the epilogue operands, and only then the wait for x ----
@@ -377,10 +401,10 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     // constant columns "all ones" (column 0 -> X) and "the slot bases" (column 1 -> the base
     // part to subtract).  In the compact layout t = 0 is the masked tile (groups < 16) and
     // t = 1 the unmasked one (all groups): groups >= 16 are their difference.
-    f4 acc[M][TPM][4];
-    f4 accx[M][TPM];
+    f4 acc[MA][TPM][4];
+    f4 accx[MA][TPM];
 #pragma unroll
-    for (int m = 0; m < M; m++)
+    for (int m = 0; m < MA; m++)
 #pragma unroll
         for (int t = 0; t < TPM; t++) {
             accx[m][t] = (f4){0.f, 0.f, 0.f, 0.f};
@@ -420,8 +444,14 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
 #pragma unroll
                 for (int nb = 0; nb < F::NB; nb++) {
                     const int b8 = b * F::NB + nb;
-                    h8 a[M][TPM];
-                    if constexpr (LITE) {
+                    h8 a[MA][TPM];
+                    if constexpr (PACK) {
+                        // lane i feeds row i of the tile: activation row i / 4, group i % 4 of the wave
+                        const uint32_t lb = (uint32_t)((st0 + s) * 4 + lq);
+                        const int row = (int)(__umulhi(lb, p.gdiv_magic) + (p.gdiv_add ? lb : 0u)) - g_base;
+                        const uint32_t off = row == (li & 3) ? (uint32_t)((li >> 2) * kspan + b8 * 8) * 2u : zero_off;
+                        a[0][0] = *(const h8 *)(smem + off);
+                    } else if constexpr (LITE) {
                         // the group of this lane block, as a row of the wave's tile
                         const uint32_t lb = (uint32_t)((st0 + s) * 4 + lq);
                         const int row = (int)(__umulhi(lb, p.gdiv_magic) + (p.gdiv_add ? lb : 0u)) - g_base;
@@ -449,7 +479,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
                     for (int c = 0; c < 4; c++) {
                         const h8 bop = __builtin_bit_cast(h8, bq[c][nb]);
 #pragma unroll
-                        for (int m = 0; m < M; m++)
+                        for (int m = 0; m < MA; m++)
 #pragma unroll
                             for (int t = 0; t < TPM; t++) {
                                 acc[m][t][c] =
@@ -457,25 +487,29 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
                             }
                     }
 #pragma unroll
-                    for (int m = 0; m < M; m++)
+                    for (int m = 0; m < MA; m++)
 #pragma unroll
                         for (int t = 0; t < TPM; t++) {
                             accx[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[m][t], cb, accx[m][t], 0, 0, 0);
                         }
                 }
             }
+            if constexpr (LITE) {
+                if (s == 0) prep_epilogue();
+            }
         }
     }
+    if (!LITE || ws >= we) prep_epilogue();  // (a wave without steps still multiplies its zero sums by finite numbers)
 
     // ---- 7. scales and zero points once per group, then sum over groups ------------------
     // row v of tile t in lane group q is group g_base + 16 t + 4 q + v
-    float tot[M][4];
+    float tot[MA][4];
 #pragma unroll
-    for (int m = 0; m < M; m++)
+    for (int m = 0; m < MA; m++)
 #pragma unroll
         for (int c = 0; c < 4; c++) tot[m][c] = 0.f;
 #pragma unroll
-    for (int m = 0; m < M; m++) {
+    for (int m = 0; m < MA; m++) {
         float xs_prev[4] = {0.f, 0.f, 0.f, 0.f}, bs_prev[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int t = 0; t < TPM; t++) {
@@ -497,26 +531,28 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
                         for (int c = 0; c < 4; c++) pv[c] -= acc[m][0][c][v];
                     }
                 }
-                float z[4];
-                zeros_from_words<BITS>(zwa[t][v], zwb[t][v], n_ld, z);
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
-                    tot[m][c] += (float)sc[t][v][c] * ((pv[c] - bsum) - z[c] * xsum);
+                    tot[m][c] += sf[t][v][c] * ((pv[c] - bsum) - zf[t][v][c] * xsum);
                 }
             }
         }
     }
+    if constexpr (!PACK) {  // (PACK: a lane group's rows are the groups of ITS activation row)
 #pragma unroll
-    for (int m = 0; m < M; m++) {
+        for (int m = 0; m < M; m++) {
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            tot[m][c] += __shfl_xor(tot[m][c], 16);
-            tot[m][c] += __shfl_xor(tot[m][c], 32);
+            for (int c = 0; c < 4; c++) {
+                tot[m][c] += __shfl_xor(tot[m][c], 16);
+                tot[m][c] += __shfl_xor(tot[m][c], 32);
+            }
         }
     }
 
     // ---- 8. waves along K meet in LDS; one thread per four output columns finishes --------
-    if (lq == 0) {
+    if constexpr (PACK) {
+        *(f4 *)(red + (((size_t)wk * WN + wn) * M + lq) * 64 + 4 * li) = (f4){tot[0][0], tot[0][1], tot[0][2], tot[0][3]};
+    } else if (lq == 0) {
 #pragma unroll
         for (int m = 0; m < M; m++) {
             *(f4 *)(red + (((size_t)wk * WN + wn) * M + m) * 64 + 4 * li) =
@@ -528,7 +564,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     const int f_wn = tid / (M * 16);
     const int f_m = (tid >> 4) % M;
     const int f_n = blockIdx.x * BN + f_wn * 64 + 4 * (tid & 15);
-    const bool writer = fin && f_n < p.N;
+    const bool writer = fin && f_n < p.N && (!PACK || f_m < p.M);
     f4 sum = {0.f, 0.f, 0.f, 0.f};
     if (writer) {
         for (int k = 0; k < WK; k++) {
@@ -591,10 +627,31 @@ static int launch_grouped_one(const Params &p, const gptq_hip_plan &plan, hipStr
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 
+// three or four activation rows packed into one operand tile
+template <int BITS>
+static int launch_grouped_packed(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
+{
+    constexpr int NSTEP = BITS == 4 ? 16 : 4;
+    if (p.kmap || p.xsrc || !grouped_packable(BITS, p.K, p.group_size, p.g_idx != nullptr, p.M, plan.k_chunk, plan.waves_k))
+        return GPTQ_HIP_ERR_UNSUPPORTED;
+    auto kern = grouped_kernel<BITS, kPackedRows, 1, false, NSTEP, true, true, true>;
+    const int lds_bytes = plan.lds_bytes;
+    if (lds_bytes > 65536) {
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) !=
+            hipSuccess) {
+            (void)hipGetLastError();
+            return GPTQ_HIP_ERR_LAUNCH;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, 1), dim3(plan.block), lds_bytes, stream, p);
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+}
+
 template <int BITS>
 static int launch_grouped_bits(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
     const int tpm = p.gpad / 16;
+    if (p.M == 3 || p.M == 4) return tpm == 1 ? launch_grouped_packed<BITS>(p, plan, stream) : GPTQ_HIP_ERR_UNSUPPORTED;
     if (p.M == 1) {
         switch (tpm) {
             case 1: return launch_grouped_one<BITS, 1, 1, false>(p, plan, stream);

@@ -77,6 +77,22 @@ inline bool grouped_lite(int bits, int K, int gs, bool has_g_idx, int tpm, int M
 // channels of a sorted layer up per wave instead (two dependent round trips) loses to the shared
 // scatter with its one barrier (7.9 against 7.6 us).
 inline bool grouped_wavex(bool lite, int wave_channels) { return lite && wave_channels <= 512; }
+// Packed rows in the GROUPED kernel (three or four activation rows for the matrix instructions of one):
+// the lean operand with wave-private staging, and at most four groups in a wave's K range, counted
+// exactly (a wave's range starts at a multiple of its length).  Such plans are sized for four rows.
+static const int kPackedRows = 4;
+inline int wave_groups_exact(int wave_channels, int gs)
+{
+    if (gs % wave_channels == 0) return 1;
+    return wave_channels % gs == 0 ? wave_channels / gs : 0;  // 0: not a whole number
+}
+inline bool grouped_packable(int bits, int K, int gs, bool has_g_idx, int M, int kr, int waves_k)
+{
+    const int klane = bits == 4 ? 8 : 32;
+    if (M < 3 || M > kPackedRows || has_g_idx || gs % klane != 0 || K / klane >= 65536) return false;
+    const int groups = wave_groups_exact(kr / waves_k, gs);
+    return grouped_wavex(true, kr / waves_k) && groups >= 1 && groups <= 4;
+}
 // Input channels of x the GATHER kernel stages per K wave at a time: fixed per (bits, row tiles) so
 // that the kernel's unrolled step loop knows its chunk boundaries at compile time.  The chunk is a
 // whole number of steps that divides the weight prefetch depth (8 steps int4, 4 steps int3).

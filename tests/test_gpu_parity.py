@@ -193,6 +193,48 @@ def test_grouped_forced_split_k(dev, bits, desc_act, M, split):
 
 
 @pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("K,N,gs", [(512, 96, 128), (1024, 416, 32), (2048, 1056, 256), (4096, 352, 128), (1024, 160, -1),
+                                    (11008, 256, 128), (4096, 16480, 128)])
+@pytest.mark.parametrize("M", [3, 4])
+def test_grouped_packed_rows(dev, bits, K, N, gs, M):
+    """Three or four rows in the one operand tile of the GROUPED kernel (contiguous groups): against the
+    oracle, against the STREAM kernel on the same inputs, and with a forced split of K."""
+    L = layer(760 + K + M, K, N, bits, gs, False, M=M, bias=True)
+    D = to_dev(L, dev)
+    try:
+        plan = _lib.plan_for(_lib.KERNEL_GROUPED, M, K, N, bits, gs, False)
+    except _lib.GptqHipError as e:
+        assert e.status == _lib.ERR_UNSUPPORTED   # e.g. more than four groups in a wave's K range
+        pytest.skip("no packed-row plan for the shape")
+    assert plan.kernel == _lib.KERNEL_GROUPED and plan.row_tiles == 4
+    want = expected_output(L)
+    y = run_gemm(D, plan=plan)
+    assert_close(y, want, "packed rows")
+    assert_tight(y, want, "packed rows")
+    assert torch.equal(y, run_gemm(D, plan=plan))
+    assert_tight(y, run_gemm(D, plan=_lib.plan_for(_lib.KERNEL_STREAM, M, K, N, bits, gs, False)).cpu(), "packed rows vs STREAM")
+    assert_close(run_gemm(D), want, "dispatcher's choice")
+    for split in (2, 4):
+        try:
+            ps = _lib.plan_for(_lib.KERNEL_GROUPED, M, K, N, bits, gs, False, split_k=split)
+        except _lib.GptqHipError:
+            continue
+        ys = run_gemm(D, plan=ps)
+        assert_close(ys, want, f"packed rows split={split}")
+        assert_tight(ys, want, f"packed rows split={split}")
+
+
+def test_grouped_packed_rows_rejects_what_it_cannot_hold(dev):
+    # an activation order, or a fifth row, is outside the packed-row plans
+    with pytest.raises(_lib.GptqHipError) as e:
+        _lib.plan_for(_lib.KERNEL_GROUPED, 4, 1024, 128, 4, 128, True)
+    assert e.value.status == _lib.ERR_UNSUPPORTED
+    with pytest.raises(_lib.GptqHipError) as e:
+        _lib.plan_for(_lib.KERNEL_GROUPED, 5, 1024, 128, 4, 128, False)
+    assert e.value.status == _lib.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("bits", [3, 4])
 @pytest.mark.parametrize("desc_act", [False, True])
 @pytest.mark.parametrize("M", [1, 2])
 @pytest.mark.parametrize("N,wn", [(16480, 2), (32864, 4)])
@@ -377,7 +419,9 @@ def test_sorted_small_batch_matches_oracle(dev, bits, K, N, gs, M):
     plan = ops.sorted_plan(M, K, N, bits, gs)
     if plan is None:
         pytest.skip("not covered by the sorted path")
-    assert plan.kernel == _lib.KERNEL_STREAM and plan.row_tiles == 1
+    # (three rows may also go to the GROUPED kernel with packed rows, behind the same reordering pass)
+    assert (plan.kernel == _lib.KERNEL_STREAM and plan.row_tiles == 1) or \
+        (plan.kernel == _lib.KERNEL_GROUPED and M in (3, 4) and plan.row_tiles == 4)
     want = expected_output(L)
     y = run_sorted(D)
     assert_close(y, want, "sorted small batch")
