@@ -76,11 +76,11 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
         if (pl.k_chunk < kstep * pl.waves_k || pl.k_chunk % (kstep * pl.waves_k) != 0) return GPTQ_HIP_ERR_BAD_ARG;
         const int kr = pl.k_chunk;
         if ((long long)kr * pl.split_k < (long long)steps_total * kstep) return GPTQ_HIP_ERR_BAD_ARG;
-        if (M > 2) {
+        const bool packed = pl.row_tiles == gptq::packed_rows_of(M) && gptq::grouped_packable(bits, K, gs, act_order != 0, M, kr, pl.waves_k);
+        if (M > 2 || packed) {
             // packed rows: one operand tile, LDS and partial sums sized for four rows
-            if (pl.row_tiles != gptq::kPackedRows || !gptq::grouped_packable(bits, K, gs, act_order != 0, M, kr, pl.waves_k))
-                return GPTQ_HIP_ERR_UNSUPPORTED;
-            if (pl.lds_bytes < gptq::grouped_lds_bytes(kr, gptq::kPackedRows, 1, pl.waves_n, pl.waves_k, true))
+            if (!packed) return GPTQ_HIP_ERR_UNSUPPORTED;
+            if (pl.lds_bytes < gptq::grouped_lds_bytes(kr, gptq::packed_rows_of(M), 1, pl.waves_n, pl.waves_k, true))
                 return GPTQ_HIP_ERR_BAD_ARG;
             return GPTQ_HIP_OK;
         }
@@ -142,7 +142,9 @@ static int run_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros
     p.wave_steps = plan->kernel == GPTQ_HIP_KERNEL_GROUPED
                        ? plan->k_chunk / kstep / plan->waves_k
                        : (p.steps_total + plan->split_k * plan->waves_k - 1) / (plan->split_k * plan->waves_k);
-    p.gpad = plan->kernel == GPTQ_HIP_KERNEL_GROUPED ? (M > 2 ? 16 : 16 * (plan->row_tiles / M)) : 0;
+    const bool packed_rows = plan->kernel == GPTQ_HIP_KERNEL_GROUPED && plan->row_tiles == gptq::packed_rows_of(M) &&
+                             gptq::grouped_packable(bits, K, gs, act_order != 0, M, plan->k_chunk, plan->waves_k);
+    p.gpad = plan->kernel == GPTQ_HIP_KERNEL_GROUPED ? (packed_rows ? 16 : 16 * (plan->row_tiles / M)) : 0;
     p.xpack = nullptr;
     p.gpack = nullptr;
     p.rt_total = 0;
@@ -164,7 +166,7 @@ static int run_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros
         }
     }
     size_t ws_plan = workspace_bytes;  // bytes of the workspace the plan itself may use
-    if (kmap && (plan->kernel == GPTQ_HIP_KERNEL_STREAM || (plan->kernel == GPTQ_HIP_KERNEL_GROUPED && M > 2))) {
+    if (kmap && (plan->kernel == GPTQ_HIP_KERNEL_STREAM || packed_rows)) {
         // small batches on a sorted layer: x goes into the sorted channel order first (one small pass
         // into the tail of the workspace), then the kernel for contiguous groups reads it directly
         if (plan->kernel == GPTQ_HIP_KERNEL_STREAM &&
@@ -291,8 +293,10 @@ extern "C" size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits,
 {
     gptq_hip_plan plan;
     if (gptq_hip_select(M, K, N, bits, group_size, 0, &plan) != GPTQ_HIP_OK) return 0;
-    if ((plan.kernel == GPTQ_HIP_KERNEL_STREAM && M <= gptq::kSortedMaxRows) ||
-        (plan.kernel == GPTQ_HIP_KERNEL_GROUPED && M > 2))
+    const int gs = group_size == -1 ? K : group_size;
+    const bool packed_rows = plan.kernel == GPTQ_HIP_KERNEL_GROUPED && plan.row_tiles == gptq::packed_rows_of(M) &&
+                             gptq::grouped_packable(bits, K, gs, false, M, plan.k_chunk, plan.waves_k);
+    if ((plan.kernel == GPTQ_HIP_KERNEL_STREAM && M <= gptq::kSortedMaxRows) || packed_rows)
         return gptq::sorted_x_offset(plan.workspace_bytes) + (size_t)M * K * 2;
     return plan.workspace_bytes;
 }

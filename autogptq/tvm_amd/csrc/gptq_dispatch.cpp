@@ -234,8 +234,8 @@ bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, i
     return false;
 }
 
-// GROUPED with three or four activation rows packed into the one operand tile (contiguous groups only).
-// The plan is sized for four rows whatever M is.
+// GROUPED with up to four activation rows packed into one operand tile, or up to eight into two
+// (contiguous groups only).  The plan is sized for four or eight rows.
 bool plan_grouped_packed(int M, int K, int N, int bits, int gs, int force_split, int force_waves, gptq_hip_plan *plan)
 {
     const int kstep = gptq::kstep_of(bits);
@@ -255,10 +255,10 @@ bool plan_grouped_packed(int M, int K, int N, int bits, int gs, int force_split,
         const int split = ceil_div(steps_total, wg_steps);
         const int kr = wg_steps * kstep;
         if (!gptq::grouped_packable(bits, K, gs, false, M, kr, waves_k)) continue;
-        const int lds = gptq::grouped_lds_bytes(kr, gptq::kPackedRows, 1, waves_n, waves_k, true);
+        const int lds = gptq::grouped_lds_bytes(kr, gptq::packed_rows_of(M), 1, waves_n, waves_k, true);
         if (lds > gptq::kGroupedLdsCap) continue;
         plan->kernel = GPTQ_HIP_KERNEL_GROUPED;
-        plan->row_tiles = gptq::kPackedRows;
+        plan->row_tiles = gptq::packed_rows_of(M);
         plan->m_blocks = 1;
         plan->waves_n = waves_n;
         plan->waves_k = waves_k;
@@ -270,7 +270,7 @@ bool plan_grouped_packed(int M, int K, int N, int bits, int gs, int force_split,
         plan->block = 64 * waves_n * waves_k;
         plan->lds_bytes = lds;
         plan->workspace_bytes =
-            split > 1 ? gptq::kCounterBytes + (size_t)split * gptq::kPackedRows * N * sizeof(float) : 0;
+            split > 1 ? gptq::kCounterBytes + (size_t)split * gptq::packed_rows_of(M) * N * sizeof(float) : 0;
         return true;
     }
     return false;
@@ -390,16 +390,25 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
         }
     }
     bool packed = false;
-    if ((M == 3 || M == 4) && !act_order) {
-        // three or four rows for the matrix instructions of one (contiguous groups, short K ranges per wave)
-        gptq_hip_plan narrow;
-        memset(&narrow, 0, sizeof(narrow));
-        const bool have_narrow = plan_grouped_packed(M, K, N, bits, gs, 0, 0, &narrow);
-        const bool have_wide = wide && plan_grouped_packed(M, K, N, bits, gs, 0, wide, plan);
-        if (have_wide && (!have_narrow || plan->split_k <= narrow.split_k)) {
-            grouped = packed = true;
+    if (M >= 2 && M <= gptq::kPackedRows && !act_order) {
+        // two to four rows for the matrix instructions of one (five to eight: of two) (contiguous groups, short K ranges per wave).
+        // Against STREAM, int3 4096 x 11008: 7.9 us against 9.8 for two to four rows; int4: 8.9 against 10.2;
+        // int3 9216 x 9216 in three K ranges: 15.7 against 24.  With K cut into four or more ranges the sum
+        // across workgroups costs more than the packing saves (int4 4096 x 4096 in four: 9.0 against 8.6;
+        // 11008 x 4096 in six: 16.7 against 11.8).
+        gptq_hip_plan pn, pw;
+        memset(&pn, 0, sizeof(pn));
+        memset(&pw, 0, sizeof(pw));
+        const bool have_narrow = plan_grouped_packed(M, K, N, bits, gs, 0, 0, &pn);
+        const bool have_wide = wide && plan_grouped_packed(M, K, N, bits, gs, 0, wide, &pw);
+        const gptq_hip_plan *best = nullptr;
+        if (have_wide && (!have_narrow || pw.split_k <= pn.split_k)) {
+            best = &pw;
         } else if (have_narrow) {
-            *plan = narrow;
+            best = &pn;
+        }
+        if (best && best->split_k <= 3) {
+            *plan = *best;
             grouped = packed = true;
         }
     }
@@ -443,7 +452,7 @@ extern "C" int gptq_hip_plan_for(int kernel, int M, int K, int N, int bits, int 
     }
     if (kernel == GPTQ_HIP_KERNEL_GROUPED) {
         if (M <= 2 && plan_grouped(M, K, N, bits, gs, G, act_order, split_k, waves_n, plan)) return GPTQ_HIP_OK;
-        if ((M == 3 || M == 4) && !act_order && plan_grouped_packed(M, K, N, bits, gs, split_k, waves_n, plan))
+        if (M >= 2 && M <= gptq::kPackedRows && !act_order && plan_grouped_packed(M, K, N, bits, gs, split_k, waves_n, plan))
             return GPTQ_HIP_OK;
         memset(plan, 0, sizeof(*plan));
         return GPTQ_HIP_ERR_UNSUPPORTED;

@@ -67,8 +67,8 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     static_assert(!COMPACT || TPM == 2, "compact layout is for two row tiles");
     static_assert(!LITE || (TPM == 1 && !COMPACT), "the lite operand is one row tile of contiguous groups");
     static_assert(!WAVEX || LITE, "wave-private staging is for the lean operand");
-    static_assert(!PACK || (WAVEX && M == 4), "packed rows: four activation rows x four groups in one tile");
-    constexpr int MA = PACK ? 1 : M;  // operand tiles (and accumulator sets) per row tile
+    static_assert(!PACK || (WAVEX && (M == 4 || M == 8)), "packed rows: four activation rows x four groups per tile");
+    constexpr int MA = PACK ? M / 4 : M;  // operand tiles (and accumulator sets) per row tile
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -172,10 +172,12 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     int wpos[XP];  // where the quad's lane block starts in xlds
     if constexpr (WAVEX) {
         const int wq = wave_k / 4;  // quads per activation row in this wave's range
+        // q / wq as a multiply: exact for q < 8192 and wq <= 128 (the error term q * (wq - 1) stays below 2^20)
+        const uint32_t wq_inv = M == 1 ? 0u : ((1u << 20) + (uint32_t)wq - 1u) / (uint32_t)wq;
 #pragma unroll
         for (int ps = 0; ps < XP; ps++) {
             const int q = lane + 64 * ps;
-            const int m = M == 1 ? 0 : min(q / wq, M - 1);
+            const int m = M == 1 ? 0 : min((int)(((uint32_t)q * wq_inv) >> 20), M - 1);
             const int kc = wk * wave_k + 4 * (q - m * wq);  // position inside the workgroup's K range
             const int k = k_base + kc;
             wqv[ps] = q < M * wq && k < p.K && (!PACK || m < p.M);  // PACK: rows past p.M stay zero
@@ -449,8 +451,12 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
                         // lane i feeds row i of the tile: activation row i / 4, group i % 4 of the wave
                         const uint32_t lb = (uint32_t)((st0 + s) * 4 + lq);
                         const int row = (int)(__umulhi(lb, p.gdiv_magic) + (p.gdiv_add ? lb : 0u)) - g_base;
-                        const uint32_t off = row == (li & 3) ? (uint32_t)((li >> 2) * kspan + b8 * 8) * 2u : zero_off;
-                        a[0][0] = *(const h8 *)(smem + off);
+#pragma unroll
+                        for (int j = 0; j < MA; j++) {  // tile j: activation rows 4 j .. 4 j + 3
+                            const uint32_t off =
+                                row == (li & 3) ? (uint32_t)((4 * j + (li >> 2)) * kspan + b8 * 8) * 2u : zero_off;
+                            a[j][0] = *(const h8 *)(smem + off);
+                        }
                     } else if constexpr (LITE) {
                         // the group of this lane block, as a row of the wave's tile
                         const uint32_t lb = (uint32_t)((st0 + s) * 4 + lq);
@@ -551,7 +557,11 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
 
     // ---- 8. waves along K meet in LDS; one thread per four output columns finishes --------
     if constexpr (PACK) {
-        *(f4 *)(red + (((size_t)wk * WN + wn) * M + lq) * 64 + 4 * li) = (f4){tot[0][0], tot[0][1], tot[0][2], tot[0][3]};
+#pragma unroll
+        for (int j = 0; j < MA; j++) {
+            *(f4 *)(red + (((size_t)wk * WN + wn) * M + 4 * j + lq) * 64 + 4 * li) =
+                (f4){tot[j][0], tot[j][1], tot[j][2], tot[j][3]};
+        }
     } else if (lq == 0) {
 #pragma unroll
         for (int m = 0; m < M; m++) {
@@ -627,14 +637,15 @@ static int launch_grouped_one(const Params &p, const gptq_hip_plan &plan, hipStr
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 
-// three or four activation rows packed into one operand tile
-template <int BITS>
+// two to four activation rows packed into one operand tile (ROWS = 4), five to eight into two (ROWS = 8)
+template <int BITS, int ROWS>
 static int launch_grouped_packed(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
     constexpr int NSTEP = BITS == 4 ? 16 : 4;
-    if (p.kmap || p.xsrc || !grouped_packable(BITS, p.K, p.group_size, p.g_idx != nullptr, p.M, plan.k_chunk, plan.waves_k))
+    if (p.kmap || p.xsrc || plan.row_tiles != ROWS ||
+        !grouped_packable(BITS, p.K, p.group_size, p.g_idx != nullptr, p.M, plan.k_chunk, plan.waves_k))
         return GPTQ_HIP_ERR_UNSUPPORTED;
-    auto kern = grouped_kernel<BITS, kPackedRows, 1, false, NSTEP, true, true, true>;
+    auto kern = grouped_kernel<BITS, ROWS, 1, false, NSTEP, true, true, true>;
     const int lds_bytes = plan.lds_bytes;
     if (lds_bytes > 65536) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) !=
@@ -651,7 +662,11 @@ template <int BITS>
 static int launch_grouped_bits(const Params &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
     const int tpm = p.gpad / 16;
-    if (p.M == 3 || p.M == 4) return tpm == 1 ? launch_grouped_packed<BITS>(p, plan, stream) : GPTQ_HIP_ERR_UNSUPPORTED;
+    if (p.M > 4) return tpm == 1 ? launch_grouped_packed<BITS, 8>(p, plan, stream) : GPTQ_HIP_ERR_UNSUPPORTED;
+    if (p.M > 2) return tpm == 1 ? launch_grouped_packed<BITS, 4>(p, plan, stream) : GPTQ_HIP_ERR_UNSUPPORTED;
+    if (p.M == 2 && plan.row_tiles == packed_rows_of(2) &&
+        grouped_packable(BITS, p.K, p.group_size, p.g_idx != nullptr, p.M, plan.k_chunk, plan.waves_k))
+        return launch_grouped_packed<BITS, 4>(p, plan, stream);
     if (p.M == 1) {
         switch (tpm) {
             case 1: return launch_grouped_one<BITS, 1, 1, false>(p, plan, stream);

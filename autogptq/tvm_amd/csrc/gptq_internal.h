@@ -77,10 +77,15 @@ inline bool grouped_lite(int bits, int K, int gs, bool has_g_idx, int tpm, int M
 // channels of a sorted layer up per wave instead (two dependent round trips) loses to the shared
 // scatter with its one barrier (7.9 against 7.6 us).
 inline bool grouped_wavex(bool lite, int wave_channels) { return lite && wave_channels <= 512; }
-// Packed rows in the GROUPED kernel (three or four activation rows for the matrix instructions of one):
+// Packed rows in the GROUPED kernel (two to four activation rows for the matrix instructions of one, five
+// to eight for those of two):
 // the lean operand with wave-private staging, and at most four groups in a wave's K range, counted
-// exactly (a wave's range starts at a multiple of its length).  Such plans are sized for four rows.
-static const int kPackedRows = 4;
+// exactly (a wave's range starts at a multiple of its length).  Such plans are sized for four or eight rows and
+// say so in row_tiles; a two-row plan of the unpacked kind with four row tiles meets more than 16 groups
+// per wave and is therefore never packable, so the two cannot be mistaken for each other.
+static const int kPackedRows = 8;  // the most rows a packed plan holds
+// rows a packed plan for M activation rows is sized for (its row_tiles): one tile of four, or two
+inline int packed_rows_of(int M) { return M <= 4 ? 4 : 8; }
 inline int wave_groups_exact(int wave_channels, int gs)
 {
     if (gs % wave_channels == 0) return 1;
@@ -89,7 +94,8 @@ inline int wave_groups_exact(int wave_channels, int gs)
 inline bool grouped_packable(int bits, int K, int gs, bool has_g_idx, int M, int kr, int waves_k)
 {
     const int klane = bits == 4 ? 8 : 32;
-    if (M < 3 || M > kPackedRows || has_g_idx || gs % klane != 0 || K / klane >= 65536) return false;
+    if (M < 2 || M > kPackedRows || has_g_idx || gs % klane != 0 || K / klane >= 65536) return false;
+    if (M > 4 && waves_k < 2) return false;  // the last stage has a thread per 4 outputs of 64 columns: 128 for 8 rows
     const int groups = wave_groups_exact(kr / waves_k, gs);
     return grouped_wavex(true, kr / waves_k) && groups >= 1 && groups <= 4;
 }

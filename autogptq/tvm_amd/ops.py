@@ -163,8 +163,10 @@ def gemm_sorted(x: torch.Tensor, qweight_sorted: torch.Tensor, qzeros: torch.Ten
         if plan is None:
             raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, f"gptq_hip_gemm_sorted(M={M}, K={K}, N={N}, bits={bits})")
     ws_bytes = plan.workspace_bytes
-    if plan.kernel == _lib.KERNEL_STREAM:   # x in the sorted order goes behind what the plan itself uses
-        ws_bytes = _lib.lib().gptq_hip_sorted_workspace_bytes(M, K, N, bits, group_size)
+    if plan.kernel == _lib.KERNEL_STREAM or (plan.kernel == _lib.KERNEL_GROUPED and M >= 2):
+        # kernels that want x in the sorted order (STREAM, GROUPED with packed rows): a small pass puts it
+        # behind what the plan itself uses
+        ws_bytes = max(ws_bytes, _lib.lib().gptq_hip_sorted_workspace_bytes(M, K, N, bits, group_size))
     ws = _workspace(dev, ws_bytes) if ws_bytes else None
     with torch.cuda.device(dev):
         rc = _lib.lib().gptq_hip_gemm_sorted(

@@ -131,8 +131,8 @@ def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int =
         plan = _lib.select(M, K, N, bits, gs, desc_act)
     case["plan"] = plan
     ws_bytes = plan.workspace_bytes
-    if prepared and plan.kernel == _lib.KERNEL_STREAM:   # x in the sorted order goes behind the plan's own bytes
-        ws_bytes = _lib.lib().gptq_hip_sorted_workspace_bytes(M, K, N, bits, gs)
+    if prepared:   # kernels that want x in the sorted order find it behind the plan's own bytes
+        ws_bytes = max(ws_bytes, _lib.lib().gptq_hip_sorted_workspace_bytes(M, K, N, bits, gs))
     case["ws_bytes"] = ws_bytes
     case["ws"] = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
     return case

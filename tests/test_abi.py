@@ -52,7 +52,7 @@ def test_strerror_texts():
 
 
 @pytest.mark.parametrize("bits", [3, 4])
-@pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 64, 128, 256, 1000])
+@pytest.mark.parametrize("M", [1, 2, 3, 5, 8, 16, 17, 64, 128, 256, 1000])
 @pytest.mark.parametrize("KN", [(4096, 4096), (4096, 11008), (11008, 4096), (9216, 36864), (36864, 9216), (64, 32)])
 @pytest.mark.parametrize("gs", [128, -1])
 def test_select_plans_are_consistent(bits, M, KN, gs):
@@ -63,7 +63,11 @@ def test_select_plans_are_consistent(bits, M, KN, gs):
         p = _lib.select(M, K, N, bits, gs, act)
         assert p.kernel in (_lib.KERNEL_GATHER, _lib.KERNEL_GROUPED, _lib.KERNEL_STREAM)
         if p.kernel == _lib.KERNEL_GROUPED:
-            assert M <= 2 and 1 <= p.row_tiles <= 6 and p.m_blocks == 1
+            # one or two rows, or up to eight packed into one or two operand tiles (contiguous groups only)
+            assert M <= 8 and 1 <= p.row_tiles <= 8 and p.m_blocks == 1
+            if M > 2:
+                assert not act or gs == -1
+                assert p.row_tiles == (4 if M <= 4 else 8) and p.split_k <= 3 and p.block >= 16 * p.row_tiles
         else:
             assert p.row_tiles in (1, 2, 4, 8)
             assert p.m_blocks * 16 * p.row_tiles >= M
@@ -76,6 +80,8 @@ def test_select_plans_are_consistent(bits, M, KN, gs):
         assert p.grid_x >= 1 and p.grid_y >= 1 and p.grid_z >= 1
         if p.split_k > 1:
             assert p.workspace_bytes >= p.split_k * M * N * 4
+            if p.kernel == _lib.KERNEL_GROUPED and M > 2:   # packed rows: partial sums of all the plan's rows
+                assert p.workspace_bytes >= p.split_k * p.row_tiles * N * 4
             # partial sums stay in proportion to the packed weights (or there is a single split)
             assert p.split_k * M * N * 4 <= 3 * K * N * bits // 8 or p.split_k == 2
         elif p.kernel == _lib.KERNEL_STREAM:
@@ -185,9 +191,17 @@ def test_plan_for_forces_family_split_and_waves():
 
 
 def test_dispatcher_families_by_m():
-    # decode: GROUPED; M = 2 only while one workgroup holds all of K; batches: STREAM, direct up to 16 rows
+    # decode: GROUPED; two to four rows on contiguous groups: GROUPED with the rows packed into one operand
+    # tile (a plan sized for four rows); under an activation order M = 2 only while one workgroup holds all
+    # of K; batches: STREAM, direct up to 16 rows
     assert _lib.select(1, 4096, 11008, 4, 128, True).kernel == _lib.KERNEL_GROUPED
-    assert _lib.select(2, 4096, 11008, 4, 128, False).kernel == _lib.KERNEL_STREAM
+    for m in (2, 3, 4, 5, 8):
+        p = _lib.select(m, 4096, 11008, 4, 128, False)
+        assert p.kernel == _lib.KERNEL_GROUPED and p.row_tiles == (4 if m <= 4 else 8) and p.split_k == 1 and p.grid_x == 172
+    assert _lib.select(9, 4096, 11008, 4, 128, False).kernel == _lib.KERNEL_STREAM
+    # ... unless K would be cut into four or more ranges
+    assert _lib.select(4, 11008, 4096, 4, 128, False).kernel == _lib.KERNEL_STREAM
+    assert _lib.select(4, 4096, 11008, 4, 128, True).kernel == _lib.KERNEL_STREAM
     p = _lib.select(8, 4096, 11008, 4, 128, True)
     assert p.kernel == _lib.KERNEL_STREAM and p.row_tiles == 1 and p.workspace_bytes == 0 and p.split_k == 1
     p = _lib.select(128, 4096, 11008, 3, 128, True)

@@ -195,18 +195,24 @@ def test_grouped_forced_split_k(dev, bits, desc_act, M, split):
 @pytest.mark.parametrize("bits", [3, 4])
 @pytest.mark.parametrize("K,N,gs", [(512, 96, 128), (1024, 416, 32), (2048, 1056, 256), (4096, 352, 128), (1024, 160, -1),
                                     (11008, 256, 128), (4096, 16480, 128)])
-@pytest.mark.parametrize("M", [3, 4])
+@pytest.mark.parametrize("M", [2, 3, 4, 5, 7, 8])
 def test_grouped_packed_rows(dev, bits, K, N, gs, M):
-    """Three or four rows in the one operand tile of the GROUPED kernel (contiguous groups): against the
-    oracle, against the STREAM kernel on the same inputs, and with a forced split of K."""
+    """Two to four rows in one operand tile of the GROUPED kernel, five to eight in two (contiguous groups):
+    against the oracle, against the STREAM kernel on the same inputs, and with a forced split of K."""
     L = layer(760 + K + M, K, N, bits, gs, False, M=M, bias=True)
     D = to_dev(L, dev)
-    try:
-        plan = _lib.plan_for(_lib.KERNEL_GROUPED, M, K, N, bits, gs, False)
-    except _lib.GptqHipError as e:
-        assert e.status == _lib.ERR_UNSUPPORTED   # e.g. more than four groups in a wave's K range
-        pytest.skip("no packed-row plan for the shape")
-    assert plan.kernel == _lib.KERNEL_GROUPED and plan.row_tiles == 4
+    if M == 2:
+        # (a forced GROUPED plan for two rows is the unpacked one; the dispatcher prefers the packed one)
+        plan = _lib.select(M, K, N, bits, gs, False)
+        if not (plan.kernel == _lib.KERNEL_GROUPED and plan.row_tiles == 4):
+            pytest.skip("no packed-row plan for the shape")
+    else:
+        try:
+            plan = _lib.plan_for(_lib.KERNEL_GROUPED, M, K, N, bits, gs, False)
+        except _lib.GptqHipError as e:
+            assert e.status == _lib.ERR_UNSUPPORTED   # e.g. more than four groups in a wave's K range
+            pytest.skip("no packed-row plan for the shape")
+    assert plan.kernel == _lib.KERNEL_GROUPED and plan.row_tiles == (4 if M <= 4 else 8)
     want = expected_output(L)
     y = run_gemm(D, plan=plan)
     assert_close(y, want, "packed rows")
@@ -225,12 +231,12 @@ def test_grouped_packed_rows(dev, bits, K, N, gs, M):
 
 
 def test_grouped_packed_rows_rejects_what_it_cannot_hold(dev):
-    # an activation order, or a fifth row, is outside the packed-row plans
+    # an activation order, or a ninth row, is outside the packed-row plans
     with pytest.raises(_lib.GptqHipError) as e:
         _lib.plan_for(_lib.KERNEL_GROUPED, 4, 1024, 128, 4, 128, True)
     assert e.value.status == _lib.ERR_UNSUPPORTED
     with pytest.raises(_lib.GptqHipError) as e:
-        _lib.plan_for(_lib.KERNEL_GROUPED, 5, 1024, 128, 4, 128, False)
+        _lib.plan_for(_lib.KERNEL_GROUPED, 9, 1024, 128, 4, 128, False)
     assert e.value.status == _lib.ERR_UNSUPPORTED
 
 
@@ -421,7 +427,7 @@ def test_sorted_small_batch_matches_oracle(dev, bits, K, N, gs, M):
         pytest.skip("not covered by the sorted path")
     # (three rows may also go to the GROUPED kernel with packed rows, behind the same reordering pass)
     assert (plan.kernel == _lib.KERNEL_STREAM and plan.row_tiles == 1) or \
-        (plan.kernel == _lib.KERNEL_GROUPED and M in (3, 4) and plan.row_tiles == 4)
+        (plan.kernel == _lib.KERNEL_GROUPED and M <= 8 and plan.row_tiles == (4 if M <= 4 else 8))
     want = expected_output(L)
     y = run_sorted(D)
     assert_close(y, want, "sorted small batch")
