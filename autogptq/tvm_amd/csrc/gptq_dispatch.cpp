@@ -180,7 +180,8 @@ int grouped_lds_bytes(int kr, int M, int tpm, int waves_n, int waves_k, bool lit
 
 namespace {
 
-// GROUPED: rows expanded by group, M of 1 or 2.  Returns false when the shape does not fit
+// GROUPED: rows expanded by group, M of 1 or 2 (one set of operand tiles per activation row; the packed
+// layout for up to eight rows is plan_grouped_packed's).  Returns false when the shape does not fit
 // (too many groups for the row tiles, or an LDS operand that no split makes small enough).
 bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, int force_split, int force_waves,
                   gptq_hip_plan *plan)
@@ -390,8 +391,9 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
         }
     }
     bool packed = false;
-    if (M >= 2 && M <= gptq::kPackedRows && !act_order) {
-        // two to four rows for the matrix instructions of one (five to eight: of two) (contiguous groups, short K ranges per wave).
+    if (M >= 2 && M <= (bits == 3 ? gptq::kPackedRows : 4) && !act_order) {
+        // two to four rows for the matrix instructions of one (five to eight: of two; int4 gains nothing from
+        // two tiles: 4096 x 11008, M = 8: 11.6 us against 10.6 on STREAM, while int3 takes 9.8 against 10.5) (contiguous groups, short K ranges per wave).
         // Against STREAM, int3 4096 x 11008: 7.9 us against 9.8 for two to four rows; int4: 8.9 against 10.2;
         // int3 9216 x 9216 in three K ranges: 15.7 against 24.  With K cut into four or more ranges the sum
         // across workgroups costs more than the packing saves (int4 4096 x 4096 in four: 9.0 against 8.6;

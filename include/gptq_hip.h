@@ -37,7 +37,9 @@ typedef enum gptq_hip_status {
 /* kernel families the dispatcher chooses between */
 enum {
     GPTQ_HIP_KERNEL_GATHER = 1, /* exact fp16 weights, x staged through LDS by the workgroup; any g_idx, any M */
-    GPTQ_HIP_KERNEL_GROUPED = 2, /* rows expanded by group, scales applied once per group; M <= 2, few groups */
+    GPTQ_HIP_KERNEL_GROUPED = 2, /* rows expanded by group, scales applied once per group; M <= 2 with few groups,
+                                    or M <= 8 with contiguous groups (activation rows packed into the
+                                    operand tile: such plans have row_tiles = 4 or 8) */
     GPTQ_HIP_KERNEL_STREAM = 3  /* exact fp16 weights, independent waves along K; any g_idx, any M.  M > 16: x is
                                    pre-packed into matrix-instruction fragment order (needs the workspace);
                                    M <= 16: the kernel reads x itself.  split_k > 1 adds a reduce launch. */
@@ -115,10 +117,10 @@ int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const int32_t *qze
  *                                      kmap[K + j] = the channel whose codes are j-th along K in qweight_sorted
  * tells the kernel where each x[m, k] belongs.  x and y are in the layer's original channel order.
  * qzeros and scales are unchanged.  plan: NULL lets the dispatcher choose, else a plan for
- * (M, K, N, bits, group_size, act_order = 0) of the GROUPED family (one launch; the scatter of x into
- * LDS follows the map) or, for M <= 16, of the STREAM family with one row tile (a small pass first
- * writes x in the sorted order into the tail of the workspace, then the kernel for contiguous groups
- * runs: two or three launches).  workspace: gptq_hip_sorted_workspace_bytes, zeroed like any other.
+ * (M, K, N, bits, group_size, act_order = 0) of the GROUPED family (M <= 2 without packed rows: one
+ * launch, the scatter of x into LDS follows the map) or, for M <= 16, of the STREAM family with one row
+ * tile or of the GROUPED family with packed rows (a small pass first writes x in the sorted order into
+ * the tail of the workspace, then the kernel for contiguous groups runs: two or three launches).  workspace: gptq_hip_sorted_workspace_bytes, zeroed like any other.
  * Needs K < 65536, equal groups and group_size a multiple of 8 (int4) or 32 (int3);
  * GPTQ_HIP_ERR_UNSUPPORTED otherwise, or for larger batches (they run on the checkpoint's own
  * tensors through gptq_hip_gemm).

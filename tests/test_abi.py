@@ -195,10 +195,11 @@ def test_dispatcher_families_by_m():
     # tile (a plan sized for four rows); under an activation order M = 2 only while one workgroup holds all
     # of K; batches: STREAM, direct up to 16 rows
     assert _lib.select(1, 4096, 11008, 4, 128, True).kernel == _lib.KERNEL_GROUPED
-    for m in (2, 3, 4, 5, 8):
-        p = _lib.select(m, 4096, 11008, 4, 128, False)
+    for bits, m in [(4, 2), (4, 3), (4, 4), (3, 2), (3, 4), (3, 5), (3, 8)]:
+        p = _lib.select(m, 4096, 11008, bits, 128, False)
         assert p.kernel == _lib.KERNEL_GROUPED and p.row_tiles == (4 if m <= 4 else 8) and p.split_k == 1 and p.grid_x == 172
-    assert _lib.select(9, 4096, 11008, 4, 128, False).kernel == _lib.KERNEL_STREAM
+    assert _lib.select(5, 4096, 11008, 4, 128, False).kernel == _lib.KERNEL_STREAM   # two tiles: int3 only
+    assert _lib.select(9, 4096, 11008, 3, 128, False).kernel == _lib.KERNEL_STREAM
     # ... unless K would be cut into four or more ranges
     assert _lib.select(4, 11008, 4096, 4, 128, False).kernel == _lib.KERNEL_STREAM
     assert _lib.select(4, 4096, 11008, 4, 128, True).kernel == _lib.KERNEL_STREAM
