@@ -195,6 +195,11 @@ bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, i
     // a column tile per workgroup and no split is best (nothing crosses workgroups) unless
     // that leaves most of the 256 CUs idle
     int want = force_split > 0 ? force_split : (col_tiles >= 128 ? 1 : ceil_div(256, col_tiles));
+    // A workgroup's time is a chain of load latencies (~0.85 us per step of a wave) rather than its share of the
+    // HBM bandwidth, and the sum across workgroups costs 2-4 us: while a wave's share of an unsplit K stays within
+    // 512 channels (K <= 4096) one workgroup per column tile is faster than filling the chip, however few tiles
+    // there are (4096 x 4096 on 64 CUs: int3 6.4 us against 7.6 in four ranges, int4 7.0 against 8.2).
+    if (force_split == 0 && !act_order && ceil_div(steps_total, 8 / waves_n) * kstep <= 512) want = 1;
     if (want > steps_total) want = steps_total;
     for (int want_split = want; want_split <= steps_total && want_split <= 256; want_split++) {
         if (force_split > 0 && want_split != want) return false;
@@ -245,6 +250,7 @@ bool plan_grouped_packed(int M, int K, int N, int bits, int gs, int force_split,
     const int col_tiles = ceil_div(N, 64 * waves_n);
     if ((size_t)col_tiles * sizeof(int) > gptq::kCounterBytes) return false;
     int want = force_split > 0 ? force_split : (col_tiles >= 128 ? 1 : ceil_div(256, col_tiles));
+    if (force_split == 0 && ceil_div(steps_total, 8 / waves_n) * kstep <= 512) want = 1;  // as in plan_grouped
     if (want > steps_total) want = steps_total;
     for (int want_split = want; want_split <= steps_total && want_split <= 256; want_split++) {
         if (force_split > 0 && want_split != want) return false;

@@ -100,6 +100,13 @@ def test_select_spreads_decode_shapes_over_the_chip():
         for (K, N) in [(4096, 4096), (4096, 11008), (11008, 4096)]:
             p = _lib.select(1, K, N, bits, 128, True)
             assert p.grid_x * p.grid_y * p.grid_z >= 128, (bits, K, N, p.as_dict())
+    # contiguous groups and K <= 4096: one workgroup per column tile even when that leaves CUs idle (a
+    # workgroup's time is a chain of load latencies, and the sum across workgroups costs more than it saves)
+    for bits in (3, 4):
+        for N in (512, 4096):
+            p = _lib.select(1, 4096, N, bits, 128, False)
+            assert p.kernel == _lib.KERNEL_GROUPED and p.split_k == 1 and p.grid_x == N // 64 and p.workspace_bytes == 0
+        assert _lib.select(1, 11008, 4096, bits, 128, False).split_k > 1
     # 4096 x 11008 with 32 groups: one workgroup per 64 columns owns all of K, nothing crosses workgroups
     p = _lib.select(1, 4096, 11008, 3, 128, True)
     assert p.kernel == _lib.KERNEL_GROUPED and p.split_k == 1 and p.workspace_bytes == 0 and p.grid_x == 172
@@ -142,7 +149,8 @@ def test_entry_points_reject_null_and_bad_sizes_before_touching_the_gpu():
     assert lib.gptq_hip_gemm(fake, fake, fake, fake, null, null, fake, null, 0, 64, 4096, 11008, 4, 128,
                              null) == _lib.ERR_WORKSPACE
     # a split-K plan without a workspace
-    assert lib.gptq_hip_gemm(fake, fake, fake, fake, null, null, fake, null, 0, 1, 4096, 4096, 4, 128,
+    assert _lib.select(1, 11008, 4096, 4, 128, False).split_k > 1
+    assert lib.gptq_hip_gemm(fake, fake, fake, fake, null, null, fake, null, 0, 1, 11008, 4096, 4, 128,
                              null) == _lib.ERR_WORKSPACE
     # the sorted entry: no map, a misaligned map, a shape outside the decode family, K past the map's 16-bit positions,
     # groups that are not whole lane blocks

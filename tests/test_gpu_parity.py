@@ -436,8 +436,9 @@ def test_sorted_small_batch_matches_oracle(dev, bits, K, N, gs, M):
     # x in the sorted order sits behind the counters at the head of the shared workspace: a split-K
     # call on the same stream right after still finds them zero
     L2 = layer(931, 512, 192, bits, 128, False, M=1)
-    assert _lib.select(1, 512, 192, bits, 128, False).split_k > 1
-    assert_close(run_gemm(to_dev(L2, dev)), expected_output(L2), "split-K call after a sorted small batch")
+    p2 = _lib.plan_for(_lib.KERNEL_GROUPED, 1, 512, 192, bits, 128, False, split_k=2)
+    assert p2.split_k == 2 and p2.workspace_bytes > 0
+    assert_close(run_gemm(to_dev(L2, dev), plan=p2), expected_output(L2), "split-K call after a sorted small batch")
     with pytest.raises(_lib.GptqHipError) as e:    # larger batches are not for this entry point
         qs, kmap = pack.sort_channels_by_group(D["qweight"], D["g_idx"], bits, gs)
         x17 = torch.zeros((17, K), dtype=torch.float16, device=dev)
