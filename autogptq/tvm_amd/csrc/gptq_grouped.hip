@@ -59,7 +59,7 @@ __device__ __forceinline__ h8 and_h8(h8 a, u4 m)
 // PACK (WAVEX, at most four groups in a wave's K range, M = 4 rows of which p.M are real): row 4 m + g of
 // the ONE operand tile holds x[m] for group g of the wave, so three or four activation rows cost the
 // matrix instructions of one; lane group q of the result is activation row q, register v its group v.
-template <int BITS, int M, int TPM, bool COMPACT, int NSTEP, bool LITE, bool WAVEX = false, bool PACK = false, int PFX = 0>
+template <int BITS, int M, int TPM, bool COMPACT, int NSTEP, bool LITE, bool WAVEX = false, bool PACK = false>
 __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
 {
     using F = Fmt<BITS>;
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(512) void grouped_kernel(const Params p)
     // step being consumed (int4, 1 KB steps, 4096 x 11008: 1 ahead 9.4 us, 2: 7.9, 3: 7.5, 4: 7.45, 5: 7.6, 6: 7.8,
     // 8: 8.1, 12: 8.8, 16: 9.4; int3, 3 KB steps: 1 ahead 6.85 us, 2: 7.3, 3: 7.7, 4: 8.1): deeper queues delay
     // every wave's next request behind the others' and the waves of a workgroup drift apart.
-    constexpr int PF = PFX > 0 ? PFX : (BITS == 4 ? (LITE ? 4 : 8) : 1);
+    constexpr int PF = BITS == 4 ? (LITE ? 4 : 8) : 1;
     u4 w[NSTEP][F::WORDS];
     auto load_step = [&](int s, int st) {  // register slot s <- step st
         const int prow = 4 * st + lq;

@@ -84,10 +84,10 @@ DEFAULT_WORKLOAD = "c2-int3-4096x11008-act-m1"
 # same counter reads for a plain 256 MiB device copy); a profiler run is needed to refresh them, so
 # they are recorded here per workload.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "c2-int3-4096x11008-act-m1": 18_357 * 1024 + 22_016,        # GROUPED kernel (prepared path): read + written
-    "c3-int4-4096x11008-m4": (23_862 + 86) * 1024,               # GROUPED kernel, four packed rows
+    "c2-int3-4096x11008-act-m1": 18_356 * 1024 + 22_016,        # GROUPED kernel (prepared path): read + written
+    "c3-int4-4096x11008-m4": (23_857 + 86) * 1024,               # GROUPED kernel, four packed rows
     "int4-9216x36864-g1-m1": (167_123 + 954) * 1024,             # GROUPED kernel, 256-column workgroups
-    "c4-int4-4096x11008-act-m128": (56_363 + 2_752) * 1024,     # STREAM matmul kernel alone (pack pass: 3,154 KiB more)
+    "c4-int4-4096x11008-act-m128": (56_360 + 2_752) * 1024,     # STREAM matmul kernel alone (pack pass: 3,154 KiB more)
 }
 
 
