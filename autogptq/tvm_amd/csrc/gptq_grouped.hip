@@ -14,8 +14,8 @@
 //
 // Work split: a workgroup owns 64 * waves_n columns and one K range (all of K when
 // split_k == 1); its waves_k waves along K each take a share of that range, keep their
-// weight loads one (int3) or eight (int4) steps ahead of the matrix instructions, and meet
-// in LDS for the reduction.  With split_k == 1 nothing crosses workgroups.
+// weight loads one (int3), four (int4, lean operand) or eight (int4, tiles) steps ahead of the matrix
+// instructions, and meet in LDS for the reduction.  With split_k == 1 nothing crosses workgroups.
 //
 // LDS holds the expanded activation operand of the workgroup's K range, laid out as
 // the MFMA wants it: a tile is 16 rows x 8 slots of fp16 = 256 bytes, lane i reads its
@@ -30,8 +30,9 @@
 // LITE: with contiguous groups that are whole lane blocks (8 channels int4, 32 int3) all 8 slots
 // of an operand tile belong to one group, so the tile is "x in row r, zeros elsewhere".  LDS then
 // holds just x in unpack order (2 bytes per channel instead of 32) plus 16 zero bytes: a lane reads
-// x when its row is the block's group and the zeros otherwise.  Only x itself is zero-filled (8 KB
-// instead of 128 KB at K = 4096), and the scatter's 2-byte stores spread over the banks instead of
+// x when its row is the block's group and the zeros otherwise.  Nothing but the positions past the end
+// of K is zero-filled (instead of 128 KB of tiles at K = 4096), which the scatter never writes, so one
+// barrier (after the scatter) suffices; the scatter's 2-byte stores spread over the banks instead of
 // hitting the two banks of one tile row.  Used for int3, and for int4 where one workgroup holds all
 // of K (grouped_lite in gptq_internal.h).
 //
@@ -42,6 +43,12 @@
 // (p.kmap: one memory round trip), or looks up where the x of each of its positions comes from
 // (p.xsrc: two dependent round trips, but no scatter work on channels of other K ranges; the
 // host picks it when K is split and long).
+//
+// Wave-private staging (WAVEX: lean operand, no channel map, at most 512 channels per wave): every
+// wave loads and stages the x of its own K range, so the prologue has no workgroup barrier at all.
+// Packed rows (PACK, on top of WAVEX, at most four groups per wave): row 4 m + g of an operand tile
+// holds activation row m for group g, so up to four activation rows cost the matrix instructions of
+// one, up to eight those of two.
 #include "gptq_device.h"
 
 namespace gptq {
