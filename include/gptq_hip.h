@@ -48,7 +48,8 @@ enum {
 /* What the dispatcher decided for one problem; filled by gptq_hip_select. */
 typedef struct gptq_hip_plan {
     int kernel;             /* GPTQ_HIP_KERNEL_* */
-    int row_tiles;          /* 16-row MFMA tiles held per wave */
+    int row_tiles;          /* 16-row MFMA tiles held per wave (GROUPED with packed activation rows, M = 2..8 on
+                               contiguous groups: the rows the plan is sized for, 4 or 8) */
     int m_blocks;           /* grid extent along M */
     int waves_n;            /* waves of a workgroup laid along N (64 columns each) */
     int waves_k;            /* waves of a workgroup laid along K */
