@@ -199,7 +199,9 @@ bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, i
     // HBM bandwidth, and the sum across workgroups costs 2-4 us: while a wave's share of an unsplit K stays within
     // 512 channels (K <= 4096) one workgroup per column tile is faster than filling the chip, however few tiles
     // there are (4096 x 4096 on 64 CUs: int3 6.4 us against 7.6 in four ranges, int4 7.0 against 8.2).
-    if (force_split == 0 && !act_order && ceil_div(steps_total, 8 / waves_n) * kstep <= 512) want = 1;
+    // Under an activation order (operand tiles, two barriers) the same holds up to 256 channels per wave
+    // (2048 x 4096 int3: 5.9 us against 7.3 in four ranges; at 4096 x 4096 one range and four are level).
+    if (force_split == 0 && ceil_div(steps_total, 8 / waves_n) * kstep <= (act_order ? 256 : 512)) want = 1;
     if (want > steps_total) want = steps_total;
     for (int want_split = want; want_split <= steps_total && want_split <= 256; want_split++) {
         if (force_split > 0 && want_split != want) return false;
