@@ -34,7 +34,9 @@ ABI_SYMBOLS = (
     "gptq_hip_dequant",
     "gptq_hip_strerror",
     "gptq_hip_abi_version",
+    "gptq_hip_build_id",
 )
+ABI_VERSION = 2
 
 
 class Plan(ctypes.Structure):
@@ -105,6 +107,16 @@ def lib() -> ctypes.CDLL:
     l.gptq_hip_strerror.argtypes = [i]
     l.gptq_hip_abi_version.restype = i
     l.gptq_hip_abi_version.argtypes = []
+    l.gptq_hip_build_id.restype = ctypes.c_char_p
+    l.gptq_hip_build_id.argtypes = []
+    if l.gptq_hip_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH} has ABI version {l.gptq_hip_abi_version()}, this package expects "
+                           f"{ABI_VERSION}: rebuild it with `python -m autogptq.tvm_amd.build`")
+    from . import build as _build
+    built, now = l.gptq_hip_build_id().decode(), _build.source_hash()
+    if built != now:
+        raise RuntimeError(f"{LIB_PATH} was built from other sources (build id {built}, sources now {now}): "
+                           "rebuild it with `python -m autogptq.tvm_amd.build`")
     _lib = l
     return l
 

@@ -5,6 +5,7 @@
 """
 from __future__ import annotations
 
+import hashlib
 import json
 import os
 import shutil
@@ -35,6 +36,16 @@ def flags() -> list:
         # keep the compiler from forming packed-fp32 instructions
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     ]
+
+
+def source_hash() -> str:
+    """Digest of every source and header the library is built from; the library reports the digest it
+    was built with (gptq_hip_build_id), so a library older than its sources is noticed when it is loaded."""
+    h = hashlib.sha256()
+    for name in sorted(SOURCES + HEADERS):
+        with open(os.path.join(CSRC, name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read() + b"\0")
+    return h.hexdigest()[:16]
 
 
 def is_stale() -> bool:
@@ -68,7 +79,8 @@ def parse_resource_remarks(text: str) -> dict:
 
 
 def build(verbose: bool = False) -> str:
-    cmd = ([hipcc()] + flags() + ["-Rpass-analysis=kernel-resource-usage", "-o", LIB] +
+    cmd = ([hipcc()] + flags() + [f'-DGPTQ_HIP_BUILD_ID="{source_hash()}"',
+                                   "-Rpass-analysis=kernel-resource-usage", "-o", LIB] +
            [os.path.join(CSRC, s) for s in SOURCES])
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     report = parse_resource_remarks(proc.stdout)

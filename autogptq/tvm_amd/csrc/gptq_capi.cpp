@@ -53,8 +53,7 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
         return GPTQ_HIP_ERR_UNSUPPORTED;
     if (pl.kernel == GPTQ_HIP_KERNEL_GATHER) {
         if (pl.waves_n * pl.waves_k > 4) return GPTQ_HIP_ERR_UNSUPPORTED;
-        if (pl.row_tiles != 1 && pl.row_tiles != 2 && pl.row_tiles != 4 && pl.row_tiles != 8)
-            return GPTQ_HIP_ERR_UNSUPPORTED;
+        if (pl.row_tiles != 1 && pl.row_tiles != 2 && pl.row_tiles != 4) return GPTQ_HIP_ERR_UNSUPPORTED;
         if (pl.k_chunk < kstep || pl.k_chunk % kstep != 0) return GPTQ_HIP_ERR_BAD_ARG;
         if (pl.m_blocks * 16 * pl.row_tiles < M || pl.grid_z != pl.m_blocks) return GPTQ_HIP_ERR_BAD_ARG;
         if (pl.split_k * pl.waves_k > steps_total && pl.split_k * pl.waves_k > 1) return GPTQ_HIP_ERR_BAD_ARG;
@@ -202,6 +201,8 @@ static int run_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros
         const size_t part =
             plan->split_k > 1 ? ((size_t)plan->split_k * M * N * sizeof(float) + 255) / 256 * 256 : 0;
         p.direct = gptq::stream_direct(bits, K, plan->row_tiles, p.act_table, g_idx != nullptr);
+        // the kernel that reads x itself covers one tile of 16 rows and ignores the grid's M extent
+        if (plan->row_tiles == 1 && (M > 16 || plan->m_blocks != 1)) return GPTQ_HIP_ERR_BAD_ARG;
         p.gdiv_magic = 0;
         p.gdiv_add = 0;
         if (p.direct) {
@@ -234,8 +235,10 @@ static int run_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros
         return gptq::launch_stream(p, bits, *plan, stream);
     }
     if (plan->split_k > 1) {
-        const size_t need = gptq::kCounterBytes + (size_t)plan->split_k * M * N * sizeof(float);
-        if (!workspace || workspace_bytes < need || !aligned(workspace, 16)) return GPTQ_HIP_ERR_WORKSPACE;
+        // a packed-row plan indexes its partial sums by the rows it is sized for (4 or 8), not by M
+        const size_t part_rows = packed_rows ? (size_t)gptq::packed_rows_of(M) : (size_t)M;
+        const size_t need = gptq::kCounterBytes + (size_t)plan->split_k * part_rows * N * sizeof(float);
+        if (!workspace || ws_plan < need || !aligned(workspace, 16)) return GPTQ_HIP_ERR_WORKSPACE;
         p.counters = (int *)workspace;
         p.partial = (float *)((char *)workspace + gptq::kCounterBytes);
     }
@@ -346,4 +349,9 @@ extern "C" const char *gptq_hip_strerror(int status)
     }
 }
 
-extern "C" int gptq_hip_abi_version(void) { return 1; }
+extern "C" int gptq_hip_abi_version(void) { return GPTQ_HIP_ABI_VERSION; }
+
+#ifndef GPTQ_HIP_BUILD_ID
+#define GPTQ_HIP_BUILD_ID "unknown"
+#endif
+extern "C" const char *gptq_hip_build_id(void) { return GPTQ_HIP_BUILD_ID; }

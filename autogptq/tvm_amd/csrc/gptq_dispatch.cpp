@@ -22,7 +22,7 @@ int plan_gather(int M, int K, int N, int bits, int G, int force_split, int force
 {
     // the tallest tile that fits; shorter tiles (more M blocks) when LDS or staging registers
     // cannot hold it, e.g. with hundreds of groups in the (scale, zero) table
-    int rt = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8));
+    int rt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);  // (128-row tiles spilled)
     for (; rt >= 1; rt >>= 1) {
         memset(plan, 0, sizeof(*plan));
         const int rc = plan_gather_rt(rt, M, K, N, bits, G, force_split, force_waves, plan);
@@ -107,9 +107,8 @@ namespace gptq {
 // Row tiles (of 16 groups) per activation row that the GROUPED kernel is built for.
 int grouped_tpm(int groups, int M)
 {
-    int tpm = ceil_div(groups, 16);
-    if (tpm == 5) tpm = 6;
-    const int max_tpm = M == 1 ? 6 : 2;
+    const int tpm = ceil_div(groups, 16);
+    const int max_tpm = M == 1 ? 4 : 2;  // (a six-tile instantiation spilled 60-70 registers and lost to STREAM)
     return tpm <= max_tpm ? tpm : 0;
 }
 

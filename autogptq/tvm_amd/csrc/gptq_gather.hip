@@ -428,7 +428,6 @@ static int launch_gather_rt(const Params &p, const gptq_hip_plan &plan, hipStrea
         case 1: return launch_gather_one<BITS, 1, ACT>(p, plan, stream);
         case 2: return launch_gather_one<BITS, 2, ACT>(p, plan, stream);
         case 4: return launch_gather_one<BITS, 4, ACT>(p, plan, stream);
-        case 8: return launch_gather_one<BITS, 8, ACT>(p, plan, stream);
         default: return GPTQ_HIP_ERR_UNSUPPORTED;
     }
 }

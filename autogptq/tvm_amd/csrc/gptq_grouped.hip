@@ -684,7 +684,6 @@ static int launch_grouped_bits(const Params &p, const gptq_hip_plan &plan, hipSt
             case 2: return launch_grouped_one<BITS, 1, 2, true>(p, plan, stream);
             case 3: return launch_grouped_one<BITS, 1, 3, false>(p, plan, stream);
             case 4: return launch_grouped_one<BITS, 1, 4, false>(p, plan, stream);
-            case 6: return launch_grouped_one<BITS, 1, 6, false>(p, plan, stream);
             default: return GPTQ_HIP_ERR_UNSUPPORTED;
         }
     }

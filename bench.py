@@ -79,16 +79,27 @@ WORKLOADS = {
     "int3-8192x28672-act-m1": (3, 8192, 28672, 128, True, 1),
 }
 DEFAULT_WORKLOAD = "c2-int3-4096x11008-act-m1"
+# timed in the default run next to the headline: the int4 decode product and the M = 128 products of the
+# same 4096 x 11008 activation-order layer (the metric is quoted on all of them)
+SECONDARY_WORKLOADS = ("int4-4096x11008-act-m1", "c4-int4-4096x11008-act-m128", "c4-int3-4096x11008-act-m128")
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the
-# same counter reads for a plain 256 MiB device copy); a profiler run is needed to refresh them, so
-# they are recorded here per workload.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {
-    "c2-int3-4096x11008-act-m1": 18_356 * 1024 + 22_016,        # GROUPED kernel (prepared path): read + written
-    "c3-int4-4096x11008-m4": (23_857 + 86) * 1024,               # GROUPED kernel, four packed rows
-    "int4-9216x36864-g1-m1": (167_123 + 954) * 1024,             # GROUPED kernel, 256-column workgroups
-    "c4-int4-4096x11008-act-m128": (56_360 + 2_752) * 1024,     # STREAM matmul kernel alone (pack pass: 3,154 KiB more)
-}
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the same
+# counter reads for a plain 256 MiB device copy): profiles/traffic.json holds, per workload, the bytes, the
+# kernel they were measured on and the summary under profiles/ they come from.  A workload without an entry,
+# or whose entry names another kernel plan than the one timed here, reports null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def measured_traffic(workload: str, plan_kernel: int):
+    try:
+        with open(TRAFFIC_FILE, encoding="utf-8") as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None, None
+    e = table.get(workload)
+    if not e or e.get("plan_kernel") != plan_kernel:
+        return None, None
+    return int(e["fetch_bytes"]) + int(e["write_bytes"]), e.get("source")
 
 
 def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int = 0, prepared: bool = False):
@@ -176,10 +187,22 @@ def make_step(case, dev):
     return step
 
 
+_scrub = {}
+
+
+def scrub_cache(dev):
+    """Overwrites twice the Infinity Cache with zeros, so that nothing a later step reads is still cached."""
+    if dev not in _scrub:
+        _scrub[dev] = torch.empty(2 * INFINITY_CACHE_BYTES, dtype=torch.uint8, device=dev)
+    _scrub[dev].zero_()
+
+
 def time_case(case, dev, steps: int, warmup: int):
     """Average duration of one step in microseconds: K steps captured once in a HIP graph and
-    replayed inside one event-bracketed region (no host launch cost between the kernels), plus
-    the same K steps launched eagerly for comparison."""
+    replayed inside one event-bracketed region (no host launch cost between the kernels; reported as
+    ``graph_us`` and as ``us``), plus the same K steps launched eagerly (``eager_us``).  The weight copy
+    of step i is (warmup + i) mod copies, continuing the warm-up's rotation, and the cache is scrubbed
+    before every timed region, so no timed step finds its weights cached."""
     step = make_step(case, dev)
     stream = torch.cuda.Stream(device=dev)
     res = {}
@@ -187,13 +210,14 @@ def time_case(case, dev, steps: int, warmup: int):
         sp = ctypes.c_void_p(stream.cuda_stream)
         for i in range(warmup):
             step(i, sp)
+        scrub_cache(dev)
         stream.synchronize()
         # eager
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize(dev)
         e0.record(stream)
         for i in range(steps):
-            step(i, sp)
+            step(warmup + i, sp)
         e1.record(stream)
         torch.cuda.synchronize(dev)
         res["eager_us"] = e0.elapsed_time(e1) * 1e3 / steps
@@ -203,12 +227,13 @@ def time_case(case, dev, steps: int, warmup: int):
         with torch.cuda.graph(g, stream=stream):
             spg = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
             for i in range(steps):
-                step(i, spg)
+                step(warmup + i, spg)
         g.replay()
         torch.cuda.synchronize(dev)
         times = []
         for _ in range(3):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            scrub_cache(dev)
             torch.cuda.synchronize(dev)
             e0.record()
             g.replay()
@@ -218,7 +243,7 @@ def time_case(case, dev, steps: int, warmup: int):
         res["graph_us"] = min(times)
     except Exception as exc:  # graph capture unavailable: report the eager figure only
         res["graph_error"] = repr(exc)[:200]
-    res["us"] = min(v for k, v in res.items() if k in ("eager_us", "graph_us"))
+    res["us"] = res.get("graph_us", res["eager_us"])
     return res
 
 
@@ -250,6 +275,20 @@ def summarize(case, t):
     out["plan"] = {k: v for k, v in case["plan"].as_dict().items()
                    if k in ("kernel", "row_tiles", "waves_n", "waves_k", "split_k", "grid_x", "grid_y", "grid_z")}
     return out
+
+
+def roofline_of(name: str, s: dict) -> dict:
+    """The roofline object of one timed workload: HBM-bound for decode sizes (M <= 8), MFMA-bound above."""
+    M = WORKLOADS[name][5]
+    traffic, source = measured_traffic(name, s["plan"]["kernel"])
+    if M <= 8:
+        r = {"bound": "hbm", "achieved": s["weight_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s["hbm_frac"]}
+    else:
+        r = {"bound": "mfma", "achieved": s["TFLOPs"], "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
+             "frac": s["mfma_frac"], "hbm_frac": s["hbm_frac"]}
+    r["traffic"] = traffic
+    r["traffic_source"] = source
+    return r
 
 
 def cpu_baseline(case, budget_s: float = 20.0):
@@ -287,6 +326,7 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument("--sweep", action="store_true", help="also time every workload in WORKLOADS")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true", help="default workload only: skip the secondary records")
     ap.add_argument("--unprepared", action="store_true",
                     help="decode on activation-order layers: time gptq_hip_gemm on the checkpoint's tensors "
                          "instead of gptq_hip_gemm_sorted on the load-time prepared ones")
@@ -348,13 +388,26 @@ def main():
         "timing": {k: s[k] for k in ("eager_us", "graph_us", "graph_error", "unprepared_us") if k in s},
         "hbm_frac": s["hbm_frac"], "tflops": s["TFLOPs"],
     }
-    if gemv:
-        line["roofline"] = {"bound": "hbm", "achieved": s["weight_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                            "frac": s["hbm_frac"], "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
-    else:
-        line["roofline"] = {"bound": "mfma", "achieved": s["TFLOPs"], "peak": MFMA_FP16_PEAK_TFLOPS,
-                            "unit": "TFLOP/s", "frac": s["mfma_frac"],
-                            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
+    line["roofline"] = roofline_of(args.workload, s)
+    if args.workload == DEFAULT_WORKLOAD and not forced and not args.unprepared and not args.no_secondary:
+        # the other halves of the metric, each a timed record of its own with its roofline and parity
+        secondary = []
+        for name in SECONDARY_WORKLOADS:
+            prep = prepared_applies(name)
+            c = build_case(name, dev, prepared=prep)
+            okc, errc = check_case(c, dev)
+            r = summarize(c, time_case(c, dev, args.steps, args.warmup))
+            secondary.append({
+                "workload": name, "value": r["us"], "unit": "us", "steps": args.steps, "warmup": args.warmup,
+                "timing": {k: r[k] for k in ("eager_us", "graph_us", "graph_error") if k in r},
+                "entry": "gptq_hip_gemm_sorted" if prep else "gptq_hip_gemm_plan", "plan": r["plan"],
+                "hbm_frac": r["hbm_frac"], "tflops": r["TFLOPs"], "mfma_frac": r["mfma_frac"],
+                "roofline": roofline_of(name, r),
+                "parity": {"ok": okc, "max_abs_err": round(errc, 6), "rtol": 1e-2, "atol": 1e-2},
+            })
+            del c
+            torch.cuda.empty_cache()
+        line["secondary"] = secondary
     if args.sweep:
         sweep = []
         for name, prep in [(n, pr) for n in sorted(WORKLOADS) for pr in (False, True)]:

@@ -160,8 +160,13 @@ int gptq_hip_dequant(const int32_t *qweight, const int32_t *qzeros, const void *
 /* Human-readable text for a gptq_hip_status. */
 const char *gptq_hip_strerror(int status);
 
-/* ABI version of this library (bumped when a signature changes). */
+/* ABI version of this library (bumped when a signature or gptq_hip_plan changes). */
+#define GPTQ_HIP_ABI_VERSION 2
 int gptq_hip_abi_version(void);
+
+/* Digest of the sources this library was built from (set by the build script; "unknown" otherwise), so that a
+ * loader can tell a library that is older than the sources beside it. */
+const char *gptq_hip_build_id(void);
 
 #ifdef __cplusplus
 }

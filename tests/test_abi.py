@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(_lib.ABI_SYMBOLS)
     for name in names:
         assert getattr(lib, name) is not None
-    assert lib.gptq_hip_abi_version() == 1
+    assert lib.gptq_hip_abi_version() == _lib.ABI_VERSION
 
 
 def test_plan_struct_matches_header():
@@ -152,6 +152,23 @@ def test_entry_points_reject_null_and_bad_sizes_before_touching_the_gpu():
     assert _lib.select(1, 11008, 4096, 4, 128, False).split_k > 1
     assert lib.gptq_hip_gemm(fake, fake, fake, fake, null, null, fake, null, 0, 1, 11008, 4096, 4, 128,
                              null) == _lib.ERR_WORKSPACE
+    # packed rows with K split: the partial sums are indexed by the rows the plan is sized for (4 or 8), so a
+    # workspace sized for the real M is refused
+    pk = _lib.plan_for(_lib.KERNEL_GROUPED, 2, 2048, 320, 4, 128, False, split_k=2)
+    pk3 = _lib.plan_for(_lib.KERNEL_GROUPED, 3, 2048, 320, 4, 128, False, split_k=2)
+    for M, pl in ((3, pk3),):
+        assert pl.row_tiles == 4 and pl.split_k == 2
+        small = 16384 + pl.split_k * M * 320 * 4
+        assert small < pl.workspace_bytes
+        assert lib.gptq_hip_gemm_plan(fake, fake, fake, fake, null, null, fake, fake, small, M, 2048, 320, 4, 128,
+                                      ctypes.byref(pl), null) == _lib.ERR_WORKSPACE
+    del pk
+    # a hand-edited STREAM plan: one row tile but several M blocks (the kernel that reads x itself covers 16 rows)
+    ps = _lib.plan_for(_lib.KERNEL_STREAM, 16, 4096, 352, 4, 128, False)
+    assert ps.row_tiles == 1 and ps.m_blocks == 1
+    ps.m_blocks, ps.grid_z = 2, 2
+    assert lib.gptq_hip_gemm_plan(fake, fake, fake, fake, null, null, fake, fake, 1 << 24, 32, 4096, 352, 4, 128,
+                                  ctypes.byref(ps), null) == _lib.ERR_BAD_ARG
     # the sorted entry: no map, a misaligned map, a shape outside the decode family, K past the map's 16-bit positions,
     # groups that are not whole lane blocks
     srt = lib.gptq_hip_gemm_sorted

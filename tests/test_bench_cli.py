@@ -32,5 +32,17 @@ def test_workload_table_covers_the_baseline_configurations():
     assert bench.WORKLOADS["c1-int4-4096x4096-m1"] == (4, 4096, 4096, 128, False, 1)  # configs[0]
     assert any(v[5] == 128 and v[4] for v in bench.WORKLOADS.values())     # act-order GEMM at M = 128
     assert any(v[3] == -1 and v[1] == 36864 for v in bench.WORKLOADS.values())  # OPT-66B long K
-    for name in bench.MEASURED_TRAFFIC_BYTES:
+    for name in bench.SECONDARY_WORKLOADS:
         assert name in names
+    # the measured-traffic table names workloads that exist and the profile summaries its figures come from
+    import json
+    with open(bench.TRAFFIC_FILE) as f:
+        table = json.load(f)
+    for name, e in table.items():
+        assert name in names
+        assert os.path.exists(os.path.join(ROOT, e["source"])), e["source"]
+        assert e["fetch_bytes"] > 0 and e["write_bytes"] >= 0
+    total, source = bench.measured_traffic("c2-int3-4096x11008-act-m1", table["c2-int3-4096x11008-act-m1"]["plan_kernel"])
+    assert total == table["c2-int3-4096x11008-act-m1"]["fetch_bytes"] + table["c2-int3-4096x11008-act-m1"]["write_bytes"]
+    assert source.startswith("profiles/")
+    assert bench.measured_traffic("c2-int3-4096x11008-act-m1", 99) == (None, None)   # another kernel than the one measured

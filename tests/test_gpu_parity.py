@@ -297,14 +297,18 @@ def test_gemm_does_not_write_outside_y(dev):
 
 # ------------------------------------------------------------------ the benchmark configurations
 FULL = [
-    # (name, bits, K, N, gs, desc_act, Ms)
-    ("c1-int4-4096x4096", 4, 4096, 4096, 128, False, [1]),
+    # (name, bits, K, N, gs, desc_act, Ms): every shape x M of the benchmark configurations
+    ("c1-int4-4096x4096", 4, 4096, 4096, 128, False, [1, 2, 4, 8]),
     ("c2-int3-4096x11008-act", 3, 4096, 11008, 128, True, [1]),
     ("c3-int4-4096x11008", 4, 4096, 11008, 128, False, [1, 2, 4, 8]),
-    ("c3-int4-11008x4096", 4, 11008, 4096, 128, False, [1, 8]),
-    ("c4-int4-4096x11008-act", 4, 4096, 11008, 128, True, [16, 128]),
-    ("c4-int3-11008x4096-act", 3, 11008, 4096, 128, True, [64, 256]),
+    ("c3-int4-11008x4096", 4, 11008, 4096, 128, False, [1, 2, 4, 8]),
+    ("c4-int4-4096x11008-act", 4, 4096, 11008, 128, True, [16, 64, 128, 256]),
+    ("c4-int3-4096x11008-act", 3, 4096, 11008, 128, True, [16, 64, 128, 256]),
+    ("c4-int4-11008x4096-act", 4, 11008, 4096, 128, True, [16, 64, 128, 256]),
+    ("c4-int3-11008x4096-act", 3, 11008, 4096, 128, True, [16, 64, 128, 256]),
     ("c5-int3-9216x9216-act-g1", 3, 9216, 9216, -1, True, [1, 32]),
+    ("c5-int3-9216x36864-act-g1", 3, 9216, 36864, -1, True, [1, 32]),
+    ("c5-int3-36864x9216-act-g1", 3, 36864, 9216, -1, True, [1, 32]),
 ]
 
 
@@ -413,6 +417,27 @@ def test_sorted_decode_matches_oracle_and_unsorted_kernel(dev, bits, K, N, gs, M
     assert_tight(y, want, "sorted decode")
     assert torch.equal(y, run_sorted(D))
     assert_tight(y, run_gemm(D).cpu(), "sorted vs unsorted kernel")
+
+
+@pytest.mark.parametrize("K,N", [(4096, 11008), (11008, 4096)])
+def test_sorted_path_at_full_size(dev, K, N):
+    """The benchmark's own path at its own size: gptq_hip_gemm_sorted on the 3-bit activation-order layer,
+    decode and small batches, against the oracle and against the unsorted kernels; two calls must agree."""
+    bits, gs = 3, 128
+    L = layer(7100 + K // 1000, K, N, bits, gs, True, M=16)
+    D = to_dev(L, dev)
+    w16 = expected_weight(L)
+    qs, kmap = ops.sort_channels(D["qweight"], D["g_idx"], bits, gs)
+    for M in (1, 2, 8, 16):
+        x = L["x"][:M].contiguous()
+        xd = x.to(dev)
+        assert ops.sorted_plan(M, K, N, bits, gs) is not None
+        y = ops.gemm_sorted(xd, qs, D["qzeros"], D["scales"], kmap, None, bits, gs)
+        want = expected_output(L, x=x, w16=w16)
+        assert_close(y, want, f"sorted {K}x{N} M={M}")
+        assert_tight(y, want, f"sorted {K}x{N} M={M}")
+        assert torch.equal(y, ops.gemm_sorted(xd, qs, D["qzeros"], D["scales"], kmap, None, bits, gs))
+        assert_tight(y, run_gemm(D, x=xd).cpu(), f"sorted vs unsorted {K}x{N} M={M}")
 
 
 @pytest.mark.parametrize("bits", [3, 4])
