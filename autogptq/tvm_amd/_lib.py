@@ -28,6 +28,8 @@ ABI_SYMBOLS = (
     "gptq_hip_workspace_init",
     "gptq_hip_gemm",
     "gptq_hip_gemm_plan",
+    "gptq_hip_gemm_static",
+    "gptq_hip_static_workspace_limit",
     "gptq_hip_gemm_sorted",
     "gptq_hip_sorted_workspace_bytes",
     "gptq_hip_sort_channels",
@@ -95,6 +97,10 @@ def lib() -> ctypes.CDLL:
     l.gptq_hip_gemm.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, vp]
     l.gptq_hip_gemm_plan.restype = i
     l.gptq_hip_gemm_plan.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
+    l.gptq_hip_gemm_static.restype = i
+    l.gptq_hip_gemm_static.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
+    l.gptq_hip_static_workspace_limit.restype = sz
+    l.gptq_hip_static_workspace_limit.argtypes = []
     l.gptq_hip_gemm_sorted.restype = i
     l.gptq_hip_gemm_sorted.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
     l.gptq_hip_sorted_workspace_bytes.restype = sz

@@ -15,7 +15,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(CSRC, "libgptq_hip.so")
-SOURCES = ["gptq_gather.hip", "gptq_stream.hip", "gptq_grouped.hip", "gptq_dequant.hip", "gptq_dispatch.cpp", "gptq_capi.cpp"]
+SOURCES = ["gptq_gather.hip", "gptq_stream.hip", "gptq_grouped.hip", "gptq_dequant.hip", "gptq_static.hip", "gptq_dispatch.cpp", "gptq_capi.cpp"]
 HEADERS = ["gptq_unpack.h", "gptq_internal.h", "gptq_device.h", os.path.join("..", "..", "..", "include", "gptq_hip.h")]
 
 

@@ -109,6 +109,21 @@ int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const int32_t *qze
                        int M, int K, int N, int bits, int group_size, const gptq_hip_plan *plan, void *stream);
 
 /*
+ * gptq_hip_gemm without a workspace argument and without any allocation.  No counterpart in the reference:
+ * it is for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  The workspace is an array of gptq_hip_static_workspace_limit() bytes
+ * (16 MiB) inside the library, one copy per GPU, held until the process ends.  A problem whose plan needs more
+ * returns GPTQ_HIP_ERR_WORKSPACE (use gptq_hip_gemm with a workspace of your own).  Every call on a GPU uses that
+ * GPU's one array: calls that overlap on the same GPU (different streams or threads) race; calls on one
+ * stream, or otherwise ordered, are fine.  The first call on a device looks the array's address up and zeroes
+ * its counters with a fill kernel on `stream`.
+ */
+int gptq_hip_gemm_static(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                         const int32_t *g_idx, const void *bias, void *y, int M, int K, int N, int bits,
+                         int group_size, void *stream);
+size_t gptq_hip_static_workspace_limit(void);
+
+/*
  * The decode product (one row, or a batch of up to 16) for a layer prepared when it was loaded: an activation-order g_idx makes
  * every weight look its group up (qlinear.py:200-242 gathers scales and zeros by g_idx), so the
  * loader sorts the input channels by group once; qweight_sorted holds the same codes with groups
