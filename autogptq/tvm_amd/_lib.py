@@ -20,6 +20,7 @@ ERR_LAUNCH = -4
 KERNEL_GATHER = 1
 KERNEL_GROUPED = 2
 KERNEL_STREAM = 3
+KERNEL_TILED = 4
 
 ABI_SYMBOLS = (
     "gptq_hip_select",
@@ -33,6 +34,10 @@ ABI_SYMBOLS = (
     "gptq_hip_gemm_sorted",
     "gptq_hip_sorted_workspace_bytes",
     "gptq_hip_sort_channels",
+    "gptq_hip_tiled_bytes",
+    "gptq_hip_tile_prepare",
+    "gptq_hip_select_tiled",
+    "gptq_hip_gemm_tiled",
     "gptq_hip_dequant",
     "gptq_hip_strerror",
     "gptq_hip_abi_version",
@@ -107,6 +112,14 @@ def lib() -> ctypes.CDLL:
     l.gptq_hip_sorted_workspace_bytes.argtypes = [i, i, i, i, i]
     l.gptq_hip_sort_channels.restype = i
     l.gptq_hip_sort_channels.argtypes = [vp, vp, vp, vp, i, i, i, i, vp]
+    l.gptq_hip_tiled_bytes.restype = sz
+    l.gptq_hip_tiled_bytes.argtypes = [i, i, i]
+    l.gptq_hip_tile_prepare.restype = i
+    l.gptq_hip_tile_prepare.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
+    l.gptq_hip_select_tiled.restype = i
+    l.gptq_hip_select_tiled.argtypes = [i, i, i, i, i, ctypes.POINTER(Plan)]
+    l.gptq_hip_gemm_tiled.restype = i
+    l.gptq_hip_gemm_tiled.argtypes = [vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
     l.gptq_hip_dequant.restype = i
     l.gptq_hip_dequant.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
     l.gptq_hip_strerror.restype = ctypes.c_char_p
@@ -136,6 +149,14 @@ def select(M: int, K: int, N: int, bits: int, group_size: int, act_order: bool) 
     rc = lib().gptq_hip_select(M, K, N, bits, group_size, int(bool(act_order)), ctypes.byref(plan))
     if rc != OK:
         raise GptqHipError(rc, f"gptq_hip_select(M={M}, K={K}, N={N}, bits={bits}, group_size={group_size})")
+    return plan
+
+
+def select_tiled(M: int, K: int, N: int, bits: int, group_size: int) -> Plan:
+    plan = Plan()
+    rc = lib().gptq_hip_select_tiled(M, K, N, bits, group_size, ctypes.byref(plan))
+    if rc != OK:
+        raise GptqHipError(rc, f"gptq_hip_select_tiled(M={M}, K={K}, N={N}, bits={bits}, group_size={group_size})")
     return plan
 
 

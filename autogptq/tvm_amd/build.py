@@ -15,7 +15,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(CSRC, "libgptq_hip.so")
-SOURCES = ["gptq_gather.hip", "gptq_stream.hip", "gptq_grouped.hip", "gptq_dequant.hip", "gptq_static.hip", "gptq_dispatch.cpp", "gptq_capi.cpp"]
+SOURCES = ["gptq_gather.hip", "gptq_stream.hip", "gptq_grouped.hip", "gptq_dequant.hip", "gptq_static.hip", "gptq_tiled.hip", "gptq_dispatch.cpp", "gptq_capi.cpp"]
 HEADERS = ["gptq_unpack.h", "gptq_internal.h", "gptq_device.h", os.path.join("..", "..", "..", "include", "gptq_hip.h")]
 
 
@@ -78,15 +78,28 @@ def parse_resource_remarks(text: str) -> dict:
     return res
 
 
-def build(verbose: bool = False) -> str:
-    cmd = ([hipcc()] + flags() + [f'-DGPTQ_HIP_BUILD_ID="{source_hash()}"',
-                                   "-Rpass-analysis=kernel-resource-usage", "-o", LIB] +
-           [os.path.join(CSRC, s) for s in SOURCES])
-    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    report = parse_resource_remarks(proc.stdout)
+def _compile_one(src: str, obj: str, build_id: str):
+    cmd = [hipcc()] + [f for f in flags() if f != "-shared"] + [
+        f'-DGPTQ_HIP_BUILD_ID="{build_id}"', "-Rpass-analysis=kernel-resource-usage", "-c", "-o", obj, src]
+    return subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+
+
+def build(verbose: bool = False, jobs: int = 0) -> str:
+    """Compiles every source to an object file (in parallel, at most 8 at a time) and links the library."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    build_id = source_hash()
+    objdir = os.path.join(CSRC, "build")
+    os.makedirs(objdir, exist_ok=True)
+    pairs = [(os.path.join(CSRC, s), os.path.join(objdir, os.path.splitext(s)[0] + ".o")) for s in SOURCES]
+    jobs = jobs or min(8, len(pairs), os.cpu_count() or 1)
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        procs = list(pool.map(lambda so: _compile_one(so[0], so[1], build_id), pairs))
+    text = "\n".join(p.stdout for p in procs)
+    report = parse_resource_remarks(text)
     noise = ("is not a recognized feature", "remark:", "-Rpass-analysis")
     lines, skip = [], 0
-    for l in proc.stdout.splitlines():
+    for l in text.splitlines():
         if skip:          # the two source-echo lines that follow every remark
             skip -= 1
             continue
@@ -95,8 +108,12 @@ def build(verbose: bool = False) -> str:
         if not any(n in l for n in noise):
             lines.append(l)
     out = "\n".join(lines)
-    if proc.returncode != 0:
+    if any(p.returncode != 0 for p in procs):
         raise RuntimeError("hipcc failed:\n" + out)
+    link = subprocess.run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + [o for _, o in pairs],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if link.returncode != 0:
+        raise RuntimeError("link failed:\n" + link.stdout)
     with open(REPORT, "w", encoding="utf-8") as f:   # registers, scratch and spills per kernel
         json.dump(report, f, indent=1, sort_keys=True)
     spilled = sorted(k for k, v in report.items() if v.get("vgpr_spill", 0) or v.get("scratch", 0))

@@ -304,6 +304,65 @@ extern "C" size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits,
     return plan.workspace_bytes;
 }
 
+extern "C" size_t gptq_hip_tiled_bytes(int K, int N, int bits)
+{
+    if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0 || (bits != 3 && bits != 4)) return 0;
+    return (size_t)((K + 63) / 64 * 64) * (size_t)N * bits / 8;
+}
+
+extern "C" int gptq_hip_tile_prepare(const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                                     const int32_t *g_idx, void *qtile, uint32_t *sz, int32_t *xsrc, int K, int N,
+                                     int bits, int group_size, void *stream)
+{
+    if (!qtile || !sz || !xsrc || (const void *)qweight == qtile) return GPTQ_HIP_ERR_BAD_ARG;
+    const int rc = check_common(qweight, qzeros, scales, K, N, bits, group_size);
+    if (rc != GPTQ_HIP_OK) return rc;
+    if (!aligned(qtile, 16) || !aligned(sz, 4) || !aligned(xsrc, 16) || (g_idx && !aligned(g_idx, 4)))
+        return GPTQ_HIP_ERR_BAD_ARG;
+    const int gs = group_size == -1 ? K : group_size;
+    if (!gptq::tiled_qualifies(K, N, bits, gs)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    return gptq::launch_tile_prepare((const uint32_t *)qweight, (const uint32_t *)qzeros, scales, g_idx, (uint32_t *)qtile,
+                                     sz, xsrc, K, N, K / gs, bits, gs, stream);
+}
+
+extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint32_t *sz, const int32_t *xsrc,
+                                   const void *bias, void *y, void *workspace, size_t workspace_bytes, int M, int K,
+                                   int N, int bits, int group_size, const gptq_hip_plan *plan, void *stream)
+{
+    if (!x || !qtile || !sz || !y || M < 1) return GPTQ_HIP_ERR_BAD_ARG;
+    if (bits != 3 && bits != 4) return GPTQ_HIP_ERR_BAD_ARG;
+    if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;
+    if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
+    if (!aligned(x, 16) || !aligned(qtile, 16) || !aligned(sz, 4) || !aligned(y, 8) || (bias && !aligned(bias, 8)) ||
+        (xsrc && !aligned(xsrc, 16)))
+        return GPTQ_HIP_ERR_BAD_ARG;
+    const int gs = group_size == -1 ? K : group_size;
+    if (!gptq::tiled_qualifies(K, N, bits, gs)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    if ((long long)((K + 63) / 64 * 64) * N * bits / 8 >= (1LL << 32)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    gptq_hip_plan chosen;
+    if (!plan) {
+        const int rc = gptq_hip_select_tiled(M, K, N, bits, group_size, &chosen);
+        if (rc != GPTQ_HIP_OK) return rc;
+        plan = &chosen;
+    }
+    // the plan must be one this family runs, sized for this problem
+    const int at = plan->row_tiles;
+    const int S_total = (K + 63) / 64;
+    if (plan->kernel != GPTQ_HIP_KERNEL_TILED || (at != 1 && at != 2 && at != 4)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    if (plan->block != 256 || plan->waves_k != 4 || plan->split_k < 1 || plan->k_chunk < 1 || plan->m_blocks < 1 ||
+        plan->grid_x != (N / 32 + 1) / 2 || plan->grid_y != plan->split_k || plan->grid_z != plan->m_blocks ||
+        (long long)plan->m_blocks * 32 * at < M || (long long)plan->split_k * 4 * plan->k_chunk < S_total ||
+        plan->lds_bytes < 4 * at * 2 * 4096 || plan->lds_bytes > 160 * 1024)
+        return GPTQ_HIP_ERR_BAD_ARG;
+    if (plan->split_k > 1 && (long long)M * N >= (1LL << 32)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    const size_t part = plan->split_k > 1 ? ((size_t)plan->split_k * M * N * sizeof(float) + 255) / 256 * 256 : 0;
+    const size_t xb = (size_t)gptq::tiled_pack_blocks(plan->split_k, plan->k_chunk, at) * 4 * (size_t)(at * plan->m_blocks) * 1024;
+    if (!workspace || !aligned(workspace, 16) || workspace_bytes < gptq::kCounterBytes + part + xb) return GPTQ_HIP_ERR_WORKSPACE;
+    float *partial = (float *)((char *)workspace + gptq::kCounterBytes);
+    char *xpack = (char *)workspace + gptq::kCounterBytes + part;
+    return gptq::launch_tiled(x, qtile, sz, xsrc, bias, y, xpack, partial, M, K, N, K / gs, bits, gs, *plan, stream);
+}
+
 extern "C" int gptq_hip_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                              const int32_t *g_idx, const void *bias, void *y, void *workspace,
                              size_t workspace_bytes, int M, int K, int N, int bits, int group_size, void *stream)

@@ -469,6 +469,52 @@ extern "C" int gptq_hip_plan_for(int kernel, int M, int K, int N, int bits, int 
     return GPTQ_HIP_ERR_UNSUPPORTED;
 }
 
+// TILED: a workgroup per 64 columns and block of 32 * row_tiles rows, four waves along K; workgroups along K
+// when the column tiles alone leave most CUs idle (their fp32 tiles cross the workspace, so the split stays
+// within 3x the packed weights of traffic).
+extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan)
+{
+    if (!plan) return GPTQ_HIP_ERR_BAD_ARG;
+    memset(plan, 0, sizeof(*plan));
+    if (bits != 3 && bits != 4) return GPTQ_HIP_ERR_BAD_ARG;
+    if (M < 1 || K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;
+    if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
+    const int gs = group_size == -1 ? K : group_size;
+    if (!gptq::tiled_qualifies(K, N, bits, gs)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    const int at = gptq::tiled_row_tiles(M);
+    const int m_blocks = ceil_div(M, 32 * at);
+    const int col_pairs = ceil_div(N / 32, 2);
+    const int S_total = ceil_div(K, 64);
+    const long long tiles = (long long)col_pairs * m_blocks;
+    int split = (int)((256 + tiles / 2) / tiles);
+    if (split < 1) split = 1;
+    int cap = (int)((3LL * K * bits) / (128LL * M));
+    if (cap < 1) cap = 1;
+    if (split > cap) split = cap;
+    if ((long long)M * N >= (1LL << 32)) split = 1;  // indexing of the pass that adds the partial tiles
+    // every wave gets at least a ring of blocks
+    while (split > 1 && S_total / (split * 4) < gptq::tiled_ring(at)) split--;
+    const int wave_steps = ceil_div(S_total, split * 4);
+    split = ceil_div(S_total, wave_steps * 4);
+    plan->kernel = GPTQ_HIP_KERNEL_TILED;
+    plan->row_tiles = at;
+    plan->m_blocks = m_blocks;
+    plan->waves_n = 1;
+    plan->waves_k = 4;
+    plan->split_k = split;
+    plan->k_chunk = wave_steps;  // blocks of 64 positions per wave
+    plan->grid_x = col_pairs;
+    plan->grid_y = split;
+    plan->grid_z = m_blocks;
+    plan->block = 256;
+    plan->lds_bytes = 4 * at * 2 * 4096;
+    size_t ws = gptq::kCounterBytes;
+    if (split > 1) ws += ((size_t)split * M * N * sizeof(float) + 255) / 256 * 256;
+    ws += (size_t)gptq::tiled_pack_blocks(split, wave_steps, at) * 4 * (size_t)(at * m_blocks) * 1024;
+    plan->workspace_bytes = ws;
+    return GPTQ_HIP_OK;
+}
+
 extern "C" size_t gptq_hip_workspace_bytes(int M, int K, int N, int bits, int group_size, int act_order)
 {
     gptq_hip_plan plan;

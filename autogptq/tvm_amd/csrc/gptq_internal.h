@@ -167,4 +167,24 @@ inline size_t sorted_x_offset(size_t plan_bytes)
     return (head + 255) / 256 * 256;
 }
 
+
+// ---- TILED family (a layer re-laid by gptq_hip_tile_prepare) ----------------------------------------
+// blocks (64 positions) the register rings of a wave run ahead, by 32-row tiles per wave: the taller the
+// tile the longer a block takes, and the fewer blocks cover the memory latency
+constexpr int tiled_ring(int at) { return at >= 4 ? 3 : (at == 2 ? 4 : 6); }
+// 32-row tiles a wave holds for M rows
+inline int tiled_row_tiles(int M) { return M <= 32 ? 1 : (M <= 64 ? 2 : 4); }
+// blocks of x the pack pass writes: what the waves of all K ranges walk, plus the ring their refills run ahead
+inline int tiled_pack_blocks(int split_k, int wave_steps, int at) { return split_k * 4 * wave_steps + tiled_ring(at); }
+inline bool tiled_qualifies(int K, int N, int bits, int gs)
+{
+    return (bits == 3 || bits == 4) && K % 32 == 0 && N % 32 == 0 && gs % 32 == 0 && K % gs == 0;
+}
+int launch_tile_prepare(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
+                        uint32_t *qtile, uint32_t *sz, int32_t *xsrc, int K, int N, int G, int bits, int group_size,
+                        void *stream);
+int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int32_t *xsrc, const void *bias, void *y,
+                 char *xpack, float *partial, int M, int K, int N, int G, int bits, int group_size,
+                 const gptq_hip_plan &plan, void *stream);
+
 }  // namespace gptq

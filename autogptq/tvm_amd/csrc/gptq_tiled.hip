@@ -1,0 +1,475 @@
+// TILED kernel family: the product on a layer that was re-laid once, when it was loaded, into the
+// order the matrix instructions consume (gptq_hip_tile_prepare), for any number of rows of x.
+//
+// The tiled format (also stated in torch ops by pack.tile_layout, which the tests compare with):
+//   * the input channels are sorted by group (stable; the identity without an activation order), so
+//     position p of the sorted order holds channel xsrc[p] and its group is p / group_size;
+//   * qtile is a sequence of blocks, column tile T (32 columns) outermost, then block S (64 positions);
+//     block (T, S) is 64 lanes x BITS words, exactly one coalesced wave load.  Lane (n = lane % 32,
+//     h = lane / 32) holds the 32 codes of column 32 T + n at positions 64 S + 32 h .. + 31, permuted
+//     inside the lane so that the register unpack of gptq_unpack.h yields them in position order:
+//     the lane's words are the B operand of four v_mfma_f32_32x32x16_f16 (positions 8 j .. 8 j + 7 of
+//     the lane for j = 0..3) with no shuffle;
+//   * sz[g][n] = (fp16 scale, fp16 zero point) of group g, column n, one 32-bit word.
+//
+// tiled_gemm_kernel: a workgroup owns 64 columns (two tiles), 32 * AT rows of x and one K range; its
+// four waves (one per SIMD) split that range and never talk until the end.  A wave holds the whole
+// 32 AT x 64 result in registers, dequantises every weight of its range exactly once, as the reference
+// does (fp16(scale * (q - zero)), one rounding), and reads x as ready-made A fragments that a small
+// pack pass wrote (rows past M and positions past K as zeros).  One wave per SIMD overlaps its own
+// vector and matrix instructions: the dequantisation of the next B operand is interleaved with the
+// matrix instructions of the current one.  Weights and fragments ride in register rings RING blocks
+// deep, requested in the order they are consumed (loads return in order, one counter).
+// The four waves add their tiles through LDS at the end; workgroups along K (split_k > 1) leave fp32
+// tiles in the workspace for reduce_kernel.
+#include "gptq_device.h"
+
+namespace gptq {
+
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+struct alignas(4) W3 {
+    uint32_t a, b, c;
+};
+
+// ---------------------------------------------------------------------------------------------------
+// Preparation, pass 1: xsrc[p] = the channel at position p of the stable sort by group (the rank of a
+// channel inside its group is the number of earlier channels of the same group), -1 for p >= K.
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void tile_map_kernel(const int32_t *__restrict__ g_idx, int32_t *__restrict__ xsrc,
+                                                       int K, int Kp, int G, int group_size)
+{
+    __shared__ int tile[256];
+    const int k = blockIdx.x * 256 + threadIdx.x;
+    if (!g_idx) {
+        if (k < Kp) xsrc[k] = k < K ? k : -1;
+        return;
+    }
+    const int g = k < K ? min(max(g_idx[k], 0), G - 1) : -1;
+    int rank = 0;
+    for (int t0 = 0; t0 <= (int)blockIdx.x * 256; t0 += 256) {
+        const int j = t0 + threadIdx.x;
+        __syncthreads();
+        tile[threadIdx.x] = j < K ? min(max(g_idx[j], 0), G - 1) : -2;
+        __syncthreads();
+        const int upto = min(256, k - t0);
+        for (int i = 0; i < upto; i++) rank += tile[i] == g ? 1 : 0;
+    }
+    if (k < K) {
+        // a group with more than group_size members would leave its range: keep every index in bounds
+        xsrc[g * group_size + min(rank, group_size - 1)] = k;
+    } else if (k < Kp) {
+        xsrc[k] = -1;
+    }
+}
+
+// Pass 2: one thread per (column tile, block, lane) gathers its 32 codes through xsrc and writes its words.
+template <int BITS>
+__global__ __launch_bounds__(256) void tile_retile_kernel(const uint32_t *__restrict__ qweight,
+                                                          const int32_t *__restrict__ xsrc, uint32_t *__restrict__ qtile,
+                                                          int K, int N, int S_total, int T_total)
+{
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    const int lane = t & 63;
+    const uint32_t blk = t >> 6;  // T * S_total + S
+    if (blk >= (uint32_t)T_total * (uint32_t)S_total) return;
+    const int T = blk / S_total, S = blk - T * S_total;
+    const int n = 32 * T + (lane & 31), h = lane >> 5;
+    uint32_t words[BITS];
+#pragma unroll
+    for (int i = 0; i < BITS; i++) words[i] = 0u;
+    for (int s = 0; s < 32; s++) {
+        const int src = xsrc[64 * S + 32 * h + s];
+        uint32_t q = 0u;
+        if (src >= 0 && src < K) {
+            const uint32_t *b = qweight + (size_t)(src >> 5) * BITS * N + n;  // the packed block of 32 channels
+            const int bit = BITS * (src & 31);
+            const int wd = bit >> 5, sh = bit & 31;
+            q = b[(size_t)wd * N] >> sh;
+            if (sh + BITS > 32) q |= b[(size_t)(wd + 1) * N] << (32 - sh);
+            q &= (1u << BITS) - 1u;
+        }
+        // the stream field that the register unpack hands out as position s
+        const int field = BITS == 4 ? (s & ~7) + SLOT4[s & 7] : SLOT3[s];
+        const int obit = BITS * field;
+        const int owd = obit >> 5, osh = obit & 31;
+        words[owd] |= q << osh;
+        if (osh + BITS > 32) words[owd + 1] |= q >> (32 - osh);
+    }
+#pragma unroll
+    for (int i = 0; i < BITS; i++) qtile[((size_t)blk * 64 + lane) * BITS + i] = words[i];
+}
+
+// Pass 3: sz[g][n] = fp16 scale | fp16 zero point << 16.
+template <int BITS>
+__global__ __launch_bounds__(256) void tile_sz_kernel(const uint32_t *__restrict__ qzeros,
+                                                      const _Float16 *__restrict__ scales, uint32_t *__restrict__ sz,
+                                                      int N, int G)
+{
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= (uint32_t)G * (uint32_t)N) return;
+    const int g = t / N, n = t - g * N;
+    const int z = zero_of<BITS>(qzeros + (size_t)g * (N / 32 * BITS), n);
+    const h2 v = {scales[t], (_Float16)(float)z};
+    sz[t] = as_u32(v);
+}
+
+int launch_tile_prepare(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
+                        uint32_t *qtile, uint32_t *sz, int32_t *xsrc, int K, int N, int G, int bits, int group_size,
+                        void *stream_v)
+{
+    hipStream_t stream = (hipStream_t)stream_v;
+    const int Kp = (K + 63) / 64 * 64;
+    const int S_total = Kp / 64, T_total = N / 32;
+    hipLaunchKernelGGL(tile_map_kernel, dim3((Kp + 255) / 256), dim3(256), 0, stream, g_idx, xsrc, K, Kp, G, group_size);
+    const unsigned threads = (unsigned)T_total * (unsigned)S_total * 64u;
+    const unsigned szt = (unsigned)G * (unsigned)N;
+    if (bits == 4) {
+        hipLaunchKernelGGL(tile_retile_kernel<4>, dim3((threads + 255u) / 256u), dim3(256), 0, stream, qweight, xsrc, qtile,
+                           K, N, S_total, T_total);
+        hipLaunchKernelGGL(tile_sz_kernel<4>, dim3((szt + 255u) / 256u), dim3(256), 0, stream, qzeros,
+                           (const _Float16 *)scales, sz, N, G);
+    } else {
+        hipLaunchKernelGGL(tile_retile_kernel<3>, dim3((threads + 255u) / 256u), dim3(256), 0, stream, qweight, xsrc, qtile,
+                           K, N, S_total, T_total);
+        hipLaunchKernelGGL(tile_sz_kernel<3>, dim3((szt + 255u) / 256u), dim3(256), 0, stream, qzeros,
+                           (const _Float16 *)scales, sz, N, G);
+    }
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Pack pass: x [M, K] -> A fragments of v_mfma_f32_32x32x16_f16.  Fragment (block S, j, row tile rt) is
+// 64 lanes x 16 bytes; lane (m = lane % 32, h = lane / 32) holds x[32 rt + m][xsrc[64 S + 32 h + 8 j + e]],
+// e = 0..7.  Rows past M and positions past K are zeros; blocks up to S_pack are written (the kernel's
+// waves walk whole ranges, and their refills run a ring past the end).
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void tile_pack_x_kernel(const _Float16 *__restrict__ x, const int32_t *__restrict__ xsrc,
+                                                          char *__restrict__ xpack, int M, int K, int Kp, int rt_total,
+                                                          int S_pack)
+{
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    const int lane = t & 63;
+    const uint32_t frag = t >> 6;
+    if (frag >= (uint32_t)S_pack * 4u * (uint32_t)rt_total) return;
+    const uint32_t sj = frag / rt_total;
+    const int rt = frag - sj * rt_total;
+    const int S = sj >> 2, j = sj & 3;
+    const int row = 32 * rt + (lane & 31);
+    const int p0 = 64 * S + 32 * (lane >> 5) + 8 * j;
+    h8 o = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (row < M && p0 < Kp) {
+        const _Float16 *xr = x + (size_t)row * K;
+        if (xsrc) {
+            const int4 a = *(const int4 *)(xsrc + p0);
+            const int4 b = *(const int4 *)(xsrc + p0 + 4);
+            const int idx[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const _Float16 v = xr[min((uint32_t)max(idx[e], 0), (uint32_t)K - 1u)];  // a bad map must not fault
+                o[e] = idx[e] >= 0 ? v : (_Float16)0;
+            }
+        } else if (p0 < K) {  // K is a multiple of 32: a run of 8 is inside or outside as a whole
+            o = *(const h8 *)(xr + p0);
+        }
+    }
+    *(h8 *)(xpack + (size_t)frag * 1024 + lane * 16) = o;
+}
+
+// ---------------------------------------------------------------------------------------------------
+struct TiledParams {
+    const char *xpack;     // A fragments, [S_pack * 4][rt_total][64 lanes][16 bytes]
+    const char *qtile;     // [T_total][S_total][64 lanes][BITS words]
+    const uint32_t *sz;    // [G][N]
+    const void *bias;      // fp16 [N] or nullptr
+    void *y;               // fp16 [M, N]
+    float *partial;        // [split_k][M][N] when split_k > 1
+    int M, N, G;
+    int S_total, T_total;
+    int wave_steps;        // blocks per wave
+    int rt_total;          // 32-row tiles over all M blocks
+    int split_k;
+    int lb_per_group;      // group_size / 32
+};
+
+// One B operand: positions 8 j .. 8 j + 7 of the lane, as fp16(scale * (q - zero)) exactly as the
+// reference rounds it: (base + q) - (base + zero) is exact, the product rounds once.
+template <int BITS>
+__device__ __forceinline__ h8 tiled_bop(const uint32_t (&w)[BITS], int j, h2 s2, h2 zb_a, h2 zb_b, uint32_t magic_a,
+                                        uint32_t magic_b)
+{
+    u4 q;
+    if constexpr (BITS == 4) {
+        u4 tmp[1];
+        biased4(w[j], tmp, magic_a, magic_b);
+        q = tmp[0];
+    } else {
+        biased3_block(w[0], w[1], w[2], j, q, magic_a, magic_b);
+    }
+    u4 o;
+#pragma unroll
+    for (int r = 0; r < 4; r++) o[r] = as_u32((as_h2(q[r]) - ((r & 1) ? zb_b : zb_a)) * s2);
+    return __builtin_bit_cast(h8, o);
+}
+
+template <int BITS, int AT, int RING>
+__global__ __launch_bounds__(256) void tiled_gemm_kernel(const TiledParams p)
+{
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, h = lane >> 5;
+    const int T0 = 2 * blockIdx.x;
+    const int split = blockIdx.y;
+    const int rt0 = blockIdx.z * AT;
+    const int S_begin = (split * 4 + wave) * p.wave_steps;
+    const int S_last = p.S_total - 1;
+    const int lb_last = 2 * p.S_total - 1;
+
+    // per-lane offsets that never change; the block number lives in scalar registers
+    uint32_t tile_off[2], col[2];
+#pragma unroll
+    for (int ct = 0; ct < 2; ct++) {
+        const int T = min(T0 + ct, p.T_total - 1);  // a missing second tile repeats the first; it is never stored
+        tile_off[ct] = (uint32_t)T * (uint32_t)p.S_total;
+        col[ct] = (uint32_t)(32 * T + n);
+    }
+    const uint32_t b_lane = (uint32_t)lane * (4u * BITS);
+    const uint32_t a_lane = (uint32_t)rt0 * 1024u + (uint32_t)lane * 16u;
+    const uint32_t a_frag_row = (uint32_t)p.rt_total * 1024u;  // bytes between consecutive (S, j)
+
+    uint32_t w[RING][2][BITS];
+    uint32_t szr[RING][2];
+    h8 a[RING][4][AT];
+    auto load_b = [&](int S, uint32_t (&wr)[2][BITS], uint32_t (&sr)[2]) {
+        const int Sc = min(S, S_last);  // blocks past K repeat the last one (their x is zero)
+        const uint32_t lb = (uint32_t)min(2 * S + h, lb_last);
+        const uint32_t g = min(lb / (uint32_t)p.lb_per_group, (uint32_t)p.G - 1u);
+#pragma unroll
+        for (int ct = 0; ct < 2; ct++) {
+            const char *src = p.qtile + ((size_t)(tile_off[ct] + (uint32_t)Sc) * (256u * BITS) + b_lane);
+            if constexpr (BITS == 4) {
+                const u4 v = __builtin_nontemporal_load((const u4 *)src);
+                wr[ct][0] = v[0];
+                wr[ct][1] = v[1];
+                wr[ct][2] = v[2];
+                wr[ct][3] = v[3];
+            } else {
+                const W3 v = *(const W3 *)src;
+                wr[ct][0] = v.a;
+                wr[ct][1] = v.b;
+                wr[ct][2] = v.c;
+            }
+            sr[ct] = p.sz[(size_t)g * p.N + col[ct]];
+        }
+    };
+    auto load_a = [&](int S, int j, h8 (&ar)[AT]) {
+        const char *src = p.xpack + (size_t)(4 * S + j) * a_frag_row + a_lane;
+#pragma unroll
+        for (int rt = 0; rt < AT; rt++) ar[rt] = __builtin_bit_cast(h8, *(const u4 *)(src + rt * 1024));
+    };
+
+    // prologue, in consumption order
+#pragma unroll
+    for (int u = 0; u < RING; u++) {
+        load_b(S_begin + u, w[u], szr[u]);
+#pragma unroll
+        for (int j = 0; j < 4; j++) load_a(S_begin + u, j, a[u][j]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    f16v acc[AT][2];
+#pragma unroll
+    for (int rt = 0; rt < AT; rt++)
+#pragma unroll
+        for (int ct = 0; ct < 2; ct++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[rt][ct][v] = 0.f;
+
+    const uint32_t magic_a = opaque_vgpr(BITS == 4 ? MAGIC4_LO : MAGIC3_EVEN);
+    const uint32_t magic_b = opaque_vgpr(BITS == 4 ? MAGIC4_HI : MAGIC3_ODD);
+    // (base + zero) per register kind: even registers of an operand carry bases (BASE[0], BASE[1]), odd (BASE[2], BASE[3])
+    const h2 base_a = BITS == 4 ? (h2){(_Float16)1024.f, (_Float16)1024.f} : (h2){(_Float16)1024.f, (_Float16)256.f};
+    const h2 base_b = BITS == 4 ? (h2){(_Float16)64.f, (_Float16)64.f} : (h2){(_Float16)128.f, (_Float16)32.f};
+    auto consts_of = [&](uint32_t e, h2 &s2, h2 &za, h2 &zb) {
+        const h2 v = as_h2(e);
+        s2 = (h2){v[0], v[0]};
+        const h2 z2 = {v[1], v[1]};
+        za = z2 + base_a;  // exact: small integers
+        zb = z2 + base_b;
+    };
+
+    // the first operand of the walk
+    h2 cs[2], cza[2], czb[2];  // (scale, base + zero) of the block being dequantised, per column tile
+    consts_of(szr[0][0], cs[0], cza[0], czb[0]);
+    h8 bop_next = tiled_bop<BITS>(w[0][0], 0, cs[0], cza[0], czb[0], magic_a, magic_b);
+
+    for (int i0 = 0; i0 < p.wave_steps; i0 += RING) {
+#pragma unroll
+        for (int u = 0; u < RING; u++) {
+            if (i0 + u >= p.wave_steps) break;  // (no load sits behind this branch)
+            const int S = S_begin + i0 + u;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++) {
+                    const h8 bop = bop_next;
+                    // the operand of the next (j, ct) of the walk, dequantised while this one multiplies
+                    {
+                        const int jn = ct == 1 ? (j + 1) & 3 : j;
+                        const int ctn = ct ^ 1;
+                        const int un = (ct == 1 && j == 3) ? (u + 1) % RING : u;
+                        if (jn == 0) consts_of(szr[un][ctn], cs[ctn], cza[ctn], czb[ctn]);  // first operand of a block
+                        bop_next = tiled_bop<BITS>(w[un][ctn], jn, cs[ctn], cza[ctn], czb[ctn], magic_a, magic_b);
+                    }
+#pragma unroll
+                    for (int rt = 0; rt < AT; rt++) {
+                        acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[u][j][rt], bop, acc[rt][ct], 0, 0, 0);
+                    }
+                    if (ct == 1) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (j == 3) load_b(S + RING, w[u], szr[u]);  // (its last reader, the operand of (3, 1), is done)
+                        load_a(S + RING, j, a[u][j]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- the four waves meet in LDS: [wave][tile rt * 2 + ct][v][lane] floats ----------------------
+    float *red = (float *)smem;
+    {
+        float *dst = red + (size_t)wave * (AT * 2) * 1024 + lane;
+#pragma unroll
+        for (int rt = 0; rt < AT; rt++)
+#pragma unroll
+            for (int ct = 0; ct < 2; ct++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) dst[((rt * 2 + ct) * 16 + v) * 64] = acc[rt][ct][v];
+    }
+    __syncthreads();
+    // one item = four adjacent columns of one row: element v of lane (n, h) of tile (rt, ct) is row
+    // 32 rt + 8 (v / 4) + 4 h + v % 4, column 32 ct + n
+    const int m0 = 32 * rt0;
+    const _Float16 *bias = (const _Float16 *)p.bias;
+    _Float16 *y = (_Float16 *)p.y;
+#pragma unroll
+    for (int it = 0; it < 2 * AT; it++) {
+        const int item = tid + 256 * it;
+        const int r = item >> 4, c4 = (item & 15) * 4;
+        const int ct = c4 >> 5, nn = c4 & 31;
+        const int rt = r >> 5, rr = r & 31;
+        const int v = 4 * (rr >> 3) + (rr & 3), hh = (rr >> 2) & 1;
+        const float *src = red + ((size_t)(rt * 2 + ct) * 16 + v) * 64 + hh * 32 + nn;
+        f4 sum = *(const f4 *)src;
+#pragma unroll
+        for (int wv = 1; wv < 4; wv++) sum += *(const f4 *)(src + (size_t)wv * (AT * 2) * 1024);
+        const int row = m0 + r;
+        const int T = T0 + ct;
+        if (row < p.M && T < p.T_total) {
+            const size_t o = (size_t)row * p.N + 32 * T + nn;
+            if (p.split_k == 1) {
+                if (bias) {
+                    const h4 b4 = *(const h4 *)(bias + 32 * T + nn);
+#pragma unroll
+                    for (int c = 0; c < 4; c++) sum[c] += (float)b4[c];
+                }
+                h4 ov;
+#pragma unroll
+                for (int c = 0; c < 4; c++) ov[c] = (_Float16)sum[c];
+                *(h4 *)(y + o) = ov;
+            } else {
+                *(f4 *)(p.partial + (size_t)split * p.M * p.N + o) = sum;
+            }
+        }
+    }
+}
+
+// y = fp16(sum over split of partial[split] (+ bias)), four columns per thread, in split order.
+__global__ __launch_bounds__(256) void tiled_reduce_kernel(const float *__restrict__ partial, const _Float16 *bias,
+                                                           _Float16 *__restrict__ y, int M, int N, int split_k)
+{
+    const uint32_t q = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t nq = (uint32_t)N / 4u;
+    if (q >= (uint32_t)M * nq) return;
+    const uint32_t row = q / nq;
+    const uint32_t c = 4u * (q - row * nq);
+    f4 sum = {0.f, 0.f, 0.f, 0.f};
+    if (bias) {
+        const h4 b4 = *(const h4 *)(bias + c);
+        sum = (f4){(float)b4[0], (float)b4[1], (float)b4[2], (float)b4[3]};
+    }
+    for (int s = 0; s < split_k; s++) sum += *(const f4 *)(partial + ((size_t)s * M + row) * N + c);
+    h4 o;
+#pragma unroll
+    for (int e = 0; e < 4; e++) o[e] = (_Float16)sum[e];
+    *(h4 *)(y + (size_t)row * N + c) = o;
+}
+
+template <int BITS, int AT, int RING>
+static int launch_tiled_one(const TiledParams &p, const gptq_hip_plan &plan, hipStream_t stream)
+{
+    auto kern = tiled_gemm_kernel<BITS, AT, RING>;
+    const int lds_bytes = 4 * AT * 2 * 4096;
+    if (plan.lds_bytes < lds_bytes) return GPTQ_HIP_ERR_BAD_ARG;
+    if (lds_bytes > 65536) {
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return GPTQ_HIP_ERR_LAUNCH;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, plan.grid_z), dim3(256), lds_bytes, stream, p);
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+}
+
+// x is packed into the workspace, the matmul runs, and a reduce pass follows when K is split over workgroups.
+int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int32_t *xsrc, const void *bias, void *y,
+                 char *xpack, float *partial, int M, int K, int N, int G, int bits, int group_size,
+                 const gptq_hip_plan &plan, void *stream_v)
+{
+    hipStream_t stream = (hipStream_t)stream_v;
+    const int Kp = (K + 63) / 64 * 64;
+    TiledParams p;
+    p.xpack = xpack;
+    p.qtile = (const char *)qtile;
+    p.sz = sz;
+    p.bias = bias;
+    p.y = y;
+    p.partial = partial;
+    p.M = M;
+    p.N = N;
+    p.G = G;
+    p.S_total = Kp / 64;
+    p.T_total = N / 32;
+    p.wave_steps = plan.k_chunk;
+    p.rt_total = plan.row_tiles * plan.m_blocks;
+    p.split_k = plan.split_k;
+    p.lb_per_group = group_size / 32;
+    const int S_pack = tiled_pack_blocks(plan.split_k, plan.k_chunk, plan.row_tiles);
+    const unsigned threads = (unsigned)S_pack * 4u * (unsigned)p.rt_total * 64u;
+    hipLaunchKernelGGL(tile_pack_x_kernel, dim3((threads + 255u) / 256u), dim3(256), 0, stream, (const _Float16 *)x, xsrc,
+                       xpack, M, K, Kp, p.rt_total, S_pack);
+    if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ERR_LAUNCH;
+    int rc = GPTQ_HIP_ERR_UNSUPPORTED;
+#define GPTQ_TILED_CASE(B, A)                                                                  \
+    if (bits == B && plan.row_tiles == A)                                                      \
+        rc = launch_tiled_one<B, A, tiled_ring(A)>(p, plan, stream)
+    GPTQ_TILED_CASE(4, 1);
+    GPTQ_TILED_CASE(4, 2);
+    GPTQ_TILED_CASE(4, 4);
+    GPTQ_TILED_CASE(3, 1);
+    GPTQ_TILED_CASE(3, 2);
+    GPTQ_TILED_CASE(3, 4);
+#undef GPTQ_TILED_CASE
+    if (rc != GPTQ_HIP_OK) return rc;
+    if (plan.split_k > 1) {
+        const uint32_t quads = (uint32_t)M * ((uint32_t)N / 4u);
+        hipLaunchKernelGGL(tiled_reduce_kernel, dim3((quads + 255u) / 256u), dim3(256), 0, stream, partial,
+                           (const _Float16 *)bias, (_Float16 *)y, M, N, plan.split_k);
+        if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ERR_LAUNCH;
+    }
+    return GPTQ_HIP_OK;
+}
+
+}  // namespace gptq

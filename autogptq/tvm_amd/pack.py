@@ -148,6 +148,74 @@ def sort_channels_by_group(qweight: torch.Tensor, g_idx: torch.Tensor, bits: int
     return qweight_sorted.contiguous(), kmap.contiguous()
 
 
+TILE_COLS = 32     # columns of one tile of the tiled format: the N extent of one 32x32x16 matrix instruction
+TILE_CHANNELS = 64  # input channels of one block of the tiled format: two lane halves x 32 codes
+
+
+def tiled_qualifies(K: int, N: int, bits: int, group_size: int) -> bool:
+    """Layers the tiled format covers: 3 or 4 bits, whole groups made of whole 32-channel lane blocks."""
+    gs = K if group_size == -1 else group_size
+    return bits in (3, 4) and K % 32 == 0 and N % 32 == 0 and gs % 32 == 0 and K % gs == 0
+
+
+def tile_layout(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor, g_idx, bits: int, group_size: int):
+    """The load-time re-layout for the tiled kernels, in torch ops (the statement the library's own
+    preparation, ``gptq_hip_tile_prepare``, is tested against; the reference's TVM module re-lays its
+    weights once in the same spirit, auto_gptq/nn_modules/qlinear_tvm.py:25-40,105-107).
+
+    Returns ``(qtile int32 [N/32 * Kp/64 * 64 * bits], sz int32 [G, N], xsrc int32 [Kp])`` with
+    Kp = K rounded up to 64, or None when the layer does not qualify.
+
+    * The input channels are sorted by group (stable; the identity for contiguous groups); position p of
+      the sorted order holds channel ``xsrc[p]`` (-1 for the padding positions p >= K, whose codes are 0).
+    * ``qtile`` is a sequence of blocks, column tile T (32 columns) outermost, then block S (64 positions):
+      block (T, S) is 64 lanes x ``bits`` words; lane (n = lane % 32, h = lane // 32) holds the 32 codes of
+      column 32 T + n at positions 64 S + 32 h .. + 31 as the usual little-endian stream of ``bits``-bit
+      fields, with the codes permuted inside the lane (each 8 positions for 4 bits, all 32 for 3 bits) so
+      that the kernels' register unpack yields them in position order: stream field ``code_of_slot[s]``
+      holds position s.
+    * ``sz[g, n]`` = fp16 bits of ``scales[g, n]`` | fp16 bits of the zero point (stored value + 1) << 16.
+    """
+    from . import _slots
+
+    rows, N = qweight.shape
+    K = rows * 32 // bits
+    if not tiled_qualifies(K, N, bits, group_size):
+        return None
+    gs = K if group_size == -1 else group_size
+    dev = qweight.device
+    ar = torch.arange(K, dtype=torch.int64, device=dev)
+    if g_idx is None:
+        perm = ar
+    else:
+        g = g_idx.detach().to(device=dev, dtype=torch.int64)
+        perm = torch.argsort(g, stable=True)
+        if not torch.equal(g[perm], ar // gs):
+            return None
+    Kp = (K + TILE_CHANNELS - 1) // TILE_CHANNELS * TILE_CHANNELS
+    S, T = Kp // TILE_CHANNELS, N // TILE_COLS
+    codes = unpack_rows_torch(qweight.detach(), bits)[perm]                      # [K, N], sorted order
+    if Kp > K:
+        codes = torch.cat([codes, torch.zeros((Kp - K, N), dtype=codes.dtype, device=dev)])
+    # stream field i of a lane holds the position slot_of_code[i] (of each 8 for 4 bits, of the 32 for 3 bits)
+    inv = torch.tensor(_slots.slot_of_code(bits), dtype=torch.int64, device=dev)
+    if bits == 4:
+        order = (torch.arange(32, device=dev) // 8) * 8 + inv[torch.arange(32, device=dev) % 8]
+    else:
+        order = inv
+    blocks = codes.view(S * 2, 32, N)[:, order, :]                                # [(S, h), field, N]
+    words = pack_rows_torch(blocks.reshape(S * 2 * 32, N), bits)                  # [(S, h, word), N]
+    qtile = words.view(S, 2, bits, T, TILE_COLS).permute(3, 0, 1, 4, 2).contiguous().view(-1)
+    zeros = unpack_rows_torch(qzeros.detach().t().contiguous(), bits).t() + 1     # [G, N]
+    zbits = zeros.to(torch.float16).view(torch.int16).to(torch.int64) & 0xFFFF
+    sbits = scales.detach().contiguous().view(torch.int16).to(torch.int64) & 0xFFFF
+    both = sbits | (zbits << 16)
+    sz = torch.where(both >= (1 << 31), both - (1 << 32), both).to(torch.int32).contiguous()
+    xsrc = torch.full((Kp,), -1, dtype=torch.int32, device=dev)
+    xsrc[:K] = perm.to(torch.int32)
+    return qtile, sz, xsrc
+
+
 def num_groups(k: int, group_size: int) -> int:
     gs = k if group_size == -1 else group_size
     return math.ceil(k / gs)

@@ -40,9 +40,12 @@ enum {
     GPTQ_HIP_KERNEL_GROUPED = 2, /* rows expanded by group, scales applied once per group; M <= 2 with few groups,
                                     or M <= 8 with contiguous groups (activation rows packed into the
                                     operand tile: such plans have row_tiles = 4 or 8) */
-    GPTQ_HIP_KERNEL_STREAM = 3  /* exact fp16 weights, independent waves along K; any g_idx, any M.  M > 16: x is
+    GPTQ_HIP_KERNEL_STREAM = 3, /* exact fp16 weights, independent waves along K; any g_idx, any M.  M > 16: x is
                                    pre-packed into matrix-instruction fragment order (needs the workspace);
                                    M <= 16: the kernel reads x itself.  split_k > 1 adds a reduce launch. */
+    GPTQ_HIP_KERNEL_TILED = 4   /* a layer re-laid by gptq_hip_tile_prepare: exact fp16 weights, 32 * row_tiles rows x
+                                   64 columns per workgroup, four waves along K (k_chunk = blocks of 64 channels per
+                                   wave); x is pre-packed into the workspace; split_k > 1 adds a reduce launch */
 };
 
 /* What the dispatcher decided for one problem; filled by gptq_hip_select. */
@@ -162,6 +165,41 @@ int gptq_hip_sort_channels(const int32_t *qweight, const int32_t *g_idx, int32_t
  * groups needs and, when that plan is a STREAM one, M*K*2 bytes for x in the sorted order behind it (at
  * max(plan bytes, 16 KiB) rounded up to 256: the counters at the head of a workspace stay untouched). */
 size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits, int group_size);
+
+/*
+ * The tiled format: a layer re-laid once, when it is loaded, into the order the matrix instructions consume,
+ * for any number of rows of x (the reference's TVM module likewise keeps only its own re-laid copy of the
+ * weights, auto_gptq/nn_modules/qlinear_tvm.py:25-40,105-107).  With Kp = K rounded up to 64:
+ *   qtile  gptq_hip_tiled_bytes(K, N, bits) bytes, 16-byte aligned: blocks of 64 lanes x `bits` words, column tile
+ *          (32 columns) outermost, then block of 64 sorted positions; lane (n = lane % 32, h = lane / 32) holds the 32
+ *          codes of column 32 T + n at positions 64 S + 32 h .. + 31, permuted inside the lane into the order in
+ *          which the kernels' register unpack hands them to the matrix instruction
+ *   sz     uint32 [G, N]: fp16 scale | fp16 (zero point) << 16
+ *   xsrc   int32 [Kp], 16-byte aligned: the channel of x at sorted position p (stable sort of the channels by
+ *          group; the identity without an activation order), -1 for p >= K
+ * gptq_hip_tile_prepare writes the three from the checkpoint tensors (g_idx may be NULL = contiguous groups); it
+ * needs whole groups of equal size that are multiples of 32 channels (GPTQ_HIP_ERR_UNSUPPORTED otherwise) and
+ * a g_idx that gives every group exactly group_size channels (other contents stay in bounds but do not describe
+ * the layer).  Three launches; the sort costs K * K / 2 compares.
+ */
+size_t gptq_hip_tiled_bytes(int K, int N, int bits);
+int gptq_hip_tile_prepare(const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *g_idx,
+                          void *qtile, uint32_t *sz, int32_t *xsrc, int K, int N, int bits, int group_size,
+                          void *stream);
+
+/* The plan of the TILED family for a problem (workspace_bytes included); takes the place of the reference's
+ * tile table per M bucket (pycuda_warpper.py:77-127,150-189). */
+int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan);
+
+/*
+ * y = x @ W (+ bias) on a layer in the tiled format, any M; replaces the same handler call as gptq_hip_gemm
+ * (pycuda_warpper.py:138, qlinear_tvm.py:123,150).  x and y are in the layer's own channel order (xsrc = NULL
+ * means the identity).  plan: NULL = gptq_hip_select_tiled.  workspace: plan.workspace_bytes.  Two launches
+ * (pack pass, matmul), three when the plan splits K.
+ */
+int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint32_t *sz, const int32_t *xsrc, const void *bias,
+                        void *y, void *workspace, size_t workspace_bytes, int M, int K, int N, int bits,
+                        int group_size, const gptq_hip_plan *plan, void *stream);
 
 /*
  * W fp16 [K, N] = scales[g] * (q - (zq[g] + 1)), one rounding per element:

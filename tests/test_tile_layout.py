@@ -1,0 +1,59 @@
+"""The tiled format's definition (pack.tile_layout), pinned on the CPU: decoding every lane of every block by
+plain bit extraction, with the register unpack's slot table, must give back the codes of the layer in the
+order xsrc states; xsrc must be the stable sort of the channels by group; sz must hold the scales and the
+zero points (+1) the oracle unpacks."""
+import numpy as np
+import pytest
+import torch
+
+from autogptq.tvm_amd import _slots, pack
+from oracle import gptq_oracle as orc
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("K,N,gs,act", [(64, 32, 32, False), (192, 64, 64, True), (1056, 96, 32, True),
+                                        (2048, 64, 128, True), (96, 32, -1, True), (160, 32, 32, False)])
+def test_tile_layout_decodes_to_the_layer(bits, K, N, gs, act):
+    L = pack.synth_layer(5 + K, K, N, bits, gs, act)
+    qtile, sz, xsrc = pack.tile_layout(L["qweight"], L["qzeros"], L["scales"], L["g_idx"] if act else None, bits, gs)
+    Kp = (K + 63) // 64 * 64
+    S, T = Kp // 64, N // 32
+    assert qtile.numel() == T * S * 64 * bits and tuple(xsrc.shape) == (Kp,)
+    qt = qtile.numpy().view(np.uint32).reshape(T, S, 64, bits).astype(np.uint64)
+    stream_lo = qt[..., 0] | (qt[..., 1] << np.uint64(32))          # bits 0..63 of every lane's stream
+    stream_hi = qt[..., 2] if bits == 3 else (qt[..., 2] | (qt[..., 3] << np.uint64(32)))   # bits 64..
+    codes = orc.unpack_qweight_ref(L["qweight"], bits).numpy()      # the oracle's unpack, [K, N]
+    assert np.array_equal(codes, L["codes"].numpy())
+    code_of_slot = _slots.code_of_slot(bits)
+    x = xsrc.numpy()
+    for s in range(32):
+        field = (s // 8) * 8 + code_of_slot[s % 8] if bits == 4 else code_of_slot[s]
+        bit = bits * field
+        if bit + bits <= 64:
+            q = (stream_lo >> np.uint64(bit)) & np.uint64((1 << bits) - 1)
+        elif bit >= 64:
+            q = (stream_hi >> np.uint64(bit - 64)) & np.uint64((1 << bits) - 1)
+        else:   # a 3-bit field across bit 64
+            q = ((stream_lo >> np.uint64(bit)) | (stream_hi << np.uint64(64 - bit))) & np.uint64(7)
+        for h in range(2):
+            pos = 64 * np.arange(S) + 32 * h + s                     # [S]
+            src = x[pos]
+            want = np.where(src[None, :, None] >= 0, codes[np.maximum(src, 0)].reshape(S, T, 32).transpose(1, 0, 2), 0)
+            got = q[:, :, 32 * h: 32 * h + 32]                        # [T, S, n]
+            assert np.array_equal(got, want), (s, h)
+    g = L["g_idx"].numpy().astype(np.int64)
+    perm = np.argsort(g, kind="stable") if act else np.arange(K)
+    assert np.array_equal(x[:K], perm) and (x[K:] == -1).all()
+    szn = sz.numpy().view(np.uint32)
+    assert np.array_equal((szn & 0xFFFF).astype(np.uint16).view(np.float16), L["scales"].numpy())
+    zeros = orc.unpack_qzeros_ref(L["qzeros"], bits, N).numpy()       # already +1
+    assert np.array_equal((szn >> 16).astype(np.uint16).view(np.float16).astype(np.int64), zeros)
+
+
+def test_tile_layout_refuses_what_the_format_does_not_cover():
+    L = pack.synth_layer(9, 96, 32, 4, 16, False)      # groups narrower than a 32-channel lane block
+    assert pack.tile_layout(L["qweight"], L["qzeros"], L["scales"], None, 4, 16) is None
+    L = pack.synth_layer(9, 128, 32, 4, 64, True)
+    bad = L["g_idx"].clone()
+    bad[:] = 0                                          # not an activation order of equal groups
+    assert pack.tile_layout(L["qweight"], L["qzeros"], L["scales"], bad, 4, 64) is None

@@ -1,0 +1,167 @@
+"""GPU parity of the TILED family: the library's preparation against the torch statement of the format, and
+gptq_hip_gemm_tiled (through the C ABI) against the CPU oracle on the same seeded inputs.  The kernel forms the
+reference's rounded fp16 weights, so the tight bound applies as well as the contract's rtol = atol = 1e-2."""
+import ctypes
+
+import pytest
+import torch
+
+from autogptq.tvm_amd import _lib, ops, pack
+from tests.parity_util import assert_close, assert_tight, expected_output, expected_weight, layer, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+def prepare(D):
+    g = D["g_idx"] if D["desc_act"] else None
+    return ops.tile_prepare(D["qweight"], D["qzeros"], D["scales"], g, D["bits"], D["group_size"])
+
+
+def run_tiled(D, prep, x=None, plan=None):
+    qtile, sz, xsrc = prep
+    return ops.gemm_tiled(D["x"] if x is None else x, qtile, sz, xsrc if D["desc_act"] else None, D.get("bias"),
+                          D["bits"], D["group_size"], plan=plan)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("K,N,gs", [(64, 32, 32), (96, 32, 32), (1024, 416, 32), (2048, 1056, 256), (11008, 256, 128),
+                                    (1024, 160, -1), (4096, 352, 128)])
+@pytest.mark.parametrize("desc_act", [False, True])
+def test_library_preparation_equals_the_torch_statement(dev, bits, K, N, gs, desc_act):
+    L = layer(1100 + K, K, N, bits, gs, desc_act)
+    D = to_dev(L, dev)
+    g = D["g_idx"] if desc_act else None
+    want = pack.tile_layout(D["qweight"], D["qzeros"], D["scales"], g, bits, gs)
+    got = ops.tile_prepare(D["qweight"], D["qzeros"], D["scales"], g, bits, gs)
+    for a, b, what in zip(got, want, ("qtile", "sz", "xsrc")):
+        assert torch.equal(a, b), what
+    # an explicit contiguous g_idx is its own sorted order
+    if not desc_act:
+        again = ops.tile_prepare(D["qweight"], D["qzeros"], D["scales"], D["g_idx"], bits, gs)
+        for a, b in zip(again, want):
+            assert torch.equal(a, b)
+
+
+M_EDGES = [1, 2, 5, 16, 17, 31, 32, 33, 64, 65, 127, 128, 129, 257]
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("desc_act", [False, True])
+@pytest.mark.parametrize("M", M_EDGES)
+def test_tiled_ragged_m(dev, bits, desc_act, M):
+    L = layer(1200 + M, 512, 192, bits, 128, desc_act, M=M, bias=(M % 2 == 1))
+    D = to_dev(L, dev)
+    y = run_tiled(D, prepare(D))
+    assert y.shape == (M, 192) and y.dtype == torch.float16
+    assert_close(y, expected_output(L), f"tiled bits={bits} act={desc_act} M={M}")
+    assert_tight(y, expected_output(L), f"tiled bits={bits} act={desc_act} M={M}")
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("K,N,gs", [(32, 32, 32), (96, 32, 32), (160, 96, -1), (384, 64, 64), (1024, 416, 32),
+                                    (2048, 1056, 256), (4096, 352, 128)])
+@pytest.mark.parametrize("M", [1, 7, 40, 130])
+def test_tiled_odd_shapes(dev, bits, K, N, gs, M):
+    # K that is not a multiple of 64 (a padded last block), an odd number of column tiles, every tile height
+    for desc_act in (False, True):
+        L = layer(1300 + K + N, K, N, bits, gs, desc_act, M=M, bias=True)
+        D = to_dev(L, dev)
+        prep = prepare(D)
+        y = run_tiled(D, prep)
+        assert_close(y, expected_output(L), f"tiled bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
+        assert_tight(y, expected_output(L), f"tiled bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
+        assert torch.equal(y, run_tiled(D, prep)), "two identical calls differ"
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("split", [1, 2, 3, 5])
+@pytest.mark.parametrize("M", [20, 130])
+def test_tiled_forced_split_k(dev, bits, split, M):
+    K, N, gs = 4096, 352, 128
+    L = layer(1400 + split, K, N, bits, gs, True, M=M, bias=True)
+    D = to_dev(L, dev)
+    plan = _lib.select_tiled(M, K, N, bits, gs)
+    blocks = K // 64
+    plan.split_k, plan.grid_y = split, split
+    plan.k_chunk = -(-blocks // (4 * split))
+    part = (split * M * N * 4 + 255) // 256 * 256 if split > 1 else 0
+    ring = {1: 6, 2: 4, 4: 3}[plan.row_tiles]
+    plan.workspace_bytes = 16384 + part + (split * 4 * plan.k_chunk + ring) * 4 * plan.row_tiles * plan.m_blocks * 1024
+    prep = prepare(D)
+    y1 = run_tiled(D, prep, plan=plan)
+    y2 = run_tiled(D, prep, plan=plan)
+    assert_close(y1, expected_output(L), f"tiled split={split}")
+    assert_tight(y1, expected_output(L), f"tiled split={split}")
+    assert torch.equal(y1, y2)
+
+
+def test_tiled_integer_exact_and_guard_bands(dev):
+    # x = 1, scales = 1, one group: y[n] = sum_k (q - z), exactly representable
+    for bits in (3, 4):
+        L = layer(1500, 64, 64, bits, -1, False, M=2)
+        L["scales"] = torch.ones_like(L["scales"])
+        L["x"] = torch.ones_like(L["x"])
+        D = to_dev(L, dev)
+        y = run_tiled(D, prepare(D)).float().cpu()
+        want = (L["codes"].float() - L["zeros"][0].float()[None, :]).sum(dim=0)
+        assert torch.equal(y[0], want) and torch.equal(y[1], want)
+    M, K, N = 37, 512, 96
+    L = layer(1501, K, N, 4, 128, True, M=M)
+    D = to_dev(L, dev)
+    qtile, sz, xsrc = prepare(D)
+    guard = 4096
+    buf = torch.full((guard + M * N + guard,), 1234.0, dtype=torch.float16, device=dev)
+    out = buf[guard: guard + M * N].view(M, N)
+    ops.gemm_tiled(D["x"], qtile, sz, xsrc, None, 4, 128, out=out)
+    assert_close(out, expected_output(L), "guarded out")
+    assert bool((buf[:guard] == 1234.0).all()) and bool((buf[guard + M * N:] == 1234.0).all())
+
+
+def test_tiled_rejections(dev):
+    lib = _lib.lib()
+    fake, null = ctypes.c_void_p(0x1000), ctypes.c_void_p(None)
+    # no workspace; groups that are not whole 32-channel lane blocks; a plan of another family
+    assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, fake, null, 0, 8, 4096, 352, 4, 128, None, null) == _lib.ERR_WORKSPACE
+    assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, fake, fake, 1 << 24, 8, 4096, 352, 4, 16, None, null) == _lib.ERR_UNSUPPORTED
+    p = _lib.select(8, 4096, 352, 4, 128, False)
+    assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, fake, fake, 1 << 24, 8, 4096, 352, 4, 128, ctypes.byref(p),
+                                   null) == _lib.ERR_UNSUPPORTED
+    other = ctypes.c_void_p(0x2000)
+    assert lib.gptq_hip_tile_prepare(fake, fake, fake, null, other, fake, fake, 4096, 352, 4, 16, null) == _lib.ERR_UNSUPPORTED
+    assert lib.gptq_hip_tile_prepare(fake, fake, fake, null, null, fake, fake, 4096, 352, 4, 128, null) == _lib.ERR_BAD_ARG
+    assert lib.gptq_hip_tile_prepare(fake, fake, fake, null, fake, fake, fake, 4096, 352, 4, 128, null) == _lib.ERR_BAD_ARG  # in place
+    assert lib.gptq_hip_tiled_bytes(4096, 11008, 3) == 4096 * 11008 * 3 // 8
+    assert lib.gptq_hip_tiled_bytes(96, 32, 4) == 128 * 32 // 2
+
+
+TILED_FULL = [
+    ("c4-int4-4096x11008-act", 4, 4096, 11008, 128, True, [16, 64, 128, 256]),
+    ("c4-int3-4096x11008-act", 3, 4096, 11008, 128, True, [16, 64, 128, 256]),
+    ("c4-int4-11008x4096-act", 4, 11008, 4096, 128, True, [16, 64, 128, 256]),
+    ("c4-int3-11008x4096-act", 3, 11008, 4096, 128, True, [16, 64, 128, 256]),
+    ("c3-int4-4096x4096", 4, 4096, 4096, 128, False, [8, 1024]),
+    ("c5-int3-9216x36864-act-g1", 3, 9216, 36864, -1, True, [32]),
+    ("c5-int3-36864x9216-act-g1", 3, 36864, 9216, -1, True, [32]),
+]
+
+
+@pytest.mark.parametrize("name,bits,K,N,gs,desc_act,Ms", TILED_FULL, ids=[f[0] for f in TILED_FULL])
+def test_tiled_full_size(dev, name, bits, K, N, gs, desc_act, Ms):
+    L = layer(7200 + [f[0] for f in TILED_FULL].index(name), K, N, bits, gs, desc_act, M=max(Ms))
+    D = to_dev(L, dev)
+    w16 = expected_weight(L)
+    prep = prepare(D)
+    for M in Ms:
+        x = L["x"][:M].contiguous()
+        y = run_tiled(D, prep, x=x.to(dev))
+        want = expected_output(L, x=x, w16=w16)
+        assert_close(y, want, f"tiled {name} M={M}")
+        assert_tight(y, want, f"tiled {name} M={M}")
+        assert torch.equal(y, run_tiled(D, prep, x=x.to(dev))), f"tiled {name} M={M}: two identical calls differ"
