@@ -30,7 +30,7 @@ def flags() -> list:
     return [
         "--offload-arch=gfx950",
         "-O3",
-        "-std=c++17",
+        "-std=c++20",
         "-fPIC",
         "-shared",
         # keep the compiler from forming packed-fp32 instructions

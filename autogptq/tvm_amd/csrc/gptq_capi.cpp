@@ -346,17 +346,18 @@ extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint3
         plan = &chosen;
     }
     // the plan must be one this family runs, sized for this problem
-    const int at = plan->row_tiles;
+    const int rts = plan->row_tiles;  // 32-row tiles per workgroup
     const int S_total = (K + 63) / 64;
-    if (plan->kernel != GPTQ_HIP_KERNEL_TILED || (at != 1 && at != 2 && at != 4)) return GPTQ_HIP_ERR_UNSUPPORTED;
-    if (plan->block != 256 || plan->waves_k != 4 || plan->split_k < 1 || plan->k_chunk < 1 || plan->m_blocks < 1 ||
+    if (plan->kernel != GPTQ_HIP_KERNEL_TILED || (rts != 1 && rts != 2 && rts != 4)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    const int kwv = 4;
+    if (plan->block != 64 * kwv || plan->waves_k != kwv || plan->split_k < 1 || plan->k_chunk < 1 || plan->m_blocks < 1 ||
         plan->grid_x != (N / 32 + 1) / 2 || plan->grid_y != plan->split_k || plan->grid_z != plan->m_blocks ||
-        (long long)plan->m_blocks * 32 * at < M || (long long)plan->split_k * 4 * plan->k_chunk < S_total ||
-        plan->lds_bytes < 4 * at * 2 * 4096 || plan->lds_bytes > 160 * 1024)
+        (long long)plan->m_blocks * 32 * rts < M || (long long)plan->split_k * kwv * plan->k_chunk < S_total ||
+        plan->lds_bytes < gptq::tiled_lds_bytes(rts, kwv) || plan->lds_bytes > 160 * 1024)
         return GPTQ_HIP_ERR_BAD_ARG;
     if (plan->split_k > 1 && (long long)M * N >= (1LL << 32)) return GPTQ_HIP_ERR_UNSUPPORTED;
     const size_t part = plan->split_k > 1 ? ((size_t)plan->split_k * M * N * sizeof(float) + 255) / 256 * 256 : 0;
-    const size_t xb = (size_t)gptq::tiled_pack_blocks(plan->split_k, plan->k_chunk, at) * 4 * (size_t)(at * plan->m_blocks) * 1024;
+    const size_t xb = (size_t)gptq::tiled_pack_blocks(plan->split_k, kwv, plan->k_chunk) * 4 * (size_t)(rts * plan->m_blocks) * 1024;
     if (!workspace || !aligned(workspace, 16) || workspace_bytes < gptq::kCounterBytes + part + xb) return GPTQ_HIP_ERR_WORKSPACE;
     float *partial = (float *)((char *)workspace + gptq::kCounterBytes);
     char *xpack = (char *)workspace + gptq::kCounterBytes + part;

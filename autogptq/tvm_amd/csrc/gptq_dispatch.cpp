@@ -481,8 +481,9 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
     const int gs = group_size == -1 ? K : group_size;
     if (!gptq::tiled_qualifies(K, N, bits, gs)) return GPTQ_HIP_ERR_UNSUPPORTED;
-    const int at = gptq::tiled_row_tiles(M);
-    const int m_blocks = ceil_div(M, 32 * at);
+    const int at = gptq::tiled_row_tiles(M), rw = 1, kwv = 4;
+    const int rows = 32 * at * rw;
+    const int m_blocks = ceil_div(M, rows);
     const int col_pairs = ceil_div(N / 32, 2);
     const int S_total = ceil_div(K, 64);
     const long long tiles = (long long)col_pairs * m_blocks;
@@ -493,24 +494,24 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     if (split > cap) split = cap;
     if ((long long)M * N >= (1LL << 32)) split = 1;  // indexing of the pass that adds the partial tiles
     // every wave gets at least a ring of blocks
-    while (split > 1 && S_total / (split * 4) < gptq::tiled_ring(at)) split--;
-    const int wave_steps = ceil_div(S_total, split * 4);
-    split = ceil_div(S_total, wave_steps * 4);
+    while (split > 1 && S_total / (split * kwv) < gptq::tiled_ring(at)) split--;
+    const int wave_steps = ceil_div(S_total, split * kwv);
+    split = ceil_div(S_total, wave_steps * kwv);
     plan->kernel = GPTQ_HIP_KERNEL_TILED;
-    plan->row_tiles = at;
+    plan->row_tiles = at * rw;
     plan->m_blocks = m_blocks;
     plan->waves_n = 1;
-    plan->waves_k = 4;
+    plan->waves_k = kwv;
     plan->split_k = split;
     plan->k_chunk = wave_steps;  // blocks of 64 positions per wave
     plan->grid_x = col_pairs;
     plan->grid_y = split;
     plan->grid_z = m_blocks;
-    plan->block = 256;
-    plan->lds_bytes = 4 * at * 2 * 4096;
+    plan->block = 64 * rw * kwv;
+    plan->lds_bytes = gptq::tiled_lds_bytes(at * rw, kwv);
     size_t ws = gptq::kCounterBytes;
     if (split > 1) ws += ((size_t)split * M * N * sizeof(float) + 255) / 256 * 256;
-    ws += (size_t)gptq::tiled_pack_blocks(split, wave_steps, at) * 4 * (size_t)(at * m_blocks) * 1024;
+    ws += (size_t)gptq::tiled_pack_blocks(split, kwv, wave_steps) * 4 * (size_t)(at * rw * m_blocks) * 1024;
     plan->workspace_bytes = ws;
     return GPTQ_HIP_OK;
 }

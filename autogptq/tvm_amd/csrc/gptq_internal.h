@@ -169,16 +169,19 @@ inline size_t sorted_x_offset(size_t plan_bytes)
 
 
 // ---- TILED family (a layer re-laid by gptq_hip_tile_prepare) ----------------------------------------
-// blocks (64 positions) the register rings of a wave run ahead, by 32-row tiles per wave: the taller the
-// tile the longer a block takes, and the fewer blocks cover the memory latency
-constexpr int tiled_ring(int at) { return at >= 4 ? 3 : (at == 2 ? 4 : 6); }
-// 32-row tiles a wave holds for M rows
+// A workgroup is four waves along K; a wave holds AT 32-row tiles (row_tiles of the plan).
 inline int tiled_row_tiles(int M) { return M <= 32 ? 1 : (M <= 64 ? 2 : 4); }
-// blocks of x the pack pass writes: what the waves of all K ranges walk, plus the ring their refills run ahead
-inline int tiled_pack_blocks(int split_k, int wave_steps, int at) { return split_k * 4 * wave_steps + tiled_ring(at); }
+// blocks (64 positions) the register rings of a wave run ahead: the taller the tile, the longer a block
+// takes and the fewer of them cover the memory latency (and fit the registers)
+constexpr int tiled_ring(int at) { return at >= 4 ? 3 : (at == 2 ? 4 : 6); }
+// blocks of x the pack pass writes: what the waves of all K ranges walk
+inline int tiled_pack_blocks(int split_k, int waves_k, int wave_steps) { return split_k * waves_k * wave_steps; }
+// LDS of a workgroup: the result tiles (32 x 32 floats, two per 32 rows) of its waves
+inline int tiled_lds_bytes(int row_tiles, int waves_k) { return waves_k * row_tiles * 2 * 4096; }
 inline bool tiled_qualifies(int K, int N, int bits, int gs)
 {
-    return (bits == 3 || bits == 4) && K % 32 == 0 && N % 32 == 0 && gs % 32 == 0 && K % gs == 0;
+    // (the pack pass stages one row of x in LDS: K * 2 bytes)
+    return (bits == 3 || bits == 4) && K % 32 == 0 && N % 32 == 0 && gs % 32 == 0 && K % gs == 0 && K <= 65536;
 }
 int launch_tile_prepare(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
                         uint32_t *qtile, uint32_t *sz, int32_t *xsrc, int K, int N, int G, int bits, int group_size,

@@ -12,16 +12,27 @@
 //     the lane for j = 0..3) with no shuffle;
 //   * sz[g][n] = (fp16 scale, fp16 zero point) of group g, column n, one 32-bit word.
 //
-// tiled_gemm_kernel: a workgroup owns 64 columns (two tiles), 32 * AT rows of x and one K range; its
-// four waves (one per SIMD) split that range and never talk until the end.  A wave holds the whole
-// 32 AT x 64 result in registers, dequantises every weight of its range exactly once, as the reference
-// does (fp16(scale * (q - zero)), one rounding), and reads x as ready-made A fragments that a small
-// pack pass wrote (rows past M and positions past K as zeros).  One wave per SIMD overlaps its own
-// vector and matrix instructions: the dequantisation of the next B operand is interleaved with the
-// matrix instructions of the current one.  Weights and fragments ride in register rings RING blocks
-// deep, requested in the order they are consumed (loads return in order, one counter).
-// The four waves add their tiles through LDS at the end; workgroups along K (split_k > 1) leave fp32
-// tiles in the workspace for reduce_kernel.
+// tiled_gemm_kernel: a workgroup owns 64 columns (two tiles), 32 * AT rows of x and one K range; its four
+// waves (one per SIMD) split that range and never talk until the end.  A wave holds its whole 32 AT x 64
+// result in registers (AT = 4: 128 rows, 128 accumulator registers), dequantises every weight of its slice
+// exactly once, as the reference does (fp16(scale * (q - zero)), one rounding), and reads x as ready-made A
+// fragments that a small pack pass wrote (rows past M and positions past K as zeros).  One wave per SIMD
+// overlaps its own vector and matrix instructions (measured: up to six packed-fp16 instructions per
+// 32x32x16 matrix instruction are free), so the dequantisation of the next B operand is interleaved with the
+// matrix instructions of the current one.  Weights, (scale, zero) words and fragments ride in register
+// rings RING blocks deep, requested in the order they are consumed (vector loads return in order on one
+// counter, so a wait for a fragment also waits for every older load).
+// Measured alternatives that were no faster: eight waves per workgroup (two per SIMD, 64-row waves, two row
+// halves x four K slices or eight K slices); a wave's whole weight range brought into LDS up front with
+// global_load_lds (a CU draws ~35 GB/s from HBM, and those 3.7 us then stand in front of the first matrix
+// instruction).  What bounds the 128-row kernel is the A stream (every workgroup reads all of x through its
+// CU's L1: 1 MB at ~130 GB/s), the matrix pipes of the 172 CUs that 11008 columns give work to, and the
+// fixed costs around the loop.
+// The four waves add their tiles through LDS at the end; workgroups along K (split_k > 1) leave fp32 tiles
+// in the workspace for tiled_reduce_kernel.
+#include <type_traits>
+#include <utility>
+
 #include "gptq_device.h"
 
 namespace gptq {
@@ -143,37 +154,57 @@ int launch_tile_prepare(const uint32_t *qweight, const uint32_t *qzeros, const v
 // 64 lanes x 16 bytes; lane (m = lane % 32, h = lane / 32) holds x[32 rt + m][xsrc[64 S + 32 h + 8 j + e]],
 // e = 0..7.  Rows past M and positions past K are zeros; blocks up to S_pack are written (the kernel's
 // waves walk whole ranges, and their refills run a ring past the end).
+// One workgroup per row: the row goes to LDS with coalesced loads and the gather through xsrc reads LDS
+// (lanes that gather from global memory with one row per lane touch 64 cache lines per instruction).
 // ---------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void tile_pack_x_kernel(const _Float16 *__restrict__ x, const int32_t *__restrict__ xsrc,
                                                           char *__restrict__ xpack, int M, int K, int Kp, int rt_total,
                                                           int S_pack)
 {
-    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
-    const int lane = t & 63;
-    const uint32_t frag = t >> 6;
-    if (frag >= (uint32_t)S_pack * 4u * (uint32_t)rt_total) return;
-    const uint32_t sj = frag / rt_total;
-    const int rt = frag - sj * rt_total;
-    const int S = sj >> 2, j = sj & 3;
-    const int row = 32 * rt + (lane & 31);
-    const int p0 = 64 * S + 32 * (lane >> 5) + 8 * j;
-    h8 o = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (row < M && p0 < Kp) {
-        const _Float16 *xr = x + (size_t)row * K;
-        if (xsrc) {
-            const int4 a = *(const int4 *)(xsrc + p0);
-            const int4 b = *(const int4 *)(xsrc + p0 + 4);
-            const int idx[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    const int row = blockIdx.x;
+    const int rt = row >> 5, m = row & 31;
+    const int tid = threadIdx.x;
+    _Float16 *xl = (_Float16 *)smem;
+    const bool live = row < M;
+    const _Float16 *xr = x + (size_t)row * K;
+    const int octets = S_pack * 8;
+    int4 ia[2], ib[2];  // the map entries of this thread's first two octets, requested before the row is staged
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const _Float16 v = xr[min((uint32_t)max(idx[e], 0), (uint32_t)K - 1u)];  // a bad map must not fault
-                o[e] = idx[e] >= 0 ? v : (_Float16)0;
-            }
-        } else if (p0 < K) {  // K is a multiple of 32: a run of 8 is inside or outside as a whole
-            o = *(const h8 *)(xr + p0);
-        }
+    for (int i = 0; i < 2; i++) {
+        const int p0 = min(8 * (tid + 256 * i), Kp - 8);
+        ia[i] = xsrc ? *(const int4 *)(xsrc + p0) : make_int4(0, 0, 0, 0);
+        ib[i] = xsrc ? *(const int4 *)(xsrc + p0 + 4) : make_int4(0, 0, 0, 0);
     }
-    *(h8 *)(xpack + (size_t)frag * 1024 + lane * 16) = o;
+    if (live && xsrc) {
+        for (int i = tid; i < K / 8; i += 256) ((u4 *)xl)[i] = ((const u4 *)xr)[i];
+    }
+    __syncthreads();
+    for (int o = tid, it = 0; o < octets; o += 256, it++) {
+        const int p0 = 8 * o;
+        const int S = p0 >> 6, h = (p0 >> 5) & 1, j = (p0 >> 3) & 3;
+        h8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (live && p0 < Kp) {
+            if (xsrc) {
+                int4 a, b;
+                if (it < 2) {
+                    a = ia[it];
+                    b = ib[it];
+                } else {
+                    a = *(const int4 *)(xsrc + p0);
+                    b = *(const int4 *)(xsrc + p0 + 4);
+                }
+                const int idx[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const _Float16 t = xl[min((uint32_t)max(idx[e], 0), (uint32_t)K - 1u)];  // a bad map must not fault
+                    v[e] = idx[e] >= 0 ? t : (_Float16)0;
+                }
+            } else if (p0 < K) {  // K is a multiple of 32: a run of 8 is inside or outside as a whole
+                v = *(const h8 *)(xr + p0);
+            }
+        }
+        *(h8 *)(xpack + ((size_t)(4 * S + j) * rt_total + rt) * 1024 + (h * 32 + m) * 16) = v;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -212,17 +243,20 @@ __device__ __forceinline__ h8 tiled_bop(const uint32_t (&w)[BITS], int j, h2 s2,
     return __builtin_bit_cast(h8, o);
 }
 
-template <int BITS, int AT, int RING>
-__global__ __launch_bounds__(256) void tiled_gemm_kernel(const TiledParams p)
+// AT: 32-row tiles per wave.  RW x KW: waves of the workgroup along M and along K: the workgroup holds
+// 32 * AT * RW rows, and its KW waves along K split the workgroup's K range.
+template <int BITS, int AT, int RW, int KW, int RING>
+__global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledParams p)
 {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rw = wave % RW, kw = wave / RW;
     const int n = lane & 31, h = lane >> 5;
     const int T0 = 2 * blockIdx.x;
     const int split = blockIdx.y;
-    const int rt0 = blockIdx.z * AT;
-    const int S_begin = (split * 4 + wave) * p.wave_steps;
+    const int rt0 = (blockIdx.z * RW + rw) * AT;
+    const int S_begin = (split * KW + kw) * p.wave_steps;
     const int S_last = p.S_total - 1;
     const int lb_last = 2 * p.S_total - 1;
 
@@ -250,10 +284,8 @@ __global__ __launch_bounds__(256) void tiled_gemm_kernel(const TiledParams p)
             const char *src = p.qtile + ((size_t)(tile_off[ct] + (uint32_t)Sc) * (256u * BITS) + b_lane);
             if constexpr (BITS == 4) {
                 const u4 v = __builtin_nontemporal_load((const u4 *)src);
-                wr[ct][0] = v[0];
-                wr[ct][1] = v[1];
-                wr[ct][2] = v[2];
-                wr[ct][3] = v[3];
+#pragma unroll
+                for (int e = 0; e < 4; e++) wr[ct][e] = v[e];
             } else {
                 const W3 v = *(const W3 *)src;
                 wr[ct][0] = v.a;
@@ -269,12 +301,22 @@ __global__ __launch_bounds__(256) void tiled_gemm_kernel(const TiledParams p)
         for (int rt = 0; rt < AT; rt++) ar[rt] = __builtin_bit_cast(h8, *(const u4 *)(src + rt * 1024));
     };
 
+    // Every workgroup starts its walk at another block of its waves' ranges and wraps around, so that the
+    // workgroups, which all read the same A fragments, do not ask the same L2 channels at the same time.
+    const int ws_n = p.wave_steps;
+    int ahead = (int)((blockIdx.x + 3u * blockIdx.z) % (uint32_t)ws_n);  // block (inside the range) the next request is for
+    auto next_block = [&]() {
+        const int S = S_begin + ahead;
+        ahead = ahead + 1 == ws_n ? 0 : ahead + 1;
+        return S;
+    };
     // prologue, in consumption order
 #pragma unroll
     for (int u = 0; u < RING; u++) {
-        load_b(S_begin + u, w[u], szr[u]);
+        const int S = next_block();
+        load_b(S, w[u], szr[u]);
 #pragma unroll
-        for (int j = 0; j < 4; j++) load_a(S_begin + u, j, a[u][j]);
+        for (int j = 0; j < 4; j++) load_a(S, j, a[u][j]);
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -304,40 +346,57 @@ __global__ __launch_bounds__(256) void tiled_gemm_kernel(const TiledParams p)
     consts_of(szr[0][0], cs[0], cza[0], czb[0]);
     h8 bop_next = tiled_bop<BITS>(w[0][0], 0, cs[0], cza[0], czb[0], magic_a, magic_b);
 
-    for (int i0 = 0; i0 < p.wave_steps; i0 += RING) {
+    // One block of the walk (ring slot u): the eight (j, ct) operands, each multiplied with the AT row tiles
+    // while the next operand of the walk is dequantised.  REFILL: the slot's registers are requested again
+    // for the block a ring ahead as soon as their last reader is done.
+    auto block = [&](auto u_c, auto refill_c) {
+        constexpr int u = decltype(u_c)::value;
+        constexpr bool REFILL = decltype(refill_c)::value;
+        const int S_refill = REFILL ? next_block() : 0;  // the block a ring ahead of this one in the walk
 #pragma unroll
-        for (int u = 0; u < RING; u++) {
-            if (i0 + u >= p.wave_steps) break;  // (no load sits behind this branch)
-            const int S = S_begin + i0 + u;
+        for (int j = 0; j < 4; j++) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+            for (int ct = 0; ct < 2; ct++) {
+                const h8 bop = bop_next;
+                {
+                    const int jn = ct == 1 ? (j + 1) & 3 : j;
+                    const int ctn = ct ^ 1;
+                    constexpr int u1 = (u + 1) % RING;
+                    const bool wrap_u = ct == 1 && j == 3;
+                    if (jn == 0) consts_of(wrap_u ? szr[u1][ctn] : szr[u][ctn], cs[ctn], cza[ctn], czb[ctn]);  // first operand of a block
+                    bop_next = wrap_u ? tiled_bop<BITS>(w[u1][ctn], jn, cs[ctn], cza[ctn], czb[ctn], magic_a, magic_b)
+                                      : tiled_bop<BITS>(w[u][ctn], jn, cs[ctn], cza[ctn], czb[ctn], magic_a, magic_b);
+                }
 #pragma unroll
-                for (int ct = 0; ct < 2; ct++) {
-                    const h8 bop = bop_next;
-                    // the operand of the next (j, ct) of the walk, dequantised while this one multiplies
-                    {
-                        const int jn = ct == 1 ? (j + 1) & 3 : j;
-                        const int ctn = ct ^ 1;
-                        const int un = (ct == 1 && j == 3) ? (u + 1) % RING : u;
-                        if (jn == 0) consts_of(szr[un][ctn], cs[ctn], cza[ctn], czb[ctn]);  // first operand of a block
-                        bop_next = tiled_bop<BITS>(w[un][ctn], jn, cs[ctn], cza[ctn], czb[ctn], magic_a, magic_b);
-                    }
-#pragma unroll
-                    for (int rt = 0; rt < AT; rt++) {
-                        acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[u][j][rt], bop, acc[rt][ct], 0, 0, 0);
-                    }
-                    if (ct == 1) {
-                        __builtin_amdgcn_sched_barrier(0);
-                        if (j == 3) load_b(S + RING, w[u], szr[u]);  // (its last reader, the operand of (3, 1), is done)
-                        load_a(S + RING, j, a[u][j]);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
+                for (int rt = 0; rt < AT; rt++) {
+                    acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[u][j][rt], bop, acc[rt][ct], 0, 0, 0);
+                }
+                if (REFILL && ct == 1) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (j == 3) load_b(S_refill, w[u], szr[u]);  // (its last reader, the operand of (3, 1), is done)
+                    load_a(S_refill, j, a[u][j]);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
+    };
+    // whole turns of the ring, then what is left without refills (no load sits behind a branch, and the loop
+    // has no early exit: an exit into its latch would make the compiler wait at the head of every turn for
+    // almost every load in flight)
+    const int full = p.wave_steps / RING * RING;
+    for (int i0 = 0; i0 < full; i0 += RING) {
+        [&]<int... U>(std::integer_sequence<int, U...>) {
+            (block(std::integral_constant<int, U>{}, std::true_type{}), ...);
+        }(std::make_integer_sequence<int, RING>{});
+    }
+    {
+        const int rem = p.wave_steps - full;
+        [&]<int... U>(std::integer_sequence<int, U...>) {
+            ((U < RING - 1 && U < rem ? block(std::integral_constant<int, U>{}, std::false_type{}) : (void)0), ...);
+        }(std::make_integer_sequence<int, RING>{});
     }
 
-    // ---- the four waves meet in LDS: [wave][tile rt * 2 + ct][v][lane] floats ----------------------
+    // ---- the waves along K meet in LDS: [wave][tile rt * 2 + ct][v][lane] floats --------------------
     float *red = (float *)smem;
     {
         float *dst = red + (size_t)wave * (AT * 2) * 1024 + lane;
@@ -349,22 +408,24 @@ __global__ __launch_bounds__(256) void tiled_gemm_kernel(const TiledParams p)
                 for (int v = 0; v < 16; v++) dst[((rt * 2 + ct) * 16 + v) * 64] = acc[rt][ct][v];
     }
     __syncthreads();
-    // one item = four adjacent columns of one row: element v of lane (n, h) of tile (rt, ct) is row
-    // 32 rt + 8 (v / 4) + 4 h + v % 4, column 32 ct + n
-    const int m0 = 32 * rt0;
+    // one item = four adjacent columns of one row: element v of lane (n, h) of tile (rt, ct) of a wave in row
+    // group rw is row 32 (AT rw + rt) + 8 (v / 4) + 4 h + v % 4, column 32 ct + n
+    const int m0 = 32 * AT * RW * blockIdx.z;
     const _Float16 *bias = (const _Float16 *)p.bias;
     _Float16 *y = (_Float16 *)p.y;
+    constexpr int NT = 64 * RW * KW;
 #pragma unroll
-    for (int it = 0; it < 2 * AT; it++) {
-        const int item = tid + 256 * it;
+    for (int it = 0; it < 512 * AT * RW / NT; it++) {
+        const int item = tid + NT * it;
         const int r = item >> 4, c4 = (item & 15) * 4;
         const int ct = c4 >> 5, nn = c4 & 31;
-        const int rt = r >> 5, rr = r & 31;
+        const int rtw = r >> 5, rr = r & 31;          // 32-row tile of the workgroup
+        const int rwi = rtw / AT, rt = rtw % AT;      // its row group and tile inside the wave
         const int v = 4 * (rr >> 3) + (rr & 3), hh = (rr >> 2) & 1;
-        const float *src = red + ((size_t)(rt * 2 + ct) * 16 + v) * 64 + hh * 32 + nn;
+        const float *src = red + ((size_t)rwi * (AT * 2) + rt * 2 + ct) * 1024 + v * 64 + hh * 32 + nn;
         f4 sum = *(const f4 *)src;
 #pragma unroll
-        for (int wv = 1; wv < 4; wv++) sum += *(const f4 *)(src + (size_t)wv * (AT * 2) * 1024);
+        for (int k = 1; k < KW; k++) sum += *(const f4 *)(src + (size_t)k * RW * (AT * 2) * 1024);
         const int row = m0 + r;
         const int T = T0 + ct;
         if (row < p.M && T < p.T_total) {
@@ -407,19 +468,19 @@ __global__ __launch_bounds__(256) void tiled_reduce_kernel(const float *__restri
     *(h4 *)(y + (size_t)row * N + c) = o;
 }
 
-template <int BITS, int AT, int RING>
+template <int BITS, int AT, int RW, int KW, int RING>
 static int launch_tiled_one(const TiledParams &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
-    auto kern = tiled_gemm_kernel<BITS, AT, RING>;
-    const int lds_bytes = 4 * AT * 2 * 4096;
-    if (plan.lds_bytes < lds_bytes) return GPTQ_HIP_ERR_BAD_ARG;
+    auto kern = tiled_gemm_kernel<BITS, AT, RW, KW, RING>;
+    const int lds_bytes = tiled_lds_bytes(AT * RW, KW);
+    if (plan.lds_bytes < lds_bytes || plan.waves_k != KW || plan.block != 64 * RW * KW) return GPTQ_HIP_ERR_BAD_ARG;
     if (lds_bytes > 65536) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) {
             (void)hipGetLastError();
             return GPTQ_HIP_ERR_LAUNCH;
         }
     }
-    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, plan.grid_z), dim3(256), lds_bytes, stream, p);
+    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, plan.grid_z), dim3(64 * RW * KW), lds_bytes, stream, p);
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 
@@ -446,15 +507,22 @@ int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int
     p.rt_total = plan.row_tiles * plan.m_blocks;
     p.split_k = plan.split_k;
     p.lb_per_group = group_size / 32;
-    const int S_pack = tiled_pack_blocks(plan.split_k, plan.k_chunk, plan.row_tiles);
-    const unsigned threads = (unsigned)S_pack * 4u * (unsigned)p.rt_total * 64u;
-    hipLaunchKernelGGL(tile_pack_x_kernel, dim3((threads + 255u) / 256u), dim3(256), 0, stream, (const _Float16 *)x, xsrc,
+    const int S_pack = tiled_pack_blocks(plan.split_k, plan.waves_k, plan.k_chunk);
+    const int pack_lds = xsrc ? K * 2 : 0;  // one row of x
+    if (pack_lds > 65536) {
+        if (hipFuncSetAttribute((const void *)tile_pack_x_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, pack_lds) !=
+            hipSuccess) {
+            (void)hipGetLastError();
+            return GPTQ_HIP_ERR_LAUNCH;
+        }
+    }
+    hipLaunchKernelGGL(tile_pack_x_kernel, dim3(32 * p.rt_total), dim3(256), pack_lds, stream, (const _Float16 *)x, xsrc,
                        xpack, M, K, Kp, p.rt_total, S_pack);
     if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ERR_LAUNCH;
     int rc = GPTQ_HIP_ERR_UNSUPPORTED;
 #define GPTQ_TILED_CASE(B, A)                                                                  \
     if (bits == B && plan.row_tiles == A)                                                      \
-        rc = launch_tiled_one<B, A, tiled_ring(A)>(p, plan, stream)
+        rc = launch_tiled_one<B, A, 1, 4, tiled_ring(A)>(p, plan, stream)
     GPTQ_TILED_CASE(4, 1);
     GPTQ_TILED_CASE(4, 2);
     GPTQ_TILED_CASE(4, 4);

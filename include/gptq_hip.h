@@ -43,9 +43,10 @@ enum {
     GPTQ_HIP_KERNEL_STREAM = 3, /* exact fp16 weights, independent waves along K; any g_idx, any M.  M > 16: x is
                                    pre-packed into matrix-instruction fragment order (needs the workspace);
                                    M <= 16: the kernel reads x itself.  split_k > 1 adds a reduce launch. */
-    GPTQ_HIP_KERNEL_TILED = 4   /* a layer re-laid by gptq_hip_tile_prepare: exact fp16 weights, 32 * row_tiles rows x
-                                   64 columns per workgroup, four waves along K (k_chunk = blocks of 64 channels per
-                                   wave); x is pre-packed into the workspace; split_k > 1 adds a reduce launch */
+    GPTQ_HIP_KERNEL_TILED = 4   /* a layer re-laid by gptq_hip_tile_prepare: exact fp16 weights, 32 * row_tiles rows
+                                   (row_tiles = 1, 2 or 4) x 64 columns per workgroup of waves_k = 4 waves along K
+                                   (k_chunk = blocks of 64 channels per wave); x is pre-packed into the
+                                   workspace; split_k > 1 adds a reduce launch */
 };
 
 /* What the dispatcher decided for one problem; filled by gptq_hip_select. */

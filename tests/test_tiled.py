@@ -90,10 +90,9 @@ def test_tiled_forced_split_k(dev, bits, split, M):
     plan = _lib.select_tiled(M, K, N, bits, gs)
     blocks = K // 64
     plan.split_k, plan.grid_y = split, split
-    plan.k_chunk = -(-blocks // (4 * split))
+    plan.k_chunk = -(-blocks // (plan.waves_k * split))
     part = (split * M * N * 4 + 255) // 256 * 256 if split > 1 else 0
-    ring = {1: 6, 2: 4, 4: 3}[plan.row_tiles]
-    plan.workspace_bytes = 16384 + part + (split * 4 * plan.k_chunk + ring) * 4 * plan.row_tiles * plan.m_blocks * 1024
+    plan.workspace_bytes = 16384 + part + split * plan.waves_k * plan.k_chunk * 4 * plan.row_tiles * plan.m_blocks * 1024
     prep = prepare(D)
     y1 = run_tiled(D, prep, plan=plan)
     y2 = run_tiled(D, prep, plan=plan)
