@@ -21,6 +21,7 @@ KERNEL_GATHER = 1
 KERNEL_GROUPED = 2
 KERNEL_STREAM = 3
 KERNEL_TILED = 4
+KERNEL_TILED_DECODE = 5
 
 ABI_SYMBOLS = (
     "gptq_hip_select",
@@ -115,11 +116,11 @@ def lib() -> ctypes.CDLL:
     l.gptq_hip_tiled_bytes.restype = sz
     l.gptq_hip_tiled_bytes.argtypes = [i, i, i]
     l.gptq_hip_tile_prepare.restype = i
-    l.gptq_hip_tile_prepare.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
+    l.gptq_hip_tile_prepare.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
     l.gptq_hip_select_tiled.restype = i
     l.gptq_hip_select_tiled.argtypes = [i, i, i, i, i, ctypes.POINTER(Plan)]
     l.gptq_hip_gemm_tiled.restype = i
-    l.gptq_hip_gemm_tiled.argtypes = [vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
+    l.gptq_hip_gemm_tiled.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
     l.gptq_hip_dequant.restype = i
     l.gptq_hip_dequant.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
     l.gptq_hip_strerror.restype = ctypes.c_char_p

@@ -311,24 +311,26 @@ extern "C" size_t gptq_hip_tiled_bytes(int K, int N, int bits)
 }
 
 extern "C" int gptq_hip_tile_prepare(const int32_t *qweight, const int32_t *qzeros, const void *scales,
-                                     const int32_t *g_idx, void *qtile, uint32_t *sz, int32_t *xsrc, int K, int N,
-                                     int bits, int group_size, void *stream)
+                                     const int32_t *g_idx, void *qtile, uint32_t *sz, int32_t *xsrc, uint16_t *kinv,
+                                     int K, int N, int bits, int group_size, void *stream)
 {
-    if (!qtile || !sz || !xsrc || (const void *)qweight == qtile) return GPTQ_HIP_ERR_BAD_ARG;
+    if (!qtile || !sz || !xsrc || !kinv || (const void *)qweight == qtile) return GPTQ_HIP_ERR_BAD_ARG;
     const int rc = check_common(qweight, qzeros, scales, K, N, bits, group_size);
     if (rc != GPTQ_HIP_OK) return rc;
-    if (!aligned(qtile, 16) || !aligned(sz, 4) || !aligned(xsrc, 16) || (g_idx && !aligned(g_idx, 4)))
+    if (!aligned(qtile, 16) || !aligned(sz, 4) || !aligned(xsrc, 16) || !aligned(kinv, 16) || (g_idx && !aligned(g_idx, 4)))
         return GPTQ_HIP_ERR_BAD_ARG;
     const int gs = group_size == -1 ? K : group_size;
     if (!gptq::tiled_qualifies(K, N, bits, gs)) return GPTQ_HIP_ERR_UNSUPPORTED;
     return gptq::launch_tile_prepare((const uint32_t *)qweight, (const uint32_t *)qzeros, scales, g_idx, (uint32_t *)qtile,
-                                     sz, xsrc, K, N, K / gs, bits, gs, stream);
+                                     sz, xsrc, kinv, K, N, K / gs, bits, gs, stream);
 }
 
 extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint32_t *sz, const int32_t *xsrc,
-                                   const void *bias, void *y, void *workspace, size_t workspace_bytes, int M, int K,
-                                   int N, int bits, int group_size, const gptq_hip_plan *plan, void *stream)
+                                   const uint16_t *kinv, const void *bias, void *y, void *workspace,
+                                   size_t workspace_bytes, int M, int K, int N, int bits, int group_size,
+                                   const gptq_hip_plan *plan, void *stream)
 {
+    if ((xsrc == nullptr) != (kinv == nullptr) || (kinv && !aligned(kinv, 16))) return GPTQ_HIP_ERR_BAD_ARG;
     if (!x || !qtile || !sz || !y || M < 1) return GPTQ_HIP_ERR_BAD_ARG;
     if (bits != 3 && bits != 4) return GPTQ_HIP_ERR_BAD_ARG;
     if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;
@@ -344,6 +346,29 @@ extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint3
         const int rc = gptq_hip_select_tiled(M, K, N, bits, group_size, &chosen);
         if (rc != GPTQ_HIP_OK) return rc;
         plan = &chosen;
+    }
+    if (plan->kernel == GPTQ_HIP_KERNEL_TILED_DECODE) {
+        const int mr = plan->row_tiles, kw = plan->waves_k;
+        const int S_all = (K + 63) / 64;
+        if (M > gptq::kDecodeMaxRows || mr != gptq::tiled_decode_rows(M)) return GPTQ_HIP_ERR_UNSUPPORTED;
+        if ((kw != 4 && kw != 8 && kw != 16) || plan->block != 64 * kw || plan->split_k < 1 || plan->k_chunk < 1 ||
+            plan->grid_x != N / 32 || plan->grid_y != plan->split_k || plan->grid_z != 1 ||
+            (long long)plan->split_k * kw * plan->k_chunk < S_all ||
+            (long long)(plan->split_k - 1) * kw * plan->k_chunk >= S_all)  // every workgroup starts inside K
+            return GPTQ_HIP_ERR_BAD_ARG;
+        const int span = plan->k_chunk * kw * 64;
+        const int G_all = K / gs;
+        const int groups = (span - 1) / gs + 2 < G_all ? (span - 1) / gs + 2 : G_all;
+        if (plan->lds_bytes < gptq::tiled_decode_lds_bytes(mr, span, groups, kw) || plan->lds_bytes > 160 * 1024)
+            return GPTQ_HIP_ERR_BAD_ARG;
+        float *part = nullptr;
+        if (plan->split_k > 1) {
+            if ((long long)M * N >= (1LL << 32)) return GPTQ_HIP_ERR_UNSUPPORTED;
+            const size_t need = gptq::kCounterBytes + (size_t)plan->split_k * M * N * sizeof(float);
+            if (!workspace || !aligned(workspace, 16) || workspace_bytes < need) return GPTQ_HIP_ERR_WORKSPACE;
+            part = (float *)((char *)workspace + gptq::kCounterBytes);
+        }
+        return gptq::launch_tiled_decode(x, qtile, sz, kinv, bias, y, part, M, K, N, G_all, bits, gs, *plan, stream);
     }
     // the plan must be one this family runs, sized for this problem
     const int rts = plan->row_tiles;  // 32-row tiles per workgroup

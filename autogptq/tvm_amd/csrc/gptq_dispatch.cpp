@@ -481,6 +481,39 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
     const int gs = group_size == -1 ? K : group_size;
     if (!gptq::tiled_qualifies(K, N, bits, gs)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    if (M <= gptq::kDecodeMaxRows) {
+        // Decode: a workgroup per column tile of 32, enough waves along K to give the chip ~1000 waves, K cut
+        // over workgroups only when the staged x would not fit LDS.
+        const int mr = gptq::tiled_decode_rows(M);
+        const int tiles = N / 32;
+        const int S_total = ceil_div(K, 64);
+        int kw = tiles * 4 >= 1024 ? 4 : (tiles * 8 >= 1024 ? 8 : 16);
+        while (kw > 4 && kw > S_total) kw >>= 1;
+        for (int split = 1; split <= S_total; split++) {
+            const int wave_steps = ceil_div(S_total, split * kw);
+            if (ceil_div(S_total, wave_steps * kw) != split) continue;  // (the split this partition really needs)
+            const int span = wave_steps * kw * 64;
+            const int groups = (span - 1) / gs + 2 < ceil_div(K, gs) ? (span - 1) / gs + 2 : ceil_div(K, gs);
+            const int lds = gptq::tiled_decode_lds_bytes(mr, span, groups, kw);
+            if (lds > 128 * 1024) continue;
+            if (split > 1 && (long long)M * N >= (1LL << 32)) return GPTQ_HIP_ERR_UNSUPPORTED;
+            plan->kernel = GPTQ_HIP_KERNEL_TILED_DECODE;
+            plan->row_tiles = mr;
+            plan->m_blocks = 1;
+            plan->waves_n = 1;
+            plan->waves_k = kw;
+            plan->split_k = split;
+            plan->k_chunk = wave_steps;
+            plan->grid_x = tiles;
+            plan->grid_y = split;
+            plan->grid_z = 1;
+            plan->block = 64 * kw;
+            plan->lds_bytes = lds;
+            plan->workspace_bytes = split > 1 ? gptq::kCounterBytes + (size_t)split * M * N * sizeof(float) : 0;
+            return GPTQ_HIP_OK;
+        }
+        return GPTQ_HIP_ERR_UNSUPPORTED;
+    }
     const int at = gptq::tiled_row_tiles(M), rw = 1, kwv = 4;
     const int rows = 32 * at * rw;
     const int m_blocks = ceil_div(M, rows);

@@ -183,9 +183,20 @@ inline bool tiled_qualifies(int K, int N, int bits, int gs)
     // (the pack pass stages one row of x in LDS: K * 2 bytes)
     return (bits == 3 || bits == 4) && K % 32 == 0 && N % 32 == 0 && gs % 32 == 0 && K % gs == 0 && K <= 65536;
 }
+// decode kernel on the tiled format: rows it is built for, and the LDS of a workgroup whose waves cover
+// `span` positions of `groups` groups
+static const int kDecodeMaxRows = 8;
+inline int tiled_decode_rows(int M) { return M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8)); }
+inline int tiled_decode_lds_bytes(int mr, int span, int groups, int waves_k)
+{
+    return mr * span * 2 + 64 + (span / 32) * mr * 8 + groups * 128 + waves_k * mr * 128;
+}
 int launch_tile_prepare(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
-                        uint32_t *qtile, uint32_t *sz, int32_t *xsrc, int K, int N, int G, int bits, int group_size,
-                        void *stream);
+                        uint32_t *qtile, uint32_t *sz, int32_t *xsrc, uint16_t *kinv, int K, int N, int G, int bits,
+                        int group_size, void *stream);
+int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, const uint16_t *kinv, const void *bias,
+                        void *y, float *partial, int M, int K, int N, int G, int bits, int group_size,
+                        const gptq_hip_plan &plan, void *stream);
 int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int32_t *xsrc, const void *bias, void *y,
                  char *xpack, float *partial, int M, int K, int N, int G, int bits, int group_size,
                  const gptq_hip_plan &plan, void *stream);

@@ -45,15 +45,17 @@ struct alignas(4) W3 {
 
 // ---------------------------------------------------------------------------------------------------
 // Preparation, pass 1: xsrc[p] = the channel at position p of the stable sort by group (the rank of a
-// channel inside its group is the number of earlier channels of the same group), -1 for p >= K.
+// channel inside its group is the number of earlier channels of the same group), -1 for p >= K; and its
+// inverse kinv[k] = the position of channel k (positions are below 65536).
 // ---------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void tile_map_kernel(const int32_t *__restrict__ g_idx, int32_t *__restrict__ xsrc,
-                                                       int K, int Kp, int G, int group_size)
+                                                       uint16_t *__restrict__ kinv, int K, int Kp, int G, int group_size)
 {
     __shared__ int tile[256];
     const int k = blockIdx.x * 256 + threadIdx.x;
     if (!g_idx) {
         if (k < Kp) xsrc[k] = k < K ? k : -1;
+        if (k < K) kinv[k] = (uint16_t)k;
         return;
     }
     const int g = k < K ? min(max(g_idx[k], 0), G - 1) : -1;
@@ -68,7 +70,9 @@ __global__ __launch_bounds__(256) void tile_map_kernel(const int32_t *__restrict
     }
     if (k < K) {
         // a group with more than group_size members would leave its range: keep every index in bounds
-        xsrc[g * group_size + min(rank, group_size - 1)] = k;
+        const int pos = g * group_size + min(rank, group_size - 1);
+        xsrc[pos] = k;
+        kinv[k] = (uint16_t)pos;
     } else if (k < Kp) {
         xsrc[k] = -1;
     }
@@ -126,13 +130,14 @@ __global__ __launch_bounds__(256) void tile_sz_kernel(const uint32_t *__restrict
 }
 
 int launch_tile_prepare(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
-                        uint32_t *qtile, uint32_t *sz, int32_t *xsrc, int K, int N, int G, int bits, int group_size,
-                        void *stream_v)
+                        uint32_t *qtile, uint32_t *sz, int32_t *xsrc, uint16_t *kinv, int K, int N, int G, int bits,
+                        int group_size, void *stream_v)
 {
     hipStream_t stream = (hipStream_t)stream_v;
     const int Kp = (K + 63) / 64 * 64;
     const int S_total = Kp / 64, T_total = N / 32;
-    hipLaunchKernelGGL(tile_map_kernel, dim3((Kp + 255) / 256), dim3(256), 0, stream, g_idx, xsrc, K, Kp, G, group_size);
+    hipLaunchKernelGGL(tile_map_kernel, dim3((Kp + 255) / 256), dim3(256), 0, stream, g_idx, xsrc, kinv, K, Kp, G,
+                       group_size);
     const unsigned threads = (unsigned)T_total * (unsigned)S_total * 64u;
     const unsigned szt = (unsigned)G * (unsigned)N;
     if (bits == 4) {
@@ -447,6 +452,301 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// tiled_decode_kernel: M <= 8 rows of x on the tiled format, bound by the weight stream from HBM.
+//
+// A workgroup owns ONE column tile (32 columns) and one K range; its KW waves split that range.  With one
+// small workgroup per tile every CU gets work whatever N is (11008 columns: 344 workgroups of 4 waves,
+// 4096 columns: 128 of 16), and what a wave keeps in flight (PF blocks of 1 KB / 768 B) adds up over the
+// many waves of a CU.
+// The dots run on v_mfma_f32_4x4x4_16B_f16: sixteen independent 4-lane blocks, lane 4 b + i supplies
+// row i of A and column i of B of block b, and result register v of lane 4 b + j is row v of column j.
+// A lane of the tiled format holds 32 codes of ONE column, so its unpacked registers are B operands as
+// they are (four positions each), the A operand of lane 4 b + i is x[row i] at the same four positions
+// (read from LDS: rows past M read zeros), and the four result registers of a lane are the rows of its
+// own column.  Up to four rows of x cost one matrix instruction per four positions, five to eight two.
+// Per weight the vector ALU only unpacks.
+// The codes enter as (base + q) with the bases of the register unpack; per block of 32 positions the
+// epilogue takes y += scale * (P - Bsum - zero * Xsum), with Xsum = sum x and Bsum = sum x * base of the
+// block computed once per workgroup when x is staged.  Like GROUPED, and unlike the TILED matmul, this
+// does not reproduce the fp16 rounding of each dequantised weight: products are exact, sums are fp32.
+// x reaches LDS in position order: a layer with an activation order scatters it through kinv (16-bit
+// position per channel, one round trip; every workgroup walks all of x and keeps its K range).
+// ---------------------------------------------------------------------------------------------------
+struct DecodeParams {
+    const _Float16 *x;      // [M, K]
+    const uint16_t *kinv;   // [K] position of channel k, or nullptr (identity)
+    const char *qtile;
+    const uint32_t *sz;     // [G][N]
+    const void *bias;
+    void *y;                // fp16 [M, N]
+    float *partial;         // [split_k][M][N] when split_k > 1
+    int M, K, N, G;
+    int S_total, T_total;
+    int wave_steps;         // blocks (64 positions) per wave
+    int split_k;
+    int lb_per_group;       // group_size / 32
+    uint32_t lbg_magic;     // lane block -> group: umulhi(lb, magic) + (add ? lb : 0)
+    int lbg_add;
+};
+
+typedef float f2 __attribute__((ext_vector_type(2)));
+
+template <int BITS, int MR, int KW>
+__global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParams p)
+{
+    constexpr int NT = 64 * KW;
+    constexpr int PF = 4;              // blocks of weights a wave requests ahead
+    constexpr int MA = (MR + 3) / 4;   // matrix instructions per four positions (rows 0..3, rows 4..7)
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, h = lane >> 5;
+    const int T = blockIdx.x;
+    const int split = blockIdx.y;
+    const int wg_steps = p.wave_steps * KW;              // blocks of the workgroup's K range
+    const int S_wg = split * wg_steps;                   // its first block
+    const int S_begin = S_wg + wave * p.wave_steps;      // this wave's first block
+    const int S_last = p.S_total - 1;
+    const int span = wg_steps * 64;                      // positions the workgroup stages
+    const int p0 = S_wg * 64;                            // its first position
+
+    // LDS: x in position order [MR][span] fp16 | 64 zero bytes | block sums [span / 32][MR] (Xsum, Bsum) |
+    //      (scale, zero) words of the range's groups [groups][32] | partial results [KW][MR][32]
+    _Float16 *xl = (_Float16 *)smem;
+    const uint32_t zero_off = (uint32_t)MR * (uint32_t)span * 2u;
+    f2 *xs = (f2 *)(smem + zero_off + 64);
+    const int lbs = span / 32;
+    const uint32_t g_first = __umulhi((uint32_t)(2 * S_wg), p.lbg_magic) + (p.lbg_add ? (uint32_t)(2 * S_wg) : 0u);
+    const uint32_t lb_end = (uint32_t)min(2 * (S_wg + wg_steps), 2 * p.S_total) - 1u;
+    const uint32_t g_lastr = min(__umulhi(lb_end, p.lbg_magic) + (p.lbg_add ? lb_end : 0u), (uint32_t)p.G - 1u);
+    const int n_groups = (int)(g_lastr - g_first) + 1;
+    uint32_t *szl = (uint32_t *)(xs + (size_t)lbs * MR);
+    float *red = (float *)(szl + (size_t)n_groups * 32);
+
+    // ---- 1. x and the map first (a wait for them would also wait for every older load: vector loads return
+    //         in order), then the first weights of this wave, then the (scale, zero) words ----------------
+    // (without a map the channels of the range are the range itself)
+    const int k8_lo = p.kinv ? 0 : p0 / 8, k8_hi = p.kinv ? p.K / 8 : min(p0 + span, p.K) / 8;
+    constexpr int QP = 2;  // passes over x kept in registers
+    u4 kq[QP];
+    h8 xq[QP][MR];
+#pragma unroll
+    for (int ps = 0; ps < QP; ps++) {
+        const int k = 8 * min(k8_lo + tid + ps * NT, k8_hi - 1);  // (clamped: the pass is skipped below when outside)
+        kq[ps] = p.kinv ? *(const u4 *)(p.kinv + k) : (u4){0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int m = 0; m < MR; m++) xq[ps][m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
+    }
+    // the (scale, zero) words of the range's groups for this tile's 32 columns: SZP passes in registers
+    constexpr int SZP = 4;
+    uint32_t szq[SZP];
+#pragma unroll
+    for (int ps = 0; ps < SZP; ps++) {
+        const int i = min(tid + ps * NT, n_groups * 32 - 1);
+        szq[ps] = p.sz[(size_t)(g_first + (uint32_t)(i >> 5)) * p.N + 32 * T + (i & 31)];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    const uint32_t b_lane = (uint32_t)lane * (4u * BITS);
+    const uint32_t tile_off = (uint32_t)T * (uint32_t)p.S_total;
+    uint32_t w[2][PF][BITS];
+    const int steps = min(p.wave_steps, max(p.S_total - S_begin, 0));  // blocks of this wave that lie inside K
+    auto load_w = [&](int i, uint32_t (&wr)[BITS]) {
+        // block i of the wave's range; past its end: its first block again (a cache hit that is never multiplied)
+        const int Sc = min(S_begin + (i < steps ? i : 0), S_last);
+        const char *src = p.qtile + ((size_t)(tile_off + (uint32_t)Sc) * (256u * BITS) + b_lane);
+        if constexpr (BITS == 4) {
+            const u4 v = __builtin_nontemporal_load((const u4 *)src);
+#pragma unroll
+            for (int e = 0; e < 4; e++) wr[e] = v[e];
+        } else {
+            const W3 v = *(const W3 *)src;
+            wr[0] = v.a;
+            wr[1] = v.b;
+            wr[2] = v.c;
+        }
+    };
+    // two chunks of PF blocks are in flight from here on, through the staging of x as well
+#pragma unroll
+    for (int u = 0; u < PF; u++) load_w(u, w[0][u]);
+#pragma unroll
+    for (int u = 0; u < PF; u++) load_w(PF + u, w[1][u]);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- 2. stage x in position order ------------------------------------------------------------------
+    if (tid < 16) ((uint32_t *)(smem + zero_off))[tid] = 0u;
+    {
+        // positions of the range that lie past K (the padding of the last block) read as zeros
+        const int tail0 = max(p.K - p0, 0);
+        for (int i = tail0 + tid; i < span; i += NT)
+#pragma unroll
+            for (int m = 0; m < MR; m++) xl[m * span + i] = (_Float16)0;
+    }
+    auto scatter8 = [&](int k, const u4 &kv, const h8 (&xv)[MR]) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int pos = p.kinv ? (int)((kv[e >> 1] >> (16 * (e & 1))) & 0xffffu) : k + e;
+            const int pl = pos - p0;
+            if ((unsigned)pl < (unsigned)span) {
+#pragma unroll
+                for (int m = 0; m < MR; m++) xl[m * span + pl] = xv[m][e];
+            }
+        }
+    };
+#pragma unroll
+    for (int ps = 0; ps < QP; ps++) {
+        const int k8 = k8_lo + tid + ps * NT;
+        if (k8 < k8_hi) scatter8(8 * k8, kq[ps], xq[ps]);
+    }
+    for (int k8 = k8_lo + tid + QP * NT; k8 < k8_hi; k8 += NT) {  // long layers: the rest, a pass at a time
+        const int k = 8 * k8;
+        u4 kv = {0u, 0u, 0u, 0u};
+        if (p.kinv) kv = *(const u4 *)(p.kinv + k);
+        h8 xv[MR];
+#pragma unroll
+        for (int m = 0; m < MR; m++) xv[m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
+        scatter8(k, kv, xv);
+    }
+#pragma unroll
+    for (int ps = 0; ps < SZP; ps++) {
+        const int i = tid + ps * NT;
+        if (i < n_groups * 32) szl[i] = szq[ps];
+    }
+    for (int i = tid + SZP * NT; i < n_groups * 32; i += NT) {  // more groups than the register passes hold
+        szl[i] = p.sz[(size_t)(g_first + (uint32_t)(i >> 5)) * p.N + 32 * T + (i & 31)];
+    }
+    lds_barrier();
+    // ---- 3. per block of 32 positions and row: Xsum = sum x, Bsum = sum x * base(position); every wave for
+    //         the blocks of its own slice (LDS serves one wave's accesses in order: no barrier needed) ------
+    {
+        const int lb0 = 2 * (S_begin - S_wg);
+        for (int i = lane; i < 2 * p.wave_steps * MR; i += 64) {
+            const int lb = lb0 + i / MR, m = i % MR;
+            float X = 0.f, B = 0.f;
+            if (m < p.M) {
+                const h8 *src = (const h8 *)(xl + m * span + 32 * lb);
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const h8 q = src[v];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const float xf = (float)q[e];
+                        X += xf;
+                        B += xf * (BITS == 4 ? BASE4[e] : BASE3[e]);
+                    }
+                }
+            }
+            xs[lb * MR + m] = (f2){X, B};
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+
+    // ---- 4. the walk ----------------------------------------------------------------------------------
+    const uint32_t magic_a = opaque_vgpr(BITS == 4 ? MAGIC4_LO : MAGIC3_EVEN);
+    const uint32_t magic_b = opaque_vgpr(BITS == 4 ? MAGIC4_HI : MAGIC3_ODD);
+    const int row_i = lane & 3;  // the row of x this lane supplies to its 4-lane block
+    float ysum[MR];
+#pragma unroll
+    for (int m = 0; m < MR; m++) ysum[m] = 0.f;
+    // Per-lane byte offsets that never change; what changes per block is wave-uniform and stays in scalar
+    // registers.  A lane whose row lies past M reads the 64 zero bytes whatever the block (stride 0).
+    uint32_t x_base[MA], x_stride[MA];
+#pragma unroll
+    for (int a = 0; a < MA; a++) {
+        const int row = 4 * a + row_i;
+        x_base[a] = row < p.M ? (uint32_t)(row * span + 32 * h) * 2u : zero_off;
+        x_stride[a] = row < p.M ? 128u : 0u;
+    }
+    const uint32_t xs_lane = zero_off + 64u + (uint32_t)(h * MR) * 8u;   // block sums of lane block 2 sb + h
+    const uint32_t sz_lane = (uint32_t)((const unsigned char *)szl - smem) + (uint32_t)n * 4u;
+
+    auto do_block = [&](int S, const uint32_t (&wr)[BITS]) {
+        // unpack: sixteen registers, positions (2 r, 2 r + 1) of the lane in register r
+        u4 q[4];
+        if constexpr (BITS == 4) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                u4 t[1];
+                biased4(wr[j], t, magic_a, magic_b);
+                q[j] = t[0];
+            }
+        } else {
+            biased3(wr[0], wr[1], wr[2], q, magic_a, magic_b);
+        }
+        const uint32_t sb = (uint32_t)(S - S_wg);  // block inside the workgroup's range (wave-uniform)
+        f4 acc[MA];
+#pragma unroll
+        for (int a = 0; a < MA; a++) {
+            // (two chains: a matrix instruction waits for the one it adds to)
+            f4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};
+            const uint32_t xoff = x_base[a] + x_stride[a] * sb;
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const u4 xv = *(const u4 *)(smem + xoff + 16 * v);  // positions 8 v .. 8 v + 7 of the lane block
+                const u2 a0 = {xv[0], xv[1]}, a1 = {xv[2], xv[3]};
+                const u2 b0 = {q[v][0], q[v][1]}, b1 = {q[v][2], q[v][3]};
+                c0 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a0), __builtin_bit_cast(h4, b0), c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a1), __builtin_bit_cast(h4, b1), c1, 0, 0, 0);
+            }
+            acc[a] = c0 + c1;
+        }
+        // scale and zero point of the lane block's group (the two halves of the wave may differ), and its sums
+        const uint32_t l0 = 2u * (uint32_t)S, l1 = l0 + 1u;
+        const uint32_t g0 = min(__umulhi(l0, p.lbg_magic) + (p.lbg_add ? l0 : 0u), (uint32_t)p.G - 1u) - g_first;
+        const uint32_t g1 = min(__umulhi(l1, p.lbg_magic) + (p.lbg_add ? l1 : 0u), (uint32_t)p.G - 1u) - g_first;
+        const h2 e = as_h2(*(const uint32_t *)(smem + sz_lane + (h ? g1 : g0) * 128u));
+        const float sc = (float)e[0], zp = (float)e[1];
+        const f2 *xb = (const f2 *)(smem + xs_lane + sb * (uint32_t)(2 * MR * 8));
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            const f2 t = xb[m];
+            ysum[m] += sc * ((acc[m >> 2][m & 3] - t[1]) - zp * t[0]);
+        }
+    };
+
+    for (int c = 0; c < steps; c += 2 * PF) {
+#pragma unroll
+        for (int u = 0; u < PF; u++)
+            if (c + u < steps) do_block(S_begin + c + u, w[0][u]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < PF; u++) load_w(c + 2 * PF + u, w[0][u]);  // the chunk after the one in flight
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < PF; u++)
+            if (c + PF + u < steps) do_block(S_begin + c + PF + u, w[1][u]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < PF; u++) load_w(c + 3 * PF + u, w[1][u]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // ---- 5. the two halves of a column (lanes n and n + 32), then the waves along K ---------------------
+#pragma unroll
+    for (int m = 0; m < MR; m++) ysum[m] += __shfl_xor(ysum[m], 32);
+    if (h == 0) {
+#pragma unroll
+        for (int m = 0; m < MR; m++) red[(wave * MR + m) * 32 + n] = ysum[m];
+    }
+    lds_barrier();
+    if (tid < MR * 32) {
+        const int m = tid >> 5, nn = tid & 31;
+        if (m < p.M) {
+            float sum = 0.f;
+            for (int k = 0; k < KW; k++) sum += red[(k * MR + m) * 32 + nn];
+            const size_t o = (size_t)m * p.N + 32 * T + nn;
+            if (p.split_k == 1) {
+                if (p.bias) sum += (float)((const _Float16 *)p.bias)[32 * T + nn];
+                ((_Float16 *)p.y)[o] = (_Float16)sum;
+            } else {
+                p.partial[(size_t)split * p.M * p.N + o] = sum;
+            }
+        }
+    }
+}
+
 // y = fp16(sum over split of partial[split] (+ bias)), four columns per thread, in split order.
 __global__ __launch_bounds__(256) void tiled_reduce_kernel(const float *__restrict__ partial, const _Float16 *bias,
                                                            _Float16 *__restrict__ y, int M, int N, int split_k)
@@ -530,6 +830,81 @@ int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int
     GPTQ_TILED_CASE(3, 2);
     GPTQ_TILED_CASE(3, 4);
 #undef GPTQ_TILED_CASE
+    if (rc != GPTQ_HIP_OK) return rc;
+    if (plan.split_k > 1) {
+        const uint32_t quads = (uint32_t)M * ((uint32_t)N / 4u);
+        hipLaunchKernelGGL(tiled_reduce_kernel, dim3((quads + 255u) / 256u), dim3(256), 0, stream, partial,
+                           (const _Float16 *)bias, (_Float16 *)y, M, N, plan.split_k);
+        if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ERR_LAUNCH;
+    }
+    return GPTQ_HIP_OK;
+}
+
+
+template <int BITS, int MR, int KW>
+static int launch_decode_one(const DecodeParams &p, const gptq_hip_plan &plan, hipStream_t stream)
+{
+    auto kern = tiled_decode_kernel<BITS, MR, KW>;
+    if (plan.lds_bytes > 65536) {
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, plan.lds_bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return GPTQ_HIP_ERR_LAUNCH;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, 1), dim3(64 * KW), plan.lds_bytes, stream, p);
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+}
+
+template <int BITS, int MR>
+static int launch_decode_kw(const DecodeParams &p, const gptq_hip_plan &plan, hipStream_t stream)
+{
+    switch (plan.waves_k) {
+        case 4: return launch_decode_one<BITS, MR, 4>(p, plan, stream);
+        case 8: return launch_decode_one<BITS, MR, 8>(p, plan, stream);
+        case 16: return launch_decode_one<BITS, MR, 16>(p, plan, stream);
+        default: return GPTQ_HIP_ERR_UNSUPPORTED;
+    }
+}
+
+// The decode product on the tiled format: one launch, plus a reduce pass when K is split over workgroups.
+int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, const uint16_t *kinv, const void *bias,
+                        void *y, float *partial, int M, int K, int N, int G, int bits, int group_size,
+                        const gptq_hip_plan &plan, void *stream_v)
+{
+    hipStream_t stream = (hipStream_t)stream_v;
+    DecodeParams p;
+    p.x = (const _Float16 *)x;
+    p.kinv = kinv;
+    p.qtile = (const char *)qtile;
+    p.sz = sz;
+    p.bias = bias;
+    p.y = y;
+    p.partial = partial;
+    p.M = M;
+    p.K = K;
+    p.N = N;
+    p.G = G;
+    p.S_total = (K + 63) / 64;
+    p.T_total = N / 32;
+    p.wave_steps = plan.k_chunk;
+    p.split_k = plan.split_k;
+    p.lb_per_group = group_size / 32;
+    // lane block -> group as a multiply-high (lane blocks are below 2^16 / 32 * 2)
+    p.lbg_add = p.lb_per_group == 1;
+    p.lbg_magic = p.lbg_add ? 0u : (uint32_t)((1ull << 32) / (uint32_t)p.lb_per_group) + 1u;
+    const int mr = tiled_decode_rows(M);
+    int rc = GPTQ_HIP_ERR_UNSUPPORTED;
+#define GPTQ_DECODE_CASE(B, R) \
+    if (bits == B && mr == R) rc = launch_decode_kw<B, R>(p, plan, stream)
+    GPTQ_DECODE_CASE(4, 1);
+    GPTQ_DECODE_CASE(4, 2);
+    GPTQ_DECODE_CASE(4, 4);
+    GPTQ_DECODE_CASE(4, 8);
+    GPTQ_DECODE_CASE(3, 1);
+    GPTQ_DECODE_CASE(3, 2);
+    GPTQ_DECODE_CASE(3, 4);
+    GPTQ_DECODE_CASE(3, 8);
+#undef GPTQ_DECODE_CASE
     if (rc != GPTQ_HIP_OK) return rc;
     if (plan.split_k > 1) {
         const uint32_t quads = (uint32_t)M * ((uint32_t)N / 4u);

@@ -201,7 +201,7 @@ def sort_channels(qweight: torch.Tensor, g_idx: torch.Tensor, bits: int, group_s
 def tile_prepare(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor, g_idx: Optional[torch.Tensor],
                  bits: int, group_size: int):
     """``pack.tile_layout`` on the library's own kernels (gptq_hip_tile_prepare): ``(qtile int32 1-D,
-    sz int32 [G, N], xsrc int32 [Kp])`` on the GPU.  The caller vouches that every group has exactly
+    sz int32 [G, N], xsrc int32 [Kp], kinv int16 [K] holding unsigned 16-bit positions)`` on the GPU.  The caller vouches that every group has exactly
     ``group_size`` channels.  Raises ``GptqHipError`` (UNSUPPORTED) for layers the tiled format does not cover."""
     _need_gpu("qweight", qweight, torch.int32)
     _need_gpu("qzeros", qzeros, torch.int32)
@@ -214,24 +214,28 @@ def tile_prepare(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tens
     qtile = torch.empty(nbytes // 4, dtype=torch.int32, device=dev)
     sz = torch.empty((G, N), dtype=torch.int32, device=dev)
     xsrc = torch.empty((K + 63) // 64 * 64, dtype=torch.int32, device=dev)
+    kinv = torch.empty(K, dtype=torch.int16, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().gptq_hip_tile_prepare(_ptr(qweight), _ptr(qzeros), _ptr(scales), _ptr(g_idx), _ptr(qtile),
-                                              _ptr(sz), _ptr(xsrc), K, N, bits, group_size, _stream(dev))
+                                              _ptr(sz), _ptr(xsrc), _ptr(kinv), K, N, bits, group_size, _stream(dev))
     if rc != _lib.OK:
         raise _lib.GptqHipError(rc, f"gptq_hip_tile_prepare(K={K}, N={N}, bits={bits}, group_size={group_size})")
-    return qtile, sz, xsrc
+    return qtile, sz, xsrc, kinv
 
 
 def gemm_tiled(x: torch.Tensor, qtile: torch.Tensor, sz: torch.Tensor, xsrc: Optional[torch.Tensor],
-               bias: Optional[torch.Tensor], bits: int, group_size: int, plan: Optional[_lib.Plan] = None,
-               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+               kinv: Optional[torch.Tensor], bias: Optional[torch.Tensor], bits: int, group_size: int,
+               plan: Optional[_lib.Plan] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y[M, N] fp16 = x[M, K] @ W (+ bias) on a layer in the tiled format (``tile_prepare``); x and y in the
-    layer's own channel order; ``xsrc=None`` means no activation order."""
+    layer's own channel order; ``xsrc = kinv = None`` means no activation order."""
     _need_gpu("x", x, torch.float16)
     _need_gpu("qtile", qtile, torch.int32)
     _need_gpu("sz", sz, torch.int32)
+    if (xsrc is None) != (kinv is None):
+        raise ValueError("xsrc and kinv go together: pass both (activation order) or neither")
     if xsrc is not None:
         _need_gpu("xsrc", xsrc, torch.int32)
+        _need_gpu("kinv", kinv, torch.int16)
     if bias is not None:
         _need_gpu("bias", bias, torch.float16)
     if x.dim() != 2 or sz.dim() != 2:
@@ -241,8 +245,8 @@ def gemm_tiled(x: torch.Tensor, qtile: torch.Tensor, sz: torch.Tensor, xsrc: Opt
     Kp = (K + 63) // 64 * 64
     if qtile.numel() * 4 != Kp * N * bits // 8:
         raise ValueError(f"qtile holds {qtile.numel() * 4} bytes, a {K} x {N} layer of {bits} bits needs {Kp * N * bits // 8}")
-    if xsrc is not None and tuple(xsrc.shape) != (Kp,):
-        raise ValueError(f"xsrc must be [{Kp}], got {tuple(xsrc.shape)}")
+    if xsrc is not None and (tuple(xsrc.shape) != (Kp,) or tuple(kinv.shape) != (K,)):
+        raise ValueError(f"xsrc must be [{Kp}] and kinv [{K}], got {tuple(xsrc.shape)} and {tuple(kinv.shape)}")
     if bias is not None and tuple(bias.shape) != (N,):
         raise ValueError(f"bias must be [{N}], got {tuple(bias.shape)}")
     dev = x.device
@@ -252,10 +256,11 @@ def gemm_tiled(x: torch.Tensor, qtile: torch.Tensor, sz: torch.Tensor, xsrc: Opt
         return out
     if plan is None:
         plan = _lib.select_tiled(M, K, N, bits, group_size)
-    ws = _workspace(dev, plan.workspace_bytes)
+    ws = _workspace(dev, plan.workspace_bytes) if plan.workspace_bytes else None
     with torch.cuda.device(dev):
-        rc = _lib.lib().gptq_hip_gemm_tiled(_ptr(x), _ptr(qtile), _ptr(sz), _ptr(xsrc), _ptr(bias), _ptr(out), _ptr(ws),
-                                            ws.numel(), M, K, N, bits, group_size, ctypes.byref(plan), _stream(dev))
+        rc = _lib.lib().gptq_hip_gemm_tiled(_ptr(x), _ptr(qtile), _ptr(sz), _ptr(xsrc), _ptr(kinv), _ptr(bias), _ptr(out),
+                                            _ptr(ws), ws.numel() if ws is not None else 0, M, K, N, bits, group_size,
+                                            ctypes.byref(plan), _stream(dev))
     if rc != _lib.OK:
         raise _lib.GptqHipError(rc, f"gptq_hip_gemm_tiled(M={M}, K={K}, N={N}, bits={bits}, group_size={group_size})")
     return out

@@ -155,7 +155,7 @@ TILE_CHANNELS = 64  # input channels of one block of the tiled format: two lane 
 def tiled_qualifies(K: int, N: int, bits: int, group_size: int) -> bool:
     """Layers the tiled format covers: 3 or 4 bits, whole groups made of whole 32-channel lane blocks."""
     gs = K if group_size == -1 else group_size
-    return bits in (3, 4) and K % 32 == 0 and N % 32 == 0 and gs % 32 == 0 and K % gs == 0
+    return bits in (3, 4) and K % 32 == 0 and N % 32 == 0 and gs % 32 == 0 and K % gs == 0 and K <= 65536
 
 
 def tile_layout(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor, g_idx, bits: int, group_size: int):
@@ -163,8 +163,9 @@ def tile_layout(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tenso
     preparation, ``gptq_hip_tile_prepare``, is tested against; the reference's TVM module re-lays its
     weights once in the same spirit, auto_gptq/nn_modules/qlinear_tvm.py:25-40,105-107).
 
-    Returns ``(qtile int32 [N/32 * Kp/64 * 64 * bits], sz int32 [G, N], xsrc int32 [Kp])`` with
-    Kp = K rounded up to 64, or None when the layer does not qualify.
+    Returns ``(qtile int32 [N/32 * Kp/64 * 64 * bits], sz int32 [G, N], xsrc int32 [Kp], kinv int16 [K])``
+    with Kp = K rounded up to 64, or None when the layer does not qualify (K must not exceed 65536: ``kinv``
+    holds the position of every channel, the inverse of ``xsrc``, as an unsigned 16-bit value).
 
     * The input channels are sorted by group (stable; the identity for contiguous groups); position p of
       the sorted order holds channel ``xsrc[p]`` (-1 for the padding positions p >= K, whose codes are 0).
@@ -213,7 +214,10 @@ def tile_layout(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tenso
     sz = torch.where(both >= (1 << 31), both - (1 << 32), both).to(torch.int32).contiguous()
     xsrc = torch.full((Kp,), -1, dtype=torch.int32, device=dev)
     xsrc[:K] = perm.to(torch.int32)
-    return qtile, sz, xsrc
+    inv = torch.empty(K, dtype=torch.int64, device=dev)
+    inv[perm] = ar
+    kinv = torch.where(inv >= (1 << 15), inv - (1 << 16), inv).to(torch.int16)   # unsigned 16-bit positions
+    return qtile, sz, xsrc, kinv
 
 
 def num_groups(k: int, group_size: int) -> int:

@@ -43,10 +43,14 @@ enum {
     GPTQ_HIP_KERNEL_STREAM = 3, /* exact fp16 weights, independent waves along K; any g_idx, any M.  M > 16: x is
                                    pre-packed into matrix-instruction fragment order (needs the workspace);
                                    M <= 16: the kernel reads x itself.  split_k > 1 adds a reduce launch. */
-    GPTQ_HIP_KERNEL_TILED = 4   /* a layer re-laid by gptq_hip_tile_prepare: exact fp16 weights, 32 * row_tiles rows
+    GPTQ_HIP_KERNEL_TILED = 4,  /* a layer re-laid by gptq_hip_tile_prepare: exact fp16 weights, 32 * row_tiles rows
                                    (row_tiles = 1, 2 or 4) x 64 columns per workgroup of waves_k = 4 waves along K
                                    (k_chunk = blocks of 64 channels per wave); x is pre-packed into the
                                    workspace; split_k > 1 adds a reduce launch */
+    GPTQ_HIP_KERNEL_TILED_DECODE = 5 /* the same layer for M <= 8 rows: a workgroup per 32 columns, waves_k (4, 8 or 16)
+                                   waves along K, x staged in LDS in the layer's sorted order; scales applied per
+                                   block of 32 channels; row_tiles = the rows the kernel is built for (1, 2, 4 or 8);
+                                   split_k > 1 (an x that does not fit LDS) adds a reduce launch */
 };
 
 /* What the dispatcher decided for one problem; filled by gptq_hip_select. */
@@ -178,6 +182,7 @@ size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits, int group_
  *   sz     uint32 [G, N]: fp16 scale | fp16 (zero point) << 16
  *   xsrc   int32 [Kp], 16-byte aligned: the channel of x at sorted position p (stable sort of the channels by
  *          group; the identity without an activation order), -1 for p >= K
+ *   kinv   uint16 [K], 16-byte aligned: its inverse, the position of channel k (K <= 65536)
  * gptq_hip_tile_prepare writes the three from the checkpoint tensors (g_idx may be NULL = contiguous groups); it
  * needs whole groups of equal size that are multiples of 32 channels (GPTQ_HIP_ERR_UNSUPPORTED otherwise) and
  * a g_idx that gives every group exactly group_size channels (other contents stay in bounds but do not describe
@@ -185,8 +190,8 @@ size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits, int group_
  */
 size_t gptq_hip_tiled_bytes(int K, int N, int bits);
 int gptq_hip_tile_prepare(const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *g_idx,
-                          void *qtile, uint32_t *sz, int32_t *xsrc, int K, int N, int bits, int group_size,
-                          void *stream);
+                          void *qtile, uint32_t *sz, int32_t *xsrc, uint16_t *kinv, int K, int N, int bits,
+                          int group_size, void *stream);
 
 /* The plan of the TILED family for a problem (workspace_bytes included); takes the place of the reference's
  * tile table per M bucket (pycuda_warpper.py:77-127,150-189). */
@@ -194,13 +199,14 @@ int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_size, gptq_hi
 
 /*
  * y = x @ W (+ bias) on a layer in the tiled format, any M; replaces the same handler call as gptq_hip_gemm
- * (pycuda_warpper.py:138, qlinear_tvm.py:123,150).  x and y are in the layer's own channel order (xsrc = NULL
- * means the identity).  plan: NULL = gptq_hip_select_tiled.  workspace: plan.workspace_bytes.  Two launches
- * (pack pass, matmul), three when the plan splits K.
+ * (pycuda_warpper.py:138, qlinear_tvm.py:123,150).  x and y are in the layer's own channel order (xsrc = kinv =
+ * NULL means no activation order; pass both or neither).  plan: NULL = gptq_hip_select_tiled.  workspace:
+ * plan.workspace_bytes (none for most decode plans).  M <= 8: one launch (the decode kernel); above: two
+ * (pack pass, matmul); one more when the plan splits K.
  */
-int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint32_t *sz, const int32_t *xsrc, const void *bias,
-                        void *y, void *workspace, size_t workspace_bytes, int M, int K, int N, int bits,
-                        int group_size, const gptq_hip_plan *plan, void *stream);
+int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint32_t *sz, const int32_t *xsrc, const uint16_t *kinv,
+                        const void *bias, void *y, void *workspace, size_t workspace_bytes, int M, int K, int N,
+                        int bits, int group_size, const gptq_hip_plan *plan, void *stream);
 
 /*
  * W fp16 [K, N] = scales[g] * (q - (zq[g] + 1)), one rounding per element:

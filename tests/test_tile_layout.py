@@ -15,7 +15,7 @@ from oracle import gptq_oracle as orc
                                         (2048, 64, 128, True), (96, 32, -1, True), (160, 32, 32, False)])
 def test_tile_layout_decodes_to_the_layer(bits, K, N, gs, act):
     L = pack.synth_layer(5 + K, K, N, bits, gs, act)
-    qtile, sz, xsrc = pack.tile_layout(L["qweight"], L["qzeros"], L["scales"], L["g_idx"] if act else None, bits, gs)
+    qtile, sz, xsrc, kinv = pack.tile_layout(L["qweight"], L["qzeros"], L["scales"], L["g_idx"] if act else None, bits, gs)
     Kp = (K + 63) // 64 * 64
     S, T = Kp // 64, N // 32
     assert qtile.numel() == T * S * 64 * bits and tuple(xsrc.shape) == (Kp,)
@@ -44,6 +44,7 @@ def test_tile_layout_decodes_to_the_layer(bits, K, N, gs, act):
     g = L["g_idx"].numpy().astype(np.int64)
     perm = np.argsort(g, kind="stable") if act else np.arange(K)
     assert np.array_equal(x[:K], perm) and (x[K:] == -1).all()
+    assert np.array_equal(kinv.numpy().view(np.uint16).astype(np.int64)[perm], np.arange(K))   # the inverse map
     szn = sz.numpy().view(np.uint32)
     assert np.array_equal((szn & 0xFFFF).astype(np.uint16).view(np.float16), L["scales"].numpy())
     zeros = orc.unpack_qzeros_ref(L["qzeros"], bits, N).numpy()       # already +1

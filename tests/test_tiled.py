@@ -25,9 +25,10 @@ def prepare(D):
 
 
 def run_tiled(D, prep, x=None, plan=None):
-    qtile, sz, xsrc = prep
-    return ops.gemm_tiled(D["x"] if x is None else x, qtile, sz, xsrc if D["desc_act"] else None, D.get("bias"),
-                          D["bits"], D["group_size"], plan=plan)
+    qtile, sz, xsrc, kinv = prep
+    act = D["desc_act"]
+    return ops.gemm_tiled(D["x"] if x is None else x, qtile, sz, xsrc if act else None, kinv if act else None,
+                          D.get("bias"), D["bits"], D["group_size"], plan=plan)
 
 
 @pytest.mark.parametrize("bits", [3, 4])
@@ -40,7 +41,7 @@ def test_library_preparation_equals_the_torch_statement(dev, bits, K, N, gs, des
     g = D["g_idx"] if desc_act else None
     want = pack.tile_layout(D["qweight"], D["qzeros"], D["scales"], g, bits, gs)
     got = ops.tile_prepare(D["qweight"], D["qzeros"], D["scales"], g, bits, gs)
-    for a, b, what in zip(got, want, ("qtile", "sz", "xsrc")):
+    for a, b, what in zip(got, want, ("qtile", "sz", "xsrc", "kinv")):
         assert torch.equal(a, b), what
     # an explicit contiguous g_idx is its own sorted order
     if not desc_act:
@@ -114,11 +115,11 @@ def test_tiled_integer_exact_and_guard_bands(dev):
     M, K, N = 37, 512, 96
     L = layer(1501, K, N, 4, 128, True, M=M)
     D = to_dev(L, dev)
-    qtile, sz, xsrc = prepare(D)
+    qtile, sz, xsrc, kinv = prepare(D)
     guard = 4096
     buf = torch.full((guard + M * N + guard,), 1234.0, dtype=torch.float16, device=dev)
     out = buf[guard: guard + M * N].view(M, N)
-    ops.gemm_tiled(D["x"], qtile, sz, xsrc, None, 4, 128, out=out)
+    ops.gemm_tiled(D["x"], qtile, sz, xsrc, kinv, None, 4, 128, out=out)
     assert_close(out, expected_output(L), "guarded out")
     assert bool((buf[:guard] == 1234.0).all()) and bool((buf[guard + M * N:] == 1234.0).all())
 
@@ -127,17 +128,88 @@ def test_tiled_rejections(dev):
     lib = _lib.lib()
     fake, null = ctypes.c_void_p(0x1000), ctypes.c_void_p(None)
     # no workspace; groups that are not whole 32-channel lane blocks; a plan of another family
-    assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, fake, null, 0, 8, 4096, 352, 4, 128, None, null) == _lib.ERR_WORKSPACE
-    assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, fake, fake, 1 << 24, 8, 4096, 352, 4, 16, None, null) == _lib.ERR_UNSUPPORTED
+    assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, null, fake, null, 0, 40, 4096, 352, 4, 128, None, null) == _lib.ERR_WORKSPACE
+    assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, null, fake, fake, 1 << 24, 8, 4096, 352, 4, 16, None, null) == _lib.ERR_UNSUPPORTED
+    assert lib.gptq_hip_gemm_tiled(fake, fake, fake, fake, null, null, fake, fake, 1 << 24, 8, 4096, 352, 4, 128, None, null) == _lib.ERR_BAD_ARG   # a map without its inverse
     p = _lib.select(8, 4096, 352, 4, 128, False)
-    assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, fake, fake, 1 << 24, 8, 4096, 352, 4, 128, ctypes.byref(p),
+    assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, null, fake, fake, 1 << 24, 8, 4096, 352, 4, 128, ctypes.byref(p),
                                    null) == _lib.ERR_UNSUPPORTED
     other = ctypes.c_void_p(0x2000)
-    assert lib.gptq_hip_tile_prepare(fake, fake, fake, null, other, fake, fake, 4096, 352, 4, 16, null) == _lib.ERR_UNSUPPORTED
-    assert lib.gptq_hip_tile_prepare(fake, fake, fake, null, null, fake, fake, 4096, 352, 4, 128, null) == _lib.ERR_BAD_ARG
-    assert lib.gptq_hip_tile_prepare(fake, fake, fake, null, fake, fake, fake, 4096, 352, 4, 128, null) == _lib.ERR_BAD_ARG  # in place
+    assert lib.gptq_hip_tile_prepare(fake, fake, fake, null, other, fake, fake, fake, 4096, 352, 4, 16, null) == _lib.ERR_UNSUPPORTED
+    assert lib.gptq_hip_tile_prepare(fake, fake, fake, null, null, fake, fake, fake, 4096, 352, 4, 128, null) == _lib.ERR_BAD_ARG
+    assert lib.gptq_hip_tile_prepare(fake, fake, fake, null, fake, fake, fake, fake, 4096, 352, 4, 128, null) == _lib.ERR_BAD_ARG  # in place
     assert lib.gptq_hip_tiled_bytes(4096, 11008, 3) == 4096 * 11008 * 3 // 8
     assert lib.gptq_hip_tiled_bytes(96, 32, 4) == 128 * 32 // 2
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("K,N,gs", [(32, 32, 32), (96, 32, 32), (160, 96, -1), (384, 64, 64), (1024, 416, 32),
+                                    (2048, 1056, 256), (4096, 352, 128), (11008, 256, 128), (4096, 64, 64)])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 7, 8])
+def test_tiled_decode_rows_and_shapes(dev, bits, K, N, gs, M):
+    """The decode kernel of the tiled format (M <= 8): every row count, K that is not a multiple of 64, one
+    and many column tiles, group sizes from one lane block to the whole layer, with and without an activation
+    order; against the oracle and against the unprepared kernels on the same inputs."""
+    for desc_act in (False, True):
+        L = layer(1600 + K + M, K, N, bits, gs, desc_act, M=M, bias=(M % 2 == 0))
+        D = to_dev(L, dev)
+        plan = _lib.select_tiled(M, K, N, bits, gs)
+        assert plan.kernel == _lib.KERNEL_TILED_DECODE and plan.row_tiles in (1, 2, 4, 8) and plan.row_tiles >= M
+        prep = prepare(D)
+        y = run_tiled(D, prep)
+        want = expected_output(L)
+        assert_close(y, want, f"decode bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
+        assert_tight(y, want, f"decode bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
+        assert torch.equal(y, run_tiled(D, prep)), "two identical calls differ"
+        g = D["g_idx"] if desc_act else None
+        assert_tight(y, ops.gemm(D["x"], D["qweight"], D["qzeros"], D["scales"], g, D.get("bias"), bits, gs).cpu(),
+                     "decode vs the unprepared kernels")
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("M", [1, 8])
+def test_tiled_decode_split_k(dev, bits, M):
+    # a forced split of K over workgroups (what a long K with many rows needs): partial sums and the reduce pass
+    K, N, gs = 4096, 352, 128
+    L = layer(1700 + M, K, N, bits, gs, True, M=M, bias=True)
+    D = to_dev(L, dev)
+    prep = prepare(D)
+    plan = _lib.select_tiled(M, K, N, bits, gs)
+    for split in (2, 4):
+        plan.split_k = plan.grid_y = split
+        plan.k_chunk = -(-(K // 64) // (split * plan.waves_k))
+        plan.workspace_bytes = 16384 + split * M * N * 4
+        y = run_tiled(D, prep, plan=plan)
+        assert_close(y, expected_output(L), f"decode split={split}")
+        assert_tight(y, expected_output(L), f"decode split={split}")
+        assert torch.equal(y, run_tiled(D, prep, plan=plan))
+
+
+DECODE_FULL = [
+    ("c1-int4-4096x4096", 4, 4096, 4096, 128, False, [1, 2, 4, 8]),
+    ("c2-int3-4096x11008-act", 3, 4096, 11008, 128, True, [1, 2, 8]),
+    ("int4-4096x11008-act", 4, 4096, 11008, 128, True, [1, 4]),
+    ("c3-int4-11008x4096", 4, 11008, 4096, 128, False, [1, 2, 4, 8]),
+    ("int3-11008x4096-act", 3, 11008, 4096, 128, True, [1, 8]),
+    ("c5-int3-9216x9216-act-g1", 3, 9216, 9216, -1, True, [1]),
+    ("c5-int3-9216x36864-act-g1", 3, 9216, 36864, -1, True, [1]),
+    ("c5-int3-36864x9216-act-g1", 3, 36864, 9216, -1, True, [1]),
+]
+
+
+@pytest.mark.parametrize("name,bits,K,N,gs,desc_act,Ms", DECODE_FULL, ids=[f[0] for f in DECODE_FULL])
+def test_tiled_decode_full_size(dev, name, bits, K, N, gs, desc_act, Ms):
+    L = layer(7300 + [f[0] for f in DECODE_FULL].index(name), K, N, bits, gs, desc_act, M=max(Ms))
+    D = to_dev(L, dev)
+    w16 = expected_weight(L)
+    prep = prepare(D)
+    for M in Ms:
+        x = L["x"][:M].contiguous()
+        y = run_tiled(D, prep, x=x.to(dev))
+        want = expected_output(L, x=x, w16=w16)
+        assert_close(y, want, f"decode {name} M={M}")
+        assert_tight(y, want, f"decode {name} M={M}")
+        assert torch.equal(y, run_tiled(D, prep, x=x.to(dev))), f"decode {name} M={M}: two identical calls differ"
 
 
 TILED_FULL = [
