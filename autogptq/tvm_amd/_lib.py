@@ -38,6 +38,7 @@ ABI_SYMBOLS = (
     "gptq_hip_tiled_bytes",
     "gptq_hip_tile_prepare",
     "gptq_hip_select_tiled",
+    "gptq_hip_select_tiled_decode",
     "gptq_hip_gemm_tiled",
     "gptq_hip_dequant",
     "gptq_hip_strerror",
@@ -119,6 +120,8 @@ def lib() -> ctypes.CDLL:
     l.gptq_hip_tile_prepare.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
     l.gptq_hip_select_tiled.restype = i
     l.gptq_hip_select_tiled.argtypes = [i, i, i, i, i, ctypes.POINTER(Plan)]
+    l.gptq_hip_select_tiled_decode.restype = i
+    l.gptq_hip_select_tiled_decode.argtypes = [i, i, i, i, i, ctypes.POINTER(Plan)]
     l.gptq_hip_gemm_tiled.restype = i
     l.gptq_hip_gemm_tiled.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
     l.gptq_hip_dequant.restype = i
@@ -153,9 +156,11 @@ def select(M: int, K: int, N: int, bits: int, group_size: int, act_order: bool) 
     return plan
 
 
-def select_tiled(M: int, K: int, N: int, bits: int, group_size: int) -> Plan:
+def select_tiled(M: int, K: int, N: int, bits: int, group_size: int, decode: bool = False) -> Plan:
+    """The plan of the tiled family; ``decode=True`` asks for its decode kernel (M <= 8) whatever M."""
     plan = Plan()
-    rc = lib().gptq_hip_select_tiled(M, K, N, bits, group_size, ctypes.byref(plan))
+    fn = lib().gptq_hip_select_tiled_decode if decode else lib().gptq_hip_select_tiled
+    rc = fn(M, K, N, bits, group_size, ctypes.byref(plan))
     if rc != OK:
         raise GptqHipError(rc, f"gptq_hip_select_tiled(M={M}, K={K}, N={N}, bits={bits}, group_size={group_size})")
     return plan

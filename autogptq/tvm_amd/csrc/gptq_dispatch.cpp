@@ -472,16 +472,24 @@ extern "C" int gptq_hip_plan_for(int kernel, int M, int K, int N, int bits, int 
 // TILED: a workgroup per 64 columns and block of 32 * row_tiles rows, four waves along K; workgroups along K
 // when the column tiles alone leave most CUs idle (their fp32 tiles cross the workspace, so the split stays
 // within 3x the packed weights of traffic).
-extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan)
+static int tiled_args_ok(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan)
 {
     if (!plan) return GPTQ_HIP_ERR_BAD_ARG;
     memset(plan, 0, sizeof(*plan));
     if (bits != 3 && bits != 4) return GPTQ_HIP_ERR_BAD_ARG;
     if (M < 1 || K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;
     if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
+    if (!gptq::tiled_qualifies(K, N, bits, group_size == -1 ? K : group_size)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    return GPTQ_HIP_OK;
+}
+
+extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan)
+{
+    const int ok = tiled_args_ok(M, K, N, bits, group_size, plan);
+    if (ok != GPTQ_HIP_OK) return ok;
+    if (M > gptq::kDecodeMaxRows) return GPTQ_HIP_ERR_UNSUPPORTED;
     const int gs = group_size == -1 ? K : group_size;
-    if (!gptq::tiled_qualifies(K, N, bits, gs)) return GPTQ_HIP_ERR_UNSUPPORTED;
-    if (M <= gptq::kDecodeMaxRows) {
+    {
         // Decode: a workgroup per column tile of 32, enough waves along K to give the chip ~1000 waves, K cut
         // over workgroups only when the staged x would not fit LDS.
         const int mr = gptq::tiled_decode_rows(M);
@@ -514,6 +522,19 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
         }
         return GPTQ_HIP_ERR_UNSUPPORTED;
     }
+}
+
+extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan)
+{
+    // Up to four rows the decode kernel (one matrix instruction set per lane block); from five rows on its
+    // cost grows with the rows (two sets, x staged per row) and the matmul kernel with one 32-row tile is
+    // faster: 14.6 against 24.6 us at eight rows of a 4096 x 11008 layer.
+    if (M >= 1 && M <= gptq::kDecodeSelectRows) {
+        const int rc = gptq_hip_select_tiled_decode(M, K, N, bits, group_size, plan);
+        if (rc != GPTQ_HIP_ERR_UNSUPPORTED || !plan) return rc;
+    }
+    const int ok = tiled_args_ok(M, K, N, bits, group_size, plan);
+    if (ok != GPTQ_HIP_OK) return ok;
     const int at = gptq::tiled_row_tiles(M), rw = 1, kwv = 4;
     const int rows = 32 * at * rw;
     const int m_blocks = ceil_div(M, rows);

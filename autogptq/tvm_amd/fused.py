@@ -38,7 +38,7 @@ def concat_qlinears(layers: Sequence[QuantLinear]) -> QuantLinear:
     out = sum(l.outfeatures for l in layers)
     fused = QuantLinear(first.bits, first.groupsize, first.infeatures, out, first.bias is not None,
                         kernel_switch_threshold=first.kernel_switch_threshold,
-                        sort_for_decode=first.sort_for_decode)
+                        sort_for_decode=first.sort_for_decode, tile_for_prefill=first.tile_for_prefill)
     fused.qweight = torch.cat([l.qweight for l in layers], dim=1).contiguous()
     fused.qzeros = torch.cat([l.qzeros for l in layers], dim=1).contiguous()    # 32 columns per `bits` words
     fused.scales = torch.cat([l.scales for l in layers], dim=1).contiguous()

@@ -131,7 +131,7 @@ def load_quantized_state(model: nn.Module, state: Dict[str, torch.Tensor], devic
 def from_quantized(save_dir: str, device="cuda:0", model_basename: Optional[str] = None,
                    use_safetensors: bool = True, ignore_layers: Iterable[str] = ("lm_head",),
                    trust_remote_code: bool = False, fuse_shared_inputs: bool = False,
-                   prepare_decode: bool = False):
+                   prepare_decode: bool = False, prepare_tiled: bool = False, compact: bool = False):
     """Builds the ``transformers`` causal LM described by ``save_dir/config.json`` with every linear
     layer (except ``ignore_layers`` prefixes: the reference skips ``lm_head`` and the modules outside
     the decoder stack) replaced by ``QuantLinear``, and fills it from
@@ -139,7 +139,10 @@ def from_quantized(save_dir: str, device="cuda:0", model_basename: Optional[str]
     q/k/v and gate/up projections into one product each (``fused.fuse_shared_input_layers``; an inference
     optimisation the reference does not have: the state-dict names of those layers change).
     ``prepare_decode`` builds the sorted copies of activation-order layers now instead of on their first
-    decode-size call (needed before capturing the model in a graph: the preparation allocates).
+    decode-size call (needed before capturing the model in a graph: the preparation allocates);
+    ``prepare_tiled`` does the same for the copies in the tiled format that prompt-size calls use.
+    ``compact`` keeps the tiled copy as the only weights of every layer it covers (``QuantLinear.compact``:
+    no second or third copy in device memory, and no checkpoint tensors left to save).
     Returns ``(model, quantize_config)``."""
     import accelerate
     from transformers import AutoConfig, AutoModelForCausalLM
@@ -176,10 +179,15 @@ def from_quantized(save_dir: str, device="cuda:0", model_basename: Optional[str]
         from .fused import fuse_shared_input_layers
 
         fuse_shared_input_layers(model)
-    if prepare_decode:
-        for mod in model.modules():
-            if isinstance(mod, QuantLinear) and mod.sort_for_decode:
-                mod.prepare_decode()
+    for mod in model.modules():
+        if not isinstance(mod, QuantLinear):
+            continue
+        if compact and mod.compact():
+            continue
+        if prepare_decode and mod.sort_for_decode:
+            mod.prepare_decode()
+        if prepare_tiled and mod.tile_for_prefill:
+            mod.prepare_tiled()
     seqlen = 4096
     for key in ("max_position_embeddings", "seq_length", "n_positions"):
         if key in model.config.to_dict():

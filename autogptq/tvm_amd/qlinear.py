@@ -16,7 +16,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib, ops
-from .pack import pack_qweight, pack_qzeros
+from .pack import pack_qweight, pack_qzeros, tiled_qualifies
 
 
 class _ProductWithInputGrad(torch.autograd.Function):
@@ -41,7 +41,7 @@ class QuantLinear(nn.Module):
     FUSED_BITS = (3, 4)             # those the fused kernels cover; 2 and 8 run as dequant + library GEMM
 
     def __init__(self, bits, groupsize, infeatures, outfeatures, bias, kernel_switch_threshold=1024,
-                 sort_for_decode=True):
+                 sort_for_decode=True, tile_for_prefill=True):
         super().__init__()
         if bits not in self.SUPPORTED_BITS:
             raise NotImplementedError("Only 2,3,4,8 bits are supported.")
@@ -78,6 +78,13 @@ class QuantLinear(nn.Module):
         self.sort_for_decode = sort_for_decode
         self._sorted = None   # (key, (qweight_sorted, kmap) or None)
         self._sorted_plans = {}  # M -> plan of the sorted path, or None where it does not apply
+        # Every fused layer whose groups are whole multiples of 32 channels: on the first call with a row count
+        # the tiled kernels are faster at (see _tiled_wins), keep a copy of the layer in the order the matrix
+        # instructions consume (gptq_hip_tile_prepare).  Costs the layer's packed size again; False keeps
+        # the checkpoint's tensors (and the sorted copy) only.  compact() makes it the only copy.
+        self.tile_for_prefill = tile_for_prefill
+        self._tiled = None    # (key, (qtile, sz, xsrc, kinv) or None)
+        self._compact = False
 
     # ------------------------------------------------------------------ packing
     def pack(self, linear, scales, zeros, g_idx=None):
@@ -142,17 +149,83 @@ class QuantLinear(nn.Module):
             self._sorted = (key, tensors)
         return self._sorted[1]
 
+    def _whole_groups(self, g):
+        """The one check the preparation kernels cannot make: every group holds exactly ``groupsize`` channels."""
+        K, gs = self.infeatures, self.groupsize
+        counts = torch.bincount(g.to(torch.int64), minlength=K // gs)
+        return counts.numel() == K // gs and bool((counts == gs).all())
+
     def _sort_on_gpu(self, q, g):
-        """``pack.sort_channels_by_group`` through the library's own kernels (gptq_hip_sort_channels), after
-        the one check they cannot make: that every group holds exactly ``groupsize`` channels."""
+        """``pack.sort_channels_by_group`` through the library's own kernels (gptq_hip_sort_channels)."""
         K, gs = self.infeatures, self.groupsize
         klane = 8 if self.bits == 4 else 32
-        if K >= 65536 or K % gs != 0 or gs % klane != 0:
-            return None
-        counts = torch.bincount(g.to(torch.int64), minlength=K // gs)
-        if counts.numel() != K // gs or not bool((counts == gs).all()):
+        if K >= 65536 or K % gs != 0 or gs % klane != 0 or not self._whole_groups(g):
             return None
         return ops.sort_channels(q, g, self.bits, self.groupsize)
+
+    def prepare_tiled(self):
+        """Builds (once per distinct storage of the packed tensors) the layer in the tiled format; returns
+        ``(qtile, sz, xsrc, kinv)`` or None when the format does not cover the layer.  ``forward`` calls this
+        lazily; loaders may call it up front (it synchronises once, for the check of the group sizes)."""
+        if self._compact:
+            return self._tiled[1]
+        g = self._kernel_g_idx()
+        key = tuple((t.data_ptr(), t._version) for t in (self.qweight, self.qzeros, self.scales)) + (
+            None if g is None else (g.data_ptr(), g._version),)
+        if self._tiled is None or self._tiled[0] != key:
+            tensors = None
+            if (self.qweight.device.type == "cuda" and self.bits in self.FUSED_BITS
+                    and tiled_qualifies(self.infeatures, self.outfeatures, self.bits, self.groupsize)
+                    and (g is None or self._whole_groups(g))):
+                tensors = ops.tile_prepare(self.qweight, self.qzeros, self.scales, g, self.bits, self.groupsize)
+            self._tiled = (key, tensors)
+        return self._tiled[1]
+
+    def compact(self):
+        """Keeps the tiled copy as the layer's ONLY weights: every row count then runs on the tiled kernels and
+        the checkpoint's tensors are released (empty buffers stay in their place, so ``state_dict`` no longer
+        holds the layer: save before, or reload).  Returns True when the layer is compact afterwards."""
+        if self._compact:
+            return True
+        tensors = self.prepare_tiled()
+        if tensors is None:
+            return False
+        act = self._kernel_g_idx() is not None
+        self._tiled = (None, tensors if act else (tensors[0], tensors[1], None, None))
+        self._compact = True
+        self._sorted = None
+        dev = self.qweight.device
+        self.qweight = torch.empty((0, self.outfeatures), dtype=torch.int32, device=dev)
+        self.qzeros = torch.empty((0, self.qzeros.shape[1]), dtype=torch.int32, device=dev)
+        self.scales = torch.empty((0, self.outfeatures), dtype=torch.float16, device=dev)
+        return True
+
+    def _apply(self, fn, *args, **kwargs):
+        # the tiled copy of a compact layer is its weights: it moves with the module (a prepared copy beside
+        # the checkpoint tensors is rebuilt instead, when their storage changes)
+        super()._apply(fn, *args, **kwargs)
+        if self._compact:
+            self._tiled = (None, tuple(None if t is None else fn(t) for t in self._tiled[1]))
+        return self
+
+    def _tiled_wins(self, M, act_order):
+        """Where the tiled kernels were measured faster than the ones that read the checkpoint layout (or its
+        sorted copy), on MI355X with the weights cold, group size 128, 3 and 4 bits:
+          * up to 4 rows (its decode kernel, one workgroup per 32 columns): layers of up to 8192 columns, where
+            every workgroup has a CU to itself: 4096 x 4096 6.2-7.9 us against 7.1-10.9; 11008 x 4096 with an
+            activation order 11.9/13.0 against 13.4/15.5 at one and two rows, behind from four rows on and
+            without an activation order (14.8 against 12.9); 4096 x 11008 9.2 against 8.2;
+          * 5 to 16 rows: never (4096 x 11008, 8 rows: 14.6 against 13.4);
+          * 17 to 128 rows: everywhere within 4 % or better (4096 x 11008 with an activation order, 32/64/128
+            rows: 14.8/19.2/26.6 against 18.1/22.1/34.1 us);
+          * above 128 rows: K up to 8192 (4096 x 11008, 512 rows: 75 against 95; 11008 x 4096: 127 against 81,
+            where every workgroup pulls 2.8 MB of x fragments and they no longer stay in one L2)."""
+        K, N = self.infeatures, self.outfeatures
+        if M <= 4:
+            return N <= 8192 and (K <= 4096 or (act_order and M <= 2))
+        if M <= 16:
+            return False
+        return M <= 128 or K <= 8192
 
     def _decode_sorted(self, x2):
         """The decode product through the sorted copy, or None when that path does not apply."""
@@ -183,15 +256,27 @@ class QuantLinear(nn.Module):
 
     def _product(self, x2: torch.Tensor) -> torch.Tensor:
         """y[M, N] = x2[M, K] @ W + bias for a contiguous fp16 x2."""
+        M = x2.shape[0]
+        if self._compact:
+            qtile, sz, xsrc, kinv = self._tiled[1]
+            return ops.gemm_tiled(x2, qtile, sz, xsrc, kinv, self.bias, self.bits, self.groupsize)
         try:
             if self.bits not in self.FUSED_BITS:
                 raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, "width without a fused kernel")
+            g = self._kernel_g_idx()
+            tiled = None
+            if self.tile_for_prefill and M > 0 and self._tiled_wins(M, g is not None):
+                tiled = self.prepare_tiled()
             threshold = self.kernel_switch_threshold
-            if threshold and self.act_order_switch_threshold and self._kernel_g_idx() is not None:
-                threshold = min(threshold, self.act_order_switch_threshold)
-            if threshold and x2.shape[0] >= threshold:
+            if threshold and self.act_order_switch_threshold and g is not None and tiled is None:
+                threshold = min(threshold, self.act_order_switch_threshold)   # (the tiled kernels do not pay for the order)
+            if threshold and M >= threshold:
                 raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, "above kernel_switch_threshold")
-            out = self._decode_sorted(x2) if (self.sort_for_decode and 0 < x2.shape[0] <= ops.SORTED_MAX_ROWS) else None
+            if tiled is not None:
+                act = g is not None
+                return ops.gemm_tiled(x2, tiled[0], tiled[1], tiled[2] if act else None, tiled[3] if act else None,
+                                      self.bias, self.bits, self.groupsize)
+            out = self._decode_sorted(x2) if (self.sort_for_decode and 0 < M <= ops.SORTED_MAX_ROWS) else None
             if out is None:
                 out = ops.gemm(x2, self.qweight, self.qzeros, self.scales, self._kernel_g_idx(), self.bias,
                                self.bits, self.groupsize)
@@ -209,6 +294,11 @@ class QuantLinear(nn.Module):
 
     def dequantize(self) -> torch.Tensor:
         """fp16 [infeatures, outfeatures], the weight the reference materialises on every call."""
+        if self._compact:
+            # the tiled kernels form the same rounded fp16 weights: the product with the identity is W itself
+            eye = torch.eye(self.infeatures, dtype=torch.float16, device=self._tiled[1][0].device)
+            qtile, sz, xsrc, kinv = self._tiled[1]
+            return ops.gemm_tiled(eye, qtile, sz, xsrc, kinv, None, self.bits, self.groupsize)
         return ops.dequant(self.qweight, self.qzeros, self.scales, self._kernel_g_idx(), self.bits, self.groupsize)
 
     def extra_repr(self) -> str:

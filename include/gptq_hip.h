@@ -197,6 +197,11 @@ int gptq_hip_tile_prepare(const int32_t *qweight, const int32_t *qzeros, const v
  * tile table per M bucket (pycuda_warpper.py:77-127,150-189). */
 int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan);
 
+/* The plan of the family's decode kernel (GPTQ_HIP_KERNEL_TILED_DECODE) for M <= 8 rows; gptq_hip_select_tiled
+ * chooses it by itself up to four rows and the matmul kernel above that.  No counterpart in the reference, whose
+ * GEMV handler takes one row (pycuda_warpper.py:150-152). */
+int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan);
+
 /*
  * y = x @ W (+ bias) on a layer in the tiled format, any M; replaces the same handler call as gptq_hip_gemm
  * (pycuda_warpper.py:138, qlinear_tvm.py:123,150).  x and y are in the layer's own channel order (xsrc = kinv =

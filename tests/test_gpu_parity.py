@@ -538,7 +538,8 @@ def test_sorted_decode_integer_exact_and_rejections(dev):
 
 @pytest.mark.parametrize("bits", [3, 4])
 def test_quantlinear_decode_uses_the_sorted_copy(dev, bits):
-    K, N, gs = 2048, 8192, 128   # wide enough for the decode family to take two rows as well
+    K, N, gs = 2048, 12288, 128   # wide enough for the decode family to take two rows as well (and for the
+    #                               module to prefer the sorted copy over the tiled one at these row counts)
     L = layer(44, K, N, bits, gs, True, M=2, bias=True)
     q = QuantLinear(bits, gs, K, N, True)
     q.load_state_dict({k: L[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})

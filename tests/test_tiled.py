@@ -7,6 +7,7 @@ import pytest
 import torch
 
 from autogptq.tvm_amd import _lib, ops, pack
+from autogptq.tvm_amd.qlinear import QuantLinear
 from tests.parity_util import assert_close, assert_tight, expected_output, expected_weight, layer, to_dev
 
 pytestmark = pytest.mark.gpu
@@ -153,14 +154,17 @@ def test_tiled_decode_rows_and_shapes(dev, bits, K, N, gs, M):
     for desc_act in (False, True):
         L = layer(1600 + K + M, K, N, bits, gs, desc_act, M=M, bias=(M % 2 == 0))
         D = to_dev(L, dev)
-        plan = _lib.select_tiled(M, K, N, bits, gs)
+        plan = _lib.select_tiled(M, K, N, bits, gs, decode=True)
         assert plan.kernel == _lib.KERNEL_TILED_DECODE and plan.row_tiles in (1, 2, 4, 8) and plan.row_tiles >= M
+        # the family's own choice: this kernel up to four rows, the matmul kernel above
+        own = _lib.select_tiled(M, K, N, bits, gs)
+        assert own.kernel == (_lib.KERNEL_TILED_DECODE if M <= 4 else _lib.KERNEL_TILED)
         prep = prepare(D)
-        y = run_tiled(D, prep)
+        y = run_tiled(D, prep, plan=plan)
         want = expected_output(L)
         assert_close(y, want, f"decode bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
         assert_tight(y, want, f"decode bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
-        assert torch.equal(y, run_tiled(D, prep)), "two identical calls differ"
+        assert torch.equal(y, run_tiled(D, prep, plan=plan)), "two identical calls differ"
         g = D["g_idx"] if desc_act else None
         assert_tight(y, ops.gemm(D["x"], D["qweight"], D["qzeros"], D["scales"], g, D.get("bias"), bits, gs).cpu(),
                      "decode vs the unprepared kernels")
@@ -174,7 +178,7 @@ def test_tiled_decode_split_k(dev, bits, M):
     L = layer(1700 + M, K, N, bits, gs, True, M=M, bias=True)
     D = to_dev(L, dev)
     prep = prepare(D)
-    plan = _lib.select_tiled(M, K, N, bits, gs)
+    plan = _lib.select_tiled(M, K, N, bits, gs, decode=True)
     for split in (2, 4):
         plan.split_k = plan.grid_y = split
         plan.k_chunk = -(-(K // 64) // (split * plan.waves_k))
@@ -205,11 +209,12 @@ def test_tiled_decode_full_size(dev, name, bits, K, N, gs, desc_act, Ms):
     prep = prepare(D)
     for M in Ms:
         x = L["x"][:M].contiguous()
-        y = run_tiled(D, prep, x=x.to(dev))
+        plan = _lib.select_tiled(M, K, N, bits, gs, decode=True)
+        y = run_tiled(D, prep, x=x.to(dev), plan=plan)
         want = expected_output(L, x=x, w16=w16)
         assert_close(y, want, f"decode {name} M={M}")
         assert_tight(y, want, f"decode {name} M={M}")
-        assert torch.equal(y, run_tiled(D, prep, x=x.to(dev))), f"decode {name} M={M}: two identical calls differ"
+        assert torch.equal(y, run_tiled(D, prep, x=x.to(dev), plan=plan)), f"decode {name} M={M}: two identical calls differ"
 
 
 TILED_FULL = [
@@ -236,3 +241,63 @@ def test_tiled_full_size(dev, name, bits, K, N, gs, desc_act, Ms):
         assert_close(y, want, f"tiled {name} M={M}")
         assert_tight(y, want, f"tiled {name} M={M}")
         assert torch.equal(y, run_tiled(D, prep, x=x.to(dev))), f"tiled {name} M={M}: two identical calls differ"
+
+
+def module_of(L, dev, **kw):
+    q = QuantLinear(L["bits"], L["group_size"], L["K"], L["N"], L.get("bias") is not None, **kw)
+    q.load_state_dict({k: L[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias") if L.get(k) is not None})
+    return q.to(dev)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("desc_act", [False, True])
+def test_quantlinear_routes_prompt_sizes_to_the_tiled_copy(dev, bits, desc_act):
+    K, N, gs = 1024, 416, 128
+    L = layer(1800 + bits, K, N, bits, gs, desc_act, M=150, bias=True)
+    q = module_of(L, dev)
+    assert q._tiled is None
+    x = L["x"].to(dev)
+    y8 = q(x[:8])                                  # 5..16 rows stay on the checkpoint layout (or its sorted copy)
+    assert q._tiled is None
+    y40, y150, y2 = q(x[:40]), q(x), q(x[:2])      # prompt sizes, and a narrow layer's decode sizes
+    assert q._tiled is not None and q._tiled[1] is not None
+    want = expected_output(L)
+    for y, M in ((y2, 2), (y8, 8), (y40, 40), (y150, 150)):
+        assert_close(y, want[:M], f"module, {M} rows")
+        assert_tight(y, want[:M], f"module, {M} rows")
+    # the same numbers (to the tight bound) from the checkpoint's own tensors
+    q.tile_for_prefill = False
+    assert_tight(q(x[:40]), y40.cpu(), "module, tiled against unprepared")
+    q.tile_for_prefill = True
+    # new weights invalidate the copy
+    L2 = layer(1810 + bits, K, N, bits, gs, desc_act, M=40, bias=True)
+    q.load_state_dict({k: L2[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})
+    assert_close(q(L2["x"].to(dev)), expected_output(L2), "module after reload")
+    # a layer the format does not cover (groups of 16 channels) keeps working
+    L3 = layer(1820, 256, 64, 4, 16, False, M=40)
+    q3 = module_of(L3, dev)
+    assert_close(q3(L3["x"].to(dev)), expected_output(L3), "module, uncovered by the format")
+    assert q3._tiled is not None and q3._tiled[1] is None and not q3.compact()
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("desc_act", [False, True])
+def test_quantlinear_compact_keeps_one_copy(dev, bits, desc_act):
+    K, N, gs = 1024, 416, 128
+    L = layer(1900 + bits, K, N, bits, gs, desc_act, M=300, bias=True)
+    q = module_of(L, dev, kernel_switch_threshold=256)
+    assert q.compact() and q.compact()
+    assert q.qweight.numel() == 0 and q.qzeros.numel() == 0 and q.scales.numel() == 0 and q._sorted is None
+    x = L["x"].to(dev)
+    want = expected_output(L)
+    for M in (1, 3, 8, 40, 300):                   # 300 rows: above the threshold, still the tiled kernels
+        y = q(x[:M])
+        assert_close(y, want[:M], f"compact module, {M} rows")
+        assert_tight(y, want[:M], f"compact module, {M} rows")
+    assert torch.equal(q.dequantize().cpu().view(torch.int16), expected_weight(L).view(torch.int16))
+    q = q.to(dev)                                  # moving the module keeps the copy
+    assert_close(q(x[:40]), want[:40], "compact module after .to()")
+    # the gradient for x still works (adapters on top of frozen layers)
+    xg = x[:4].clone().requires_grad_(True)
+    q(xg).float().sum().backward()
+    assert xg.grad is not None and xg.grad.shape == xg.shape
