@@ -266,6 +266,25 @@ def gemm_tiled(x: torch.Tensor, qtile: torch.Tensor, sz: torch.Tensor, xsrc: Opt
     return out
 
 
+def tiled_wins(M: int, K: int, N: int, act_order: bool) -> bool:
+    """Where the tiled kernels were measured faster than the ones that read the checkpoint layout (or its
+    sorted copy), on MI355X with the weights cold, group size 128, 3 and 4 bits:
+      * up to 4 rows (its decode kernel, one workgroup per 32 columns): layers of up to 8192 columns, where
+        every workgroup has a CU to itself: 4096 x 4096 6.2-7.9 us against 7.1-10.9; 11008 x 4096 with an
+        activation order 11.9/13.0 against 13.4/15.5 at one and two rows, behind from four rows on and
+        without an activation order (14.8 against 12.9); 4096 x 11008 9.2 against 8.2;
+      * 5 to 16 rows: never (4096 x 11008, 8 rows: 14.6 against 13.4);
+      * 17 to 128 rows: everywhere within 4 % or better (4096 x 11008 with an activation order, 32/64/128
+        rows: 14.8/19.2/26.6 against 18.1/22.1/34.1 us);
+      * above 128 rows: K up to 8192 (4096 x 11008, 512 rows: 75 against 95; 11008 x 4096: 127 against 81,
+        where every workgroup pulls 2.8 MB of x fragments and they no longer stay in one L2)."""
+    if M <= 4:
+        return N <= 8192 and (K <= 4096 or (act_order and M <= 2))
+    if M <= 16:
+        return False
+    return M <= 128 or K <= 8192
+
+
 def dequant(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
             g_idx: Optional[torch.Tensor], bits: int, group_size: int) -> torch.Tensor:
     """The materialised fp16 weight [K, N], bit-exact with the reference's dequantisation."""

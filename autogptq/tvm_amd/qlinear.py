@@ -79,7 +79,7 @@ class QuantLinear(nn.Module):
         self._sorted = None   # (key, (qweight_sorted, kmap) or None)
         self._sorted_plans = {}  # M -> plan of the sorted path, or None where it does not apply
         # Every fused layer whose groups are whole multiples of 32 channels: on the first call with a row count
-        # the tiled kernels are faster at (see _tiled_wins), keep a copy of the layer in the order the matrix
+        # the tiled kernels are faster at (ops.tiled_wins), keep a copy of the layer in the order the matrix
         # instructions consume (gptq_hip_tile_prepare).  Costs the layer's packed size again; False keeps
         # the checkpoint's tensors (and the sorted copy) only.  compact() makes it the only copy.
         self.tile_for_prefill = tile_for_prefill
@@ -208,24 +208,6 @@ class QuantLinear(nn.Module):
             self._tiled = (None, tuple(None if t is None else fn(t) for t in self._tiled[1]))
         return self
 
-    def _tiled_wins(self, M, act_order):
-        """Where the tiled kernels were measured faster than the ones that read the checkpoint layout (or its
-        sorted copy), on MI355X with the weights cold, group size 128, 3 and 4 bits:
-          * up to 4 rows (its decode kernel, one workgroup per 32 columns): layers of up to 8192 columns, where
-            every workgroup has a CU to itself: 4096 x 4096 6.2-7.9 us against 7.1-10.9; 11008 x 4096 with an
-            activation order 11.9/13.0 against 13.4/15.5 at one and two rows, behind from four rows on and
-            without an activation order (14.8 against 12.9); 4096 x 11008 9.2 against 8.2;
-          * 5 to 16 rows: never (4096 x 11008, 8 rows: 14.6 against 13.4);
-          * 17 to 128 rows: everywhere within 4 % or better (4096 x 11008 with an activation order, 32/64/128
-            rows: 14.8/19.2/26.6 against 18.1/22.1/34.1 us);
-          * above 128 rows: K up to 8192 (4096 x 11008, 512 rows: 75 against 95; 11008 x 4096: 127 against 81,
-            where every workgroup pulls 2.8 MB of x fragments and they no longer stay in one L2)."""
-        K, N = self.infeatures, self.outfeatures
-        if M <= 4:
-            return N <= 8192 and (K <= 4096 or (act_order and M <= 2))
-        if M <= 16:
-            return False
-        return M <= 128 or K <= 8192
 
     def _decode_sorted(self, x2):
         """The decode product through the sorted copy, or None when that path does not apply."""
@@ -265,7 +247,7 @@ class QuantLinear(nn.Module):
                 raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, "width without a fused kernel")
             g = self._kernel_g_idx()
             tiled = None
-            if self.tile_for_prefill and M > 0 and self._tiled_wins(M, g is not None):
+            if self.tile_for_prefill and M > 0 and ops.tiled_wins(M, self.infeatures, self.outfeatures, g is not None):
                 tiled = self.prepare_tiled()
             threshold = self.kernel_switch_threshold
             if threshold and self.act_order_switch_threshold and g is not None and tiled is None:

@@ -5,9 +5,11 @@ Default workload: the headline configuration of the reference's benchmarks -- 3-
 desc_act=True (g_idx from a random permutation), synthetic seeded tensors.  One "step" is one
 call of the C-ABI entry point that ``QuantLinear.forward`` makes for that shape, on tensors already
 resident in HBM: ``gptq_hip_gemm_sorted`` for decode sizes on activation-order layers (the layer
-as the module holds it after its one-time load preparation, the channel sort; ``--unprepared``
-times ``gptq_hip_gemm`` on the checkpoint's own tensors instead, and the default run reports that
-figure too under ``timing.unprepared_us``), ``gptq_hip_gemm`` otherwise.  Steps rotate
+as the module holds it after its one-time load preparation, the channel sort),
+``gptq_hip_gemm_tiled`` where the module routes to its copy in the tiled format (prompt sizes; decode
+sizes of layers up to 8192 columns wide), ``gptq_hip_gemm`` otherwise; ``--unprepared`` times
+``gptq_hip_gemm`` on the checkpoint's own tensors instead, and the default run reports that figure
+too under ``timing.unprepared_us``.  Steps rotate
 over enough distinct weight copies to exceed twice the 256 MB Infinity Cache, so every step
 streams its packed weights from HBM (cache-cold).
 
@@ -102,11 +104,12 @@ def measured_traffic(workload: str, plan_kernel: int):
     return int(e["fetch_bytes"]) + int(e["write_bytes"]), e.get("source")
 
 
-def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int = 0, prepared: bool = False):
-    """prepared: the layer as QuantLinear holds it for decode-size calls after its one-time
-    preparation (channels of an activation-order layer sorted by group), run through
-    gptq_hip_gemm_sorted; only for workloads that path covers (see prepared_applies)."""
-    from autogptq.tvm_amd import _lib
+def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int = 0, prepared=None):
+    """prepared: the layer as QuantLinear holds it after its one-time preparation: "sorted" (channels of
+    an activation-order layer sorted by group, run through gptq_hip_gemm_sorted), "tiled" (the tiled
+    format, run through gptq_hip_gemm_tiled), or None (the checkpoint's tensors, gptq_hip_gemm);
+    prepared_mode(name) is the module's own choice."""
+    from autogptq.tvm_amd import _lib, ops
     from autogptq.tvm_amd.pack import sort_channels_by_group, synth_layer
 
     bits, K, N, gs, desc_act, M = WORKLOADS[name]
@@ -114,26 +117,33 @@ def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int =
     wbytes = K * N * bits // 8
     copies = max(2, -(-2 * INFINITY_CACHE_BYTES // wbytes))
     gen = torch.Generator().manual_seed(99)
-    qweights = [L["qweight"].to(dev)]
-    for _ in range(copies - 1):
-        # distinct random packed words: every int32 pattern is a valid block of codes
-        qweights.append(torch.randint(-(1 << 31), (1 << 31) - 1, L["qweight"].shape, generator=gen,
-                                      dtype=torch.int64).to(torch.int32).to(dev))
     case = {
         "name": name, "bits": bits, "K": K, "N": N, "gs": gs, "desc_act": desc_act, "M": M, "L": L,
-        "qweights": qweights,
         "qzeros": L["qzeros"].to(dev), "scales": L["scales"].to(dev),
         "g_idx": L["g_idx"].to(dev) if desc_act else None,
         "x": L["x"].to(dev), "y": torch.empty((M, N), dtype=torch.float16, device=dev),
-        "wbytes": wbytes, "flops": 2 * M * K * N, "kmap": None,
+        "wbytes": wbytes, "flops": 2 * M * K * N, "kmap": None, "tiled": None, "prepared": prepared,
     }
-    if prepared:
-        case["qweights"][0], case["kmap"] = sort_channels_by_group(qweights[0], case["g_idx"], bits, gs)
+    qweights = []
+    for c in range(copies):
+        # copy 0 is the seeded layer; the others are distinct random packed words (every int32 pattern is a
+        # valid block of codes)
+        q = L["qweight"].to(dev) if c == 0 else torch.randint(
+            -(1 << 31), (1 << 31) - 1, L["qweight"].shape, generator=gen, dtype=torch.int64).to(torch.int32).to(dev)
+        if prepared == "tiled":
+            qtile, sz, xsrc, kinv = ops.tile_prepare(q, case["qzeros"], case["scales"], case["g_idx"], bits, gs)
+            if c == 0:
+                case["tiled"] = (sz, xsrc if desc_act else None, kinv if desc_act else None)
+            q = qtile
+        qweights.append(q)
+    case["qweights"] = qweights
+    if prepared == "sorted":
+        qweights[0], case["kmap"] = sort_channels_by_group(qweights[0], case["g_idx"], bits, gs)
         case["g_idx"] = None
         desc_act = False  # the plan is that of contiguous groups
-    if prepared and not (kernel or split_k or waves_n):
-        from autogptq.tvm_amd import ops
-
+    if prepared == "tiled":
+        plan = _lib.select_tiled(M, K, N, bits, gs)
+    elif prepared == "sorted" and not (kernel or split_k or waves_n):
         plan = ops.sorted_plan(M, K, N, bits, gs)
     elif kernel or split_k or waves_n:
         if not kernel:
@@ -143,14 +153,19 @@ def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int =
         plan = _lib.select(M, K, N, bits, gs, desc_act)
     case["plan"] = plan
     ws_bytes = plan.workspace_bytes
-    if prepared:   # kernels that want x in the sorted order find it behind the plan's own bytes
+    if prepared == "sorted":   # kernels that want x in the sorted order find it behind the plan's own bytes
         ws_bytes = max(ws_bytes, _lib.lib().gptq_hip_sorted_workspace_bytes(M, K, N, bits, gs))
     case["ws_bytes"] = ws_bytes
     case["ws"] = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
     return case
 
 
-def prepared_applies(name: str) -> bool:
+ENTRY = {None: "gptq_hip_gemm_plan", "sorted": "gptq_hip_gemm_sorted", "tiled": "gptq_hip_gemm_tiled"}
+PREPARED_NOTE = {None: None, "sorted": "input channels sorted by group once at load",
+                 "tiled": "layer re-laid once at load into the tiled format (gptq_hip_tile_prepare)"}
+
+
+def sorted_applies(name: str) -> bool:
     from autogptq.tvm_amd import ops
 
     bits, K, N, gs, desc_act, M = WORKLOADS[name]
@@ -158,29 +173,51 @@ def prepared_applies(name: str) -> bool:
     return bool(desc_act and G > 1 and M <= ops.SORTED_MAX_ROWS and ops.sorted_plan(M, K, N, bits, gs) is not None)
 
 
+def tiled_applies(name: str) -> bool:
+    from autogptq.tvm_amd.pack import tiled_qualifies
+
+    bits, K, N, gs, desc_act, M = WORKLOADS[name]
+    return tiled_qualifies(K, N, bits, gs)
+
+
+def prepared_mode(name: str):
+    """The prepared copy QuantLinear.forward uses for this workload (qlinear.py: _product), or None."""
+    from autogptq.tvm_amd import ops
+
+    bits, K, N, gs, desc_act, M = WORKLOADS[name]
+    if tiled_applies(name) and ops.tiled_wins(M, K, N, desc_act):
+        return "tiled"
+    return "sorted" if sorted_applies(name) else None
+
+
 def make_step(case, dev):
-    """Returns step(i): one gptq_hip_gemm_plan (or gptq_hip_gemm_sorted) call on weight copy i
-    (pre-marshalled arguments)."""
+    """Returns step(i): one call of the case's entry point on weight copy i (pre-marshalled arguments)."""
     from autogptq.tvm_amd import _lib
 
     lib = _lib.lib()
-    fn = lib.gptq_hip_gemm_sorted if case["kmap"] is not None else lib.gptq_hip_gemm_plan
     vp = ctypes.c_void_p
-    gmap = case["kmap"] if case["kmap"] is not None else case["g_idx"]
-    common = dict(
-        x=vp(case["x"].data_ptr()), qz=vp(case["qzeros"].data_ptr()), sc=vp(case["scales"].data_ptr()),
-        g=vp(gmap.data_ptr()) if gmap is not None else None,
-        y=vp(case["y"].data_ptr()), ws=vp(case["ws"].data_ptr()) if case["ws_bytes"] else None,
-    )
+    ptr = lambda t: vp(t.data_ptr()) if t is not None else None
     qws = [vp(q.data_ptr()) for q in case["qweights"]]
-    wsb = case["ws_bytes"]
+    x, y = ptr(case["x"]), ptr(case["y"])
+    ws, wsb = (ptr(case["ws"]) if case["ws_bytes"] else None), case["ws_bytes"]
     M, K, N, bits, gs = case["M"], case["K"], case["N"], case["bits"], case["gs"]
     planp = ctypes.byref(case["plan"])
     n = len(qws)
+    if case["prepared"] == "tiled":
+        sz, xsrc, kinv = (ptr(t) for t in case["tiled"])
+
+        def step(i, stream):
+            rc = lib.gptq_hip_gemm_tiled(x, qws[i % n], sz, xsrc, kinv, None, y, ws, wsb, M, K, N, bits, gs, planp, stream)
+            if rc != 0:
+                raise RuntimeError(f"gptq_hip_gemm_tiled failed: {_lib.strerror(rc)}")
+
+        return step
+    fn = lib.gptq_hip_gemm_sorted if case["kmap"] is not None else lib.gptq_hip_gemm_plan
+    qz, sc = ptr(case["qzeros"]), ptr(case["scales"])
+    g = ptr(case["kmap"] if case["kmap"] is not None else case["g_idx"])
 
     def step(i, stream):
-        rc = fn(common["x"], qws[i % n], common["qz"], common["sc"], common["g"], None, common["y"],
-                common["ws"], wsb, M, K, N, bits, gs, planp, stream)
+        rc = fn(x, qws[i % n], qz, sc, g, None, y, ws, wsb, M, K, N, bits, gs, planp, stream)
         if rc != 0:
             raise RuntimeError(f"gptq_hip_gemm failed: {_lib.strerror(rc)}")
 
@@ -330,6 +367,9 @@ def main():
     ap.add_argument("--unprepared", action="store_true",
                     help="decode on activation-order layers: time gptq_hip_gemm on the checkpoint's tensors "
                          "instead of gptq_hip_gemm_sorted on the load-time prepared ones")
+    ap.add_argument("--prepared", default="auto", choices=("auto", "none", "sorted", "tiled"),
+                    help="which copy of the layer to run on: the module's own choice (auto), the checkpoint's "
+                         "tensors, the sorted copy or the tiled copy")
     ap.add_argument("--kernel", type=int, default=0, help="force a kernel family (1 gather, 2 grouped, 3 blocked)")
     ap.add_argument("--split-k", type=int, default=0, help="force the split-K factor")
     ap.add_argument("--waves-n", type=int, default=0, help="force the waves per workgroup along N (STREAM kernel: along K)")
@@ -358,7 +398,9 @@ def main():
                                                "kernel": "torch elementwise copy (int32)"}}))
         return
     forced = bool(args.kernel or args.split_k or args.waves_n)
-    prepared = prepared_applies(args.workload) and not args.unprepared and not forced
+    prepared = None if (args.unprepared or forced) else prepared_mode(args.workload)
+    if args.prepared != "auto" and not forced:
+        prepared = None if args.prepared == "none" else args.prepared
     case = build_case(args.workload, dev, args.kernel, args.split_k, args.waves_n, prepared=prepared)
     ok, max_err = check_case(case, dev)
     torch.cuda.synchronize(dev)
@@ -382,8 +424,7 @@ def main():
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": args.workload, "bits": bits, "K": K, "N": N, "M": M, "group_size": gs,
                    "desc_act": desc_act, "weight_copies": len(case["qweights"]), "plan": s["plan"],
-                   "entry": "gptq_hip_gemm_sorted" if prepared else "gptq_hip_gemm_plan",
-                   "prepared": "input channels sorted by group once at load" if prepared else None},
+                   "entry": ENTRY[prepared], "prepared": PREPARED_NOTE[prepared]},
         "parity": {"ok": ok, "max_abs_err": round(max_err, 6), "rtol": 1e-2, "atol": 1e-2},
         "timing": {k: s[k] for k in ("eager_us", "graph_us", "graph_error", "unprepared_us") if k in s},
         "hbm_frac": s["hbm_frac"], "tflops": s["TFLOPs"],
@@ -393,14 +434,14 @@ def main():
         # the other halves of the metric, each a timed record of its own with its roofline and parity
         secondary = []
         for name in SECONDARY_WORKLOADS:
-            prep = prepared_applies(name)
+            prep = prepared_mode(name)
             c = build_case(name, dev, prepared=prep)
             okc, errc = check_case(c, dev)
             r = summarize(c, time_case(c, dev, args.steps, args.warmup))
             secondary.append({
                 "workload": name, "value": r["us"], "unit": "us", "steps": args.steps, "warmup": args.warmup,
                 "timing": {k: r[k] for k in ("eager_us", "graph_us", "graph_error") if k in r},
-                "entry": "gptq_hip_gemm_sorted" if prep else "gptq_hip_gemm_plan", "plan": r["plan"],
+                "entry": ENTRY[prep], "prepared": PREPARED_NOTE[prep], "plan": r["plan"],
                 "hbm_frac": r["hbm_frac"], "tflops": r["TFLOPs"], "mfma_frac": r["mfma_frac"],
                 "roofline": roofline_of(name, r),
                 "parity": {"ok": okc, "max_abs_err": round(errc, 6), "rtol": 1e-2, "atol": 1e-2},
@@ -410,13 +451,14 @@ def main():
         line["secondary"] = secondary
     if args.sweep:
         sweep = []
-        for name, prep in [(n, pr) for n in sorted(WORKLOADS) for pr in (False, True)]:
-            if prep and not prepared_applies(name):
+        for name, prep in [(n, pr) for n in sorted(WORKLOADS) for pr in (None, "sorted", "tiled")]:
+            if (prep == "sorted" and not sorted_applies(name)) or (prep == "tiled" and not tiled_applies(name)):
                 continue
             c = build_case(name, dev, prepared=prep)
             okc, errc = check_case(c, dev)
             r = summarize(c, time_case(c, dev, min(args.steps, 100), min(args.warmup, 10)))
             r["prepared"] = prep
+            r["module_choice"] = prep == prepared_mode(name)
             r["parity_ok"] = okc
             r["max_abs_err"] = round(errc, 6)
             sweep.append(r)
