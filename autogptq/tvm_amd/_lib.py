@@ -135,7 +135,7 @@ def lib() -> ctypes.CDLL:
     if l.gptq_hip_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{LIB_PATH} has ABI version {l.gptq_hip_abi_version()}, this package expects "
                            f"{ABI_VERSION}: rebuild it with `python -m autogptq.tvm_amd.build`")
-    from . import build as _build
+    from . import _sources as _build
     built, now = l.gptq_hip_build_id().decode(), _build.source_hash()
     if built != now:
         raise RuntimeError(f"{LIB_PATH} was built from other sources (build id {built}, sources now {now}): "
@@ -154,6 +154,11 @@ def select(M: int, K: int, N: int, bits: int, group_size: int, act_order: bool) 
     if rc != OK:
         raise GptqHipError(rc, f"gptq_hip_select(M={M}, K={K}, N={N}, bits={bits}, group_size={group_size})")
     return plan
+
+
+def build_id() -> str:
+    """The digest of the sources the loaded kernel library was built from."""
+    return lib().gptq_hip_build_id().decode()
 
 
 def select_tiled(M: int, K: int, N: int, bits: int, group_size: int, decode: bool = False) -> Plan:

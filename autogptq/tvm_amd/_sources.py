@@ -1,0 +1,22 @@
+"""The sources the two in-tree libraries are built from, and their digest."""
+from __future__ import annotations
+
+import hashlib
+import os
+
+CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+SOURCES = ["gptq_gather.hip", "gptq_stream.hip", "gptq_grouped.hip", "gptq_dequant.hip", "gptq_static.hip", "gptq_tiled.hip", "gptq_dispatch.cpp", "gptq_capi.cpp"]
+HEADERS = ["gptq_unpack.h", "gptq_internal.h", "gptq_device.h", os.path.join("..", "..", "..", "include", "gptq_hip.h"),
+           "binding.cpp"]   # (hashed with the rest: both libraries carry one build id)
+
+
+def source_hash() -> str:
+    """Digest of every source and header the library is built from; the library reports the digest it
+    was built with (gptq_hip_build_id), so a library older than its sources is noticed when it is loaded."""
+    h = hashlib.sha256()
+    for name in sorted(SOURCES + HEADERS):
+        with open(os.path.join(CSRC, name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read() + b"\0")
+    return h.hexdigest()[:16]
+
+

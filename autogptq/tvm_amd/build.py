@@ -1,22 +1,22 @@
-"""Builds the C-ABI shared library of HIP kernels for gfx950, in-tree, with hipcc.
+"""Builds the C-ABI shared library of HIP kernels for gfx950, in-tree, with hipcc, and the torch operator
+library on top of it.
 
 ``python -m autogptq.tvm_amd.build`` compiles ``csrc/*.hip`` and ``csrc/*.cpp`` into
-``csrc/libgptq_hip.so``.  hipcc cross-compiles without a GPU.
+``csrc/libgptq_hip.so`` (no torch in it), then ``csrc/binding.cpp`` against the installed torch headers into
+``csrc/libgptq_hip_torch.so`` (``torch.ops.gptq_hip.*``).  hipcc cross-compiles without a GPU.
 """
 from __future__ import annotations
 
-import hashlib
 import json
 import os
 import shutil
 import subprocess
 import sys
 
-HERE = os.path.dirname(os.path.abspath(__file__))
-CSRC = os.path.join(HERE, "csrc")
+from ._sources import CSRC, HEADERS, SOURCES, source_hash  # noqa: F401
+
 LIB = os.path.join(CSRC, "libgptq_hip.so")
-SOURCES = ["gptq_gather.hip", "gptq_stream.hip", "gptq_grouped.hip", "gptq_dequant.hip", "gptq_static.hip", "gptq_tiled.hip", "gptq_dispatch.cpp", "gptq_capi.cpp"]
-HEADERS = ["gptq_unpack.h", "gptq_internal.h", "gptq_device.h", os.path.join("..", "..", "..", "include", "gptq_hip.h")]
+BINDING_LIB = os.path.join(CSRC, "libgptq_hip_torch.so")
 
 
 def hipcc() -> str:
@@ -36,16 +36,6 @@ def flags() -> list:
         # keep the compiler from forming packed-fp32 instructions
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     ]
-
-
-def source_hash() -> str:
-    """Digest of every source and header the library is built from; the library reports the digest it
-    was built with (gptq_hip_build_id), so a library older than its sources is noticed when it is loaded."""
-    h = hashlib.sha256()
-    for name in sorted(SOURCES + HEADERS):
-        with open(os.path.join(CSRC, name), "rb") as f:
-            h.update(name.encode() + b"\0" + f.read() + b"\0")
-    return h.hexdigest()[:16]
 
 
 def is_stale() -> bool:
@@ -84,6 +74,25 @@ def _compile_one(src: str, obj: str, build_id: str):
     return subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
 
 
+def build_binding(build_id: str) -> str:
+    """binding.cpp -> libgptq_hip_torch.so: host C++ only (no device code), against torch's headers and
+    libraries, linked to libgptq_hip.so beside it."""
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    inc = [f"-I{d}" for d in ce.include_paths()] + ["-I/opt/rocm/include", f"-I{os.path.join(CSRC, '..', '..', '..', 'include')}"]
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [hipcc(), "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", f'-DGPTQ_HIP_BUILD_ID="{build_id}"',
+           "-Wno-deprecated-declarations"] + inc + [
+        os.path.join(CSRC, "binding.cpp"), "-o", BINDING_LIB, f"-L{CSRC}", "-lgptq_hip", f"-L{tlib}", "-lc10", "-lc10_hip",
+        "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building the torch operator library failed:\n" + r.stdout)
+    return BINDING_LIB
+
+
 def build(verbose: bool = False, jobs: int = 0) -> str:
     """Compiles every source to an object file (in parallel, at most 8 at a time) and links the library."""
     from concurrent.futures import ThreadPoolExecutor
@@ -114,6 +123,7 @@ def build(verbose: bool = False, jobs: int = 0) -> str:
                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if link.returncode != 0:
         raise RuntimeError("link failed:\n" + link.stdout)
+    build_binding(build_id)
     with open(REPORT, "w", encoding="utf-8") as f:   # registers, scratch and spills per kernel
         json.dump(report, f, indent=1, sort_keys=True)
     spilled = sorted(k for k, v in report.items() if v.get("vgpr_spill", 0) or v.get("scratch", 0))

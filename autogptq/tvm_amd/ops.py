@@ -2,6 +2,7 @@
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional
 
 import torch
@@ -305,28 +306,74 @@ def dequant(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
 
 
 # ---------------------------------------------------------------------------------------------
-# torch.ops.gptq_hip.{gemm, dequant}: the same two calls as dispatcher-visible operators (GPU kernels
-# and shape-only "meta" versions; no CPU kernel is registered, so a CPU tensor fails in the dispatcher
-# instead of falling back).
+# torch.ops.gptq_hip.{gemm, gemm_sorted, gemm_tiled, dequant}: the same calls as dispatcher-visible
+# operators.  csrc/binding.cpp defines them in C++ (libgptq_hip_torch.so, built beside the kernel library);
+# only GPU kernels and shape-only "meta" versions exist; a CPU tensor raises ("no CPU fallback").  Without the built operator library the same operators are registered from here, as thin
+# wrappers of the functions above (ctypes into the same C ABI).
 def _meta_gemm(x, qweight, qzeros, scales, g_idx, bias, bits, group_size):
     return x.new_empty((x.shape[0], qweight.shape[1]), dtype=torch.float16)
+
+
+def _meta_gemm_sorted(x, qweight_sorted, qzeros, scales, kmap, bias, bits, group_size):
+    return x.new_empty((x.shape[0], qweight_sorted.shape[1]), dtype=torch.float16)
+
+
+def _meta_gemm_tiled(x, qtile, sz, xsrc, kinv, bias, bits, group_size):
+    return x.new_empty((x.shape[0], sz.shape[1]), dtype=torch.float16)
 
 
 def _meta_dequant(qweight, qzeros, scales, g_idx, bits, group_size):
     return scales.new_empty((qweight.shape[0] * 32 // bits, qweight.shape[1]), dtype=torch.float16)
 
 
+BINDING_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libgptq_hip_torch.so")
+NATIVE_OPS = False   # True when torch.ops.gptq_hip.* are the C++ operators
+
+
 def _register_torch_ops():
-    lib = torch.library.Library("gptq_hip", "DEF")
-    lib.define("gemm(Tensor x, Tensor qweight, Tensor qzeros, Tensor scales, Tensor? g_idx, Tensor? bias, "
-               "int bits, int group_size) -> Tensor")
-    lib.define("dequant(Tensor qweight, Tensor qzeros, Tensor scales, Tensor? g_idx, int bits, int group_size) "
-               "-> Tensor")
-    lib.impl("gemm", lambda x, qw, qz, sc, g, b, bits, gs: gemm(x, qw, qz, sc, g, b, bits, gs), "CUDA")
-    lib.impl("dequant", lambda qw, qz, sc, g, bits, gs: dequant(qw, qz, sc, g, bits, gs), "CUDA")
-    lib.impl("gemm", _meta_gemm, "Meta")
-    lib.impl("dequant", _meta_dequant, "Meta")
-    return lib
+    global NATIVE_OPS
+    keep = []
+    native = False
+    if os.path.exists(BINDING_PATH) and os.path.exists(_lib.LIB_PATH):
+        try:
+            _lib.lib()                  # the kernel library first (checks that it matches its sources)
+            native = True
+        except RuntimeError:
+            pass                        # stale: the Python operators below report it on their first call
+    if native:
+        torch.ops.load_library(BINDING_PATH)
+        built = torch.ops.gptq_hip.binding_build_id()
+        if built != _lib.build_id():
+            raise RuntimeError(f"{BINDING_PATH} was built from other sources ({built}) than the kernel library "
+                               f"({_lib.build_id()}): run python -m autogptq.tvm_amd.build")
+        NATIVE_OPS = True
+    else:
+        lib = torch.library.Library("gptq_hip", "DEF")
+        lib.define("gemm(Tensor x, Tensor qweight, Tensor qzeros, Tensor scales, Tensor? g_idx, Tensor? bias, "
+                   "int bits, int group_size) -> Tensor")
+        lib.define("gemm_sorted(Tensor x, Tensor qweight_sorted, Tensor qzeros, Tensor scales, Tensor kmap, "
+                   "Tensor? bias, int bits, int group_size) -> Tensor")
+        lib.define("gemm_tiled(Tensor x, Tensor qtile, Tensor sz, Tensor? xsrc, Tensor? kinv, Tensor? bias, "
+                   "int bits, int group_size) -> Tensor")
+        lib.define("dequant(Tensor qweight, Tensor qzeros, Tensor scales, Tensor? g_idx, int bits, int group_size) "
+                   "-> Tensor")
+        lib.impl("gemm", lambda x, qw, qz, sc, g, b, bits, gs: gemm(x, qw, qz, sc, g, b, bits, gs), "CUDA")
+        lib.impl("gemm_sorted", lambda x, qw, qz, sc, km, b, bits, gs: gemm_sorted(x, qw, qz, sc, km, b, bits, gs), "CUDA")
+        lib.impl("gemm_tiled", lambda x, qt, sz, xs, ki, b, bits, gs: gemm_tiled(x, qt, sz, xs, ki, b, bits, gs), "CUDA")
+        lib.impl("dequant", lambda qw, qz, sc, g, bits, gs: dequant(qw, qz, sc, g, bits, gs), "CUDA")
+        # CPU tensors reach the same functions, whose first check raises ("no CPU fallback")
+        lib.impl("gemm", lambda x, qw, qz, sc, g, b, bits, gs: gemm(x, qw, qz, sc, g, b, bits, gs), "CPU")
+        lib.impl("gemm_sorted", lambda x, qw, qz, sc, km, b, bits, gs: gemm_sorted(x, qw, qz, sc, km, b, bits, gs), "CPU")
+        lib.impl("gemm_tiled", lambda x, qt, sz, xs, ki, b, bits, gs: gemm_tiled(x, qt, sz, xs, ki, b, bits, gs), "CPU")
+        lib.impl("dequant", lambda qw, qz, sc, g, bits, gs: dequant(qw, qz, sc, g, bits, gs), "CPU")
+        keep.append(lib)
+    meta = torch.library.Library("gptq_hip", "IMPL", "Meta")
+    meta.impl("gemm", _meta_gemm)
+    meta.impl("gemm_sorted", _meta_gemm_sorted)
+    meta.impl("gemm_tiled", _meta_gemm_tiled)
+    meta.impl("dequant", _meta_dequant)
+    keep.append(meta)
+    return keep
 
 
 _TORCH_OPS = _register_torch_ops()  # kept alive for the life of the module

@@ -85,6 +85,7 @@ class QuantLinear(nn.Module):
         self.tile_for_prefill = tile_for_prefill
         self._tiled = None    # (key, (qtile, sz, xsrc, kinv) or None)
         self._compact = False
+        self._routes = {}     # M -> (watched buffers, sum of their versions, path name, fn(x2)): see _route
 
     # ------------------------------------------------------------------ packing
     def pack(self, linear, scales, zeros, g_idx=None):
@@ -204,26 +205,116 @@ class QuantLinear(nn.Module):
         # the tiled copy of a compact layer is its weights: it moves with the module (a prepared copy beside
         # the checkpoint tensors is rebuilt instead, when their storage changes)
         super()._apply(fn, *args, **kwargs)
+        self._routes.clear()
         if self._compact:
             self._tiled = (None, tuple(None if t is None else fn(t) for t in self._tiled[1]))
         return self
 
-
-    def _decode_sorted(self, x2):
-        """The decode product through the sorted copy, or None when that path does not apply."""
+    def _sorted_tensors(self, M):
+        """The sorted copy when the decode path through it covers M rows, else None."""
         plans = self._sorted_plans
-        M = x2.shape[0]
         if M not in plans:
             plans[M] = ops.sorted_plan(M, self.infeatures, self.outfeatures, self.bits, self.groupsize)
-        if plans[M] is None:
-            return None
-        tensors = self.prepare_decode()
-        if tensors is None:
-            return None
-        return ops.gemm_sorted(x2, tensors[0], self.qzeros, self.scales, tensors[1], self.bias, self.bits,
-                               self.groupsize, plan=plans[M])
+        return self.prepare_decode() if plans[M] is not None else None
+
+    # ------------------------------------------------------------------ routing
+    def __setattr__(self, name, value):
+        # any change of a buffer or a switch may change where a row count goes: forget the routes
+        if name != "_routes":
+            routes = self.__dict__.get("_routes")
+            if routes:
+                routes.clear()
+        super().__setattr__(name, value)
+
+    def _watched(self):
+        """The buffers whose contents a route may have baked into a prepared copy."""
+        return (self.qweight, self.qzeros, self.scales, self.g_idx)
+
+    def _route(self, M):
+        """(what, fn): the product for M rows as one call fn(x2), and the name of the path it takes: "tiled",
+        "sorted", "plain" (the checkpoint's own tensors) or "library" (dequant kernel + library GEMM).  Decided
+        once per row count and state of the buffers; the operators are torch.ops.gptq_hip.* (csrc/binding.cpp)."""
+        t = torch.ops.gptq_hip
+        bits, gs, bias = self.bits, self.groupsize, self.bias
+
+        def bind(kind, a, b, c, d, e):
+            if ops.NATIVE_OPS:
+                # the C++ operator library binds a layer's constant tensors once: one argument per call
+                return torch.classes.gptq_hip.Layer(kind, a, b, c, d, e, bias, bits, gs).forward
+            if kind == 0:
+                return lambda x2: t.gemm.default(x2, a, b, c, d, bias, bits, gs)
+            if kind == 1:
+                return lambda x2: t.gemm_sorted.default(x2, a, b, c, d, bias, bits, gs)
+            return lambda x2: t.gemm_tiled.default(x2, a, b, d, e, bias, bits, gs)
+
+        if self._compact:
+            qtile, sz, xsrc, kinv = self._tiled[1]
+            return "tiled", bind(2, qtile, sz, None, xsrc, kinv)
+
+        def library(x2):
+            # Long prompts (kernel_switch_threshold), 2- and 8-bit layers, or a shape the fused kernels do
+            # not cover (activation order with more groups than their LDS table holds): materialise W with
+            # the HIP dequant kernel and multiply with the library GEMM, which is what the reference
+            # does above its threshold (auto_gptq/nn_modules/qlinear.py:198-245).  Still GPU only.
+            out = torch.matmul(x2, self.dequantize())
+            return out if bias is None else out + bias
+
+        if self.bits not in self.FUSED_BITS:
+            return "library", library
+        g = self._kernel_g_idx()
+        K, N = self.infeatures, self.outfeatures
+        tiled = None
+        if self.tile_for_prefill and ops.tiled_wins(M, K, N, g is not None):
+            tiled = self.prepare_tiled()
+        threshold = self.kernel_switch_threshold
+        if threshold and self.act_order_switch_threshold and g is not None and tiled is None:
+            threshold = min(threshold, self.act_order_switch_threshold)   # (the tiled kernels do not pay for the order)
+        if threshold and M >= threshold:
+            return "library", library
+        if tiled is not None:
+            qtile, sz = tiled[0], tiled[1]
+            xsrc, kinv = (tiled[2], tiled[3]) if g is not None else (None, None)
+            return "tiled", bind(2, qtile, sz, None, xsrc, kinv)
+        qzeros, scales = self.qzeros, self.scales
+        srt = self._sorted_tensors(M) if (self.sort_for_decode and M <= ops.SORTED_MAX_ROWS) else None
+        if srt is not None:
+            qs, kmap = srt
+            return "sorted", bind(1, qs, qzeros, scales, kmap, None)
+        try:
+            _lib.select(M, K, N, bits, gs, g is not None)
+        except _lib.GptqHipError as e:
+            if e.status != _lib.ERR_UNSUPPORTED:
+                raise
+            return "library", library
+        qweight = self.qweight
+        return "plain", bind(0, qweight, qzeros, scales, g, None)
+
+    def route(self, M: int) -> str:
+        """The path a call with M rows takes (see ``_route``); builds the prepared copy it needs."""
+        return self._routed(M)[2]
+
+    def _routed(self, M):
+        r = self._routes.get(M)
+        if r is not None:
+            a, b, c, d = r[0]
+            if a._version + b._version + c._version + d._version == r[1]:
+                return r
+        what, fn = self._route(M)
+        w = self._watched()               # (read after routing: the preparations may have re-made g_idx)
+        r = (w, sum(t._version for t in w), what, fn)
+        self._routes[M] = r
+        return r
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        # the common case first: a contiguous fp16 matrix, no gradient wanted, a row count seen before and
+        # buffers not written since (replacing a buffer or moving the module empties the table)
+        if x.dim() == 2 and x.dtype is torch.float16 and x.is_contiguous() and not (
+                x.requires_grad and torch.is_grad_enabled()):
+            r = self._routes.get(x.size(0))
+            if r is not None:
+                a, b, c, d = r[0]
+                if a._version + b._version + c._version + d._version == r[1]:
+                    return r[3](x)
         out_shape = x.shape[:-1] + (self.outfeatures,)
         x2 = x.reshape(-1, x.shape[-1])
         if x2.dtype != torch.float16:
@@ -239,40 +330,9 @@ class QuantLinear(nn.Module):
     def _product(self, x2: torch.Tensor) -> torch.Tensor:
         """y[M, N] = x2[M, K] @ W + bias for a contiguous fp16 x2."""
         M = x2.shape[0]
-        if self._compact:
-            qtile, sz, xsrc, kinv = self._tiled[1]
-            return ops.gemm_tiled(x2, qtile, sz, xsrc, kinv, self.bias, self.bits, self.groupsize)
-        try:
-            if self.bits not in self.FUSED_BITS:
-                raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, "width without a fused kernel")
-            g = self._kernel_g_idx()
-            tiled = None
-            if self.tile_for_prefill and M > 0 and ops.tiled_wins(M, self.infeatures, self.outfeatures, g is not None):
-                tiled = self.prepare_tiled()
-            threshold = self.kernel_switch_threshold
-            if threshold and self.act_order_switch_threshold and g is not None and tiled is None:
-                threshold = min(threshold, self.act_order_switch_threshold)   # (the tiled kernels do not pay for the order)
-            if threshold and M >= threshold:
-                raise _lib.GptqHipError(_lib.ERR_UNSUPPORTED, "above kernel_switch_threshold")
-            if tiled is not None:
-                act = g is not None
-                return ops.gemm_tiled(x2, tiled[0], tiled[1], tiled[2] if act else None, tiled[3] if act else None,
-                                      self.bias, self.bits, self.groupsize)
-            out = self._decode_sorted(x2) if (self.sort_for_decode and 0 < M <= ops.SORTED_MAX_ROWS) else None
-            if out is None:
-                out = ops.gemm(x2, self.qweight, self.qzeros, self.scales, self._kernel_g_idx(), self.bias,
-                               self.bits, self.groupsize)
-        except _lib.GptqHipError as e:
-            if e.status != _lib.ERR_UNSUPPORTED:
-                raise
-            # Long prompts (kernel_switch_threshold), 2- and 8-bit layers, or a shape the fused kernels do
-            # not cover (activation order with more groups than their LDS table holds): materialise W with
-            # the HIP dequant kernel and multiply with the library GEMM, which is what the reference
-            # does above its threshold (auto_gptq/nn_modules/qlinear.py:198-245).  Still GPU only.
-            out = torch.matmul(x2, self.dequantize())
-            if self.bias is not None:
-                out = out + self.bias
-        return out
+        if M == 0:
+            return x2.new_empty((0, self.outfeatures))
+        return self._routed(M)[3](x2)
 
     def dequantize(self) -> torch.Tensor:
         """fp16 [infeatures, outfeatures], the weight the reference materialises on every call."""

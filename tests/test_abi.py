@@ -262,3 +262,24 @@ def test_single_group_ignores_act_order():
     a = _lib.select(1, 9216, 9216, 3, -1, True).as_dict()
     b = _lib.select(1, 9216, 9216, 3, -1, False).as_dict()
     assert a == b
+
+
+def test_torch_operator_library_is_built_and_matches_the_kernel_library():
+    """csrc/binding.cpp: built beside the kernel library, from the same sources (one build id), and it
+    defines every operator the module calls, with the schemas the Python front end has."""
+    import torch
+
+    from autogptq.tvm_amd import ops
+
+    assert os.path.exists(ops.BINDING_PATH), "run python -m autogptq.tvm_amd.build"
+    assert ops.NATIVE_OPS
+    assert torch.ops.gptq_hip.binding_build_id() == _lib.build_id()
+    for name in ("gemm", "gemm_sorted", "gemm_tiled", "dequant"):
+        schema = str(getattr(torch.ops.gptq_hip, name).default._schema)
+        assert schema.startswith(f"gptq_hip::{name}(Tensor ") and schema.endswith("-> Tensor"), schema
+    assert hasattr(torch.classes.gptq_hip, "Layer")
+    # shape-only versions for tracing
+    m = torch.ops.gptq_hip.gemm_tiled(torch.empty(5, 64, dtype=torch.float16, device="meta"),
+                                      torch.empty(64 * 32 // 8, dtype=torch.int32, device="meta"),
+                                      torch.empty(1, 32, dtype=torch.int32, device="meta"), None, None, None, 4, 64)
+    assert m.shape == (5, 32) and m.device.type == "meta"

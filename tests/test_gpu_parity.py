@@ -663,3 +663,28 @@ def test_torch_operator_equals_the_python_front_end(dev):
     assert torch.equal(a, run_gemm(D))
     w = torch.ops.gptq_hip.dequant(D["qweight"], D["qzeros"], D["scales"], D["g_idx"], 3, 128)
     assert torch.equal(w.cpu().view(torch.int16), expected_weight(L).view(torch.int16))
+    # the operators are the C++ ones of csrc/binding.cpp (built beside the kernel library), and each gives what
+    # the ctypes front end gives on the same tensors
+    assert ops.NATIVE_OPS
+    qs, kmap = ops.sort_channels(D["qweight"], D["g_idx"], 3, 128)
+    b = torch.ops.gptq_hip.gemm_sorted(D["x"], qs, D["qzeros"], D["scales"], kmap, D["bias"], 3, 128)
+    assert torch.equal(b, ops.gemm_sorted(D["x"], qs, D["qzeros"], D["scales"], kmap, D["bias"], 3, 128))
+    qtile, sz, xsrc, kinv = ops.tile_prepare(D["qweight"], D["qzeros"], D["scales"], D["g_idx"], 3, 128)
+    for M in (5, 3):
+        c = torch.ops.gptq_hip.gemm_tiled(D["x"][:M], qtile, sz, xsrc, kinv, D["bias"], 3, 128)
+        assert torch.equal(c, ops.gemm_tiled(D["x"][:M], qtile, sz, xsrc, kinv, D["bias"], 3, 128))
+    assert_close(a, expected_output(L), "C++ operator")
+    # a layer's tensors bound once (what QuantLinear calls): first call checked, later calls on the kept plan
+    for kind, args in ((0, (D["qweight"], D["qzeros"], D["scales"], D["g_idx"], None)),
+                       (1, (qs, D["qzeros"], D["scales"], kmap, None)), (2, (qtile, sz, None, xsrc, kinv))):
+        bound = torch.classes.gptq_hip.Layer(kind, *args, D["bias"], 3, 128)
+        for x in (D["x"], D["x"], D["x"][:2], D["x"]):
+            assert_close(bound.forward(x), expected_output(L)[: x.shape[0]], f"bound layer, kind {kind}")
+        with pytest.raises(RuntimeError, match="no CPU fallback"):
+            bound.forward(D["x"].cpu())
+        with pytest.raises(RuntimeError):
+            bound.forward(D["x"][:, :256].contiguous())
+    with pytest.raises(RuntimeError, match="must be"):
+        torch.ops.gptq_hip.gemm(D["x"].float(), D["qweight"], D["qzeros"], D["scales"], D["g_idx"], D["bias"], 3, 128)
+    with pytest.raises(RuntimeError, match="UNSUPPORTED|unsupported|not supported|status"):
+        torch.ops.gptq_hip.gemm_tiled(D["x"], qtile, sz, xsrc, kinv, D["bias"], 3, 16)
