@@ -526,9 +526,9 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
 
 extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan)
 {
-    // Up to four rows the decode kernel (one matrix instruction set per lane block); from five rows on its
-    // cost grows with the rows (two sets, x staged per row) and the matmul kernel with one 32-row tile is
-    // faster: 14.6 against 24.6 us at eight rows of a 4096 x 11008 layer.
+    // Up to four rows the decode kernel (one 4-row matrix instruction set per lane block); from five rows on
+    // the matmul kernel with one 32-row tile (a decode kernel with two sets took 24.6 us at eight rows of a
+    // 4096 x 11008 layer against 14.6).
     if (M >= 1 && M <= gptq::kDecodeSelectRows) {
         const int rc = gptq_hip_select_tiled_decode(M, K, N, bits, group_size, plan);
         if (rc != GPTQ_HIP_ERR_UNSUPPORTED || !plan) return rc;

@@ -453,7 +453,7 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
 }
 
 // ---------------------------------------------------------------------------------------------------
-// tiled_decode_kernel: M <= 8 rows of x on the tiled format, bound by the weight stream from HBM.
+// tiled_decode_kernel: M <= 4 rows of x on the tiled format.
 //
 // A workgroup owns ONE column tile (32 columns) and one K range; its KW waves split that range.  With one
 // small workgroup per tile every CU gets work whatever N is (11008 columns: 344 workgroups of 4 waves,
@@ -464,7 +464,7 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
 // A lane of the tiled format holds 32 codes of ONE column, so its unpacked registers are B operands as
 // they are (four positions each), the A operand of lane 4 b + i is x[row i] at the same four positions
 // (read from LDS: rows past M read zeros), and the four result registers of a lane are the rows of its
-// own column.  Up to four rows of x cost one matrix instruction per four positions, five to eight two.
+// own column: up to four rows of x cost one matrix instruction per four positions.
 // Per weight the vector ALU only unpacks.
 // The codes enter as (base + q) with the bases of the register unpack; per block of 32 positions the
 // epilogue takes y += scale * (P - Bsum - zero * Xsum), with Xsum = sum x and Bsum = sum x * base of the
@@ -492,12 +492,14 @@ struct DecodeParams {
 
 typedef float f2 __attribute__((ext_vector_type(2)));
 
-template <int BITS, int MR, int KW>
+// E: blocks of 64 positions that share one epilogue (1, or 2 when the groups are multiples of 128 channels and
+// every wave has an even number of blocks: both lane blocks of both blocks then lie in one group).
+template <int BITS, int MR, int KW, int E>
 __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParams p)
 {
+    static_assert(MR <= 4 && (E == 1 || E == 2), "one matrix instruction set per lane block");
     constexpr int NT = 64 * KW;
-    constexpr int PF = 4;              // blocks of weights a wave requests ahead
-    constexpr int MA = (MR + 3) / 4;   // matrix instructions per four positions (rows 0..3, rows 4..7)
+    constexpr int PF = 2;              // blocks of weights per chunk; two chunks are in flight
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -616,27 +618,33 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
         szl[i] = p.sz[(size_t)(g_first + (uint32_t)(i >> 5)) * p.N + 32 * T + (i & 31)];
     }
     lds_barrier();
-    // ---- 3. per block of 32 positions and row: Xsum = sum x, Bsum = sum x * base(position); every wave for
-    //         the blocks of its own slice (LDS serves one wave's accesses in order: no barrier needed) ------
+    // ---- 3. per epilogue unit (E blocks), half and row: Xsum = sum x, Bsum = sum x * base(position) over the
+    //         unit's 32 E positions of that half; every wave for the units of its own slice (LDS serves one
+    //         wave's accesses in order: no barrier needed).  Entry ((sb / E) * 2 + h) * MR + m, sb = the unit's
+    //         first block inside the workgroup's range ------------------------------------------------------
     {
-        const int lb0 = 2 * (S_begin - S_wg);
-        for (int i = lane; i < 2 * p.wave_steps * MR; i += 64) {
-            const int lb = lb0 + i / MR, m = i % MR;
+        const int sb0 = S_begin - S_wg;
+        for (int i = lane; i < 2 * (p.wave_steps / E) * MR; i += 64) {
+            const int uh = i / MR, m = i % MR;
+            const int sb = sb0 + E * (uh >> 1), hh = uh & 1;
             float X = 0.f, B = 0.f;
             if (m < p.M) {
-                const h8 *src = (const h8 *)(xl + m * span + 32 * lb);
 #pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    const h8 q = src[v];
+                for (int b = 0; b < E; b++) {
+                    const h8 *src = (const h8 *)(xl + m * span + 64 * (sb + b) + 32 * hh);
 #pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        const float xf = (float)q[e];
-                        X += xf;
-                        B += xf * (BITS == 4 ? BASE4[e] : BASE3[e]);
+                    for (int v = 0; v < 4; v++) {
+                        const h8 q = src[v];
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            const float xf = (float)q[e];
+                            X += xf;
+                            B += xf * (BITS == 4 ? BASE4[e] : BASE3[e]);
+                        }
                     }
                 }
             }
-            xs[lb * MR + m] = (f2){X, B};
+            xs[((sb / E) * 2 + hh) * MR + m] = (f2){X, B};
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -652,17 +660,39 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     for (int m = 0; m < MR; m++) ysum[m] = 0.f;
     // Per-lane byte offsets that never change; what changes per block is wave-uniform and stays in scalar
     // registers.  A lane whose row lies past M reads the 64 zero bytes whatever the block (stride 0).
-    uint32_t x_base[MA], x_stride[MA];
-#pragma unroll
-    for (int a = 0; a < MA; a++) {
-        const int row = 4 * a + row_i;
-        x_base[a] = row < p.M ? (uint32_t)(row * span + 32 * h) * 2u : zero_off;
-        x_stride[a] = row < p.M ? 128u : 0u;
-    }
-    const uint32_t xs_lane = zero_off + 64u + (uint32_t)(h * MR) * 8u;   // block sums of lane block 2 sb + h
+    const uint32_t x_base = row_i < p.M ? (uint32_t)(row_i * span + 32 * h) * 2u : zero_off;
+    const uint32_t x_stride = row_i < p.M ? 128u : 0u;
+    const uint32_t xs_lane = zero_off + 64u + (uint32_t)(h * MR) * 8u;   // sums of half h of unit 0
     const uint32_t sz_lane = (uint32_t)((const unsigned char *)szl - smem) + (uint32_t)n * 4u;
 
-    auto do_block = [&](int S, const uint32_t (&wr)[BITS]) {
+    // x of a block: the 32 positions of the lane block, row row_i; read one block ahead of its use
+    auto load_x = [&](uint32_t sb, u4 (&xv)[4]) {
+        const uint32_t xoff = x_base + x_stride * sb;
+#pragma unroll
+        for (int v = 0; v < 4; v++) xv[v] = *(const u4 *)(smem + xoff + 16 * v);
+    };
+    f4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};  // two chains: a matrix instruction waits for the one it adds to
+    uint32_t szw = 0u;   // (scale, zero) word and sums of the unit in flight, read when the unit starts
+    f2 xsv[MR];
+    auto block = [&](auto uu_c, int S, const uint32_t (&wr)[BITS], const u4 (&xc)[4], u4 (&xn)[4]) {
+        constexpr int uu = decltype(uu_c)::value;                 // block inside its unit
+        const uint32_t sb = (uint32_t)(S - S_wg);                  // block inside the workgroup's range (wave-uniform)
+        if constexpr (uu == 0) {
+            // group of the unit's lane blocks (E = 1: the two halves of the wave may differ)
+            const uint32_t l0 = 2u * (uint32_t)S;
+            const uint32_t g0 = min(__umulhi(l0, p.lbg_magic) + (p.lbg_add ? l0 : 0u), (uint32_t)p.G - 1u) - g_first;
+            uint32_t goff = g0 * 128u;
+            if constexpr (E == 1) {
+                const uint32_t l1 = l0 + 1u;
+                const uint32_t g1 = min(__umulhi(l1, p.lbg_magic) + (p.lbg_add ? l1 : 0u), (uint32_t)p.G - 1u) - g_first;
+                goff = (h ? g1 : g0) * 128u;
+            }
+            szw = *(const uint32_t *)(smem + sz_lane + goff);
+            const f2 *xb = (const f2 *)(smem + xs_lane + (sb / E) * (uint32_t)(2 * MR * 8));
+#pragma unroll
+            for (int m = 0; m < MR; m++) xsv[m] = xb[m];
+        }
+        load_x(sb + 1u, xn);
         // unpack: sixteen registers, positions (2 r, 2 r + 1) of the lane in register r
         u4 q[4];
         if constexpr (BITS == 4) {
@@ -675,52 +705,54 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
         } else {
             biased3(wr[0], wr[1], wr[2], q, magic_a, magic_b);
         }
-        const uint32_t sb = (uint32_t)(S - S_wg);  // block inside the workgroup's range (wave-uniform)
-        f4 acc[MA];
-#pragma unroll
-        for (int a = 0; a < MA; a++) {
-            // (two chains: a matrix instruction waits for the one it adds to)
-            f4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};
-            const uint32_t xoff = x_base[a] + x_stride[a] * sb;
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const u4 xv = *(const u4 *)(smem + xoff + 16 * v);  // positions 8 v .. 8 v + 7 of the lane block
-                const u2 a0 = {xv[0], xv[1]}, a1 = {xv[2], xv[3]};
-                const u2 b0 = {q[v][0], q[v][1]}, b1 = {q[v][2], q[v][3]};
-                c0 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a0), __builtin_bit_cast(h4, b0), c0, 0, 0, 0);
-                c1 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a1), __builtin_bit_cast(h4, b1), c1, 0, 0, 0);
-            }
-            acc[a] = c0 + c1;
+        if constexpr (uu == 0) {
+            c0 = (f4){0.f, 0.f, 0.f, 0.f};
+            c1 = (f4){0.f, 0.f, 0.f, 0.f};
         }
-        // scale and zero point of the lane block's group (the two halves of the wave may differ), and its sums
-        const uint32_t l0 = 2u * (uint32_t)S, l1 = l0 + 1u;
-        const uint32_t g0 = min(__umulhi(l0, p.lbg_magic) + (p.lbg_add ? l0 : 0u), (uint32_t)p.G - 1u) - g_first;
-        const uint32_t g1 = min(__umulhi(l1, p.lbg_magic) + (p.lbg_add ? l1 : 0u), (uint32_t)p.G - 1u) - g_first;
-        const h2 e = as_h2(*(const uint32_t *)(smem + sz_lane + (h ? g1 : g0) * 128u));
-        const float sc = (float)e[0], zp = (float)e[1];
-        const f2 *xb = (const f2 *)(smem + xs_lane + sb * (uint32_t)(2 * MR * 8));
 #pragma unroll
-        for (int m = 0; m < MR; m++) {
-            const f2 t = xb[m];
-            ysum[m] += sc * ((acc[m >> 2][m & 3] - t[1]) - zp * t[0]);
+        for (int v = 0; v < 4; v++) {
+            const u2 a0 = {xc[v][0], xc[v][1]}, a1 = {xc[v][2], xc[v][3]};
+            const u2 b0 = {q[v][0], q[v][1]}, b1 = {q[v][2], q[v][3]};
+            c0 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a0), __builtin_bit_cast(h4, b0), c0, 0, 0, 0);
+            c1 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a1), __builtin_bit_cast(h4, b1), c1, 0, 0, 0);
+        }
+        if constexpr (uu == E - 1) {
+            const h2 e = as_h2(szw);
+            const float sc = (float)e[0], zp = (float)e[1];
+#pragma unroll
+            for (int m = 0; m < MR; m++) ysum[m] += sc * (((c0[m] + c1[m]) - xsv[m][1]) - zp * xsv[m][0]);
         }
     };
 
-    for (int c = 0; c < steps; c += 2 * PF) {
-#pragma unroll
-        for (int u = 0; u < PF; u++)
-            if (c + u < steps) do_block(S_begin + c + u, w[0][u]);
+    // Chunks of PF blocks, two in flight; x rides one block ahead in two register sets.  Blocks past the end
+    // of K inside a wave's range are harmless (their x and sums are zeros), blocks past the range are skipped.
+    u4 xr[2][4];
+    load_x((uint32_t)(S_begin - S_wg), xr[0]);
+    auto chunk = [&](int c, uint32_t (&wc)[PF][BITS], auto all_c) {
+        constexpr bool ALL = decltype(all_c)::value;
+        [&]<int... U>(std::integer_sequence<int, U...>) {
+            ((ALL || c + U < p.wave_steps
+                  ? block(std::integral_constant<int, U % E>{}, S_begin + c + U, wc[U], xr[U & 1], xr[(U + 1) & 1])
+                  : (void)0),
+             ...);
+        }(std::make_integer_sequence<int, PF>{});
+    };
+    int c = 0;
+    for (; c + 2 * PF <= p.wave_steps; c += 2 * PF) {
+        chunk(c, w[0], std::true_type{});
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < PF; u++) load_w(c + 2 * PF + u, w[0][u]);  // the chunk after the one in flight
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int u = 0; u < PF; u++)
-            if (c + PF + u < steps) do_block(S_begin + c + PF + u, w[1][u]);
+        chunk(c + PF, w[1], std::true_type{});
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < PF; u++) load_w(c + 3 * PF + u, w[1][u]);
         __builtin_amdgcn_sched_barrier(0);
+    }
+    if (c < p.wave_steps) {   // what is left of the range: fewer than two chunks, nothing more to request
+        chunk(c, w[0], std::false_type{});
+        chunk(c + PF, w[1], std::false_type{});
     }
 
     // ---- 5. the two halves of a column (lanes n and n + 32), then the waves along K ---------------------
@@ -841,10 +873,10 @@ int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int
 }
 
 
-template <int BITS, int MR, int KW>
+template <int BITS, int MR, int KW, int E>
 static int launch_decode_one(const DecodeParams &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
-    auto kern = tiled_decode_kernel<BITS, MR, KW>;
+    auto kern = tiled_decode_kernel<BITS, MR, KW, E>;
     if (plan.lds_bytes > 65536) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, plan.lds_bytes) != hipSuccess) {
             (void)hipGetLastError();
@@ -855,13 +887,13 @@ static int launch_decode_one(const DecodeParams &p, const gptq_hip_plan &plan, h
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 
-template <int BITS, int MR>
+template <int BITS, int MR, int E>
 static int launch_decode_kw(const DecodeParams &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
     switch (plan.waves_k) {
-        case 4: return launch_decode_one<BITS, MR, 4>(p, plan, stream);
-        case 8: return launch_decode_one<BITS, MR, 8>(p, plan, stream);
-        case 16: return launch_decode_one<BITS, MR, 16>(p, plan, stream);
+        case 4: return launch_decode_one<BITS, MR, 4, E>(p, plan, stream);
+        case 8: return launch_decode_one<BITS, MR, 8, E>(p, plan, stream);
+        case 16: return launch_decode_one<BITS, MR, 16, E>(p, plan, stream);
         default: return GPTQ_HIP_ERR_UNSUPPORTED;
     }
 }
@@ -894,16 +926,16 @@ int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, co
     p.lbg_magic = p.lbg_add ? 0u : (uint32_t)((1ull << 32) / (uint32_t)p.lb_per_group) + 1u;
     const int mr = tiled_decode_rows(M);
     int rc = GPTQ_HIP_ERR_UNSUPPORTED;
+    // two blocks per epilogue where every unit of two blocks lies in one group
+    const bool pairs = group_size % 128 == 0 && plan.k_chunk % 2 == 0;
 #define GPTQ_DECODE_CASE(B, R) \
-    if (bits == B && mr == R) rc = launch_decode_kw<B, R>(p, plan, stream)
+    if (bits == B && mr == R) rc = pairs ? launch_decode_kw<B, R, 2>(p, plan, stream) : launch_decode_kw<B, R, 1>(p, plan, stream)
     GPTQ_DECODE_CASE(4, 1);
     GPTQ_DECODE_CASE(4, 2);
     GPTQ_DECODE_CASE(4, 4);
-    GPTQ_DECODE_CASE(4, 8);
     GPTQ_DECODE_CASE(3, 1);
     GPTQ_DECODE_CASE(3, 2);
     GPTQ_DECODE_CASE(3, 4);
-    GPTQ_DECODE_CASE(3, 8);
 #undef GPTQ_DECODE_CASE
     if (rc != GPTQ_HIP_OK) return rc;
     if (plan.split_k > 1) {
