@@ -492,6 +492,13 @@ struct DecodeParams {
 
 typedef float f2 __attribute__((ext_vector_type(2)));
 
+// v of lane l + N inside its row of 16 lanes (zero past the row's end)
+template <int N>
+__device__ __forceinline__ float row_shl(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x100 + N, 0xf, 0xf, true));
+}
+
 // E: blocks of 64 positions that share one epilogue (1, or 2 when the groups are multiples of 128 channels and
 // every wave has an even number of blocks: both lane blocks of both blocks then lie in one group).
 template <int BITS, int MR, int KW, int E>
@@ -623,17 +630,20 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     //         wave's accesses in order: no barrier needed).  Entry ((sb / E) * 2 + h) * MR + m, sb = the unit's
     //         first block inside the workgroup's range ------------------------------------------------------
     {
+        // a lane sums 16 consecutive positions; a run of 32 positions (one half of one block) is two lanes,
+        // a unit-half 2 E lanes: l, l + 1 (the other half of the run) and, E = 2, l + 4, l + 5 (the other block)
         const int sb0 = S_begin - S_wg;
-        for (int i = lane; i < 2 * (p.wave_steps / E) * MR; i += 64) {
-            const int uh = i / MR, m = i % MR;
-            const int sb = sb0 + E * (uh >> 1), hh = uh & 1;
-            float X = 0.f, B = 0.f;
-            if (m < p.M) {
+        for (int q0 = 0; q0 < 4 * p.wave_steps; q0 += 64) {   // 16-position pieces of the wave's range
+            const int piece = q0 + lane;
+            const int sb = sb0 + (piece >> 2), hh = (piece >> 1) & 1;
+            const bool live = piece < 4 * p.wave_steps;
 #pragma unroll
-                for (int b = 0; b < E; b++) {
-                    const h8 *src = (const h8 *)(xl + m * span + 64 * (sb + b) + 32 * hh);
+            for (int m = 0; m < MR; m++) {
+                float X = 0.f, B = 0.f;
+                if (live && m < p.M) {
+                    const h8 *src = (const h8 *)(xl + m * span + 64 * sb0 + 16 * piece);
 #pragma unroll
-                    for (int v = 0; v < 4; v++) {
+                    for (int v = 0; v < 2; v++) {
                         const h8 q = src[v];
 #pragma unroll
                         for (int e = 0; e < 8; e++) {
@@ -643,8 +653,16 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
                         }
                     }
                 }
+                // lane l takes l + 1 (and, E = 2, l + 4 and l + 5): the lanes that store (l % 8 in {0, 2}) stay
+                // inside their row of 16, so a row shift in the data path does (no LDS round trip)
+                X += row_shl<1>(X);
+                B += row_shl<1>(B);
+                if constexpr (E == 2) {
+                    X += row_shl<4>(X);
+                    B += row_shl<4>(B);
+                }
+                if (live && (lane & (E == 2 ? 5 : 1)) == 0) xs[((sb / E) * 2 + hh) * MR + m] = (f2){X, B};
             }
-            xs[((sb / E) * 2 + hh) * MR + m] = (f2){X, B};
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
