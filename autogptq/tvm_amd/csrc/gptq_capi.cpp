@@ -347,6 +347,20 @@ extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint3
         if (rc != GPTQ_HIP_OK) return rc;
         plan = &chosen;
     }
+    if (plan->kernel == GPTQ_HIP_KERNEL_TILED_DECODE && plan->waves_n == 2) {
+        // one workgroup per CU, 16-column units
+        const int mr = plan->row_tiles;
+        if (M > gptq::kDecodeMaxRows || mr != gptq::tiled_decode_rows(M)) return GPTQ_HIP_ERR_UNSUPPORTED;
+        const int units = N / 16;
+        const int V_all = ((K + 63) / 64 + 1) / 2;
+        if (plan->block != 1024 || plan->waves_k != 16 || plan->split_k != 1 || plan->grid_x < 1 || plan->grid_x > units ||
+            plan->grid_y != 1 || plan->grid_z != 1 || plan->k_chunk != (V_all + 15) / 16)
+            return GPTQ_HIP_ERR_BAD_ARG;
+        const int upw = (units + plan->grid_x - 1) / plan->grid_x;
+        if (plan->lds_bytes < gptq::tiled_decode16_lds_bytes(mr, K, K / gs, upw) || plan->lds_bytes > 160 * 1024)
+            return GPTQ_HIP_ERR_BAD_ARG;
+        return gptq::launch_tiled_decode16(x, qtile, sz, kinv, bias, y, M, K, N, K / gs, bits, gs, *plan, stream);
+    }
     if (plan->kernel == GPTQ_HIP_KERNEL_TILED_DECODE) {
         const int mr = plan->row_tiles, kw = plan->waves_k;
         const int S_all = (K + 63) / 64;

@@ -490,7 +490,32 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
     if (M > gptq::kDecodeMaxRows) return GPTQ_HIP_ERR_UNSUPPORTED;
     const int gs = group_size == -1 ? K : group_size;
     {
-        // Decode: a workgroup per column tile of 32, enough waves along K to give the chip ~1000 waves, K cut
+        // One workgroup of sixteen waves per CU, units of 16 columns dealt out evenly, all of K staged once per
+        // workgroup (waves_n = 2 marks this kernel): whenever that fits LDS.
+        const int mr = gptq::tiled_decode_rows(M);
+        const int units = N / 16;
+        const int nwg = units < gptq::kNumCUs ? units : gptq::kNumCUs;
+        const int upw = ceil_div(units, nwg);
+        const long long lds = gptq::tiled_decode16_lds_bytes(mr, K, K / gs, upw);
+        if (lds <= 128 * 1024) {
+            plan->kernel = GPTQ_HIP_KERNEL_TILED_DECODE;
+            plan->row_tiles = mr;
+            plan->m_blocks = 1;
+            plan->waves_n = 2;
+            plan->waves_k = 16;
+            plan->split_k = 1;
+            plan->k_chunk = ceil_div(ceil_div(ceil_div(K, 64), 2), 16);  // virtual blocks per unit and wave
+            plan->grid_x = nwg;
+            plan->grid_y = 1;
+            plan->grid_z = 1;
+            plan->block = 1024;
+            plan->lds_bytes = (int)lds;
+            plan->workspace_bytes = 0;
+            return GPTQ_HIP_OK;
+        }
+    }
+    {
+        // Otherwise: a workgroup per column tile of 32, enough waves along K to give the chip ~1000 waves, K cut
         // over workgroups only when the staged x would not fit LDS.
         const int mr = gptq::tiled_decode_rows(M);
         const int tiles = N / 32;

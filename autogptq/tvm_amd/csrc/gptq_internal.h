@@ -192,12 +192,24 @@ inline int tiled_decode_lds_bytes(int mr, int span, int groups, int waves_k)
 {
     return mr * span * 2 + 64 + (span / 32) * mr * 8 + groups * 128 + waves_k * mr * 128;
 }
+// decode kernel with one workgroup per CU (16-column units, all of K staged): LDS of a workgroup that takes
+// `units_per_wg` units
+constexpr int kNumCUs = 256;   // MI355X
+inline long long tiled_decode16_lds_bytes(int mr, int K, int groups, int units_per_wg)
+{
+    const long long span = ((K + 63) / 64 + 1) / 2 * 128;
+    return mr * span * 2 + 64 + (span / 32) * mr * 8 + (long long)units_per_wg * groups * 128 +
+           (long long)units_per_wg * 16 * mr * 256;
+}
 int launch_tile_prepare(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
                         uint32_t *qtile, uint32_t *sz, int32_t *xsrc, uint16_t *kinv, int K, int N, int G, int bits,
                         int group_size, void *stream);
 int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, const uint16_t *kinv, const void *bias,
                         void *y, float *partial, int M, int K, int N, int G, int bits, int group_size,
                         const gptq_hip_plan &plan, void *stream);
+int launch_tiled_decode16(const void *x, const void *qtile, const uint32_t *sz, const uint16_t *kinv, const void *bias,
+                          void *y, int M, int K, int N, int G, int bits, int group_size, const gptq_hip_plan &plan,
+                          void *stream);
 int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int32_t *xsrc, const void *bias, void *y,
                  char *xpack, float *partial, int M, int K, int N, int G, int bits, int group_size,
                  const gptq_hip_plan &plan, void *stream);

@@ -25,6 +25,28 @@ def prepare(D):
     return ops.tile_prepare(D["qweight"], D["qzeros"], D["scales"], g, D["bits"], D["group_size"])
 
 
+def tile_decode_plan(M, K, N, bits, gs):
+    """The plan of the workgroup-per-tile decode kernel (the family's choice when x does not fit the LDS of the
+    one-workgroup-per-CU kernel), made by hand so that both kernels are tested on every shape."""
+    plan = _lib.select_tiled(M, K, N, bits, gs, decode=True)
+    if plan.waves_n != 2:
+        return plan
+    g = K if gs == -1 else gs
+    mr = 1 if M <= 1 else (2 if M <= 2 else 4)
+    tiles, S_total = N // 32, -(-K // 64)
+    kw = 4 if tiles * 4 >= 1024 else (8 if tiles * 8 >= 1024 else 16)
+    while kw > 4 and kw > S_total:
+        kw >>= 1
+    steps = -(-S_total // kw)
+    span = steps * kw * 64
+    groups = min((span - 1) // g + 2, K // g)
+    plan.waves_n, plan.waves_k, plan.split_k, plan.k_chunk = 1, kw, 1, steps
+    plan.grid_x, plan.grid_y, plan.grid_z, plan.block = tiles, 1, 1, 64 * kw
+    plan.lds_bytes = mr * span * 2 + 64 + (span // 32) * mr * 8 + groups * 128 + kw * mr * 128
+    plan.workspace_bytes = 0
+    return plan
+
+
 def run_tiled(D, prep, x=None, plan=None):
     qtile, sz, xsrc, kinv = prep
     act = D["desc_act"]
@@ -156,20 +178,28 @@ def test_tiled_decode_rows_and_shapes(dev, bits, K, N, gs, M):
     for desc_act in (False, True):
         L = layer(1600 + K + M, K, N, bits, gs, desc_act, M=M, bias=(M % 2 == 0))
         D = to_dev(L, dev)
-        plan = _lib.select_tiled(M, K, N, bits, gs, decode=True)
-        assert plan.kernel == _lib.KERNEL_TILED_DECODE and plan.row_tiles in (1, 2, 4) and plan.row_tiles >= M
-        # the family's own choice: this kernel up to four rows, the matmul kernel above
-        own = _lib.select_tiled(M, K, N, bits, gs)
-        assert own.kernel == (_lib.KERNEL_TILED_DECODE if M <= 4 else _lib.KERNEL_TILED)
+        own = _lib.select_tiled(M, K, N, bits, gs)   # the family's own choice: a decode kernel up to four rows
+        assert own.kernel == _lib.KERNEL_TILED_DECODE and own.row_tiles in (1, 2, 4) and own.row_tiles >= M
+        assert own.waves_n == 2                      # (these shapes fit the one-workgroup-per-CU kernel)
         prep = prepare(D)
-        y = run_tiled(D, prep, plan=plan)
         want = expected_output(L)
-        assert_close(y, want, f"decode bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
-        assert_tight(y, want, f"decode bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
-        assert torch.equal(y, run_tiled(D, prep, plan=plan)), "two identical calls differ"
         g = D["g_idx"] if desc_act else None
-        assert_tight(y, ops.gemm(D["x"], D["qweight"], D["qzeros"], D["scales"], g, D.get("bias"), bits, gs).cpu(),
-                     "decode vs the unprepared kernels")
+        plain = ops.gemm(D["x"], D["qweight"], D["qzeros"], D["scales"], g, D.get("bias"), bits, gs).cpu()
+        plans = [("cu", own), ("tile", tile_decode_plan(M, K, N, bits, gs))]
+        few = _lib.select_tiled(M, K, N, bits, gs)   # the same kernel on fewer workgroups: several units each
+        few.grid_x = max(1, (N // 16) // 5)
+        upw = -(-(N // 16) // few.grid_x)
+        span = -(-(-(-K // 64)) // 2) * 128
+        g = K if gs == -1 else gs
+        few.lds_bytes = few.row_tiles * span * 2 + 64 + span // 32 * few.row_tiles * 8 + upw * (K // g) * 128 + upw * 16 * few.row_tiles * 256
+        if few.lds_bytes <= 128 * 1024:
+            plans.append(("cu, few workgroups", few))
+        for what, plan in plans:
+            y = run_tiled(D, prep, plan=plan)
+            assert_close(y, want, f"decode ({what}) bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
+            assert_tight(y, want, f"decode ({what}) bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
+            assert torch.equal(y, run_tiled(D, prep, plan=plan)), "two identical calls differ"
+            assert_tight(y, plain, "decode vs the unprepared kernels")
 
 
 @pytest.mark.parametrize("bits", [3, 4])
@@ -180,7 +210,7 @@ def test_tiled_decode_split_k(dev, bits, M):
     L = layer(1700 + M, K, N, bits, gs, True, M=M, bias=True)
     D = to_dev(L, dev)
     prep = prepare(D)
-    plan = _lib.select_tiled(M, K, N, bits, gs, decode=True)
+    plan = tile_decode_plan(M, K, N, bits, gs)
     for split in (2, 4):           # two blocks per wave (paired epilogue) and one (the one-block epilogue)
         plan.split_k = plan.grid_y = split
         plan.k_chunk = -(-(K // 64) // (split * plan.waves_k))
@@ -211,12 +241,13 @@ def test_tiled_decode_full_size(dev, name, bits, K, N, gs, desc_act, Ms):
     prep = prepare(D)
     for M in Ms:
         x = L["x"][:M].contiguous()
-        plan = _lib.select_tiled(M, K, N, bits, gs, decode=True)
-        y = run_tiled(D, prep, x=x.to(dev), plan=plan)
         want = expected_output(L, x=x, w16=w16)
-        assert_close(y, want, f"decode {name} M={M}")
-        assert_tight(y, want, f"decode {name} M={M}")
-        assert torch.equal(y, run_tiled(D, prep, x=x.to(dev), plan=plan)), f"decode {name} M={M}: two identical calls differ"
+        for plan in (_lib.select_tiled(M, K, N, bits, gs, decode=True), tile_decode_plan(M, K, N, bits, gs)):
+            y = run_tiled(D, prep, x=x.to(dev), plan=plan)
+            what = f"decode {name} M={M} ({'cu' if plan.waves_n == 2 else 'tile'})"
+            assert_close(y, want, what)
+            assert_tight(y, want, what)
+            assert torch.equal(y, run_tiled(D, prep, x=x.to(dev), plan=plan)), f"{what}: two identical calls differ"
 
 
 TILED_FULL = [
