@@ -490,14 +490,17 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
     if (M > gptq::kDecodeMaxRows) return GPTQ_HIP_ERR_UNSUPPORTED;
     const int gs = group_size == -1 ? K : group_size;
     {
-        // One workgroup of sixteen waves per CU, units of 16 columns dealt out evenly, all of K staged once per
-        // workgroup (waves_n = 2 marks this kernel): whenever that fits LDS.
+        // Layers of up to 16 columns per CU (N <= 4096): one workgroup of sixteen waves per 16-column unit, all of
+        // K staged once per workgroup (waves_n = 2 marks this kernel), when that fits LDS.  Every CU then has
+        // work (a workgroup per 32-column tile leaves half of them idle): 11008 x 4096, one row, 9.0 / 9.3 us
+        // (int4 / int3) against 10.4 / 11.0; 4096 x 4096 5.3 against 5.4-5.5.  Wider layers would give a workgroup
+        // several units; there the kernel below is faster (4096 x 11008: 7.7 / 7.8 us against 9.0 / 9.3).
         const int mr = gptq::tiled_decode_rows(M);
         const int units = N / 16;
         const int nwg = units < gptq::kNumCUs ? units : gptq::kNumCUs;
         const int upw = ceil_div(units, nwg);
         const long long lds = gptq::tiled_decode16_lds_bytes(mr, K, K / gs, upw);
-        if (lds <= 128 * 1024) {
+        if (upw == 1 && lds <= 128 * 1024) {
             plan->kernel = GPTQ_HIP_KERNEL_TILED_DECODE;
             plan->row_tiles = mr;
             plan->m_blocks = 1;

@@ -31,6 +31,10 @@ def tile_decode_plan(M, K, N, bits, gs):
     plan = _lib.select_tiled(M, K, N, bits, gs, decode=True)
     if plan.waves_n != 2:
         return plan
+    return tile_decode_plan_of(plan, M, K, N, bits, gs)
+
+
+def tile_decode_plan_of(plan, M, K, N, bits, gs):
     g = K if gs == -1 else gs
     mr = 1 if M <= 1 else (2 if M <= 2 else 4)
     tiles, S_total = N // 32, -(-K // 64)
@@ -44,6 +48,25 @@ def tile_decode_plan(M, K, N, bits, gs):
     plan.grid_x, plan.grid_y, plan.grid_z, plan.block = tiles, 1, 1, 64 * kw
     plan.lds_bytes = mr * span * 2 + 64 + (span // 32) * mr * 8 + groups * 128 + kw * mr * 128
     plan.workspace_bytes = 0
+    return plan
+
+
+def cu_decode_plan(M, K, N, bits, gs, grid=None):
+    """The plan of the one-workgroup-per-CU decode kernel (16-column units), whatever the family would choose;
+    ``grid`` workgroups (default: one per unit up to 256).  None when x and the tables do not fit LDS."""
+    plan = _lib.select_tiled(M, K, N, bits, gs, decode=True)
+    g = K if gs == -1 else gs
+    units = N // 16
+    grid = grid or min(units, 256)
+    upw = -(-units // grid)
+    mr = 1 if M <= 1 else (2 if M <= 2 else 4)
+    V = -(-(-(-K // 64)) // 2)
+    span = V * 128
+    lds = mr * span * 2 + 64 + span // 32 * mr * 8 + upw * (K // g) * 128 + upw * 16 * mr * 256
+    if lds > 150 * 1024:
+        return None
+    plan.row_tiles, plan.waves_n, plan.waves_k, plan.split_k, plan.k_chunk = mr, 2, 16, 1, -(-V // 16)
+    plan.grid_x, plan.grid_y, plan.grid_z, plan.block, plan.lds_bytes, plan.workspace_bytes = grid, 1, 1, 1024, lds, 0
     return plan
 
 
@@ -180,21 +203,16 @@ def test_tiled_decode_rows_and_shapes(dev, bits, K, N, gs, M):
         D = to_dev(L, dev)
         own = _lib.select_tiled(M, K, N, bits, gs)   # the family's own choice: a decode kernel up to four rows
         assert own.kernel == _lib.KERNEL_TILED_DECODE and own.row_tiles in (1, 2, 4) and own.row_tiles >= M
-        assert own.waves_n == 2                      # (these shapes fit the one-workgroup-per-CU kernel)
         prep = prepare(D)
         want = expected_output(L)
         g = D["g_idx"] if desc_act else None
         plain = ops.gemm(D["x"], D["qweight"], D["qzeros"], D["scales"], g, D.get("bias"), bits, gs).cpu()
-        plans = [("cu", own), ("tile", tile_decode_plan(M, K, N, bits, gs))]
-        few = _lib.select_tiled(M, K, N, bits, gs)   # the same kernel on fewer workgroups: several units each
-        few.grid_x = max(1, (N // 16) // 5)
-        upw = -(-(N // 16) // few.grid_x)
-        span = -(-(-(-K // 64)) // 2) * 128
-        g = K if gs == -1 else gs
-        few.lds_bytes = few.row_tiles * span * 2 + 64 + span // 32 * few.row_tiles * 8 + upw * (K // g) * 128 + upw * 16 * few.row_tiles * 256
-        if few.lds_bytes <= 128 * 1024:
-            plans.append(("cu, few workgroups", few))
+        # both decode kernels, and the one-workgroup-per-CU kernel on fewer workgroups (several units each)
+        plans = [("own", own), ("tile", tile_decode_plan(M, K, N, bits, gs)), ("cu", cu_decode_plan(M, K, N, bits, gs)),
+                 ("cu, few workgroups", cu_decode_plan(M, K, N, bits, gs, grid=max(1, (N // 16) // 5)))]
         for what, plan in plans:
+            if plan is None:
+                continue
             y = run_tiled(D, prep, plan=plan)
             assert_close(y, want, f"decode ({what}) bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
             assert_tight(y, want, f"decode ({what}) bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
@@ -242,7 +260,9 @@ def test_tiled_decode_full_size(dev, name, bits, K, N, gs, desc_act, Ms):
     for M in Ms:
         x = L["x"][:M].contiguous()
         want = expected_output(L, x=x, w16=w16)
-        for plan in (_lib.select_tiled(M, K, N, bits, gs, decode=True), tile_decode_plan(M, K, N, bits, gs)):
+        for plan in (tile_decode_plan(M, K, N, bits, gs), cu_decode_plan(M, K, N, bits, gs)):
+            if plan is None:
+                continue
             y = run_tiled(D, prep, x=x.to(dev), plan=plan)
             what = f"decode {name} M={M} ({'cu' if plan.waves_n == 2 else 'tile'})"
             assert_close(y, want, what)
