@@ -267,20 +267,28 @@ def gemm_tiled(x: torch.Tensor, qtile: torch.Tensor, sz: torch.Tensor, xsrc: Opt
     return out
 
 
-def tiled_wins(M: int, K: int, N: int, act_order: bool) -> bool:
+def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
     """Where the tiled kernels were measured faster than the ones that read the checkpoint layout (or its
-    sorted copy), on MI355X with the weights cold, group size 128, 3 and 4 bits:
-      * up to 4 rows (its decode kernel, one workgroup per 32 columns): layers of up to 8192 columns, where
-        every workgroup has a CU to itself: 4096 x 4096 6.2-7.9 us against 7.1-10.9; 11008 x 4096 with an
-        activation order 11.9/13.0 against 13.4/15.5 at one and two rows, behind from four rows on and
-        without an activation order (14.8 against 12.9); 4096 x 11008 9.2 against 8.2;
+    sorted copy), on MI355X with the weights cold, group size 128 (us, graph replay):
+      * up to 4 rows, layers of up to 4096 columns (decode kernel with a workgroup per 16 columns, every CU at
+        work): always.  4096 x 4096: 5.3-5.6 at one row, 7.4-8.0 at four, against 6.8-7.5 and 7.8-10.5;
+        11008 x 4096: 9.5-9.7 / 12.7-14.4 against 9.4-13.3 / 12.7-15.3;
+      * up to 4 rows, wider layers (a workgroup per 32 columns, x staged per workgroup): K up to 6144 and at
+        most two rows, for 4-bit layers and for two rows under an activation order.  4096 x 11008 with an
+        activation order, one / two rows: int4 7.9 / 8.9 against 8.2 / 11.0, int3 8.0 / 8.9 against 7.7 / 10.3;
+        without: int4 7.9 / 8.5 against 7.9 / 9.0, int3 8.0 / 8.3 against 7.3 / 8.2; three and four rows are
+        behind by 0.5-2 us; 5120 x 5120 int4 6.3 against 13.4-15.2; 8192 x 8192 int3 13.2-13.9 against 11.2;
       * 5 to 16 rows: never (4096 x 11008, 8 rows: 14.6 against 13.4);
       * 17 to 128 rows: everywhere within 4 % or better (4096 x 11008 with an activation order, 32/64/128
-        rows: 14.8/19.2/26.6 against 18.1/22.1/34.1 us);
+        rows: 14.8/19.2/26.6 against 18.1/22.1/34.1);
       * above 128 rows: K up to 8192 (4096 x 11008, 512 rows: 75 against 95; 11008 x 4096: 127 against 81,
         where every workgroup pulls 2.8 MB of x fragments and they no longer stay in one L2)."""
     if M <= 4:
-        return N <= 8192 and (K <= 4096 or (act_order and M <= 2))
+        if N <= 4096:
+            return True
+        if K > 6144:
+            return False
+        return M <= 2 and (bits == 4 or (act_order and M == 2))
     if M <= 16:
         return False
     return M <= 128 or K <= 8192

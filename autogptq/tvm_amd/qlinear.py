@@ -264,7 +264,7 @@ class QuantLinear(nn.Module):
         g = self._kernel_g_idx()
         K, N = self.infeatures, self.outfeatures
         tiled = None
-        if self.tile_for_prefill and ops.tiled_wins(M, K, N, g is not None):
+        if self.tile_for_prefill and ops.tiled_wins(M, K, N, g is not None, bits):
             tiled = self.prepare_tiled()
         threshold = self.kernel_switch_threshold
         if threshold and self.act_order_switch_threshold and g is not None and tiled is None:

@@ -185,7 +185,7 @@ def prepared_mode(name: str):
     from autogptq.tvm_amd import ops
 
     bits, K, N, gs, desc_act, M = WORKLOADS[name]
-    if tiled_applies(name) and ops.tiled_wins(M, K, N, desc_act):
+    if tiled_applies(name) and ops.tiled_wins(M, K, N, desc_act, bits):
         return "tiled"
     return "sorted" if sorted_applies(name) else None
 

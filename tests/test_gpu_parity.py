@@ -541,7 +541,7 @@ def test_quantlinear_decode_uses_the_sorted_copy(dev, bits):
     K, N, gs = 2048, 12288, 128   # wide enough for the decode family to take two rows as well (and for the
     #                               module to prefer the sorted copy over the tiled one at these row counts)
     L = layer(44, K, N, bits, gs, True, M=2, bias=True)
-    q = QuantLinear(bits, gs, K, N, True)
+    q = QuantLinear(bits, gs, K, N, True, tile_for_prefill=False)   # (this test is about the sorted copy)
     q.load_state_dict({k: L[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})
     q = q.to(dev)
     assert q._sorted is None
