@@ -354,3 +354,23 @@ def test_quantlinear_compact_keeps_one_copy(dev, bits, desc_act):
     xg = x[:4].clone().requires_grad_(True)
     q(xg).float().sum().backward()
     assert xg.grad is not None and xg.grad.shape == xg.shape
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_long_prompts_run_fused_on_the_tiled_kernels(dev, bits):
+    """1024 and 4096 rows stay on the fused path when the switch to the library GEMM is off (and always on a
+    compact layer): the matmul kernel walks the row blocks itself."""
+    K, N, gs = 512, 192, 128
+    L = layer(2000 + bits, K, N, bits, gs, True, M=4096, bias=True)
+    q = module_of(L, dev, kernel_switch_threshold=None)
+    x = L["x"].to(dev)
+    want = expected_output(L)
+    for M in (1024, 4096):
+        assert q.route(M) == "tiled"
+        y = q(x[:M])
+        assert_close(y, want[:M], f"module, {M} rows")
+        assert_tight(y, want[:M], f"module, {M} rows")
+    q.kernel_switch_threshold = 1024
+    assert q.route(1024) == "library" and q.route(1023) == "tiled"
+    assert q.compact() and q.route(4096) == "tiled"
+    assert_tight(q(x), want, "compact module, 4096 rows")
