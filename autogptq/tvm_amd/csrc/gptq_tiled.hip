@@ -22,7 +22,8 @@
 // matrix instructions of the current one.  Weights, (scale, zero) words and fragments ride in register
 // rings RING blocks deep, requested in the order they are consumed (vector loads return in order on one
 // counter, so a wait for a fragment also waits for every older load).
-// Measured alternatives that were no faster: eight waves per workgroup (two per SIMD, 64-row waves, two row
+// Measured alternatives that were no faster: an L2 prefetch of the weights through scalar loads (slower: the
+// scalar path does not sustain the rate); eight waves per workgroup (two per SIMD, 64-row waves, two row
 // halves x four K slices or eight K slices); a wave's whole weight range brought into LDS up front with
 // global_load_lds (a CU draws ~35 GB/s from HBM, and those 3.7 us then stand in front of the first matrix
 // instruction).  What bounds the 128-row kernel is the A stream (every workgroup reads all of x through its
