@@ -45,7 +45,7 @@ ABI_SYMBOLS = (
     "gptq_hip_abi_version",
     "gptq_hip_build_id",
 )
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class Plan(ctypes.Structure):

@@ -47,10 +47,14 @@ enum {
                                    (row_tiles = 1, 2 or 4) x 64 columns per workgroup of waves_k = 4 waves along K
                                    (k_chunk = blocks of 64 channels per wave); x is pre-packed into the
                                    workspace; split_k > 1 adds a reduce launch */
-    GPTQ_HIP_KERNEL_TILED_DECODE = 5 /* the same layer for M <= 4 rows: a workgroup per 32 columns, waves_k (4, 8 or 16)
-                                   waves along K, x staged in LDS in the layer's sorted order; scales applied per
-                                   block of 32 channels; row_tiles = the rows the kernel is built for (1, 2, 4 or 8);
-                                   split_k > 1 (an x that does not fit LDS) adds a reduce launch */
+    GPTQ_HIP_KERNEL_TILED_DECODE = 5 /* the same layer for M <= 4 rows, x staged in LDS in the layer's sorted order,
+                                   scales applied per 32 or 64 channels; row_tiles = the rows the kernel is built
+                                   for (1, 2 or 4).  waves_n = 1: a workgroup per 32 columns, waves_k (4, 8 or 16)
+                                   waves along K with k_chunk blocks of 64 channels each; split_k > 1 (an x that
+                                   does not fit LDS) adds a reduce launch.  waves_n = 2: units of 16 columns dealt
+                                   out evenly over grid_x workgroups of 16 waves, all of K staged per workgroup
+                                   (k_chunk = blocks of 128 channels per unit and wave); chosen for layers of up to
+                                   4096 columns */
 };
 
 /* What the dispatcher decided for one problem; filled by gptq_hip_select. */
@@ -226,7 +230,7 @@ int gptq_hip_dequant(const int32_t *qweight, const int32_t *qzeros, const void *
 const char *gptq_hip_strerror(int status);
 
 /* ABI version of this library (bumped when a signature or gptq_hip_plan changes). */
-#define GPTQ_HIP_ABI_VERSION 2
+#define GPTQ_HIP_ABI_VERSION 3
 int gptq_hip_abi_version(void);
 
 /* Digest of the sources this library was built from (set by the build script; "unknown" otherwise), so that a
