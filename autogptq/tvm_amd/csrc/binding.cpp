@@ -15,6 +15,7 @@
 #include <torch/custom_class.h>
 #include <torch/library.h>
 
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <optional>
@@ -238,26 +239,30 @@ struct Layer : torch::CustomClassHolder {
         TORCH_CHECK(kind != 1 || has(d), "the sorted copy needs its kmap");
     }
 
-    // What the last fully checked call fixed for its row count: later calls with the same M check x only.
-    int64_t fast_M = -1, K = 0, N = 0;
+    // What the first fully checked call fixed for its row count: later calls with the same M check x only.
+    // Written once, under the mutex, before fast_M is published; calls with another M take the checked path.
+    std::atomic<int64_t> fast_M{-1};
+    int64_t K = 0, N = 0;
     gptq_hip_plan plan{};
     size_t ws_need = 0;
+    std::mutex fix_mutex;
 
     Tensor forward(const Tensor &x)
     {
-        if (x.dim() == 2 && x.size(0) == fast_M) {
+        const int64_t fast_rows = fast_M.load(std::memory_order_acquire);
+        if (x.dim() == 2 && x.size(0) == fast_rows) {
             TORCH_CHECK(x.is_cuda() && x.device() == a.device(), "x is on ", x.device(), ", the layer on ", a.device(),
                         ": the GPTQ kernels run on a ROCm GPU only and there is no CPU fallback");
             TORCH_CHECK(x.scalar_type() == at::kHalf && x.is_contiguous() && x.size(1) == K,
                         "x must be a contiguous fp16 [M, ", K, "] matrix");
-            Tensor y = at::empty({fast_M, N}, x.options());
+            Tensor y = at::empty({fast_rows, N}, x.options());
             const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
             void *stream = (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(x.get_device()).stream();
             Tensor ws;
             if (ws_need) ws = workspace(x, ws_need, stream);
             void *wsp = ws.defined() ? ws.data_ptr() : nullptr;
             const size_t wsb = ws.defined() ? (size_t)ws.numel() : 0;
-            const int M = (int)fast_M, bi = (int)bits, gs = (int)group_size;
+            const int M = (int)fast_rows, bi = (int)bits, gs = (int)group_size;
             int rc;
             if (kind == 0)
                 rc = gptq_hip_gemm_plan(x.data_ptr(), (const int32_t *)a.data_ptr(), (const int32_t *)b.data_ptr(), c.data_ptr(),
@@ -271,7 +276,7 @@ struct Layer : torch::CustomClassHolder {
                 rc = gptq_hip_gemm_tiled(x.data_ptr(), a.data_ptr(), (const uint32_t *)b.data_ptr(), (const int32_t *)ptr(d),
                                          (const uint16_t *)ptr(e), ptr(bias), y.data_ptr(), wsp, wsb, M, (int)K, (int)N, bi, gs,
                                          &plan, stream);
-            raise(rc, "gptq_hip.Layer.forward", fast_M, K, N, bits, group_size);
+            raise(rc, "gptq_hip.Layer.forward", fast_rows, K, N, bits, group_size);
             return y;
         }
         // the checked path; what it selects is what the operators select
@@ -286,18 +291,19 @@ struct Layer : torch::CustomClassHolder {
         default:
             y = gemm_tiled(x, a, b, d, e, bias, bits, group_size);
         }
-        if (x.size(0) > 0) {
+        if (x.size(0) > 0 && fast_rows < 0) {
             const int M = (int)x.size(0), Ki = (int)x.size(1), Ni = (int)y.size(1), bi = (int)bits, gs = (int)group_size;
             gptq_hip_plan p;
             const int rc = kind == 2 ? gptq_hip_select_tiled(M, Ki, Ni, bi, gs, &p)
                                      : gptq_hip_select(M, Ki, Ni, bi, gs, kind == 0 && has(d), &p);
-            if (rc == GPTQ_HIP_OK) {
+            const std::lock_guard<std::mutex> lock(fix_mutex);
+            if (rc == GPTQ_HIP_OK && fast_M.load(std::memory_order_relaxed) < 0) {
                 plan = p;
                 ws_need = p.workspace_bytes;
                 if (kind == 1) ws_need = std::max(ws_need, gptq_hip_sorted_workspace_bytes(M, Ki, Ni, bi, gs));
                 K = Ki;
                 N = Ni;
-                fast_M = M;
+                fast_M.store(M, std::memory_order_release);
             }
         }
         return y;

@@ -389,8 +389,10 @@ extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint3
     const int S_total = (K + 63) / 64;
     if (plan->kernel != GPTQ_HIP_KERNEL_TILED || (rts != 1 && rts != 2 && rts != 4)) return GPTQ_HIP_ERR_UNSUPPORTED;
     const int kwv = 4;
+    const int ct = 2 * plan->waves_n;   // 32-column tiles per wave: 2, or 4 (with four row tiles only)
+    if ((ct != 2 && ct != 4) || (ct == 4 && rts != 4)) return GPTQ_HIP_ERR_BAD_ARG;
     if (plan->block != 64 * kwv || plan->waves_k != kwv || plan->split_k < 1 || plan->k_chunk < 1 || plan->m_blocks < 1 ||
-        plan->grid_x != (N / 32 + 1) / 2 || plan->grid_y != plan->split_k || plan->grid_z != plan->m_blocks ||
+        plan->grid_x != (N / 32 + ct - 1) / ct || plan->grid_y != plan->split_k || plan->grid_z != plan->m_blocks ||
         (long long)plan->m_blocks * 32 * rts < M || (long long)plan->split_k * kwv * plan->k_chunk < S_total ||
         plan->lds_bytes < gptq::tiled_lds_bytes(rts, kwv) || plan->lds_bytes > 160 * 1024)
         return GPTQ_HIP_ERR_BAD_ARG;

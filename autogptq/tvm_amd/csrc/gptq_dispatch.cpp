@@ -566,7 +566,15 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     const int at = gptq::tiled_row_tiles(M), rw = 1, kwv = 4;
     const int rows = 32 * at * rw;
     const int m_blocks = ceil_div(M, rows);
-    const int col_pairs = ceil_div(N / 32, 2);
+    // several row blocks: 128 columns per wave (waves_n = 2), which halves the x fragments a matrix instruction
+    // needs; one row block keeps 64 columns, for more workgroups
+    // (when that still leaves a workgroup for two of three CUs, or when K is long: the fragments of a row block
+    // then need the larger share of L2 that fewer, wider workgroups leave them.  4096 x 11008: 256 rows 49.6 ->
+    // 41.9 us, 1024 rows 142 -> 123; 11008 x 4096, 512 rows: 127 -> 88; 4096 x 4096, 512 rows, 128 workgroups:
+    // 33.5 -> 40.4, so not there)
+    const bool wide = m_blocks >= 2 && ((long long)ceil_div(N / 32, 4) * m_blocks >= 172 || K > 8192);
+    const int ct = wide ? 4 : 2;
+    const int col_pairs = ceil_div(N / 32, ct);
     const int S_total = ceil_div(K, 64);
     const long long tiles = (long long)col_pairs * m_blocks;
     int split = (int)((256 + tiles / 2) / tiles);
@@ -582,7 +590,7 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     plan->kernel = GPTQ_HIP_KERNEL_TILED;
     plan->row_tiles = at * rw;
     plan->m_blocks = m_blocks;
-    plan->waves_n = 1;
+    plan->waves_n = ct / 2;
     plan->waves_k = kwv;
     plan->split_k = split;
     plan->k_chunk = wave_steps;  // blocks of 64 positions per wave

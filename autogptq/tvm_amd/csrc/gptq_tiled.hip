@@ -250,8 +250,11 @@ __device__ __forceinline__ h8 tiled_bop(const uint32_t (&w)[BITS], int j, h2 s2,
 }
 
 // AT: 32-row tiles per wave.  RW x KW: waves of the workgroup along M and along K: the workgroup holds
-// 32 * AT * RW rows, and its KW waves along K split the workgroup's K range.
-template <int BITS, int AT, int RW, int KW, int RING>
+// 32 * AT * RW rows, and its KW waves along K split the workgroup's K range.  CT: 32-column tiles per wave (2, or
+// 4 for problems of several row blocks: a fragment of x then feeds four matrix instructions instead of two,
+// which halves the fragment traffic per flop, and the 256 accumulator registers fill the wave's second
+// register file).
+template <int BITS, int AT, int RW, int KW, int RING, int CT>
 __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledParams p)
 {
     const int tid = threadIdx.x;
@@ -259,7 +262,7 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int rw = wave % RW, kw = wave / RW;
     const int n = lane & 31, h = lane >> 5;
-    const int T0 = 2 * blockIdx.x;
+    const int T0 = CT * blockIdx.x;
     const int split = blockIdx.y;
     const int rt0 = (blockIdx.z * RW + rw) * AT;
     const int S_begin = (split * KW + kw) * p.wave_steps;
@@ -267,10 +270,10 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
     const int lb_last = 2 * p.S_total - 1;
 
     // per-lane offsets that never change; the block number lives in scalar registers
-    uint32_t tile_off[2], col[2];
+    uint32_t tile_off[CT], col[CT];
 #pragma unroll
-    for (int ct = 0; ct < 2; ct++) {
-        const int T = min(T0 + ct, p.T_total - 1);  // a missing second tile repeats the first; it is never stored
+    for (int ct = 0; ct < CT; ct++) {
+        const int T = min(T0 + ct, p.T_total - 1);  // a missing tile repeats the last one; it is never stored
         tile_off[ct] = (uint32_t)T * (uint32_t)p.S_total;
         col[ct] = (uint32_t)(32 * T + n);
     }
@@ -278,15 +281,15 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
     const uint32_t a_lane = (uint32_t)rt0 * 1024u + (uint32_t)lane * 16u;
     const uint32_t a_frag_row = (uint32_t)p.rt_total * 1024u;  // bytes between consecutive (S, j)
 
-    uint32_t w[RING][2][BITS];
-    uint32_t szr[RING][2];
+    uint32_t w[RING][CT][BITS];
+    uint32_t szr[RING][CT];
     h8 a[RING][4][AT];
-    auto load_b = [&](int S, uint32_t (&wr)[2][BITS], uint32_t (&sr)[2]) {
+    auto load_b = [&](int S, uint32_t (&wr)[CT][BITS], uint32_t (&sr)[CT]) {
         const int Sc = min(S, S_last);  // blocks past K repeat the last one (their x is zero)
         const uint32_t lb = (uint32_t)min(2 * S + h, lb_last);
         const uint32_t g = min(lb / (uint32_t)p.lb_per_group, (uint32_t)p.G - 1u);
 #pragma unroll
-        for (int ct = 0; ct < 2; ct++) {
+        for (int ct = 0; ct < CT; ct++) {
             const char *src = p.qtile + ((size_t)(tile_off[ct] + (uint32_t)Sc) * (256u * BITS) + b_lane);
             if constexpr (BITS == 4) {
                 const u4 v = __builtin_nontemporal_load((const u4 *)src);
@@ -326,11 +329,11 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    f16v acc[AT][2];
+    f16v acc[AT][CT];
 #pragma unroll
     for (int rt = 0; rt < AT; rt++)
 #pragma unroll
-        for (int ct = 0; ct < 2; ct++)
+        for (int ct = 0; ct < CT; ct++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[rt][ct][v] = 0.f;
 
@@ -348,11 +351,11 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
     };
 
     // the first operand of the walk
-    h2 cs[2], cza[2], czb[2];  // (scale, base + zero) of the block being dequantised, per column tile
+    h2 cs[CT], cza[CT], czb[CT];  // (scale, base + zero) of the block being dequantised, per column tile
     consts_of(szr[0][0], cs[0], cza[0], czb[0]);
     h8 bop_next = tiled_bop<BITS>(w[0][0], 0, cs[0], cza[0], czb[0], magic_a, magic_b);
 
-    // One block of the walk (ring slot u): the eight (j, ct) operands, each multiplied with the AT row tiles
+    // One block of the walk (ring slot u): the 4 CT (j, ct) operands, each multiplied with the AT row tiles
     // while the next operand of the walk is dequantised.  REFILL: the slot's registers are requested again
     // for the block a ring ahead as soon as their last reader is done.
     auto block = [&](auto u_c, auto refill_c) {
@@ -362,13 +365,13 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
 #pragma unroll
         for (int j = 0; j < 4; j++) {
 #pragma unroll
-            for (int ct = 0; ct < 2; ct++) {
+            for (int ct = 0; ct < CT; ct++) {
                 const h8 bop = bop_next;
                 {
-                    const int jn = ct == 1 ? (j + 1) & 3 : j;
-                    const int ctn = ct ^ 1;
+                    const int jn = ct == CT - 1 ? (j + 1) & 3 : j;
+                    const int ctn = ct == CT - 1 ? 0 : ct + 1;
                     constexpr int u1 = (u + 1) % RING;
-                    const bool wrap_u = ct == 1 && j == 3;
+                    const bool wrap_u = ct == CT - 1 && j == 3;
                     if (jn == 0) consts_of(wrap_u ? szr[u1][ctn] : szr[u][ctn], cs[ctn], cza[ctn], czb[ctn]);  // first operand of a block
                     bop_next = wrap_u ? tiled_bop<BITS>(w[u1][ctn], jn, cs[ctn], cza[ctn], czb[ctn], magic_a, magic_b)
                                       : tiled_bop<BITS>(w[u][ctn], jn, cs[ctn], cza[ctn], czb[ctn], magic_a, magic_b);
@@ -377,9 +380,9 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
                 for (int rt = 0; rt < AT; rt++) {
                     acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[u][j][rt], bop, acc[rt][ct], 0, 0, 0);
                 }
-                if (REFILL && ct == 1) {
+                if (REFILL && ct == CT - 1) {
                     __builtin_amdgcn_sched_barrier(0);
-                    if (j == 3) load_b(S_refill, w[u], szr[u]);  // (its last reader, the operand of (3, 1), is done)
+                    if (j == 3) load_b(S_refill, w[u], szr[u]);  // (its last reader, the last operand of the block, is done)
                     load_a(S_refill, j, a[u][j]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -402,52 +405,57 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
         }(std::make_integer_sequence<int, RING>{});
     }
 
-    // ---- the waves along K meet in LDS: [wave][tile rt * 2 + ct][v][lane] floats --------------------
+    // ---- the waves along K meet in LDS, EP row tiles at a time: [wave][tile rtp * CT + ct][v][lane] floats ----
+    constexpr int EP = AT * CT <= 8 ? AT : 8 / CT;   // row tiles per pass (at most eight 4 KB tiles per wave in LDS)
     float *red = (float *)smem;
-    {
-        float *dst = red + (size_t)wave * (AT * 2) * 1024 + lane;
-#pragma unroll
-        for (int rt = 0; rt < AT; rt++)
-#pragma unroll
-            for (int ct = 0; ct < 2; ct++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) dst[((rt * 2 + ct) * 16 + v) * 64] = acc[rt][ct][v];
-    }
-    __syncthreads();
-    // one item = four adjacent columns of one row: element v of lane (n, h) of tile (rt, ct) of a wave in row
-    // group rw is row 32 (AT rw + rt) + 8 (v / 4) + 4 h + v % 4, column 32 ct + n
     const int m0 = 32 * AT * RW * blockIdx.z;
     const _Float16 *bias = (const _Float16 *)p.bias;
     _Float16 *y = (_Float16 *)p.y;
     constexpr int NT = 64 * RW * KW;
 #pragma unroll
-    for (int it = 0; it < 512 * AT * RW / NT; it++) {
-        const int item = tid + NT * it;
-        const int r = item >> 4, c4 = (item & 15) * 4;
-        const int ct = c4 >> 5, nn = c4 & 31;
-        const int rtw = r >> 5, rr = r & 31;          // 32-row tile of the workgroup
-        const int rwi = rtw / AT, rt = rtw % AT;      // its row group and tile inside the wave
-        const int v = 4 * (rr >> 3) + (rr & 3), hh = (rr >> 2) & 1;
-        const float *src = red + ((size_t)rwi * (AT * 2) + rt * 2 + ct) * 1024 + v * 64 + hh * 32 + nn;
-        f4 sum = *(const f4 *)src;
+    for (int rp = 0; rp < AT; rp += EP) {
+        if (rp > 0) __syncthreads();   // the previous pass has been read
+        {
+            float *dst = red + (size_t)wave * (EP * CT) * 1024 + lane;
 #pragma unroll
-        for (int k = 1; k < KW; k++) sum += *(const f4 *)(src + (size_t)k * RW * (AT * 2) * 1024);
-        const int row = m0 + r;
-        const int T = T0 + ct;
-        if (row < p.M && T < p.T_total) {
-            const size_t o = (size_t)row * p.N + 32 * T + nn;
-            if (p.split_k == 1) {
-                if (bias) {
-                    const h4 b4 = *(const h4 *)(bias + 32 * T + nn);
+            for (int rt = 0; rt < EP; rt++)
 #pragma unroll
-                    for (int c = 0; c < 4; c++) sum[c] += (float)b4[c];
+                for (int ct = 0; ct < CT; ct++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) dst[((rt * CT + ct) * 16 + v) * 64] = acc[rp + rt][ct][v];
+        }
+        __syncthreads();
+        // one item = four adjacent columns of one row: element v of lane (n, h) of tile (rt, ct) of a wave in row
+        // group rw is row 32 (AT rw + rt) + 8 (v / 4) + 4 h + v % 4, column 32 ct + n
+#pragma unroll
+        for (int it = 0; it < 32 * EP * RW * 8 * CT / NT; it++) {
+            const int item = tid + NT * it;
+            const int r = item / (8 * CT), c4 = (item % (8 * CT)) * 4;
+            const int ct = c4 >> 5, nn = c4 & 31;
+            const int rtw = r >> 5, rr = r & 31;          // 32-row tile of the pass
+            const int rwi = rtw / EP, rt = rtw % EP;      // its row group and tile inside the wave's pass
+            const int v = 4 * (rr >> 3) + (rr & 3), hh = (rr >> 2) & 1;
+            const float *src = red + ((size_t)rwi * (EP * CT) + rt * CT + ct) * 1024 + v * 64 + hh * 32 + nn;
+            f4 sum = *(const f4 *)src;
+#pragma unroll
+            for (int k = 1; k < KW; k++) sum += *(const f4 *)(src + (size_t)k * RW * (EP * CT) * 1024);
+            const int row = m0 + 32 * (AT * rwi + rp + rt) + rr;
+            const int T = T0 + ct;
+            if (row < p.M && T < p.T_total) {
+                const size_t o = (size_t)row * p.N + 32 * T + nn;
+                if (p.split_k == 1) {
+                    if (bias) {
+                        const h4 b4 = *(const h4 *)(bias + 32 * T + nn);
+#pragma unroll
+                        for (int c = 0; c < 4; c++) sum[c] += (float)b4[c];
+                    }
+                    h4 ov;
+#pragma unroll
+                    for (int c = 0; c < 4; c++) ov[c] = (_Float16)sum[c];
+                    *(h4 *)(y + o) = ov;
+                } else {
+                    *(f4 *)(p.partial + (size_t)split * p.M * p.N + o) = sum;
                 }
-                h4 ov;
-#pragma unroll
-                for (int c = 0; c < 4; c++) ov[c] = (_Float16)sum[c];
-                *(h4 *)(y + o) = ov;
-            } else {
-                *(f4 *)(p.partial + (size_t)split * p.M * p.N + o) = sum;
             }
         }
     }
@@ -1129,10 +1137,10 @@ __global__ __launch_bounds__(256) void tiled_reduce_kernel(const float *__restri
     *(h4 *)(y + (size_t)row * N + c) = o;
 }
 
-template <int BITS, int AT, int RW, int KW, int RING>
+template <int BITS, int AT, int RW, int KW, int RING, int CT>
 static int launch_tiled_one(const TiledParams &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
-    auto kern = tiled_gemm_kernel<BITS, AT, RW, KW, RING>;
+    auto kern = tiled_gemm_kernel<BITS, AT, RW, KW, RING, CT>;
     const int lds_bytes = tiled_lds_bytes(AT * RW, KW);
     if (plan.lds_bytes < lds_bytes || plan.waves_k != KW || plan.block != 64 * RW * KW) return GPTQ_HIP_ERR_BAD_ARG;
     if (lds_bytes > 65536) {
@@ -1182,8 +1190,8 @@ int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int
     if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ERR_LAUNCH;
     int rc = GPTQ_HIP_ERR_UNSUPPORTED;
 #define GPTQ_TILED_CASE(B, A)                                                                  \
-    if (bits == B && plan.row_tiles == A)                                                      \
-        rc = launch_tiled_one<B, A, 1, 4, tiled_ring(A)>(p, plan, stream)
+    if (bits == B && plan.row_tiles == A && plan.waves_n == 1)                                 \
+        rc = launch_tiled_one<B, A, 1, 4, tiled_ring(A), 2>(p, plan, stream)
     GPTQ_TILED_CASE(4, 1);
     GPTQ_TILED_CASE(4, 2);
     GPTQ_TILED_CASE(4, 4);
@@ -1191,6 +1199,9 @@ int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int
     GPTQ_TILED_CASE(3, 2);
     GPTQ_TILED_CASE(3, 4);
 #undef GPTQ_TILED_CASE
+    // 128 x 128 per wave (waves_n = 2): a ring of two blocks
+    if (plan.row_tiles == 4 && plan.waves_n == 2)
+        rc = bits == 4 ? launch_tiled_one<4, 4, 1, 4, 2, 4>(p, plan, stream) : launch_tiled_one<3, 4, 1, 4, 2, 4>(p, plan, stream);
     if (rc != GPTQ_HIP_OK) return rc;
     if (plan.split_k > 1) {
         const uint32_t quads = (uint32_t)M * ((uint32_t)N / 4u);

@@ -40,7 +40,7 @@ class QuantLinear(nn.Module):
     SUPPORTED_BITS = (2, 3, 4, 8)   # the widths of the format (qlinear.py:31-32)
     FUSED_BITS = (3, 4)             # those the fused kernels cover; 2 and 8 run as dequant + library GEMM
 
-    def __init__(self, bits, groupsize, infeatures, outfeatures, bias, kernel_switch_threshold=1024,
+    def __init__(self, bits, groupsize, infeatures, outfeatures, bias, kernel_switch_threshold=1152,
                  sort_for_decode=True, tile_for_prefill=True):
         super().__init__()
         if bits not in self.SUPPORTED_BITS:
@@ -54,11 +54,16 @@ class QuantLinear(nn.Module):
         self.maxq = 2 ** self.bits - 1
         # Rows of x from which forward() materialises W (HIP dequant kernel) and calls the library
         # GEMM instead of the fused kernels, as the reference does (qlinear.py:25,198: default 128
-        # there).  Measured on MI355X at 4096x11008, fused against dequant + library GEMM: contiguous
-        # groups 124 vs 139 us at 768 rows, 152 vs 146 at 1024 (int4; int3 136 vs 146); activation
-        # order 126 vs 130 at 640 rows, 139 vs 133 at 768, 169 vs 142 at 1024.  Hence 1024, and 640 for
-        # layers with an activation order.  0 or None disables the switch.
+        # there).  Measured on MI355X, fused against dequant + library GEMM, weights cold:
+        #   * tiled kernels (act-order or not), 4096x11008 int4 / int3: 117 / 117 vs 148 / 135 us at 768 rows,
+        #     125 / 118 vs 141 / 140 at 1024, 165 / 152 vs 152 / 148 at 1280; 4096x4096: 54 vs 67 at 1024, 86 vs
+        #     73 at 1280; 8192x8192: 172 vs 193 at 1024, 226 vs 219 at 1280.  Hence 1152 (nine row blocks);
+        #   * kernels on the checkpoint layout (layers off the tiled route): contiguous groups 124 vs 139 us
+        #     at 768 rows, 152 vs 146 at 1024; activation order 126 vs 130 at 640 rows, 139 vs 133 at 768.
+        #     Hence 1024 and 640 there.
+        # 0 or None disables the switch.
         self.kernel_switch_threshold = kernel_switch_threshold
+        self.plain_switch_threshold = 1024
         self.act_order_switch_threshold = 640
 
         groups = math.ceil(infeatures / self.groupsize)
@@ -267,8 +272,11 @@ class QuantLinear(nn.Module):
         if self.tile_for_prefill and ops.tiled_wins(M, K, N, g is not None, bits):
             tiled = self.prepare_tiled()
         threshold = self.kernel_switch_threshold
-        if threshold and self.act_order_switch_threshold and g is not None and tiled is None:
-            threshold = min(threshold, self.act_order_switch_threshold)   # (the tiled kernels do not pay for the order)
+        if threshold and tiled is None:   # off the tiled route the library wins earlier
+            if self.plain_switch_threshold:
+                threshold = min(threshold, self.plain_switch_threshold)
+            if self.act_order_switch_threshold and g is not None:
+                threshold = min(threshold, self.act_order_switch_threshold)
         if threshold and M >= threshold:
             return "library", library
         if tiled is not None:
