@@ -278,6 +278,9 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
         activation order, one / two rows: int4 7.9 / 8.9 against 8.2 / 11.0, int3 8.0 / 8.9 against 7.7 / 10.3;
         without: int4 7.9 / 8.5 against 7.9 / 9.0, int3 8.0 / 8.3 against 7.3 / 8.2; three and four rows are
         behind by 0.5-2 us; 5120 x 5120 int4 6.3 against 13.4-15.2; 8192 x 8192 int3 13.2-13.9 against 11.2;
+        and very wide layers (from 16384 columns, K up to 12288), where many tiles per CU even the load out:
+        4096 x 22016 int3 / int4 10.1 / 10.6 against 11.6 / 12.8, 8192 x 28672 int4 24.2 against 27.5,
+        9216 x 36864 int3 / int4 29.1 / 31.8 against 32.9 / 34.6 (36864 x 9216: 79 against 36, hence the bound on K);
       * 5 to 16 rows: never (4096 x 11008, 8 rows: 14.6 against 13.4);
       * 17 to 128 rows: everywhere within 4 % or better (4096 x 11008 with an activation order, 32/64/128
         rows: 14.8/19.2/26.6 against 18.1/22.1/34.1);
@@ -285,6 +288,8 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
         where every workgroup pulls 2.8 MB of x fragments and they no longer stay in one L2)."""
     if M <= 4:
         if N <= 4096:
+            return True
+        if M <= 2 and N >= 16384 and K <= 12288:
             return True
         if K > 6144:
             return False

@@ -66,6 +66,8 @@ WORKLOADS = {
     "c4-int4-4096x11008-act-m64": (4, 4096, 11008, 128, True, 64),
     "c4-int4-4096x11008-act-m128": (4, 4096, 11008, 128, True, 128),
     "c4-int4-4096x11008-act-m256": (4, 4096, 11008, 128, True, 256),
+    "c4-int4-4096x11008-act-m1024": (4, 4096, 11008, 128, True, 1024),
+    "c4-int3-4096x11008-act-m1024": (3, 4096, 11008, 128, True, 1024),
     "c4-int3-4096x11008-act-m128": (3, 4096, 11008, 128, True, 128),
     "int4-4096x11008-m128": (4, 4096, 11008, 128, False, 128),
     "int4-4096x11008-m256": (4, 4096, 11008, 128, False, 256),
