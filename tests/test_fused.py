@@ -147,3 +147,26 @@ def test_fused_model_matches_the_unfused_one(tmp_path):
     assert np.isfinite(b.numpy()).all()
     assert float((a - b).abs().max()) <= 1e-2 + 1e-2 * float(a.abs().max())
     assert float((a1 - b1).abs().max()) <= 1e-2 + 1e-2 * float(a1.abs().max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fuse", [False, True])
+def test_compact_model_matches_the_plain_one(tmp_path, fuse):
+    """from_quantized(compact=True): every layer keeps the tiled copy as its only weights (checkpoint tensors
+    released, fused projections included) and the model gives the same logits for a prompt and for one token."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from autogptq.tvm_amd.loader import from_quantized
+
+    cfg, _, _ = build_checkpoint(str(tmp_path), bits=4, gs=32, act_order=True, seed=6, shared_order=True)
+    plain, _ = from_quantized(str(tmp_path), device="cuda:0")
+    compact, _ = from_quantized(str(tmp_path), device="cuda:0", fuse_shared_inputs=fuse, compact=True)
+    quant = [m for m in compact.modules() if isinstance(m, QuantLinear)]
+    assert quant and all(m._compact and m.qweight.numel() == 0 and m.route(1) == "tiled" for m in quant)
+    ids = torch.randint(0, cfg.vocab_size, (2, 9), generator=torch.Generator().manual_seed(7)).to("cuda:0")
+    for part in (ids, ids[:, :1]):
+        with torch.no_grad():
+            a = plain(part).logits.float().cpu()
+            b = compact(part).logits.float().cpu()
+        assert np.isfinite(b.numpy()).all()
+        assert float((a - b).abs().max()) <= 1e-2 + 1e-2 * float(a.abs().max())
