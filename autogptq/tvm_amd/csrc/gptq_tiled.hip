@@ -601,9 +601,15 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
             for (int m = 0; m < MR; m++) xl[m * span + i] = (_Float16)0;
     }
     auto scatter8 = [&](int k, const u4 &kv, const h8 (&xv)[MR]) {
+        if (!p.kinv) {   // no activation order: the eight channels are eight consecutive positions, one store
+            // (k8_lo .. k8_hi is the workgroup's own range here, a multiple of 8 away from p0)
+#pragma unroll
+            for (int m = 0; m < MR; m++) *(h8 *)(xl + m * span + (k - p0)) = xv[m];
+            return;
+        }
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const int pos = p.kinv ? (int)((kv[e >> 1] >> (16 * (e & 1))) & 0xffffu) : k + e;
+            const int pos = (int)((kv[e >> 1] >> (16 * (e & 1))) & 0xffffu);
             const int pl = pos - p0;
             if ((unsigned)pl < (unsigned)span) {
 #pragma unroll
@@ -929,9 +935,14 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
 #pragma unroll
         for (int m = 0; m < MR; m++) xl[m * span + i] = (_Float16)0;
     auto scatter8 = [&](int k, const u4 &kv, const h8 (&xv)[MR]) {
+        if (!p.kinv) {   // no activation order: the eight channels are eight consecutive positions, one store
+#pragma unroll
+            for (int m = 0; m < MR; m++) *(h8 *)(xl + m * span + k) = xv[m];
+            return;
+        }
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const int pos = p.kinv ? min((int)((kv[e >> 1] >> (16 * (e & 1))) & 0xffffu), span - 1) : k + e;
+            const int pos = min((int)((kv[e >> 1] >> (16 * (e & 1))) & 0xffffu), span - 1);
 #pragma unroll
             for (int m = 0; m < MR; m++) xl[m * span + pos] = xv[m][e];
         }
