@@ -170,7 +170,7 @@ Tensor gemm_tiled(const Tensor &x, const Tensor &qtile, const Tensor &sz, const 
         need(*kinv, "kinv", at::kShort, x);
     }
     if (has(bias)) need(*bias, "bias", at::kHalf, x);
-    TORCH_CHECK(bits == 3 || bits == 4, "Only 3, 4 bits are supported here.");
+    TORCH_CHECK(bits == 2 || bits == 3 || bits == 4 || bits == 8, "Only 2, 3, 4, 8 bits are supported.");
     TORCH_CHECK(x.dim() == 2 && sz.dim() == 2, "x must be [M, K] and sz [G, N]");
     const int64_t M = x.size(0), K = x.size(1), N = sz.size(1);
     TORCH_CHECK(M < (1LL << 31) && K <= 65536 && N < (1LL << 31), "layer too large");

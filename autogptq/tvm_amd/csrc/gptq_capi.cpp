@@ -8,7 +8,7 @@ namespace {
 
 bool aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
 
-// wide: also the widths only the dequant kernel covers (2 and 8 bits)
+// wide: also 2 and 8 bits (the dequant kernel and the tiled format cover them, the kernels on the checkpoint layout do not)
 int check_common(const int32_t *qweight, const int32_t *qzeros, const void *scales, int K, int N, int bits,
                  int group_size, bool wide = false)
 {
@@ -306,7 +306,7 @@ extern "C" size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits,
 
 extern "C" size_t gptq_hip_tiled_bytes(int K, int N, int bits)
 {
-    if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0 || (bits != 3 && bits != 4)) return 0;
+    if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0 || (bits != 2 && bits != 3 && bits != 4 && bits != 8)) return 0;
     return (size_t)((K + 63) / 64 * 64) * (size_t)N * bits / 8;
 }
 
@@ -315,7 +315,7 @@ extern "C" int gptq_hip_tile_prepare(const int32_t *qweight, const int32_t *qzer
                                      int K, int N, int bits, int group_size, void *stream)
 {
     if (!qtile || !sz || !xsrc || !kinv || (const void *)qweight == qtile) return GPTQ_HIP_ERR_BAD_ARG;
-    const int rc = check_common(qweight, qzeros, scales, K, N, bits, group_size);
+    const int rc = check_common(qweight, qzeros, scales, K, N, bits, group_size, true);
     if (rc != GPTQ_HIP_OK) return rc;
     if (!aligned(qtile, 16) || !aligned(sz, 4) || !aligned(xsrc, 16) || !aligned(kinv, 16) || (g_idx && !aligned(g_idx, 4)))
         return GPTQ_HIP_ERR_BAD_ARG;
@@ -332,7 +332,7 @@ extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint3
 {
     if ((xsrc == nullptr) != (kinv == nullptr) || (kinv && !aligned(kinv, 16))) return GPTQ_HIP_ERR_BAD_ARG;
     if (!x || !qtile || !sz || !y || M < 1) return GPTQ_HIP_ERR_BAD_ARG;
-    if (bits != 3 && bits != 4) return GPTQ_HIP_ERR_BAD_ARG;
+    if (bits != 2 && bits != 3 && bits != 4 && bits != 8) return GPTQ_HIP_ERR_BAD_ARG;
     if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;
     if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
     if (!aligned(x, 16) || !aligned(qtile, 16) || !aligned(sz, 4) || !aligned(y, 8) || (bias && !aligned(bias, 8)) ||

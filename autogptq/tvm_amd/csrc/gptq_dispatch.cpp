@@ -476,7 +476,7 @@ static int tiled_args_ok(int M, int K, int N, int bits, int group_size, gptq_hip
 {
     if (!plan) return GPTQ_HIP_ERR_BAD_ARG;
     memset(plan, 0, sizeof(*plan));
-    if (bits != 3 && bits != 4) return GPTQ_HIP_ERR_BAD_ARG;
+    if (bits != 2 && bits != 3 && bits != 4 && bits != 8) return GPTQ_HIP_ERR_BAD_ARG;
     if (M < 1 || K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;
     if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
     if (!gptq::tiled_qualifies(K, N, bits, group_size == -1 ? K : group_size)) return GPTQ_HIP_ERR_UNSUPPORTED;

@@ -181,7 +181,8 @@ inline int tiled_lds_bytes(int row_tiles, int waves_k) { return waves_k * row_ti
 inline bool tiled_qualifies(int K, int N, int bits, int gs)
 {
     // (the pack pass stages one row of x in LDS: K * 2 bytes)
-    return (bits == 3 || bits == 4) && K % 32 == 0 && N % 32 == 0 && gs % 32 == 0 && K % gs == 0 && K <= 65536;
+    return (bits == 2 || bits == 3 || bits == 4 || bits == 8) && K % 32 == 0 && N % 32 == 0 && gs % 32 == 0 &&
+           K % gs == 0 && K <= 65536;
 }
 // decode kernel on the tiled format: rows it is built for, and the LDS of a workgroup whose waves cover
 // `span` positions of `groups` groups

@@ -5,11 +5,12 @@
 //   * the input channels are sorted by group (stable; the identity without an activation order), so
 //     position p of the sorted order holds channel xsrc[p] and its group is p / group_size;
 //   * qtile is a sequence of blocks, column tile T (32 columns) outermost, then block S (64 positions);
-//     block (T, S) is 64 lanes x BITS words, exactly one coalesced wave load.  Lane (n = lane % 32,
-//     h = lane / 32) holds the 32 codes of column 32 T + n at positions 64 S + 32 h .. + 31, permuted
-//     inside the lane so that the register unpack of gptq_unpack.h yields them in position order:
-//     the lane's words are the B operand of four v_mfma_f32_32x32x16_f16 (positions 8 j .. 8 j + 7 of
-//     the lane for j = 0..3) with no shuffle;
+//     block (T, S) is 64 lanes x BITS words, one coalesced wave load (two for 8 bits, whose block is laid
+//     out as two halves of 64 lanes x 4 words).  Lane (n = lane % 32, h = lane / 32) holds the 32 codes of
+//     column 32 T + n at positions 64 S + 32 h .. + 31, permuted inside the lane so that the register
+//     unpack of gptq_unpack.h (TileCodec) yields them in position order: the lane's words are the B
+//     operand of four v_mfma_f32_32x32x16_f16 (positions 8 j .. 8 j + 7 of the lane for j = 0..3) with
+//     no shuffle;
 //   * sz[g][n] = (fp16 scale, fp16 zero point) of group g, column n, one 32-bit word.
 //
 // tiled_gemm_kernel: a workgroup owns 64 columns (two tiles), 32 * AT rows of x and one K range; its four
@@ -43,6 +44,49 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 struct alignas(4) W3 {
     uint32_t a, b, c;
 };
+
+// Byte offset of lane l's words inside a block, and the lane's load.  Word i of a lane sits at
+// l * BITS + i, except for 8 bits: (i / 4) * 256 + l * 4 + i % 4, so that each of the two loads is coalesced.
+template <int BITS>
+__device__ __forceinline__ constexpr uint32_t tile_lane_bytes(uint32_t l)
+{
+    return BITS == 8 ? l * 16u : l * (4u * BITS);
+}
+
+template <int BITS>
+__device__ __forceinline__ void tile_load(const char *src, uint32_t (&wr)[BITS])
+{
+    if constexpr (BITS == 4) {
+        const u4 v = __builtin_nontemporal_load((const u4 *)src);
+#pragma unroll
+        for (int e = 0; e < 4; e++) wr[e] = v[e];
+    } else if constexpr (BITS == 8) {
+        const u4 v0 = __builtin_nontemporal_load((const u4 *)src);
+        const u4 v1 = __builtin_nontemporal_load((const u4 *)(src + 1024));
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            wr[e] = v0[e];
+            wr[4 + e] = v1[e];
+        }
+    } else if constexpr (BITS == 2) {
+        const u2 v = __builtin_nontemporal_load((const u2 *)src);
+        wr[0] = v[0];
+        wr[1] = v[1];
+    } else {
+        const W3 v = *(const W3 *)src;
+        wr[0] = v.a;
+        wr[1] = v.b;
+        wr[2] = v.c;
+    }
+}
+
+// The magic constants of the width's unpack, each held in a vector register.
+template <int BITS>
+__device__ __forceinline__ void tile_magic(uint32_t (&mg)[TileCodec<BITS>::KINDS])
+{
+#pragma unroll
+    for (int k = 0; k < TileCodec<BITS>::KINDS; k++) mg[k] = opaque_vgpr(TileCodec<BITS>::MAGIC[k]);
+}
 
 // ---------------------------------------------------------------------------------------------------
 // Preparation, pass 1: xsrc[p] = the channel at position p of the stable sort by group (the rank of a
@@ -106,14 +150,17 @@ __global__ __launch_bounds__(256) void tile_retile_kernel(const uint32_t *__rest
             q &= (1u << BITS) - 1u;
         }
         // the stream field that the register unpack hands out as position s
-        const int field = BITS == 4 ? (s & ~7) + SLOT4[s & 7] : SLOT3[s];
+        const int field = TileCodec<BITS>::field(s);
         const int obit = BITS * field;
         const int owd = obit >> 5, osh = obit & 31;
         words[owd] |= q << osh;
         if (osh + BITS > 32) words[owd + 1] |= q >> (32 - osh);
     }
 #pragma unroll
-    for (int i = 0; i < BITS; i++) qtile[((size_t)blk * 64 + lane) * BITS + i] = words[i];
+    for (int i = 0; i < BITS; i++) {
+        const int at = BITS == 8 ? (i >> 2) * 256 + lane * 4 + (i & 3) : lane * BITS + i;
+        qtile[(size_t)blk * (64 * BITS) + at] = words[i];
+    }
 }
 
 // Pass 3: sz[g][n] = fp16 scale | fp16 zero point << 16.
@@ -141,16 +188,19 @@ int launch_tile_prepare(const uint32_t *qweight, const uint32_t *qzeros, const v
                        group_size);
     const unsigned threads = (unsigned)T_total * (unsigned)S_total * 64u;
     const unsigned szt = (unsigned)G * (unsigned)N;
-    if (bits == 4) {
-        hipLaunchKernelGGL(tile_retile_kernel<4>, dim3((threads + 255u) / 256u), dim3(256), 0, stream, qweight, xsrc, qtile,
+    auto go = [&](auto bits_c) {
+        constexpr int B = decltype(bits_c)::value;
+        hipLaunchKernelGGL(tile_retile_kernel<B>, dim3((threads + 255u) / 256u), dim3(256), 0, stream, qweight, xsrc, qtile,
                            K, N, S_total, T_total);
-        hipLaunchKernelGGL(tile_sz_kernel<4>, dim3((szt + 255u) / 256u), dim3(256), 0, stream, qzeros,
+        hipLaunchKernelGGL(tile_sz_kernel<B>, dim3((szt + 255u) / 256u), dim3(256), 0, stream, qzeros,
                            (const _Float16 *)scales, sz, N, G);
-    } else {
-        hipLaunchKernelGGL(tile_retile_kernel<3>, dim3((threads + 255u) / 256u), dim3(256), 0, stream, qweight, xsrc, qtile,
-                           K, N, S_total, T_total);
-        hipLaunchKernelGGL(tile_sz_kernel<3>, dim3((szt + 255u) / 256u), dim3(256), 0, stream, qzeros,
-                           (const _Float16 *)scales, sz, N, G);
+    };
+    switch (bits) {
+        case 2: go(std::integral_constant<int, 2>{}); break;
+        case 3: go(std::integral_constant<int, 3>{}); break;
+        case 4: go(std::integral_constant<int, 4>{}); break;
+        case 8: go(std::integral_constant<int, 8>{}); break;
+        default: return GPTQ_HIP_ERR_BAD_ARG;
     }
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
@@ -232,20 +282,14 @@ struct TiledParams {
 // One B operand: positions 8 j .. 8 j + 7 of the lane, as fp16(scale * (q - zero)) exactly as the
 // reference rounds it: (base + q) - (base + zero) is exact, the product rounds once.
 template <int BITS>
-__device__ __forceinline__ h8 tiled_bop(const uint32_t (&w)[BITS], int j, h2 s2, h2 zb_a, h2 zb_b, uint32_t magic_a,
-                                        uint32_t magic_b)
+__device__ __forceinline__ h8 tiled_bop(const uint32_t (&w)[BITS], int j, h2 s2, const h2 (&zb)[TileCodec<BITS>::KINDS],
+                                        const uint32_t (&mg)[TileCodec<BITS>::KINDS])
 {
     u4 q;
-    if constexpr (BITS == 4) {
-        u4 tmp[1];
-        biased4(w[j], tmp, magic_a, magic_b);
-        q = tmp[0];
-    } else {
-        biased3_block(w[0], w[1], w[2], j, q, magic_a, magic_b);
-    }
+    TileCodec<BITS>::operand(w, j, q, mg);
     u4 o;
 #pragma unroll
-    for (int r = 0; r < 4; r++) o[r] = as_u32((as_h2(q[r]) - ((r & 1) ? zb_b : zb_a)) * s2);
+    for (int r = 0; r < 4; r++) o[r] = as_u32((as_h2(q[r]) - zb[r % TileCodec<BITS>::KINDS]) * s2);
     return __builtin_bit_cast(h8, o);
 }
 
@@ -277,7 +321,7 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
         tile_off[ct] = (uint32_t)T * (uint32_t)p.S_total;
         col[ct] = (uint32_t)(32 * T + n);
     }
-    const uint32_t b_lane = (uint32_t)lane * (4u * BITS);
+    const uint32_t b_lane = tile_lane_bytes<BITS>((uint32_t)lane);
     const uint32_t a_lane = (uint32_t)rt0 * 1024u + (uint32_t)lane * 16u;
     const uint32_t a_frag_row = (uint32_t)p.rt_total * 1024u;  // bytes between consecutive (S, j)
 
@@ -290,17 +334,7 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
         const uint32_t g = min(lb / (uint32_t)p.lb_per_group, (uint32_t)p.G - 1u);
 #pragma unroll
         for (int ct = 0; ct < CT; ct++) {
-            const char *src = p.qtile + ((size_t)(tile_off[ct] + (uint32_t)Sc) * (256u * BITS) + b_lane);
-            if constexpr (BITS == 4) {
-                const u4 v = __builtin_nontemporal_load((const u4 *)src);
-#pragma unroll
-                for (int e = 0; e < 4; e++) wr[ct][e] = v[e];
-            } else {
-                const W3 v = *(const W3 *)src;
-                wr[ct][0] = v.a;
-                wr[ct][1] = v.b;
-                wr[ct][2] = v.c;
-            }
+            tile_load<BITS>(p.qtile + ((size_t)(tile_off[ct] + (uint32_t)Sc) * (256u * BITS) + b_lane), wr[ct]);
             sr[ct] = p.sz[(size_t)g * p.N + col[ct]];
         }
     };
@@ -337,23 +371,24 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[rt][ct][v] = 0.f;
 
-    const uint32_t magic_a = opaque_vgpr(BITS == 4 ? MAGIC4_LO : MAGIC3_EVEN);
-    const uint32_t magic_b = opaque_vgpr(BITS == 4 ? MAGIC4_HI : MAGIC3_ODD);
-    // (base + zero) per register kind: even registers of an operand carry bases (BASE[0], BASE[1]), odd (BASE[2], BASE[3])
-    const h2 base_a = BITS == 4 ? (h2){(_Float16)1024.f, (_Float16)1024.f} : (h2){(_Float16)1024.f, (_Float16)256.f};
-    const h2 base_b = BITS == 4 ? (h2){(_Float16)64.f, (_Float16)64.f} : (h2){(_Float16)128.f, (_Float16)32.f};
-    auto consts_of = [&](uint32_t e, h2 &s2, h2 &za, h2 &zb) {
+    using Codec = TileCodec<BITS>;
+    constexpr int KINDS = Codec::KINDS;
+    uint32_t mg[KINDS];
+    tile_magic<BITS>(mg);
+    // (base + zero) per register kind: register r of an operand carries the bases of positions 2 r, 2 r + 1
+    auto consts_of = [&](uint32_t e, h2 &s2, h2 (&zb)[KINDS]) {
         const h2 v = as_h2(e);
         s2 = (h2){v[0], v[0]};
         const h2 z2 = {v[1], v[1]};
-        za = z2 + base_a;  // exact: small integers
-        zb = z2 + base_b;
+#pragma unroll
+        for (int k = 0; k < KINDS; k++)
+            zb[k] = z2 + (h2){(_Float16)Codec::base(2 * k), (_Float16)Codec::base(2 * k + 1)};  // exact: small integers
     };
 
     // the first operand of the walk
-    h2 cs[CT], cza[CT], czb[CT];  // (scale, base + zero) of the block being dequantised, per column tile
-    consts_of(szr[0][0], cs[0], cza[0], czb[0]);
-    h8 bop_next = tiled_bop<BITS>(w[0][0], 0, cs[0], cza[0], czb[0], magic_a, magic_b);
+    h2 cs[CT], czb[CT][KINDS];  // (scale, base + zero) of the block being dequantised, per column tile
+    consts_of(szr[0][0], cs[0], czb[0]);
+    h8 bop_next = tiled_bop<BITS>(w[0][0], 0, cs[0], czb[0], mg);
 
     // One block of the walk (ring slot u): the 4 CT (j, ct) operands, each multiplied with the AT row tiles
     // while the next operand of the walk is dequantised.  REFILL: the slot's registers are requested again
@@ -372,9 +407,9 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
                     const int ctn = ct == CT - 1 ? 0 : ct + 1;
                     constexpr int u1 = (u + 1) % RING;
                     const bool wrap_u = ct == CT - 1 && j == 3;
-                    if (jn == 0) consts_of(wrap_u ? szr[u1][ctn] : szr[u][ctn], cs[ctn], cza[ctn], czb[ctn]);  // first operand of a block
-                    bop_next = wrap_u ? tiled_bop<BITS>(w[u1][ctn], jn, cs[ctn], cza[ctn], czb[ctn], magic_a, magic_b)
-                                      : tiled_bop<BITS>(w[u][ctn], jn, cs[ctn], cza[ctn], czb[ctn], magic_a, magic_b);
+                    if (jn == 0) consts_of(wrap_u ? szr[u1][ctn] : szr[u][ctn], cs[ctn], czb[ctn]);  // first operand of a block
+                    bop_next = wrap_u ? tiled_bop<BITS>(w[u1][ctn], jn, cs[ctn], czb[ctn], mg)
+                                      : tiled_bop<BITS>(w[u][ctn], jn, cs[ctn], czb[ctn], mg);
                 }
 #pragma unroll
                 for (int rt = 0; rt < AT; rt++) {
@@ -474,11 +509,13 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
 // they are (four positions each), the A operand of lane 4 b + i is x[row i] at the same four positions
 // (read from LDS: rows past M read zeros), and the four result registers of a lane are the rows of its
 // own column: up to four rows of x cost one matrix instruction per four positions.
-// Per weight the vector ALU only unpacks.
+// Per weight the vector ALU only unpacks (2, 3, 4 bits).
 // The codes enter as (base + q) with the bases of the register unpack; per block of 32 positions the
 // epilogue takes y += scale * (P - Bsum - zero * Xsum), with Xsum = sum x and Bsum = sum x * base of the
 // block computed once per workgroup when x is staged.  Like GROUPED, and unlike the TILED matmul, this
 // does not reproduce the fp16 rounding of each dequantised weight: products are exact, sums are fp32.
+// 8-bit layers instead dequantise every weight in registers, as the matmul does (tiled_decode_exact), and add
+// the products as they are.
 // x reaches LDS in position order: a layer with an activation order scatters it through kinv (16-bit
 // position per channel, one round trip; every workgroup walks all of x and keeps its K range).
 // ---------------------------------------------------------------------------------------------------
@@ -501,6 +538,29 @@ struct DecodeParams {
 
 typedef float f2 __attribute__((ext_vector_type(2)));
 
+// 8-bit layers: the decode kernels dequantise every weight as the reference rounds it (fp16(scale * (q - zero)),
+// the matmul kernel's arithmetic).  Their weights are sixteen times those of a 4-bit layer, and so is the
+// distance between exact products and the reference's rounded ones; the extra packed instructions hide
+// behind a stream that is twice as long per weight.
+constexpr bool tiled_decode_exact(int bits) { return bits == 8; }
+
+// the sixteen unpacked registers of a lane -> fp16(scale * (q - zero)); sz = fp16 scale | fp16 zero << 16
+template <int BITS>
+__device__ __forceinline__ void tiled_dequant_exact(u4 (&q)[4], uint32_t sz)
+{
+    using Codec = TileCodec<BITS>;
+    const h2 e = as_h2(sz);
+    const h2 s2 = {e[0], e[0]};
+    h2 zb[Codec::KINDS];
+#pragma unroll
+    for (int k = 0; k < Codec::KINDS; k++)
+        zb[k] = (h2){e[1], e[1]} + (h2){(_Float16)Codec::base(2 * k), (_Float16)Codec::base(2 * k + 1)};
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) q[j][r] = as_u32((as_h2(q[j][r]) - zb[r % Codec::KINDS]) * s2);
+}
+
 // v of lane l + N inside its row of 16 lanes (zero past the row's end)
 template <int N>
 __device__ __forceinline__ float row_shl(float v)
@@ -514,6 +574,7 @@ template <int BITS, int MR, int KW, int E>
 __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParams p)
 {
     static_assert(MR <= 4 && (E == 1 || E == 2), "one matrix instruction set per lane block");
+    constexpr bool EXACT = tiled_decode_exact(BITS);
     constexpr int NT = 64 * KW;
     constexpr int PF = 2;              // blocks of weights per chunk; two chunks are in flight
     const int tid = threadIdx.x;
@@ -565,24 +626,14 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
         szq[ps] = p.sz[(size_t)(g_first + (uint32_t)(i >> 5)) * p.N + 32 * T + (i & 31)];
     }
     __builtin_amdgcn_sched_barrier(0);
-    const uint32_t b_lane = (uint32_t)lane * (4u * BITS);
+    const uint32_t b_lane = tile_lane_bytes<BITS>((uint32_t)lane);
     const uint32_t tile_off = (uint32_t)T * (uint32_t)p.S_total;
     uint32_t w[2][PF][BITS];
     const int steps = min(p.wave_steps, max(p.S_total - S_begin, 0));  // blocks of this wave that lie inside K
     auto load_w = [&](int i, uint32_t (&wr)[BITS]) {
         // block i of the wave's range; past its end: its first block again (a cache hit that is never multiplied)
         const int Sc = min(S_begin + (i < steps ? i : 0), S_last);
-        const char *src = p.qtile + ((size_t)(tile_off + (uint32_t)Sc) * (256u * BITS) + b_lane);
-        if constexpr (BITS == 4) {
-            const u4 v = __builtin_nontemporal_load((const u4 *)src);
-#pragma unroll
-            for (int e = 0; e < 4; e++) wr[e] = v[e];
-        } else {
-            const W3 v = *(const W3 *)src;
-            wr[0] = v.a;
-            wr[1] = v.b;
-            wr[2] = v.c;
-        }
+        tile_load<BITS>(p.qtile + ((size_t)(tile_off + (uint32_t)Sc) * (256u * BITS) + b_lane), wr);
     };
     // two chunks of PF blocks are in flight from here on, through the staging of x as well
 #pragma unroll
@@ -644,7 +695,7 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     //         unit's 32 E positions of that half; every wave for the units of its own slice (LDS serves one
     //         wave's accesses in order: no barrier needed).  Entry ((sb / E) * 2 + h) * MR + m, sb = the unit's
     //         first block inside the workgroup's range ------------------------------------------------------
-    {
+    if constexpr (!EXACT) {
         // a lane sums 16 consecutive positions; a run of 32 positions (one half of one block) is two lanes,
         // a unit-half 2 E lanes: l, l + 1 (the other half of the run) and, E = 2, l + 4, l + 5 (the other block)
         const int sb0 = S_begin - S_wg;
@@ -664,7 +715,7 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
                         for (int e = 0; e < 8; e++) {
                             const float xf = (float)q[e];
                             X += xf;
-                            B += xf * (BITS == 4 ? BASE4[e] : BASE3[e]);
+                            B += xf * TileCodec<BITS>::base(e);
                         }
                     }
                 }
@@ -685,8 +736,8 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     }
 
     // ---- 4. the walk ----------------------------------------------------------------------------------
-    const uint32_t magic_a = opaque_vgpr(BITS == 4 ? MAGIC4_LO : MAGIC3_EVEN);
-    const uint32_t magic_b = opaque_vgpr(BITS == 4 ? MAGIC4_HI : MAGIC3_ODD);
+    uint32_t mg[TileCodec<BITS>::KINDS];
+    tile_magic<BITS>(mg);
     const int row_i = lane & 3;  // the row of x this lane supplies to its 4-lane block
     float ysum[MR];
 #pragma unroll
@@ -721,23 +772,18 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
                 goff = (h ? g1 : g0) * 128u;
             }
             szw = *(const uint32_t *)(smem + sz_lane + goff);
-            const f2 *xb = (const f2 *)(smem + xs_lane + (sb / E) * (uint32_t)(2 * MR * 8));
+            if constexpr (!EXACT) {
+                const f2 *xb = (const f2 *)(smem + xs_lane + (sb / E) * (uint32_t)(2 * MR * 8));
 #pragma unroll
-            for (int m = 0; m < MR; m++) xsv[m] = xb[m];
+                for (int m = 0; m < MR; m++) xsv[m] = xb[m];
+            }
         }
         load_x(sb + 1u, xn);
         // unpack: sixteen registers, positions (2 r, 2 r + 1) of the lane in register r
         u4 q[4];
-        if constexpr (BITS == 4) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                u4 t[1];
-                biased4(wr[j], t, magic_a, magic_b);
-                q[j] = t[0];
-            }
-        } else {
-            biased3(wr[0], wr[1], wr[2], q, magic_a, magic_b);
-        }
+        for (int j = 0; j < 4; j++) TileCodec<BITS>::operand(wr, j, q[j], mg);
+        if constexpr (EXACT) tiled_dequant_exact<BITS>(q, szw);
         if constexpr (uu == 0) {
             c0 = (f4){0.f, 0.f, 0.f, 0.f};
             c1 = (f4){0.f, 0.f, 0.f, 0.f};
@@ -750,10 +796,15 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
             c1 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a1), __builtin_bit_cast(h4, b1), c1, 0, 0, 0);
         }
         if constexpr (uu == E - 1) {
-            const h2 e = as_h2(szw);
-            const float sc = (float)e[0], zp = (float)e[1];
+            if constexpr (EXACT) {
 #pragma unroll
-            for (int m = 0; m < MR; m++) ysum[m] += sc * (((c0[m] + c1[m]) - xsv[m][1]) - zp * xsv[m][0]);
+                for (int m = 0; m < MR; m++) ysum[m] += c0[m] + c1[m];
+            } else {
+                const h2 e = as_h2(szw);
+                const float sc = (float)e[0], zp = (float)e[1];
+#pragma unroll
+                for (int m = 0; m < MR; m++) ysum[m] += sc * (((c0[m] + c1[m]) - xsv[m][1]) - zp * xsv[m][0]);
+            }
         }
     };
 
@@ -847,6 +898,7 @@ template <int BITS, int MR, bool G128>
 __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Params p)
 {
     static_assert(MR <= 4, "one matrix instruction set per lane block");
+    constexpr bool EXACT = tiled_decode_exact(BITS);
     constexpr int NT = 1024, NW = 16;
     constexpr int PF = 2;               // items of weights per chunk; two chunks are in flight
     const int tid = threadIdx.x;
@@ -893,7 +945,7 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     const int n_items = n_units * vpu;
     // lane offset inside a virtual block: its lane of the real block, and the second real block for q >= 2
     // (a last, odd virtual block has no second real block: those lanes repeat the first; their x is zero)
-    const uint32_t b_lane = (uint32_t)(n16 + 32 * (lbv & 1)) * (4u * BITS);
+    const uint32_t b_lane = tile_lane_bytes<BITS>((uint32_t)(n16 + 32 * (lbv & 1)));
     const uint32_t b_lane2 = b_lane + (uint32_t)(lbv >> 1) * (256u * BITS);
     // cursors: (unit, V) of the next item to request and of the next item to compute
     int rq_u = 0, rq_v = wave;
@@ -905,18 +957,8 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
         const int V = valid ? rq_v : min(wave, p.V_total - 1);
         const int T = unit >> 1, c = unit & 1;
         const char *base = p.qtile + ((size_t)((uint32_t)T * (uint32_t)p.S_total + 2u * (uint32_t)V) * (256u * BITS) +
-                                      (uint32_t)c * (64u * BITS));   // wave-uniform
-        const char *src = base + (2 * V + 1 <= S_last ? b_lane2 : b_lane);
-        if constexpr (BITS == 4) {
-            const u4 v = __builtin_nontemporal_load((const u4 *)src);
-#pragma unroll
-            for (int e = 0; e < 4; e++) wr[e] = v[e];
-        } else {
-            const W3 v = *(const W3 *)src;
-            wr[0] = v.a;
-            wr[1] = v.b;
-            wr[2] = v.c;
-        }
+                                      tile_lane_bytes<BITS>(16u * (uint32_t)c));   // wave-uniform
+        tile_load<BITS>(base + (2 * V + 1 <= S_last ? b_lane2 : b_lane), wr);
         rq_v += NW;
         if (rq_v >= p.V_total) {
             rq_v = wave;
@@ -972,7 +1014,7 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     lds_barrier();
     // ---- 3. per 32 positions and row: Xsum = sum x, Bsum = sum x * base(position).  A thread sums 16
     //         positions, the lane next to it the other half of the run -------------------------------------
-    for (int q0 = 0; q0 < span / 16; q0 += NT) {
+    for (int q0 = 0; !EXACT && q0 < span / 16; q0 += NT) {
         const int piece = q0 + tid;
         const bool live = piece < span / 16;
 #pragma unroll
@@ -987,7 +1029,7 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
                     for (int e = 0; e < 8; e++) {
                         const float xf = (float)q[e];
                         X += xf;
-                        B += xf * (BITS == 4 ? BASE4[e] : BASE3[e]);
+                        B += xf * TileCodec<BITS>::base(e);
                     }
                 }
             }
@@ -999,8 +1041,8 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     lds_barrier();
 
     // ---- 4. the walk ----------------------------------------------------------------------------------
-    const uint32_t magic_a = opaque_vgpr(BITS == 4 ? MAGIC4_LO : MAGIC3_EVEN);
-    const uint32_t magic_b = opaque_vgpr(BITS == 4 ? MAGIC4_HI : MAGIC3_ODD);
+    uint32_t mg[TileCodec<BITS>::KINDS];
+    tile_magic<BITS>(mg);
     const int row_i = lane & 3;  // the row of x this lane supplies to its 4-lane block
     float ysum[MR];
 #pragma unroll
@@ -1030,10 +1072,12 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
             goff = min(__umulhi(lb, p.lbg_magic) + (p.lbg_add ? lb : 0u), (uint32_t)p.G - 1u) * 128u;
         }
         const f2 szf = *(const f2 *)(smem + sz_lane + (uint32_t)ul * (uint32_t)p.G * 128u + goff);
-        const f2 *xb = (const f2 *)(smem + xs_lane + (uint32_t)V * (uint32_t)(4 * MR * 8));
         f2 xsv[MR];
+        if constexpr (!EXACT) {
+            const f2 *xb = (const f2 *)(smem + xs_lane + (uint32_t)V * (uint32_t)(4 * MR * 8));
 #pragma unroll
-        for (int m = 0; m < MR; m++) xsv[m] = xb[m];
+            for (int m = 0; m < MR; m++) xsv[m] = xb[m];
+        }
         // advance to the next item and read its x
         cv += NW;
         const bool unit_done = cv >= p.V_total;
@@ -1043,15 +1087,11 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
         }
         load_x(cv, xn);
         u4 q[4];
-        if constexpr (BITS == 4) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                u4 t[1];
-                biased4(wr[j], t, magic_a, magic_b);
-                q[j] = t[0];
-            }
-        } else {
-            biased3(wr[0], wr[1], wr[2], q, magic_a, magic_b);
+        for (int j = 0; j < 4; j++) TileCodec<BITS>::operand(wr, j, q[j], mg);
+        if constexpr (EXACT) {   // (both floats came from fp16 values: the conversions back are exact)
+            const h2 e = {(_Float16)szf[0], (_Float16)szf[1]};
+            tiled_dequant_exact<BITS>(q, as_u32(e));
         }
         f4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};  // two chains
 #pragma unroll
@@ -1061,9 +1101,14 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
             c0 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a0), __builtin_bit_cast(h4, b0), c0, 0, 0, 0);
             c1 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a1), __builtin_bit_cast(h4, b1), c1, 0, 0, 0);
         }
-        const float sc = szf[0], zp = szf[1];
+        if constexpr (EXACT) {
 #pragma unroll
-        for (int m = 0; m < MR; m++) ysum[m] += sc * (((c0[m] + c1[m]) - xsv[m][1]) - zp * xsv[m][0]);
+            for (int m = 0; m < MR; m++) ysum[m] += c0[m] + c1[m];
+        } else {
+            const float sc = szf[0], zp = szf[1];
+#pragma unroll
+            for (int m = 0; m < MR; m++) ysum[m] += sc * (((c0[m] + c1[m]) - xsv[m][1]) - zp * xsv[m][0]);
+        }
         if (unit_done) {   // (wave-uniform) the wave's share of this unit is complete
 #pragma unroll
             for (int m = 0; m < MR; m++) {
@@ -1209,10 +1254,23 @@ int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int
     GPTQ_TILED_CASE(3, 1);
     GPTQ_TILED_CASE(3, 2);
     GPTQ_TILED_CASE(3, 4);
+    GPTQ_TILED_CASE(2, 1);
+    GPTQ_TILED_CASE(2, 2);
+    GPTQ_TILED_CASE(2, 4);
+    GPTQ_TILED_CASE(8, 1);
+    GPTQ_TILED_CASE(8, 2);
+    GPTQ_TILED_CASE(8, 4);
 #undef GPTQ_TILED_CASE
     // 128 x 128 per wave (waves_n = 2): a ring of two blocks
-    if (plan.row_tiles == 4 && plan.waves_n == 2)
-        rc = bits == 4 ? launch_tiled_one<4, 4, 1, 4, 2, 4>(p, plan, stream) : launch_tiled_one<3, 4, 1, 4, 2, 4>(p, plan, stream);
+    if (plan.row_tiles == 4 && plan.waves_n == 2) {
+        switch (bits) {
+            case 2: rc = launch_tiled_one<2, 4, 1, 4, 2, 4>(p, plan, stream); break;
+            case 3: rc = launch_tiled_one<3, 4, 1, 4, 2, 4>(p, plan, stream); break;
+            case 4: rc = launch_tiled_one<4, 4, 1, 4, 2, 4>(p, plan, stream); break;
+            case 8: rc = launch_tiled_one<8, 4, 1, 4, 2, 4>(p, plan, stream); break;
+            default: break;
+        }
+    }
     if (rc != GPTQ_HIP_OK) return rc;
     if (plan.split_k > 1) {
         const uint32_t quads = (uint32_t)M * ((uint32_t)N / 4u);
@@ -1287,6 +1345,12 @@ int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, co
     GPTQ_DECODE_CASE(3, 1);
     GPTQ_DECODE_CASE(3, 2);
     GPTQ_DECODE_CASE(3, 4);
+    GPTQ_DECODE_CASE(2, 1);
+    GPTQ_DECODE_CASE(2, 2);
+    GPTQ_DECODE_CASE(2, 4);
+    GPTQ_DECODE_CASE(8, 1);
+    GPTQ_DECODE_CASE(8, 2);
+    GPTQ_DECODE_CASE(8, 4);
 #undef GPTQ_DECODE_CASE
     if (rc != GPTQ_HIP_OK) return rc;
     if (plan.split_k > 1) {
@@ -1347,6 +1411,12 @@ int launch_tiled_decode16(const void *x, const void *qtile, const uint32_t *sz, 
     GPTQ_DECODE16_CASE(3, 1);
     GPTQ_DECODE16_CASE(3, 2);
     GPTQ_DECODE16_CASE(3, 4);
+    GPTQ_DECODE16_CASE(2, 1);
+    GPTQ_DECODE16_CASE(2, 2);
+    GPTQ_DECODE16_CASE(2, 4);
+    GPTQ_DECODE16_CASE(8, 1);
+    GPTQ_DECODE16_CASE(8, 2);
+    GPTQ_DECODE16_CASE(8, 4);
 #undef GPTQ_DECODE16_CASE
     return rc;
 }

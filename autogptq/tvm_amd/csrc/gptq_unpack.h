@@ -216,6 +216,85 @@ GPTQ_HD void biased3_block(uint32_t w0, uint32_t w1, uint32_t w2, int nb, u4 &ou
     out[3] = and_or(hi, 0x00e00038u, magic_odd);
 }
 
+// int8: two registers per word.  Register r of a word holds fields (r, r + 2): both halves carry their code at
+// mantissa bit 0, so every base is 1024.
+static constexpr int SLOT8[4] = {0, 2, 1, 3};
+static constexpr uint32_t MAGIC8 = 0x64006400u;
+
+// int2: eight registers per word.  The word, and the word shifted right by 8, each give four registers:
+// register r masks bits 2 r, 2 r + 1 of both halves, so its codes sit at mantissa bit 2 r and read
+// (1024 >> 2 r) + code.  Register r of the unshifted word holds fields (r, 8 + r), of the shifted word
+// (4 + r, 12 + r).
+static constexpr int SLOT2[16] = {0, 8, 1, 9, 2, 10, 3, 11, 4, 12, 5, 13, 6, 14, 7, 15};
+static constexpr uint32_t MAGIC2[4] = {0x64006400u, 0x5c005c00u, 0x54005400u, 0x4c004c00u};
+
+// ---- the tiled format, per width ------------------------------------------------------------------
+// A lane of the tiled format holds 32 codes in BITS words; operand j (j = 0..3) is the lane's positions
+// 8 j .. 8 j + 7 as four registers of (base + code) pairs, register r holding positions (8 j + 2 r, 8 j + 2 r + 1).
+//   field(s)   the stream field (of the lane's 32) that the unpack hands out as position s
+//   base(e)    the base of position e (period 8)
+//   KINDS      registers r and r + KINDS of an operand share their magic constant and their bases
+//   operand()  the unpack of operand j; mg[k] = MAGIC[k] held in a vector register
+template <int BITS>
+struct TileCodec;
+
+template <>
+struct TileCodec<4> {
+    static constexpr int KINDS = 2;
+    static constexpr uint32_t MAGIC[4] = {MAGIC4_LO, MAGIC4_HI, MAGIC4_LO, MAGIC4_HI};
+    static GPTQ_HD constexpr float base(int e) { return ((e >> 1) & 1) ? 64.f : 1024.f; }
+    static GPTQ_HD constexpr int field(int s) { return (s & ~7) + SLOT4[s & 7]; }
+    static GPTQ_HD void operand(const uint32_t (&w)[4], int j, u4 &q, const uint32_t (&mg)[KINDS])
+    {
+        u4 t[1];
+        biased4(w[j], t, mg[0], mg[1]);
+        q = t[0];
+    }
+};
+
+template <>
+struct TileCodec<3> {
+    static constexpr int KINDS = 2;
+    static constexpr uint32_t MAGIC[4] = {MAGIC3_EVEN, MAGIC3_ODD, MAGIC3_EVEN, MAGIC3_ODD};
+    static GPTQ_HD constexpr float base(int e) { return BASE3[e & 7]; }
+    static GPTQ_HD constexpr int field(int s) { return SLOT3[s]; }
+    static GPTQ_HD void operand(const uint32_t (&w)[3], int j, u4 &q, const uint32_t (&mg)[KINDS])
+    {
+        biased3_block(w[0], w[1], w[2], j, q, mg[0], mg[1]);
+    }
+};
+
+template <>
+struct TileCodec<8> {
+    static constexpr int KINDS = 1;
+    static constexpr uint32_t MAGIC[4] = {MAGIC8, MAGIC8, MAGIC8, MAGIC8};
+    static GPTQ_HD constexpr float base(int) { return 1024.f; }
+    static GPTQ_HD constexpr int field(int s) { return (s & ~3) + SLOT8[s & 3]; }
+    static GPTQ_HD void operand(const uint32_t (&w)[8], int j, u4 &q, const uint32_t (&mg)[KINDS])
+    {
+        q[0] = and_or(w[2 * j], 0x00ff00ffu, mg[0]);
+        q[1] = and_or(w[2 * j] >> 8, 0x00ff00ffu, mg[0]);
+        q[2] = and_or(w[2 * j + 1], 0x00ff00ffu, mg[0]);
+        q[3] = and_or(w[2 * j + 1] >> 8, 0x00ff00ffu, mg[0]);
+    }
+};
+
+template <>
+struct TileCodec<2> {
+    static constexpr int KINDS = 4;
+    static constexpr uint32_t MAGIC[4] = {MAGIC2[0], MAGIC2[1], MAGIC2[2], MAGIC2[3]};
+    static GPTQ_HD constexpr float base(int e) { return (float)(1024 >> (2 * ((e >> 1) & 3))); }
+    static GPTQ_HD constexpr int field(int s) { return (s & ~15) + SLOT2[s & 15]; }
+    static GPTQ_HD void operand(const uint32_t (&w)[2], int j, u4 &q, const uint32_t (&mg)[KINDS])
+    {
+        const uint32_t t = (j & 1) ? w[j >> 1] >> 8 : w[j >> 1];
+        q[0] = and_or(t, 0x00030003u, mg[0]);
+        q[1] = and_or(t, 0x000c000cu, mg[1]);
+        q[2] = and_or(t, 0x00300030u, mg[2]);
+        q[3] = and_or(t, 0x00c000c0u, mg[3]);
+    }
+};
+
 // The dequantised weight of the reference (qlinear.py:242): fp16 scale times the
 // integer (q - zero), rounded once.  (q - zero) is exact in fp16, so one fp16 multiply
 // is that rounding, signed zeros and subnormals included.  (Going through an fp32

@@ -31,8 +31,8 @@ def _stream(device: torch.device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
-FUSED_BITS = (3, 4)        # widths the matmul kernels cover
-FORMAT_BITS = (2, 3, 4, 8)  # widths of the checkpoint format; 2 and 8 run as dequant + library GEMM
+FUSED_BITS = (3, 4)        # widths the matmul kernels on the checkpoint layout (and its sorted copy) cover
+FORMAT_BITS = (2, 3, 4, 8)  # widths of the checkpoint format; all four run fused on the tiled format
 
 
 def check_shapes(qweight, qzeros, scales, g_idx, bias, bits: int, group_size: int, widths=FUSED_BITS):
@@ -209,7 +209,7 @@ def tile_prepare(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tens
     _need_gpu("scales", scales, torch.float16)
     if g_idx is not None:
         _need_gpu("g_idx", g_idx, torch.int32)
-    K, N, G = check_shapes(qweight, qzeros, scales, g_idx, None, bits, group_size)
+    K, N, G = check_shapes(qweight, qzeros, scales, g_idx, None, bits, group_size, widths=FORMAT_BITS)
     dev = qweight.device
     nbytes = _lib.lib().gptq_hip_tiled_bytes(K, N, bits)
     qtile = torch.empty(nbytes // 4, dtype=torch.int32, device=dev)

@@ -84,9 +84,10 @@ def unpack_rows_torch(words: torch.Tensor, bits: int) -> torch.Tensor:
     [R//32*bits, C] -> codes int64 [R, C]."""
     rows, cols = words.shape
     w = words.to(torch.int64) & 0xFFFFFFFF
-    if bits == 4:
-        shifts = (4 * torch.arange(8, device=words.device)).view(1, 8, 1)
-        return ((w.unsqueeze(1) >> shifts) & 15).reshape(rows * 8, cols)
+    if bits != 3:
+        per = 32 // bits
+        shifts = (bits * torch.arange(per, device=words.device)).view(1, per, 1)
+        return ((w.unsqueeze(1) >> shifts) & ((1 << bits) - 1)).reshape(rows * per, cols)
     b = w.view(rows // 3, 3, cols)
     out = torch.empty((rows // 3, 32, cols), dtype=torch.int64, device=words.device)
     for j in range(32):
@@ -155,7 +156,7 @@ TILE_CHANNELS = 64  # input channels of one block of the tiled format: two lane 
 def tiled_qualifies(K: int, N: int, bits: int, group_size: int) -> bool:
     """Layers the tiled format covers: 3 or 4 bits, whole groups made of whole 32-channel lane blocks."""
     gs = K if group_size == -1 else group_size
-    return bits in (3, 4) and K % 32 == 0 and N % 32 == 0 and gs % 32 == 0 and K % gs == 0 and K <= 65536
+    return bits in (2, 3, 4, 8) and K % 32 == 0 and N % 32 == 0 and gs % 32 == 0 and K % gs == 0 and K <= 65536
 
 
 def tile_layout(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor, g_idx, bits: int, group_size: int):
@@ -172,9 +173,10 @@ def tile_layout(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tenso
     * ``qtile`` is a sequence of blocks, column tile T (32 columns) outermost, then block S (64 positions):
       block (T, S) is 64 lanes x ``bits`` words; lane (n = lane % 32, h = lane // 32) holds the 32 codes of
       column 32 T + n at positions 64 S + 32 h .. + 31 as the usual little-endian stream of ``bits``-bit
-      fields, with the codes permuted inside the lane (each 8 positions for 4 bits, all 32 for 3 bits) so
-      that the kernels' register unpack yields them in position order: stream field ``code_of_slot[s]``
-      holds position s.
+      fields, with the codes permuted inside the lane (each 4 / 8 / 16 positions for 8 / 4 / 2 bits, all 32
+      for 3 bits) so that the kernels' register unpack yields them in position order: stream field
+      ``lane_field_of_position[s]`` holds position s.  Word i of lane l sits at l * bits + i of the block,
+      except for 8 bits, whose block is two halves of 64 lanes x 4 words: (i // 4) * 256 + l * 4 + i % 4.
     * ``sz[g, n]`` = fp16 bits of ``scales[g, n]`` | fp16 bits of the zero point (stored value + 1) << 16.
     """
     from . import _slots
@@ -198,15 +200,17 @@ def tile_layout(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tenso
     codes = unpack_rows_torch(qweight.detach(), bits)[perm]                      # [K, N], sorted order
     if Kp > K:
         codes = torch.cat([codes, torch.zeros((Kp - K, N), dtype=codes.dtype, device=dev)])
-    # stream field i of a lane holds the position slot_of_code[i] (of each 8 for 4 bits, of the 32 for 3 bits)
-    inv = torch.tensor(_slots.slot_of_code(bits), dtype=torch.int64, device=dev)
-    if bits == 4:
-        order = (torch.arange(32, device=dev) // 8) * 8 + inv[torch.arange(32, device=dev) % 8]
-    else:
-        order = inv
+    # stream field f of a lane holds the position order[f]
+    field_of = _slots.lane_field_of_position(bits)
+    order = torch.empty(32, dtype=torch.int64, device=dev)
+    order[torch.tensor(field_of, dtype=torch.int64, device=dev)] = torch.arange(32, device=dev)
     blocks = codes.view(S * 2, 32, N)[:, order, :]                                # [(S, h), field, N]
     words = pack_rows_torch(blocks.reshape(S * 2 * 32, N), bits)                  # [(S, h, word), N]
-    qtile = words.view(S, 2, bits, T, TILE_COLS).permute(3, 0, 1, 4, 2).contiguous().view(-1)
+    words = words.view(S, 2, bits, T, TILE_COLS)
+    if bits == 8:   # [T, S, word // 4, (h, n), word % 4]
+        qtile = words.view(S, 2, 2, 4, T, TILE_COLS).permute(4, 0, 2, 1, 5, 3).contiguous().view(-1)
+    else:           # [T, S, (h, n), word]
+        qtile = words.permute(3, 0, 1, 4, 2).contiguous().view(-1)
     zeros = unpack_rows_torch(qzeros.detach().t().contiguous(), bits).t() + 1     # [G, N]
     zbits = zeros.to(torch.float16).view(torch.int16).to(torch.int64) & 0xFFFF
     sbits = scales.detach().contiguous().view(torch.int16).to(torch.int64) & 0xFFFF

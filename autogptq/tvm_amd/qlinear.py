@@ -38,7 +38,8 @@ class _ProductWithInputGrad(torch.autograd.Function):
 
 class QuantLinear(nn.Module):
     SUPPORTED_BITS = (2, 3, 4, 8)   # the widths of the format (qlinear.py:31-32)
-    FUSED_BITS = (3, 4)             # those the fused kernels cover; 2 and 8 run as dequant + library GEMM
+    FUSED_BITS = (3, 4)             # those the kernels on the checkpoint layout cover; 2 and 8 run fused on the
+                                    # tiled format only (else as dequant + library GEMM)
 
     def __init__(self, bits, groupsize, infeatures, outfeatures, bias, kernel_switch_threshold=1152,
                  sort_for_decode=True, tile_for_prefill=True):
@@ -180,7 +181,7 @@ class QuantLinear(nn.Module):
             None if g is None else (g.data_ptr(), g._version),)
         if self._tiled is None or self._tiled[0] != key:
             tensors = None
-            if (self.qweight.device.type == "cuda" and self.bits in self.FUSED_BITS
+            if (self.qweight.device.type == "cuda"
                     and tiled_qualifies(self.infeatures, self.outfeatures, self.bits, self.groupsize)
                     and (g is None or self._whole_groups(g))):
                 tensors = ops.tile_prepare(self.qweight, self.qzeros, self.scales, g, self.bits, self.groupsize)
@@ -264,12 +265,15 @@ class QuantLinear(nn.Module):
             out = torch.matmul(x2, self.dequantize())
             return out if bias is None else out + bias
 
-        if self.bits not in self.FUSED_BITS:
-            return "library", library
         g = self._kernel_g_idx()
         K, N = self.infeatures, self.outfeatures
         tiled = None
-        if self.tile_for_prefill and ops.tiled_wins(M, K, N, g is not None, bits):
+        if self.bits not in self.FUSED_BITS:
+            # 2 and 8 bits: the tiled kernels are the only fused ones
+            tiled = self.prepare_tiled() if self.tile_for_prefill else None
+            if tiled is None:
+                return "library", library
+        elif self.tile_for_prefill and ops.tiled_wins(M, K, N, g is not None, bits):
             tiled = self.prepare_tiled()
         threshold = self.kernel_switch_threshold
         if threshold and tiled is None:   # off the tiled route the library wins earlier

@@ -81,6 +81,11 @@ WORKLOADS = {
     "int4-9216x36864-g1-m1": (4, 9216, 36864, -1, True, 1),
     "int4-8192x28672-m1": (4, 8192, 28672, 128, False, 1),
     "int3-8192x28672-act-m1": (3, 8192, 28672, 128, True, 1),
+    # the other widths of the format: fused on the tiled format only
+    "int8-4096x11008-act-m1": (8, 4096, 11008, 128, True, 1),
+    "int2-4096x11008-act-m1": (2, 4096, 11008, 128, True, 1),
+    "int8-4096x11008-act-m128": (8, 4096, 11008, 128, True, 128),
+    "int2-4096x11008-act-m128": (2, 4096, 11008, 128, True, 128),
 }
 DEFAULT_WORKLOAD = "c2-int3-4096x11008-act-m1"
 # timed in the default run next to the headline: the int4 decode product and the M = 128 products of the
@@ -167,11 +172,20 @@ PREPARED_NOTE = {None: None, "sorted": "input channels sorted by group once at l
                  "tiled": "layer re-laid once at load into the tiled format (gptq_hip_tile_prepare)"}
 
 
+def plain_applies(name: str) -> bool:
+    """The kernels on the checkpoint layout (and its sorted copy) cover 3 and 4 bits."""
+    from autogptq.tvm_amd import ops
+
+    return WORKLOADS[name][0] in ops.FUSED_BITS
+
+
 def sorted_applies(name: str) -> bool:
     from autogptq.tvm_amd import ops
 
     bits, K, N, gs, desc_act, M = WORKLOADS[name]
     G = 1 if gs == -1 else -(-K // gs)
+    if not plain_applies(name):
+        return False
     return bool(desc_act and G > 1 and M <= ops.SORTED_MAX_ROWS and ops.sorted_plan(M, K, N, bits, gs) is not None)
 
 
@@ -187,7 +201,7 @@ def prepared_mode(name: str):
     from autogptq.tvm_amd import ops
 
     bits, K, N, gs, desc_act, M = WORKLOADS[name]
-    if tiled_applies(name) and ops.tiled_wins(M, K, N, desc_act, bits):
+    if tiled_applies(name) and (not plain_applies(name) or ops.tiled_wins(M, K, N, desc_act, bits)):
         return "tiled"
     return "sorted" if sorted_applies(name) else None
 
@@ -409,7 +423,7 @@ def main():
     t = time_case(case, dev, args.steps, args.warmup)
     torch.cuda.synchronize(dev)
     s = summarize(case, t)
-    if prepared:
+    if prepared and plain_applies(args.workload):
         plain = build_case(args.workload, dev)
         okp, _ = check_case(plain, dev)
         s["unprepared_us"] = round(time_case(plain, dev, min(args.steps, 100), min(args.warmup, 10))["us"], 3)
@@ -454,7 +468,8 @@ def main():
     if args.sweep:
         sweep = []
         for name, prep in [(n, pr) for n in sorted(WORKLOADS) for pr in (None, "sorted", "tiled")]:
-            if (prep == "sorted" and not sorted_applies(name)) or (prep == "tiled" and not tiled_applies(name)):
+            if ((prep is None and not plain_applies(name)) or (prep == "sorted" and not sorted_applies(name))
+                    or (prep == "tiled" and not tiled_applies(name))):
                 continue
             c = build_case(name, dev, prepared=prep)
             okc, errc = check_case(c, dev)

@@ -28,7 +28,7 @@ extern "C" {
 
 typedef enum gptq_hip_status {
     GPTQ_HIP_OK = 0,
-    GPTQ_HIP_ERR_BAD_ARG = -1,     /* null pointer, non-positive size, bits not in {3,4}, misaligned */
+    GPTQ_HIP_ERR_BAD_ARG = -1,     /* null pointer, non-positive size, a width the entry point does not take, misaligned */
     GPTQ_HIP_ERR_UNSUPPORTED = -2, /* shape outside what the kernels cover (see gptq_hip_select) */
     GPTQ_HIP_ERR_WORKSPACE = -3,   /* workspace missing or smaller than the plan needs */
     GPTQ_HIP_ERR_LAUNCH = -4       /* the HIP runtime refused the launch */
@@ -183,7 +183,8 @@ size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits, int group_
  *   qtile  gptq_hip_tiled_bytes(K, N, bits) bytes, 16-byte aligned: blocks of 64 lanes x `bits` words, column tile
  *          (32 columns) outermost, then block of 64 sorted positions; lane (n = lane % 32, h = lane / 32) holds the 32
  *          codes of column 32 T + n at positions 64 S + 32 h .. + 31, permuted inside the lane into the order in
- *          which the kernels' register unpack hands them to the matrix instruction
+ *          which the kernels' register unpack hands them to the matrix instruction (word i of lane l at
+ *          l * bits + i of the block; 8 bits: at (i / 4) * 256 + l * 4 + i % 4)
  *   sz     uint32 [G, N]: fp16 scale | fp16 (zero point) << 16
  *   xsrc   int32 [Kp], 16-byte aligned: the channel of x at sorted position p (stable sort of the channels by
  *          group; the identity without an activation order), -1 for p >= K
@@ -192,6 +193,8 @@ size_t gptq_hip_sorted_workspace_bytes(int M, int K, int N, int bits, int group_
  * needs whole groups of equal size that are multiples of 32 channels (GPTQ_HIP_ERR_UNSUPPORTED otherwise) and
  * a g_idx that gives every group exactly group_size channels (other contents stay in bounds but do not describe
  * the layer).  Three launches; the sort costs K * K / 2 compares.
+ * bits: 2, 3, 4 or 8, every width of the format (qlinear.py:31-32): the tiled entry points are the fused path
+ * of 2- and 8-bit layers, which the entry points on the checkpoint layout above do not take.
  */
 size_t gptq_hip_tiled_bytes(int K, int N, int bits);
 int gptq_hip_tile_prepare(const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *g_idx,
@@ -221,8 +224,8 @@ int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint32_t *sz, co
 /*
  * W fp16 [K, N] = scales[g] * (q - (zq[g] + 1)), one rounding per element:
  * the materialised weight of qlinear.py:198-242, for the bit-exact check.  bits may also be 2 or 8
- * here (the other widths of the format, qlinear.py:31-32,211-215): those layers run as this kernel
- * followed by a library GEMM.
+ * here (the other widths of the format, qlinear.py:31-32,211-215): without a tiled copy those layers run as
+ * this kernel followed by a library GEMM.
  */
 int gptq_hip_dequant(const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *g_idx,
                      void *w, int K, int N, int bits, int group_size, void *stream);

@@ -3,6 +3,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <initializer_list>
+
 #include "gptq_unpack.h"
 
 using namespace gptq;
@@ -14,6 +16,57 @@ static uint32_t rnd()
     state ^= state >> 7;
     state ^= state << 17;
     return (uint32_t)(state >> 16);
+}
+
+// field f (BITS wide) of the little-endian stream held in the lane's words
+template <int BITS>
+static int stream_field(const uint32_t *w, int f)
+{
+    const int bit = BITS * f, wd = bit >> 5, sh = bit & 31;
+    uint64_t v = w[wd];
+    if (wd + 1 < BITS) v |= (uint64_t)w[wd + 1] << 32;
+    return (int)((v >> sh) & ((1u << BITS) - 1u));
+}
+
+// The tiled format's codec: register r, half h of operand j reads base(2 r + h) + the code in stream field
+// field(8 j + 2 r + h), and field() is a permutation of the lane's 32 fields.
+template <int BITS>
+static bool check_codec(const uint32_t (&w)[BITS], long &checked)
+{
+    using C = TileCodec<BITS>;
+    uint32_t mg[C::KINDS];
+    for (int k = 0; k < C::KINDS; k++) mg[k] = C::MAGIC[k];
+    uint32_t seen = 0u;
+    for (int j = 0; j < 4; j++) {
+        u4 q;
+        C::operand(w, j, q, mg);
+        for (int r = 0; r < 4; r++) {
+            const h2 v = as_h2(q[r]);
+            for (int h = 0; h < 2; h++) {
+                const int s = 8 * j + 2 * r + h;
+                seen |= 1u << C::field(s);
+                if (C::base(2 * r + h) != C::base(s) ||
+                    (float)v[h] - C::base(s) != (float)stream_field<BITS>(w, C::field(s))) {
+                    printf("codec<%d> mismatch operand %d reg %d half %d got %f\n", BITS, j, r, h, (float)v[h]);
+                    return false;
+                }
+                // the matmul's dequantisation: (v - (base + zero)) is exact for every zero point of the width
+                for (int z = 1; z <= (1 << BITS); z += (1 << BITS) - 1) {
+                    const _Float16 zb = (_Float16)(C::base(s) + (float)z);
+                    if ((float)(_Float16)(v[h] - zb) != (float)(stream_field<BITS>(w, C::field(s)) - z)) {
+                        printf("codec<%d> zero-point subtraction is not exact\n", BITS);
+                        return false;
+                    }
+                }
+                checked++;
+            }
+        }
+    }
+    if (seen != 0xffffffffu) {
+        printf("codec<%d>: field() is not a permutation\n", BITS);
+        return false;
+    }
+    return true;
 }
 
 int main()
@@ -77,6 +130,14 @@ int main()
                 checked++;
             }
         }
+        {
+            const uint32_t a2[2] = {w0, w1}, a3[3] = {w0, w1, w2}, a4[4] = {w0, w1, w2, rnd()};
+            uint32_t a8[8] = {w0, w1, w2, rnd(), rnd(), rnd(), rnd(), rnd()};
+            if (it == 0) for (auto &v : a8) v = 0xffffffffu;
+            if (!check_codec<2>(a2, checked) || !check_codec<3>(a3, checked) || !check_codec<4>(a4, checked) ||
+                !check_codec<8>(a8, checked))
+                return 1;
+        }
         // code3 itself against the reference's straddle formulas (qlinear.py:233-234)
         const int c10 = (int)(((w0 >> 30) & 0x3u) | ((w1 << 2) & 0x4u));
         const int c21 = (int)(((w1 >> 31) & 0x1u) | ((w2 << 1) & 0x6u));
@@ -108,6 +169,15 @@ int main()
     for (int i = 0; i < 8; i++) printf(" %d", SLOT4[i]);
     printf("\nslot3");
     for (int i = 0; i < 32; i++) printf(" %d", SLOT3[i]);
+    printf("\nslot8");
+    for (int i = 0; i < 4; i++) printf(" %d", SLOT8[i]);
+    printf("\nslot2");
+    for (int i = 0; i < 16; i++) printf(" %d", SLOT2[i]);
+    for (int bits : {2, 3, 4, 8}) {
+        printf("\nfield%d", bits);
+        for (int s = 0; s < 32; s++)
+            printf(" %d", bits == 2 ? TileCodec<2>::field(s) : bits == 3 ? TileCodec<3>::field(s) : bits == 4 ? TileCodec<4>::field(s) : TileCodec<8>::field(s));
+    }
     printf("\n");
     return 0;
 }

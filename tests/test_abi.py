@@ -283,3 +283,42 @@ def test_torch_operator_library_is_built_and_matches_the_kernel_library():
                                       torch.empty(64 * 32 // 8, dtype=torch.int32, device="meta"),
                                       torch.empty(1, 32, dtype=torch.int32, device="meta"), None, None, None, 4, 64)
     assert m.shape == (5, 32) and m.device.type == "meta"
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
+@pytest.mark.parametrize("KN", [(4096, 4096), (4096, 11008), (11008, 4096), (96, 32), (9216, 36864)])
+def test_tiled_plans_are_consistent(bits, KN):
+    """The tiled family plans every width of the format; the launches it describes cover the problem and stay
+    within a workgroup's LDS (no GPU needed: the plans are host arithmetic)."""
+    K, N = KN
+    gs = 128 if K % 128 == 0 else 32
+    blocks = -(-K // 64)
+    for M in (1, 2, 4, 5, 16, 17, 128, 129, 1024):
+        p = _lib.select_tiled(M, K, N, bits, gs)
+        assert p.lds_bytes <= 160 * 1024 and p.block in (256, 512, 1024) and p.split_k == p.grid_y >= 1
+        if M <= 4:
+            assert p.kernel == _lib.KERNEL_TILED_DECODE and p.row_tiles >= M
+            if p.waves_n == 2:       # a workgroup per CU, 16-column units, sixteen waves over the 128-position blocks
+                assert p.block == 1024 and 1 <= p.grid_x <= min(N // 16, 256) and p.k_chunk * 16 >= -(-blocks // 2)
+            else:                    # a workgroup per 32-column tile
+                assert p.grid_x == N // 32 and p.split_k * p.waves_k * p.k_chunk >= blocks
+        else:
+            assert p.kernel == _lib.KERNEL_TILED
+            cols = 64 * p.waves_n
+            assert p.grid_x * cols >= N and p.grid_z == p.m_blocks and p.m_blocks * p.row_tiles * 32 >= M
+            assert p.split_k * p.waves_k * p.k_chunk >= blocks
+            assert p.workspace_bytes >= p.split_k * p.waves_k * p.k_chunk * 4 * p.row_tiles * p.m_blocks * 1024
+    assert _lib.lib().gptq_hip_tiled_bytes(K, N, bits) == blocks * 64 * N * bits // 8
+
+
+def test_tiled_plans_reject_what_the_format_does_not_cover():
+    for args, status in [((1, 4096, 4096, 5, 128), _lib.ERR_BAD_ARG),      # a width the format does not have
+                         ((1, 4096, 4096, 4, 16), _lib.ERR_UNSUPPORTED),   # groups narrower than a lane block
+                         ((1, 4096, 4100, 4, 128), _lib.ERR_BAD_ARG),
+                         ((0, 4096, 4096, 4, 128), _lib.ERR_BAD_ARG)]:
+        with pytest.raises(_lib.GptqHipError) as e:
+            _lib.select_tiled(*args)
+        assert e.value.status == status, args
+    with pytest.raises(_lib.GptqHipError):
+        _lib.select_tiled(5, 4096, 4096, 8, 128, decode=True)             # the decode kernels take up to four rows
+    assert _lib.lib().gptq_hip_tiled_bytes(4096, 4096, 5) == 0

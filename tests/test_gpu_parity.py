@@ -360,14 +360,15 @@ def test_dequant_bit_exact_two_and_eight_bits(dev, bits, desc_act, shape):
 def test_module_runs_two_and_eight_bit_layers_as_dequant_plus_gemm(dev, bits, M):
     K, N, gs = 512, 256, 128
     L = layer(130 + bits, K, N, bits, gs, True, M=M, bias=True)
-    q = QuantLinear(bits, gs, K, N, True)
+    q = QuantLinear(bits, gs, K, N, True, tile_for_prefill=False)   # (with the tiled copy these widths run fused)
     q.load_state_dict({k: L[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})
     q = q.to(dev)
+    assert q.route(M) == "library"
     y = q(L["x"].to(dev))
     assert y.shape == (M, N) and y.dtype == torch.float16
     assert_close(y, expected_output(L), f"module forward, {bits} bits")
     assert torch.equal(q.dequantize().cpu().view(torch.int16), expected_weight(L).view(torch.int16))
-    # the fused entry points do not take these widths
+    # the entry points on the checkpoint layout do not take these widths
     with pytest.raises(NotImplementedError):
         run_gemm(to_dev(L, dev))
 

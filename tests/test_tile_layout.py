@@ -10,7 +10,7 @@ from autogptq.tvm_amd import _slots, pack
 from oracle import gptq_oracle as orc
 
 
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 @pytest.mark.parametrize("K,N,gs,act", [(64, 32, 32, False), (192, 64, 64, True), (1056, 96, 32, True),
                                         (2048, 64, 128, True), (96, 32, -1, True), (160, 32, 32, False)])
 def test_tile_layout_decodes_to_the_layer(bits, K, N, gs, act):
@@ -19,22 +19,21 @@ def test_tile_layout_decodes_to_the_layer(bits, K, N, gs, act):
     Kp = (K + 63) // 64 * 64
     S, T = Kp // 64, N // 32
     assert qtile.numel() == T * S * 64 * bits and tuple(xsrc.shape) == (Kp,)
-    qt = qtile.numpy().view(np.uint32).reshape(T, S, 64, bits).astype(np.uint64)
-    stream_lo = qt[..., 0] | (qt[..., 1] << np.uint64(32))          # bits 0..63 of every lane's stream
-    stream_hi = qt[..., 2] if bits == 3 else (qt[..., 2] | (qt[..., 3] << np.uint64(32)))   # bits 64..
+    if bits == 8:   # the block is two halves of 64 lanes x 4 words
+        qt = qtile.numpy().view(np.uint32).reshape(T, S, 2, 64, 4).transpose(0, 1, 3, 2, 4).reshape(T, S, 64, 8)
+    else:
+        qt = qtile.numpy().view(np.uint32).reshape(T, S, 64, bits)
+    qt = np.concatenate([qt, np.zeros_like(qt[..., :1])], axis=-1).astype(np.uint64)   # (a zero word past the end)
     codes = orc.unpack_qweight_ref(L["qweight"], bits).numpy()      # the oracle's unpack, [K, N]
     assert np.array_equal(codes, L["codes"].numpy())
-    code_of_slot = _slots.code_of_slot(bits)
+    field_of = _slots.lane_field_of_position(bits)
+    assert sorted(field_of) == list(range(32))
     x = xsrc.numpy()
     for s in range(32):
-        field = (s // 8) * 8 + code_of_slot[s % 8] if bits == 4 else code_of_slot[s]
-        bit = bits * field
-        if bit + bits <= 64:
-            q = (stream_lo >> np.uint64(bit)) & np.uint64((1 << bits) - 1)
-        elif bit >= 64:
-            q = (stream_hi >> np.uint64(bit - 64)) & np.uint64((1 << bits) - 1)
-        else:   # a 3-bit field across bit 64
-            q = ((stream_lo >> np.uint64(bit)) | (stream_hi << np.uint64(64 - bit))) & np.uint64(7)
+        bit = bits * field_of[s]
+        wd, sh = bit // 32, bit % 32
+        two = qt[..., wd] | (qt[..., wd + 1] << np.uint64(32))       # the field may straddle two words (3 bits)
+        q = (two >> np.uint64(sh)) & np.uint64((1 << bits) - 1)
         for h in range(2):
             pos = 64 * np.arange(S) + 32 * h + s                     # [S]
             src = x[pos]

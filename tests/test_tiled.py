@@ -77,7 +77,7 @@ def run_tiled(D, prep, x=None, plan=None):
                           D.get("bias"), D["bits"], D["group_size"], plan=plan)
 
 
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 @pytest.mark.parametrize("K,N,gs", [(64, 32, 32), (96, 32, 32), (1024, 416, 32), (2048, 1056, 256), (11008, 256, 128),
                                     (1024, 160, -1), (4096, 352, 128)])
 @pytest.mark.parametrize("desc_act", [False, True])
@@ -99,7 +99,7 @@ def test_library_preparation_equals_the_torch_statement(dev, bits, K, N, gs, des
 M_EDGES = [1, 2, 5, 16, 17, 31, 32, 33, 64, 65, 127, 128, 129, 257]
 
 
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 @pytest.mark.parametrize("desc_act", [False, True])
 @pytest.mark.parametrize("M", M_EDGES)
 def test_tiled_ragged_m(dev, bits, desc_act, M):
@@ -111,7 +111,7 @@ def test_tiled_ragged_m(dev, bits, desc_act, M):
     assert_tight(y, expected_output(L), f"tiled bits={bits} act={desc_act} M={M}")
 
 
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 @pytest.mark.parametrize("K,N,gs", [(32, 32, 32), (96, 32, 32), (160, 96, -1), (384, 64, 64), (1024, 416, 32),
                                     (2048, 1056, 256), (4096, 352, 128)])
 @pytest.mark.parametrize("M", [1, 7, 40, 130])
@@ -127,7 +127,7 @@ def test_tiled_odd_shapes(dev, bits, K, N, gs, M):
         assert torch.equal(y, run_tiled(D, prep)), "two identical calls differ"
 
 
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 @pytest.mark.parametrize("split", [1, 2, 3, 5])
 @pytest.mark.parametrize("M", [20, 130])
 def test_tiled_forced_split_k(dev, bits, split, M):
@@ -149,14 +149,14 @@ def test_tiled_forced_split_k(dev, bits, split, M):
 
 
 def test_tiled_integer_exact_and_guard_bands(dev):
-    # x = 1, scales = 1, one group: y[n] = sum_k (q - z), exactly representable
-    for bits in (3, 4):
+    # x = 1, scales = 1, one group: y[n] = sum_k (q - z), an integer (8-bit sums pass 2048: one fp16 rounding)
+    for bits in (2, 3, 4, 8):
         L = layer(1500, 64, 64, bits, -1, False, M=2)
         L["scales"] = torch.ones_like(L["scales"])
         L["x"] = torch.ones_like(L["x"])
         D = to_dev(L, dev)
         y = run_tiled(D, prepare(D)).float().cpu()
-        want = (L["codes"].float() - L["zeros"][0].float()[None, :]).sum(dim=0)
+        want = (L["codes"].float() - L["zeros"][0].float()[None, :]).sum(dim=0).half().float()
         assert torch.equal(y[0], want) and torch.equal(y[1], want)
     M, K, N = 37, 512, 96
     L = layer(1501, K, N, 4, 128, True, M=M)
@@ -190,7 +190,7 @@ def test_tiled_rejections(dev):
     assert lib.gptq_hip_tiled_bytes(96, 32, 4) == 128 * 32 // 2
 
 
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 @pytest.mark.parametrize("K,N,gs", [(32, 32, 32), (96, 32, 32), (160, 96, -1), (384, 64, 64), (1024, 416, 32),
                                     (2048, 1056, 256), (4096, 352, 128), (11008, 256, 128), (4096, 64, 64)])
 @pytest.mark.parametrize("M", [1, 2, 3, 4])
@@ -206,7 +206,9 @@ def test_tiled_decode_rows_and_shapes(dev, bits, K, N, gs, M):
         prep = prepare(D)
         want = expected_output(L)
         g = D["g_idx"] if desc_act else None
-        plain = ops.gemm(D["x"], D["qweight"], D["qzeros"], D["scales"], g, D.get("bias"), bits, gs).cpu()
+        # (the kernels on the checkpoint layout cover 3 and 4 bits)
+        plain = (ops.gemm(D["x"], D["qweight"], D["qzeros"], D["scales"], g, D.get("bias"), bits, gs).cpu()
+                 if bits in ops.FUSED_BITS else None)
         # both decode kernels, and the one-workgroup-per-CU kernel on fewer workgroups (several units each)
         plans = [("own", own), ("tile", tile_decode_plan(M, K, N, bits, gs)), ("cu", cu_decode_plan(M, K, N, bits, gs)),
                  ("cu, few workgroups", cu_decode_plan(M, K, N, bits, gs, grid=max(1, (N // 16) // 5)))]
@@ -217,10 +219,11 @@ def test_tiled_decode_rows_and_shapes(dev, bits, K, N, gs, M):
             assert_close(y, want, f"decode ({what}) bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
             assert_tight(y, want, f"decode ({what}) bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
             assert torch.equal(y, run_tiled(D, prep, plan=plan)), "two identical calls differ"
-            assert_tight(y, plain, "decode vs the unprepared kernels")
+            if plain is not None:
+                assert_tight(y, plain, "decode vs the unprepared kernels")
 
 
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 @pytest.mark.parametrize("M", [1, 4])
 def test_tiled_decode_split_k(dev, bits, M):
     # a forced split of K over workgroups (what a long K with many rows needs): partial sums and the reduce pass
@@ -248,6 +251,10 @@ DECODE_FULL = [
     ("c5-int3-9216x9216-act-g1", 3, 9216, 9216, -1, True, [1]),
     ("c5-int3-9216x36864-act-g1", 3, 9216, 36864, -1, True, [1]),
     ("c5-int3-36864x9216-act-g1", 3, 36864, 9216, -1, True, [1]),
+    ("int8-4096x11008-act", 8, 4096, 11008, 128, True, [1, 4]),
+    ("int2-4096x11008-act", 2, 4096, 11008, 128, True, [1, 3]),
+    ("int8-11008x4096", 8, 11008, 4096, 128, False, [2]),
+    ("int2-4096x4096-g64", 2, 4096, 4096, 64, False, [1]),
 ]
 
 
@@ -278,6 +285,10 @@ TILED_FULL = [
     ("c3-int4-4096x4096", 4, 4096, 4096, 128, False, [8, 1024]),
     ("c5-int3-9216x36864-act-g1", 3, 9216, 36864, -1, True, [32]),
     ("c5-int3-36864x9216-act-g1", 3, 36864, 9216, -1, True, [32]),
+    ("int8-4096x11008-act", 8, 4096, 11008, 128, True, [16, 128, 256]),
+    ("int2-4096x11008-act", 2, 4096, 11008, 128, True, [16, 128, 256]),
+    ("int8-11008x4096", 8, 11008, 4096, 128, False, [64]),
+    ("int2-11008x4096-act", 2, 11008, 4096, 128, True, [64]),
 ]
 
 
@@ -333,7 +344,32 @@ def test_quantlinear_routes_prompt_sizes_to_the_tiled_copy(dev, bits, desc_act):
     assert q3._tiled is not None and q3._tiled[1] is None and not q3.compact()
 
 
-@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("bits", [2, 8])
+@pytest.mark.parametrize("desc_act", [False, True])
+def test_quantlinear_runs_2_and_8_bits_fused_on_the_tiled_copy(dev, bits, desc_act):
+    """2- and 8-bit layers have no kernels on the checkpoint layout: every row count below the switch to the
+    library GEMM runs on the tiled copy; without it (or above the switch) the layer is dequantised."""
+    K, N, gs = 1024, 416, 128
+    L = layer(1850 + bits, K, N, bits, gs, desc_act, M=150, bias=True)
+    q = module_of(L, dev, kernel_switch_threshold=128)
+    x = L["x"].to(dev)
+    want = expected_output(L)
+    for M in (1, 3, 8, 40, 127):
+        assert q.route(M) == "tiled"
+        y = q(x[:M])
+        assert_close(y, want[:M], f"module, {M} rows")
+        assert_tight(y, want[:M], f"module, {M} rows")
+    assert q.route(150) == "library"
+    assert_close(q(x), want, "module, 150 rows (library)")
+    off = module_of(L, dev, tile_for_prefill=False)
+    assert off.route(1) == "library" and off._tiled is None
+    assert_close(off(x[:3]), want[:3], "module without the tiled copy")
+    assert q.compact() and q.route(150) == "tiled"
+    assert_tight(q(x), want, "compact module, 150 rows")
+    assert torch.equal(q.dequantize().cpu().view(torch.int16), expected_weight(L).view(torch.int16))
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 @pytest.mark.parametrize("desc_act", [False, True])
 def test_quantlinear_compact_keeps_one_copy(dev, bits, desc_act):
     K, N, gs = 1024, 416, 128

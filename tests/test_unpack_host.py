@@ -33,3 +33,8 @@ def test_magic_unpack_matches_bit_extraction(tmp_path):
     lines = {l.split()[0]: [int(v) for v in l.split()[1:]] for l in out.stdout.splitlines()[1:]}
     assert lines["slot4"] == _slots.CODE_OF_SLOT4
     assert lines["slot3"] == _slots.CODE_OF_SLOT3
+    assert lines["slot8"] == _slots.CODE_OF_SLOT8
+    assert lines["slot2"] == _slots.CODE_OF_SLOT2
+    # the tiled format's permutation per width, as the kernels' codec states it
+    for bits in (2, 3, 4, 8):
+        assert lines[f"field{bits}"] == _slots.lane_field_of_position(bits)
