@@ -39,6 +39,11 @@ ABI_SYMBOLS = (
     "gptq_hip_tile_prepare",
     "gptq_hip_select_tiled",
     "gptq_hip_select_tiled_decode",
+    "gptq_hip_tiled_transposed_bytes",
+    "gptq_hip_tiled_transposed_table_bytes",
+    "gptq_hip_tile_prepare_transposed",
+    "gptq_hip_select_tiled_transposed",
+    "gptq_hip_gemm_tiled_transposed",
     "gptq_hip_gemm_tiled",
     "gptq_hip_dequant",
     "gptq_hip_strerror",
@@ -124,6 +129,16 @@ def lib() -> ctypes.CDLL:
     l.gptq_hip_select_tiled_decode.argtypes = [i, i, i, i, i, ctypes.POINTER(Plan)]
     l.gptq_hip_gemm_tiled.restype = i
     l.gptq_hip_gemm_tiled.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
+    l.gptq_hip_tiled_transposed_bytes.restype = sz
+    l.gptq_hip_tiled_transposed_bytes.argtypes = [i, i, i]
+    l.gptq_hip_tiled_transposed_table_bytes.restype = sz
+    l.gptq_hip_tiled_transposed_table_bytes.argtypes = [i, i, i]
+    l.gptq_hip_tile_prepare_transposed.restype = i
+    l.gptq_hip_tile_prepare_transposed.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
+    l.gptq_hip_select_tiled_transposed.restype = i
+    l.gptq_hip_select_tiled_transposed.argtypes = [i, i, i, i, i, ctypes.POINTER(Plan)]
+    l.gptq_hip_gemm_tiled_transposed.restype = i
+    l.gptq_hip_gemm_tiled_transposed.argtypes = [vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
     l.gptq_hip_dequant.restype = i
     l.gptq_hip_dequant.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
     l.gptq_hip_strerror.restype = ctypes.c_char_p
@@ -168,6 +183,16 @@ def select_tiled(M: int, K: int, N: int, bits: int, group_size: int, decode: boo
     rc = fn(M, K, N, bits, group_size, ctypes.byref(plan))
     if rc != OK:
         raise GptqHipError(rc, f"gptq_hip_select_tiled(M={M}, K={K}, N={N}, bits={bits}, group_size={group_size})")
+    return plan
+
+
+def select_tiled_transposed(M: int, K: int, N: int, bits: int, group_size: int) -> Plan:
+    """The plan of the transposed product gx[M, K] = gy[M, N] @ W^T on the tiled family."""
+    plan = Plan()
+    rc = lib().gptq_hip_select_tiled_transposed(M, K, N, bits, group_size, ctypes.byref(plan))
+    if rc != OK:
+        raise GptqHipError(rc, f"gptq_hip_select_tiled_transposed(M={M}, K={K}, N={N}, bits={bits}, "
+                               f"group_size={group_size})")
     return plan
 
 

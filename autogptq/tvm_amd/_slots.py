@@ -10,6 +10,14 @@ CODE_OF_SLOT2 = [0, 8, 1, 9, 2, 10, 3, 11, 4, 12, 5, 13, 6, 14, 7, 15]
 
 _TABLES = {2: CODE_OF_SLOT2, 3: CODE_OF_SLOT3, 4: CODE_OF_SLOT4, 8: CODE_OF_SLOT8}
 
+# The register unpack leaves (base + code) in each half register; the base of position e of an octet:
+BASE_OF_POSITION = {
+    2: [1024, 1024, 256, 256, 64, 64, 16, 16],
+    3: [1024, 256, 128, 32, 1024, 256, 128, 32],
+    4: [1024, 1024, 64, 64, 1024, 1024, 64, 64],
+    8: [1024] * 8,
+}
+
 
 def code_of_slot(bits: int):
     """The table of one period of the width's permutation (4, 8, 16 or 32 codes)."""

@@ -405,6 +405,75 @@ extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint3
     return gptq::launch_tiled(x, qtile, sz, xsrc, bias, y, xpack, partial, M, K, N, K / gs, bits, gs, *plan, stream);
 }
 
+extern "C" size_t gptq_hip_tiled_transposed_bytes(int K, int N, int bits)
+{
+    if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0 || (bits != 2 && bits != 3 && bits != 4 && bits != 8)) return 0;
+    return (size_t)K * (size_t)((N + 63) / 64 * 64) * bits / 8;
+}
+
+extern "C" size_t gptq_hip_tiled_transposed_table_bytes(int K, int N, int group_size)
+{
+    if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0 || group_size == 0 || group_size < -1) return 0;
+    const int gs = group_size == -1 ? K : group_size;
+    if (K % gs != 0) return 0;
+    return (size_t)(K / gs) * (size_t)((N + 63) / 64) * 256;
+}
+
+extern "C" int gptq_hip_tile_prepare_transposed(const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                                                const int32_t *xsrc, void *qtile_t, uint32_t *szt, int K, int N, int bits,
+                                                int group_size, void *stream)
+{
+    if (!qtile_t || !szt || (const void *)qweight == qtile_t) return GPTQ_HIP_ERR_BAD_ARG;
+    const int rc = check_common(qweight, qzeros, scales, K, N, bits, group_size, true);
+    if (rc != GPTQ_HIP_OK) return rc;
+    if (!aligned(qtile_t, 16) || !aligned(szt, 16) || (xsrc && !aligned(xsrc, 16))) return GPTQ_HIP_ERR_BAD_ARG;
+    const int gs = group_size == -1 ? K : group_size;
+    if (!gptq::tiled_qualifies(K, N, bits, gs)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    if ((long long)K * ((N + 63) / 64 * 64) * bits / 8 >= (1LL << 32)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    return gptq::launch_tile_prepare_t((const uint32_t *)qweight, (const uint32_t *)qzeros, scales, xsrc,
+                                       (uint32_t *)qtile_t, szt, K, N, K / gs, bits, stream);
+}
+
+extern "C" int gptq_hip_gemm_tiled_transposed(const void *gy, const void *qtile_t, const uint32_t *szt,
+                                              const int32_t *xsrc, void *gx, void *workspace, size_t workspace_bytes,
+                                              int M, int K, int N, int bits, int group_size, const gptq_hip_plan *plan,
+                                              void *stream)
+{
+    if (!gy || !qtile_t || !szt || !gx || M < 1) return GPTQ_HIP_ERR_BAD_ARG;
+    if (bits != 2 && bits != 3 && bits != 4 && bits != 8) return GPTQ_HIP_ERR_BAD_ARG;
+    if (K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;
+    if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
+    if (!aligned(gy, 16) || !aligned(qtile_t, 16) || !aligned(szt, 16) || !aligned(gx, 8) || (xsrc && !aligned(xsrc, 16)))
+        return GPTQ_HIP_ERR_BAD_ARG;
+    const int gs = group_size == -1 ? K : group_size;
+    if (!gptq::tiled_qualifies(K, N, bits, gs)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    if ((long long)K * ((N + 63) / 64 * 64) * bits / 8 >= (1LL << 32)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    gptq_hip_plan chosen;
+    if (!plan) {
+        const int rc = gptq_hip_select_tiled_transposed(M, K, N, bits, group_size, &chosen);
+        if (rc != GPTQ_HIP_OK) return rc;
+        plan = &chosen;
+    }
+    // the plan must be one this product runs, sized for this problem
+    const int rts = plan->row_tiles, kwv = 4;
+    const int S_total = (N + 63) / 64;
+    if (plan->kernel != GPTQ_HIP_KERNEL_TILED || (rts != 1 && rts != 2 && rts != 4) || plan->waves_n != 1)
+        return GPTQ_HIP_ERR_UNSUPPORTED;
+    if (plan->block != 64 * kwv || plan->waves_k != kwv || plan->split_k < 1 || plan->k_chunk < 1 || plan->m_blocks < 1 ||
+        plan->grid_x != (K / 32 + 1) / 2 || plan->grid_y != plan->split_k || plan->grid_z != plan->m_blocks ||
+        (long long)plan->m_blocks * 32 * rts < M || (long long)plan->split_k * kwv * plan->k_chunk < S_total ||
+        kwv * plan->k_chunk > gptq::kTiledTMaxBlocks || plan->lds_bytes < gptq::tiled_t_lds_bytes(rts, kwv, plan->k_chunk) ||
+        plan->lds_bytes > 160 * 1024)
+        return GPTQ_HIP_ERR_BAD_ARG;
+    if (plan->split_k > 1 && (long long)M * K >= (1LL << 32)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    const size_t part = plan->split_k > 1 ? ((size_t)plan->split_k * M * K * sizeof(float) + 255) / 256 * 256 : 0;
+    const size_t xb = (size_t)gptq::tiled_pack_blocks(plan->split_k, kwv, plan->k_chunk) * 4 * (size_t)(rts * plan->m_blocks) * 1024;
+    if (!workspace || !aligned(workspace, 16) || workspace_bytes < gptq::kCounterBytes + part + xb) return GPTQ_HIP_ERR_WORKSPACE;
+    float *partial = (float *)((char *)workspace + gptq::kCounterBytes);
+    char *xpack = (char *)workspace + gptq::kCounterBytes + part;
+    return gptq::launch_tiled_t(gy, qtile_t, szt, xsrc, gx, xpack, partial, M, K, N, bits, gs, *plan, stream);
+}
+
 extern "C" int gptq_hip_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                              const int32_t *g_idx, const void *bias, void *y, void *workspace,
                              size_t workspace_bytes, int M, int K, int N, int bits, int group_size, void *stream)

@@ -606,6 +606,48 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     return GPTQ_HIP_OK;
 }
 
+// The transposed product gx[M, K] = gy[M, N] @ W^T on the matmul kernel: the reduction runs over the layer's N
+// columns (blocks of 64), the result has K columns (tiles of 32 positions, two per workgroup).
+extern "C" int gptq_hip_select_tiled_transposed(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan)
+{
+    const int ok = tiled_args_ok(M, K, N, bits, group_size, plan);
+    if (ok != GPTQ_HIP_OK) return ok;
+    const int at = gptq::tiled_row_tiles(M), kwv = 4, ct = 2;
+    const int m_blocks = ceil_div(M, 32 * at);
+    const int col_pairs = ceil_div(K / 32, ct);
+    const int S_total = ceil_div(N, 64);
+    const long long tiles = (long long)col_pairs * m_blocks;
+    int split = (int)((256 + tiles / 2) / tiles);
+    if (split < 1) split = 1;
+    int cap = (int)((3LL * N * bits) / (128LL * M));   // the fp32 tiles of a split stay within 3x the packed weights
+    if (cap < 1) cap = 1;
+    if (split > cap) split = cap;
+    if ((long long)M * K >= (1LL << 32)) split = 1;
+    while (split > 1 && S_total / (split * kwv) < gptq::tiled_ring(at)) split--;
+    // the table of a workgroup's K range must fit its LDS
+    while (ceil_div(S_total, split * kwv) * kwv > gptq::kTiledTMaxBlocks) split++;
+    if (split > 1 && (long long)M * K >= (1LL << 32)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    const int wave_steps = ceil_div(S_total, split * kwv);
+    split = ceil_div(S_total, wave_steps * kwv);
+    plan->kernel = GPTQ_HIP_KERNEL_TILED;
+    plan->row_tiles = at;
+    plan->m_blocks = m_blocks;
+    plan->waves_n = 1;
+    plan->waves_k = kwv;
+    plan->split_k = split;
+    plan->k_chunk = wave_steps;
+    plan->grid_x = col_pairs;
+    plan->grid_y = split;
+    plan->grid_z = m_blocks;
+    plan->block = 64 * kwv;
+    plan->lds_bytes = gptq::tiled_t_lds_bytes(at, kwv, wave_steps);
+    size_t ws = gptq::kCounterBytes;
+    if (split > 1) ws += ((size_t)split * M * K * sizeof(float) + 255) / 256 * 256;
+    ws += (size_t)gptq::tiled_pack_blocks(split, kwv, wave_steps) * 4 * (size_t)(at * m_blocks) * 1024;
+    plan->workspace_bytes = ws;
+    return GPTQ_HIP_OK;
+}
+
 extern "C" size_t gptq_hip_workspace_bytes(int M, int K, int N, int bits, int group_size, int act_order)
 {
     gptq_hip_plan plan;

@@ -178,6 +178,14 @@ constexpr int tiled_ring(int at) { return at >= 4 ? 3 : (at == 2 ? 4 : 6); }
 inline int tiled_pack_blocks(int split_k, int waves_k, int wave_steps) { return split_k * waves_k * wave_steps; }
 // LDS of a workgroup: the result tiles (32 x 32 floats, two per 32 rows) of its waves
 inline int tiled_lds_bytes(int row_tiles, int waves_k) { return waves_k * row_tiles * 2 * 4096; }
+// the transposed product: the result tiles, or the table of (scale, base + zero) pairs of the workgroup's K range
+// for its two column tiles (256 bytes per block and tile), whichever is larger: they share the memory
+inline int tiled_t_lds_bytes(int row_tiles, int waves_k, int wave_steps)
+{
+    const int red = tiled_lds_bytes(row_tiles, waves_k), tbl = 2 * waves_k * wave_steps * 256;
+    return red > tbl ? red : tbl;
+}
+constexpr int kTiledTMaxBlocks = 304;   // blocks of 64 columns a workgroup of the transposed product may walk (LDS)
 inline bool tiled_qualifies(int K, int N, int bits, int gs)
 {
     // (the pack pass stages one row of x in LDS: K * 2 bytes)
@@ -211,6 +219,11 @@ int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, co
 int launch_tiled_decode16(const void *x, const void *qtile, const uint32_t *sz, const uint16_t *kinv, const void *bias,
                           void *y, int M, int K, int N, int G, int bits, int group_size, const gptq_hip_plan &plan,
                           void *stream);
+int launch_tile_prepare_t(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *xsrc,
+                          uint32_t *qtile_t, uint32_t *szt, int K, int N, int G, int bits, void *stream);
+int launch_tiled_t(const void *gy, const void *qtile_t, const uint32_t *szt, const int32_t *xsrc, void *gx, char *xpack,
+                   float *partial, int M, int K, int N, int bits, int group_size, const gptq_hip_plan &plan,
+                   void *stream);
 int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int32_t *xsrc, const void *bias, void *y,
                  char *xpack, float *partial, int M, int K, int N, int G, int bits, int group_size,
                  const gptq_hip_plan &plan, void *stream);

@@ -277,6 +277,10 @@ struct TiledParams {
     int rt_total;          // 32-row tiles over all M blocks
     int split_k;
     int lb_per_group;      // group_size / 32
+    // the transposed product only (TRANS): the roles of K and N are swapped, see tiled_gemm_kernel
+    const uint32_t *szt;   // [G][S_total][8 octets][8 words]: per octet of columns, (scale, scale) x 4 | (base + zero) x 4
+    const int32_t *out_map;  // channel of sorted position p (nullptr = identity): where column p of the result goes
+    int tiles_per_group;   // group_size / 32: output tiles (32 positions) per group
 };
 
 // One B operand: positions 8 j .. 8 j + 7 of the lane, as fp16(scale * (q - zero)) exactly as the
@@ -293,12 +297,34 @@ __device__ __forceinline__ h8 tiled_bop(const uint32_t (&w)[BITS], int j, h2 s2,
     return __builtin_bit_cast(h8, o);
 }
 
+// The same for the transposed product, where the eight values of an operand are eight COLUMNS of the layer at one
+// position: scale and (base + zero) differ per value and come as ready-made register pairs.
+template <int BITS>
+__device__ __forceinline__ h8 tiled_bop_t(const uint32_t (&w)[BITS], int j, const u4 &s2, const u4 &zb,
+                                          const uint32_t (&mg)[TileCodec<BITS>::KINDS])
+{
+    u4 q;
+    TileCodec<BITS>::operand(w, j, q, mg);
+    u4 o;
+#pragma unroll
+    for (int r = 0; r < 4; r++) o[r] = as_u32((as_h2(q[r]) - as_h2(zb[r])) * as_h2(s2[r]));
+    return __builtin_bit_cast(h8, o);
+}
+
 // AT: 32-row tiles per wave.  RW x KW: waves of the workgroup along M and along K: the workgroup holds
 // 32 * AT * RW rows, and its KW waves along K split the workgroup's K range.  CT: 32-column tiles per wave (2, or
 // 4 for problems of several row blocks: a fragment of x then feeds four matrix instructions instead of two,
 // which halves the fragment traffic per flop, and the 256 accumulator registers fill the wave's second
 // register file).
-template <int BITS, int AT, int RW, int KW, int RING, int CT>
+// TRANS: gx = gy @ W^T, the gradient of the product with respect to x.  The kernel is handed the tiled format of the
+// TRANSPOSED code matrix (gptq_hip_tile_prepare_transposed): its "positions" are the layer's columns n (the
+// reduction runs over them; x here is gy, packed like any x), its "columns" are the layer's sorted positions p, so
+// a lane holds 32 columns of one position and a column tile (32 positions) lies in one group.  Scale and zero
+// point then differ per value of an operand instead of per lane: the table p.szt holds them as register pairs
+// per octet of columns; the workgroup copies the part of its tiles' groups and of its K range into LDS, and
+// every operand reads its 32 bytes from there, one operand ahead of the arithmetic.  The weights are formed
+// exactly as in the forward product.  The result's column p goes to channel out_map[p].
+template <int BITS, int AT, int RW, int KW, int RING, int CT, bool TRANS = false>
 __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledParams p)
 {
     const int tid = threadIdx.x;
@@ -335,7 +361,7 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
 #pragma unroll
         for (int ct = 0; ct < CT; ct++) {
             tile_load<BITS>(p.qtile + ((size_t)(tile_off[ct] + (uint32_t)Sc) * (256u * BITS) + b_lane), wr[ct]);
-            sr[ct] = p.sz[(size_t)g * p.N + col[ct]];
+            if constexpr (!TRANS) sr[ct] = p.sz[(size_t)g * p.N + col[ct]];
         }
     };
     auto load_a = [&](int S, int j, h8 (&ar)[AT]) {
@@ -354,14 +380,30 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
         return S;
     };
     // prologue, in consumption order
+    int S_of[RING];   // the block each ring slot holds (TRANS: its table entries are looked up by block)
 #pragma unroll
     for (int u = 0; u < RING; u++) {
         const int S = next_block();
+        S_of[u] = S;
         load_b(S, w[u], szr[u]);
 #pragma unroll
         for (int j = 0; j < 4; j++) load_a(S, j, a[u][j]);
     }
     __builtin_amdgcn_sched_barrier(0);
+    // TRANS: the (scale, base + zero) pairs of the workgroup's K range for the groups of its CT tiles -> LDS,
+    // [ct][block of the range][octet][8 words]
+    const int wg_blocks = KW * p.wave_steps;
+    const int S_wg0 = split * wg_blocks;
+    if constexpr (TRANS) {
+        u4 *tbl = (u4 *)smem;
+        for (int i = tid; i < CT * wg_blocks * 16; i += 64 * RW * KW) {
+            const int ct = i / (wg_blocks * 16), r = i - ct * (wg_blocks * 16);
+            const int Sc = min(S_wg0 + (r >> 4), S_last);   // (blocks past K repeat the last one: their x is zero)
+            const int g = min(T0 + ct, p.T_total - 1) / p.tiles_per_group;
+            tbl[i] = *(const u4 *)(p.szt + ((size_t)g * p.S_total + Sc) * 64 + (r & 15) * 4);
+        }
+        __syncthreads();
+    }
 
     f16v acc[AT][CT];
 #pragma unroll
@@ -385,10 +427,25 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
             zb[k] = z2 + (h2){(_Float16)Codec::base(2 * k), (_Float16)Codec::base(2 * k + 1)};  // exact: small integers
     };
 
+    // TRANS: the table entry of (block S, operand j, tile ct) for this lane's half
+    u4 tq_s, tq_z;
+    auto tbl_read = [&](int S, int j, int ct) {
+        const uint32_t off = (uint32_t)(((ct * wg_blocks + (S - S_wg0)) * 8 + 4 * h + j) * 32);
+        tq_s = *(const u4 *)(smem + off);
+        tq_z = *(const u4 *)(smem + off + 16);
+    };
+
     // the first operand of the walk
     h2 cs[CT], czb[CT][KINDS];  // (scale, base + zero) of the block being dequantised, per column tile
-    consts_of(szr[0][0], cs[0], czb[0]);
-    h8 bop_next = tiled_bop<BITS>(w[0][0], 0, cs[0], czb[0], mg);
+    h8 bop_next;
+    if constexpr (TRANS) {
+        tbl_read(S_of[0], 0, 0);
+        bop_next = tiled_bop_t<BITS>(w[0][0], 0, tq_s, tq_z, mg);
+        tbl_read(S_of[0], CT > 1 ? 0 : 1, CT > 1 ? 1 : 0);   // the entry of the operand after it
+    } else {
+        consts_of(szr[0][0], cs[0], czb[0]);
+        bop_next = tiled_bop<BITS>(w[0][0], 0, cs[0], czb[0], mg);
+    }
 
     // One block of the walk (ring slot u): the 4 CT (j, ct) operands, each multiplied with the AT row tiles
     // while the next operand of the walk is dequantised.  REFILL: the slot's registers are requested again
@@ -407,9 +464,19 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
                     const int ctn = ct == CT - 1 ? 0 : ct + 1;
                     constexpr int u1 = (u + 1) % RING;
                     const bool wrap_u = ct == CT - 1 && j == 3;
-                    if (jn == 0) consts_of(wrap_u ? szr[u1][ctn] : szr[u][ctn], cs[ctn], czb[ctn]);  // first operand of a block
-                    bop_next = wrap_u ? tiled_bop<BITS>(w[u1][ctn], jn, cs[ctn], czb[ctn], mg)
-                                      : tiled_bop<BITS>(w[u][ctn], jn, cs[ctn], czb[ctn], mg);
+                    if constexpr (TRANS) {
+                        // tq_* hold the entry of the next operand; then the entry of the one after it is requested
+                        bop_next = wrap_u ? tiled_bop_t<BITS>(w[u1][ctn], jn, tq_s, tq_z, mg)
+                                          : tiled_bop_t<BITS>(w[u][ctn], jn, tq_s, tq_z, mg);
+                        const int i2 = j * CT + ct + 2;
+                        const bool wrap2 = i2 >= 4 * CT;
+                        const int i2w = wrap2 ? i2 - 4 * CT : i2;
+                        tbl_read(wrap2 ? S_of[u1] : S_of[u], i2w / CT, i2w % CT);
+                    } else {
+                        if (jn == 0) consts_of(wrap_u ? szr[u1][ctn] : szr[u][ctn], cs[ctn], czb[ctn]);  // first operand of a block
+                        bop_next = wrap_u ? tiled_bop<BITS>(w[u1][ctn], jn, cs[ctn], czb[ctn], mg)
+                                          : tiled_bop<BITS>(w[u][ctn], jn, cs[ctn], czb[ctn], mg);
+                    }
                 }
 #pragma unroll
                 for (int rt = 0; rt < AT; rt++) {
@@ -417,7 +484,10 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
                 }
                 if (REFILL && ct == CT - 1) {
                     __builtin_amdgcn_sched_barrier(0);
-                    if (j == 3) load_b(S_refill, w[u], szr[u]);  // (its last reader, the last operand of the block, is done)
+                    if (j == 3) {
+                        load_b(S_refill, w[u], szr[u]);  // (its last reader, the last operand of the block, is done)
+                        S_of[u] = S_refill;
+                    }
                     load_a(S_refill, j, a[u][j]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -447,6 +517,7 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
     const _Float16 *bias = (const _Float16 *)p.bias;
     _Float16 *y = (_Float16 *)p.y;
     constexpr int NT = 64 * RW * KW;
+    if constexpr (TRANS) __syncthreads();   // the table shares this memory: every wave is done reading it
 #pragma unroll
     for (int rp = 0; rp < AT; rp += EP) {
         if (rp > 0) __syncthreads();   // the previous pass has been read
@@ -478,7 +549,13 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
             const int T = T0 + ct;
             if (row < p.M && T < p.T_total) {
                 const size_t o = (size_t)row * p.N + 32 * T + nn;
-                if (p.split_k == 1) {
+                if (TRANS && p.split_k == 1 && p.out_map) {
+                    // (the reduce pass of a split applies the map itself)
+                    const int4 dst = *(const int4 *)(p.out_map + 32 * T + nn);
+                    const int d[4] = {dst.x, dst.y, dst.z, dst.w};
+#pragma unroll
+                    for (int c = 0; c < 4; c++) y[(size_t)row * p.N + min(max(d[c], 0), p.N - 1)] = (_Float16)sum[c];
+                } else if (p.split_k == 1) {
                     if (bias) {
                         const h4 b4 = *(const h4 *)(bias + 32 * T + nn);
 #pragma unroll
@@ -1174,7 +1251,8 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
 
 // y = fp16(sum over split of partial[split] (+ bias)), four columns per thread, in split order.
 __global__ __launch_bounds__(256) void tiled_reduce_kernel(const float *__restrict__ partial, const _Float16 *bias,
-                                                           _Float16 *__restrict__ y, int M, int N, int split_k)
+                                                           _Float16 *__restrict__ y, int M, int N, int split_k,
+                                                           const int32_t *__restrict__ out_map = nullptr)
 {
     const uint32_t q = blockIdx.x * 256u + threadIdx.x;
     const uint32_t nq = (uint32_t)N / 4u;
@@ -1187,6 +1265,13 @@ __global__ __launch_bounds__(256) void tiled_reduce_kernel(const float *__restri
         sum = (f4){(float)b4[0], (float)b4[1], (float)b4[2], (float)b4[3]};
     }
     for (int s = 0; s < split_k; s++) sum += *(const f4 *)(partial + ((size_t)s * M + row) * N + c);
+    if (out_map) {   // the transposed product: column c is a sorted position, its channel is out_map[c]
+        const int4 dst = *(const int4 *)(out_map + c);
+        const int d[4] = {dst.x, dst.y, dst.z, dst.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) y[(size_t)row * N + min(max(d[e], 0), N - 1)] = (_Float16)sum[e];
+        return;
+    }
     h4 o;
 #pragma unroll
     for (int e = 0; e < 4; e++) o[e] = (_Float16)sum[e];
@@ -1232,6 +1317,9 @@ int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int
     p.rt_total = plan.row_tiles * plan.m_blocks;
     p.split_k = plan.split_k;
     p.lb_per_group = group_size / 32;
+    p.szt = nullptr;
+    p.out_map = nullptr;
+    p.tiles_per_group = 1;
     const int S_pack = tiled_pack_blocks(plan.split_k, plan.waves_k, plan.k_chunk);
     const int pack_lds = xsrc ? K * 2 : 0;  // one row of x
     if (pack_lds > 65536) {
@@ -1281,6 +1369,177 @@ int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int
     return GPTQ_HIP_OK;
 }
 
+
+// ---------------------------------------------------------------------------------------------------
+// The transposed product gx[M, K] = gy[M, N] @ W^T.
+// Preparation: the tiled format of the transposed code matrix (a lane holds, for sorted position
+// p = 32 T + lane % 32, the codes of columns 64 S + 32 (lane / 32) .. + 31; columns past N are zeros), and the table
+// of (scale, base + zero) register pairs per group and octet of columns.
+// ---------------------------------------------------------------------------------------------------
+template <int BITS>
+__global__ __launch_bounds__(256) void tile_retile_t_kernel(const uint32_t *__restrict__ qweight,
+                                                            const int32_t *__restrict__ xsrc, uint32_t *__restrict__ qtile,
+                                                            int K, int N, int S_total, int T_total)
+{
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    const int lane = t & 63;
+    const uint32_t blk = t >> 6;  // T * S_total + S
+    if (blk >= (uint32_t)T_total * (uint32_t)S_total) return;
+    const int T = blk / S_total, S = blk - T * S_total;
+    const int pos = 32 * T + (lane & 31), h = lane >> 5;
+    int src = xsrc ? xsrc[pos] : pos;
+    src = min(max(src, 0), K - 1);   // a bad map must not fault
+    const uint32_t *b = qweight + (size_t)(src >> 5) * BITS * N;   // the packed block of 32 channels
+    const int bit = BITS * (src & 31);
+    const int wd = bit >> 5, sh = bit & 31;
+    uint32_t words[BITS];
+#pragma unroll
+    for (int i = 0; i < BITS; i++) words[i] = 0u;
+    for (int s = 0; s < 32; s++) {
+        const int n = 64 * S + 32 * h + s;
+        uint32_t q = 0u;
+        if (n < N) {
+            q = b[(size_t)wd * N + n] >> sh;
+            if (sh + BITS > 32) q |= b[(size_t)(wd + 1) * N + n] << (32 - sh);
+            q &= (1u << BITS) - 1u;
+        }
+        const int obit = BITS * TileCodec<BITS>::field(s);
+        const int owd = obit >> 5, osh = obit & 31;
+        words[owd] |= q << osh;
+        if (osh + BITS > 32) words[owd + 1] |= q >> (32 - osh);
+    }
+#pragma unroll
+    for (int i = 0; i < BITS; i++) {
+        const int at = BITS == 8 ? (i >> 2) * 256 + lane * 4 + (i & 3) : lane * BITS + i;
+        qtile[(size_t)blk * (64 * BITS) + at] = words[i];
+    }
+}
+
+// szt[g][o] for octet o of columns (8 o .. 8 o + 7): words 0..3 = (scale, scale) of columns (8 o + 2 r, 8 o + 2 r + 1),
+// words 4..7 = (base + zero) of the same, with the bases of the register unpack; columns past N: zeros.
+template <int BITS>
+__global__ __launch_bounds__(256) void tile_szt_kernel(const uint32_t *__restrict__ qzeros,
+                                                       const _Float16 *__restrict__ scales, uint32_t *__restrict__ szt,
+                                                       int N, int G, int octets)
+{
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= (uint32_t)G * (uint32_t)octets) return;
+    const int g = t / octets, o = t - g * octets;
+    uint32_t out[8];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        h2 s2 = {(_Float16)0, (_Float16)0}, zb = {(_Float16)0, (_Float16)0};
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const int n = 8 * o + 2 * r + e;
+            if (n < N) {
+                s2[e] = scales[(size_t)g * N + n];
+                zb[e] = (_Float16)((float)zero_of<BITS>(qzeros + (size_t)g * (N / 32 * BITS), n) + TileCodec<BITS>::base(2 * r + e));
+            }
+        }
+        out[r] = as_u32(s2);
+        out[4 + r] = as_u32(zb);
+    }
+    u4 *dst = (u4 *)(szt + (size_t)t * 8);
+    dst[0] = (u4){out[0], out[1], out[2], out[3]};
+    dst[1] = (u4){out[4], out[5], out[6], out[7]};
+}
+
+int launch_tile_prepare_t(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *xsrc,
+                          uint32_t *qtile_t, uint32_t *szt, int K, int N, int G, int bits, void *stream_v)
+{
+    hipStream_t stream = (hipStream_t)stream_v;
+    const int S_total = (N + 63) / 64, T_total = K / 32;
+    const unsigned threads = (unsigned)T_total * (unsigned)S_total * 64u;
+    const unsigned tbl = (unsigned)G * (unsigned)S_total * 8u;
+    auto go = [&](auto bits_c) {
+        constexpr int B = decltype(bits_c)::value;
+        hipLaunchKernelGGL(tile_retile_t_kernel<B>, dim3((threads + 255u) / 256u), dim3(256), 0, stream, qweight, xsrc,
+                           qtile_t, K, N, S_total, T_total);
+        hipLaunchKernelGGL(tile_szt_kernel<B>, dim3((tbl + 255u) / 256u), dim3(256), 0, stream, qzeros,
+                           (const _Float16 *)scales, szt, N, G, S_total * 8);
+    };
+    switch (bits) {
+        case 2: go(std::integral_constant<int, 2>{}); break;
+        case 3: go(std::integral_constant<int, 3>{}); break;
+        case 4: go(std::integral_constant<int, 4>{}); break;
+        case 8: go(std::integral_constant<int, 8>{}); break;
+        default: return GPTQ_HIP_ERR_BAD_ARG;
+    }
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+}
+
+template <int BITS, int AT>
+static int launch_tiled_t_one(const TiledParams &p, const gptq_hip_plan &plan, hipStream_t stream)
+{
+    auto kern = tiled_gemm_kernel<BITS, AT, 1, 4, tiled_ring(AT), 2, true>;
+    if (plan.lds_bytes < tiled_t_lds_bytes(AT, 4, plan.k_chunk) || plan.waves_k != 4 || plan.block != 256) return GPTQ_HIP_ERR_BAD_ARG;
+    if (plan.lds_bytes > 65536) {
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, plan.lds_bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return GPTQ_HIP_ERR_LAUNCH;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, plan.grid_z), dim3(256), plan.lds_bytes, stream, p);
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+}
+
+// gy is packed into the workspace (as x is for the forward product), the matmul runs on the transposed copy, and a
+// reduce pass follows when the reduction over N is split over workgroups.
+int launch_tiled_t(const void *gy, const void *qtile_t, const uint32_t *szt, const int32_t *xsrc, void *gx, char *xpack,
+                   float *partial, int M, int K, int N, int bits, int group_size, const gptq_hip_plan &plan,
+                   void *stream_v)
+{
+    hipStream_t stream = (hipStream_t)stream_v;
+    const int Np = (N + 63) / 64 * 64;
+    TiledParams p;
+    p.xpack = xpack;
+    p.qtile = (const char *)qtile_t;
+    p.sz = nullptr;
+    p.bias = nullptr;
+    p.y = gx;
+    p.partial = partial;
+    p.M = M;
+    p.N = K;                 // the result has K columns
+    p.G = K / group_size;
+    p.S_total = Np / 64;     // the reduction runs over the layer's N columns
+    p.T_total = K / 32;
+    p.wave_steps = plan.k_chunk;
+    p.rt_total = plan.row_tiles * plan.m_blocks;
+    p.split_k = plan.split_k;
+    p.lb_per_group = 1;
+    p.szt = szt;
+    p.out_map = xsrc;
+    p.tiles_per_group = group_size / 32;
+    const int S_pack = tiled_pack_blocks(plan.split_k, plan.waves_k, plan.k_chunk);
+    hipLaunchKernelGGL(tile_pack_x_kernel, dim3(32 * p.rt_total), dim3(256), 0, stream, (const _Float16 *)gy,
+                       (const int32_t *)nullptr, xpack, M, N, Np, p.rt_total, S_pack);
+    if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ERR_LAUNCH;
+    int rc = GPTQ_HIP_ERR_UNSUPPORTED;
+#define GPTQ_TILED_T_CASE(B, A) \
+    if (bits == B && plan.row_tiles == A) rc = launch_tiled_t_one<B, A>(p, plan, stream)
+    GPTQ_TILED_T_CASE(2, 1);
+    GPTQ_TILED_T_CASE(2, 2);
+    GPTQ_TILED_T_CASE(2, 4);
+    GPTQ_TILED_T_CASE(3, 1);
+    GPTQ_TILED_T_CASE(3, 2);
+    GPTQ_TILED_T_CASE(3, 4);
+    GPTQ_TILED_T_CASE(4, 1);
+    GPTQ_TILED_T_CASE(4, 2);
+    GPTQ_TILED_T_CASE(4, 4);
+    GPTQ_TILED_T_CASE(8, 1);
+    GPTQ_TILED_T_CASE(8, 2);
+    GPTQ_TILED_T_CASE(8, 4);
+#undef GPTQ_TILED_T_CASE
+    if (rc != GPTQ_HIP_OK) return rc;
+    if (plan.split_k > 1) {
+        const uint32_t quads = (uint32_t)M * ((uint32_t)K / 4u);
+        hipLaunchKernelGGL(tiled_reduce_kernel, dim3((quads + 255u) / 256u), dim3(256), 0, stream, partial,
+                           (const _Float16 *)nullptr, (_Float16 *)gx, M, K, plan.split_k, xsrc);
+        if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ERR_LAUNCH;
+    }
+    return GPTQ_HIP_OK;
+}
 
 template <int BITS, int MR, int KW, int E>
 static int launch_decode_one(const DecodeParams &p, const gptq_hip_plan &plan, hipStream_t stream)

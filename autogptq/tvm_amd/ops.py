@@ -267,6 +267,76 @@ def gemm_tiled(x: torch.Tensor, qtile: torch.Tensor, sz: torch.Tensor, xsrc: Opt
     return out
 
 
+def tile_prepare_transposed(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
+                            xsrc: Optional[torch.Tensor], bits: int, group_size: int):
+    """``pack.tile_layout_transposed`` on the library's own kernels (gptq_hip_tile_prepare_transposed): the copy the
+    transposed product runs on, ``(qtile_t int32 1-D, szt int32 [G, ceil64(N) / 8, 8])``.  ``xsrc``: the map
+    ``tile_prepare`` returned for the layer (the channel at each sorted position), None without an activation
+    order."""
+    _need_gpu("qweight", qweight, torch.int32)
+    _need_gpu("qzeros", qzeros, torch.int32)
+    _need_gpu("scales", scales, torch.float16)
+    K, N, G = check_shapes(qweight, qzeros, scales, None, None, bits, group_size, widths=FORMAT_BITS)
+    if xsrc is not None:
+        _need_gpu("xsrc", xsrc, torch.int32)
+        if tuple(xsrc.shape) != ((K + 63) // 64 * 64,):
+            raise ValueError(f"xsrc must be [{(K + 63) // 64 * 64}], got {tuple(xsrc.shape)}")
+    dev = qweight.device
+    lib = _lib.lib()
+    qtile_t = torch.empty(lib.gptq_hip_tiled_transposed_bytes(K, N, bits) // 4, dtype=torch.int32, device=dev)
+    szt = torch.empty((G, (N + 63) // 64 * 8, 8), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.gptq_hip_tile_prepare_transposed(_ptr(qweight), _ptr(qzeros), _ptr(scales), _ptr(xsrc), _ptr(qtile_t),
+                                                  _ptr(szt), K, N, bits, group_size, _stream(dev))
+    if rc != _lib.OK:
+        raise _lib.GptqHipError(rc, f"gptq_hip_tile_prepare_transposed(K={K}, N={N}, bits={bits}, "
+                                    f"group_size={group_size})")
+    return qtile_t, szt
+
+
+def gemm_tiled_transposed(gy: torch.Tensor, qtile_t: torch.Tensor, szt: torch.Tensor, xsrc: Optional[torch.Tensor],
+                          K: int, bits: int, group_size: int, plan: Optional[_lib.Plan] = None,
+                          out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """gx[M, K] fp16 = gy[M, N] @ W^T on the transposed tiled copy (``tile_prepare_transposed``): the gradient of
+    ``y = x @ W`` with respect to x (the reference's transpose_matmul248, qlinear_triton.py:298-317); gy and gx in
+    the layer's own channel order."""
+    _need_gpu("gy", gy, torch.float16)
+    _need_gpu("qtile_t", qtile_t, torch.int32)
+    _need_gpu("szt", szt, torch.int32)
+    if xsrc is not None:
+        _need_gpu("xsrc", xsrc, torch.int32)
+    if gy.dim() != 2 or szt.dim() != 3:
+        raise ValueError("gy must be [M, N] and szt [G, ceil64(N) / 8, 8]")
+    M, N = gy.shape
+    Np = (N + 63) // 64 * 64
+    gs = K if group_size == -1 else group_size
+    if K % 32 != 0 or N % 32 != 0 or K % gs != 0:
+        raise ValueError(f"a {K} x {N} layer with groups of {gs} is not one the tiled format covers")
+    if qtile_t.numel() * 4 != K * Np * bits // 8:
+        raise ValueError(f"qtile_t holds {qtile_t.numel() * 4} bytes, a {K} x {N} layer of {bits} bits needs "
+                         f"{K * Np * bits // 8}")
+    if tuple(szt.shape) != (K // gs, Np // 8, 8):
+        raise ValueError(f"szt must be [{K // gs}, {Np // 8}, 8], got {tuple(szt.shape)}")
+    if xsrc is not None and tuple(xsrc.shape) != ((K + 63) // 64 * 64,):
+        raise ValueError(f"xsrc must be [{(K + 63) // 64 * 64}], got {tuple(xsrc.shape)}")
+    dev = gy.device
+    if out is None:
+        out = torch.empty((M, K), dtype=torch.float16, device=dev)
+    if M == 0:
+        return out
+    if plan is None:
+        plan = _lib.select_tiled_transposed(M, K, N, bits, group_size)
+    ws = _workspace(dev, plan.workspace_bytes)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().gptq_hip_gemm_tiled_transposed(_ptr(gy), _ptr(qtile_t), _ptr(szt), _ptr(xsrc), _ptr(out), _ptr(ws),
+                                                       ws.numel(), M, K, N, bits, group_size, ctypes.byref(plan),
+                                                       _stream(dev))
+    if rc != _lib.OK:
+        raise _lib.GptqHipError(rc, f"gptq_hip_gemm_tiled_transposed(M={M}, K={K}, N={N}, bits={bits}, "
+                                    f"group_size={group_size})")
+    return out
+
+
 def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
     """Where the tiled kernels were measured faster than the ones that read the checkpoint layout (or its
     sorted copy), on MI355X with the weights cold, group size 128 (us, graph replay):

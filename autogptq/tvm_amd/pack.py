@@ -196,21 +196,8 @@ def tile_layout(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tenso
         if not torch.equal(g[perm], ar // gs):
             return None
     Kp = (K + TILE_CHANNELS - 1) // TILE_CHANNELS * TILE_CHANNELS
-    S, T = Kp // TILE_CHANNELS, N // TILE_COLS
     codes = unpack_rows_torch(qweight.detach(), bits)[perm]                      # [K, N], sorted order
-    if Kp > K:
-        codes = torch.cat([codes, torch.zeros((Kp - K, N), dtype=codes.dtype, device=dev)])
-    # stream field f of a lane holds the position order[f]
-    field_of = _slots.lane_field_of_position(bits)
-    order = torch.empty(32, dtype=torch.int64, device=dev)
-    order[torch.tensor(field_of, dtype=torch.int64, device=dev)] = torch.arange(32, device=dev)
-    blocks = codes.view(S * 2, 32, N)[:, order, :]                                # [(S, h), field, N]
-    words = pack_rows_torch(blocks.reshape(S * 2 * 32, N), bits)                  # [(S, h, word), N]
-    words = words.view(S, 2, bits, T, TILE_COLS)
-    if bits == 8:   # [T, S, word // 4, (h, n), word % 4]
-        qtile = words.view(S, 2, 2, 4, T, TILE_COLS).permute(4, 0, 2, 1, 5, 3).contiguous().view(-1)
-    else:           # [T, S, (h, n), word]
-        qtile = words.permute(3, 0, 1, 4, 2).contiguous().view(-1)
+    qtile = _tile_words(codes, bits)
     zeros = unpack_rows_torch(qzeros.detach().t().contiguous(), bits).t() + 1     # [G, N]
     zbits = zeros.to(torch.float16).view(torch.int16).to(torch.int64) & 0xFFFF
     sbits = scales.detach().contiguous().view(torch.int16).to(torch.int64) & 0xFFFF
@@ -222,6 +209,82 @@ def tile_layout(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tenso
     inv[perm] = ar
     kinv = torch.where(inv >= (1 << 15), inv - (1 << 16), inv).to(torch.int16)   # unsigned 16-bit positions
     return qtile, sz, xsrc, kinv
+
+
+def _tile_words(codes: torch.Tensor, bits: int) -> torch.Tensor:
+    """The blocks of the tiled format for a code matrix [positions, columns] (columns a multiple of 32; the
+    positions are padded with zero codes to a multiple of 64): int32, 1-D."""
+    from . import _slots
+
+    P, C = codes.shape
+    dev = codes.device
+    Pp = (P + TILE_CHANNELS - 1) // TILE_CHANNELS * TILE_CHANNELS
+    S, T = Pp // TILE_CHANNELS, C // TILE_COLS
+    if Pp > P:
+        codes = torch.cat([codes, torch.zeros((Pp - P, C), dtype=codes.dtype, device=dev)])
+    # stream field f of a lane holds the position order[f]
+    field_of = _slots.lane_field_of_position(bits)
+    order = torch.empty(32, dtype=torch.int64, device=dev)
+    order[torch.tensor(field_of, dtype=torch.int64, device=dev)] = torch.arange(32, device=dev)
+    blocks = codes.reshape(S * 2, 32, C)[:, order, :]                             # [(S, h), field, C]
+    words = pack_rows_torch(blocks.reshape(S * 2 * 32, C), bits)                  # [(S, h, word), C]
+    words = words.view(S, 2, bits, T, TILE_COLS)
+    if bits == 8:   # [T, S, word // 4, (h, n), word % 4]
+        return words.view(S, 2, 2, 4, T, TILE_COLS).permute(4, 0, 2, 1, 5, 3).contiguous().view(-1)
+    return words.permute(3, 0, 1, 4, 2).contiguous().view(-1)                     # [T, S, (h, n), word]
+
+
+def tile_layout_transposed(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor, g_idx, bits: int,
+                           group_size: int):
+    """The second prepared copy, for the transposed product gx = gy @ W^T (the gradient with respect to x; the
+    reference's Triton back end, auto_gptq/nn_modules/qlinear_triton.py:195-273,298-317), in torch ops: the
+    statement ``gptq_hip_tile_prepare_transposed`` is tested against.
+
+    Returns ``(qtile_t int32 [K/32 * Np/64 * 64 * bits], szt int32 [G, Np/8, 8])`` with Np = N rounded up to 64,
+    or None when the tiled format does not cover the layer.
+
+    * ``qtile_t`` is the tiled format of the TRANSPOSED code matrix: its positions are the layer's columns n (padded
+      with zero codes to Np), its columns are the layer's sorted positions p; block (T, S) holds, in lane
+      (lane % 32, h), the codes of position 32 T + lane % 32 at columns 64 S + 32 h .. + 31.
+    * ``szt[g, o]``, for the octet of columns 8 o .. 8 o + 7: words r = 0..3 are the fp16 pairs
+      (scale[g, 8 o + 2 r], scale[g, 8 o + 2 r + 1]), words 4 + r the pairs (base + zero) of the same columns, with
+      the bases of the register unpack (``_slots.BASE_OF_POSITION``); zeros for columns past N.
+    """
+    from . import _slots
+
+    rows, N = qweight.shape
+    K = rows * 32 // bits
+    if not tiled_qualifies(K, N, bits, group_size):
+        return None
+    gs = K if group_size == -1 else group_size
+    dev = qweight.device
+    ar = torch.arange(K, dtype=torch.int64, device=dev)
+    if g_idx is None:
+        perm = ar
+    else:
+        g = g_idx.detach().to(device=dev, dtype=torch.int64)
+        perm = torch.argsort(g, stable=True)
+        if not torch.equal(g[perm], ar // gs):
+            return None
+    codes = unpack_rows_torch(qweight.detach(), bits)[perm]                      # [K, N], sorted order
+    qtile_t = _tile_words(codes.t().contiguous(), bits)
+    G = K // gs
+    Np = (N + 63) // 64 * 64
+    zeros = (unpack_rows_torch(qzeros.detach().t().contiguous(), bits).t() + 1).to(torch.float32)   # [G, N]
+    base = torch.tensor(_slots.BASE_OF_POSITION[bits], dtype=torch.float32, device=dev).repeat(N // 8)
+    zb = (zeros + base[None, :]).to(torch.float16)                               # exact: small integers
+    s = scales.detach().contiguous()
+
+    def pairs(v):   # fp16 [G, N] -> int64 [G, Np/8, 4]: (v[2 i], v[2 i + 1]) as one word
+        bits16 = v.view(torch.int16).to(torch.int64) & 0xFFFF
+        if Np > N:
+            bits16 = torch.cat([bits16, torch.zeros((G, Np - N), dtype=torch.int64, device=dev)], dim=1)
+        b = bits16.view(G, Np // 8, 4, 2)
+        return b[..., 0] | (b[..., 1] << 16)
+
+    both = torch.cat([pairs(s), pairs(zb)], dim=2)                               # [G, Np/8, 8]
+    szt = torch.where(both >= (1 << 31), both - (1 << 32), both).to(torch.int32).contiguous()
+    return qtile_t, szt
 
 
 def num_groups(k: int, group_size: int) -> int:

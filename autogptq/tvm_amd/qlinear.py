@@ -20,10 +20,11 @@ from .pack import pack_qweight, pack_qzeros, tiled_qualifies
 
 
 class _ProductWithInputGrad(torch.autograd.Function):
-    """The product with a gradient for x (the packed weights are constants): grad_x = grad_y @ W^T on
-    the dequantised weight, which is what the reference's Triton back end offers for training on top
-    of quantised layers (auto_gptq/nn_modules/qlinear_triton.py:195-273), here with the HIP dequant
-    kernel and the library GEMM."""
+    """The product with a gradient for x (the packed weights are constants): grad_x = grad_y @ W^T, which
+    is what the reference's Triton back end offers for training on top of quantised layers
+    (auto_gptq/nn_modules/qlinear_triton.py:195-273,298-336): fused on the transposed tiled copy
+    (``QuantLinear.grad_input``), or the HIP dequant kernel and the library GEMM for long batches and
+    layers the format does not cover."""
 
     @staticmethod
     def forward(ctx, x2, layer):
@@ -32,8 +33,7 @@ class _ProductWithInputGrad(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_out):
-        w = ctx.layer.dequantize()                                   # [K, N] fp16
-        return torch.matmul(grad_out.to(w.dtype), w.t()), None
+        return ctx.layer.grad_input(grad_out), None
 
 
 class QuantLinear(nn.Module):
@@ -90,6 +90,8 @@ class QuantLinear(nn.Module):
         # the checkpoint's tensors (and the sorted copy) only.  compact() makes it the only copy.
         self.tile_for_prefill = tile_for_prefill
         self._tiled = None    # (key, (qtile, sz, xsrc, kinv) or None)
+        self._tiled_t = None  # (key, (qtile_t, szt, xsrc) or None): the copy the gradient for x runs on
+        self.grad_switch_threshold = 384   # rows of grad_y from which the gradient for x takes the library GEMM
         self._compact = False
         self._routes = {}     # M -> (watched buffers, sum of their versions, path name, fn(x2)): see _route
 
@@ -188,6 +190,47 @@ class QuantLinear(nn.Module):
             self._tiled = (key, tensors)
         return self._tiled[1]
 
+    def prepare_transposed(self):
+        """Builds (once per distinct storage of the packed tensors) the copy the transposed product runs on;
+        returns ``(qtile_t, szt, xsrc)`` or None when the tiled format does not cover the layer.  A compact layer
+        keeps the copy it had when it was compacted (its checkpoint tensors are gone)."""
+        if self._compact:
+            return None if self._tiled_t is None else self._tiled_t[1]
+        tiled = self.prepare_tiled()
+        if tiled is None:
+            return None
+        key = self._tiled[0]
+        if self._tiled_t is None or self._tiled_t[0] != key:
+            xsrc = tiled[2] if self._kernel_g_idx() is not None else None
+            qtile_t, szt = ops.tile_prepare_transposed(self.qweight, self.qzeros, self.scales, xsrc, self.bits,
+                                                       self.groupsize)
+            self._tiled_t = (key, (qtile_t, szt, xsrc))
+        return self._tiled_t[1]
+
+    def grad_input(self, grad_out: torch.Tensor) -> torch.Tensor:
+        """grad_out[..., outfeatures] @ W^T: below the switch to the library GEMM the fused transposed product
+        (gptq_hip_gemm_tiled_transposed), else W from the dequant kernel and the library GEMM."""
+        gy = grad_out.reshape(-1, self.outfeatures)
+        if gy.dtype != torch.float16:
+            gy = gy.half()
+        if not gy.is_contiguous():
+            gy = gy.contiguous()
+        M = gy.size(0)
+        # Measured on MI355X (us, eager, int4 with an activation order; fused against dequant + library GEMM):
+        # 4096 x 11008: 22 / 64 at 16 rows, 37 / 90 at 128, 140 / 102 at 512; 11008 x 4096: 35 / 66 at 128,
+        # 106 / 89 at 512; 4096 x 4096: 27 / 44 at 128, 46 / 47 at 512.
+        threshold = self.kernel_switch_threshold
+        if threshold:
+            threshold = min(threshold, self.grad_switch_threshold)
+        gx = None
+        if self.tile_for_prefill and gy.is_cuda and M > 0 and not (threshold and M >= threshold):
+            t = self.prepare_transposed()
+            if t is not None:
+                gx = ops.gemm_tiled_transposed(gy, t[0], t[1], t[2], self.infeatures, self.bits, self.groupsize)
+        if gx is None:
+            gx = torch.matmul(gy, self.dequantize().t())
+        return gx.reshape(grad_out.shape[:-1] + (self.infeatures,))
+
     def compact(self):
         """Keeps the tiled copy as the layer's ONLY weights: every row count then runs on the tiled kernels and
         the checkpoint's tensors are released (empty buffers stay in their place, so ``state_dict`` no longer
@@ -201,6 +244,8 @@ class QuantLinear(nn.Module):
         self._tiled = (None, tensors if act else (tensors[0], tensors[1], None, None))
         self._compact = True
         self._sorted = None
+        if self._tiled_t is not None:   # a copy for the gradient that exists stays with the layer
+            self._tiled_t = (None, self._tiled_t[1])
         dev = self.qweight.device
         self.qweight = torch.empty((0, self.outfeatures), dtype=torch.int32, device=dev)
         self.qzeros = torch.empty((0, self.qzeros.shape[1]), dtype=torch.int32, device=dev)
@@ -214,6 +259,8 @@ class QuantLinear(nn.Module):
         self._routes.clear()
         if self._compact:
             self._tiled = (None, tuple(None if t is None else fn(t) for t in self._tiled[1]))
+            if self._tiled_t is not None and self._tiled_t[1] is not None:
+                self._tiled_t = (None, tuple(None if t is None else fn(t) for t in self._tiled_t[1]))
         return self
 
     def _sorted_tensors(self, M):

@@ -222,6 +222,32 @@ int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint32_t *sz, co
                         int bits, int group_size, const gptq_hip_plan *plan, void *stream);
 
 /*
+ * The transposed product gx[M, K] = gy[M, N] @ W^T: the gradient of y = x @ W with respect to x, for training on
+ * top of frozen quantised layers (the reference's Triton back end: transpose_matmul_248_kernel and
+ * transpose_matmul248, auto_gptq/nn_modules/qlinear_triton.py:195-273,298-317, used by its backward, :329-336).  It
+ * runs the matmul kernel on a
+ * second prepared copy, the tiled format of the transposed code matrix:
+ *   qtile_t  gptq_hip_tiled_transposed_bytes(K, N, bits) bytes, 16-byte aligned: blocks of 64 lanes x `bits` words, tile
+ *            of 32 sorted positions outermost, then block of 64 columns; lane (lane % 32, h = lane / 32) holds, for
+ *            position 32 T + lane % 32, the codes of columns 64 S + 32 h .. + 31 (zeros past N)
+ *   szt      gptq_hip_tiled_transposed_table_bytes(K, N, group_size) bytes, 16-byte aligned: per group and octet of
+ *            columns, four (scale, scale) and four (base + zero) fp16 pairs in the order of the register unpack
+ * gptq_hip_tile_prepare_transposed writes both (two launches).  xsrc: the map of gptq_hip_tile_prepare (the channel at
+ * each sorted position), NULL without an activation order; gy and gx are in the layer's own channel order.  The
+ * weights are formed exactly as in the forward product (fp16(scale * (q - zero)), one rounding), sums are fp32.
+ * plan: NULL = gptq_hip_select_tiled_transposed.  workspace: plan.workspace_bytes, zeroed once.
+ */
+size_t gptq_hip_tiled_transposed_bytes(int K, int N, int bits);
+size_t gptq_hip_tiled_transposed_table_bytes(int K, int N, int group_size);
+int gptq_hip_tile_prepare_transposed(const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                                     const int32_t *xsrc, void *qtile_t, uint32_t *szt, int K, int N, int bits,
+                                     int group_size, void *stream);
+int gptq_hip_select_tiled_transposed(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan);
+int gptq_hip_gemm_tiled_transposed(const void *gy, const void *qtile_t, const uint32_t *szt, const int32_t *xsrc,
+                                   void *gx, void *workspace, size_t workspace_bytes, int M, int K, int N, int bits,
+                                   int group_size, const gptq_hip_plan *plan, void *stream);
+
+/*
  * W fp16 [K, N] = scales[g] * (q - (zq[g] + 1)), one rounding per element:
  * the materialised weight of qlinear.py:198-242, for the bit-exact check.  bits may also be 2 or 8
  * here (the other widths of the format, qlinear.py:31-32,211-215): without a tiled copy those layers run as

@@ -174,6 +174,9 @@ int main()
     printf("\nslot2");
     for (int i = 0; i < 16; i++) printf(" %d", SLOT2[i]);
     for (int bits : {2, 3, 4, 8}) {
+        printf("\nbase%d", bits);
+        for (int e = 0; e < 8; e++)
+            printf(" %d", (int)(bits == 2 ? TileCodec<2>::base(e) : bits == 3 ? TileCodec<3>::base(e) : bits == 4 ? TileCodec<4>::base(e) : TileCodec<8>::base(e)));
         printf("\nfield%d", bits);
         for (int s = 0; s < 32; s++)
             printf(" %d", bits == 2 ? TileCodec<2>::field(s) : bits == 3 ? TileCodec<3>::field(s) : bits == 4 ? TileCodec<4>::field(s) : TileCodec<8>::field(s));

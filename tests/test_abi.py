@@ -322,3 +322,27 @@ def test_tiled_plans_reject_what_the_format_does_not_cover():
     with pytest.raises(_lib.GptqHipError):
         _lib.select_tiled(5, 4096, 4096, 8, 128, decode=True)             # the decode kernels take up to four rows
     assert _lib.lib().gptq_hip_tiled_bytes(4096, 4096, 5) == 0
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
+@pytest.mark.parametrize("KN", [(4096, 4096), (4096, 11008), (11008, 4096), (96, 32), (9216, 36864), (352, 65536)])
+def test_transposed_plans_are_consistent(bits, KN):
+    """The plans of the transposed product gx[M, K] = gy[M, N] @ W^T: the grid covers the K columns of the result,
+    the waves cover the N columns of the reduction, and the table of a workgroup's range fits its LDS."""
+    K, N = KN
+    gs = 128 if K % 128 == 0 else 32
+    blocks = -(-N // 64)
+    for M in (1, 5, 33, 128, 129, 1024):
+        p = _lib.select_tiled_transposed(M, K, N, bits, gs)
+        assert p.kernel == _lib.KERNEL_TILED and p.waves_n == 1 and p.waves_k == 4 and p.block == 256
+        assert p.grid_x == -(-(K // 32) // 2) and p.grid_z == p.m_blocks and p.m_blocks * p.row_tiles * 32 >= M
+        assert p.split_k == p.grid_y >= 1 and p.split_k * p.waves_k * p.k_chunk >= blocks
+        assert 2 * p.waves_k * p.k_chunk * 256 <= p.lds_bytes <= 160 * 1024
+        assert p.lds_bytes >= p.waves_k * p.row_tiles * 2 * 4096
+        part = (p.split_k * M * K * 4 + 255) // 256 * 256 if p.split_k > 1 else 0
+        assert p.workspace_bytes >= 16384 + part + p.split_k * p.waves_k * p.k_chunk * 4 * p.row_tiles * p.m_blocks * 1024
+    lib = _lib.lib()
+    assert lib.gptq_hip_tiled_transposed_bytes(K, N, bits) == K * blocks * 64 * bits // 8
+    assert lib.gptq_hip_tiled_transposed_table_bytes(K, N, gs) == (K // gs) * blocks * 256
+    with pytest.raises(_lib.GptqHipError):
+        _lib.select_tiled_transposed(1, K, N, bits, 16)

@@ -38,3 +38,4 @@ def test_magic_unpack_matches_bit_extraction(tmp_path):
     # the tiled format's permutation per width, as the kernels' codec states it
     for bits in (2, 3, 4, 8):
         assert lines[f"field{bits}"] == _slots.lane_field_of_position(bits)
+        assert lines[f"base{bits}"] == _slots.BASE_OF_POSITION[bits]
