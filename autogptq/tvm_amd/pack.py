@@ -175,12 +175,10 @@ def tile_layout(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tenso
       column 32 T + n at positions 64 S + 32 h .. + 31 as the usual little-endian stream of ``bits``-bit
       fields, with the codes permuted inside the lane (each 4 / 8 / 16 positions for 8 / 4 / 2 bits, all 32
       for 3 bits) so that the kernels' register unpack yields them in position order: stream field
-      ``lane_field_of_position[s]`` holds position s.  Word i of lane l sits at l * bits + i of the block,
+      ``_slots.lane_field_of_position(bits)[s]`` holds position s.  Word i of lane l sits at l * bits + i of the block,
       except for 8 bits, whose block is two halves of 64 lanes x 4 words: (i // 4) * 256 + l * 4 + i % 4.
     * ``sz[g, n]`` = fp16 bits of ``scales[g, n]`` | fp16 bits of the zero point (stored value + 1) << 16.
     """
-    from . import _slots
-
     rows, N = qweight.shape
     K = rows * 32 // bits
     if not tiled_qualifies(K, N, bits, group_size):
