@@ -143,6 +143,7 @@ FULL = [
     ("int8-4096x11008-act", 8, 4096, 11008, 128, True, [128]),
     ("int2-11008x4096", 2, 11008, 4096, 128, False, [64]),
     ("c5-int3-9216x36864-act-g1", 3, 9216, 36864, -1, True, [32]),
+    ("int4-352x65536-act", 4, 352, 65536, 32, True, [40]),   # a reduction longer than one workgroup's table
 ]
 
 
