@@ -583,9 +583,12 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
 // The dots run on v_mfma_f32_4x4x4_16B_f16: sixteen independent 4-lane blocks, lane 4 b + i supplies
 // row i of A and column i of B of block b, and result register v of lane 4 b + j is row v of column j.
 // A lane of the tiled format holds 32 codes of ONE column, so its unpacked registers are B operands as
-// they are (four positions each), the A operand of lane 4 b + i is x[row i] at the same four positions
-// (read from LDS: rows past M read zeros), and the four result registers of a lane are the rows of its
-// own column: up to four rows of x cost one matrix instruction per four positions.
+// they are (four positions each), the A operand of row i is x[row i] at the same four positions (rows past
+// M are zeros), and the four result registers of a lane are the rows of its own column: up to four rows of
+// x cost one matrix instruction per four positions.  All 4-lane blocks of a half wave share their positions,
+// and the instruction can broadcast the A operand of one block to the others (cbsz / abid): block b of the
+// half keeps positions 4 b .. 4 b + 3 in its A registers and the instruction for positions 4 i .. 4 i + 3
+// names block i, so x costs one 8-byte LDS read per lane and block.
 // Per weight the vector ALU only unpacks (2, 3, 4 bits).
 // The codes enter as (base + q) with the bases of the register unpack; per block of 32 positions the
 // epilogue takes y += scale * (P - Bsum - zero * Xsum), with Xsum = sum x and Bsum = sum x * base of the
@@ -821,21 +824,22 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     for (int m = 0; m < MR; m++) ysum[m] = 0.f;
     // Per-lane byte offsets that never change; what changes per block is wave-uniform and stays in scalar
     // registers.  A lane whose row lies past M reads the 64 zero bytes whatever the block (stride 0).
-    const uint32_t x_base = row_i < p.M ? (uint32_t)(row_i * span + 32 * h) * 2u : zero_off;
+    // The matrix instruction broadcasts A: with cbsz = 3 the eight 4-lane blocks of a half wave all take their A
+    // operand from block `abid` of the half.  So lane block b of a half holds only positions 4 b .. 4 b + 3 of the
+    // half's 32 (one 8-byte read per lane and block instead of 64 bytes), and the instruction for positions
+    // 4 i .. 4 i + 3 names abid = i.
+    const int lb8 = (lane >> 2) & 7;
+    const uint32_t x_base = row_i < p.M ? (uint32_t)(row_i * span + 32 * h + 4 * lb8) * 2u : zero_off;
     const uint32_t x_stride = row_i < p.M ? 128u : 0u;
     const uint32_t xs_lane = zero_off + 64u + (uint32_t)(h * MR) * 8u;   // sums of half h of unit 0
     const uint32_t sz_lane = (uint32_t)((const unsigned char *)szl - smem) + (uint32_t)n * 4u;
 
-    // x of a block: the 32 positions of the lane block, row row_i; read one block ahead of its use
-    auto load_x = [&](uint32_t sb, u4 (&xv)[4]) {
-        const uint32_t xoff = x_base + x_stride * sb;
-#pragma unroll
-        for (int v = 0; v < 4; v++) xv[v] = *(const u4 *)(smem + xoff + 16 * v);
-    };
+    // x of a block: this lane's four positions of row row_i; read one block ahead of its use
+    auto load_x = [&](uint32_t sb, u2 &xv) { xv = *(const u2 *)(smem + x_base + x_stride * sb); };
     f4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};  // two chains: a matrix instruction waits for the one it adds to
     uint32_t szw = 0u;   // (scale, zero) word and sums of the unit in flight, read when the unit starts
     f2 xsv[MR];
-    auto block = [&](auto uu_c, int S, const uint32_t (&wr)[BITS], const u4 (&xc)[4], u4 (&xn)[4]) {
+    auto block = [&](auto uu_c, int S, const uint32_t (&wr)[BITS], const u2 &xc, u2 &xn) {
         constexpr int uu = decltype(uu_c)::value;                 // block inside its unit
         const uint32_t sb = (uint32_t)(S - S_wg);                  // block inside the workgroup's range (wave-uniform)
         if constexpr (uu == 0) {
@@ -865,13 +869,12 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
             c0 = (f4){0.f, 0.f, 0.f, 0.f};
             c1 = (f4){0.f, 0.f, 0.f, 0.f};
         }
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const u2 a0 = {xc[v][0], xc[v][1]}, a1 = {xc[v][2], xc[v][3]};
-            const u2 b0 = {q[v][0], q[v][1]}, b1 = {q[v][2], q[v][3]};
-            c0 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a0), __builtin_bit_cast(h4, b0), c0, 0, 0, 0);
-            c1 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a1), __builtin_bit_cast(h4, b1), c1, 0, 0, 0);
-        }
+        const h4 xa = __builtin_bit_cast(h4, xc);
+        [&]<int... V>(std::integer_sequence<int, V...>) {
+            ((c0 = __builtin_amdgcn_mfma_f32_4x4x4f16(xa, __builtin_bit_cast(h4, (u2){q[V][0], q[V][1]}), c0, 3, 2 * V, 0),
+              c1 = __builtin_amdgcn_mfma_f32_4x4x4f16(xa, __builtin_bit_cast(h4, (u2){q[V][2], q[V][3]}), c1, 3, 2 * V + 1, 0)),
+             ...);
+        }(std::make_integer_sequence<int, 4>{});
         if constexpr (uu == E - 1) {
             if constexpr (EXACT) {
 #pragma unroll
@@ -887,7 +890,7 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
 
     // Chunks of PF blocks, two in flight; x rides one block ahead in two register sets.  Blocks past the end
     // of K inside a wave's range are harmless (their x and sums are zeros), blocks past the range are skipped.
-    u4 xr[2][4];
+    u2 xr[2];
     load_x((uint32_t)(S_begin - S_wg), xr[0]);
     auto chunk = [&](int c, uint32_t (&wc)[PF][BITS], auto all_c) {
         constexpr bool ALL = decltype(all_c)::value;
@@ -1124,20 +1127,25 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     float ysum[MR];
 #pragma unroll
     for (int m = 0; m < MR; m++) ysum[m] = 0.f;
-    // per-lane byte offsets that never change; a lane whose row lies past M reads the 64 zero bytes (stride 0)
-    const uint32_t x_base = row_i < p.M ? (uint32_t)(row_i * span + 32 * lbv) * 2u : zero_off;
+    // per-lane byte offsets that never change; a lane whose row lies past M reads the 64 zero bytes (stride 0).
+    // A is broadcast inside each group of four 4-lane blocks (cbsz = 2), the sixteen lanes that share their 32
+    // positions: block b of a group holds positions 4 b .. 4 b + 3 and 16 + 4 b .. 16 + 4 b + 3 (two 8-byte reads
+    // per lane and item), and the instruction for positions 4 i .. 4 i + 3 takes register set i / 4 with abid = i % 4.
+    const int lb4 = (lane >> 2) & 3;
+    const uint32_t x_base = row_i < p.M ? (uint32_t)(row_i * span + 32 * lbv + 4 * lb4) * 2u : zero_off;
     const uint32_t x_stride = row_i < p.M ? 256u : 0u;
+    const uint32_t x_second = row_i < p.M ? 32u : 0u;   // bytes to positions 16 ..
     const uint32_t xs_lane = zero_off + 64u + (uint32_t)(lbv * MR) * 8u;
     const uint32_t sz_lane = (uint32_t)((const unsigned char *)szl - smem) + (uint32_t)n16 * 8u;
     const uint32_t red_lane = (uint32_t)((const unsigned char *)red - smem) + (uint32_t)lane * 4u;
 
-    auto load_x = [&](int V, u4 (&xv)[4]) {
+    auto load_x = [&](int V, u2 (&xv)[2]) {
         const uint32_t xoff = x_base + x_stride * (uint32_t)V;
-#pragma unroll
-        for (int v = 0; v < 4; v++) xv[v] = *(const u4 *)(smem + xoff + 16 * v);
+        xv[0] = *(const u2 *)(smem + xoff);
+        xv[1] = *(const u2 *)(smem + xoff + x_second);
     };
     int cu = 0, cv = wave;   // (unit, V) of the item being computed
-    auto item = [&](const uint32_t (&wr)[BITS], const u4 (&xc)[4], u4 (&xn)[4]) {
+    auto item = [&](const uint32_t (&wr)[BITS], const u2 (&xc)[2], u2 (&xn)[2]) {
         const int V = cv, ul = cu;
         // this item's scale, zero point and sums
         uint32_t goff;
@@ -1171,13 +1179,12 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
             tiled_dequant_exact<BITS>(q, as_u32(e));
         }
         f4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};  // two chains
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const u2 a0 = {xc[v][0], xc[v][1]}, a1 = {xc[v][2], xc[v][3]};
-            const u2 b0 = {q[v][0], q[v][1]}, b1 = {q[v][2], q[v][3]};
-            c0 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a0), __builtin_bit_cast(h4, b0), c0, 0, 0, 0);
-            c1 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a1), __builtin_bit_cast(h4, b1), c1, 0, 0, 0);
-        }
+        const h4 xa[2] = {__builtin_bit_cast(h4, xc[0]), __builtin_bit_cast(h4, xc[1])};
+        [&]<int... V>(std::integer_sequence<int, V...>) {
+            ((c0 = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[V / 2], __builtin_bit_cast(h4, (u2){q[V][0], q[V][1]}), c0, 2, (2 * V) % 4, 0),
+              c1 = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[V / 2], __builtin_bit_cast(h4, (u2){q[V][2], q[V][3]}), c1, 2, (2 * V + 1) % 4, 0)),
+             ...);
+        }(std::make_integer_sequence<int, 4>{});
         if constexpr (EXACT) {
 #pragma unroll
             for (int m = 0; m < MR; m++) ysum[m] += c0[m] + c1[m];
@@ -1194,7 +1201,7 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
             }
         }
     };
-    u4 xr[2][4];
+    u2 xr[2][2];
     load_x(cv, xr[0]);
     auto chunk = [&](int c, uint32_t (&wc)[PF][BITS], auto all_c) {
         constexpr bool ALL = decltype(all_c)::value;
