@@ -371,6 +371,94 @@ def cpu_baseline(case, budget_s: float = 20.0):
     }
 
 
+def run_transposed(args, dev):
+    """``--transposed``: the gradient for x of the workload's layer, gx[M, K] = gy[M, N] @ W^T
+    (gptq_hip_gemm_tiled_transposed on the transposed tiled copy), timed like a forward step and checked against
+    the oracle's dequantised weight.  One JSON line; no secondary records."""
+    from autogptq.tvm_amd import _lib, ops
+    from autogptq.tvm_amd.pack import synth_layer
+    from oracle import c_oracle
+
+    bits, K, N, gs, desc_act, M = WORKLOADS[args.workload]
+    L = synth_layer(2000 + sorted(WORKLOADS).index(args.workload), K, N, bits, gs, desc_act, M=1)
+    qz, sc = L["qzeros"].to(dev), L["scales"].to(dev)
+    g = L["g_idx"].to(dev) if desc_act else None
+    wbytes = K * N * bits // 8
+    copies = max(2, -(-2 * INFINITY_CACHE_BYTES // wbytes))
+    gen = torch.Generator().manual_seed(99)
+    xsrc, qts, szt = None, [], None
+    for c in range(copies):
+        q = L["qweight"].to(dev) if c == 0 else torch.randint(
+            -(1 << 31), (1 << 31) - 1, L["qweight"].shape, generator=gen, dtype=torch.int64).to(torch.int32).to(dev)
+        if c == 0 and desc_act:
+            xsrc = ops.tile_prepare(q, qz, sc, g, bits, gs)[2]
+        qt, t = ops.tile_prepare_transposed(q, qz, sc, xsrc, bits, gs)
+        qts.append(qt)
+        szt = t if c == 0 else szt
+    gy_cpu = torch.randn(M, N, generator=torch.Generator().manual_seed(7)).half()
+    gy, gx = gy_cpu.to(dev), torch.empty((M, K), dtype=torch.float16, device=dev)
+    plan = _lib.select_tiled_transposed(M, K, N, bits, gs)
+    ws = torch.zeros(max(plan.workspace_bytes, 16), dtype=torch.uint8, device=dev)
+    lib = _lib.lib()
+    vp = ctypes.c_void_p
+    ptr = lambda t: vp(t.data_ptr()) if t is not None else None
+    qps = [ptr(q) for q in qts]
+    a_gy, a_szt, a_xsrc, a_gx, a_ws = ptr(gy), ptr(szt), ptr(xsrc), ptr(gx), ptr(ws)
+    planp = ctypes.byref(plan)
+
+    def step(i, stream):
+        rc = lib.gptq_hip_gemm_tiled_transposed(a_gy, qps[i % copies], a_szt, a_xsrc, a_gx, a_ws, ws.numel(), M, K, N, bits,
+                                                gs, planp, stream)
+        if rc != 0:
+            raise RuntimeError(f"gptq_hip_gemm_tiled_transposed failed: {_lib.strerror(rc)}")
+
+    step(0, vp(torch.cuda.current_stream(dev).cuda_stream))
+    torch.cuda.synchronize(dev)
+    w16 = torch.from_numpy(c_oracle.dequant(L["qweight"].numpy(), L["qzeros"].numpy(), L["scales"].numpy(),
+                                            L["g_idx"].numpy(), bits).copy())
+    want = gy_cpu.float() @ w16.float().t()
+    err = (gx.float().cpu() - want).abs()
+    ok = bool((err <= 1e-2 + 1e-2 * want.abs()).all())
+    stream = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(stream):
+        sp = vp(stream.cuda_stream)
+        for i in range(args.warmup):
+            step(i, sp)
+        stream.synchronize()
+    gr = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gr, stream=stream):
+        spg = vp(torch.cuda.current_stream(dev).cuda_stream)
+        for i in range(args.steps):
+            step(args.warmup + i, spg)
+    gr.replay()
+    torch.cuda.synchronize(dev)
+    times = []
+    for _ in range(3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        scrub_cache(dev)
+        torch.cuda.synchronize(dev)
+        e0.record()
+        gr.replay()
+        e1.record()
+        torch.cuda.synchronize(dev)
+        times.append(e0.elapsed_time(e1) * 1e3 / args.steps)
+    us = min(times)
+    tflops = 2 * M * K * N / us * 1e-6
+    print(json.dumps({
+        "metric": f"transposed GEMM latency (gradient for x), int{bits} {K}x{N} M={M}", "value": round(us, 3), "unit": "us",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us * 1e-3, 6),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": args.workload + " (transposed)", "bits": bits, "K": K, "N": N, "M": M, "group_size": gs,
+                   "desc_act": desc_act, "weight_copies": copies, "entry": "gptq_hip_gemm_tiled_transposed",
+                   "plan": {k: v for k, v in plan.as_dict().items()
+                            if k in ("kernel", "row_tiles", "waves_n", "waves_k", "split_k", "grid_x", "grid_y", "grid_z")}},
+        "parity": {"ok": ok, "max_abs_err": round(float(err.max()), 6), "rtol": 1e-2, "atol": 1e-2},
+        "tflops": round(tflops, 2),
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -389,6 +477,9 @@ def main():
     ap.add_argument("--kernel", type=int, default=0, help="force a kernel family (1 gather, 2 grouped, 3 blocked)")
     ap.add_argument("--split-k", type=int, default=0, help="force the split-K factor")
     ap.add_argument("--waves-n", type=int, default=0, help="force the waves per workgroup along N (STREAM kernel: along K)")
+    ap.add_argument("--transposed", action="store_true",
+                    help="time the gradient for x of the workload's layer (gy[M, N] @ W^T on the transposed tiled "
+                         "copy) instead of the forward product")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 256 MiB device copy a few times (known traffic, for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters of a profiler run) and exit")
@@ -412,6 +503,9 @@ def main():
         torch.cuda.synchronize(dev)
         print(json.dumps({"copy_calibration": {"bytes_read": nbytes, "bytes_written": nbytes, "launches": 5,
                                                "kernel": "torch elementwise copy (int32)"}}))
+        return
+    if args.transposed:
+        run_transposed(args, dev)
         return
     forced = bool(args.kernel or args.split_k or args.waves_n)
     prepared = None if (args.unprepared or forced) else prepared_mode(args.workload)
