@@ -66,7 +66,7 @@ def test_from_quantized_reports_missing_files_and_tensors(tmp_path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("bits,act_order", [(4, True), (3, True), (4, False)])
+@pytest.mark.parametrize("bits,act_order", [(4, True), (3, True), (4, False), (8, True), (2, False)])
 def test_loaded_model_matches_the_dequantised_float_model(tmp_path, bits, act_order):
     """End to end: logits of the loaded quantised model on the GPU against the same architecture
     with every quantised layer replaced by a float Linear holding the oracle's dequantised weight."""
