@@ -954,8 +954,8 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
 // 32 T + 16 c + n at positions 128 V + 32 q .. + 31 (two 256-byte runs per real block).  Everything per lane
 // is as in tiled_decode_kernel: the unpacked registers are B operands of v_mfma_f32_4x4x4_16B_f16, four
 // consecutive lanes share their positions, and the epilogue takes scale * (P - Bsum - zero * Xsum) per
-// 32 positions.  The sixteen waves take the virtual blocks V = wave, wave + 16, ... of every unit of the
-// workgroup, unit after unit, and meet in LDS at the end.
+// 32 positions.  The workgroup's (unit, virtual block) pairs are dealt out to the sixteen waves as contiguous
+// ranges; a wave leaves its partial results per unit in LDS, where all meet at the end.
 // G128: groups are multiples of 128 channels, so a virtual block lies in one group (scalar group index).
 // ---------------------------------------------------------------------------------------------------
 struct Decode16Params {
@@ -1020,29 +1020,38 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     for (int ps = 0; ps < SZP; ps++) szq[ps] = *sz_src(min(tid + ps * NT, sz_words - 1));
     __builtin_amdgcn_sched_barrier(0);
 
-    // items of this wave: for every unit the virtual blocks V = wave, wave + 16, ...
-    const int vpu = (p.V_total - wave + NW - 1) / NW;   // per unit (may be 0 for the last waves of a short K)
-    const int n_items = n_units * vpu;
+    // items of the workgroup: (unit, virtual block) pairs, unit after unit; wave w takes the contiguous range
+    // [I w / 16, I (w + 1) / 16) of them: consecutive virtual blocks of one unit, with a change of unit once or
+    // twice per wave (waves that stride over the virtual blocks would change unit after every K / 2048 items)
+    const int items_all = n_units * p.V_total;
+    const int i0 = (int)(((long long)items_all * wave) / NW);
+    const int n_items = (int)(((long long)items_all * (wave + 1)) / NW) - i0;   // (may be 0 for a short K)
     // lane offset inside a virtual block: its lane of the real block, and the second real block for q >= 2
     // (a last, odd virtual block has no second real block: those lanes repeat the first; their x is zero)
     const uint32_t b_lane = tile_lane_bytes<BITS>((uint32_t)(n16 + 32 * (lbv & 1)));
     const uint32_t b_lane2 = b_lane + (uint32_t)(lbv >> 1) * (256u * BITS);
     // cursors: (unit, V) of the next item to request and of the next item to compute
-    int rq_u = 0, rq_v = wave;
+    const int first_u = min(i0 / p.V_total, n_units - 1), first_v = n_items > 0 ? i0 % p.V_total : 0;
+    int rq_u = first_u, rq_v = first_v, rq_left = n_items;
+    auto unit_base = [&](int ul) {   // the first block of a unit's 16 columns (wave-uniform)
+        const int unit = u0 + ul;
+        return p.qtile + ((size_t)((uint32_t)(unit >> 1) * (uint32_t)p.S_total) * (256u * BITS) +
+                          tile_lane_bytes<BITS>(16u * (uint32_t)(unit & 1)));
+    };
+    const char *rq_ptr = unit_base(rq_u) + (size_t)rq_v * (512u * BITS);
     uint32_t w[2][PF][BITS];
     auto load_w = [&](uint32_t (&wr)[BITS]) {
-        // past the wave's items: its first item again (a cache hit that is never multiplied)
-        const bool valid = rq_u < n_units && vpu > 0;
-        const int unit = u0 + (valid ? rq_u : 0);
-        const int V = valid ? rq_v : min(wave, p.V_total - 1);
-        const int T = unit >> 1, c = unit & 1;
-        const char *base = p.qtile + ((size_t)((uint32_t)T * (uint32_t)p.S_total + 2u * (uint32_t)V) * (256u * BITS) +
-                                      tile_lane_bytes<BITS>(16u * (uint32_t)c));   // wave-uniform
-        tile_load<BITS>(base + (2 * V + 1 <= S_last ? b_lane2 : b_lane), wr);
-        rq_v += NW;
-        if (rq_v >= p.V_total) {
-            rq_v = wave;
-            rq_u++;
+        tile_load<BITS>(rq_ptr + (2 * rq_v + 1 <= S_last ? b_lane2 : b_lane), wr);
+        // past the wave's items: its last item again (a cache hit that is never multiplied)
+        if (rq_left > 1) {
+            rq_left--;
+            rq_v++;
+            rq_ptr += 512u * BITS;
+            if (rq_v == p.V_total) {
+                rq_v = 0;
+                rq_u++;
+                rq_ptr = unit_base(rq_u);
+            }
         }
     };
 #pragma unroll
@@ -1091,6 +1100,8 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
         const h2 e = as_h2(*sz_src(i));
         szl[i] = (f2){(float)e[0], (float)e[1]};
     }
+    // a wave writes the partial results of the units it walks: the others read as zeros
+    for (int i = tid; i < n_units * NW * MR * 64; i += NT) red[i] = 0.f;
     lds_barrier();
     // ---- 3. per 32 positions and row: Xsum = sum x, Bsum = sum x * base(position).  A thread sums 16
     //         positions, the lane next to it the other half of the run -------------------------------------
@@ -1144,7 +1155,7 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
         xv[0] = *(const u2 *)(smem + xoff);
         xv[1] = *(const u2 *)(smem + xoff + x_second);
     };
-    int cu = 0, cv = wave;   // (unit, V) of the item being computed
+    int cu = first_u, cv = first_v, c_left = n_items;   // (unit, V) of the item being computed, items still to compute
     auto item = [&](const uint32_t (&wr)[BITS], const u2 (&xc)[2], u2 (&xn)[2]) {
         const int V = cv, ul = cu;
         // this item's scale, zero point and sums
@@ -1164,10 +1175,11 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
             for (int m = 0; m < MR; m++) xsv[m] = xb[m];
         }
         // advance to the next item and read its x
-        cv += NW;
-        const bool unit_done = cv >= p.V_total;
-        if (unit_done) {
-            cv = wave;
+        c_left--;
+        cv++;
+        const bool unit_done = cv == p.V_total || c_left == 0;   // the wave's share of this unit ends here
+        if (cv == p.V_total) {
+            cv = 0;
             cu++;
         }
         load_x(cv, xn);
@@ -1225,11 +1237,6 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     if (c < n_items) {
         chunk(c, w[0], std::false_type{});
         chunk(c + PF, w[1], std::false_type{});
-    }
-    if (vpu == 0) {   // a wave without virtual blocks (K shorter than sixteen of them) adds zeros
-        for (int ul = 0; ul < n_units; ul++)
-#pragma unroll
-            for (int m = 0; m < MR; m++) *(float *)(smem + red_lane + (uint32_t)((ul * NW + wave) * MR + m) * 256u) = 0.f;
     }
     lds_barrier();
 
