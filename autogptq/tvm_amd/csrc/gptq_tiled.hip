@@ -974,7 +974,7 @@ struct Decode16Params {
     int lbg_add;
 };
 
-template <int BITS, int MR, bool G128>
+template <int BITS, int MR, bool G128, bool CONTIG>
 __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Params p)
 {
     static_assert(MR <= 4, "one matrix instruction set per lane block");
@@ -1020,18 +1020,22 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     for (int ps = 0; ps < SZP; ps++) szq[ps] = *sz_src(min(tid + ps * NT, sz_words - 1));
     __builtin_amdgcn_sched_barrier(0);
 
-    // items of the workgroup: (unit, virtual block) pairs, unit after unit; wave w takes the contiguous range
-    // [I w / 16, I (w + 1) / 16) of them: consecutive virtual blocks of one unit, with a change of unit once or
-    // twice per wave (waves that stride over the virtual blocks would change unit after every K / 2048 items)
+    // items of the workgroup: (unit, virtual block) pairs, unit after unit.
+    // CONTIG: wave w takes the contiguous range [I w / 16, I (w + 1) / 16) of them: consecutive virtual blocks of
+    // one unit, with a change of unit once or twice per wave.  Otherwise the waves stride over the virtual blocks
+    // of every unit (V = wave, wave + 16, ...), which changes unit after every K / 2048 items: measured 0.2 us
+    // ahead for one unit of 32 virtual blocks (4096 x 4096), 0.4 us behind for 86 (11008 x 4096).
     const int items_all = n_units * p.V_total;
-    const int i0 = (int)(((long long)items_all * wave) / NW);
-    const int n_items = (int)(((long long)items_all * (wave + 1)) / NW) - i0;   // (may be 0 for a short K)
+    const int i0 = CONTIG ? (int)(((long long)items_all * wave) / NW) : 0;
+    const int vpu = (p.V_total - wave + NW - 1) / NW;   // strided: per unit (may be 0 for the last waves of a short K)
+    const int n_items = CONTIG ? (int)(((long long)items_all * (wave + 1)) / NW) - i0 : n_units * vpu;
     // lane offset inside a virtual block: its lane of the real block, and the second real block for q >= 2
     // (a last, odd virtual block has no second real block: those lanes repeat the first; their x is zero)
     const uint32_t b_lane = tile_lane_bytes<BITS>((uint32_t)(n16 + 32 * (lbv & 1)));
     const uint32_t b_lane2 = b_lane + (uint32_t)(lbv >> 1) * (256u * BITS);
     // cursors: (unit, V) of the next item to request and of the next item to compute
-    const int first_u = min(i0 / p.V_total, n_units - 1), first_v = n_items > 0 ? i0 % p.V_total : 0;
+    const int first_u = CONTIG ? min(i0 / p.V_total, n_units - 1) : 0;
+    const int first_v = CONTIG ? (n_items > 0 ? i0 % p.V_total : 0) : min(wave, p.V_total - 1);
     int rq_u = first_u, rq_v = first_v, rq_left = n_items;
     auto unit_base = [&](int ul) {   // the first block of a unit's 16 columns (wave-uniform)
         const int unit = u0 + ul;
@@ -1045,12 +1049,22 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
         // past the wave's items: its last item again (a cache hit that is never multiplied)
         if (rq_left > 1) {
             rq_left--;
-            rq_v++;
-            rq_ptr += 512u * BITS;
-            if (rq_v == p.V_total) {
-                rq_v = 0;
-                rq_u++;
-                rq_ptr = unit_base(rq_u);
+            if constexpr (CONTIG) {
+                rq_v++;
+                rq_ptr += 512u * BITS;
+                if (rq_v == p.V_total) {
+                    rq_v = 0;
+                    rq_u++;
+                    rq_ptr = unit_base(rq_u);
+                }
+            } else {
+                rq_v += NW;
+                rq_ptr += (size_t)NW * (512u * BITS);
+                if (rq_v >= p.V_total) {
+                    rq_v = wave;
+                    rq_u++;
+                    rq_ptr = unit_base(rq_u) + (size_t)wave * (512u * BITS);
+                }
             }
         }
     };
@@ -1100,8 +1114,9 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
         const h2 e = as_h2(*sz_src(i));
         szl[i] = (f2){(float)e[0], (float)e[1]};
     }
-    // a wave writes the partial results of the units it walks: the others read as zeros
-    for (int i = tid; i < n_units * NW * MR * 64; i += NT) red[i] = 0.f;
+    // CONTIG: a wave writes the partial results of the units it walks: the others read as zeros
+    if constexpr (CONTIG)
+        for (int i = tid; i < n_units * NW * MR * 64; i += NT) red[i] = 0.f;
     lds_barrier();
     // ---- 3. per 32 positions and row: Xsum = sum x, Bsum = sum x * base(position).  A thread sums 16
     //         positions, the lane next to it the other half of the run -------------------------------------
@@ -1176,10 +1191,10 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
         }
         // advance to the next item and read its x
         c_left--;
-        cv++;
-        const bool unit_done = cv == p.V_total || c_left == 0;   // the wave's share of this unit ends here
-        if (cv == p.V_total) {
-            cv = 0;
+        cv += CONTIG ? 1 : NW;
+        const bool unit_done = cv >= p.V_total || c_left == 0;   // the wave's share of this unit ends here
+        if (cv >= p.V_total) {
+            cv = CONTIG ? 0 : wave;
             cu++;
         }
         load_x(cv, xn);
@@ -1237,6 +1252,11 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     if (c < n_items) {
         chunk(c, w[0], std::false_type{});
         chunk(c + PF, w[1], std::false_type{});
+    }
+    if (!CONTIG && vpu == 0) {   // strided: a wave without virtual blocks (K shorter than sixteen of them) adds zeros
+        for (int ul = 0; ul < n_units; ul++)
+#pragma unroll
+            for (int m = 0; m < MR; m++) *(float *)(smem + red_lane + (uint32_t)((ul * NW + wave) * MR + m) * 256u) = 0.f;
     }
     lds_barrier();
 
@@ -1635,10 +1655,10 @@ int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, co
     return GPTQ_HIP_OK;
 }
 
-template <int BITS, int MR, bool G128>
+template <int BITS, int MR, bool G128, bool CONTIG>
 static int launch_decode16_one(const Decode16Params &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
-    auto kern = tiled_decode16_kernel<BITS, MR, G128>;
+    auto kern = tiled_decode16_kernel<BITS, MR, G128, CONTIG>;
     if (plan.lds_bytes > 65536) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, plan.lds_bytes) != hipSuccess) {
             (void)hipGetLastError();
@@ -1676,8 +1696,14 @@ int launch_tiled_decode16(const void *x, const void *qtile, const uint32_t *sz, 
     const int mr = tiled_decode_rows(M);
     const bool g128 = group_size % 128 == 0;
     int rc = GPTQ_HIP_ERR_UNSUPPORTED;
-#define GPTQ_DECODE16_CASE(B, R) \
-    if (bits == B && mr == R) rc = g128 ? launch_decode16_one<B, R, true>(p, plan, stream) : launch_decode16_one<B, R, false>(p, plan, stream)
+    // contiguous ranges per wave when a wave has more than two items (a long K, or several units per workgroup)
+    const bool contig = (long long)((p.units + plan.grid_x - 1) / plan.grid_x) * p.V_total > 32;
+#define GPTQ_DECODE16_CASE(B, R)                                                                              \
+    if (bits == B && mr == R)                                                                                 \
+        rc = g128 ? (contig ? launch_decode16_one<B, R, true, true>(p, plan, stream)                          \
+                            : launch_decode16_one<B, R, true, false>(p, plan, stream))                        \
+                  : (contig ? launch_decode16_one<B, R, false, true>(p, plan, stream)                         \
+                            : launch_decode16_one<B, R, false, false>(p, plan, stream))
     GPTQ_DECODE16_CASE(4, 1);
     GPTQ_DECODE16_CASE(4, 2);
     GPTQ_DECODE16_CASE(4, 4);
