@@ -524,9 +524,19 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
         const int tiles = N / 32;
         const int S_total = ceil_div(K, 64);
         int kw = tiles * 4 >= 1024 ? 4 : (tiles * 8 >= 1024 ? 8 : 16);
+        // and enough of them that a wave walks about sixteen blocks at most: a wave issues one instruction per
+        // four clocks, so a long K wants more, shorter waves.  One row, us, kw = 4 / 8 / 16: 8192 x 8192
+        // 12.1 / 9.4 / 9.5, 5120 x 13824 10.9 / 9.4 / 11.6, 6144 x 16384 12.7 / 11.0 / 12.4, 9216 x 9216
+        // 16.3 / 13.6 / 14.6, 11008 x 11008 21.1 / 17.2 / 18.0, 13824 x 5120 19.9 / 12.6 / 10.6 (4096 x 11008
+        // keeps four: 8.2 / 8.2 / 10.1): eight whenever four would walk more than sixteen blocks, sixteen only
+        // while that keeps a CU at about twelve waves
+        if (kw == 4 && ceil_div(S_total, 4) > 16) kw = 8;
+        if (kw == 8 && ceil_div(S_total, 8) > 16 && (long long)tiles * 16 <= 12LL * gptq::kNumCUs) kw = 16;
         while (kw > 4 && kw > S_total) kw >>= 1;
         for (int split = 1; split <= S_total; split++) {
-            const int wave_steps = ceil_div(S_total, split * kw);
+            int wave_steps = ceil_div(S_total, split * kw);
+            // an even number of blocks per wave keeps the paired epilogue (groups that are multiples of 128 channels)
+            if (gs % 128 == 0 && wave_steps > 1 && (wave_steps & 1) && split == 1) wave_steps++;
             if (ceil_div(S_total, wave_steps * kw) != split) continue;  // (the split this partition really needs)
             const int span = wave_steps * kw * 64;
             const int groups = (span - 1) / gs + 2 < ceil_div(K, gs) ? (span - 1) / gs + 2 : ceil_div(K, gs);

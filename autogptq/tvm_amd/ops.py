@@ -343,14 +343,22 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
       * up to 4 rows, layers of up to 4096 columns (decode kernel with a workgroup per 16 columns, every CU at
         work): always.  4096 x 4096: 5.3-5.6 at one row, 7.4-8.0 at four, against 6.8-7.5 and 7.8-10.5;
         11008 x 4096: 9.5-9.7 / 12.7-14.4 against 9.4-13.3 / 12.7-15.3;
-      * up to 4 rows, wider layers (a workgroup per 32 columns, x staged per workgroup): K up to 6144 and at
-        most two rows, for 4-bit layers and for two rows under an activation order.  4096 x 11008 with an
-        activation order, one / two rows: int4 7.9 / 8.9 against 8.2 / 11.0, int3 8.0 / 8.9 against 7.7 / 10.3;
-        without: int4 7.9 / 8.5 against 7.9 / 9.0, int3 8.0 / 8.3 against 7.3 / 8.2; three and four rows are
-        behind by 0.5-2 us; 5120 x 5120 int4 6.3 against 13.4-15.2; 8192 x 8192 int3 13.2-13.9 against 11.2;
-        and very wide layers (from 16384 columns, K up to 12288), where many tiles per CU even the load out:
-        4096 x 22016 int3 / int4 10.1 / 10.6 against 11.6 / 12.8, 8192 x 28672 int4 24.2 against 27.5,
-        9216 x 36864 int3 / int4 29.1 / 31.8 against 32.9 / 34.6 (36864 x 9216: 79 against 36, hence the bound on K);
+      * up to 4 rows, wider layers (a workgroup per 32 columns, x staged per workgroup, four to sixteen waves
+        along K so that a wave walks about sixteen blocks):
+        K = 4096: at most two rows, for 4-bit layers and for two rows under an activation order.  4096 x 11008
+        with an activation order, one / two rows: int4 7.9 / 8.8 against 8.0 / 10.9, int3 7.9 / 8.7 against
+        7.7 / 10.1; without: int4 8.2 / 8.5 against 7.9 / 8.8, int3 7.9 / 8.2 against 7.4 / 8.3; three and four
+        rows are level or behind; from 16384 columns on also int3 (4096 x 22016 int3 / int4 9.7 / 10.3 against
+        11.4 / 12.8);
+        longer K, one and two rows: always up to K = 32768 (with an activation order, int4, one / two rows:
+        5120 x 13824 9.7 / 10.5 against 18.2 / 15.2, 6656 x 17920 15.1 / 15.4 against 27.9 / 27.2, 8192 x 8192
+        9.7 / 9.9 against 14.0 / 13.3, 8192 x 28672 24.6 / 26.4 against 32.3 / 30.2, 13824 x 5120 11.6 / 12.4
+        against 21.2 / 17.6, 17920 x 6656 17.5 / 19.6 against 30.0 / 23.7, 28672 x 8192 29.2 / 30.7 against
+        49.0 / 39.8, 9216 x 36864 int3 29.7 / 33.0 against 36.0 / 49.9; 36864 x 9216: 76 against 36, hence the
+        bound), except one row of a 3-bit layer of 9216 x 9216 (13.6 against 12.5-12.9);
+        longer K, three and four rows: K up to 6656 (5120 x 13824 12.8 against 15.4, 6656 x 17920 22.3 against
+        26.8) and 8192 x 8192 (12.3 against 13.3); beyond, the four staged rows of x cost more than they save
+        (8192 x 28672 41.9 against 30.4, 17920 x 6656 29.9 against 23.9);
       * 5 to 16 rows: never (4096 x 11008, 8 rows: 14.6 against 13.4);
       * 17 to 128 rows: everywhere within 4 % or better (4096 x 11008 with an activation order, 32/64/128
         rows: 14.8/19.2/26.6 against 18.1/22.1/34.1);
@@ -359,11 +367,15 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
     if M <= 4:
         if N <= 4096:
             return True
-        if M <= 2 and N >= 16384 and K <= 12288:
-            return True
-        if K > 6144:
+        if K <= 4096:
+            if M <= 2 and N >= 16384:
+                return True
+            return M <= 2 and (bits == 4 or (act_order and M == 2))
+        if K > 32768:
             return False
-        return M <= 2 and (bits == 4 or (act_order and M == 2))
+        if M <= 2:
+            return not (bits == 3 and M == 1 and 8192 < K <= 12288 and N <= 12288)
+        return K <= 6656 or (K <= 8192 and N <= 8192)
     if M <= 16:
         return False
     return M <= 128 or K <= 8192
