@@ -255,6 +255,10 @@ DECODE_FULL = [
     ("int2-4096x11008-act", 2, 4096, 11008, 128, True, [1, 3]),
     ("int8-11008x4096", 8, 11008, 4096, 128, False, [2]),
     ("int2-4096x4096-g64", 2, 4096, 4096, 64, False, [1]),
+    # long K on wide layers: the family's own plan takes eight or sixteen waves along K
+    ("int4-8192x8192-act", 4, 8192, 8192, 128, True, [1, 2]),
+    ("int3-13824x5120-act", 3, 13824, 5120, 128, True, [1, 4]),
+    ("int4-6656x17920", 4, 6656, 17920, 128, False, [2]),
 ]
 
 
@@ -267,11 +271,12 @@ def test_tiled_decode_full_size(dev, name, bits, K, N, gs, desc_act, Ms):
     for M in Ms:
         x = L["x"][:M].contiguous()
         want = expected_output(L, x=x, w16=w16)
-        for plan in (tile_decode_plan(M, K, N, bits, gs), cu_decode_plan(M, K, N, bits, gs)):
+        for plan in (_lib.select_tiled(M, K, N, bits, gs), tile_decode_plan(M, K, N, bits, gs),
+                     cu_decode_plan(M, K, N, bits, gs)):
             if plan is None:
                 continue
             y = run_tiled(D, prep, x=x.to(dev), plan=plan)
-            what = f"decode {name} M={M} ({'cu' if plan.waves_n == 2 else 'tile'})"
+            what = f"decode {name} M={M} ({'cu' if plan.waves_n == 2 else 'tile'}, {plan.waves_k} waves)"
             assert_close(y, want, what)
             assert_tight(y, want, what)
             assert torch.equal(y, run_tiled(D, prep, x=x.to(dev), plan=plan)), f"{what}: two identical calls differ"
