@@ -1,0 +1,97 @@
+// Shared by the translation units of the TILED family (gptq_tiled.hip: preparation, pack pass, matmul and its
+// transposed form; gptq_tiled_decode.hip and gptq_tiled_decode16.hip: the two decode kernels): how a lane's words of
+// a block are addressed and loaded, the magic constants of the register unpack, and what the decode kernels share.
+#pragma once
+#include <type_traits>
+#include <utility>
+
+#include "gptq_device.h"
+
+namespace gptq {
+
+struct alignas(4) W3 {
+    uint32_t a, b, c;
+};
+
+// Byte offset of lane l's words inside a block, and the lane's load.  Word i of a lane sits at
+// l * BITS + i, except for 8 bits: (i / 4) * 256 + l * 4 + i % 4, so that each of the two loads is coalesced.
+template <int BITS>
+__device__ __forceinline__ constexpr uint32_t tile_lane_bytes(uint32_t l)
+{
+    return BITS == 8 ? l * 16u : l * (4u * BITS);
+}
+
+template <int BITS>
+__device__ __forceinline__ void tile_load(const char *src, uint32_t (&wr)[BITS])
+{
+    if constexpr (BITS == 4) {
+        const u4 v = __builtin_nontemporal_load((const u4 *)src);
+#pragma unroll
+        for (int e = 0; e < 4; e++) wr[e] = v[e];
+    } else if constexpr (BITS == 8) {
+        const u4 v0 = __builtin_nontemporal_load((const u4 *)src);
+        const u4 v1 = __builtin_nontemporal_load((const u4 *)(src + 1024));
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            wr[e] = v0[e];
+            wr[4 + e] = v1[e];
+        }
+    } else if constexpr (BITS == 2) {
+        const u2 v = __builtin_nontemporal_load((const u2 *)src);
+        wr[0] = v[0];
+        wr[1] = v[1];
+    } else {
+        const W3 v = *(const W3 *)src;
+        wr[0] = v.a;
+        wr[1] = v.b;
+        wr[2] = v.c;
+    }
+}
+
+// The magic constants of the width's unpack, each held in a vector register.
+template <int BITS>
+__device__ __forceinline__ void tile_magic(uint32_t (&mg)[TileCodec<BITS>::KINDS])
+{
+#pragma unroll
+    for (int k = 0; k < TileCodec<BITS>::KINDS; k++) mg[k] = opaque_vgpr(TileCodec<BITS>::MAGIC[k]);
+}
+
+// ---- shared by the two decode kernels ----
+typedef float f2 __attribute__((ext_vector_type(2)));
+
+// 8-bit layers: the decode kernels dequantise every weight as the reference rounds it (fp16(scale * (q - zero)),
+// the matmul kernel's arithmetic).  Their weights are sixteen times those of a 4-bit layer, and so is the
+// distance between exact products and the reference's rounded ones; the extra packed instructions hide
+// behind a stream that is twice as long per weight.
+constexpr bool tiled_decode_exact(int bits) { return bits == 8; }
+
+// the sixteen unpacked registers of a lane -> fp16(scale * (q - zero)); sz = fp16 scale | fp16 zero << 16
+template <int BITS>
+__device__ __forceinline__ void tiled_dequant_exact(u4 (&q)[4], uint32_t sz)
+{
+    using Codec = TileCodec<BITS>;
+    const h2 e = as_h2(sz);
+    const h2 s2 = {e[0], e[0]};
+    h2 zb[Codec::KINDS];
+#pragma unroll
+    for (int k = 0; k < Codec::KINDS; k++)
+        zb[k] = (h2){e[1], e[1]} + (h2){(_Float16)Codec::base(2 * k), (_Float16)Codec::base(2 * k + 1)};
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) q[j][r] = as_u32((as_h2(q[j][r]) - zb[r % Codec::KINDS]) * s2);
+}
+
+// v of lane l + N inside its row of 16 lanes (zero past the row's end)
+template <int N>
+__device__ __forceinline__ float row_shl(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x100 + N, 0xf, 0xf, true));
+}
+
+// y = fp16(sum over split of partial[split] (+ bias)): the pass after a product whose K range was cut over
+// workgroups (defined in gptq_tiled.hip); out_map: the transposed product's channel map, else nullptr.
+int launch_tiled_reduce(const float *partial, const void *bias, void *y, int M, int N, int split_k, const int32_t *out_map,
+                        hipStream_t stream);
+
+}  // namespace gptq

@@ -1,0 +1,424 @@
+// TILED family, the decode kernel with a workgroup per 32-column tile: up to four rows of x on the tiled format
+// (the format, its preparation and the matmul kernel for more rows are in gptq_tiled.hip; the decode kernel with
+// one workgroup per CU in gptq_tiled_decode16.hip).
+#include "gptq_tiled_common.h"
+
+namespace gptq {
+
+// ---------------------------------------------------------------------------------------------------
+// tiled_decode_kernel: M <= 4 rows of x on the tiled format.
+//
+// A workgroup owns ONE column tile (32 columns) and one K range; its KW waves split that range.  With one
+// small workgroup per tile every CU gets work whatever N is (11008 columns: 344 workgroups of 4 waves,
+// 4096 columns: 128 of 16), and what a wave keeps in flight (PF blocks of 1 KB / 768 B) adds up over the
+// many waves of a CU.
+// The dots run on v_mfma_f32_4x4x4_16B_f16: sixteen independent 4-lane blocks, lane 4 b + i supplies
+// row i of A and column i of B of block b, and result register v of lane 4 b + j is row v of column j.
+// A lane of the tiled format holds 32 codes of ONE column, so its unpacked registers are B operands as
+// they are (four positions each), the A operand of row i is x[row i] at the same four positions (rows past
+// M are zeros), and the four result registers of a lane are the rows of its own column: up to four rows of
+// x cost one matrix instruction per four positions.  All 4-lane blocks of a half wave share their positions,
+// and the instruction can broadcast the A operand of one block to the others (cbsz / abid): block b of the
+// half keeps positions 4 b .. 4 b + 3 in its A registers and the instruction for positions 4 i .. 4 i + 3
+// names block i, so x costs one 8-byte LDS read per lane and block.
+// Per weight the vector ALU only unpacks (2, 3, 4 bits).
+// The codes enter as (base + q) with the bases of the register unpack; per block of 32 positions the
+// epilogue takes y += scale * (P - Bsum - zero * Xsum), with Xsum = sum x and Bsum = sum x * base of the
+// block computed once per workgroup when x is staged.  Like GROUPED, and unlike the TILED matmul, this
+// does not reproduce the fp16 rounding of each dequantised weight: products are exact, sums are fp32.
+// 8-bit layers instead dequantise every weight in registers, as the matmul does (tiled_decode_exact), and add
+// the products as they are.
+// x reaches LDS in position order: a layer with an activation order scatters it through kinv (16-bit
+// position per channel, one round trip; every workgroup walks all of x and keeps its K range).
+// ---------------------------------------------------------------------------------------------------
+struct DecodeParams {
+    const _Float16 *x;      // [M, K]
+    const uint16_t *kinv;   // [K] position of channel k, or nullptr (identity)
+    const char *qtile;
+    const uint32_t *sz;     // [G][N]
+    const void *bias;
+    void *y;                // fp16 [M, N]
+    float *partial;         // [split_k][M][N] when split_k > 1
+    int M, K, N, G;
+    int S_total, T_total;
+    int wave_steps;         // blocks (64 positions) per wave
+    int split_k;
+    int lb_per_group;       // group_size / 32
+    uint32_t lbg_magic;     // lane block -> group: umulhi(lb, magic) + (add ? lb : 0)
+    int lbg_add;
+};
+
+// E: blocks of 64 positions that share one epilogue (1, or 2 when the groups are multiples of 128 channels and
+// every wave has an even number of blocks: both lane blocks of both blocks then lie in one group).
+template <int BITS, int MR, int KW, int E>
+__global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParams p)
+{
+    static_assert(MR <= 4 && (E == 1 || E == 2), "one matrix instruction set per lane block");
+    constexpr bool EXACT = tiled_decode_exact(BITS);
+    constexpr int NT = 64 * KW;
+    constexpr int PF = 2;              // blocks of weights per chunk; two chunks are in flight
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, h = lane >> 5;
+    const int T = blockIdx.x;
+    const int split = blockIdx.y;
+    const int wg_steps = p.wave_steps * KW;              // blocks of the workgroup's K range
+    const int S_wg = split * wg_steps;                   // its first block
+    const int S_begin = S_wg + wave * p.wave_steps;      // this wave's first block
+    const int S_last = p.S_total - 1;
+    const int span = wg_steps * 64;                      // positions the workgroup stages
+    const int p0 = S_wg * 64;                            // its first position
+
+    // LDS: x in position order [MR][span] fp16 | 64 zero bytes | block sums [span / 32][MR] (Xsum, Bsum) |
+    //      (scale, zero) words of the range's groups [groups][32] | partial results [KW][MR][32]
+    _Float16 *xl = (_Float16 *)smem;
+    const uint32_t zero_off = (uint32_t)MR * (uint32_t)span * 2u;
+    f2 *xs = (f2 *)(smem + zero_off + 64);
+    const int lbs = span / 32;
+    const uint32_t g_first = __umulhi((uint32_t)(2 * S_wg), p.lbg_magic) + (p.lbg_add ? (uint32_t)(2 * S_wg) : 0u);
+    const uint32_t lb_end = (uint32_t)min(2 * (S_wg + wg_steps), 2 * p.S_total) - 1u;
+    const uint32_t g_lastr = min(__umulhi(lb_end, p.lbg_magic) + (p.lbg_add ? lb_end : 0u), (uint32_t)p.G - 1u);
+    const int n_groups = (int)(g_lastr - g_first) + 1;
+    uint32_t *szl = (uint32_t *)(xs + (size_t)lbs * MR);
+    float *red = (float *)(szl + (size_t)n_groups * 32);
+
+    // ---- 1. x and the map first (a wait for them would also wait for every older load: vector loads return
+    //         in order), then the first weights of this wave, then the (scale, zero) words ----------------
+    // (without a map the channels of the range are the range itself)
+    const int k8_lo = p.kinv ? 0 : p0 / 8, k8_hi = p.kinv ? p.K / 8 : min(p0 + span, p.K) / 8;
+    constexpr int QP = 2;  // passes over x kept in registers
+    u4 kq[QP];
+    h8 xq[QP][MR];
+#pragma unroll
+    for (int ps = 0; ps < QP; ps++) {
+        const int k = 8 * min(k8_lo + tid + ps * NT, k8_hi - 1);  // (clamped: the pass is skipped below when outside)
+        kq[ps] = p.kinv ? *(const u4 *)(p.kinv + k) : (u4){0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int m = 0; m < MR; m++) xq[ps][m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
+    }
+    // the (scale, zero) words of the range's groups for this tile's 32 columns: SZP passes in registers
+    constexpr int SZP = 4;
+    uint32_t szq[SZP];
+#pragma unroll
+    for (int ps = 0; ps < SZP; ps++) {
+        const int i = min(tid + ps * NT, n_groups * 32 - 1);
+        szq[ps] = p.sz[(size_t)(g_first + (uint32_t)(i >> 5)) * p.N + 32 * T + (i & 31)];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    const uint32_t b_lane = tile_lane_bytes<BITS>((uint32_t)lane);
+    const uint32_t tile_off = (uint32_t)T * (uint32_t)p.S_total;
+    uint32_t w[2][PF][BITS];
+    const int steps = min(p.wave_steps, max(p.S_total - S_begin, 0));  // blocks of this wave that lie inside K
+    auto load_w = [&](int i, uint32_t (&wr)[BITS]) {
+        // block i of the wave's range; past its end: its first block again (a cache hit that is never multiplied)
+        const int Sc = min(S_begin + (i < steps ? i : 0), S_last);
+        tile_load<BITS>(p.qtile + ((size_t)(tile_off + (uint32_t)Sc) * (256u * BITS) + b_lane), wr);
+    };
+    // two chunks of PF blocks are in flight from here on, through the staging of x as well
+#pragma unroll
+    for (int u = 0; u < PF; u++) load_w(u, w[0][u]);
+#pragma unroll
+    for (int u = 0; u < PF; u++) load_w(PF + u, w[1][u]);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- 2. stage x in position order ------------------------------------------------------------------
+    if (tid < 16) ((uint32_t *)(smem + zero_off))[tid] = 0u;
+    {
+        // positions of the range that lie past K (the padding of the last block) read as zeros
+        const int tail0 = max(p.K - p0, 0);
+        for (int i = tail0 + tid; i < span; i += NT)
+#pragma unroll
+            for (int m = 0; m < MR; m++) xl[m * span + i] = (_Float16)0;
+    }
+    auto scatter8 = [&](int k, const u4 &kv, const h8 (&xv)[MR]) {
+        if (!p.kinv) {   // no activation order: the eight channels are eight consecutive positions, one store
+            // (k8_lo .. k8_hi is the workgroup's own range here, a multiple of 8 away from p0)
+#pragma unroll
+            for (int m = 0; m < MR; m++) *(h8 *)(xl + m * span + (k - p0)) = xv[m];
+            return;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int pos = (int)((kv[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+            const int pl = pos - p0;
+            if ((unsigned)pl < (unsigned)span) {
+#pragma unroll
+                for (int m = 0; m < MR; m++) xl[m * span + pl] = xv[m][e];
+            }
+        }
+    };
+#pragma unroll
+    for (int ps = 0; ps < QP; ps++) {
+        const int k8 = k8_lo + tid + ps * NT;
+        if (k8 < k8_hi) scatter8(8 * k8, kq[ps], xq[ps]);
+    }
+    for (int k8 = k8_lo + tid + QP * NT; k8 < k8_hi; k8 += NT) {  // long layers: the rest, a pass at a time
+        const int k = 8 * k8;
+        u4 kv = {0u, 0u, 0u, 0u};
+        if (p.kinv) kv = *(const u4 *)(p.kinv + k);
+        h8 xv[MR];
+#pragma unroll
+        for (int m = 0; m < MR; m++) xv[m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
+        scatter8(k, kv, xv);
+    }
+#pragma unroll
+    for (int ps = 0; ps < SZP; ps++) {
+        const int i = tid + ps * NT;
+        if (i < n_groups * 32) szl[i] = szq[ps];
+    }
+    for (int i = tid + SZP * NT; i < n_groups * 32; i += NT) {  // more groups than the register passes hold
+        szl[i] = p.sz[(size_t)(g_first + (uint32_t)(i >> 5)) * p.N + 32 * T + (i & 31)];
+    }
+    lds_barrier();
+    // ---- 3. per epilogue unit (E blocks), half and row: Xsum = sum x, Bsum = sum x * base(position) over the
+    //         unit's 32 E positions of that half; every wave for the units of its own slice (LDS serves one
+    //         wave's accesses in order: no barrier needed).  Entry ((sb / E) * 2 + h) * MR + m, sb = the unit's
+    //         first block inside the workgroup's range ------------------------------------------------------
+    if constexpr (!EXACT) {
+        // a lane sums 16 consecutive positions; a run of 32 positions (one half of one block) is two lanes,
+        // a unit-half 2 E lanes: l, l + 1 (the other half of the run) and, E = 2, l + 4, l + 5 (the other block)
+        const int sb0 = S_begin - S_wg;
+        for (int q0 = 0; q0 < 4 * p.wave_steps; q0 += 64) {   // 16-position pieces of the wave's range
+            const int piece = q0 + lane;
+            const int sb = sb0 + (piece >> 2), hh = (piece >> 1) & 1;
+            const bool live = piece < 4 * p.wave_steps;
+#pragma unroll
+            for (int m = 0; m < MR; m++) {
+                float X = 0.f, B = 0.f;
+                if (live && m < p.M) {
+                    const h8 *src = (const h8 *)(xl + m * span + 64 * sb0 + 16 * piece);
+#pragma unroll
+                    for (int v = 0; v < 2; v++) {
+                        const h8 q = src[v];
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            const float xf = (float)q[e];
+                            X += xf;
+                            B += xf * TileCodec<BITS>::base(e);
+                        }
+                    }
+                }
+                // lane l takes l + 1 (and, E = 2, l + 4 and l + 5): the lanes that store (l % 8 in {0, 2}) stay
+                // inside their row of 16, so a row shift in the data path does (no LDS round trip)
+                X += row_shl<1>(X);
+                B += row_shl<1>(B);
+                if constexpr (E == 2) {
+                    X += row_shl<4>(X);
+                    B += row_shl<4>(B);
+                }
+                if (live && (lane & (E == 2 ? 5 : 1)) == 0) xs[((sb / E) * 2 + hh) * MR + m] = (f2){X, B};
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+
+    // ---- 4. the walk ----------------------------------------------------------------------------------
+    uint32_t mg[TileCodec<BITS>::KINDS];
+    tile_magic<BITS>(mg);
+    const int row_i = lane & 3;  // the row of x this lane supplies to its 4-lane block
+    float ysum[MR];
+#pragma unroll
+    for (int m = 0; m < MR; m++) ysum[m] = 0.f;
+    // Per-lane byte offsets that never change; what changes per block is wave-uniform and stays in scalar
+    // registers.  A lane whose row lies past M reads the 64 zero bytes whatever the block (stride 0).
+    // The matrix instruction broadcasts A: with cbsz = 3 the eight 4-lane blocks of a half wave all take their A
+    // operand from block `abid` of the half.  So lane block b of a half holds only positions 4 b .. 4 b + 3 of the
+    // half's 32 (one 8-byte read per lane and block instead of 64 bytes), and the instruction for positions
+    // 4 i .. 4 i + 3 names abid = i.
+    const int lb8 = (lane >> 2) & 7;
+    const uint32_t x_base = row_i < p.M ? (uint32_t)(row_i * span + 32 * h + 4 * lb8) * 2u : zero_off;
+    const uint32_t x_stride = row_i < p.M ? 128u : 0u;
+    const uint32_t xs_lane = zero_off + 64u + (uint32_t)(h * MR) * 8u;   // sums of half h of unit 0
+    const uint32_t sz_lane = (uint32_t)((const unsigned char *)szl - smem) + (uint32_t)n * 4u;
+
+    // x of a block: this lane's four positions of row row_i; read one block ahead of its use
+    auto load_x = [&](uint32_t sb, u2 &xv) { xv = *(const u2 *)(smem + x_base + x_stride * sb); };
+    f4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};  // two chains: a matrix instruction waits for the one it adds to
+    uint32_t szw = 0u;   // (scale, zero) word and sums of the unit in flight, read when the unit starts
+    f2 xsv[MR];
+    auto block = [&](auto uu_c, int S, const uint32_t (&wr)[BITS], const u2 &xc, u2 &xn) {
+        constexpr int uu = decltype(uu_c)::value;                 // block inside its unit
+        const uint32_t sb = (uint32_t)(S - S_wg);                  // block inside the workgroup's range (wave-uniform)
+        if constexpr (uu == 0) {
+            // group of the unit's lane blocks (E = 1: the two halves of the wave may differ)
+            const uint32_t l0 = 2u * (uint32_t)S;
+            const uint32_t g0 = min(__umulhi(l0, p.lbg_magic) + (p.lbg_add ? l0 : 0u), (uint32_t)p.G - 1u) - g_first;
+            uint32_t goff = g0 * 128u;
+            if constexpr (E == 1) {
+                const uint32_t l1 = l0 + 1u;
+                const uint32_t g1 = min(__umulhi(l1, p.lbg_magic) + (p.lbg_add ? l1 : 0u), (uint32_t)p.G - 1u) - g_first;
+                goff = (h ? g1 : g0) * 128u;
+            }
+            szw = *(const uint32_t *)(smem + sz_lane + goff);
+            if constexpr (!EXACT) {
+                const f2 *xb = (const f2 *)(smem + xs_lane + (sb / E) * (uint32_t)(2 * MR * 8));
+#pragma unroll
+                for (int m = 0; m < MR; m++) xsv[m] = xb[m];
+            }
+        }
+        load_x(sb + 1u, xn);
+        // unpack: sixteen registers, positions (2 r, 2 r + 1) of the lane in register r
+        u4 q[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) TileCodec<BITS>::operand(wr, j, q[j], mg);
+        if constexpr (EXACT) tiled_dequant_exact<BITS>(q, szw);
+        if constexpr (uu == 0) {
+            c0 = (f4){0.f, 0.f, 0.f, 0.f};
+            c1 = (f4){0.f, 0.f, 0.f, 0.f};
+        }
+        const h4 xa = __builtin_bit_cast(h4, xc);
+        [&]<int... V>(std::integer_sequence<int, V...>) {
+            ((c0 = __builtin_amdgcn_mfma_f32_4x4x4f16(xa, __builtin_bit_cast(h4, (u2){q[V][0], q[V][1]}), c0, 3, 2 * V, 0),
+              c1 = __builtin_amdgcn_mfma_f32_4x4x4f16(xa, __builtin_bit_cast(h4, (u2){q[V][2], q[V][3]}), c1, 3, 2 * V + 1, 0)),
+             ...);
+        }(std::make_integer_sequence<int, 4>{});
+        if constexpr (uu == E - 1) {
+            if constexpr (EXACT) {
+#pragma unroll
+                for (int m = 0; m < MR; m++) ysum[m] += c0[m] + c1[m];
+            } else {
+                const h2 e = as_h2(szw);
+                const float sc = (float)e[0], zp = (float)e[1];
+#pragma unroll
+                for (int m = 0; m < MR; m++) ysum[m] += sc * (((c0[m] + c1[m]) - xsv[m][1]) - zp * xsv[m][0]);
+            }
+        }
+    };
+
+    // Chunks of PF blocks, two in flight; x rides one block ahead in two register sets.  Blocks past the end
+    // of K inside a wave's range are harmless (their x and sums are zeros), blocks past the range are skipped.
+    u2 xr[2];
+    load_x((uint32_t)(S_begin - S_wg), xr[0]);
+    auto chunk = [&](int c, uint32_t (&wc)[PF][BITS], auto all_c) {
+        constexpr bool ALL = decltype(all_c)::value;
+        [&]<int... U>(std::integer_sequence<int, U...>) {
+            ((ALL || c + U < p.wave_steps
+                  ? block(std::integral_constant<int, U % E>{}, S_begin + c + U, wc[U], xr[U & 1], xr[(U + 1) & 1])
+                  : (void)0),
+             ...);
+        }(std::make_integer_sequence<int, PF>{});
+    };
+    int c = 0;
+    for (; c + 2 * PF <= p.wave_steps; c += 2 * PF) {
+        chunk(c, w[0], std::true_type{});
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < PF; u++) load_w(c + 2 * PF + u, w[0][u]);  // the chunk after the one in flight
+        __builtin_amdgcn_sched_barrier(0);
+        chunk(c + PF, w[1], std::true_type{});
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < PF; u++) load_w(c + 3 * PF + u, w[1][u]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (c < p.wave_steps) {   // what is left of the range: fewer than two chunks, nothing more to request
+        chunk(c, w[0], std::false_type{});
+        chunk(c + PF, w[1], std::false_type{});
+    }
+
+    // ---- 5. the two halves of a column (lanes n and n + 32), then the waves along K ---------------------
+#pragma unroll
+    for (int m = 0; m < MR; m++) ysum[m] += __shfl_xor(ysum[m], 32);
+    if (h == 0) {
+#pragma unroll
+        for (int m = 0; m < MR; m++) red[(wave * MR + m) * 32 + n] = ysum[m];
+    }
+    lds_barrier();
+    if (tid < MR * 32) {
+        const int m = tid >> 5, nn = tid & 31;
+        if (m < p.M) {
+            float sum = 0.f;
+            for (int k = 0; k < KW; k++) sum += red[(k * MR + m) * 32 + nn];
+            const size_t o = (size_t)m * p.N + 32 * T + nn;
+            if (p.split_k == 1) {
+                if (p.bias) sum += (float)((const _Float16 *)p.bias)[32 * T + nn];
+                ((_Float16 *)p.y)[o] = (_Float16)sum;
+            } else {
+                p.partial[(size_t)split * p.M * p.N + o] = sum;
+            }
+        }
+    }
+}
+
+template <int BITS, int MR, int KW, int E>
+static int launch_decode_one(const DecodeParams &p, const gptq_hip_plan &plan, hipStream_t stream)
+{
+    auto kern = tiled_decode_kernel<BITS, MR, KW, E>;
+    if (plan.lds_bytes > 65536) {
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, plan.lds_bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return GPTQ_HIP_ERR_LAUNCH;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, 1), dim3(64 * KW), plan.lds_bytes, stream, p);
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+}
+
+template <int BITS, int MR, int E>
+static int launch_decode_kw(const DecodeParams &p, const gptq_hip_plan &plan, hipStream_t stream)
+{
+    switch (plan.waves_k) {
+        case 4: return launch_decode_one<BITS, MR, 4, E>(p, plan, stream);
+        case 8: return launch_decode_one<BITS, MR, 8, E>(p, plan, stream);
+        case 16: return launch_decode_one<BITS, MR, 16, E>(p, plan, stream);
+        default: return GPTQ_HIP_ERR_UNSUPPORTED;
+    }
+}
+
+// The decode product on the tiled format: one launch, plus a reduce pass when K is split over workgroups.
+int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, const uint16_t *kinv, const void *bias,
+                        void *y, float *partial, int M, int K, int N, int G, int bits, int group_size,
+                        const gptq_hip_plan &plan, void *stream_v)
+{
+    hipStream_t stream = (hipStream_t)stream_v;
+    DecodeParams p;
+    p.x = (const _Float16 *)x;
+    p.kinv = kinv;
+    p.qtile = (const char *)qtile;
+    p.sz = sz;
+    p.bias = bias;
+    p.y = y;
+    p.partial = partial;
+    p.M = M;
+    p.K = K;
+    p.N = N;
+    p.G = G;
+    p.S_total = (K + 63) / 64;
+    p.T_total = N / 32;
+    p.wave_steps = plan.k_chunk;
+    p.split_k = plan.split_k;
+    p.lb_per_group = group_size / 32;
+    // lane block -> group as a multiply-high (lane blocks are below 2^16 / 32 * 2)
+    p.lbg_add = p.lb_per_group == 1;
+    p.lbg_magic = p.lbg_add ? 0u : (uint32_t)((1ull << 32) / (uint32_t)p.lb_per_group) + 1u;
+    const int mr = tiled_decode_rows(M);
+    int rc = GPTQ_HIP_ERR_UNSUPPORTED;
+    // two blocks per epilogue where every unit of two blocks lies in one group
+    const bool pairs = group_size % 128 == 0 && plan.k_chunk % 2 == 0;
+#define GPTQ_DECODE_CASE(B, R) \
+    if (bits == B && mr == R) rc = pairs ? launch_decode_kw<B, R, 2>(p, plan, stream) : launch_decode_kw<B, R, 1>(p, plan, stream)
+    GPTQ_DECODE_CASE(4, 1);
+    GPTQ_DECODE_CASE(4, 2);
+    GPTQ_DECODE_CASE(4, 4);
+    GPTQ_DECODE_CASE(3, 1);
+    GPTQ_DECODE_CASE(3, 2);
+    GPTQ_DECODE_CASE(3, 4);
+    GPTQ_DECODE_CASE(2, 1);
+    GPTQ_DECODE_CASE(2, 2);
+    GPTQ_DECODE_CASE(2, 4);
+    GPTQ_DECODE_CASE(8, 1);
+    GPTQ_DECODE_CASE(8, 2);
+    GPTQ_DECODE_CASE(8, 4);
+#undef GPTQ_DECODE_CASE
+    if (rc != GPTQ_HIP_OK) return rc;
+    if (plan.split_k > 1) {
+        if (launch_tiled_reduce(partial, bias, y, M, N, plan.split_k, nullptr, stream) != GPTQ_HIP_OK)
+            return GPTQ_HIP_ERR_LAUNCH;
+    }
+    return GPTQ_HIP_OK;
+}
+
+}  // namespace gptq
