@@ -49,15 +49,24 @@ void raise(int rc, const char *what, int64_t M, int64_t K, int64_t N, int64_t bi
                 ") failed: ", gptq_hip_strerror(rc), " [status ", rc, "]");
 }
 
-// One workspace per (device, stream); a replaced one stays alive until the process ends only if a caller
+// One workspace per (device, stream) and kind; a replaced one stays alive until the process ends only if a caller
 // still holds it (the allocator keeps it valid for work already queued on its stream).
+// kind 1: the decode plans of the tiled family with halved tiles, whose kernel keeps their bytes zero between launches
+// (the slots of the halves): nothing else may write there, so they do not share the workspace the other plans pack x
+// or partial sums into.
 std::mutex g_ws_mutex;
-std::map<std::pair<int, void *>, Tensor> g_ws;
+std::map<std::tuple<int, void *, int>, Tensor> g_ws;
 
-Tensor workspace(const Tensor &like, size_t nbytes, void *stream)
+int workspace_kind(const gptq_hip_plan &plan)
+{
+    // (a decode plan that cuts K over workgroups leaves partial sums in its workspace like any other plan)
+    return plan.kernel == GPTQ_HIP_KERNEL_TILED_DECODE && plan.split_k == 1 ? 1 : 0;
+}
+
+Tensor workspace(const Tensor &like, size_t nbytes, void *stream, int kind = 0)
 {
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    Tensor &ws = g_ws[{(int)like.get_device(), stream}];
+    Tensor &ws = g_ws[{(int)like.get_device(), stream, kind}];
     if (!ws.defined() || (size_t)ws.numel() < nbytes) {
         const int64_t n = (int64_t)std::max(nbytes, (size_t)1 << 20);
         ws = at::zeros({n}, like.options().dtype(at::kByte));
@@ -190,7 +199,7 @@ Tensor gemm_tiled(const Tensor &x, const Tensor &qtile, const Tensor &sz, const 
     raise(rc, "gptq_hip_gemm_tiled", M, K, N, bits, group_size);
     TORCH_CHECK(sz.size(0) == (group_size == -1 ? 1 : K / group_size), "sz must have one row per group");
     Tensor ws;
-    if (plan.workspace_bytes) ws = workspace(x, plan.workspace_bytes, stream);
+    if (plan.workspace_bytes) ws = workspace(x, plan.workspace_bytes, stream, workspace_kind(plan));
     rc = gptq_hip_gemm_tiled(x.data_ptr(), qtile.data_ptr(), (const uint32_t *)sz.data_ptr(), (const int32_t *)ptr(xsrc),
                              (const uint16_t *)ptr(kinv), ptr(bias), y.data_ptr(), ws.defined() ? ws.data_ptr() : nullptr,
                              ws.defined() ? (size_t)ws.numel() : 0, (int)M, (int)K, (int)N, (int)bits, (int)group_size,
@@ -259,7 +268,7 @@ struct Layer : torch::CustomClassHolder {
             const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
             void *stream = (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(x.get_device()).stream();
             Tensor ws;
-            if (ws_need) ws = workspace(x, ws_need, stream);
+            if (ws_need) ws = workspace(x, ws_need, stream, workspace_kind(plan));
             void *wsp = ws.defined() ? ws.data_ptr() : nullptr;
             const size_t wsb = ws.defined() ? (size_t)ws.numel() : 0;
             const int M = (int)fast_rows, bi = (int)bits, gs = (int)group_size;

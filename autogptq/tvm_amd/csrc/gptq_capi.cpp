@@ -365,8 +365,12 @@ extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint3
         const int mr = plan->row_tiles, kw = plan->waves_k;
         const int S_all = (K + 63) / 64;
         if (M > gptq::kDecodeMaxRows || mr != gptq::tiled_decode_rows(M)) return GPTQ_HIP_ERR_UNSUPPORTED;
+        // grid_x: a workgroup per tile, or the planner's halved tiles on top
+        const int halved = plan->grid_x - N / 32;
+        if (halved != 0 && halved != gptq::tiled_decode_halved(N / 32, plan->k_chunk, plan->split_k, kw, S_all))
+            return GPTQ_HIP_ERR_BAD_ARG;
         if ((kw != 4 && kw != 8 && kw != 16) || plan->block != 64 * kw || plan->split_k < 1 || plan->k_chunk < 1 ||
-            plan->grid_x != N / 32 || plan->grid_y != plan->split_k || plan->grid_z != 1 ||
+            plan->grid_y != plan->split_k || plan->grid_z != 1 ||
             (long long)plan->split_k * kw * plan->k_chunk < S_all ||
             (long long)(plan->split_k - 1) * kw * plan->k_chunk >= S_all)  // every workgroup starts inside K
             return GPTQ_HIP_ERR_BAD_ARG;
@@ -382,7 +386,13 @@ extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint3
             if (!workspace || !aligned(workspace, 16) || workspace_bytes < need) return GPTQ_HIP_ERR_WORKSPACE;
             part = (float *)((char *)workspace + gptq::kCounterBytes);
         }
-        return gptq::launch_tiled_decode(x, qtile, sz, kinv, bias, y, part, M, K, N, G_all, bits, gs, *plan, stream);
+        unsigned long long *slots = nullptr;
+        if (halved > 0) {
+            const size_t need = gptq::kCounterBytes + gptq::tiled_decode_slot_bytes(halved, mr);
+            if (!workspace || !aligned(workspace, 16) || workspace_bytes < need) return GPTQ_HIP_ERR_WORKSPACE;
+            slots = (unsigned long long *)((char *)workspace + gptq::kCounterBytes);
+        }
+        return gptq::launch_tiled_decode(x, qtile, sz, kinv, bias, y, part, slots, M, K, N, G_all, bits, gs, *plan, stream);
     }
     // the plan must be one this family runs, sized for this problem
     const int rts = plan->row_tiles;  // 32-row tiles per workgroup
@@ -502,9 +512,8 @@ extern "C" int gptq_hip_workspace_init(void *workspace, size_t workspace_bytes, 
 {
     if (workspace_bytes == 0) return GPTQ_HIP_OK;
     if (!workspace || workspace_bytes % 4 != 0 || !aligned(workspace, 4)) return GPTQ_HIP_ERR_BAD_ARG;
-    // only the counters at the head need to start at zero
-    const size_t n = workspace_bytes < gptq::kCounterBytes ? workspace_bytes : gptq::kCounterBytes;
-    return gptq::launch_fill_zero(workspace, n, stream);
+    // (most plans only need the counters at the head to start at zero; a decode plan with halved tiles needs all of it)
+    return gptq::launch_fill_zero(workspace, workspace_bytes, stream);
 }
 
 extern "C" const char *gptq_hip_strerror(int status)

@@ -550,12 +550,16 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
             plan->waves_k = kw;
             plan->split_k = split;
             plan->k_chunk = wave_steps;
-            plan->grid_x = tiles;
+            // more tiles than CUs but fewer than two per CU: the last tiles - CUs tiles run as two halves along K,
+            // so that no CU holds two whole tiles (4096 x 11008: 344 tiles, 88 of them halved)
+            const int halved = gptq::tiled_decode_halved(tiles, wave_steps, split, kw, S_total);
+            plan->grid_x = tiles + halved;
             plan->grid_y = split;
             plan->grid_z = 1;
             plan->block = 64 * kw;
             plan->lds_bytes = lds;
-            plan->workspace_bytes = split > 1 ? gptq::kCounterBytes + (size_t)split * M * N * sizeof(float) : 0;
+            plan->workspace_bytes = split > 1 ? gptq::kCounterBytes + (size_t)split * M * N * sizeof(float)
+                                    : (halved ? gptq::kCounterBytes + gptq::tiled_decode_slot_bytes(halved, mr) : 0);
             return GPTQ_HIP_OK;
         }
         return GPTQ_HIP_ERR_UNSUPPORTED;

@@ -214,8 +214,18 @@ int launch_tile_prepare(const uint32_t *qweight, const uint32_t *qzeros, const v
                         uint32_t *qtile, uint32_t *sz, int32_t *xsrc, uint16_t *kinv, int K, int N, int G, int bits,
                         int group_size, void *stream);
 int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, const uint16_t *kinv, const void *bias,
-                        void *y, float *partial, int M, int K, int N, int G, int bits, int group_size,
-                        const gptq_hip_plan &plan, void *stream);
+                        void *y, float *partial, unsigned long long *slots, int M, int K, int N, int G, int bits,
+                        int group_size, const gptq_hip_plan &plan, void *stream);
+// tiles of the workgroup-per-tile decode kernel that are halved along K so that no CU holds two whole tiles
+// (more tiles than CUs, fewer than two per CU; the halves pair their blocks up where whole tiles do)
+inline int tiled_decode_halved(int tiles, int wave_steps, int split_k, int waves_k, int S_total)
+{
+    if (split_k != 1 || tiles <= kNumCUs || tiles >= 2 * kNumCUs || wave_steps % 4 != 0) return 0;
+    if (waves_k * (wave_steps / 2) >= S_total) return 0;   // the second half must start inside K
+    return tiles - kNumCUs;
+}
+// workspace of those tiles: one 64-bit slot per output of a halved tile, behind the counters
+inline size_t tiled_decode_slot_bytes(int halved, int mr) { return (size_t)halved * mr * 32 * 8; }
 int launch_tiled_decode16(const void *x, const void *qtile, const uint32_t *sz, const uint16_t *kinv, const void *bias,
                           void *y, int M, int K, int N, int G, int bits, int group_size, const gptq_hip_plan &plan,
                           void *stream);

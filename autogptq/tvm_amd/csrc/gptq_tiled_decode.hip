@@ -42,6 +42,7 @@ struct DecodeParams {
     int M, K, N, G;
     int S_total, T_total;
     int wave_steps;         // blocks (64 positions) per wave
+    unsigned long long *slots;  // halved tiles (grid_x > T_total): [tile - first halved][MR][32] (tag << 32 | fp32 bits), zero between launches
     int split_k;
     int lb_per_group;       // group_size / 32
     uint32_t lbg_magic;     // lane block -> group: umulhi(lb, magic) + (add ? lb : 0)
@@ -61,11 +62,22 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, h = lane >> 5;
-    const int T = blockIdx.x;
-    const int split = blockIdx.y;
-    const int wg_steps = p.wave_steps * KW;              // blocks of the workgroup's K range
+    // With more tiles than CUs but fewer than two per CU, the last e = tiles - CUs tiles are HALVED along K
+    // (grid_x = tiles + e): the first tiles - e workgroups take a whole tile each, one per CU, and the 2 e
+    // workgroups after them half a tile, so that no CU holds more than a tile and a half (two whole tiles on 88
+    // of the 256 CUs bound both the memory and the instruction path of 11008 columns).  The two halves of a tile
+    // meet through one 64-bit exchange per output (see the end of the kernel); they finish early, so that round
+    // trip lies under the walk of the whole tiles.
+    const int n_halved = (int)gridDim.x - p.T_total;     // e (0: no tile is halved)
+    const int n_whole = p.T_total - n_halved;
+    const bool is_half = (int)blockIdx.x >= n_whole;
+    const int half_i = (int)blockIdx.x - n_whole;        // (halved tile, half) = (half_i / 2, half_i % 2)
+    const int T = is_half ? n_whole + (half_i >> 1) : (int)blockIdx.x;
+    const int split = is_half ? (half_i & 1) : (int)blockIdx.y;
+    const int ws = is_half ? p.wave_steps / 2 : p.wave_steps;   // blocks per wave (the plan keeps the half even where blocks pair up)
+    const int wg_steps = ws * KW;                        // blocks of the workgroup's K range
     const int S_wg = split * wg_steps;                   // its first block
-    const int S_begin = S_wg + wave * p.wave_steps;      // this wave's first block
+    const int S_begin = S_wg + wave * ws;                // this wave's first block
     const int S_last = p.S_total - 1;
     const int span = wg_steps * 64;                      // positions the workgroup stages
     const int p0 = S_wg * 64;                            // its first position
@@ -109,7 +121,7 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     const uint32_t b_lane = tile_lane_bytes<BITS>((uint32_t)lane);
     const uint32_t tile_off = (uint32_t)T * (uint32_t)p.S_total;
     uint32_t w[2][PF][BITS];
-    const int steps = min(p.wave_steps, max(p.S_total - S_begin, 0));  // blocks of this wave that lie inside K
+    const int steps = min(ws, max(p.S_total - S_begin, 0));  // blocks of this wave that lie inside K
     auto load_w = [&](int i, uint32_t (&wr)[BITS]) {
         // block i of the wave's range; past its end: its first block again (a cache hit that is never multiplied)
         const int Sc = min(S_begin + (i < steps ? i : 0), S_last);
@@ -179,10 +191,10 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
         // a lane sums 16 consecutive positions; a run of 32 positions (one half of one block) is two lanes,
         // a unit-half 2 E lanes: l, l + 1 (the other half of the run) and, E = 2, l + 4, l + 5 (the other block)
         const int sb0 = S_begin - S_wg;
-        for (int q0 = 0; q0 < 4 * p.wave_steps; q0 += 64) {   // 16-position pieces of the wave's range
+        for (int q0 = 0; q0 < 4 * ws; q0 += 64) {   // 16-position pieces of the wave's range
             const int piece = q0 + lane;
             const int sb = sb0 + (piece >> 2), hh = (piece >> 1) & 1;
-            const bool live = piece < 4 * p.wave_steps;
+            const bool live = piece < 4 * ws;
 #pragma unroll
             for (int m = 0; m < MR; m++) {
                 float X = 0.f, B = 0.f;
@@ -295,14 +307,14 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     auto chunk = [&](int c, uint32_t (&wc)[PF][BITS], auto all_c) {
         constexpr bool ALL = decltype(all_c)::value;
         [&]<int... U>(std::integer_sequence<int, U...>) {
-            ((ALL || c + U < p.wave_steps
+            ((ALL || c + U < ws
                   ? block(std::integral_constant<int, U % E>{}, S_begin + c + U, wc[U], xr[U & 1], xr[(U + 1) & 1])
                   : (void)0),
              ...);
         }(std::make_integer_sequence<int, PF>{});
     };
     int c = 0;
-    for (; c + 2 * PF <= p.wave_steps; c += 2 * PF) {
+    for (; c + 2 * PF <= ws; c += 2 * PF) {
         chunk(c, w[0], std::true_type{});
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -314,7 +326,7 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
         for (int u = 0; u < PF; u++) load_w(c + 3 * PF + u, w[1][u]);
         __builtin_amdgcn_sched_barrier(0);
     }
-    if (c < p.wave_steps) {   // what is left of the range: fewer than two chunks, nothing more to request
+    if (c < ws) {   // what is left of the range: fewer than two chunks, nothing more to request
         chunk(c, w[0], std::false_type{});
         chunk(c + PF, w[1], std::false_type{});
     }
@@ -333,7 +345,21 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
             float sum = 0.f;
             for (int k = 0; k < KW; k++) sum += red[(k * MR + m) * 32 + nn];
             const size_t o = (size_t)m * p.N + 32 * T + nn;
-            if (p.split_k == 1) {
+            if (is_half) {
+                // One 64-bit exchange per output carries the half's sum and a tag: the half that finds the slot
+                // empty leaves its sum there; the other finds it, adds (a + b = b + a: the result does not depend on
+                // which half came first), writes y and empties the slot for the next launch.  The payload travels
+                // inside the atomic itself, so no other ordering is needed.
+                unsigned long long *slot = p.slots + ((size_t)(T - n_whole) * MR + m) * 32 + nn;
+                const unsigned long long mine = (1ull << 32) | (unsigned long long)__builtin_bit_cast(uint32_t, sum);
+                const unsigned long long old = __hip_atomic_exchange(slot, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((old >> 32) != 0ull) {
+                    float total = sum + __builtin_bit_cast(float, (uint32_t)old);
+                    if (p.bias) total += (float)((const _Float16 *)p.bias)[32 * T + nn];
+                    ((_Float16 *)p.y)[o] = (_Float16)total;
+                    __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            } else if (p.split_k == 1) {
                 if (p.bias) sum += (float)((const _Float16 *)p.bias)[32 * T + nn];
                 ((_Float16 *)p.y)[o] = (_Float16)sum;
             } else {
@@ -370,8 +396,8 @@ static int launch_decode_kw(const DecodeParams &p, const gptq_hip_plan &plan, hi
 
 // The decode product on the tiled format: one launch, plus a reduce pass when K is split over workgroups.
 int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, const uint16_t *kinv, const void *bias,
-                        void *y, float *partial, int M, int K, int N, int G, int bits, int group_size,
-                        const gptq_hip_plan &plan, void *stream_v)
+                        void *y, float *partial, unsigned long long *slots, int M, int K, int N, int G, int bits,
+                        int group_size, const gptq_hip_plan &plan, void *stream_v)
 {
     hipStream_t stream = (hipStream_t)stream_v;
     DecodeParams p;
@@ -389,6 +415,7 @@ int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, co
     p.S_total = (K + 63) / 64;
     p.T_total = N / 32;
     p.wave_steps = plan.k_chunk;
+    p.slots = slots;
     p.split_k = plan.split_k;
     p.lb_per_group = group_size / 32;
     // lane block -> group as a multiply-high (lane blocks are below 2^16 / 32 * 2)
@@ -397,7 +424,9 @@ int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, co
     const int mr = tiled_decode_rows(M);
     int rc = GPTQ_HIP_ERR_UNSUPPORTED;
     // two blocks per epilogue where every unit of two blocks lies in one group
-    const bool pairs = group_size % 128 == 0 && plan.k_chunk % 2 == 0;
+    // (halved tiles, grid_x > tiles: their waves walk k_chunk / 2 blocks, which must pair up as well)
+    const bool halved = plan.grid_x > N / 32;
+    const bool pairs = group_size % 128 == 0 && plan.k_chunk % (halved ? 4 : 2) == 0;
 #define GPTQ_DECODE_CASE(B, R) \
     if (bits == B && mr == R) rc = pairs ? launch_decode_kw<B, R, 2>(p, plan, stream) : launch_decode_kw<B, R, 1>(p, plan, stream)
     GPTQ_DECODE_CASE(4, 1);

@@ -62,10 +62,12 @@ def check_shapes(qweight, qzeros, scales, g_idx, bias, bits: int, group_size: in
 _workspaces = {}
 
 
-def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    """A zero-initialised workspace per (device, stream), grown on demand.  The kernels leave
-    its counters at zero, so it is cleared only when it is (re)allocated."""
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+def _workspace(device: torch.device, nbytes: int, kind: int = 0) -> torch.Tensor:
+    """A zero-initialised workspace per (device, stream) and kind, grown on demand.  The kernels leave
+    its counters at zero, so it is cleared only when it is (re)allocated.  kind 1: the decode plans of the
+    tiled family with halved tiles, whose kernel keeps ALL their bytes zero between launches (the slots through
+    which the two halves of a tile meet); they do not share the workspace other plans pack x or partial sums into."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream, kind)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
@@ -257,7 +259,8 @@ def gemm_tiled(x: torch.Tensor, qtile: torch.Tensor, sz: torch.Tensor, xsrc: Opt
         return out
     if plan is None:
         plan = _lib.select_tiled(M, K, N, bits, group_size)
-    ws = _workspace(dev, plan.workspace_bytes) if plan.workspace_bytes else None
+    slots = plan.kernel == _lib.KERNEL_TILED_DECODE and plan.split_k == 1   # (halved tiles: a workspace of their own)
+    ws = _workspace(dev, plan.workspace_bytes, 1 if slots else 0) if plan.workspace_bytes else None
     with torch.cuda.device(dev):
         rc = _lib.lib().gptq_hip_gemm_tiled(_ptr(x), _ptr(qtile), _ptr(sz), _ptr(xsrc), _ptr(kinv), _ptr(bias), _ptr(out),
                                             _ptr(ws), ws.numel() if ws is not None else 0, M, K, N, bits, group_size,

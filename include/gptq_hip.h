@@ -215,7 +215,10 @@ int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int group_size, 
  * (pycuda_warpper.py:138, qlinear_tvm.py:123,150).  x and y are in the layer's own channel order (xsrc = kinv =
  * NULL means no activation order; pass both or neither).  plan: NULL = gptq_hip_select_tiled.  workspace:
  * plan.workspace_bytes (none for most decode plans).  M <= 4: one launch (the decode kernel); above: two
- * (pack pass, matmul); one more when the plan splits K.
+ * (pack pass, matmul); one more when the plan splits K.  A decode plan (GPTQ_HIP_KERNEL_TILED_DECODE) with split_k = 1 that asks
+ * for a workspace wants ALL its bytes zero at the first call and leaves them zero (the two halves of a tile that
+ * is halved along K meet in 64-bit slots behind the counters): give such plans a workspace of their own, which no
+ * other entry point writes between the calls.
  */
 int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint32_t *sz, const int32_t *xsrc, const uint16_t *kinv,
                         const void *bias, void *y, void *workspace, size_t workspace_bytes, int M, int K, int N,

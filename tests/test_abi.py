@@ -301,7 +301,17 @@ def test_tiled_plans_are_consistent(bits, KN):
             if p.waves_n == 2:       # a workgroup per CU, 16-column units, sixteen waves over the 128-position blocks
                 assert p.block == 1024 and 1 <= p.grid_x <= min(N // 16, 256) and p.k_chunk * 16 >= -(-blocks // 2)
             else:                    # a workgroup per 32-column tile
-                assert p.grid_x == N // 32 and p.split_k * p.waves_k * p.k_chunk >= blocks
+                tiles = N // 32
+                # (more tiles than CUs, fewer than two per CU: the tiles past the 256th run as two halves along K,
+                # which meet in 64-bit slots behind the counters of the workspace)
+                halved = p.grid_x - tiles
+                assert halved in (0, tiles - 256) and p.split_k * p.waves_k * p.k_chunk >= blocks
+                if halved:
+                    assert 256 < tiles < 512 and p.split_k == 1 and p.k_chunk % 4 == 0
+                    assert p.waves_k * (p.k_chunk // 2) < blocks
+                    assert p.workspace_bytes == 16384 + halved * p.row_tiles * 32 * 8
+                elif p.split_k == 1:
+                    assert p.workspace_bytes == 0
         else:
             assert p.kernel == _lib.KERNEL_TILED
             cols = 64 * p.waves_n

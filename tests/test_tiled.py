@@ -29,9 +29,7 @@ def tile_decode_plan(M, K, N, bits, gs):
     """The plan of the workgroup-per-tile decode kernel (the family's choice when x does not fit the LDS of the
     one-workgroup-per-CU kernel), made by hand so that both kernels are tested on every shape."""
     plan = _lib.select_tiled(M, K, N, bits, gs, decode=True)
-    if plan.waves_n != 2:
-        return plan
-    return tile_decode_plan_of(plan, M, K, N, bits, gs)
+    return tile_decode_plan_of(plan, M, K, N, bits, gs)   # (a workgroup per whole tile, whatever the family halves)
 
 
 def tile_decode_plan_of(plan, M, K, N, bits, gs):
