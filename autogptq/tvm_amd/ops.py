@@ -348,11 +348,13 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
         11008 x 4096: 9.5-9.7 / 12.7-14.4 against 9.4-13.3 / 12.7-15.3;
       * up to 4 rows, wider layers (a workgroup per 32 columns, x staged per workgroup, four to sixteen waves
         along K so that a wave walks about sixteen blocks):
-        K = 4096: at most two rows, for 4-bit layers and for two rows under an activation order.  4096 x 11008
-        with an activation order, one / two rows: int4 7.9 / 8.8 against 8.0 / 10.9, int3 7.9 / 8.7 against
-        7.7 / 10.1; without: int4 8.2 / 8.5 against 7.9 / 8.8, int3 7.9 / 8.2 against 7.4 / 8.3; three and four
-        rows are level or behind; from 16384 columns on also int3 (4096 x 22016 int3 / int4 9.7 / 10.3 against
-        11.4 / 12.8);
+        K = 4096: one and two rows always, three and four up to 16384 columns.  With 257 to 511 tiles the tiles
+        past one per CU run as two halves along K (a tagged 64-bit exchange joins them), so that no CU holds two
+        whole tiles.  4096 x 11008, one / two / four rows, with an activation order: int4 7.8 / 8.1 / 9.8 against
+        8.1 / 11.0 / 11.1, int3 7.3 / 7.7 / 9.7 against 7.7 / 10.2 / 10.3; without: int4 7.8 / 8.1 / 8.7 against
+        7.9 / 8.8 / 8.9, int3 7.2 / 7.5 / 8.2 against 7.3 / 8.3 / 8.2; 4096 x 12288 int4 8.3 / 8.5 / 10.1 against
+        8.2 / 11.0 / 11.1; 4096 x 14336 int4 9.0 / 9.4 / 11.2 against 9.0 / 11.2 / 11.1; 4096 x 22016 int3 / int4,
+        one row, 9.7 / 10.3 against 11.4 / 12.8;
         longer K, one and two rows: always up to K = 32768 (with an activation order, int4, one / two rows:
         5120 x 13824 9.7 / 10.5 against 18.2 / 15.2, 6656 x 17920 15.1 / 15.4 against 27.9 / 27.2, 8192 x 8192
         9.7 / 9.9 against 14.0 / 13.3, 8192 x 28672 24.6 / 26.4 against 32.3 / 30.2, 13824 x 5120 11.6 / 12.4
@@ -371,9 +373,7 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
         if N <= 4096:
             return True
         if K <= 4096:
-            if M <= 2 and N >= 16384:
-                return True
-            return M <= 2 and (bits == 4 or (act_order and M == 2))
+            return M <= 2 or N < 16384
         if K > 32768:
             return False
         if M <= 2:
