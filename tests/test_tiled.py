@@ -240,6 +240,31 @@ def test_tiled_decode_split_k(dev, bits, M):
         assert torch.equal(y, run_tiled(D, prep, plan=plan))
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
+@pytest.mark.parametrize("K,N,gs", [(1024, 8224, 128), (1024, 11008, 128), (1024, 16352, 128), (2048, 9600, 64),
+                                    (2048, 12288, -1)])
+@pytest.mark.parametrize("desc_act", [False, True])
+def test_tiled_decode_halved_tiles(dev, bits, K, N, gs, desc_act):
+    # 257 to 511 column tiles: the family's plan runs the tiles past the 256th as two halves along K that meet
+    # through the exchange slots of a workspace of their own; the slots are zero again after every call, so the
+    # same workspace serves every row count in turn
+    L = layer(8100 + bits, K, N, bits, gs, desc_act, M=4, bias=True)
+    D = to_dev(L, dev)
+    w16 = expected_weight(L)
+    prep = prepare(D)
+    for M in (1, 4, 2, 3, 1):
+        plan = _lib.select_tiled(M, K, N, bits, gs)
+        assert plan.kernel == _lib.KERNEL_TILED_DECODE and plan.split_k == 1
+        assert plan.grid_x == 2 * (N // 32) - 256 and plan.workspace_bytes > 16384, "the plan does not halve any tile"
+        x = L["x"][:M].contiguous()
+        want = expected_output(L, x=x, w16=w16)
+        y = run_tiled(D, prep, x=x.to(dev), plan=plan)
+        what = f"halved tiles int{bits} {K}x{N} M={M}"
+        assert_close(y, want, what)
+        assert_tight(y, want, what)
+        assert torch.equal(y, run_tiled(D, prep, x=x.to(dev), plan=plan)), f"{what}: two identical calls differ"
+
+
 DECODE_FULL = [
     ("c1-int4-4096x4096", 4, 4096, 4096, 128, False, [1, 2, 4]),
     ("c2-int3-4096x11008-act", 3, 4096, 11008, 128, True, [1, 2, 3]),
