@@ -367,7 +367,7 @@ extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint3
         if (M > gptq::kDecodeMaxRows || mr != gptq::tiled_decode_rows(M)) return GPTQ_HIP_ERR_UNSUPPORTED;
         // grid_x: a workgroup per tile, or the planner's halved tiles on top
         const int halved = plan->grid_x - N / 32;
-        if (halved != 0 && halved != gptq::tiled_decode_halved(N / 32, plan->k_chunk, plan->split_k, kw, S_all))
+        if (halved != 0 && halved != gptq::tiled_decode_halved(N / 32, plan->k_chunk, plan->split_k, kw, S_all, gs))
             return GPTQ_HIP_ERR_BAD_ARG;
         if ((kw != 4 && kw != 8 && kw != 16) || plan->block != 64 * kw || plan->split_k < 1 || plan->k_chunk < 1 ||
             plan->grid_y != plan->split_k || plan->grid_z != 1 ||

@@ -536,8 +536,8 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
         for (int split = 1; split <= S_total; split++) {
             int wave_steps = ceil_div(S_total, split * kw);
             // an even number of blocks per wave keeps the paired epilogue (groups that are multiples of 128 channels)
-            // (rounding up to a multiple of four, so that more layers could halve their tiles, cost more than the
-            // halves gave: 5120 x 13824, ten blocks per wave, 9.7 -> 11.2 us with twelve and halved tiles)
+            // (rounding up to a multiple of four, so that halved tiles come out in equal halves, cost more than
+            // unequal halves do: 5120 x 13824, 9.7 -> 11.2 us with twelve blocks per wave instead of ten)
             if (gs % 128 == 0 && wave_steps > 1 && (wave_steps & 1) && split == 1) wave_steps++;
             if (ceil_div(S_total, wave_steps * kw) != split) continue;  // (the split this partition really needs)
             const int span = wave_steps * kw * 64;
@@ -552,9 +552,9 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
             plan->waves_k = kw;
             plan->split_k = split;
             plan->k_chunk = wave_steps;
-            // more tiles than CUs but fewer than two per CU: the last tiles - CUs tiles run as two halves along K,
-            // so that no CU holds two whole tiles (4096 x 11008: 344 tiles, 88 of them halved)
-            const int halved = gptq::tiled_decode_halved(tiles, wave_steps, split, kw, S_total);
+            // up to CUs / 2 tiles past a whole number per CU run as two halves along K, so that the fullest CU
+            // holds half a tile more than the others, not a whole one (4096 x 11008: 344 tiles, 88 of them halved)
+            const int halved = gptq::tiled_decode_halved(tiles, wave_steps, split, kw, S_total, gs);
             plan->grid_x = tiles + halved;
             plan->grid_y = split;
             plan->grid_z = 1;

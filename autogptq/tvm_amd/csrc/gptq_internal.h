@@ -216,13 +216,29 @@ int launch_tile_prepare(const uint32_t *qweight, const uint32_t *qzeros, const v
 int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, const uint16_t *kinv, const void *bias,
                         void *y, float *partial, unsigned long long *slots, int M, int K, int N, int G, int bits,
                         int group_size, const gptq_hip_plan &plan, void *stream);
-// tiles of the workgroup-per-tile decode kernel that are halved along K so that no CU holds two whole tiles
-// (more tiles than CUs, fewer than two per CU; the halves pair their blocks up where whole tiles do)
-inline int tiled_decode_halved(int tiles, int wave_steps, int split_k, int waves_k, int S_total)
+// the workgroup-per-tile decode kernel pairs the blocks of a wave up (one epilogue per two blocks) when groups
+// are multiples of 128 channels and a wave walks an even number of blocks
+constexpr bool tiled_decode_pairs(int group_size, int wave_steps) { return group_size % 128 == 0 && wave_steps % 2 == 0; }
+// halved tiles: blocks per wave of the first half (the larger one; an even count where blocks pair up), the
+// second half takes the rest
+constexpr int tiled_decode_first_half(int wave_steps, bool pairs)
 {
-    if (split_k != 1 || tiles <= kNumCUs || tiles >= 2 * kNumCUs || wave_steps % 4 != 0) return 0;
-    if (waves_k * (wave_steps / 2) >= S_total) return 0;   // the second half must start inside K
-    return tiles - kNumCUs;
+    return pairs ? 2 * ((wave_steps + 3) / 4) : (wave_steps + 1) / 2;
+}
+// tiles of the workgroup-per-tile decode kernel that are halved along K: the e tiles past a whole number per
+// CU, when their 2 e halves find a CU each (e <= CUs / 2), so that the fullest CU holds half a tile more than
+// the others instead of a whole one.  Both halves pair their blocks up where whole tiles do.  (With more
+// halves than CUs nothing is gained, and workgroups of eight waves lose: 5120 x 13824, 176 tiles halved,
+// 9.9 -> 11.4 us at one row, 12.8 -> 16.2 at four.)
+inline int tiled_decode_halved(int tiles, int wave_steps, int split_k, int waves_k, int S_total, int group_size)
+{
+    const int e = tiles % kNumCUs;
+    if (split_k != 1 || tiles <= kNumCUs || e == 0 || 2 * e > kNumCUs) return 0;
+    const bool pairs = tiled_decode_pairs(group_size, wave_steps);
+    const int first = tiled_decode_first_half(wave_steps, pairs);
+    if (wave_steps - first < (pairs ? 2 : 1)) return 0;    // nothing left for the second half
+    if (waves_k * first >= S_total) return 0;              // the second half must start inside K
+    return e;
 }
 // workspace of those tiles: one 64-bit slot per output of a halved tile, behind the counters
 inline size_t tiled_decode_slot_bytes(int halved, int mr) { return (size_t)halved * mr * 32 * 8; }

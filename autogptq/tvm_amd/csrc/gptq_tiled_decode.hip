@@ -62,21 +62,23 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, h = lane >> 5;
-    // With more tiles than CUs but fewer than two per CU, the last e = tiles - CUs tiles are HALVED along K
-    // (grid_x = tiles + e): the first tiles - e workgroups take a whole tile each, one per CU, and the 2 e
-    // workgroups after them half a tile, so that no CU holds more than a tile and a half (two whole tiles on 88
-    // of the 256 CUs bound both the memory and the instruction path of 11008 columns).  The two halves of a tile
-    // meet through one 64-bit exchange per output (see the end of the kernel); they finish early, so that round
-    // trip lies under the walk of the whole tiles.
+    // The e tiles past a whole number per CU (the planner: when e is at most half the CUs) are HALVED along K
+    // (grid_x = tiles + e): the first tiles - e workgroups take a whole tile each and the 2 e workgroups after
+    // them half a tile, so that the fullest CU holds half a tile more than the others instead of a whole one
+    // (two whole tiles on 88 of the 256 CUs bound both the memory and the instruction path of 11008 columns).
+    // The two halves of a tile meet through one 64-bit exchange per output (see the end of the kernel).
     const int n_halved = (int)gridDim.x - p.T_total;     // e (0: no tile is halved)
     const int n_whole = p.T_total - n_halved;
     const bool is_half = (int)blockIdx.x >= n_whole;
     const int half_i = (int)blockIdx.x - n_whole;        // (halved tile, half) = (half_i / 2, half_i % 2)
     const int T = is_half ? n_whole + (half_i >> 1) : (int)blockIdx.x;
     const int split = is_half ? (half_i & 1) : (int)blockIdx.y;
-    const int ws = is_half ? p.wave_steps / 2 : p.wave_steps;   // blocks per wave (the plan keeps the half even where blocks pair up)
+    // blocks per wave: all of them, or the first half's share (rounded up, to an even count where blocks pair
+    // up) and the rest for the second half
+    const int ws_first = tiled_decode_first_half(p.wave_steps, E == 2);
+    const int ws = is_half ? (split ? p.wave_steps - ws_first : ws_first) : p.wave_steps;
     const int wg_steps = ws * KW;                        // blocks of the workgroup's K range
-    const int S_wg = split * wg_steps;                   // its first block
+    const int S_wg = is_half ? split * ws_first * KW : split * wg_steps;   // its first block
     const int S_begin = S_wg + wave * ws;                // this wave's first block
     const int S_last = p.S_total - 1;
     const int span = wg_steps * 64;                      // positions the workgroup stages
@@ -424,9 +426,8 @@ int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, co
     const int mr = tiled_decode_rows(M);
     int rc = GPTQ_HIP_ERR_UNSUPPORTED;
     // two blocks per epilogue where every unit of two blocks lies in one group
-    // (halved tiles, grid_x > tiles: their waves walk k_chunk / 2 blocks, which must pair up as well)
-    const bool halved = plan.grid_x > N / 32;
-    const bool pairs = group_size % 128 == 0 && plan.k_chunk % (halved ? 4 : 2) == 0;
+    // (halved tiles, grid_x > tiles: their waves walk the two even shares of k_chunk that the planner checked)
+    const bool pairs = tiled_decode_pairs(group_size, plan.k_chunk);
 #define GPTQ_DECODE_CASE(B, R) \
     if (bits == B && mr == R) rc = pairs ? launch_decode_kw<B, R, 2>(p, plan, stream) : launch_decode_kw<B, R, 1>(p, plan, stream)
     GPTQ_DECODE_CASE(4, 1);

@@ -348,9 +348,9 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
         11008 x 4096: 9.5-9.7 / 12.7-14.4 against 9.4-13.3 / 12.7-15.3;
       * up to 4 rows, wider layers (a workgroup per 32 columns, x staged per workgroup, four to sixteen waves
         along K so that a wave walks about sixteen blocks):
-        K = 4096: one and two rows always, three and four up to 16384 columns.  With 257 to 511 tiles the tiles
-        past one per CU run as two halves along K (a tagged 64-bit exchange joins them), so that no CU holds two
-        whole tiles.  4096 x 11008, one / two / four rows, with an activation order: int4 7.8 / 8.1 / 9.8 against
+        K = 4096: one and two rows always, three and four up to 16384 columns.  Up to 128 tiles past a whole number
+        per CU run as two halves along K (a tagged 64-bit exchange joins them), so that the fullest CU holds half
+        a tile more than the others, not a whole one.  4096 x 11008, one / two / four rows, with an activation order: int4 7.8 / 8.1 / 9.8 against
         8.1 / 11.0 / 11.1, int3 7.3 / 7.7 / 9.7 against 7.7 / 10.2 / 10.3; without: int4 7.8 / 8.1 / 8.7 against
         7.9 / 8.8 / 8.9, int3 7.2 / 7.5 / 8.2 against 7.3 / 8.3 / 8.2; 4096 x 12288 int4 8.3 / 8.5 / 10.1 against
         8.2 / 11.0 / 11.1; 4096 x 14336 int4 9.0 / 9.4 / 11.2 against 9.0 / 11.2 / 11.1; 4096 x 22016 int3 / int4,

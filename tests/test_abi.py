@@ -302,13 +302,15 @@ def test_tiled_plans_are_consistent(bits, KN):
                 assert p.block == 1024 and 1 <= p.grid_x <= min(N // 16, 256) and p.k_chunk * 16 >= -(-blocks // 2)
             else:                    # a workgroup per 32-column tile
                 tiles = N // 32
-                # (more tiles than CUs, fewer than two per CU: the tiles past the 256th run as two halves along K,
-                # which meet in 64-bit slots behind the counters of the workspace)
+                # (the tiles past a whole number per CU, when there are at most 128 of them, run as two halves
+                # along K, which meet in 64-bit slots behind the counters of the workspace)
                 halved = p.grid_x - tiles
-                assert halved in (0, tiles - 256) and p.split_k * p.waves_k * p.k_chunk >= blocks
+                assert halved in (0, tiles % 256) and p.split_k * p.waves_k * p.k_chunk >= blocks
                 if halved:
-                    assert 256 < tiles < 512 and p.split_k == 1 and p.k_chunk % 4 == 0
-                    assert p.waves_k * (p.k_chunk // 2) < blocks
+                    assert tiles > 256 and halved <= 128 and p.split_k == 1
+                    pairs = (K if gs == -1 else gs) % 128 == 0 and p.k_chunk % 2 == 0
+                    first = 2 * ((p.k_chunk + 3) // 4) if pairs else (p.k_chunk + 1) // 2
+                    assert p.k_chunk - first >= (2 if pairs else 1) and p.waves_k * first < blocks
                     assert p.workspace_bytes == 16384 + halved * p.row_tiles * 32 * 8
                 elif p.split_k == 1:
                     assert p.workspace_bytes == 0

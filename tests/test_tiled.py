@@ -241,13 +241,14 @@ def test_tiled_decode_split_k(dev, bits, M):
 
 
 @pytest.mark.parametrize("bits", [2, 3, 4, 8])
-@pytest.mark.parametrize("K,N,gs", [(1024, 8224, 128), (1024, 11008, 128), (1024, 16352, 128), (2048, 9600, 64),
-                                    (2048, 12288, -1)])
+@pytest.mark.parametrize("K,N,gs", [(1024, 8224, 128), (1024, 11008, 128), (1280, 12288, 128), (2048, 9600, 64),
+                                    (2048, 12288, -1), (640, 18368, 128), (1152, 9216, 32)])
 @pytest.mark.parametrize("desc_act", [False, True])
 def test_tiled_decode_halved_tiles(dev, bits, K, N, gs, desc_act):
-    # 257 to 511 column tiles: the family's plan runs the tiles past the 256th as two halves along K that meet
-    # through the exchange slots of a workspace of their own; the slots are zero again after every call, so the
-    # same workspace serves every row count in turn
+    # Up to 128 column tiles past a whole number per CU (256): the family's plan runs them as two halves along K
+    # (equal, or the first one larger: 1280 and 1152 channels) that meet through the exchange slots of a
+    # workspace of their own; the slots are zero again after every call, so the same workspace serves every row
+    # count in turn
     L = layer(8100 + bits, K, N, bits, gs, desc_act, M=4, bias=True)
     D = to_dev(L, dev)
     w16 = expected_weight(L)
@@ -255,7 +256,7 @@ def test_tiled_decode_halved_tiles(dev, bits, K, N, gs, desc_act):
     for M in (1, 4, 2, 3, 1):
         plan = _lib.select_tiled(M, K, N, bits, gs)
         assert plan.kernel == _lib.KERNEL_TILED_DECODE and plan.split_k == 1
-        assert plan.grid_x == 2 * (N // 32) - 256 and plan.workspace_bytes > 16384, "the plan does not halve any tile"
+        assert plan.grid_x == N // 32 + (N // 32) % 256 and plan.workspace_bytes > 16384, "the plan does not halve any tile"
         x = L["x"][:M].contiguous()
         want = expected_output(L, x=x, w16=w16)
         y = run_tiled(D, prep, x=x.to(dev), plan=plan)
