@@ -621,17 +621,19 @@ def test_bad_g_idx_is_rejected_by_the_module(dev):
 
 
 @pytest.mark.parametrize("bits", [3, 4])
-def test_module_forward_replays_in_a_graph(dev, bits):
-    """Decoding loops replay a captured graph: the module's calls (sorted decode, small batch behind the
+@pytest.mark.parametrize("K,N", [(2048, 4096), (1024, 11008)])
+def test_module_forward_replays_in_a_graph(dev, bits, K, N):
+    """Decoding loops replay a captured graph: the module's calls (decode kernels, among them the one whose
+    halved tiles meet in the slots of a workspace of their own (11008 columns), small batch behind the
     reorder pass, pack pass + matmul + reduce pass) must give the eager result on every replay, with the
     program's own eager work between replays."""
-    K, N, gs = 2048, 4096, 128
+    gs = 128
     L = layer(970 + bits, K, N, bits, gs, True, M=40, bias=True)
     q = QuantLinear(bits, gs, K, N, True)
     q.load_state_dict({k: L[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})
     q = q.to(dev)
     gen = torch.Generator().manual_seed(12)
-    xs = {M: torch.randn(M, K, generator=gen).half().to(dev) for M in (1, 8, 40)}
+    xs = {M: torch.randn(M, K, generator=gen).half().to(dev) for M in (1, 4, 8, 40)}
     for M in xs:          # eager first: workspaces and the sorted copy are allocated outside the capture
         q(xs[M])
     torch.cuda.synchronize(dev)
@@ -655,6 +657,38 @@ def test_module_forward_replays_in_a_graph(dev, bits):
         for M in xs:
             assert torch.equal(outs[M], want[M]), (rep, M)
             assert_close(outs[M], expected_output(L, x=xs[M].cpu()), f"graph replay {rep}, M={M}")
+
+
+def test_module_runs_on_two_streams_at_once(dev):
+    """Two host streams run the same layers back to back without waiting for each other: every (device, stream)
+    has workspaces of its own (also the one whose exchange slots the halved tiles of 11008 columns use), so the
+    results equal those of one stream alone."""
+    K, gs = 1024, 128
+    layers = []
+    for i, (bits, N) in enumerate(((4, 11008), (3, 11008), (4, 4096))):
+        L = layer(1200 + i, K, N, bits, gs, True, M=40, bias=True)
+        q = QuantLinear(bits, gs, K, N, True)
+        q.load_state_dict({k: L[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})
+        layers.append((L, q.to(dev)))
+    gen = torch.Generator().manual_seed(5)
+    xs = {M: torch.randn(M, K, generator=gen).half().to(dev) for M in (1, 4, 40)}
+    want = {(i, M): q(x).clone() for i, (L, q) in enumerate(layers) for M, x in xs.items()}
+    torch.cuda.synchronize(dev)
+    streams = [torch.cuda.Stream(device=dev) for _ in range(2)]
+    got = [{}, {}]
+    for rep in range(6):
+        for si, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                for i, (L, q) in enumerate(layers):
+                    for M, x in xs.items():
+                        got[si][(i, M, rep)] = q(x)
+    torch.cuda.synchronize(dev)
+    for si in range(2):
+        for (i, M, rep), y in got[si].items():
+            assert torch.equal(y, want[(i, M)]), (si, i, M, rep)
+    for i, (L, q) in enumerate(layers):
+        for M, x in xs.items():
+            assert_close(want[(i, M)], expected_output(L, x=x.cpu()), f"layer {i}, M={M}")
 
 
 def test_torch_operator_equals_the_python_front_end(dev):
