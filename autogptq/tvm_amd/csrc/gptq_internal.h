@@ -178,6 +178,16 @@ constexpr int tiled_ring(int at) { return at >= 4 ? 3 : (at == 2 ? 4 : 6); }
 inline int tiled_pack_blocks(int split_k, int waves_k, int wave_steps) { return split_k * waves_k * wave_steps; }
 // LDS of a workgroup: the result tiles (32 x 32 floats, two per 32 rows) of its waves
 inline int tiled_lds_bytes(int row_tiles, int waves_k) { return waves_k * row_tiles * 2 * 4096; }
+// the matmul kernel reads its x fragments from x itself, without the pack pass: up to 16 rows of layers without an
+// activation order, when K is a whole number of blocks that the waves' ranges cover exactly (no zero padding is
+// read)
+constexpr int kTiledDirectRows = 16;
+inline bool tiled_reads_x_directly(bool act_order, int M, int K, const gptq_hip_plan &plan)
+{
+    return !act_order && M <= kTiledDirectRows && plan.kernel == GPTQ_HIP_KERNEL_TILED && plan.row_tiles == 1 &&
+           plan.m_blocks == 1 && plan.waves_n == 1 && K % 64 == 0 &&
+           plan.split_k * plan.waves_k * plan.k_chunk == K / 64;
+}
 // the transposed product: the result tiles, or the table of (scale, base + zero) pairs of the workgroup's K range
 // for its two column tiles (256 bytes per block and tile), whichever is larger: they share the memory
 inline int tiled_t_lds_bytes(int row_tiles, int waves_k, int wave_steps)

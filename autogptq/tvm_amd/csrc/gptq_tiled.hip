@@ -233,6 +233,9 @@ struct TiledParams {
     const uint32_t *szt;   // [G][S_total][8 octets][8 words]: per octet of columns, (scale, scale) x 4 | (base + zero) x 4
     const int32_t *out_map;  // channel of sorted position p (nullptr = identity): where column p of the result goes
     int tiles_per_group;   // group_size / 32: output tiles (32 positions) per group
+    // DIRECT: the A fragments are read from x itself (no pack pass)
+    const _Float16 *x;     // fp16 [M, K]
+    int K;
 };
 
 // One B operand: positions 8 j .. 8 j + 7 of the lane, as fp16(scale * (q - zero)) exactly as the
@@ -276,7 +279,14 @@ __device__ __forceinline__ h8 tiled_bop_t(const uint32_t (&w)[BITS], int j, cons
 // per octet of columns; the workgroup copies the part of its tiles' groups and of its K range into LDS, and
 // every operand reads its 32 bytes from there, one operand ahead of the arithmetic.  The weights are formed
 // exactly as in the forward product.  The result's column p goes to channel out_map[p].
-template <int BITS, int AT, int RW, int KW, int RING, int CT, bool TRANS = false>
+// DIRECT: no pack pass.  Without an activation order position p is channel p, so lane (m, h) of fragment (S, j) finds
+// its eight values in row m of x at 64 S + 32 h + 8 j: sixteen bytes of a 128-byte line that the lane's other seven
+// fragments of the block share.  Rows past M read row M - 1 (a row of the result depends on its own row of x only,
+// and those rows are never stored), so a wave's load touches M lines; the launcher takes this form up to 16 rows
+// (4096 x 11008, us with / without the pack pass: 8 rows 14.0 / 10.7, 16 rows 14.5 / 11.5; with 32 distinct rows
+// per load 14.8 / 16.2, 64 rows 19 / 29.5: every lane then asks for a line of its own), and only when K is a whole
+// number of blocks that the waves' ranges cover exactly: there is no zero padding to read.
+template <int BITS, int AT, int RW, int KW, int RING, int CT, bool TRANS = false, bool DIRECT = false>
 __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledParams p)
 {
     const int tid = threadIdx.x;
@@ -316,10 +326,23 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledPar
             if constexpr (!TRANS) sr[ct] = p.sz[(size_t)g * p.N + col[ct]];
         }
     };
-    auto load_a = [&](int S, int j, h8 (&ar)[AT]) {
-        const char *src = p.xpack + (size_t)(4 * S + j) * a_frag_row + a_lane;
+    // DIRECT: the lane's rows of x, at its half of a block
+    const _Float16 *a_row[AT];
+    if constexpr (DIRECT) {
 #pragma unroll
-        for (int rt = 0; rt < AT; rt++) ar[rt] = __builtin_bit_cast(h8, *(const u4 *)(src + rt * 1024));
+        for (int rt = 0; rt < AT; rt++)
+            a_row[rt] = p.x + (size_t)min(32 * (rt0 + rt) + n, p.M - 1) * (size_t)p.K + 32 * h;
+    }
+    auto load_a = [&](int S, int j, h8 (&ar)[AT]) {
+        if constexpr (DIRECT) {
+            const int off = 64 * S + 8 * j;
+#pragma unroll
+            for (int rt = 0; rt < AT; rt++) ar[rt] = *(const h8 *)(a_row[rt] + off);
+        } else {
+            const char *src = p.xpack + (size_t)(4 * S + j) * a_frag_row + a_lane;
+#pragma unroll
+            for (int rt = 0; rt < AT; rt++) ar[rt] = __builtin_bit_cast(h8, *(const u4 *)(src + rt * 1024));
+        }
     };
 
     // Every workgroup starts its walk at another block of its waves' ranges and wraps around, so that the
@@ -563,10 +586,10 @@ int launch_tiled_reduce(const float *partial, const void *bias, void *y, int M, 
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 
-template <int BITS, int AT, int RW, int KW, int RING, int CT>
+template <int BITS, int AT, int RW, int KW, int RING, int CT, bool DIRECT = false>
 static int launch_tiled_one(const TiledParams &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
-    auto kern = tiled_gemm_kernel<BITS, AT, RW, KW, RING, CT>;
+    auto kern = tiled_gemm_kernel<BITS, AT, RW, KW, RING, CT, false, DIRECT>;
     const int lds_bytes = tiled_lds_bytes(AT * RW, KW);
     if (plan.lds_bytes < lds_bytes || plan.waves_k != KW || plan.block != 64 * RW * KW) return GPTQ_HIP_ERR_BAD_ARG;
     if (lds_bytes > 65536) {
@@ -605,22 +628,37 @@ int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int
     p.szt = nullptr;
     p.out_map = nullptr;
     p.tiles_per_group = 1;
+    p.x = (const _Float16 *)x;
+    p.K = K;
     const int S_pack = tiled_pack_blocks(plan.split_k, plan.waves_k, plan.k_chunk);
-    const int pack_lds = xsrc ? K * 2 : 0;  // one row of x
-    if (pack_lds > 65536) {
-        if (hipFuncSetAttribute((const void *)tile_pack_x_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, pack_lds) !=
-            hipSuccess) {
-            (void)hipGetLastError();
-            return GPTQ_HIP_ERR_LAUNCH;
+    // without an activation order the fragments can be read from x itself: one launch less
+    const bool direct = tiled_reads_x_directly(xsrc != nullptr, M, K, plan);
+    if (!direct) {
+        const int pack_lds = xsrc ? K * 2 : 0;  // one row of x
+        if (pack_lds > 65536) {
+            if (hipFuncSetAttribute((const void *)tile_pack_x_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    pack_lds) != hipSuccess) {
+                (void)hipGetLastError();
+                return GPTQ_HIP_ERR_LAUNCH;
+            }
         }
+        hipLaunchKernelGGL(tile_pack_x_kernel, dim3(32 * p.rt_total), dim3(256), pack_lds, stream, (const _Float16 *)x,
+                           xsrc, xpack, M, K, Kp, p.rt_total, S_pack);
+        if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ERR_LAUNCH;
     }
-    hipLaunchKernelGGL(tile_pack_x_kernel, dim3(32 * p.rt_total), dim3(256), pack_lds, stream, (const _Float16 *)x, xsrc,
-                       xpack, M, K, Kp, p.rt_total, S_pack);
-    if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ERR_LAUNCH;
     int rc = GPTQ_HIP_ERR_UNSUPPORTED;
 #define GPTQ_TILED_CASE(B, A)                                                                  \
     if (bits == B && plan.row_tiles == A && plan.waves_n == 1)                                 \
         rc = launch_tiled_one<B, A, 1, 4, tiled_ring(A), 2>(p, plan, stream)
+    if (direct) {
+        switch (bits) {
+            case 2: rc = launch_tiled_one<2, 1, 1, 4, tiled_ring(1), 2, true>(p, plan, stream); break;
+            case 3: rc = launch_tiled_one<3, 1, 1, 4, tiled_ring(1), 2, true>(p, plan, stream); break;
+            case 4: rc = launch_tiled_one<4, 1, 1, 4, tiled_ring(1), 2, true>(p, plan, stream); break;
+            case 8: rc = launch_tiled_one<8, 1, 1, 4, tiled_ring(1), 2, true>(p, plan, stream); break;
+            default: break;
+        }
+    } else {
     GPTQ_TILED_CASE(4, 1);
     GPTQ_TILED_CASE(4, 2);
     GPTQ_TILED_CASE(4, 4);
@@ -633,6 +671,7 @@ int launch_tiled(const void *x, const void *qtile, const uint32_t *sz, const int
     GPTQ_TILED_CASE(8, 1);
     GPTQ_TILED_CASE(8, 2);
     GPTQ_TILED_CASE(8, 4);
+    }
 #undef GPTQ_TILED_CASE
     // 128 x 128 per wave (waves_n = 2): a ring of two blocks
     if (plan.row_tiles == 4 && plan.waves_n == 2) {

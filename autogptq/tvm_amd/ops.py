@@ -364,7 +364,11 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
         longer K, three and four rows: K up to 6656 (5120 x 13824 12.8 against 15.4, 6656 x 17920 22.3 against
         26.8) and 8192 x 8192 (12.3 against 13.3); beyond, the four staged rows of x cost more than they save
         (8192 x 28672 41.9 against 30.4, 17920 x 6656 29.9 against 23.9);
-      * 5 to 16 rows: never (4096 x 11008, 8 rows: 14.6 against 13.4);
+      * 5 to 16 rows: only layers without an activation order, K up to 4096 and more than 4096 columns (the
+        matmul kernel then reads x itself, one launch; 4096 x 11008 int4, 5 / 8 / 16 rows: 10.6 / 10.7 / 11.5
+        against 11.2 / 11.3 / 12.5; int3 from nine rows: 11.5 against 12.8 at sixteen, 10.9 against 10.4 at
+        eight); with an activation order the pack pass makes it 14.6 against 13.4 at 8 rows, and narrower or
+        longer layers split K and add a pass (11008 x 4096: 17.3 against 13.1);
       * 17 to 128 rows: everywhere within 4 % or better (4096 x 11008 with an activation order, 32/64/128
         rows: 14.8/19.2/26.6 against 18.1/22.1/34.1);
       * above 128 rows: K up to 8192 (4096 x 11008, 512 rows: 75 against 95; 11008 x 4096: 127 against 81,
@@ -380,7 +384,7 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
             return not (bits == 3 and M == 1 and 8192 < K <= 12288 and N <= 12288)
         return K <= 6656 or (K <= 8192 and N <= 8192)
     if M <= 16:
-        return False
+        return not act_order and K <= 4096 and N > 4096 and (M >= 9 or bits == 4)
     return M <= 128 or K <= 8192
 
 

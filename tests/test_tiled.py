@@ -126,6 +126,26 @@ def test_tiled_odd_shapes(dev, bits, K, N, gs, M):
 
 
 @pytest.mark.parametrize("bits", [2, 3, 4, 8])
+@pytest.mark.parametrize("K,N,gs", [(1024, 416, 128), (4096, 352, 64), (2048, 11008, 128)])
+def test_tiled_small_batches_read_x_without_the_pack_pass(dev, bits, K, N, gs):
+    # 5 to 16 rows of a layer without an activation order: the matmul kernel reads its fragments from x itself.
+    # Handing the same layer over with its (identity) channel maps forces the pack pass: same fragments, so the
+    # two results are the same bits.
+    L = layer(2500 + bits, K, N, bits, gs, False, M=16, bias=True)
+    D = to_dev(L, dev)
+    qtile, sz, xsrc, kinv = prepare(D)
+    w16 = expected_weight(L)
+    for M in (5, 9, 16):
+        x = L["x"][:M].contiguous()
+        direct = ops.gemm_tiled(x.to(dev), qtile, sz, None, None, D["bias"], bits, gs)
+        packed = ops.gemm_tiled(x.to(dev), qtile, sz, xsrc, kinv, D["bias"], bits, gs)
+        want = expected_output(L, x=x, w16=w16)
+        assert_close(direct, want, f"direct M={M}")
+        assert_tight(direct, want, f"direct M={M}")
+        assert torch.equal(direct, packed), f"M={M}: reading x directly and through the pack pass differ"
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
 @pytest.mark.parametrize("split", [1, 2, 3, 5])
 @pytest.mark.parametrize("M", [20, 130])
 def test_tiled_forced_split_k(dev, bits, split, M):
