@@ -138,9 +138,11 @@ def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int =
         q = L["qweight"].to(dev) if c == 0 else torch.randint(
             -(1 << 31), (1 << 31) - 1, L["qweight"].shape, generator=gen, dtype=torch.int64).to(torch.int32).to(dev)
         if prepared == "tiled":
+            # (every copy brings its own scale / zero words and channel maps, as every layer of a model does)
             qtile, sz, xsrc, kinv = ops.tile_prepare(q, case["qzeros"], case["scales"], case["g_idx"], bits, gs)
+            case.setdefault("tiled_copies", []).append((sz, xsrc if desc_act else None, kinv if desc_act else None))
             if c == 0:
-                case["tiled"] = (sz, xsrc if desc_act else None, kinv if desc_act else None)
+                case["tiled"] = case["tiled_copies"][0]
             q = qtile
         qweights.append(q)
     case["qweights"] = qweights
@@ -148,6 +150,11 @@ def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int =
         qweights[0], case["kmap"] = sort_channels_by_group(qweights[0], case["g_idx"], bits, gs)
         case["g_idx"] = None
         desc_act = False  # the plan is that of contiguous groups
+    # the layer's other tensors, one set per copy as well (qzeros, scales, and g_idx or the sorted copy's map)
+    g_or_map = case["kmap"] if case["kmap"] is not None else case["g_idx"]
+    case["aux_copies"] = [(case["qzeros"], case["scales"], g_or_map)] + [
+        (case["qzeros"].clone(), case["scales"].clone(), g_or_map.clone() if g_or_map is not None else None)
+        for _ in range(copies - 1)]
     if prepared == "tiled":
         plan = _lib.select_tiled(M, K, N, bits, gs)
     elif prepared == "sorted" and not (kernel or split_k or waves_n):
@@ -220,19 +227,20 @@ def make_step(case, dev):
     planp = ctypes.byref(case["plan"])
     n = len(qws)
     if case["prepared"] == "tiled":
-        sz, xsrc, kinv = (ptr(t) for t in case["tiled"])
+        aux = [tuple(ptr(t) for t in c) for c in case["tiled_copies"]]
 
         def step(i, stream):
+            sz, xsrc, kinv = aux[i % n]
             rc = lib.gptq_hip_gemm_tiled(x, qws[i % n], sz, xsrc, kinv, None, y, ws, wsb, M, K, N, bits, gs, planp, stream)
             if rc != 0:
                 raise RuntimeError(f"gptq_hip_gemm_tiled failed: {_lib.strerror(rc)}")
 
         return step
     fn = lib.gptq_hip_gemm_sorted if case["kmap"] is not None else lib.gptq_hip_gemm_plan
-    qz, sc = ptr(case["qzeros"]), ptr(case["scales"])
-    g = ptr(case["kmap"] if case["kmap"] is not None else case["g_idx"])
+    aux = [tuple(ptr(t) for t in c) for c in case["aux_copies"]]
 
     def step(i, stream):
+        qz, sc, g = aux[i % n]
         rc = fn(x, qws[i % n], qz, sc, g, None, y, ws, wsb, M, K, N, bits, gs, planp, stream)
         if rc != 0:
             raise RuntimeError(f"gptq_hip_gemm failed: {_lib.strerror(rc)}")
