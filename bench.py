@@ -265,22 +265,26 @@ def scrub_cache(dev):
 def time_case(case, dev, steps: int, warmup: int):
     """Average duration of one step in microseconds: K steps captured once in a HIP graph and
     replayed inside one event-bracketed region (no host launch cost between the kernels; reported as
-    ``graph_us`` and as ``us``), plus the same K steps launched eagerly (``eager_us``).  The weight copy
-    of step i is (warmup + i) mod copies, continuing the warm-up's rotation, and the cache is scrubbed
-    right before every timed region (the region starts when the scrub kernel ends), so no timed step finds
-    its weights cached."""
+    ``graph_us`` and as ``us``), plus the same K steps launched eagerly (``eager_us``).  The W warm-up steps
+    run right in front of the timed ones, on the same stream with nothing in between, so that the K steps
+    start on a busy GPU (the first steps behind an idle or scrubbed GPU take ~2 us longer each: 5 steps
+    measure 8.8 us, steps 6 to 20 of 20 measure 7.0).  The weight copy of step i is (warmup + i) mod copies,
+    continuing the warm-up's rotation, and the cache is scrubbed before the warm-up of every timed region, so
+    no timed step finds its weights cached."""
     step = make_step(case, dev)
     stream = torch.cuda.Stream(device=dev)
     res = {}
     with torch.cuda.stream(stream):
         sp = ctypes.c_void_p(stream.cuda_stream)
-        for i in range(warmup):
+        for i in range(warmup):       # (first calls: lazy initialisation of the runtime for these kernels)
             step(i, sp)
-        scrub_cache(dev)
         stream.synchronize()
         # eager
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize(dev)
+        scrub_cache(dev)
+        for i in range(warmup):
+            step(i, sp)
         e0.record(stream)
         for i in range(steps):
             step(warmup + i, sp)
@@ -289,7 +293,12 @@ def time_case(case, dev, steps: int, warmup: int):
         res["eager_us"] = e0.elapsed_time(e1) * 1e3 / steps
     # graph replay
     try:
-        g = torch.cuda.CUDAGraph()
+        g, g_warm = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
+        if warmup > 0:
+            with torch.cuda.graph(g_warm, stream=stream):
+                spg = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+                for i in range(warmup):
+                    step(i, spg)
         with torch.cuda.graph(g, stream=stream):
             spg = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
             for i in range(steps):
@@ -300,10 +309,10 @@ def time_case(case, dev, steps: int, warmup: int):
         for _ in range(3):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize(dev)
-            # the scrub runs while the host queues the replay behind it: the K steps start when it ends, as they
-            # would behind the previous layer of a model, instead of after the launch latency of an idle GPU
-            # (~40 us, which K = 20 steps would carry as 2 us each)
+            # scrub, W warm-up steps, then the K timed steps, queued back to back
             scrub_cache(dev)
+            if warmup > 0:
+                g_warm.replay()
             e0.record()
             g.replay()
             e1.record()
