@@ -360,7 +360,8 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
         9.7 / 9.9 against 14.0 / 13.3, 8192 x 28672 24.6 / 26.4 against 32.3 / 30.2, 13824 x 5120 11.6 / 12.4
         against 21.2 / 17.6, 17920 x 6656 17.5 / 19.6 against 30.0 / 23.7, 28672 x 8192 29.2 / 30.7 against
         49.0 / 39.8, 9216 x 36864 int3 29.7 / 33.0 against 36.0 / 49.9; 36864 x 9216: 76 against 36, hence the
-        bound), except one row of a 3-bit layer of 9216 x 9216 (13.6 against 12.5-12.9);
+        bound; 9216 x 9216 int3 with one group, one row: 10.8 against 12.5 since its 32 tiles past a whole
+        number per CU are halved);
         longer K, three and four rows: K up to 6656 (5120 x 13824 12.8 against 15.4, 6656 x 17920 22.3 against
         26.8) and 8192 x 8192 (12.3 against 13.3); beyond, the four staged rows of x cost more than they save
         (8192 x 28672 41.9 against 30.4, 17920 x 6656 29.9 against 23.9);
