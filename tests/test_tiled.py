@@ -326,6 +326,30 @@ def test_tiled_decode_full_size(dev, name, bits, K, N, gs, desc_act, Ms):
             assert torch.equal(y, run_tiled(D, prep, x=x.to(dev), plan=plan)), f"{what}: two identical calls differ"
 
 
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("M", [2, 128])
+def test_tiled_linearity_at_full_size(dev, bits, M):
+    # size-independent properties on the tiled kernels at the benchmark's size (decode kernel with halved tiles,
+    # pack pass + matmul): f(2 x) = 2 f(x) exactly, f(a + b) = f(a) + f(b) up to rounding, and the rows of a batch
+    # equal the same rows computed alone
+    K, N, gs = 4096, 11008, 128
+    L = layer(905 + bits, K, N, bits, gs, True, M=M)
+    # keep fp16 subnormals out of x: doubling must stay exact on every path, matrix cores included
+    L["x"] = torch.where(L["x"].abs() < 1e-3, torch.zeros_like(L["x"]), L["x"])
+    D = to_dev(L, dev)
+    prep = prepare(D)
+    x = D["x"]
+    y = run_tiled(D, prep)
+    y2 = run_tiled(D, prep, x=(x * 2).contiguous())
+    normal = y.float().abs() >= 2.0 ** -13  # an fp16-subnormal output rounds on a fixed grid, not a relative one
+    assert torch.equal(y2.float()[normal], (y.float() * 2)[normal])
+    ysum = run_tiled(D, prep, x=(x[0:1] + x[1:2]).contiguous())
+    assert_close(ysum, (y[0:1].float() + y[1:2].float()).cpu(), "additivity", rtol=2e-2, atol=2e-2)
+    if M > 4:   # a row of the product depends on its own row of x only: the decode kernel gives the same row
+        y1 = run_tiled(D, prep, x=x[5:6].contiguous())
+        assert_tight(y1, y[5:6].cpu(), "row 5 alone against row 5 of the batch")
+
+
 TILED_FULL = [
     ("c4-int4-4096x11008-act", 4, 4096, 11008, 128, True, [16, 64, 128, 256]),
     ("c4-int3-4096x11008-act", 3, 4096, 11008, 128, True, [16, 64, 128, 256]),
