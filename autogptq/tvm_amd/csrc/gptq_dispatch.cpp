@@ -528,10 +528,11 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
         // four clocks, so a long K wants more, shorter waves.  One row, us, kw = 4 / 8 / 16: 8192 x 8192
         // 12.1 / 9.4 / 9.5, 5120 x 13824 10.9 / 9.4 / 11.6, 6144 x 16384 12.7 / 11.0 / 12.4, 9216 x 9216
         // 16.3 / 13.6 / 14.6, 11008 x 11008 21.1 / 17.2 / 18.0, 13824 x 5120 19.9 / 12.6 / 10.6 (4096 x 11008
-        // keeps four: 8.2 / 8.2 / 10.1): eight whenever four would walk more than sixteen blocks, sixteen only
-        // while that keeps a CU at about twelve waves
+        // keeps four: 8.2 / 8.2 / 10.1; 28672 x 8192 40.0 / 28.0 / 24.7, 17920 x 6656 26.0 / 17.6 / 14.6, 11008 x 8192
+        // 17.6 / 13.0 / 12.1): eight whenever four would walk more than sixteen blocks, sixteen only while that
+        // keeps a CU at sixteen waves (one tile per CU)
         if (kw == 4 && ceil_div(S_total, 4) > 16) kw = 8;
-        if (kw == 8 && ceil_div(S_total, 8) > 16 && (long long)tiles * 16 <= 12LL * gptq::kNumCUs) kw = 16;
+        if (kw == 8 && ceil_div(S_total, 8) > 16 && tiles <= gptq::kNumCUs) kw = 16;
         while (kw > 4 && kw > S_total) kw >>= 1;
         for (int split = 1; split <= S_total; split++) {
             int wave_steps = ceil_div(S_total, split * kw);

@@ -240,15 +240,19 @@ constexpr int tiled_decode_first_half(int wave_steps, bool pairs)
 // the others instead of a whole one.  Both halves pair their blocks up where whole tiles do.  (With more
 // halves than CUs nothing is gained, and workgroups of eight waves lose: 5120 x 13824, 176 tiles halved,
 // 9.9 -> 11.4 us at one row, 12.8 -> 16.2 at four.)
+inline bool tiled_decode_can_halve(int wave_steps, int split_k, int waves_k, int S_total, int group_size)
+{
+    if (split_k != 1) return false;
+    const bool pairs = tiled_decode_pairs(group_size, wave_steps);
+    const int first = tiled_decode_first_half(wave_steps, pairs);
+    if (wave_steps - first < (pairs ? 2 : 1)) return false;    // nothing left for the second half
+    return waves_k * first < S_total;                          // the second half must start inside K
+}
 inline int tiled_decode_halved(int tiles, int wave_steps, int split_k, int waves_k, int S_total, int group_size)
 {
     const int e = tiles % kNumCUs;
-    if (split_k != 1 || tiles <= kNumCUs || e == 0 || 2 * e > kNumCUs) return 0;
-    const bool pairs = tiled_decode_pairs(group_size, wave_steps);
-    const int first = tiled_decode_first_half(wave_steps, pairs);
-    if (wave_steps - first < (pairs ? 2 : 1)) return 0;    // nothing left for the second half
-    if (waves_k * first >= S_total) return 0;              // the second half must start inside K
-    return e;
+    if (tiles <= kNumCUs || e == 0 || 2 * e > kNumCUs) return 0;
+    return tiled_decode_can_halve(wave_steps, split_k, waves_k, S_total, group_size) ? e : 0;
 }
 // workspace of those tiles: one 64-bit slot per output of a halved tile, behind the counters
 inline size_t tiled_decode_slot_bytes(int halved, int mr) { return (size_t)halved * mr * 32 * 8; }

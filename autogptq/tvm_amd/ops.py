@@ -358,12 +358,13 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
         longer K, one and two rows: always up to K = 32768 (with an activation order, int4, one / two rows:
         5120 x 13824 9.7 / 10.5 against 18.2 / 15.2, 6656 x 17920 15.1 / 15.4 against 27.9 / 27.2, 8192 x 8192
         9.7 / 9.9 against 14.0 / 13.3, 8192 x 28672 24.6 / 26.4 against 32.3 / 30.2, 13824 x 5120 11.6 / 12.4
-        against 21.2 / 17.6, 17920 x 6656 17.5 / 19.6 against 30.0 / 23.7, 28672 x 8192 29.2 / 30.7 against
-        49.0 / 39.8, 9216 x 36864 int3 29.7 / 33.0 against 36.0 / 49.9; 36864 x 9216: 76 against 36, hence the
+        against 21.2 / 17.6, 17920 x 6656 14.8 / 16.2 against 31.0 / 23.8, 28672 x 8192 25.1 / 31.7 against
+        50.1 / 39.2, 9216 x 36864 int3 29.7 / 33.0 against 36.0 / 49.9; 36864 x 9216: 76 against 36, hence the
         bound; 9216 x 9216 int3 with one group, one row: 10.8 against 12.5 since its 32 tiles past a whole
         number per CU are halved);
         longer K, three and four rows: K up to 6656 (5120 x 13824 12.8 against 15.4, 6656 x 17920 22.3 against
-        26.8) and 8192 x 8192 (12.3 against 13.3); beyond, the four staged rows of x cost more than they save
+        26.8) and up to 8192 columns for K up to 11008 (8192 x 8192 12.3 against 13.3, 11008 x 8192 15.6 against
+        19.6); beyond, the four staged rows of x cost more than they save
         (8192 x 28672 41.9 against 30.4, 17920 x 6656 29.9 against 23.9);
       * 5 to 16 rows: only layers without an activation order, K up to 4096 and more than 4096 columns (the
         matmul kernel then reads x itself, one launch; 4096 x 11008 int4, 5 / 8 / 16 rows: 10.6 / 10.7 / 11.5
@@ -383,7 +384,7 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
             return False
         if M <= 2:
             return not (bits == 3 and M == 1 and 8192 < K <= 12288 and N <= 12288)
-        return K <= 6656 or (K <= 8192 and N <= 8192)
+        return K <= 6656 or (K <= 11008 and N <= 8192)
     if M <= 16:
         return not act_order and K <= 4096 and N > 4096 and (M >= 9 or bits == 4)
     return M <= 128 or K <= 8192
