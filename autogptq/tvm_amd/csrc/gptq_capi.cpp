@@ -374,7 +374,7 @@ extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint3
             (long long)plan->split_k * kw * plan->k_chunk < S_all ||
             (long long)(plan->split_k - 1) * kw * plan->k_chunk >= S_all)  // every workgroup starts inside K
             return GPTQ_HIP_ERR_BAD_ARG;
-        const int span = plan->k_chunk * kw * 64;
+        const int span = gptq::tiled_decode_span(halved, N / 32, plan->k_chunk, kw, gs);
         const int G_all = K / gs;
         const int groups = (span - 1) / gs + 2 < G_all ? (span - 1) / gs + 2 : G_all;
         if (plan->lds_bytes < gptq::tiled_decode_lds_bytes(mr, span, groups, kw) || plan->lds_bytes > 160 * 1024)

@@ -500,7 +500,8 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
         const int nwg = units < gptq::kNumCUs ? units : gptq::kNumCUs;
         const int upw = ceil_div(units, nwg);
         const long long lds = gptq::tiled_decode16_lds_bytes(mr, K, K / gs, upw);
-        if (upw == 1 && lds <= 128 * 1024) {
+        // (long K: the kernel below with every tile halved, see tiled_decode_halves_all)
+        if (upw == 1 && lds <= 128 * 1024 && !gptq::tiled_decode_halves_all(N / 32, ceil_div(K, 64))) {
             plan->kernel = GPTQ_HIP_KERNEL_TILED_DECODE;
             plan->row_tiles = mr;
             plan->m_blocks = 1;
@@ -533,6 +534,10 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
         // keeps a CU at sixteen waves (one tile per CU)
         if (kw == 4 && ceil_div(S_total, 4) > 16) kw = 8;
         if (kw == 8 && ceil_div(S_total, 8) > 16 && tiles <= gptq::kNumCUs) kw = 16;
+        // every tile in two halves: eight waves per half (14336 x 4096, one / four rows: 10.1 / 12.7 us with eight,
+        // 9.9 / 12.9 with sixteen; 11008 x 4096 int3 8.4 / 11.2 and 8.5 / 11.4)
+        const bool halves_all = gptq::tiled_decode_halves_all(tiles, S_total);
+        if (halves_all) kw = 8;
         while (kw > 4 && kw > S_total) kw >>= 1;
         for (int split = 1; split <= S_total; split++) {
             int wave_steps = ceil_div(S_total, split * kw);
@@ -541,7 +546,8 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
             // unequal halves do: 5120 x 13824, 9.7 -> 11.2 us with twelve blocks per wave instead of ten)
             if (gs % 128 == 0 && wave_steps > 1 && (wave_steps & 1) && split == 1) wave_steps++;
             if (ceil_div(S_total, wave_steps * kw) != split) continue;  // (the split this partition really needs)
-            const int span = wave_steps * kw * 64;
+            const int halved = gptq::tiled_decode_halved(tiles, wave_steps, split, kw, S_total, gs);
+            const int span = gptq::tiled_decode_span(halved, tiles, wave_steps, kw, gs);
             const int groups = (span - 1) / gs + 2 < ceil_div(K, gs) ? (span - 1) / gs + 2 : ceil_div(K, gs);
             const int lds = gptq::tiled_decode_lds_bytes(mr, span, groups, kw);
             if (lds > 128 * 1024) continue;
@@ -554,8 +560,8 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
             plan->split_k = split;
             plan->k_chunk = wave_steps;
             // up to CUs / 2 tiles past a whole number per CU run as two halves along K, so that the fullest CU
-            // holds half a tile more than the others, not a whole one (4096 x 11008: 344 tiles, 88 of them halved)
-            const int halved = gptq::tiled_decode_halved(tiles, wave_steps, split, kw, S_total, gs);
+            // holds half a tile more than the others, not a whole one (4096 x 11008: 344 tiles, 88 of them halved);
+            // long layers of up to 4096 columns halve every tile
             plan->grid_x = tiles + halved;
             plan->grid_y = split;
             plan->grid_z = 1;

@@ -248,11 +248,26 @@ inline bool tiled_decode_can_halve(int wave_steps, int split_k, int waves_k, int
     if (wave_steps - first < (pairs ? 2 : 1)) return false;    // nothing left for the second half
     return waves_k * first < S_total;                          // the second half must start inside K
 }
+// Layers of so few tiles that two workgroups per tile still find a CU each (N <= 4096), with K long enough for
+// two ranges (8192 channels): EVERY tile is halved, which gives every CU work like the 16-column kernel does, at
+// the lower cost per weight of this one (one row / four rows, us, against the 16-column kernel: 11008 x 4096 int3
+// 8.4 / 11.2 against 9.6 / 13.6, 14336 x 4096 int4 10.1 / 12.7 against 10.2 / 14.6, 8192 x 4096 7.6 / 9.1 against
+// 8.1 / 10.6; 4096 x 4096 the same 5.9, so shorter layers stay there).
+inline bool tiled_decode_halves_all(int tiles, int S_total) { return 2 * tiles <= kNumCUs && S_total >= 128; }
 inline int tiled_decode_halved(int tiles, int wave_steps, int split_k, int waves_k, int S_total, int group_size)
 {
+    if (!tiled_decode_can_halve(wave_steps, split_k, waves_k, S_total, group_size)) return 0;
+    if (tiled_decode_halves_all(tiles, S_total)) return tiles;
     const int e = tiles % kNumCUs;
     if (tiles <= kNumCUs || e == 0 || 2 * e > kNumCUs) return 0;
-    return tiled_decode_can_halve(wave_steps, split_k, waves_k, S_total, group_size) ? e : 0;
+    return e;
+}
+// positions a workgroup of the plan stages: a whole tile's range, or the larger half's when every tile is halved
+inline int tiled_decode_span(int halved, int tiles, int wave_steps, int waves_k, int group_size)
+{
+    const int ws = halved == tiles ? tiled_decode_first_half(wave_steps, tiled_decode_pairs(group_size, wave_steps))
+                                   : wave_steps;
+    return ws * waves_k * 64;
 }
 // workspace of those tiles: one 64-bit slot per output of a halved tile, behind the counters
 inline size_t tiled_decode_slot_bytes(int halved, int mr) { return (size_t)halved * mr * 32 * 8; }

@@ -304,10 +304,14 @@ def test_tiled_plans_are_consistent(bits, KN):
                 tiles = N // 32
                 # (the tiles past a whole number per CU, when there are at most 128 of them, run as two halves
                 # along K, which meet in 64-bit slots behind the counters of the workspace)
+                # (and every tile of a long layer of up to 4096 columns: two workgroups per tile still find a CU each)
                 halved = p.grid_x - tiles
-                assert halved in (0, tiles % 256) and p.split_k * p.waves_k * p.k_chunk >= blocks
-                if halved:
+                assert halved in (0, tiles % 256, tiles) and p.split_k * p.waves_k * p.k_chunk >= blocks
+                if halved == tiles:
+                    assert 2 * tiles <= 256 and blocks >= 128 and p.split_k == 1 and p.waves_k == 8
+                elif halved:
                     assert tiles > 256 and halved <= 128 and p.split_k == 1
+                if halved:
                     pairs = (K if gs == -1 else gs) % 128 == 0 and p.k_chunk % 2 == 0
                     first = 2 * ((p.k_chunk + 3) // 4) if pairs else (p.k_chunk + 1) // 2
                     assert p.k_chunk - first >= (2 if pairs else 1) and p.waves_k * first < blocks
