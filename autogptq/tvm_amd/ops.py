@@ -345,7 +345,8 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
     sorted copy), on MI355X with the weights cold, group size 128 (us, graph replay):
       * up to 4 rows, layers of up to 4096 columns (decode kernel with a workgroup per 16 columns, every CU at
         work): always.  4096 x 4096: 5.3-5.6 at one row, 7.4-8.0 at four, against 6.8-7.5 and 7.8-10.5;
-        11008 x 4096: 9.5-9.7 / 12.7-14.4 against 9.4-13.3 / 12.7-15.3;
+        11008 x 4096 (K of 8192 and more: the tile kernel with every tile in two halves along K): int4 9.0-9.4 /
+        11.5 against 13.5 / 15.3, int3 8.7 / 11.1 against 10.9 / 15.2;
       * up to 4 rows, wider layers (a workgroup per 32 columns, x staged per workgroup, four to sixteen waves
         along K so that a wave walks about sixteen blocks):
         K = 4096: one and two rows always, three and four up to 16384 columns.  Up to 128 tiles past a whole number
