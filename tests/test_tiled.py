@@ -313,6 +313,51 @@ def test_tiled_decode_halved_tiles(dev, bits, K, N, gs, desc_act):
         assert torch.equal(y, run_tiled(D, prep, x=x.to(dev), plan=plan)), f"{what}: two identical calls differ"
 
 
+def _random_decode_shapes():
+    import random
+
+    rnd = random.Random(20240)
+    shapes = []
+    for _ in range(28):
+        bits = rnd.choice([2, 3, 4, 8])
+        gs = rnd.choice([32, 64, 128, 256, -1])
+        unit = 32 if gs == -1 else gs
+        kind = rnd.choice(["long-narrow", "tail-halved", "several-per-cu", "short"])
+        if kind == "long-narrow":      # every tile in two halves
+            K = unit * rnd.randint(-(-8192 // unit), -(-8192 // unit) + 40 * 32 // unit)
+            N = 32 * rnd.randint(1, 24)
+        elif kind == "tail-halved":    # up to 128 tiles past 256
+            K = unit * rnd.randint(max(1, 256 // unit), 2048 // unit)
+            N = 32 * rnd.randint(257, 384)
+        elif kind == "several-per-cu":
+            K = unit * rnd.randint(max(1, 128 // unit), 1024 // unit)
+            N = 32 * rnd.randint(513, 700)
+        else:
+            K = unit * rnd.randint(1, max(1, 2048 // unit))
+            N = 32 * rnd.randint(1, 160)
+        shapes.append((bits, K, N, gs, rnd.random() < 0.6, rnd.randint(1, 4)))
+    return shapes
+
+
+@pytest.mark.parametrize("bits,K,N,gs,desc_act,M", _random_decode_shapes())
+def test_tiled_decode_random_shapes(dev, bits, K, N, gs, desc_act, M):
+    # the family's own decode plan (16-column units, a workgroup per tile, tail or all tiles halved, equal and
+    # unequal halves, 4 to 16 waves along K) on shapes drawn at random with a fixed seed
+    L = layer(9000 + K % 997 + N % 991, K, N, bits, gs, desc_act, M=M, bias=True)
+    D = to_dev(L, dev)
+    prep = prepare(D)
+    plan = _lib.select_tiled(M, K, N, bits, gs)
+    assert plan.kernel == _lib.KERNEL_TILED_DECODE
+    y = run_tiled(D, prep, plan=plan)
+    what = f"int{bits} {K}x{N} gs={gs} act={desc_act} M={M} (grid {plan.grid_x}, {plan.waves_k} waves, {plan.k_chunk} blocks)"
+    assert_close(y, expected_output(L), what)
+    if bits != 8:
+        assert_close(y, unrounded_output(L, L["x"]), what + " (against the unrounded weights)", rtol=1e-3, atol=1e-3)
+    else:
+        assert_tight(y, expected_output(L), what)
+    assert torch.equal(y, run_tiled(D, prep, plan=plan)), f"{what}: two identical calls differ"
+
+
 DECODE_FULL = [
     ("c1-int4-4096x4096", 4, 4096, 4096, 128, False, [1, 2, 4]),
     ("c2-int3-4096x11008-act", 3, 4096, 11008, 128, True, [1, 2, 3]),
