@@ -1,10 +1,11 @@
 """Loading a standard AutoGPTQ checkpoint onto the MI355X ``QuantLinear``.
 
-Mirrors the three pieces of the reference's loading path that touch the quantised layers:
+Mirrors the pieces of the reference's loading path that touch the quantised layers:
 
 * ``find_layers``   auto_gptq/modeling/_utils.py:38-49
 * ``make_quant``    auto_gptq/modeling/_utils.py:59-90 (the ``use_tvm=True`` branch picks this
                     package's ``QuantLinear`` instead of ``qlinear_tvm.QuantLinear``)
+* ``pack_model``    auto_gptq/modeling/_utils.py:123-157: the layers a GPTQ run quantised, packed in place
 * ``from_quantized`` auto_gptq/modeling/_base.py:478-569: read ``quantize_config.json``, build the
   model from its config with empty weights, swap the linear layers, load the checkpoint tensors
   by name onto the device.
@@ -68,6 +69,29 @@ def make_quant(module: nn.Module, names: Iterable[str], bits: int, groupsize: in
             setattr(module, child_name, new_layer.to(device))
     for child_name, child in module.named_children():
         make_quant(child, names, bits, groupsize, name + "." + child_name if name else child_name)
+
+
+def pack_model(model: nn.Module, quantizers: Dict[str, tuple], bits: int, group_size: int) -> Dict[str, QuantLinear]:
+    """Turns the layers a GPTQ run has quantised into packed ``QuantLinear`` layers, in place: the counterpart
+    of auto_gptq/modeling/_utils.py:123-157 (its ``use_tvm=True`` branch, with this package's module).
+    ``quantizers[name] = (quantizer, scale, zero, g_idx)`` as the reference's quantisation loop leaves them
+    (``scale`` and ``zero`` of shape [N, G]); the first entry is kept as it is.  Packing runs on the CPU, like
+    the reference's; every layer then returns to the device it was on.  Returns ``{name: QuantLinear}``."""
+    layers = find_layers(model)
+    layers = {n: layers[n] for n in quantizers}
+    make_quant(model, quantizers, bits, group_size)
+    qlayers = find_layers(model, [QuantLinear])
+    packed = {}
+    for name, q in qlayers.items():
+        if name not in quantizers:
+            continue
+        _, scale, zero, g_idx = quantizers[name]
+        device = q.scales.device
+        q.to("cpu")
+        q.pack(layers[name].to("cpu"), scale.to("cpu"), zero.to("cpu"), None if g_idx is None else g_idx.to("cpu"))
+        q.to(device)
+        packed[name] = q
+    return packed
 
 
 def read_quantize_config(save_dir: str) -> dict:

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from autogptq.tvm_amd import QuantLinear
-from autogptq.tvm_amd.loader import find_layers, from_quantized, make_quant
+from autogptq.tvm_amd.loader import find_layers, from_quantized, make_quant, pack_model
 from tests.loader_util import build_checkpoint
 
 
@@ -24,6 +24,36 @@ def test_find_layers_and_make_quant_on_a_plain_module():
     assert q.bias is None and q.qweight.shape == (3, 64)
     make_quant(net, ["inner.proj"], 3, 32)  # already quantised: left alone
     assert net.inner.proj is q
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
+def test_pack_model_packs_the_quantised_layers_in_place(bits):
+    """What the reference does after its GPTQ loop (auto_gptq/modeling/_utils.py:123-157): layers named in
+    ``quantizers`` become packed QuantLinear layers, other layers stay as they are.  The float weights here lie
+    on the quantisation grid, so packing must find exactly the codes they were made from."""
+    from oracle import gptq_oracle
+
+    gen = torch.Generator().manual_seed(40 + bits)
+    K, N, gs = 128, 64, 32
+    G, maxq = K // gs, 2 ** bits - 1
+    g_idx = (torch.randperm(K, generator=gen) // gs).to(torch.int32)       # an activation order
+    scale = (torch.rand(N, G, generator=gen) * 9e-3 + 1e-3).half().float()  # [N, G], as the reference passes them
+    zero = torch.randint(1, maxq + 2, (N, G), generator=gen).float()        # the format stores zero - 1
+    codes = torch.randint(0, maxq + 1, (N, K), generator=gen)
+    gl = g_idx.long()
+    net = torch.nn.Sequential()
+    net.add_module("keep", torch.nn.Linear(K, K))
+    net.add_module("q", torch.nn.Linear(K, N, bias=True))
+    net.q.weight.data = scale[:, gl] * (codes.float() - zero[:, gl])          # exact in fp32
+    packed = pack_model(net, {"q": (None, scale, zero, g_idx)}, bits, gs)
+    assert sorted(packed) == ["q"] and isinstance(net.q, QuantLinear) and isinstance(net.keep, torch.nn.Linear)
+    q = net.q
+    assert (q.bits, q.groupsize, q.infeatures, q.outfeatures) == (bits, gs, K, N) and q.bias is not None
+    assert np.array_equal(gptq_oracle.unpack_bitstream(q.qweight.numpy(), bits, axis=0), codes.t().numpy())
+    assert np.array_equal(gptq_oracle.unpack_bitstream(q.qzeros.numpy(), bits, axis=1) + 1, zero.t().numpy())
+    assert torch.equal(q.g_idx, g_idx) and torch.equal(q.scales, scale.t().half())
+    w16 = gptq_oracle.dequant_exact(q.qweight.numpy(), q.qzeros.numpy(), q.scales.numpy(), q.g_idx.numpy(), bits)
+    assert np.array_equal(w16, (scale[:, gl] * (codes.float() - zero[:, gl])).t().half().numpy())
 
 
 def test_make_quant_on_meta_allocates_nothing():
