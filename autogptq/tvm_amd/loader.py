@@ -6,6 +6,7 @@ Mirrors the pieces of the reference's loading path that touch the quantised laye
 * ``make_quant``    auto_gptq/modeling/_utils.py:59-90 (the ``use_tvm=True`` branch picks this
                     package's ``QuantLinear`` instead of ``qlinear_tvm.QuantLinear``)
 * ``pack_model``    auto_gptq/modeling/_utils.py:123-157: the layers a GPTQ run quantised, packed in place
+* ``save_quantized`` auto_gptq/modeling/_base.py:381-401: the checkpoint directory ``from_quantized`` reads
 * ``from_quantized`` auto_gptq/modeling/_base.py:478-569: read ``quantize_config.json``, build the
   model from its config with empty weights, swap the linear layers, load the checkpoint tensors
   by name onto the device.
@@ -92,6 +93,36 @@ def pack_model(model: nn.Module, quantizers: Dict[str, tuple], bits: int, group_
         q.to(device)
         packed[name] = q
     return packed
+
+
+def save_quantized(model: nn.Module, save_dir: str, bits: int, group_size: int, desc_act: bool = True,
+                   use_safetensors: bool = True, model_basename: Optional[str] = None) -> str:
+    """Writes a packed model the way the reference lays a checkpoint out (auto_gptq/modeling/_base.py:381-401):
+    ``gptq_model-{bits}bit-{group_size}g.{safetensors|bin}`` with every tensor of the state dict under its own
+    name, ``quantize_config.json`` (``_base.py:66-77``), and the model's ``config.json`` when it has one.  What
+    it writes is what ``from_quantized`` reads.  Layers that kept only their tiled copy (``QuantLinear.compact``)
+    have no checkpoint tensors left and cannot be saved.  Returns the path of the weight file."""
+    for name, mod in model.named_modules():
+        if isinstance(mod, QuantLinear) and getattr(mod, "_compact", False):
+            raise ValueError(f"{name} holds only its tiled copy (compact()): the checkpoint tensors are gone")
+    os.makedirs(save_dir, exist_ok=True)
+    if model_basename is None:
+        model_basename = f"gptq_model-{bits}bit-{group_size}g"
+    state = {k: v.detach().to("cpu").clone().contiguous() for k, v in model.state_dict().items()}
+    if use_safetensors:
+        from safetensors.torch import save_file
+
+        path = os.path.join(save_dir, model_basename + ".safetensors")
+        save_file(state, path)
+    else:
+        path = os.path.join(save_dir, model_basename + ".bin")
+        torch.save(state, path)
+    config = getattr(model, "config", None)
+    if config is not None and hasattr(config, "save_pretrained"):
+        config.save_pretrained(save_dir)
+    with open(os.path.join(save_dir, "quantize_config.json"), "w", encoding="utf-8") as f:
+        json.dump({"bits": int(bits), "group_size": int(group_size), "desc_act": bool(desc_act)}, f, indent=2)
+    return path
 
 
 def read_quantize_config(save_dir: str) -> dict:

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from autogptq.tvm_amd import QuantLinear
-from autogptq.tvm_amd.loader import find_layers, from_quantized, make_quant, pack_model
+from autogptq.tvm_amd.loader import find_layers, from_quantized, make_quant, pack_model, save_quantized
 from tests.loader_util import build_checkpoint
 
 
@@ -81,6 +81,43 @@ def test_from_quantized_restores_every_tensor(tmp_path, bits, act_order):
     assert model.seqlen == 64 and not model.training
     with pytest.raises(RuntimeError):  # no CPU path: the kernels must not be silently replaced
         model(torch.zeros((1, 4), dtype=torch.long))
+
+
+@pytest.mark.parametrize("use_safetensors", [True, False])
+def test_pack_save_load_round_trip(tmp_path, use_safetensors):
+    """The reference's whole way from a quantised float model to a loaded checkpoint, on a tiny Llama:
+    pack_model (_utils.py:123-157), save_quantized (_base.py:381-401), from_quantized (_base.py:478-569)."""
+    from transformers import AutoModelForCausalLM, LlamaConfig
+
+    from tests.loader_util import rtn_quantize
+
+    torch.manual_seed(3)
+    bits, gs = 4, 32
+    cfg = LlamaConfig(hidden_size=64, intermediate_size=128, num_hidden_layers=1, num_attention_heads=4,
+                      num_key_value_heads=4, vocab_size=128, max_position_embeddings=64, tie_word_embeddings=False)
+    model = AutoModelForCausalLM.from_config(cfg).half()
+    quantizers = {}
+    for name, lin in find_layers(model).items():
+        if name.startswith("lm_head"):
+            continue
+        scales, zeros = rtn_quantize(lin.weight.data, bits, gs)
+        g_idx = (torch.arange(lin.weight.shape[1]) // gs).to(torch.int32)
+        quantizers[name] = (None, scales, zeros, g_idx)
+    packed = pack_model(model, quantizers, bits, gs)
+    assert len(packed) == 7 and isinstance(model.lm_head, torch.nn.Linear)
+    path = save_quantized(model, str(tmp_path), bits, gs, desc_act=False, use_safetensors=use_safetensors)
+    assert path.endswith(".safetensors" if use_safetensors else ".bin")
+    loaded, qcfg = from_quantized(str(tmp_path), device="cpu", use_safetensors=use_safetensors)
+    assert (qcfg["bits"], qcfg["group_size"], qcfg["desc_act"]) == (bits, gs, False)
+    want, got = model.state_dict(), loaded.state_dict()
+    assert sorted(want) == sorted(got)
+    for name in want:
+        assert want[name].dtype == got[name].dtype and torch.equal(want[name].cpu(), got[name]), name
+    # a layer that kept only its tiled copy has nothing left to save
+    q = next(m for m in model.modules() if isinstance(m, QuantLinear))
+    q._compact = True
+    with pytest.raises(ValueError, match="compact"):
+        save_quantized(model, str(tmp_path), bits, gs)
 
 
 def test_from_quantized_reports_missing_files_and_tensors(tmp_path):
