@@ -340,7 +340,7 @@ def gemm_tiled_transposed(gy: torch.Tensor, qtile_t: torch.Tensor, szt: torch.Te
     return out
 
 
-def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
+def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4, one_group: bool = False) -> bool:
     """Where the tiled kernels were measured faster than the ones that read the checkpoint layout (or its
     sorted copy), on MI355X with the weights cold, group size 128 (us, graph replay):
       * up to 4 rows, layers of up to 4096 columns (decode kernel with a workgroup per 16 columns, every CU at
@@ -372,8 +372,14 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
         against 11.2 / 11.3 / 12.5; int3 from nine rows: 11.5 against 12.8 at sixteen, 10.9 against 10.4 at
         eight); with an activation order the pack pass makes it 14.6 against 13.4 at 8 rows, and narrower or
         longer layers split K and add a pass (11008 x 4096: 17.3 against 13.1);
-      * 17 to 128 rows: everywhere within 4 % or better (4096 x 11008 with an activation order, 32/64/128
-        rows: 14.8/19.2/26.6 against 18.1/22.1/34.1);
+      * 17 to 128 rows: almost everywhere within 4 % or better (4096 x 11008 with an activation order, 32/64/128
+        rows: 14.8/19.2/26.6 against 18.1/22.1/34.1).  Two exceptions, both with K of 8192 and more and nothing
+        for the checkpoint-layout STREAM kernel to look up per weight: 4-bit layers without an activation order
+        up to 64 rows (17 / 64 rows: 8192 x 8192 23.4 / 28.6 against 19.7 / 25.0, 8192 x 28672 44.8 / 58.9 against
+        40.4 / 55.4, 28672 x 8192 47.7 / 58.7 against 43.8 / 57.2; at 128 rows the tiled kernel is ahead again on
+        wide layers, 8192 x 28672 88 against 105; 3-bit layers stay: 9216 x 9216 28.4 against 32.6), and layers of
+        one group (``one_group``; 32 / 128 rows: 9216 x 36864 61.9 / 134 against 54.6 / 126, 36864 x 9216 86.7 / 206
+        against 72.8 / 173; 9216 x 9216 keeps the tiled copy up to 32 rows, 30.2 against 33.0);
       * above 128 rows: K up to 8192 (4096 x 11008, 512 rows: 75 against 95; 11008 x 4096: 127 against 81,
         where every workgroup pulls 2.8 MB of x fragments and they no longer stay in one L2)."""
     if M <= 4:
@@ -384,11 +390,17 @@ def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4) -> bool:
         if K > 32768:
             return False
         if M <= 2:
-            return not (bits == 3 and M == 1 and 8192 < K <= 12288 and N <= 12288)
+            return True
         return K <= 6656 or (K <= 11008 and N <= 8192)
     if M <= 16:
         return not act_order and K <= 4096 and N > 4096 and (M >= 9 or bits == 4)
-    return M <= 128 or K <= 8192
+    if M <= 128:
+        if one_group and K > 8192 and (M > 32 or K > 16384 or N > 16384):
+            return False
+        if M <= 64 and K >= 8192 and bits == 4 and not act_order:
+            return False
+        return True
+    return K <= 8192
 
 
 def dequant(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,

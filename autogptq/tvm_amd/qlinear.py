@@ -320,7 +320,7 @@ class QuantLinear(nn.Module):
             tiled = self.prepare_tiled() if self.tile_for_prefill else None
             if tiled is None:
                 return "library", library
-        elif self.tile_for_prefill and ops.tiled_wins(M, K, N, g is not None, bits):
+        elif self.tile_for_prefill and ops.tiled_wins(M, K, N, g is not None, bits, one_group=self.groupsize >= K):
             tiled = self.prepare_tiled()
         threshold = self.kernel_switch_threshold
         if threshold and tiled is None:   # off the tiled route the library wins earlier

@@ -208,7 +208,9 @@ def prepared_mode(name: str):
     from autogptq.tvm_amd import ops
 
     bits, K, N, gs, desc_act, M = WORKLOADS[name]
-    if tiled_applies(name) and (not plain_applies(name) or ops.tiled_wins(M, K, N, desc_act, bits)):
+    one_group = gs == -1 or gs >= K
+    if tiled_applies(name) and (not plain_applies(name) or ops.tiled_wins(M, K, N, desc_act and not one_group, bits,
+                                                                           one_group=one_group)):
         return "tiled"
     return "sorted" if sorted_applies(name) else None
 
