@@ -17,7 +17,6 @@ ERR_UNSUPPORTED = -2
 ERR_WORKSPACE = -3
 ERR_LAUNCH = -4
 
-KERNEL_GATHER = 1
 KERNEL_GROUPED = 2
 KERNEL_STREAM = 3
 KERNEL_TILED = 4
@@ -39,6 +38,7 @@ ABI_SYMBOLS = (
     "gptq_hip_tile_prepare",
     "gptq_hip_select_tiled",
     "gptq_hip_select_tiled_decode",
+    "gptq_hip_select_route",
     "gptq_hip_tiled_transposed_bytes",
     "gptq_hip_tiled_transposed_table_bytes",
     "gptq_hip_tile_prepare_transposed",
@@ -50,7 +50,7 @@ ABI_SYMBOLS = (
     "gptq_hip_abi_version",
     "gptq_hip_build_id",
 )
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class Plan(ctypes.Structure):
@@ -69,11 +69,25 @@ class Plan(ctypes.Structure):
         ("grid_z", ctypes.c_int),
         ("block", ctypes.c_int),
         ("lds_bytes", ctypes.c_int),
+        ("flags", ctypes.c_int),
         ("workspace_bytes", ctypes.c_size_t),
     ]
 
     def as_dict(self) -> dict:
         return {name: getattr(self, name) for name, _ in self._fields_}
+
+
+PLAN_PRIVATE_ZERO_WORKSPACE = 1
+
+COPY_CHECKPOINT, COPY_SORTED, COPY_TILED = 1, 2, 4
+ROUTE_CHECKPOINT, ROUTE_SORTED, ROUTE_TILED, ROUTE_LIBRARY = 0, 1, 2, 3
+ROUTE_NAMES = {ROUTE_CHECKPOINT: "plain", ROUTE_SORTED: "sorted", ROUTE_TILED: "tiled", ROUTE_LIBRARY: "library"}
+
+
+class Route(ctypes.Structure):
+    """Mirror of ``gptq_hip_route``."""
+
+    _fields_ = [("copy", ctypes.c_int), ("reserved", ctypes.c_int), ("plan", Plan)]
 
 
 class GptqHipError(RuntimeError):
@@ -97,6 +111,26 @@ def lib() -> ctypes.CDLL:
         )
     l = ctypes.CDLL(LIB_PATH)
     vp, i, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    # a library older than the sources beside it is refused before anything else of it is touched
+    try:
+        l.gptq_hip_abi_version.restype = i
+        l.gptq_hip_abi_version.argtypes = []
+        l.gptq_hip_build_id.restype = ctypes.c_char_p
+        l.gptq_hip_build_id.argtypes = []
+        missing = [name for name in ABI_SYMBOLS if not hasattr(l, name)]
+    except AttributeError as exc:
+        raise RuntimeError(f"{LIB_PATH} is not this package's library ({exc}): rebuild it with "
+                           "`python -m autogptq.tvm_amd.build`") from None
+    if l.gptq_hip_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH} has ABI version {l.gptq_hip_abi_version()}, this package expects "
+                           f"{ABI_VERSION}: rebuild it with `python -m autogptq.tvm_amd.build`")
+    from . import _sources as _build
+    built, now = l.gptq_hip_build_id().decode(), _build.source_hash()
+    if built != now:
+        raise RuntimeError(f"{LIB_PATH} was built from other sources (build id {built}, sources now {now}): "
+                           "rebuild it with `python -m autogptq.tvm_amd.build`")
+    if missing:
+        raise RuntimeError(f"{LIB_PATH} lacks {', '.join(missing)}: rebuild it with `python -m autogptq.tvm_amd.build`")
     l.gptq_hip_select.restype = i
     l.gptq_hip_select.argtypes = [i, i, i, i, i, i, ctypes.POINTER(Plan)]
     l.gptq_hip_plan_for.restype = i
@@ -127,6 +161,8 @@ def lib() -> ctypes.CDLL:
     l.gptq_hip_select_tiled.argtypes = [i, i, i, i, i, ctypes.POINTER(Plan)]
     l.gptq_hip_select_tiled_decode.restype = i
     l.gptq_hip_select_tiled_decode.argtypes = [i, i, i, i, i, ctypes.POINTER(Plan)]
+    l.gptq_hip_select_route.restype = i
+    l.gptq_hip_select_route.argtypes = [i, i, i, i, i, i, ctypes.c_uint, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(Route)]
     l.gptq_hip_gemm_tiled.restype = i
     l.gptq_hip_gemm_tiled.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
     l.gptq_hip_tiled_transposed_bytes.restype = sz
@@ -147,14 +183,6 @@ def lib() -> ctypes.CDLL:
     l.gptq_hip_abi_version.argtypes = []
     l.gptq_hip_build_id.restype = ctypes.c_char_p
     l.gptq_hip_build_id.argtypes = []
-    if l.gptq_hip_abi_version() != ABI_VERSION:
-        raise RuntimeError(f"{LIB_PATH} has ABI version {l.gptq_hip_abi_version()}, this package expects "
-                           f"{ABI_VERSION}: rebuild it with `python -m autogptq.tvm_amd.build`")
-    from . import _sources as _build
-    built, now = l.gptq_hip_build_id().decode(), _build.source_hash()
-    if built != now:
-        raise RuntimeError(f"{LIB_PATH} was built from other sources (build id {built}, sources now {now}): "
-                           "rebuild it with `python -m autogptq.tvm_amd.build`")
     _lib = l
     return l
 
@@ -184,6 +212,20 @@ def select_tiled(M: int, K: int, N: int, bits: int, group_size: int, decode: boo
     if rc != OK:
         raise GptqHipError(rc, f"gptq_hip_select_tiled(M={M}, K={K}, N={N}, bits={bits}, group_size={group_size})")
     return plan
+
+
+def select_route(M: int, K: int, N: int, bits: int, group_size: int, act_order: bool,
+                 copies: int = COPY_CHECKPOINT | COPY_SORTED | COPY_TILED, switch_rows=None) -> Route:
+    """Which copy of a layer a call with M rows runs on, and the plan there (gptq_hip_select_route).
+    ``switch_rows``: (tiled, checkpoint, checkpoint with an activation order) rows from which the library GEMM
+    takes over, 0 = never; None = the library's defaults."""
+    route = Route()
+    sw = None if switch_rows is None else (ctypes.c_int * 3)(*[int(v or 0) for v in switch_rows])
+    rc = lib().gptq_hip_select_route(M, K, N, bits, group_size, int(bool(act_order)), copies, sw, ctypes.byref(route))
+    if rc != OK:
+        raise GptqHipError(rc, f"gptq_hip_select_route(M={M}, K={K}, N={N}, bits={bits}, group_size={group_size}, "
+                               f"copies={copies})")
+    return route
 
 
 def select_tiled_transposed(M: int, K: int, N: int, bits: int, group_size: int) -> Plan:

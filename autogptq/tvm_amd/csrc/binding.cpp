@@ -60,7 +60,7 @@ std::map<std::tuple<int, void *, int>, Tensor> g_ws;
 int workspace_kind(const gptq_hip_plan &plan)
 {
     // (a decode plan that cuts K over workgroups leaves partial sums in its workspace like any other plan)
-    return plan.kernel == GPTQ_HIP_KERNEL_TILED_DECODE && plan.split_k == 1 ? 1 : 0;
+    return (plan.flags & GPTQ_HIP_PLAN_PRIVATE_ZERO_WORKSPACE) ? 1 : 0;
 }
 
 Tensor workspace(const Tensor &like, size_t nbytes, void *stream, int kind = 0)

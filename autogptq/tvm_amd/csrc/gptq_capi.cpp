@@ -51,24 +51,6 @@ int validate_plan(const gptq_hip_plan &pl, int M, int K, int N, int bits, int G,
     if (pl.lds_bytes > 160 * 1024) return GPTQ_HIP_ERR_BAD_ARG;
     if (pl.split_k > 1 && (size_t)pl.grid_x * (pl.grid_z > 0 ? pl.grid_z : 1) * sizeof(int) > gptq::kCounterBytes)
         return GPTQ_HIP_ERR_UNSUPPORTED;
-    if (pl.kernel == GPTQ_HIP_KERNEL_GATHER) {
-        if (pl.waves_n * pl.waves_k > 4) return GPTQ_HIP_ERR_UNSUPPORTED;
-        if (pl.row_tiles != 1 && pl.row_tiles != 2 && pl.row_tiles != 4) return GPTQ_HIP_ERR_UNSUPPORTED;
-        if (pl.k_chunk < kstep || pl.k_chunk % kstep != 0) return GPTQ_HIP_ERR_BAD_ARG;
-        if (pl.m_blocks * 16 * pl.row_tiles < M || pl.grid_z != pl.m_blocks) return GPTQ_HIP_ERR_BAD_ARG;
-        if (pl.split_k * pl.waves_k > steps_total && pl.split_k * pl.waves_k > 1) return GPTQ_HIP_ERR_BAD_ARG;
-        const int xs_rows = 16 * pl.row_tiles;
-        // chunk: a power of two; every thread stages a whole number (1 .. xv) of x vectors and
-        // at most 4 group indices
-        if (pl.k_chunk != gptq::gather_kc(bits, pl.row_tiles)) return GPTQ_HIP_ERR_BAD_ARG;
-        const int vectors = xs_rows * pl.k_chunk / 8, threads = 64 * pl.waves_n;
-        if (vectors % threads != 0 || vectors / threads > gptq::gather_xv(bits, pl.row_tiles) ||
-            pl.k_chunk > gptq::gather_gv() * threads)
-            return GPTQ_HIP_ERR_UNSUPPORTED;
-        if (pl.lds_bytes < gptq::gather_lds_bytes(G, pl.k_chunk, xs_rows, pl.row_tiles, pl.waves_n, pl.waves_k))
-            return GPTQ_HIP_ERR_BAD_ARG;
-        return GPTQ_HIP_OK;
-    }
     if (pl.kernel == GPTQ_HIP_KERNEL_GROUPED) {
         if (M > gptq::kPackedRows || pl.grid_z != 1) return GPTQ_HIP_ERR_UNSUPPORTED;
         // k_chunk is the K range of one workgroup: waves_k * wave_steps whole steps
@@ -243,7 +225,7 @@ static int run_gemm(const void *x, const int32_t *qweight, const int32_t *qzeros
         p.partial = (float *)((char *)workspace + gptq::kCounterBytes);
     }
     if (plan->kernel == GPTQ_HIP_KERNEL_GROUPED) return gptq::launch_grouped(p, bits, *plan, stream);
-    return gptq::launch_gather(p, bits, *plan, stream);
+    return GPTQ_HIP_ERR_UNSUPPORTED;
 }
 
 extern "C" int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
@@ -369,6 +351,8 @@ extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint3
         const int halved = plan->grid_x - N / 32;
         if (halved != 0 && halved != gptq::tiled_decode_halved(N / 32, plan->k_chunk, plan->split_k, kw, S_all, gs))
             return GPTQ_HIP_ERR_BAD_ARG;
+        // a caller that runs halved tiles has to know what their workspace asks for
+        if (halved != 0 && !(plan->flags & GPTQ_HIP_PLAN_PRIVATE_ZERO_WORKSPACE)) return GPTQ_HIP_ERR_BAD_ARG;
         if ((kw != 4 && kw != 8 && kw != 16) || plan->block != 64 * kw || plan->split_k < 1 || plan->k_chunk < 1 ||
             plan->grid_y != plan->split_k || plan->grid_z != 1 ||
             (long long)plan->split_k * kw * plan->k_chunk < S_all ||

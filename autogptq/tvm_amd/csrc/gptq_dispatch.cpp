@@ -14,92 +14,6 @@ const int kTargetWorkgroups = 512;  // two per CU keeps every XCD fed at M = 1
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-// GATHER: exact weights, any g_idx, any M.
-int plan_gather_rt(int row_tiles, int M, int K, int N, int bits, int G, int force_split, int force_waves,
-                   gptq_hip_plan *plan);
-
-int plan_gather(int M, int K, int N, int bits, int G, int force_split, int force_waves, gptq_hip_plan *plan)
-{
-    // the tallest tile that fits; shorter tiles (more M blocks) when LDS or staging registers
-    // cannot hold it, e.g. with hundreds of groups in the (scale, zero) table
-    int rt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);  // (128-row tiles spilled)
-    for (; rt >= 1; rt >>= 1) {
-        memset(plan, 0, sizeof(*plan));
-        const int rc = plan_gather_rt(rt, M, K, N, bits, G, force_split, force_waves, plan);
-        if (rc != GPTQ_HIP_ERR_UNSUPPORTED) return rc;
-    }
-    return GPTQ_HIP_ERR_UNSUPPORTED;
-}
-
-int plan_gather_rt(int row_tiles, int M, int K, int N, int bits, int G, int force_split, int force_waves,
-                   gptq_hip_plan *plan)
-{
-    const int kstep = gptq::kstep_of(bits);
-    const int steps_total = ceil_div(K, kstep);
-    plan->kernel = GPTQ_HIP_KERNEL_GATHER;
-    plan->row_tiles = row_tiles;
-    plan->m_blocks = ceil_div(M, 16 * plan->row_tiles);
-    // x is staged for all 16 * row_tiles rows of the tile (rows past M hold zeros)
-    const int xs_rows = 16 * plan->row_tiles;
-    // channels of x staged per K wave at a time: fixed per (bits, row tiles), see gather_kc
-    const int kc_fixed = gptq::gather_kc(bits, plan->row_tiles);
-
-    // candidate workgroup shapes, best first
-    static const int tall[][2] = {{2, 2}, {2, 1}, {1, 2}, {1, 1}};
-    static const int skinny[][2] = {{4, 1}, {2, 1}, {1, 1}};
-    const int (*cand)[2] = row_tiles == 1 ? skinny : tall;
-    const int ncand = row_tiles == 1 ? 3 : 4;
-    const int xv = gptq::gather_xv(bits, plan->row_tiles);
-    int waves_n = 0, waves_k = 0, lds = 0, kc = 0;
-    for (int i = 0; i < ncand && waves_n == 0; i++) {
-        const int wn = cand[i][0];
-        int wk = cand[i][1];
-        if (force_waves > 0 && wn != force_waves) continue;
-        if (wk > steps_total) wk = 1;
-        // every thread of a K wave group stages the same whole number of 16-byte vectors of x
-        // (1 .. xv) and at most 4 group indices per chunk
-        for (int k = kc_fixed; k == kc_fixed; k = 0) {
-            const int vectors = xs_rows * k / 8;
-            const int threads = 64 * wn;
-            if (vectors % threads != 0 || vectors / threads > xv || k > gptq::gather_gv() * threads) continue;
-            const int need = gptq::gather_lds_bytes(G, k, xs_rows, plan->row_tiles, wn, wk);
-            if (need > kLdsBudget) continue;
-            waves_n = wn;
-            waves_k = wk;
-            lds = need;
-            kc = k;
-            break;
-        }
-    }
-    if (waves_n == 0) return GPTQ_HIP_ERR_UNSUPPORTED;  // e.g. more groups than the LDS table holds
-    plan->k_chunk = kc;
-    plan->waves_n = waves_n;
-    plan->waves_k = waves_k;
-    plan->lds_bytes = lds;
-    plan->block = 64 * waves_n * waves_k;
-    const int col_tiles = ceil_div(N, 64 * waves_n);
-
-    int split = ceil_div(M <= 16 ? kTargetWorkgroups : 256, col_tiles * plan->m_blocks);
-    // partial sums cost split*M*N*4 bytes each way; keep them in proportion to the packed weights
-    int cap = (int)((3LL * K * bits) / (128LL * M));
-    if (cap < 1) cap = 1;
-    if (split > cap) split = cap;
-    if (split > 64) split = 64;
-    if (force_split > 0) split = force_split;
-    if (split * waves_k > steps_total) split = steps_total / waves_k;
-    if (split < 1) split = 1;
-    if ((size_t)col_tiles * plan->m_blocks * sizeof(int) > gptq::kCounterBytes) split = 1;
-    // uniform partition: the split actually needed once every K wave takes whole steps
-    const int wave_steps = ceil_div(steps_total, split * waves_k);
-    split = ceil_div(steps_total, wave_steps * waves_k);
-    plan->split_k = split;
-    plan->grid_x = col_tiles;
-    plan->grid_y = split;
-    plan->grid_z = plan->m_blocks;
-    plan->workspace_bytes = split > 1 ? gptq::kCounterBytes + (size_t)split * M * N * sizeof(float) : 0;
-    return GPTQ_HIP_OK;
-}
-
 }  // namespace
 
 namespace gptq {
@@ -117,17 +31,6 @@ int grouped_groups(int kr, int gs, int G, int act_order)
 {
     int groups = act_order ? G : (kr - 1) / gs + 2;
     return groups > G ? G : groups;
-}
-
-// LDS of the GATHER kernel: (scale, zero) table + per K wave the staged chunk (group offsets and
-// x rows), or the reduction buffer of the waves along K, which reuses the same bytes.
-int gather_lds_bytes(int G, int kc, int xs_rows, int row_tiles, int waves_n, int waves_k)
-{
-    const long long stage =
-        (long long)G * (64 * waves_n * 4 + 16) + 2LL * waves_k * (kc * 4 + xs_rows * (kc + 8) * 2);  // double-buffered
-    const long long red = (long long)(waves_k - 1) * waves_n * row_tiles * 16 * 64 * 4;
-    const long long need = stage > red ? stage : red;
-    return need > (1 << 30) ? (1 << 30) : (int)need;
 }
 
 // LDS of the STREAM kernel: the (scale, zero) table of 64 columns, or the reduction buffer of the
@@ -436,8 +339,7 @@ extern "C" int gptq_hip_select(int M, int K, int N, int bits, int group_size, in
     memset(plan, 0, sizeof(*plan));
     if (plan_stream(M, K, N, bits, gs, G, act_order, 0, 0, plan) == GPTQ_HIP_OK) return GPTQ_HIP_OK;
     memset(plan, 0, sizeof(*plan));
-    // last resort (its table limit is tighter than STREAM's, so this rarely finds a plan either)
-    return plan_gather(M, K, N, bits, G, 0, 0, plan);
+    return GPTQ_HIP_ERR_UNSUPPORTED;
 }
 
 extern "C" int gptq_hip_plan_for(int kernel, int M, int K, int N, int bits, int group_size, int act_order,
@@ -453,7 +355,6 @@ extern "C" int gptq_hip_plan_for(int kernel, int M, int K, int N, int bits, int 
     const int gs = group_size == -1 ? K : group_size;
     const int G = ceil_div(K, gs);
     if (G == 1) act_order = 0;
-    if (kernel == GPTQ_HIP_KERNEL_GATHER) return plan_gather(M, K, N, bits, G, split_k, waves_n, plan);
     if (kernel == GPTQ_HIP_KERNEL_STREAM) {
         const int rc2 = plan_stream(M, K, N, bits, gs, G, act_order, split_k, waves_n, plan);
         if (rc2 != GPTQ_HIP_OK) memset(plan, 0, sizeof(*plan));
@@ -569,6 +470,8 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
             plan->lds_bytes = lds;
             plan->workspace_bytes = split > 1 ? gptq::kCounterBytes + (size_t)split * M * N * sizeof(float)
                                     : (halved ? gptq::kCounterBytes + gptq::tiled_decode_slot_bytes(halved, mr) : 0);
+            // (the halves of a tile meet in slots that must be all zero between launches)
+            plan->flags = halved ? GPTQ_HIP_PLAN_PRIVATE_ZERO_WORKSPACE : 0;
             return GPTQ_HIP_OK;
         }
         return GPTQ_HIP_ERR_UNSUPPORTED;
@@ -669,6 +572,131 @@ extern "C" int gptq_hip_select_tiled_transposed(int M, int K, int N, int bits, i
     ws += (size_t)gptq::tiled_pack_blocks(split, kwv, wave_steps) * 4 * (size_t)(at * m_blocks) * 1024;
     plan->workspace_bytes = ws;
     return GPTQ_HIP_OK;
+}
+
+namespace {
+
+// Where the tiled kernels were measured faster than the ones that read the checkpoint layout or its channel-sorted
+// copy, on MI355X with the weights cold (us per call, graph replay, group size 128 unless said):
+//   * up to 4 rows, layers of up to 4096 columns (decode kernel with a workgroup per 16 columns, or every tile in two
+//     halves along K from 8192 channels): always.  4096 x 4096: 5.3-5.6 at one row, 7.4-8.0 at four, against 6.8-7.5
+//     and 7.8-10.5; 11008 x 4096: int4 9.0-9.4 / 11.5 against 13.5 / 15.3, int3 8.7 / 11.1 against 10.9 / 15.2;
+//   * up to 4 rows, wider layers (a workgroup per 32 columns): K = 4096: one and two rows always, three and four up
+//     to 16384 columns (4096 x 11008 with an activation order, one / two / four rows: int4 7.8 / 8.1 / 9.8 against
+//     8.1 / 11.0 / 11.1, int3 7.3 / 7.7 / 9.7 against 7.7 / 10.2 / 10.3; 4096 x 22016 one row 9.7 / 10.3 against
+//     11.4 / 12.8).  Longer K, one and two rows: always (8192 x 8192 9.7 / 9.9 against 14.0 / 13.3, 8192 x 28672
+//     24.6 / 26.4 against 32.3 / 30.2, 28672 x 8192 25.1 / 31.7 against 50.1 / 39.2; 36864 x 9216 int3 with one
+//     group and sixteen waves along K in two ranges: see the decode planner); three and four rows: K up to 6656, and
+//     up to 11008 for layers of up to 8192 columns (beyond, the four staged rows of x cost more than they save:
+//     8192 x 28672 41.9 against 30.4);
+//   * 5 to 16 rows: only layers without an activation order, K up to 4096 and more than 4096 columns (the matmul
+//     kernel then reads x itself, one launch: 4096 x 11008 int4, 5 / 8 / 16 rows: 10.6 / 10.7 / 11.5 against 11.2 /
+//     11.3 / 12.5; int3 from nine rows); with an activation order the pack pass makes it 14.6 against 13.4 at 8 rows;
+//   * 17 to 128 rows: almost everywhere (4096 x 11008 with an activation order, 32 / 64 / 128 rows: 14.8 / 19.2 /
+//     26.6 against 18.1 / 22.1 / 34.1), but for K of 8192 and more where the checkpoint-layout STREAM kernel has
+//     nothing to look up per weight: 4-bit layers without an activation order up to 64 rows (8192 x 8192, 17 / 64
+//     rows: 23.4 / 28.6 against 19.7 / 25.0) and layers of one group (9216 x 36864, 32 / 128 rows: 61.9 / 134 against
+//     54.6 / 126; 36864 x 9216 86.7 / 206 against 72.8 / 173; 9216 x 9216 keeps the tiled copy up to 32 rows);
+//   * above 128 rows: K up to 8192 (4096 x 11008, 512 rows: 75 against 95; 11008 x 4096: 127 against 81).
+bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
+{
+    if (M <= 4) {
+        if (N <= 4096) return true;
+        if (K <= 4096) return M <= 2 || N < 16384;
+        if (K > 32768) return false;
+        if (M <= 2) return true;
+        return K <= 6656 || (K <= 11008 && N <= 8192);
+    }
+    if (M <= 16) return !act_order && K <= 4096 && N > 4096 && (M >= 9 || bits == 4);
+    if (M <= 128) {
+        if (one_group && K > 8192 && (M > 32 || K > 16384 || N > 16384)) return false;
+        if (M <= 64 && K >= 8192 && bits == 4 && !act_order) return false;
+        return true;
+    }
+    return K <= 8192;
+}
+
+// The plan gptq_hip_gemm_sorted runs for M rows of a layer whose channels were sorted by group, if that path covers
+// the problem: the GROUPED family, or up to kSortedMaxRows rows on the STREAM kernel that reads x itself behind the
+// pass that reorders x (that pass costs a launch, ~2 us: int3 gains 2-4 us over the per-weight lookups of the
+// unsorted kernel at every size measured, int4 1-2 us at 4096 x 11008 and 11008 x 4096 but loses 0.7 us at
+// 4096 x 4096).
+bool sorted_plan(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan)
+{
+    const int gs = group_size == -1 ? K : group_size;
+    if ((bits != 3 && bits != 4) || K >= 65536 || K % gs != 0 || gs % (bits == 4 ? 8 : 32) != 0) return false;
+    if (gptq_hip_select(M, K, N, bits, group_size, 0, plan) != GPTQ_HIP_OK) return false;
+    if (plan->kernel == GPTQ_HIP_KERNEL_GROUPED) return true;
+    if (plan->kernel == GPTQ_HIP_KERNEL_STREAM && M <= gptq::kSortedMaxRows && plan->row_tiles == 1)
+        return bits == 3 || (long long)K * N >= (1LL << 25);
+    return false;
+}
+
+}  // namespace
+
+extern "C" int gptq_hip_select_route(int M, int K, int N, int bits, int group_size, int act_order, unsigned copies,
+                                     const int *switch_rows, gptq_hip_route *route)
+{
+    if (!route) return GPTQ_HIP_ERR_BAD_ARG;
+    memset(route, 0, sizeof(*route));
+    route->copy = GPTQ_HIP_ROUTE_LIBRARY;
+    if (bits != 2 && bits != 3 && bits != 4 && bits != 8) return GPTQ_HIP_ERR_BAD_ARG;
+    if (M < 1 || K < 32 || N < 32 || K % 32 != 0 || N % 32 != 0) return GPTQ_HIP_ERR_BAD_ARG;
+    if (group_size == 0 || group_size < -1) return GPTQ_HIP_ERR_BAD_ARG;
+    const unsigned all = GPTQ_HIP_COPY_CHECKPOINT | GPTQ_HIP_COPY_SORTED | GPTQ_HIP_COPY_TILED;
+    if (copies == 0 || (copies & ~all)) return GPTQ_HIP_ERR_BAD_ARG;
+    static const int kDefaultSwitch[3] = {1152, 1024, 640};
+    const int *sw = switch_rows ? switch_rows : kDefaultSwitch;
+    if (sw[0] < 0 || sw[1] < 0 || sw[2] < 0) return GPTQ_HIP_ERR_BAD_ARG;
+    const int gs = group_size == -1 ? K : group_size;
+    const bool one_group = gs >= K;
+    const bool act = act_order && !one_group;
+    const bool fused_bits = bits == 3 || bits == 4;   // the widths the kernels on the checkpoint layout take
+    const bool tiled_ok = (copies & GPTQ_HIP_COPY_TILED) && gptq::tiled_qualifies(K, N, bits, gs);
+    auto take_tiled = [&]() {
+        if (gptq_hip_select_tiled(M, K, N, bits, group_size, &route->plan) != GPTQ_HIP_OK) {
+            memset(&route->plan, 0, sizeof(route->plan));
+            return false;
+        }
+        route->copy = GPTQ_HIP_ROUTE_TILED;
+        return true;
+    };
+    if (copies == GPTQ_HIP_COPY_TILED) {
+        // the tiled copy is all the layer has: every M runs there
+        if (tiled_ok && take_tiled()) return GPTQ_HIP_OK;
+        return GPTQ_HIP_ERR_UNSUPPORTED;
+    }
+    bool tiled = false;
+    if (!fused_bits) {
+        if (!tiled_ok) return GPTQ_HIP_OK;   // 2 and 8 bits have no other fused kernels: the library
+        tiled = true;
+    } else if (tiled_ok && tiled_wins(M, K, N, act, bits, one_group)) {
+        tiled = true;
+    }
+    int threshold = sw[0];
+    if (threshold && !tiled) {   // off the tiled copy the library GEMM wins earlier
+        if (sw[1] && sw[1] < threshold) threshold = sw[1];
+        if (act && sw[2] && sw[2] < threshold) threshold = sw[2];
+    }
+    if (threshold && M >= threshold) return GPTQ_HIP_OK;
+    if (tiled && take_tiled()) return GPTQ_HIP_OK;
+    if (!fused_bits) return GPTQ_HIP_OK;
+    if ((copies & GPTQ_HIP_COPY_SORTED) && act && M <= gptq::kSortedMaxRows &&
+        sorted_plan(M, K, N, bits, group_size, &route->plan)) {
+        route->copy = GPTQ_HIP_ROUTE_SORTED;
+        return GPTQ_HIP_OK;
+    }
+    memset(&route->plan, 0, sizeof(route->plan));
+    if (copies & GPTQ_HIP_COPY_CHECKPOINT) {
+        const int rc = gptq_hip_select(M, K, N, bits, group_size, act ? 1 : 0, &route->plan);
+        if (rc == GPTQ_HIP_OK) {
+            route->copy = GPTQ_HIP_ROUTE_CHECKPOINT;
+            return GPTQ_HIP_OK;
+        }
+        memset(&route->plan, 0, sizeof(route->plan));
+        if (rc != GPTQ_HIP_ERR_UNSUPPORTED) return rc;
+    }
+    return GPTQ_HIP_OK;   // no fused kernel covers the call: dequant + library GEMM
 }
 
 extern "C" size_t gptq_hip_workspace_bytes(int M, int K, int N, int bits, int group_size, int act_order)

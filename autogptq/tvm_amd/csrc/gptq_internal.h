@@ -99,20 +99,6 @@ inline bool grouped_packable(int bits, int K, int gs, bool has_g_idx, int M, int
     const int groups = wave_groups_exact(kr / waves_k, gs);
     return grouped_wavex(true, kr / waves_k) && groups >= 1 && groups <= 4;
 }
-// Input channels of x the GATHER kernel stages per K wave at a time: fixed per (bits, row tiles) so
-// that the kernel's unrolled step loop knows its chunk boundaries at compile time.  The chunk is a
-// whole number of steps that divides the weight prefetch depth (8 steps int4, 4 steps int3).
-constexpr int gather_kc(int bits, int row_tiles)
-{
-    return bits == 4 ? (row_tiles >= 8 ? 64 : (row_tiles == 4 ? 128 : 256))
-                     : (row_tiles >= 4 ? 128 : (row_tiles == 2 ? 256 : 512));
-}
-// 16-byte vectors of x one thread of the GATHER kernel can stage per chunk
-constexpr int gather_xv(int bits, int row_tiles) { return (bits == 3 && row_tiles != 2) ? 16 : 8; }
-// group indices one thread can stage per chunk
-constexpr int gather_gv() { return 8; }
-int gather_lds_bytes(int G, int kc, int xs_rows, int row_tiles, int waves_n, int waves_k);
-
 // STREAM kernel sizing.  A row of its (scale, zero) table: 64 columns x (fp16 scale, fp16 zero),
 // padded by 16 bytes so that lane groups reading rows of different groups spread over the banks.
 static const int kStreamTableRow = 64 * 4 + 16;
@@ -148,7 +134,6 @@ size_t stream_xpack_bytes(int bits, int steps_pad, int rt_total);
 size_t stream_gpack_bytes(int bits, int steps_pad, int act_table);
 
 int launch_stream(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
-int launch_gather(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
 int launch_grouped(const Params &p, int bits, const gptq_hip_plan &plan, void *stream);
 int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
                    void *w, int K, int N, int G, int bits, int group_size, void *stream);

@@ -34,17 +34,15 @@ def _conv1d_type():
         return None
 
 
-def find_layers(module: nn.Module, layer_types=None, name: str = "", found: Optional[dict] = None) -> Dict[str, nn.Module]:
-    """``{qualified name: layer}`` of every Linear / Conv2d / Conv1D below ``module``."""
-    if found is None:
-        found = {}
-    if not layer_types:
-        layer_types = [t for t in (_conv1d_type(), nn.Conv2d, nn.Linear) if t is not None]
-    for child_name, child in module.named_children():
-        full = name + "." + child_name if name else child_name
-        if isinstance(child, tuple(layer_types)):
-            found[full] = child
-        find_layers(child, layer_types, full, found)
+def find_layers(module: nn.Module, layers=None, name: str = "") -> Dict[str, nn.Module]:
+    """``{qualified name: layer}`` of every Linear / Conv2d / Conv1D in ``module`` (``module`` itself under
+    ``name`` when it is one); ``layers`` names other layer types to look for.  Same result as the reference's
+    helper (auto_gptq/modeling/_utils.py:38-49), including its order (depth first, in registration order)."""
+    kinds = tuple(layers) if layers else tuple(t for t in (_conv1d_type(), nn.Conv2d, nn.Linear) if t is not None)
+    found = {}
+    for path, sub in module.named_modules(prefix=name, remove_duplicate=False):
+        if isinstance(sub, kinds):
+            found[path] = sub
     return found
 
 
@@ -96,15 +94,18 @@ def pack_model(model: nn.Module, quantizers: Dict[str, tuple], bits: int, group_
 
 
 def save_quantized(model: nn.Module, save_dir: str, bits: int, group_size: int, desc_act: bool = True,
-                   use_safetensors: bool = True, model_basename: Optional[str] = None) -> str:
+                   use_safetensors: bool = True, model_basename: Optional[str] = None, damp_percent: float = 0.01,
+                   sym: bool = True, true_sequential: bool = True) -> str:
     """Writes a packed model the way the reference lays a checkpoint out (auto_gptq/modeling/_base.py:381-401):
     ``gptq_model-{bits}bit-{group_size}g.{safetensors|bin}`` with every tensor of the state dict under its own
-    name, ``quantize_config.json`` (``_base.py:66-77``), and the model's ``config.json`` when it has one.  What
+    name, ``quantize_config.json`` with the six fields of the reference's ``BaseQuantizeConfig.to_dict``
+    (``_base.py:26-32,54-62``; their defaults are the reference's), and the model's ``config.json`` when it has one.  What
     it writes is what ``from_quantized`` reads.  Layers that kept only their tiled copy (``QuantLinear.compact``)
     have no checkpoint tensors left and cannot be saved.  Returns the path of the weight file."""
     for name, mod in model.named_modules():
         if isinstance(mod, QuantLinear) and getattr(mod, "_compact", False):
-            raise ValueError(f"{name} holds only its tiled copy (compact()): the checkpoint tensors are gone")
+            raise ValueError(f"{name} holds only its tiled copy (compact()): the checkpoint tensors are gone; load "
+                             f"the model with from_quantized(..., keep_checkpoint_tensors=True) to save it again")
     os.makedirs(save_dir, exist_ok=True)
     if model_basename is None:
         model_basename = f"gptq_model-{bits}bit-{group_size}g"
@@ -121,7 +122,8 @@ def save_quantized(model: nn.Module, save_dir: str, bits: int, group_size: int, 
     if config is not None and hasattr(config, "save_pretrained"):
         config.save_pretrained(save_dir)
     with open(os.path.join(save_dir, "quantize_config.json"), "w", encoding="utf-8") as f:
-        json.dump({"bits": int(bits), "group_size": int(group_size), "desc_act": bool(desc_act)}, f, indent=2)
+        json.dump({"bits": int(bits), "group_size": int(group_size), "damp_percent": float(damp_percent),
+                   "desc_act": bool(desc_act), "sym": bool(sym), "true_sequential": bool(true_sequential)}, f, indent=2)
     return path
 
 
@@ -186,18 +188,22 @@ def load_quantized_state(model: nn.Module, state: Dict[str, torch.Tensor], devic
 def from_quantized(save_dir: str, device="cuda:0", model_basename: Optional[str] = None,
                    use_safetensors: bool = True, ignore_layers: Iterable[str] = ("lm_head",),
                    trust_remote_code: bool = False, fuse_shared_inputs: bool = False,
-                   prepare_decode: bool = False, prepare_tiled: bool = False, compact: bool = False):
+                   prepare_decode: bool = False, prepare_tiled: bool = False, compact: Optional[bool] = None,
+                   keep_checkpoint_tensors: bool = False):
     """Builds the ``transformers`` causal LM described by ``save_dir/config.json`` with every linear
     layer (except ``ignore_layers`` prefixes: the reference skips ``lm_head`` and the modules outside
     the decoder stack) replaced by ``QuantLinear``, and fills it from
     ``save_dir/gptq_model-{bits}bit-{group_size}g.{safetensors|bin}``.  ``fuse_shared_inputs`` then merges
     q/k/v and gate/up projections into one product each (``fused.fuse_shared_input_layers``; an inference
     optimisation the reference does not have: the state-dict names of those layers change).
-    ``prepare_decode`` builds the sorted copies of activation-order layers now instead of on their first
-    decode-size call (needed before capturing the model in a graph: the preparation allocates);
-    ``prepare_tiled`` does the same for the copies in the tiled format that prompt-size calls use.
-    ``compact`` keeps the tiled copy as the only weights of every layer it covers (``QuantLinear.compact``:
-    no second or third copy in device memory, and no checkpoint tensors left to save).
+    Every layer the tiled format covers ends up holding ONE copy of its weights, the tiled one
+    (``QuantLinear.compact``: the reference's TVM module likewise keeps only its own re-laid weights,
+    auto_gptq/nn_modules/qlinear_tvm.py:25-40,105-107): device memory per layer is its packed size, every row count
+    runs on the tiled kernels, and no call allocates a copy later.  Such a model cannot be saved again or give
+    gradients for its inputs; ``keep_checkpoint_tensors=True`` (or ``compact=False``) keeps the checkpoint's tensors
+    instead, and the module then builds the copies it wants on first use: ``prepare_decode`` builds the sorted
+    copies of activation-order layers at load instead (needed before capturing such a model in a graph: the
+    preparation allocates), ``prepare_tiled`` the copies in the tiled format.
     Returns ``(model, quantize_config)``."""
     import accelerate
     from transformers import AutoConfig, AutoModelForCausalLM
@@ -234,6 +240,8 @@ def from_quantized(save_dir: str, device="cuda:0", model_basename: Optional[str]
         from .fused import fuse_shared_input_layers
 
         fuse_shared_input_layers(model)
+    if compact is None:
+        compact = not (keep_checkpoint_tensors or prepare_decode or prepare_tiled)
     for mod in model.modules():
         if not isinstance(mod, QuantLinear):
             continue

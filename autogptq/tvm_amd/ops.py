@@ -117,25 +117,14 @@ SORTED_MAX_ROWS = 16
 
 
 def sorted_plan(M: int, K: int, N: int, bits: int, group_size: int) -> Optional[_lib.Plan]:
-    """The plan ``gemm_sorted`` would run, or None when the sorted path does not cover the problem
-    (it is for decode sizes: the GROUPED family, or up to ``SORTED_MAX_ROWS`` rows on the STREAM kernel
-    that reads x itself)."""
-    gs = K if group_size == -1 else group_size
-    if K >= 65536 or K % gs != 0 or gs % (8 if bits == 4 else 32) != 0:
-        return None
+    """The plan ``gemm_sorted`` would run, or None when the sorted path does not cover the problem (it is for
+    decode sizes: the GROUPED family, or up to ``SORTED_MAX_ROWS`` rows on the STREAM kernel that reads x itself):
+    the library's rule (gptq_hip_select_route with only the sorted copy on offer)."""
     try:
-        plan = _lib.select(M, K, N, bits, group_size, False)
+        r = _lib.select_route(M, K, N, bits, group_size, True, copies=_lib.COPY_SORTED, switch_rows=(0, 0, 0))
     except _lib.GptqHipError:
         return None
-    if plan.kernel == _lib.KERNEL_GROUPED:
-        return plan
-    if plan.kernel == _lib.KERNEL_STREAM and M <= SORTED_MAX_ROWS and plan.row_tiles == 1:
-        # the pass that reorders x costs a launch (~2 us): int3 gains 2-4 us over the per-weight lookups
-        # of the unsorted kernel at every size measured, int4 1-2 us at 4096 x 11008 and 11008 x 4096
-        # but loses 0.7 us at 4096 x 4096
-        if bits == 3 or K * N >= (1 << 25):
-            return plan
-    return None
+    return r.plan if r.copy == _lib.ROUTE_SORTED else None
 
 
 def gemm_sorted(x: torch.Tensor, qweight_sorted: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
@@ -259,7 +248,7 @@ def gemm_tiled(x: torch.Tensor, qtile: torch.Tensor, sz: torch.Tensor, xsrc: Opt
         return out
     if plan is None:
         plan = _lib.select_tiled(M, K, N, bits, group_size)
-    slots = plan.kernel == _lib.KERNEL_TILED_DECODE and plan.split_k == 1   # (halved tiles: a workspace of their own)
+    slots = bool(plan.flags & _lib.PLAN_PRIVATE_ZERO_WORKSPACE)   # (halved tiles: a workspace of their own)
     ws = _workspace(dev, plan.workspace_bytes, 1 if slots else 0) if plan.workspace_bytes else None
     with torch.cuda.device(dev):
         rc = _lib.lib().gptq_hip_gemm_tiled(_ptr(x), _ptr(qtile), _ptr(sz), _ptr(xsrc), _ptr(kinv), _ptr(bias), _ptr(out),
@@ -341,66 +330,10 @@ def gemm_tiled_transposed(gy: torch.Tensor, qtile_t: torch.Tensor, szt: torch.Te
 
 
 def tiled_wins(M: int, K: int, N: int, act_order: bool, bits: int = 4, one_group: bool = False) -> bool:
-    """Where the tiled kernels were measured faster than the ones that read the checkpoint layout (or its
-    sorted copy), on MI355X with the weights cold, group size 128 (us, graph replay):
-      * up to 4 rows, layers of up to 4096 columns (decode kernel with a workgroup per 16 columns, every CU at
-        work): always.  4096 x 4096: 5.3-5.6 at one row, 7.4-8.0 at four, against 6.8-7.5 and 7.8-10.5;
-        11008 x 4096 (K of 8192 and more: the tile kernel with every tile in two halves along K): int4 9.0-9.4 /
-        11.5 against 13.5 / 15.3, int3 8.7 / 11.1 against 10.9 / 15.2;
-      * up to 4 rows, wider layers (a workgroup per 32 columns, x staged per workgroup, four to sixteen waves
-        along K so that a wave walks about sixteen blocks):
-        K = 4096: one and two rows always, three and four up to 16384 columns.  Up to 128 tiles past a whole number
-        per CU run as two halves along K (a tagged 64-bit exchange joins them), so that the fullest CU holds half
-        a tile more than the others, not a whole one.  4096 x 11008, one / two / four rows, with an activation order: int4 7.8 / 8.1 / 9.8 against
-        8.1 / 11.0 / 11.1, int3 7.3 / 7.7 / 9.7 against 7.7 / 10.2 / 10.3; without: int4 7.8 / 8.1 / 8.7 against
-        7.9 / 8.8 / 8.9, int3 7.2 / 7.5 / 8.2 against 7.3 / 8.3 / 8.2; 4096 x 12288 int4 8.3 / 8.5 / 10.1 against
-        8.2 / 11.0 / 11.1; 4096 x 14336 int4 9.0 / 9.4 / 11.2 against 9.0 / 11.2 / 11.1; 4096 x 22016 int3 / int4,
-        one row, 9.7 / 10.3 against 11.4 / 12.8;
-        longer K, one and two rows: always up to K = 32768 (with an activation order, int4, one / two rows:
-        5120 x 13824 9.7 / 10.5 against 18.2 / 15.2, 6656 x 17920 15.1 / 15.4 against 27.9 / 27.2, 8192 x 8192
-        9.7 / 9.9 against 14.0 / 13.3, 8192 x 28672 24.6 / 26.4 against 32.3 / 30.2, 13824 x 5120 11.6 / 12.4
-        against 21.2 / 17.6, 17920 x 6656 14.8 / 16.2 against 31.0 / 23.8, 28672 x 8192 25.1 / 31.7 against
-        50.1 / 39.2, 9216 x 36864 int3 29.7 / 33.0 against 36.0 / 49.9; 36864 x 9216: 76 against 36, hence the
-        bound; 9216 x 9216 int3 with one group, one row: 10.8 against 12.5 since its 32 tiles past a whole
-        number per CU are halved);
-        longer K, three and four rows: K up to 6656 (5120 x 13824 12.8 against 15.4, 6656 x 17920 22.3 against
-        26.8) and up to 8192 columns for K up to 11008 (8192 x 8192 12.3 against 13.3, 11008 x 8192 15.6 against
-        19.6); beyond, the four staged rows of x cost more than they save
-        (8192 x 28672 41.9 against 30.4, 17920 x 6656 29.9 against 23.9);
-      * 5 to 16 rows: only layers without an activation order, K up to 4096 and more than 4096 columns (the
-        matmul kernel then reads x itself, one launch; 4096 x 11008 int4, 5 / 8 / 16 rows: 10.6 / 10.7 / 11.5
-        against 11.2 / 11.3 / 12.5; int3 from nine rows: 11.5 against 12.8 at sixteen, 10.9 against 10.4 at
-        eight); with an activation order the pack pass makes it 14.6 against 13.4 at 8 rows, and narrower or
-        longer layers split K and add a pass (11008 x 4096: 17.3 against 13.1);
-      * 17 to 128 rows: almost everywhere within 4 % or better (4096 x 11008 with an activation order, 32/64/128
-        rows: 14.8/19.2/26.6 against 18.1/22.1/34.1).  Two exceptions, both with K of 8192 and more and nothing
-        for the checkpoint-layout STREAM kernel to look up per weight: 4-bit layers without an activation order
-        up to 64 rows (17 / 64 rows: 8192 x 8192 23.4 / 28.6 against 19.7 / 25.0, 8192 x 28672 44.8 / 58.9 against
-        40.4 / 55.4, 28672 x 8192 47.7 / 58.7 against 43.8 / 57.2; at 128 rows the tiled kernel is ahead again on
-        wide layers, 8192 x 28672 88 against 105; 3-bit layers stay: 9216 x 9216 28.4 against 32.6), and layers of
-        one group (``one_group``; 32 / 128 rows: 9216 x 36864 61.9 / 134 against 54.6 / 126, 36864 x 9216 86.7 / 206
-        against 72.8 / 173; 9216 x 9216 keeps the tiled copy up to 32 rows, 30.2 against 33.0);
-      * above 128 rows: K up to 8192 (4096 x 11008, 512 rows: 75 against 95; 11008 x 4096: 127 against 81,
-        where every workgroup pulls 2.8 MB of x fragments and they no longer stay in one L2)."""
-    if M <= 4:
-        if N <= 4096:
-            return True
-        if K <= 4096:
-            return M <= 2 or N < 16384
-        if K > 32768:
-            return False
-        if M <= 2:
-            return True
-        return K <= 6656 or (K <= 11008 and N <= 8192)
-    if M <= 16:
-        return not act_order and K <= 4096 and N > 4096 and (M >= 9 or bits == 4)
-    if M <= 128:
-        if one_group and K > 8192 and (M > 32 or K > 16384 or N > 16384):
-            return False
-        if M <= 64 and K >= 8192 and bits == 4 and not act_order:
-            return False
-        return True
-    return K <= 8192
+    """Whether a call with M rows runs on the tiled copy of a layer that holds all three copies (group size 128,
+    or one group): the library's own rule (gptq_hip_select_route), where the measurements behind it are kept."""
+    gs = -1 if one_group else 128
+    return _lib.select_route(M, K, N, bits, gs, act_order, switch_rows=(0, 0, 0)).copy == _lib.ROUTE_TILED
 
 
 def dequant(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,

@@ -83,9 +83,8 @@ class QuantLinear(nn.Module):
         # device memory; False keeps only the checkpoint's tensors.
         self.sort_for_decode = sort_for_decode
         self._sorted = None   # (key, (qweight_sorted, kmap) or None)
-        self._sorted_plans = {}  # M -> plan of the sorted path, or None where it does not apply
         # Every fused layer whose groups are whole multiples of 32 channels: on the first call with a row count
-        # the tiled kernels are faster at (ops.tiled_wins), keep a copy of the layer in the order the matrix
+        # the tiled kernels are faster at (the library's routing rule, gptq_hip_select_route), keep a copy of the layer in the order the matrix
         # instructions consume (gptq_hip_tile_prepare).  Costs the layer's packed size again; False keeps
         # the checkpoint's tensors (and the sorted copy) only.  compact() makes it the only copy.
         self.tile_for_prefill = tile_for_prefill
@@ -228,6 +227,10 @@ class QuantLinear(nn.Module):
             if t is not None:
                 gx = ops.gemm_tiled_transposed(gy, t[0], t[1], t[2], self.infeatures, self.bits, self.groupsize)
         if gx is None:
+            if self._compact:
+                raise RuntimeError("this layer keeps only its tiled copy (compact()) and has no copy for the gradient "
+                                   "of its input: call prepare_transposed() before compact(), or load the model with "
+                                   "keep_checkpoint_tensors=True")
             gx = torch.matmul(gy, self.dequantize().t())
         return gx.reshape(grad_out.shape[:-1] + (self.infeatures,))
 
@@ -263,12 +266,23 @@ class QuantLinear(nn.Module):
                 self._tiled_t = (None, tuple(None if t is None else fn(t) for t in self._tiled_t[1]))
         return self
 
-    def _sorted_tensors(self, M):
-        """The sorted copy when the decode path through it covers M rows, else None."""
-        plans = self._sorted_plans
-        if M not in plans:
-            plans[M] = ops.sorted_plan(M, self.infeatures, self.outfeatures, self.bits, self.groupsize)
-        return self.prepare_decode() if plans[M] is not None else None
+    # ------------------------------------------------------------------ copying, pickling
+    def __getstate__(self):
+        """A route holds bound C++ launch objects and closures over this module's tensors: a copy of the module
+        (``copy.deepcopy``, ``pickle``, ``torch.save(model)``) gets none of them and decides its routes again.
+        Prepared copies beside the checkpoint tensors are rebuilt by the copy as well; the tiled copy of a compact
+        layer IS its weights and travels."""
+        state = dict(self.__dict__)
+        state["_routes"] = {}
+        state["_g_state"] = None
+        state["_sorted"] = None
+        if not self._compact:
+            state["_tiled"] = None
+            state["_tiled_t"] = None
+        return state
+
+    def __setstate__(self, state):
+        super().__setstate__(state)
 
     # ------------------------------------------------------------------ routing
     def __setattr__(self, name, value):
@@ -314,50 +328,53 @@ class QuantLinear(nn.Module):
 
         g = self._kernel_g_idx()
         K, N = self.infeatures, self.outfeatures
-        tiled = None
-        if self.bits not in self.FUSED_BITS:
-            # 2 and 8 bits: the tiled kernels are the only fused ones
-            tiled = self.prepare_tiled() if self.tile_for_prefill else None
-            if tiled is None:
-                return "library", library
-        elif self.tile_for_prefill and ops.tiled_wins(M, K, N, g is not None, bits, one_group=self.groupsize >= K):
-            tiled = self.prepare_tiled()
-        threshold = self.kernel_switch_threshold
-        if threshold and tiled is None:   # off the tiled route the library wins earlier
-            if self.plain_switch_threshold:
-                threshold = min(threshold, self.plain_switch_threshold)
-            if self.act_order_switch_threshold and g is not None:
-                threshold = min(threshold, self.act_order_switch_threshold)
-        if threshold and M >= threshold:
+        # Which copy the call runs on is the library's decision (gptq_hip_select_route): this module says which
+        # copies it may hold and from how many rows it prefers the library GEMM, and builds the copy that was
+        # chosen; a copy that the layer's contents do not allow (groups of unequal size) is taken off the offer
+        # and the question asked again.
+        copies = _lib.COPY_CHECKPOINT
+        if self.sort_for_decode and self.bits in self.FUSED_BITS:
+            copies |= _lib.COPY_SORTED
+        if self.tile_for_prefill:
+            copies |= _lib.COPY_TILED
+        switch_rows = (self.kernel_switch_threshold or 0,
+                       self.plain_switch_threshold if self.kernel_switch_threshold else 0,
+                       self.act_order_switch_threshold if self.kernel_switch_threshold else 0)
+        while True:
+            r = _lib.select_route(M, K, N, bits, gs, g is not None, copies, switch_rows)
+            if r.copy == _lib.ROUTE_TILED:
+                tiled = self.prepare_tiled()
+                if tiled is None:
+                    copies &= ~_lib.COPY_TILED
+                    continue
+                xsrc, kinv = (tiled[2], tiled[3]) if g is not None else (None, None)
+                return "tiled", bind(2, tiled[0], tiled[1], None, xsrc, kinv)
+            if r.copy == _lib.ROUTE_SORTED:
+                srt = self.prepare_decode()
+                if srt is None:
+                    copies &= ~_lib.COPY_SORTED
+                    continue
+                return "sorted", bind(1, srt[0], self.qzeros, self.scales, srt[1], None)
+            if r.copy == _lib.ROUTE_CHECKPOINT:
+                return "plain", bind(0, self.qweight, self.qzeros, self.scales, g, None)
             return "library", library
-        if tiled is not None:
-            qtile, sz = tiled[0], tiled[1]
-            xsrc, kinv = (tiled[2], tiled[3]) if g is not None else (None, None)
-            return "tiled", bind(2, qtile, sz, None, xsrc, kinv)
-        qzeros, scales = self.qzeros, self.scales
-        srt = self._sorted_tensors(M) if (self.sort_for_decode and M <= ops.SORTED_MAX_ROWS) else None
-        if srt is not None:
-            qs, kmap = srt
-            return "sorted", bind(1, qs, qzeros, scales, kmap, None)
-        try:
-            _lib.select(M, K, N, bits, gs, g is not None)
-        except _lib.GptqHipError as e:
-            if e.status != _lib.ERR_UNSUPPORTED:
-                raise
-            return "library", library
-        qweight = self.qweight
-        return "plain", bind(0, qweight, qzeros, scales, g, None)
 
     def route(self, M: int) -> str:
         """The path a call with M rows takes (see ``_route``); builds the prepared copy it needs."""
         return self._routed(M)[2]
 
+    def _fresh(self, r):
+        """Whether a cached route still describes the module: the same buffer objects (code that swaps a buffer
+        through ``module._buffers[name] = t`` passes ``__setattr__`` by), not written since."""
+        a, b, c, d = r[0]
+        buf = self._buffers
+        return (a is buf["qweight"] and b is buf["qzeros"] and c is buf["scales"] and d is buf["g_idx"]
+                and a._version + b._version + c._version + d._version == r[1])
+
     def _routed(self, M):
         r = self._routes.get(M)
-        if r is not None:
-            a, b, c, d = r[0]
-            if a._version + b._version + c._version + d._version == r[1]:
-                return r
+        if r is not None and self._fresh(r):
+            return r
         what, fn = self._route(M)
         w = self._watched()               # (read after routing: the preparations may have re-made g_idx)
         r = (w, sum(t._version for t in w), what, fn)
@@ -366,14 +383,12 @@ class QuantLinear(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         # the common case first: a contiguous fp16 matrix, no gradient wanted, a row count seen before and
-        # buffers not written since (replacing a buffer or moving the module empties the table)
+        # buffers neither replaced nor written since
         if x.dim() == 2 and x.dtype is torch.float16 and x.is_contiguous() and not (
                 x.requires_grad and torch.is_grad_enabled()):
             r = self._routes.get(x.size(0))
-            if r is not None:
-                a, b, c, d = r[0]
-                if a._version + b._version + c._version + d._version == r[1]:
-                    return r[3](x)
+            if r is not None and self._fresh(r):
+                return r[3](x)
         out_shape = x.shape[:-1] + (self.outfeatures,)
         x2 = x.reshape(-1, x.shape[-1])
         if x2.dtype != torch.float16:
@@ -396,10 +411,17 @@ class QuantLinear(nn.Module):
     def dequantize(self) -> torch.Tensor:
         """fp16 [infeatures, outfeatures], the weight the reference materialises on every call."""
         if self._compact:
-            # the tiled kernels form the same rounded fp16 weights: the product with the identity is W itself
-            eye = torch.eye(self.infeatures, dtype=torch.float16, device=self._tiled[1][0].device)
+            # the tiled kernels form the same rounded fp16 weights: the product with the identity is W itself,
+            # taken 1024 rows of the identity at a time (a debugging aid: it costs a K-row product)
             qtile, sz, xsrc, kinv = self._tiled[1]
-            return ops.gemm_tiled(eye, qtile, sz, xsrc, kinv, None, self.bits, self.groupsize)
+            K, dev = self.infeatures, qtile.device
+            w = torch.empty((K, self.outfeatures), dtype=torch.float16, device=dev)
+            for k0 in range(0, K, 1024):
+                rows = min(1024, K - k0)
+                eye = torch.zeros((rows, K), dtype=torch.float16, device=dev)
+                eye[torch.arange(rows, device=dev), torch.arange(k0, k0 + rows, device=dev)] = 1
+                ops.gemm_tiled(eye, qtile, sz, xsrc, kinv, None, self.bits, self.groupsize, out=w[k0:k0 + rows])
+            return w
         return ops.dequant(self.qweight, self.qzeros, self.scales, self._kernel_g_idx(), self.bits, self.groupsize)
 
     def extra_repr(self) -> str:

@@ -36,7 +36,7 @@ typedef enum gptq_hip_status {
 
 /* kernel families the dispatcher chooses between */
 enum {
-    GPTQ_HIP_KERNEL_GATHER = 1, /* exact fp16 weights, x staged through LDS by the workgroup; any g_idx, any M */
+    /* 1: a retired family; no plan names it */
     GPTQ_HIP_KERNEL_GROUPED = 2, /* rows expanded by group, scales applied once per group; M <= 2 with few groups,
                                     or M <= 8 with contiguous groups (activation rows packed into the
                                     operand tile: such plans have row_tiles = 4 or 8) */
@@ -71,8 +71,15 @@ typedef struct gptq_hip_plan {
     int grid_x, grid_y, grid_z;
     int block;              /* threads per workgroup */
     int lds_bytes;          /* dynamic LDS per workgroup */
-    size_t workspace_bytes; /* 0 when the plan needs none (GATHER / GROUPED with split_k == 1) */
+    int flags;              /* GPTQ_HIP_PLAN_* bits */
+    size_t workspace_bytes; /* 0 when the plan needs none (e.g. GROUPED with split_k == 1) */
 } gptq_hip_plan;
+
+/* gptq_hip_plan.flags */
+/* The plan's workspace must be ALL zero at the first call, is left all zero by every call, and must not be shared
+ * with plans that lack this flag (they write theirs): give such plans a buffer of their own.  Set by the decode
+ * plans of the tiled family whose tiles are halved along K (the halves meet in 64-bit slots of the workspace). */
+#define GPTQ_HIP_PLAN_PRIVATE_ZERO_WORKSPACE 1
 
 /*
  * Shape dispatcher: a pure host function (no GPU needed).  Takes the place of
@@ -207,7 +214,8 @@ int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_size, gptq_hi
 
 /* The plan of the family's decode kernel (GPTQ_HIP_KERNEL_TILED_DECODE), M <= 4 rows (GPTQ_HIP_ERR_UNSUPPORTED
  * above); gptq_hip_select_tiled chooses it by itself for those row counts and the matmul kernel above.  No counterpart in the reference, whose
- * GEMV handler takes one row (pycuda_warpper.py:150-152). */
+ * GEMV handler takes one row (pycuda_warpper.py:150-152).  Plans with halved tiles carry
+ * GPTQ_HIP_PLAN_PRIVATE_ZERO_WORKSPACE. */
 int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan);
 
 /*
@@ -215,10 +223,10 @@ int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int group_size, 
  * (pycuda_warpper.py:138, qlinear_tvm.py:123,150).  x and y are in the layer's own channel order (xsrc = kinv =
  * NULL means no activation order; pass both or neither).  plan: NULL = gptq_hip_select_tiled.  workspace:
  * plan.workspace_bytes (none for most decode plans).  M <= 4: one launch (the decode kernel); above: two
- * (pack pass, matmul); one more when the plan splits K.  A decode plan (GPTQ_HIP_KERNEL_TILED_DECODE) with split_k = 1 that asks
- * for a workspace wants ALL its bytes zero at the first call and leaves them zero (the two halves of a tile that
- * is halved along K meet in 64-bit slots behind the counters): give such plans a workspace of their own, which no
- * other entry point writes between the calls.
+ * (pack pass, matmul); one more when the plan splits K.  A plan whose flags hold
+ * GPTQ_HIP_PLAN_PRIVATE_ZERO_WORKSPACE wants ALL bytes of its workspace zero at the first call and leaves them zero
+ * (the two halves of a tile that is halved along K meet in 64-bit slots behind the counters): give such plans a
+ * workspace of their own, which no other entry point writes between the calls.
  */
 int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint32_t *sz, const int32_t *xsrc, const uint16_t *kinv,
                         const void *bias, void *y, void *workspace, size_t workspace_bytes, int M, int K, int N,
@@ -251,6 +259,34 @@ int gptq_hip_gemm_tiled_transposed(const void *gy, const void *qtile_t, const ui
                                    int group_size, const gptq_hip_plan *plan, void *stream);
 
 /*
+ * Which copy of a layer a call with M rows runs on, and the plan there: the whole decision the reference's handler
+ * makes in one place, from the row count to a kernel and its launch geometry (TVMHandler.__call__,
+ * auto_gptq/nn_modules/tvm_untils/pycuda_warpper.py:138-189).  A pure host function.
+ *   copies       the copies of the layer the caller holds or is willing to prepare (GPTQ_HIP_COPY_* bits):
+ *                CHECKPOINT = qweight / qzeros / scales / g_idx as loaded (gptq_hip_gemm_plan), SORTED = the
+ *                channel-sorted copy (gptq_hip_sort_channels, gptq_hip_gemm_sorted), TILED = the tiled format
+ *                (gptq_hip_tile_prepare, gptq_hip_gemm_tiled).  TILED alone describes a layer that keeps only its
+ *                tiled copy: every M then runs there.
+ *   switch_rows  rows of x from which the caller prefers W from gptq_hip_dequant and its own fp16 GEMM (what the
+ *                reference does from kernel_switch_threshold rows, auto_gptq/nn_modules/qlinear.py:25,198): three
+ *                values, for calls on the tiled copy, on the checkpoint tensors, and on the checkpoint tensors of a
+ *                layer with an activation order; 0 = never.  NULL = the measured defaults {1152, 1024, 640}.
+ * route->copy names the entry point (GPTQ_HIP_ROUTE_LIBRARY: no fused kernel; dequant + library GEMM) and
+ * route->plan is the plan to hand to it (zeroed for LIBRARY).  A SORTED or TILED answer for a copy that turns out not
+ * to exist (gptq_hip_sort_channels / gptq_hip_tile_prepare refused the layer's contents) is retried with that bit
+ * cleared.
+ */
+enum { GPTQ_HIP_COPY_CHECKPOINT = 1, GPTQ_HIP_COPY_SORTED = 2, GPTQ_HIP_COPY_TILED = 4 };
+enum { GPTQ_HIP_ROUTE_CHECKPOINT = 0, GPTQ_HIP_ROUTE_SORTED = 1, GPTQ_HIP_ROUTE_TILED = 2, GPTQ_HIP_ROUTE_LIBRARY = 3 };
+typedef struct gptq_hip_route {
+    int copy;           /* GPTQ_HIP_ROUTE_* */
+    int reserved;
+    gptq_hip_plan plan;
+} gptq_hip_route;
+int gptq_hip_select_route(int M, int K, int N, int bits, int group_size, int act_order, unsigned copies,
+                          const int *switch_rows, gptq_hip_route *route);
+
+/*
  * W fp16 [K, N] = scales[g] * (q - (zq[g] + 1)), one rounding per element:
  * the materialised weight of qlinear.py:198-242, for the bit-exact check.  bits may also be 2 or 8
  * here (the other widths of the format, qlinear.py:31-32,211-215): without a tiled copy those layers run as
@@ -263,7 +299,7 @@ int gptq_hip_dequant(const int32_t *qweight, const int32_t *qzeros, const void *
 const char *gptq_hip_strerror(int status);
 
 /* ABI version of this library (bumped when a signature or gptq_hip_plan changes). */
-#define GPTQ_HIP_ABI_VERSION 3
+#define GPTQ_HIP_ABI_VERSION 4
 int gptq_hip_abi_version(void);
 
 /* Digest of the sources this library was built from (set by the build script; "unknown" otherwise), so that a

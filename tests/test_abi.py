@@ -61,7 +61,7 @@ def test_select_plans_are_consistent(bits, M, KN, gs):
         gs = 32
     for act in (False, True):
         p = _lib.select(M, K, N, bits, gs, act)
-        assert p.kernel in (_lib.KERNEL_GATHER, _lib.KERNEL_GROUPED, _lib.KERNEL_STREAM)
+        assert p.kernel in (_lib.KERNEL_GROUPED, _lib.KERNEL_STREAM)
         if p.kernel == _lib.KERNEL_GROUPED:
             # one or two rows, or up to eight packed into one or two operand tiles (contiguous groups only)
             assert M <= 8 and 1 <= p.row_tiles <= 8 and p.m_blocks == 1
@@ -198,9 +198,9 @@ def test_entry_points_reject_null_and_bad_sizes_before_touching_the_gpu():
 
 
 def test_plan_for_forces_family_split_and_waves():
-    p = _lib.plan_for(_lib.KERNEL_GATHER, 1, 4096, 11008, 3, 128, True, split_k=5, waves_n=2)
-    assert p.kernel == _lib.KERNEL_GATHER and p.split_k == 5 and p.grid_y == 5 and p.waves_n == 2
-    assert p.grid_x == 11008 // 128 and p.block == 128
+    with pytest.raises(_lib.GptqHipError) as e:      # family 1 has been retired
+        _lib.plan_for(1, 1, 4096, 11008, 3, 128, True, split_k=5, waves_n=2)
+    assert e.value.status == _lib.ERR_UNSUPPORTED
     p = _lib.plan_for(_lib.KERNEL_GROUPED, 1, 4096, 11008, 3, 128, True, split_k=8)
     assert p.kernel == _lib.KERNEL_GROUPED and p.split_k == 8 and p.row_tiles == 2
     assert p.waves_n * p.waves_k * 64 == p.block
@@ -211,7 +211,7 @@ def test_plan_for_forces_family_split_and_waves():
     with pytest.raises(_lib.GptqHipError):
         _lib.plan_for(_lib.KERNEL_GROUPED, 1, 4096, 4096, 4, 32, True)
     with pytest.raises(_lib.GptqHipError) as e:
-        _lib.plan_for(_lib.KERNEL_GATHER, 1, 4096, 4096, 4, 128, True, waves_n=3)
+        _lib.plan_for(_lib.KERNEL_GROUPED, 1, 4096, 4096, 4, 128, True, waves_n=3)
     assert e.value.status == _lib.ERR_BAD_ARG
 
 
@@ -250,12 +250,10 @@ def test_dispatcher_families_by_m():
     # forcing the STREAM family with waves along K and a split
     p = _lib.plan_for(_lib.KERNEL_STREAM, 40, 4096, 352, 3, 128, True, split_k=2, waves_n=8)
     assert p.kernel == _lib.KERNEL_STREAM and p.waves_k == 8 and p.waves_n == 1 and p.split_k == 2 and p.block == 512
-    # more groups than the LDS table of STREAM holds: the GATHER fallback, or unsupported
-    try:
-        p = _lib.select(4, 36864, 9216, 4, 32, True)
-        assert p.kernel == _lib.KERNEL_GATHER
-    except _lib.GptqHipError as e:
-        assert e.status == _lib.ERR_UNSUPPORTED
+    # more groups than the LDS table of STREAM holds: no fused kernel on the checkpoint layout
+    with pytest.raises(_lib.GptqHipError) as e:
+        _lib.select(4, 36864, 9216, 4, 32, True)
+    assert e.value.status == _lib.ERR_UNSUPPORTED
 
 
 def test_single_group_ignores_act_order():
@@ -362,3 +360,99 @@ def test_transposed_plans_are_consistent(bits, KN):
     assert lib.gptq_hip_tiled_transposed_table_bytes(K, N, gs) == (K // gs) * blocks * 256
     with pytest.raises(_lib.GptqHipError):
         _lib.select_tiled_transposed(1, K, N, bits, 16)
+
+
+# ---- which copy a call runs on (gptq_hip_select_route)
+def table_tiled_wins(M, K, N, act_order, bits, one_group):
+    """The measured table the route rule was written from, stated once more as data-like branches: which row
+    counts and shapes the tiled copy won at (group size 128 or one group)."""
+    if M <= 4:
+        if N <= 4096:
+            return True
+        if K <= 4096:
+            return M <= 2 or N < 16384
+        if K > 32768:
+            return False
+        return M <= 2 or K <= 6656 or (K <= 11008 and N <= 8192)
+    if M <= 16:
+        return (not act_order) and K <= 4096 and N > 4096 and (M >= 9 or bits == 4)
+    if M <= 128:
+        if one_group and K > 8192 and (M > 32 or K > 16384 or N > 16384):
+            return False
+        return not (M <= 64 and K >= 8192 and bits == 4 and not act_order)
+    return K <= 8192
+
+
+ROUTE_SHAPES = [(4096, 4096), (4096, 11008), (11008, 4096), (4096, 22016), (8192, 8192), (8192, 28672),
+                (9216, 9216), (9216, 36864), (36864, 9216), (5120, 13824), (6656, 17920)]
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+@pytest.mark.parametrize("KN", ROUTE_SHAPES)
+def test_route_follows_the_measured_table(bits, KN):
+    K, N = KN
+    for gs in (128, -1):
+        if gs == 128 and K % 128 != 0:
+            continue
+        one_group = gs == -1
+        for act in (False, True):
+            for M in (1, 2, 3, 4, 5, 8, 9, 16, 17, 32, 33, 64, 65, 128, 129, 256, 639, 640, 1023, 1024, 1151, 1152, 4096):
+                r = _lib.select_route(M, K, N, bits, gs, act)
+                act_eff = act and not one_group
+                tiled = table_tiled_wins(M, K, N, act_eff, bits, one_group)
+                limit = 1152 if tiled else (640 if act_eff else 1024)
+                if M >= limit:
+                    assert r.copy == _lib.ROUTE_LIBRARY and r.plan.kernel == 0, (M, K, N, gs, act)
+                    continue
+                if tiled:
+                    assert r.copy == _lib.ROUTE_TILED, (M, K, N, gs, act)
+                    assert r.plan.as_dict() == _lib.select_tiled(M, K, N, bits, gs).as_dict()
+                    continue
+                assert r.copy in (_lib.ROUTE_SORTED, _lib.ROUTE_CHECKPOINT, _lib.ROUTE_LIBRARY), (M, K, N, gs, act)
+                if r.copy == _lib.ROUTE_SORTED:
+                    assert act_eff and M <= 16
+                    assert r.plan.as_dict() == _lib.select(M, K, N, bits, gs, False).as_dict()
+                elif r.copy == _lib.ROUTE_CHECKPOINT:
+                    assert r.plan.as_dict() == _lib.select(M, K, N, bits, gs, act_eff).as_dict()
+
+
+def test_route_honours_the_copies_on_offer_and_the_switch_rows():
+    K, N = 4096, 11008
+    # a layer that keeps only its tiled copy: every row count runs there, whatever the switch says
+    for M in (1, 8, 128, 5000):
+        r = _lib.select_route(M, K, N, 4, 128, True, copies=_lib.COPY_TILED)
+        assert r.copy == _lib.ROUTE_TILED and r.plan.kernel in (_lib.KERNEL_TILED, _lib.KERNEL_TILED_DECODE)
+    # without the tiled copy: decode sizes of an activation-order layer on the sorted copy, the rest on the checkpoint
+    no_tiled = _lib.COPY_CHECKPOINT | _lib.COPY_SORTED
+    assert _lib.select_route(1, K, N, 3, 128, True, copies=no_tiled).copy == _lib.ROUTE_SORTED
+    assert _lib.select_route(1, K, N, 3, 128, False, copies=no_tiled).copy == _lib.ROUTE_CHECKPOINT
+    assert _lib.select_route(64, K, N, 3, 128, True, copies=no_tiled).copy == _lib.ROUTE_CHECKPOINT
+    assert _lib.select_route(1, K, N, 3, 128, True, copies=_lib.COPY_CHECKPOINT).copy == _lib.ROUTE_CHECKPOINT
+    # 2 and 8 bits: fused on the tiled copy only
+    assert _lib.select_route(1, K, N, 8, 128, True).copy == _lib.ROUTE_TILED
+    assert _lib.select_route(1, K, N, 8, 128, True, copies=no_tiled).copy == _lib.ROUTE_LIBRARY
+    # groups the tiled format does not cover stay off it
+    assert _lib.select_route(64, K, N, 4, 16, False).copy == _lib.ROUTE_CHECKPOINT
+    # switch rows: the caller's, 0 = never
+    assert _lib.select_route(128, K, N, 4, 128, True, switch_rows=(128, 128, 128)).copy == _lib.ROUTE_LIBRARY
+    assert _lib.select_route(127, K, N, 4, 128, True, switch_rows=(128, 128, 128)).copy == _lib.ROUTE_TILED
+    assert _lib.select_route(100000, K, N, 4, 128, True, switch_rows=(0, 0, 0)).copy == _lib.ROUTE_TILED
+    # more activation-order groups than any fused kernel on the checkpoint layout takes
+    assert _lib.select_route(4, 36864, 9216, 4, 32, True, copies=_lib.COPY_CHECKPOINT).copy == _lib.ROUTE_LIBRARY
+    with pytest.raises(_lib.GptqHipError):
+        _lib.select_route(1, K, N, 4, 128, True, copies=0)
+    with pytest.raises(_lib.GptqHipError):
+        _lib.select_route(1, K, N, 5, 128, True)
+    with pytest.raises(_lib.GptqHipError):
+        _lib.select_route(0, K, N, 4, 128, True)
+
+
+def test_plans_that_need_a_private_zero_workspace_say_so():
+    # halved tiles of the decode kernel meet in slots of the workspace: the plan carries the flag, others do not
+    p = _lib.select_tiled(1, 4096, 11008, 3, 128)
+    assert p.kernel == _lib.KERNEL_TILED_DECODE and p.grid_x > 11008 // 32
+    assert p.flags & _lib.PLAN_PRIVATE_ZERO_WORKSPACE and p.workspace_bytes > 0
+    for q in (_lib.select_tiled(1, 4096, 4096, 4, 128), _lib.select_tiled(128, 4096, 11008, 4, 128),
+              _lib.select(1, 4096, 11008, 3, 128, True), _lib.select(64, 4096, 11008, 4, 128, True)):
+        assert q.flags == 0
+    assert ctypes.sizeof(_lib.Route) == 8 + ctypes.sizeof(_lib.Plan)

@@ -134,7 +134,7 @@ def test_fused_model_matches_the_unfused_one(tmp_path):
     from autogptq.tvm_amd.loader import from_quantized
 
     cfg, _, _ = build_checkpoint(str(tmp_path), bits=4, gs=32, act_order=True, seed=4, shared_order=True)
-    plain, _ = from_quantized(str(tmp_path), device="cuda:0")
+    plain, _ = from_quantized(str(tmp_path), device="cuda:0", keep_checkpoint_tensors=True)
     merged, _ = from_quantized(str(tmp_path), device="cuda:0", fuse_shared_inputs=True, prepare_decode=True)
     assert isinstance(merged.model.layers[0].self_attn.k_proj, fused.FusedMember)
     assert merged.model.layers[0].mlp.down_proj._sorted is not None       # prepared at load
@@ -152,15 +152,17 @@ def test_fused_model_matches_the_unfused_one(tmp_path):
 @pytest.mark.gpu
 @pytest.mark.parametrize("fuse", [False, True])
 def test_compact_model_matches_the_plain_one(tmp_path, fuse):
-    """from_quantized(compact=True): every layer keeps the tiled copy as its only weights (checkpoint tensors
-    released, fused projections included) and the model gives the same logits for a prompt and for one token."""
+    """from_quantized as it loads by default: every layer keeps the tiled copy as its only weights (checkpoint
+    tensors released, fused projections included) and the model gives the same logits for a prompt and for one
+    token as the one that kept the checkpoint tensors."""
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     from autogptq.tvm_amd.loader import from_quantized
 
     cfg, _, _ = build_checkpoint(str(tmp_path), bits=4, gs=32, act_order=True, seed=6, shared_order=True)
-    plain, _ = from_quantized(str(tmp_path), device="cuda:0")
-    compact, _ = from_quantized(str(tmp_path), device="cuda:0", fuse_shared_inputs=fuse, compact=True)
+    plain, _ = from_quantized(str(tmp_path), device="cuda:0", keep_checkpoint_tensors=True)
+    assert not any(m._compact for m in plain.modules() if isinstance(m, QuantLinear))
+    compact, _ = from_quantized(str(tmp_path), device="cuda:0", fuse_shared_inputs=fuse)
     quant = [m for m in compact.modules() if isinstance(m, QuantLinear)]
     assert quant and all(m._compact and m.qweight.numel() == 0 and m.route(1) == "tiled" for m in quant)
     ids = torch.randint(0, cfg.vocab_size, (2, 9), generator=torch.Generator().manual_seed(7)).to("cuda:0")

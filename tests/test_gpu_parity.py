@@ -123,21 +123,6 @@ def test_gemm_integer_exact(dev, bits):
 
 
 @pytest.mark.parametrize("bits", [3, 4])
-@pytest.mark.parametrize("split", [1, 2, 3, 7])
-@pytest.mark.parametrize("M", [1, 20])
-@pytest.mark.parametrize("waves", [1, 2, 4])
-def test_gather_forced_split_k(dev, bits, split, M, waves):
-    K, N = 2048, 320
-    L = layer(500 + split, K, N, bits, 128, True, M=M, bias=True)
-    D = to_dev(L, dev)
-    plan = _lib.plan_for(_lib.KERNEL_GATHER, M, K, N, bits, 128, True, split_k=split, waves_n=waves)
-    y1 = run_gemm(D, plan=plan)
-    y2 = run_gemm(D, plan=plan)  # same workspace again: counters must have been left at zero
-    assert_close(y1, expected_output(L), f"split={split}")
-    assert torch.equal(y1, y2), "split-K result changed between two identical calls"
-
-
-@pytest.mark.parametrize("bits", [3, 4])
 @pytest.mark.parametrize("desc_act", [False, True])
 @pytest.mark.parametrize("waves,split", [(1, 1), (2, 1), (4, 1), (8, 1), (1, 3), (4, 2), (8, 2)])
 @pytest.mark.parametrize("M", [3, 20, 40, 130])
@@ -157,18 +142,20 @@ def test_stream_forced_waves_and_split_k(dev, bits, desc_act, waves, split, M):
 
 
 @pytest.mark.parametrize("bits", [3, 4])
-@pytest.mark.parametrize("K,N,gs", [(32, 32, 32), (160, 96, -1), (1024, 416, 32), (2048, 1056, 256), (1056, 64, 16)])
-@pytest.mark.parametrize("M", [3, 33])
-def test_stream_matches_gather(dev, bits, K, N, gs, M):
-    # two independent kernels, same exact fp16 weights: they may differ only in summation order
+@pytest.mark.parametrize("K,N,gs", [(32, 32, 32), (160, 96, -1), (1024, 416, 32), (2048, 1056, 256), (4096, 64, 64)])
+@pytest.mark.parametrize("M", [5, 33])
+def test_stream_matches_the_tiled_matmul(dev, bits, K, N, gs, M):
+    # two independent kernels on two layouts, same exact fp16 weights: they may differ only in summation order
     for desc_act in (False, True):
         L = layer(800 + M, K, N, bits, gs, desc_act, M=M)
         D = to_dev(L, dev)
         a = run_gemm(D, plan=_lib.plan_for(_lib.KERNEL_STREAM, M, K, N, bits, gs, desc_act))
-        b = run_gemm(D, plan=_lib.plan_for(_lib.KERNEL_GATHER, M, K, N, bits, gs, desc_act))
+        qtile, sz, xsrc, kinv = ops.tile_prepare(D["qweight"], D["qzeros"], D["scales"],
+                                                 D["g_idx"] if desc_act else None, bits, gs)
+        b = ops.gemm_tiled(D["x"], qtile, sz, xsrc if desc_act else None, kinv if desc_act else None, None, bits, gs)
         assert_close(a, expected_output(L), "stream")
-        assert_close(b, expected_output(L), "gather")
-        assert_close(a, b.float().cpu(), "stream vs gather")
+        assert_close(b, expected_output(L), "tiled")
+        assert_tight(a, b.float().cpu(), "stream vs tiled")
 
 
 @pytest.mark.parametrize("bits", [3, 4])
@@ -264,8 +251,8 @@ def test_grouped_wide_workgroups(dev, bits, desc_act, M, N, wn):
 @pytest.mark.parametrize("bits", [3, 4])
 @pytest.mark.parametrize("K,N,gs", [(96, 32, 32), (1024, 416, 32), (2048, 1056, 256), (11008, 256, 128), (4096, 64, 64)])
 @pytest.mark.parametrize("M", [1, 2])
-def test_grouped_matches_gather(dev, bits, K, N, gs, M):
-    """The two kernel families on the same inputs: GATHER forms the reference's rounded fp16
+def test_grouped_matches_stream(dev, bits, K, N, gs, M):
+    """The two kernel families on the same inputs: STREAM forms the reference's rounded fp16
     weights, GROUPED applies scales per group; they must agree far inside the tolerance."""
     for desc_act in (False, True):
         L = layer(700 + K, K, N, bits, gs, desc_act, M=M)
@@ -275,12 +262,12 @@ def test_grouped_matches_gather(dev, bits, K, N, gs, M):
         except _lib.GptqHipError:
             continue
         a = run_gemm(D, plan=pg)
-        b = run_gemm(D, plan=_lib.plan_for(_lib.KERNEL_GATHER, M, K, N, bits, gs, desc_act))
+        b = run_gemm(D, plan=_lib.plan_for(_lib.KERNEL_STREAM, M, K, N, bits, gs, desc_act))
         want = expected_output(L)
         assert_close(a, want, "grouped")
-        assert_close(b, want, "gather")
+        assert_close(b, want, "stream")
         assert_tight(a, want, "grouped")
-        assert_tight(b, want, "gather")
+        assert_tight(b, want, "stream")
 
 
 def test_gemm_does_not_write_outside_y(dev):
@@ -528,7 +515,7 @@ def test_sorted_decode_integer_exact_and_rejections(dev):
     qs, kmap = pack.sort_channels_by_group(D["qweight"], D["g_idx"], bits, gs)
     with pytest.raises(_lib.GptqHipError) as e:
         ops.gemm_sorted(D["x"], qs, D["qzeros"], D["scales"], kmap, None, bits, gs,
-                        plan=_lib.plan_for(_lib.KERNEL_GATHER, 1, K, N, bits, gs, False))
+                        plan=_lib.select_tiled(1, K, N, bits, gs))
     assert e.value.status == _lib.ERR_UNSUPPORTED
     shifted = torch.zeros(2 * K + 1, dtype=torch.int32, device=dev)[1:]
     shifted.copy_(kmap)

@@ -133,8 +133,9 @@ def test_from_quantized_reports_missing_files_and_tensors(tmp_path):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("keep", [False, True])
 @pytest.mark.parametrize("bits,act_order", [(4, True), (3, True), (4, False), (8, True), (2, False)])
-def test_loaded_model_matches_the_dequantised_float_model(tmp_path, bits, act_order):
+def test_loaded_model_matches_the_dequantised_float_model(tmp_path, bits, act_order, keep):
     """End to end: logits of the loaded quantised model on the GPU against the same architecture
     with every quantised layer replaced by a float Linear holding the oracle's dequantised weight."""
     if not torch.cuda.is_available():
@@ -144,7 +145,8 @@ def test_loaded_model_matches_the_dequantised_float_model(tmp_path, bits, act_or
     from oracle import gptq_oracle as orc
 
     cfg, state, dense = build_checkpoint(str(tmp_path), bits=bits, gs=32, act_order=act_order, seed=3)
-    model, _ = from_quantized(str(tmp_path), device="cuda:0")
+    model, _ = from_quantized(str(tmp_path), device="cuda:0", keep_checkpoint_tensors=keep)
+    assert all(m._compact != keep for m in model.modules() if isinstance(m, QuantLinear))
     ref = AutoModelForCausalLM.from_config(cfg).float()
     ref_state = {}
     for k, v in state.items():
@@ -164,3 +166,42 @@ def test_loaded_model_matches_the_dequantised_float_model(tmp_path, bits, act_or
     # fp16 activations through two decoder layers against an fp32 model
     assert float((got - want).abs().max()) <= 2e-2 + 2e-2 * float(want.abs().max())
     assert np.isfinite(got.numpy()).all()
+
+
+def layer_device_bytes(q):
+    """Bytes of device memory a QuantLinear holds: its buffers and whatever prepared copies it keeps."""
+    seen, total = set(), 0
+    held = [q.qweight, q.qzeros, q.scales, q.g_idx, q.bias]
+    for slot in (q._sorted, q._tiled, q._tiled_t):
+        if slot is not None and slot[1] is not None:
+            held += list(slot[1])
+    for t in held:
+        if t is None or t.device.type != "cuda" or t.data_ptr() in seen:
+            continue
+        seen.add(t.data_ptr())
+        total += t.numel() * t.element_size()
+    return total
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits,act_order", [(4, True), (3, True), (4, False)])
+def test_loaded_layers_hold_one_copy_of_their_weights(tmp_path, bits, act_order):
+    """After from_quantized and calls with 1, 8 and 128 rows, a layer holds its packed size and the small tables
+    (scale / zero words, channel maps), not a second or third copy; nothing is allocated for it by the calls."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    build_checkpoint(str(tmp_path), bits=bits, gs=32, act_order=act_order, seed=8)
+    model, _ = from_quantized(str(tmp_path), device="cuda:0")
+    layers = {n: m for n, m in model.named_modules() if isinstance(m, QuantLinear)}
+    assert layers
+    before = {n: layer_device_bytes(m) for n, m in layers.items()}
+    for rows in (1, 8, 128):
+        for m in layers.values():
+            m(torch.randn(rows, m.infeatures, dtype=torch.float16, device="cuda:0"))
+    torch.cuda.synchronize()
+    for n, m in layers.items():
+        K, N, G = m.infeatures, m.outfeatures, m.infeatures // m.groupsize
+        packed = K * N * bits // 8
+        tables = G * N * 4 + 6 * K + (2 * N if m.bias is not None else 0) + 4 * K   # sz, xsrc + kinv, bias, g_idx
+        assert layer_device_bytes(m) == before[n], n
+        assert before[n] <= 1.05 * packed + tables, (n, before[n], packed, tables)

@@ -74,3 +74,52 @@ def test_torch_ops_are_registered_without_a_cpu_kernel():
     assert tuple(w.shape) == (64, 96) and w.dtype == torch.float16
     with pytest.raises((NotImplementedError, RuntimeError)):   # no CPU fallback, not even in the dispatcher
         torch.ops.gptq_hip.gemm(x, q.qweight, q.qzeros, q.scales, None, None, 4, 32)
+
+
+def test_copies_and_pickles_drop_the_routes():
+    """A route holds bound launch objects and closures over the module's tensors; copy.deepcopy, pickle and
+    torch.save of a module that has served calls must work (the reference's module is a plain one that does) and
+    the copy decides its routes again instead of computing on the original's tensors."""
+    import copy
+    import io
+    import pickle
+    import threading
+
+    q = QuantLinear(4, 32, 64, 32, True)
+    q.qweight.random_(0, 1 << 20)
+    # what a served call leaves behind: the watched buffers, their versions, the path, a callable that cannot be copied
+    lock = threading.Lock()
+    q._g_state = (("stale",), True)      # (any attribute assignment empties the routes: set this first)
+    q._routes[1] = (q._watched(), sum(t._version for t in q._watched()), "plain", lambda x, lock=lock: x)
+    for clone in (copy.deepcopy(q), pickle.loads(pickle.dumps(q))):
+        assert clone._routes == {} and clone._g_state is None and clone._sorted is None and clone._tiled is None
+        assert torch.equal(clone.qweight, q.qweight) and clone.qweight.data_ptr() != q.qweight.data_ptr()
+        assert (clone.bits, clone.groupsize, clone.infeatures, clone.outfeatures) == (4, 32, 64, 32)
+    buf = io.BytesIO()
+    torch.save(torch.nn.Sequential(q), buf)
+    assert q._routes                      # the original keeps its routes
+    # replacing a buffer behind __setattr__'s back (what offload hooks do) makes a cached route stale
+    r = q._routes[1]
+    assert q._fresh(r)
+    q._buffers["qweight"] = q.qweight.clone()
+    assert not q._fresh(r)
+
+
+def test_find_layers_matches_the_reference_helper_on_a_nested_model():
+    """auto_gptq/modeling/_utils.py:38-49: names are dotted paths, depth first in registration order; a module
+    that is itself a layer comes back under the given name."""
+    from autogptq.tvm_amd.loader import find_layers
+
+    net = torch.nn.Sequential()
+    net.add_module("a", torch.nn.Linear(4, 4))
+    inner = torch.nn.Module()
+    inner.proj = torch.nn.Linear(4, 4)
+    inner.act = torch.nn.ReLU()
+    inner.conv = torch.nn.Conv2d(1, 1, 1)
+    net.add_module("blk", inner)
+    net.add_module("z", torch.nn.LayerNorm(4))
+    found = find_layers(net)
+    assert list(found) == ["a", "blk.proj", "blk.conv"] and found["blk.proj"] is inner.proj
+    assert list(find_layers(net, [torch.nn.LayerNorm])) == ["z"]
+    assert list(find_layers(inner.proj, name="model.q")) == ["model.q"]
+    assert find_layers(torch.nn.ReLU()) == {}

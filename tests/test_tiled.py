@@ -486,7 +486,7 @@ def test_quantlinear_routes_prompt_sizes_to_the_tiled_copy(dev, bits, desc_act):
     L3 = layer(1820, 256, 64, 4, 16, False, M=40)
     q3 = module_of(L3, dev)
     assert_close(q3(L3["x"].to(dev)), expected_output(L3), "module, uncovered by the format")
-    assert q3._tiled is not None and q3._tiled[1] is None and not q3.compact()
+    assert q3.route(40) == "plain" and not q3.compact() and q3._tiled[1] is None
 
 
 @pytest.mark.parametrize("bits", [2, 8])
@@ -531,9 +531,15 @@ def test_quantlinear_compact_keeps_one_copy(dev, bits, desc_act):
     assert torch.equal(q.dequantize().cpu().view(torch.int16), expected_weight(L).view(torch.int16))
     q = q.to(dev)                                  # moving the module keeps the copy
     assert_close(q(x[:40]), want[:40], "compact module after .to()")
-    # the gradient for x still works (adapters on top of frozen layers)
+    # a gradient for x needs the copy for it, made before the checkpoint tensors went: without one the layer says so
+    # instead of forming W through a K-row product
     xg = x[:4].clone().requires_grad_(True)
-    q(xg).float().sum().backward()
+    with pytest.raises(RuntimeError, match="prepare_transposed"):
+        q(xg).float().sum().backward()
+    q2 = module_of(L, dev)
+    assert q2.prepare_transposed() is not None and q2.compact()
+    xg = x[:4].clone().requires_grad_(True)
+    q2(xg).float().sum().backward()               # (adapters on top of frozen layers)
     assert xg.grad is not None and xg.grad.shape == xg.shape
 
 
@@ -555,3 +561,51 @@ def test_long_prompts_run_fused_on_the_tiled_kernels(dev, bits):
     assert q.route(1024) == "library" and q.route(1023) == "tiled"
     assert q.compact() and q.route(4096) == "tiled"
     assert_tight(q(x), want, "compact module, 4096 rows")
+
+
+@pytest.mark.parametrize("compact", [False, True])
+def test_quantlinear_copies_after_it_has_served_calls(dev, compact):
+    """copy.deepcopy and pickle of a module whose routes are populated (bound C++ launch objects, closures over its
+    tensors): the copy has its own tensors, decides its routes again and gives the same numbers."""
+    import copy
+    import pickle
+
+    K, N, gs = 1024, 416, 128
+    L = layer(1900, K, N, 4, gs, True, M=40, bias=True)
+    q = module_of(L, dev)
+    if compact:
+        assert q.compact()
+    x = L["x"].to(dev)
+    y1, y40 = q(x[:1]), q(x)
+    assert q._routes
+    for clone in (copy.deepcopy(q), pickle.loads(pickle.dumps(q))):
+        assert clone._routes == {} and clone._compact == compact
+        if compact:
+            assert clone._tiled[1][0].data_ptr() != q._tiled[1][0].data_ptr()
+        else:
+            assert clone.qweight.data_ptr() != q.qweight.data_ptr()
+        assert torch.equal(clone(x[:1]), y1) and torch.equal(clone(x), y40)
+        # the copy computes on its own weights: changing the original's does not reach it
+        if not compact:
+            q.qweight.zero_()
+            assert torch.equal(clone(x), y40)
+            q.load_state_dict({k: L[k] for k in ("qweight", "qzeros", "scales", "g_idx", "bias")})
+            q.to(dev)
+
+
+@pytest.mark.parametrize("bits,K,N,gs,desc_act", [(4, 1024, 416, 128, True), (3, 4096, 4096, 128, False),
+                                                   (4, 2048, 8224, 128, True), (3, 1024, 160, -1, True)])
+def test_quantlinear_takes_the_route_the_library_names(dev, bits, K, N, gs, desc_act):
+    """QuantLinear asks gptq_hip_select_route which copy a call runs on; the path it reports is that answer."""
+    L = layer(1910 + bits, K, N, bits, gs, desc_act, M=1)
+    q = module_of(L, dev)
+    for M in (1, 2, 4, 8, 16, 17, 64, 128, 300, 700, 1100, 1200):
+        r = _lib.select_route(M, K, N, bits, gs, desc_act and gs != -1)
+        assert q.route(M) == _lib.ROUTE_NAMES[r.copy], (M, q.route(M), r.copy)
+    # swapping a buffer behind the module's back (what offload hooks do) makes it decide again, on the new tensor
+    x = torch.randn(3, K, dtype=torch.float16, device=dev)
+    before = q(x)
+    q._buffers["qweight"] = torch.zeros_like(q.qweight)
+    q._g_state = None
+    after = q(x)
+    assert not torch.equal(before, after)
