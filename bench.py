@@ -2,24 +2,33 @@
 """Benchmark of the GPTQ QuantLinear hot path on one MI355X.
 
 Default workload: the headline configuration of the reference's benchmarks -- 3-bit GEMV, M=1, K=4096, N=11008, group_size=128,
-desc_act=True (g_idx from a random permutation), synthetic seeded tensors.  One "step" is one
-call of the C-ABI entry point that ``QuantLinear.forward`` makes for that shape, on tensors already
-resident in HBM: ``gptq_hip_gemm_sorted`` for decode sizes on activation-order layers (the layer
-as the module holds it after its one-time load preparation, the channel sort),
-``gptq_hip_gemm_tiled`` where the module routes to its copy in the tiled format (prompt sizes; decode
-sizes of layers up to 8192 columns wide), ``gptq_hip_gemm`` otherwise; ``--unprepared`` times
-``gptq_hip_gemm`` on the checkpoint's own tensors instead, and the default run reports that figure
-too under ``timing.unprepared_us``.  Steps rotate
-over enough distinct weight copies to exceed twice the 256 MB Infinity Cache, so every step
-streams its packed weights from HBM (cache-cold).
+desc_act=True (g_idx from a random permutation), synthetic seeded tensors.  One "step" is one call of the C-ABI
+entry point that ``gptq_hip_select_route`` names for the shape (the decision ``QuantLinear.forward`` follows), on
+tensors already resident in HBM: ``gptq_hip_gemm_tiled`` on the layer's copy in the tiled format,
+``gptq_hip_gemm_sorted`` on its channel-sorted copy, or ``gptq_hip_gemm_plan`` on the checkpoint's own tensors
+(``--prepared`` forces a copy; the default run reports the checkpoint-tensor figure too, under
+``timing.unprepared_us``).  Steps rotate over enough distinct weight copies to exceed twice the 256 MB Infinity
+Cache, so every step streams its packed weights from HBM (cache-cold).
 
-Prints ONE JSON line (see the keys below).  ``roofline.achieved`` is algorithmic bytes (packed
-qweight only, K*N*bits/8) or flops (2*M*K*N) per launch divided by the average launch duration
-measured here with HIP events on the launch stream.  ``cpu_baseline`` times the CPU oracle (the
-restatement of the reference's torch path) on this box's host cores.
+Timing: K steps, and 2 K steps, are captured once each into a HIP graph and replayed inside an event-bracketed
+region that sits behind a read of 512 MB (cache scrub), the W warm-up steps and max(K, 256) more untimed steps (a
+graph of its own), all queued back to back.  A replay carries a fixed ~10 us of start-up on the GPU whatever sits in
+front of it (t(K) = 9.6 us + 6.80 us * K fitted K = 5 ... 1000 on the headline), which at K = 20 would read as
+0.5 us per step; a decode loop replays hundreds of kernels per graph, so the figure reported is the time of K
+steps with that constant taken out: t(2 K) - t(K).  Five regions of each; ``value`` is the median of the
+differences, ``timing.min_us`` their minimum, ``timing.region_us`` the plain t(K) / K and
+``timing.replay_overhead_us`` the constant, 2 t(K) - t(2 K).
 
-Other workloads: ``--workload NAME`` (see WORKLOADS), ``--sweep`` adds a table of all of them
-under "sweep" in the same JSON line.
+Prints ONE JSON line (see the keys below).  ``roofline.achieved`` is algorithmic bytes (packed qweight only,
+K*N*bits/8) or flops (2*M*K*N) per launch divided by the median step time measured here with HIP events on the
+launch stream.  ``secondary`` holds one record like it for every other point of the configurations the metric is
+quoted on (configs[0], the 4-bit twin of the headline, the decode sweep, the prefill sweep, the one-group 3-bit
+layers), each with its own roofline and parity check.  ``cpu_baseline`` times the CPU oracle (the restatement of
+the reference's torch path) on this box's host cores: all cores, one core, and the matmul alone on a
+pre-dequantised weight.
+
+Other workloads: ``--workload NAME`` (see WORKLOADS), ``--sweep`` adds a table of every workload on every copy
+of the layer under "sweep" in the same JSON line.
 """
 from __future__ import annotations
 
@@ -87,10 +96,25 @@ WORKLOADS = {
     "int8-4096x11008-act-m128": (8, 4096, 11008, 128, True, 128),
     "int2-4096x11008-act-m128": (2, 4096, 11008, 128, True, 128),
 }
+# every point of the configurations the metric is quoted on
+for _K, _N in ((4096, 4096), (4096, 11008), (11008, 4096)):
+    for _M in (1, 2, 4, 8):
+        WORKLOADS.setdefault(f"c3-int4-{_K}x{_N}-m{_M}", (4, _K, _N, 128, False, _M))
+for _K, _N in ((4096, 11008), (11008, 4096)):
+    for _b in (4, 3):
+        for _M in (16, 64, 128, 256):
+            WORKLOADS.setdefault(f"c4-int{_b}-{_K}x{_N}-act-m{_M}", (_b, _K, _N, 128, True, _M))
+for _K, _N in ((9216, 9216), (9216, 36864), (36864, 9216)):
+    for _M in (1, 32):
+        WORKLOADS.setdefault(f"c5-int3-{_K}x{_N}-g1-m{_M}", (3, _K, _N, -1, True, _M))
 DEFAULT_WORKLOAD = "c2-int3-4096x11008-act-m1"
-# timed in the default run next to the headline: the int4 decode product and the M = 128 products of the
-# same 4096 x 11008 activation-order layer (the metric is quoted on all of them)
-SECONDARY_WORKLOADS = ("int4-4096x11008-act-m1", "c4-int4-4096x11008-act-m128", "c4-int3-4096x11008-act-m128")
+# timed in the default run next to the headline, each as a record of its own: configs[0], the headline's 4-bit twin,
+# and every point of the decode sweep (configs[2]), the prefill sweep (configs[3]) and the one-group layers (configs[4])
+SECONDARY_WORKLOADS = tuple(
+    ["c1-int4-4096x4096-m1", "int4-4096x11008-act-m1"]
+    + [f"c3-int4-{k}x{n}-m{m}" for k, n in ((4096, 4096), (4096, 11008), (11008, 4096)) for m in (1, 2, 4, 8)]
+    + [f"c4-int{b}-{k}x{n}-act-m{m}" for k, n in ((4096, 11008), (11008, 4096)) for b in (4, 3) for m in (16, 64, 128, 256)]
+    + [f"c5-int3-{k}x{n}-g1-m{m}" for k, n in ((9216, 9216), (9216, 36864), (36864, 9216)) for m in (1, 32)])
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the same
 # counter reads for a plain 256 MiB device copy): profiles/traffic.json holds, per workload, the bytes, the
@@ -111,60 +135,123 @@ def measured_traffic(workload: str, plan_kernel: int):
     return int(e["fetch_bytes"]) + int(e["write_bytes"]), e.get("source")
 
 
-def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int = 0, prepared=None):
-    """prepared: the layer as QuantLinear holds it after its one-time preparation: "sorted" (channels of
-    an activation-order layer sorted by group, run through gptq_hip_gemm_sorted), "tiled" (the tiled
-    format, run through gptq_hip_gemm_tiled), or None (the checkpoint's tensors, gptq_hip_gemm);
-    prepared_mode(name) is the module's own choice."""
+class Layer:
+    """One synthetic layer (bits, K, N, group_size, desc_act) shared by every workload on it: the seeded tensors on
+    the CPU, the oracle's dequantised weight, and per copy format ("tiled", "sorted", None = the checkpoint's own
+    tensors) enough distinct weight copies on the device to exceed twice the Infinity Cache."""
+
+    def __init__(self, key, dev, max_rows: int):
+        from autogptq.tvm_amd.pack import synth_layer
+
+        self.key = key
+        bits, K, N, gs, desc_act = key
+        self.dev = dev
+        self.L = synth_layer(2000 + (bits * 131 + K * 7 + N * 3 + (1 if desc_act else 0) + (gs & 0xff)) % 9973, K, N, bits,
+                             gs, desc_act, M=max_rows)
+        self.rows = max_rows
+        self.wbytes = K * N * bits // 8
+        self.copies = max(2, -(-2 * INFINITY_CACHE_BYTES // self.wbytes), int(os.environ.get("GPTQ_BENCH_MIN_COPIES", "0")))
+        self.qzeros, self.scales = self.L["qzeros"].to(dev), self.L["scales"].to(dev)
+        self.g_idx = self.L["g_idx"].to(dev) if desc_act else None
+        self.x = self.L["x"].to(dev)
+        self._fmt = {}
+        self._want = None
+
+    def raw_copy(self, c: int):
+        """Copy 0 is the seeded layer; the others are distinct random packed words (every int32 pattern is a valid
+        block of codes), drawn on the device."""
+        if c == 0:
+            return self.L["qweight"].to(self.dev)
+        gen = torch.Generator(device=self.dev).manual_seed(99 + c)
+        return torch.randint(-(1 << 31), (1 << 31) - 1, tuple(self.L["qweight"].shape), generator=gen, dtype=torch.int64,
+                             device=self.dev).to(torch.int32)
+
+    def fmt(self, prepared):
+        """{"qweights": [...], "aux": [per copy tuple], "kmap": ...} for a copy format, built once."""
+        from autogptq.tvm_amd import ops
+        from autogptq.tvm_amd.pack import sort_channels_by_group
+
+        if prepared in self._fmt:
+            return self._fmt[prepared]
+        bits, K, N, gs, desc_act = self.key
+        out = {"qweights": [], "aux": [], "kmap": None}
+        for c in range(self.copies):
+            q = self.raw_copy(c)
+            if prepared == "tiled":
+                # (every copy brings its own scale / zero words and channel maps, as every layer of a model does)
+                qtile, sz, xsrc, kinv = ops.tile_prepare(q, self.qzeros, self.scales, self.g_idx, bits, gs)
+                out["aux"].append((sz, xsrc if desc_act else None, kinv if desc_act else None))
+                q = qtile
+            out["qweights"].append(q)
+        if prepared == "sorted":
+            out["qweights"][0], out["kmap"] = sort_channels_by_group(out["qweights"][0], self.g_idx, bits, gs)
+        if prepared != "tiled":
+            # the layer's other tensors, one set per copy as well (qzeros, scales, and g_idx or the sorted copy's map)
+            g_or_map = out["kmap"] if out["kmap"] is not None else self.g_idx
+            out["aux"] = [(self.qzeros, self.scales, g_or_map)] + [
+                (self.qzeros.clone(), self.scales.clone(), g_or_map.clone() if g_or_map is not None else None)
+                for _ in range(self.copies - 1)]
+        self._fmt[prepared] = out
+        return out
+
+    def drop(self, prepared):
+        self._fmt.pop(prepared, None)
+        torch.cuda.empty_cache()
+
+    def want(self):
+        """x @ W in fp32 on the oracle's dequantised weight, for all rows of x."""
+        from oracle import c_oracle
+
+        if self._want is None:
+            L = self.L
+            w16 = torch.from_numpy(c_oracle.dequant(L["qweight"].numpy(), L["qzeros"].numpy(), L["scales"].numpy(),
+                                                    L["g_idx"].numpy(), self.key[0]).copy())
+            self._want = L["x"].float() @ w16.float()
+        return self._want
+
+
+_layers = {}
+
+
+def layer_of(name: str, dev, max_rows: int = 0) -> Layer:
+    """The layer of a workload, kept for the other workloads on it (one layer at a time: a new one frees the last)."""
+    bits, K, N, gs, desc_act, M = WORKLOADS[name]
+    key = (bits, K, N, gs, desc_act)
+    rows = max(M, max_rows)
+    lay = _layers.get(key)
+    if lay is None or lay.rows < rows:
+        _layers.clear()
+        torch.cuda.empty_cache()
+        lay = _layers[key] = Layer(key, dev, rows)
+    return lay
+
+
+def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int = 0, prepared=None, max_rows: int = 0):
+    """prepared: the copy of the layer the step runs on: "sorted" (channels of an activation-order layer sorted by
+    group, gptq_hip_gemm_sorted), "tiled" (the tiled format, gptq_hip_gemm_tiled), or None (the checkpoint's
+    tensors, gptq_hip_gemm_plan); prepared_mode(name) is the library's own choice."""
     from autogptq.tvm_amd import _lib, ops
-    from autogptq.tvm_amd.pack import sort_channels_by_group, synth_layer
 
     bits, K, N, gs, desc_act, M = WORKLOADS[name]
-    L = synth_layer(2000 + sorted(WORKLOADS).index(name), K, N, bits, gs, desc_act, M=M)
-    wbytes = K * N * bits // 8
-    copies = max(2, -(-2 * INFINITY_CACHE_BYTES // wbytes))
-    gen = torch.Generator().manual_seed(99)
+    lay = layer_of(name, dev, max_rows)
+    f = lay.fmt(prepared)
     case = {
-        "name": name, "bits": bits, "K": K, "N": N, "gs": gs, "desc_act": desc_act, "M": M, "L": L,
-        "qzeros": L["qzeros"].to(dev), "scales": L["scales"].to(dev),
-        "g_idx": L["g_idx"].to(dev) if desc_act else None,
-        "x": L["x"].to(dev), "y": torch.empty((M, N), dtype=torch.float16, device=dev),
-        "wbytes": wbytes, "flops": 2 * M * K * N, "kmap": None, "tiled": None, "prepared": prepared,
+        "name": name, "bits": bits, "K": K, "N": N, "gs": gs, "desc_act": desc_act, "M": M, "layer": lay,
+        "x": lay.x[:M], "y": torch.empty((M, N), dtype=torch.float16, device=dev),
+        "wbytes": lay.wbytes, "flops": 2 * M * K * N, "kmap": f["kmap"], "prepared": prepared,
+        "qweights": f["qweights"], "aux": f["aux"],
     }
-    qweights = []
-    for c in range(copies):
-        # copy 0 is the seeded layer; the others are distinct random packed words (every int32 pattern is a
-        # valid block of codes)
-        q = L["qweight"].to(dev) if c == 0 else torch.randint(
-            -(1 << 31), (1 << 31) - 1, L["qweight"].shape, generator=gen, dtype=torch.int64).to(torch.int32).to(dev)
-        if prepared == "tiled":
-            # (every copy brings its own scale / zero words and channel maps, as every layer of a model does)
-            qtile, sz, xsrc, kinv = ops.tile_prepare(q, case["qzeros"], case["scales"], case["g_idx"], bits, gs)
-            case.setdefault("tiled_copies", []).append((sz, xsrc if desc_act else None, kinv if desc_act else None))
-            if c == 0:
-                case["tiled"] = case["tiled_copies"][0]
-            q = qtile
-        qweights.append(q)
-    case["qweights"] = qweights
-    if prepared == "sorted":
-        qweights[0], case["kmap"] = sort_channels_by_group(qweights[0], case["g_idx"], bits, gs)
-        case["g_idx"] = None
-        desc_act = False  # the plan is that of contiguous groups
-    # the layer's other tensors, one set per copy as well (qzeros, scales, and g_idx or the sorted copy's map)
-    g_or_map = case["kmap"] if case["kmap"] is not None else case["g_idx"]
-    case["aux_copies"] = [(case["qzeros"], case["scales"], g_or_map)] + [
-        (case["qzeros"].clone(), case["scales"].clone(), g_or_map.clone() if g_or_map is not None else None)
-        for _ in range(copies - 1)]
+    act = desc_act and prepared != "sorted"   # the sorted copy is planned like contiguous groups
     if prepared == "tiled":
         plan = _lib.select_tiled(M, K, N, bits, gs)
     elif prepared == "sorted" and not (kernel or split_k or waves_n):
         plan = ops.sorted_plan(M, K, N, bits, gs)
     elif kernel or split_k or waves_n:
         if not kernel:
-            kernel = _lib.select(M, K, N, bits, gs, desc_act).kernel
-        plan = _lib.plan_for(kernel, M, K, N, bits, gs, desc_act, split_k, waves_n)
+            kernel = _lib.select(M, K, N, bits, gs, act).kernel
+        plan = _lib.plan_for(kernel, M, K, N, bits, gs, act, split_k, waves_n)
     else:
-        plan = _lib.select(M, K, N, bits, gs, desc_act)
+        plan = _lib.select(M, K, N, bits, gs, act)
     case["plan"] = plan
     ws_bytes = plan.workspace_bytes
     if prepared == "sorted":   # kernels that want x in the sorted order find it behind the plan's own bytes
@@ -204,15 +291,13 @@ def tiled_applies(name: str) -> bool:
 
 
 def prepared_mode(name: str):
-    """The prepared copy QuantLinear.forward uses for this workload (qlinear.py: _product), or None."""
-    from autogptq.tvm_amd import ops
+    """The copy of the layer gptq_hip_select_route names for this workload when all three are on offer (the
+    decision QuantLinear.forward follows), or None for the checkpoint's own tensors."""
+    from autogptq.tvm_amd import _lib
 
     bits, K, N, gs, desc_act, M = WORKLOADS[name]
-    one_group = gs == -1 or gs >= K
-    if tiled_applies(name) and (not plain_applies(name) or ops.tiled_wins(M, K, N, desc_act and not one_group, bits,
-                                                                           one_group=one_group)):
-        return "tiled"
-    return "sorted" if sorted_applies(name) else None
+    r = _lib.select_route(M, K, N, bits, gs, desc_act, switch_rows=(0, 0, 0))
+    return {_lib.ROUTE_TILED: "tiled", _lib.ROUTE_SORTED: "sorted"}.get(r.copy)
 
 
 def make_step(case, dev):
@@ -229,7 +314,7 @@ def make_step(case, dev):
     planp = ctypes.byref(case["plan"])
     n = len(qws)
     if case["prepared"] == "tiled":
-        aux = [tuple(ptr(t) for t in c) for c in case["tiled_copies"]]
+        aux = [tuple(ptr(t) for t in c) for c in case["aux"]]
 
         def step(i, stream):
             sz, xsrc, kinv = aux[i % n]
@@ -239,7 +324,7 @@ def make_step(case, dev):
 
         return step
     fn = lib.gptq_hip_gemm_sorted if case["kmap"] is not None else lib.gptq_hip_gemm_plan
-    aux = [tuple(ptr(t) for t in c) for c in case["aux_copies"]]
+    aux = [tuple(ptr(t) for t in c) for c in case["aux"]]
 
     def step(i, stream):
         qz, sc, g = aux[i % n]
@@ -264,80 +349,94 @@ def scrub_cache(dev):
     _scrub[dev].sum()
 
 
-def time_case(case, dev, steps: int, warmup: int):
-    """Average duration of one step in microseconds: K steps captured once in a HIP graph and
-    replayed inside one event-bracketed region (no host launch cost between the kernels; reported as
-    ``graph_us`` and as ``us``), plus the same K steps launched eagerly (``eager_us``).  The W warm-up steps
-    run right in front of the timed ones, on the same stream with nothing in between, so that the K steps
-    start on a busy GPU (the first steps behind an idle or scrubbed GPU take ~2 us longer each: 5 steps
-    measure 8.8 us, steps 6 to 20 of 20 measure 7.0).  The weight copy of step i is (warmup + i) mod copies,
-    continuing the warm-up's rotation, and the cache is scrubbed before the warm-up of every timed region, so
-    no timed step finds its weights cached."""
+REGIONS = 5
+PRE_STEPS = 256   # untimed steps queued in front of the timed graph: enough GPU work (a millisecond and more) for the
+                  # host to have submitted the timed graph before the GPU gets to it
+
+
+def time_case(case, dev, steps: int, warmup: int, eager: bool = False):
+    """Duration of one step in microseconds.  K steps, and 2 K steps, are captured once each into a HIP graph and
+    replayed inside an event-bracketed region; in front of it, queued back to back on the same stream: a read of
+    512 MB (cache scrub), the W warm-up steps and max(K, PRE_STEPS) more untimed steps, each a graph of its own, so
+    that the timed steps start on a busy GPU (the first steps behind an idle or scrubbed GPU take ~2 us longer
+    each) and the host is far ahead of the GPU.  A replay still costs the GPU a fixed ~10 us at its start, which
+    would make the figure depend on K (20 steps: +0.5 us each); ``us`` is therefore the time of K steps with that
+    constant taken out, (t(2 K) - t(K)) / K: the median over REGIONS pairs of regions, ``min_us`` their minimum.
+    ``region_us`` = t(K) / K as it stands, ``replay_overhead_us`` = 2 t(K) - t(2 K).  The weight copy of step i is
+    i mod copies over warm-up, untimed and timed steps alike, and copies * bytes is at least twice the Infinity
+    Cache, so no timed step finds its weights cached.  ``eager_us`` (on request) = the same K steps launched one
+    by one."""
     step = make_step(case, dev)
     stream = torch.cuda.Stream(device=dev)
     res = {}
     with torch.cuda.stream(stream):
         sp = ctypes.c_void_p(stream.cuda_stream)
-        for i in range(warmup):       # (first calls: lazy initialisation of the runtime for these kernels)
+        for i in range(max(warmup, 2)):       # (first calls: lazy initialisation of the runtime for these kernels)
             step(i, sp)
         stream.synchronize()
-        # eager
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize(dev)
-        scrub_cache(dev)
-        for i in range(warmup):
-            step(i, sp)
-        e0.record(stream)
-        for i in range(steps):
-            step(warmup + i, sp)
-        e1.record(stream)
-        torch.cuda.synchronize(dev)
-        res["eager_us"] = e0.elapsed_time(e1) * 1e3 / steps
-    # graph replay
-    try:
-        g, g_warm = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
-        if warmup > 0:
-            with torch.cuda.graph(g_warm, stream=stream):
-                spg = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-                for i in range(warmup):
-                    step(i, spg)
-        with torch.cuda.graph(g, stream=stream):
-            spg = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-            for i in range(steps):
-                step(warmup + i, spg)
-        g.replay()
-        torch.cuda.synchronize(dev)
-        times = []
-        for _ in range(3):
+        if eager:
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize(dev)
-            # scrub, W warm-up steps, then the K timed steps, queued back to back
             scrub_cache(dev)
-            if warmup > 0:
+            for i in range(warmup):
+                step(i, sp)
+            e0.record(stream)
+            for i in range(steps):
+                step(warmup + i, sp)
+            e1.record(stream)
+            torch.cuda.synchronize(dev)
+            res["eager_us"] = e0.elapsed_time(e1) * 1e3 / steps
+    try:
+        graphs = []
+        pre = max(steps, PRE_STEPS)
+        for first, count in ((0, warmup), (warmup, pre), (warmup + pre, steps), (warmup + pre, 2 * steps)):
+            g = torch.cuda.CUDAGraph()
+            if count > 0:
+                with torch.cuda.graph(g, stream=stream):
+                    spg = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+                    for i in range(count):
+                        step(first + i, spg)
+            graphs.append(g if count > 0 else None)
+        g_warm, g_pre, g_k, g_2k = graphs
+        g_pre.replay()
+        g_k.replay()
+        g_2k.replay()
+        torch.cuda.synchronize(dev)
+
+        def region(g):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize(dev)
+            scrub_cache(dev)
+            if g_warm is not None:
                 g_warm.replay()
+            g_pre.replay()
             e0.record()
             g.replay()
             e1.record()
             torch.cuda.synchronize(dev)
-            times.append(e0.elapsed_time(e1) * 1e3 / steps)
-        res["graph_us"] = min(times)
+            return e0.elapsed_time(e1) * 1e3
+
+        t_k = [region(g_k) for _ in range(REGIONS)]
+        t_2k = [region(g_2k) for _ in range(REGIONS)]
+        slopes = sorted((b - a) / steps for a, b in zip(sorted(t_k), sorted(t_2k)))
+        res["graph_us"] = statistics.median(slopes)
+        res["min_us"] = slopes[0]
+        res["region_us"] = statistics.median(t_k) / steps              # one replay of K steps, its start-up included
+        res["replay_overhead_us"] = max(0.0, 2 * statistics.median(t_k) - statistics.median(t_2k))
     except Exception as exc:  # graph capture unavailable: report the eager figure only
         res["graph_error"] = repr(exc)[:200]
-    res["us"] = res.get("graph_us", res["eager_us"])
+        if "eager_us" not in res:
+            return time_case(case, dev, steps, warmup, eager=True) | {"graph_error": res["graph_error"]}
+    res["us"] = res.get("graph_us", res.get("eager_us"))
     return res
 
 
 def check_case(case, dev):
     """The timed path's output against the oracle, for the first weight copy."""
-    from oracle import c_oracle
-
     step = make_step(case, dev)
     step(0, ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
     torch.cuda.synchronize(dev)
-    L = case["L"]
-    w16 = torch.from_numpy(c_oracle.dequant(L["qweight"].numpy(), L["qzeros"].numpy(), L["scales"].numpy(),
-                                            L["g_idx"].numpy(), case["bits"]).copy())
-    want = L["x"].float() @ w16.float()
+    want = case["layer"].want()[:case["M"]]
     got = case["y"].float().cpu()
     err = (got - want).abs()
     ok = bool((err <= 1e-2 + 1e-2 * want.abs()).all())
@@ -347,7 +446,9 @@ def check_case(case, dev):
 def summarize(case, t):
     us = t["us"]
     out = {"workload": case["name"], "us": round(us, 3)}
-    out.update({k: (round(v, 3) if isinstance(v, float) else v) for k, v in t.items() if k != "us"})
+    out.update({k: (round(v, 3) if isinstance(v, float) else v) for k, v in t.items() if k not in ("us", "min_us")})
+    if "min_us" in t:
+        out["min_us"] = round(t["min_us"], 3)
     out["weight_GBps"] = round(case["wbytes"] / us * 1e-3, 1)
     out["hbm_frac"] = round(case["wbytes"] / us * 1e-3 / HBM_PEAK_GBS, 4)
     out["TFLOPs"] = round(case["flops"] / us * 1e-6, 2)
@@ -371,30 +472,49 @@ def roofline_of(name: str, s: dict) -> dict:
     return r
 
 
-def cpu_baseline(case, budget_s: float = 20.0):
-    """The reference's CPU path (oracle restatement of qlinear.py:198-245: unpack + gather + dequant
-    + fp16 matmul on every call) on this box's host cores."""
-    from oracle import gptq_oracle as orc
-
-    L = case["L"]
-    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1))
-    torch.set_num_threads(threads)
-    args = (L["x"], L["qweight"], L["qzeros"], L["scales"], L["g_idx"], None, case["bits"])
+def _timed_calls(fn, warmups: int, budget_s: float, most: int = 10):
+    for _ in range(warmups):
+        fn()
     t0 = time.perf_counter()
-    orc.forward_ref(*args)
+    fn()
     first = time.perf_counter() - t0
-    n = max(3, min(10, int(budget_s / max(first, 1e-3)) - 1))
-    ts = []
+    n = max(2, min(most - 1, int(budget_s / max(first, 1e-4)) - 1))
+    ts = [first]
     for _ in range(n):
         t0 = time.perf_counter()
-        orc.forward_ref(*args)
+        fn()
         ts.append(time.perf_counter() - t0)
-    med = statistics.median(ts)
+    return statistics.median(ts), len(ts)
+
+
+def cpu_baseline(case, budget_s: float = 10.0):
+    """The reference's CPU path (oracle restatement of qlinear.py:198-245: unpack + gather + dequant + fp16 matmul
+    on every call) on this box's host cores: with all of them, with one, and the matmul alone on a weight that was
+    dequantised beforehand (what remains of a call when the unpack and dequant steps are taken out)."""
+    from oracle import gptq_oracle as orc
+
+    L = case["layer"].L
+    M = case["M"]
+    x = L["x"][:M]
+    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1))
+    args = (x, L["qweight"], L["qzeros"], L["scales"], L["g_idx"], None, case["bits"])
+    torch.set_num_threads(threads)
+    med, n = _timed_calls(lambda: orc.forward_ref(*args), 3, budget_s)
+    w16 = orc.dequant_ref(L["qweight"], L["qzeros"], L["scales"], L["g_idx"], case["bits"])
+    mm, n_mm = _timed_calls(lambda: orc.matmul_only_ref(x, w16), 3, 2.0)
+    torch.set_num_threads(1)
+    one, n_one = _timed_calls(lambda: orc.forward_ref(*args), 1, budget_s, most=5)
+    torch.set_num_threads(threads)
     return {
         "value": round(med * 1e6, 1), "unit": "us", "cores": threads, "kind": "port",
-        "sample": f"median of {n} full calls after 1 warm-up of the torch CPU path on the same "
-                  f"{case['name']} tensors (unpack+gather+dequant+fp16 matmul per call)",
+        "sample": f"median of {n} full calls after 3 warm-ups of the torch CPU path on the same {case['name']} "
+                  f"tensors (unpack+gather+dequant+fp16 matmul per call), {threads} threads",
         "weight_GBps": round(case["wbytes"] / med * 1e-9, 3),
+        "single_thread": {"value": round(one * 1e6, 1), "unit": "us", "cores": 1,
+                          "sample": f"median of {n_one} full calls after 1 warm-up, torch.set_num_threads(1)"},
+        "matmul_only": {"value": round(mm * 1e6, 1), "unit": "us", "cores": threads,
+                        "sample": f"median of {n_mm} calls of x.half() @ W on the pre-dequantised fp16 weight "
+                                  f"after 3 warm-ups"},
     }
 
 
@@ -541,7 +661,7 @@ def main():
     case = build_case(args.workload, dev, args.kernel, args.split_k, args.waves_n, prepared=prepared)
     ok, max_err = check_case(case, dev)
     torch.cuda.synchronize(dev)
-    t = time_case(case, dev, args.steps, args.warmup)
+    t = time_case(case, dev, args.steps, args.warmup, eager=True)
     torch.cuda.synchronize(dev)
     s = summarize(case, t)
     if prepared and plain_applies(args.workload):
@@ -550,7 +670,7 @@ def main():
         s["unprepared_us"] = round(time_case(plain, dev, min(args.steps, 100), min(args.warmup, 10))["us"], 3)
         ok = ok and okp
         del plain
-        torch.cuda.empty_cache()
+        case["layer"].drop(None)
     bits, K, N, gs, desc_act, M = WORKLOADS[args.workload]
     gemv = M <= 8
     line = {
@@ -563,36 +683,53 @@ def main():
                    "desc_act": desc_act, "weight_copies": len(case["qweights"]), "plan": s["plan"],
                    "entry": ENTRY[prepared], "prepared": PREPARED_NOTE[prepared]},
         "parity": {"ok": ok, "max_abs_err": round(max_err, 6), "rtol": 1e-2, "atol": 1e-2},
-        "timing": {k: s[k] for k in ("eager_us", "graph_us", "graph_error", "unprepared_us") if k in s},
+        "timing": {"statistic": f"median over {REGIONS} pairs of timed regions of t(2 K) - t(K), K = {args.steps} steps "
+                                f"(graph replay; the fixed start-up of a replay cancels)",
+                   **{k: s[k] for k in ("min_us", "region_us", "replay_overhead_us", "eager_us", "graph_us",
+                                        "graph_error", "unprepared_us") if k in s}},
         "hbm_frac": s["hbm_frac"], "tflops": s["TFLOPs"],
     }
     line["roofline"] = roofline_of(args.workload, s)
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(case)      # (while the headline's layer is still the one held)
     if args.workload == DEFAULT_WORKLOAD and not forced and not args.unprepared and not args.no_secondary:
-        # the other halves of the metric, each a timed record of its own with its roofline and parity
-        secondary = []
+        # the other points of the metric's configurations, each a timed record of its own with its roofline and
+        # parity; workloads on one layer follow each other so that the layer is built once
+        seen = {WORKLOADS[args.workload]}
+        todo = []
         for name in SECONDARY_WORKLOADS:
+            if WORKLOADS[name] not in seen:
+                seen.add(WORKLOADS[name])
+                todo.append(name)
+        rows_of = {}
+        for name in todo:
+            rows_of[WORKLOADS[name][:5]] = max(rows_of.get(WORKLOADS[name][:5], 0), WORKLOADS[name][5])
+        todo.sort(key=lambda n: (list(rows_of).index(WORKLOADS[n][:5]), WORKLOADS[n][5]))
+        secondary = []
+        for name in todo:
             prep = prepared_mode(name)
-            c = build_case(name, dev, prepared=prep)
+            c = build_case(name, dev, prepared=prep, max_rows=rows_of[WORKLOADS[name][:5]])
             okc, errc = check_case(c, dev)
             r = summarize(c, time_case(c, dev, args.steps, args.warmup))
             secondary.append({
-                "workload": name, "value": r["us"], "unit": "us", "steps": args.steps, "warmup": args.warmup,
-                "timing": {k: r[k] for k in ("eager_us", "graph_us", "graph_error") if k in r},
-                "entry": ENTRY[prep], "prepared": PREPARED_NOTE[prep], "plan": r["plan"],
+                "workload": name, "value": r["us"], "min_us": r.get("min_us"), "unit": "us", "steps": args.steps,
+                "warmup": args.warmup, "entry": ENTRY[prep], "plan": r["plan"],
                 "hbm_frac": r["hbm_frac"], "tflops": r["TFLOPs"], "mfma_frac": r["mfma_frac"],
                 "roofline": roofline_of(name, r),
                 "parity": {"ok": okc, "max_abs_err": round(errc, 6), "rtol": 1e-2, "atol": 1e-2},
             })
             del c
-            torch.cuda.empty_cache()
         line["secondary"] = secondary
     if args.sweep:
         sweep = []
-        for name, prep in [(n, pr) for n in sorted(WORKLOADS) for pr in (None, "sorted", "tiled")]:
+        names = sorted(WORKLOADS, key=lambda n: (WORKLOADS[n][:5], WORKLOADS[n][5]))
+        for name, prep in [(n, pr) for n in names for pr in (None, "sorted", "tiled")]:
             if ((prep is None and not plain_applies(name)) or (prep == "sorted" and not sorted_applies(name))
                     or (prep == "tiled" and not tiled_applies(name))):
                 continue
-            c = build_case(name, dev, prepared=prep)
+            rows = max(v[5] for v in WORKLOADS.values() if v[:5] == WORKLOADS[name][:5])
+            c = build_case(name, dev, prepared=prep, max_rows=rows)
             okc, errc = check_case(c, dev)
             r = summarize(c, time_case(c, dev, min(args.steps, 100), min(args.warmup, 10)))
             r["prepared"] = prep
@@ -601,10 +738,9 @@ def main():
             r["max_abs_err"] = round(errc, 6)
             sweep.append(r)
             del c
-            torch.cuda.empty_cache()
         line["sweep"] = sweep
-    if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(case)
+    if cpu is not None:
+        line["cpu_baseline"] = cpu
     print(json.dumps(line))
 
 
