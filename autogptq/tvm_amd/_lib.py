@@ -31,6 +31,7 @@ ABI_SYMBOLS = (
     "gptq_hip_gemm_plan",
     "gptq_hip_gemm_static",
     "gptq_hip_static_workspace_limit",
+    "gptq_hip_static_init",
     "gptq_hip_gemm_sorted",
     "gptq_hip_sorted_workspace_bytes",
     "gptq_hip_sort_channels",
@@ -145,6 +146,8 @@ def lib() -> ctypes.CDLL:
     l.gptq_hip_gemm_plan.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
     l.gptq_hip_gemm_static.restype = i
     l.gptq_hip_gemm_static.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
+    l.gptq_hip_static_init.restype = i
+    l.gptq_hip_static_init.argtypes = []
     l.gptq_hip_static_workspace_limit.restype = sz
     l.gptq_hip_static_workspace_limit.argtypes = []
     l.gptq_hip_gemm_sorted.restype = i

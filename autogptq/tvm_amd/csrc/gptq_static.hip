@@ -21,10 +21,10 @@ constexpr int kMaxDevices = 64;
 void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on device i, nullptr until first use
 std::mutex g_scratch_mutex;
 
-// The address of this device's copy of the array.  First use on a device asks the runtime for it and
-// clears the head of the array, where the split-K counters live (they must be zero before the first
-// call; every call leaves them zero).
-int scratch_of_current_device(void *stream, void **out)
+// The address of this device's copy of the array: first use on a device asks the runtime for it.  Nothing is
+// launched: an array of static storage duration starts out all zero, which is what the split-K counters at its head
+// need before the first call, and every call leaves them zero.
+int scratch_of_current_device(void **out)
 {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
@@ -38,9 +38,6 @@ int scratch_of_current_device(void *stream, void **out)
             (void)hipGetLastError();
             return GPTQ_HIP_ERR_LAUNCH;
         }
-        // a fill kernel, not a memset: this call may be recorded into a graph
-        const int rc = gptq::launch_fill_zero(ptr, gptq::kCounterBytes, stream);
-        if (rc != GPTQ_HIP_OK) return rc;
         g_scratch_ptr[dev] = ptr;
     }
     *out = g_scratch_ptr[dev];
@@ -50,6 +47,12 @@ int scratch_of_current_device(void *stream, void **out)
 }  // namespace
 
 extern "C" size_t gptq_hip_static_workspace_limit(void) { return kStaticScratchBytes; }
+
+extern "C" int gptq_hip_static_init(void)
+{
+    void *ws = nullptr;
+    return scratch_of_current_device(&ws);
+}
 
 extern "C" int gptq_hip_gemm_static(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                                     const int32_t *g_idx, const void *bias, void *y, int M, int K, int N, int bits,
@@ -61,7 +64,7 @@ extern "C" int gptq_hip_gemm_static(const void *x, const int32_t *qweight, const
     if (plan.workspace_bytes > kStaticScratchBytes) return GPTQ_HIP_ERR_WORKSPACE;  // beyond the array: use gptq_hip_gemm
     void *ws = nullptr;
     if (plan.workspace_bytes > 0) {
-        rc = scratch_of_current_device(stream, &ws);
+        rc = scratch_of_current_device(&ws);
         if (rc != GPTQ_HIP_OK) return rc;
     }
     return gptq_hip_gemm_plan(x, qweight, qzeros, scales, g_idx, bias, y, ws, ws ? kStaticScratchBytes : 0, M, K, N,

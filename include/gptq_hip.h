@@ -135,13 +135,17 @@ int gptq_hip_gemm_plan(const void *x, const int32_t *qweight, const int32_t *qze
  * (16 MiB) inside the library, one copy per GPU, held until the process ends.  A problem whose plan needs more
  * returns GPTQ_HIP_ERR_WORKSPACE (use gptq_hip_gemm with a workspace of your own).  Every call on a GPU uses that
  * GPU's one array: calls that overlap on the same GPU (different streams or threads) race; calls on one
- * stream, or otherwise ordered, are fine.  The first call on a device looks the array's address up and zeroes
- * its counters with a fill kernel on `stream`.
+ * stream, or otherwise ordered, are fine.  The first use on a device looks the array's address up (no launch, no
+ * fill: the array starts out zero and every call leaves its counters zero); the runtime may load the code object for
+ * that, so make the first call, or gptq_hip_static_init() with the device current, before a stream capture begins.
  */
 int gptq_hip_gemm_static(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                          const int32_t *g_idx, const void *bias, void *y, int M, int K, int N, int bits,
                          int group_size, void *stream);
 size_t gptq_hip_static_workspace_limit(void);
+/* Looks up the current device's array (nothing is launched); GPTQ_HIP_OK, or GPTQ_HIP_ERR_LAUNCH if the runtime
+ * refuses.  Optional: gptq_hip_gemm_static does the same on its first call on a device. */
+int gptq_hip_static_init(void);
 
 /*
  * The decode product (one row, or a batch of up to 16) for a layer prepared when it was loaded: an activation-order g_idx makes

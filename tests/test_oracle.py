@@ -214,3 +214,48 @@ def test_forward_keeps_leading_dims():
     x = torch.randn((2, 3, 64), generator=torch.Generator().manual_seed(2)).half()
     y = orc.forward_ref(x, L["qweight"], L["qzeros"], L["scales"], L["g_idx"], None, 4)
     assert y.shape == (2, 3, 32) and y.dtype == torch.float16
+
+
+# Vectors written by the reference's own QuantLinear.forward on the CPU (tests/golden/make_forward_vectors.py):
+# forward(I) without the bias is the reference's dequantised weight, forward(x) its output.
+def _forward_vectors():
+    import os
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "forward_vectors.npz")
+    data = np.load(path)
+    return data, sorted({k.split(".")[0] for k in data.files})
+
+
+_FWD, _FWD_NAMES = _forward_vectors()
+
+
+def test_forward_vectors_cover_every_width_with_and_without_an_activation_order():
+    seen = {(int(_FWD[n + ".meta"][0]), bool(_FWD[n + ".meta"][4])) for n in _FWD_NAMES}
+    assert seen == {(b, a) for b in (2, 3, 4, 8) for a in (False, True)}
+    assert any(int(_FWD[n + ".meta"][3]) == -1 for n in _FWD_NAMES)
+
+
+@pytest.mark.parametrize("name", _FWD_NAMES)
+def test_oracle_reproduces_the_reference_forward(name, c_oracle):
+    bits, K, N, gs, act, has_bias = (int(v) for v in _FWD[name + ".meta"])
+    qweight, qzeros, g_idx = _FWD[name + ".qweight"], _FWD[name + ".qzeros"], _FWD[name + ".g_idx"]
+    scales = _FWD[name + ".scales"].view(np.float16)
+    bias = _FWD[name + ".bias"].view(np.float16) if has_bias else None
+    x = _FWD[name + ".x"].view(np.float16)
+    w_ref, y_ref = _FWD[name + ".w"], _FWD[name + ".y"].view(np.float16)
+    tq, tz, ts, tg = (torch.from_numpy(a.copy()) for a in (qweight, qzeros, scales, g_idx))
+    # the dequantised weight: bit for bit, from all three statements of the oracle
+    assert np.array_equal(orc.dequant_ref(tq, tz, ts, tg, bits).numpy().view(np.uint16), w_ref)
+    assert np.array_equal(orc.dequant_exact(qweight, qzeros, scales, g_idx, bits).view(np.uint16), w_ref)
+    assert np.array_equal(c_oracle.dequant(qweight, qzeros, scales, g_idx, bits).view(np.uint16), w_ref)
+    # the output: the torch restatement runs the reference's own operations in its order (same bits on the same
+    # torch build; one fp16 ulp of slack for another build's summation order); the C restatement sums in double
+    tb = torch.from_numpy(bias.copy()) if bias is not None else None
+    y = orc.forward_ref(torch.from_numpy(x.copy()), tq, tz, ts, tg, tb, bits).numpy()
+    assert y.dtype == np.float16 and y.shape == y_ref.shape
+    ulp = np.maximum(np.abs(y_ref.astype(np.float32)), 2.0 ** -14) * 2.0 ** -10
+    assert np.all(np.abs(y.astype(np.float32) - y_ref.astype(np.float32)) <= ulp)
+    yc = c_oracle.forward(x, qweight, qzeros, scales, g_idx, bias, bits)
+    # (the reference adds in fp16-rounded steps the CPU backend chooses: K products of magnitude <= |x| |w|)
+    bound = 2e-3 + 2e-3 * np.abs(yc)
+    assert np.all(np.abs(yc - y_ref.astype(np.float32)) <= bound)

@@ -59,3 +59,36 @@ def test_static_entry_rejects_what_the_array_cannot_hold():
     assert plan.workspace_bytes > lib.gptq_hip_static_workspace_limit()
     fake, null = ctypes.c_void_p(0x1000), ctypes.c_void_p(None)
     assert lib.gptq_hip_gemm_static(fake, fake, fake, fake, fake, null, fake, 4096, 4096, 11008, 4, 128, null) == _lib.ERR_WORKSPACE
+
+
+def test_static_entry_replays_from_a_captured_graph():
+    """What the entry point is for: a call recorded into a HIP graph (no allocation, no fill, no lookup inside the
+    capture once gptq_hip_static_init has run), replayed several times with eager work in between; every replay
+    must equal the eager result."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    dev = torch.device("cuda:0")
+    assert _lib.lib().gptq_hip_static_init() == _lib.OK
+    bits, K, N, gs, act, M = 4, 4096, 1056, 128, True, 40
+    L = layer(8200, K, N, bits, gs, act, M=M, bias=True)
+    D = to_dev(L, dev)
+    D.update(K=K, N=N)
+    want = ops.gemm(D["x"], D["qweight"], D["qzeros"], D["scales"], D["g_idx"], D["bias"], bits, gs)
+    y = torch.zeros((M, N), dtype=torch.float16, device=dev)
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+    stream = torch.cuda.Stream(device=dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        rc = _lib.lib().gptq_hip_gemm_static(vp(D["x"]), vp(D["qweight"]), vp(D["qzeros"]), vp(D["scales"]), vp(D["g_idx"]),
+                                             vp(D["bias"]), vp(y), M, K, N, bits, gs,
+                                             ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+    assert rc == _lib.OK
+    for rep in range(3):
+        y.zero_()
+        torch.cuda.synchronize(dev)
+        graph.replay()
+        torch.cuda.synchronize(dev)
+        assert torch.equal(y, want), f"replay {rep} differs from the eager result"
+        # eager work of the program's own between the replays, on the same array
+        rc2, eager = _static(D, M)
+        assert rc2 == _lib.OK and torch.equal(eager, want)
