@@ -47,6 +47,7 @@ ABI_SYMBOLS = (
     "gptq_hip_gemm_tiled_transposed",
     "gptq_hip_gemm_tiled",
     "gptq_hip_dequant",
+    "gptq_hip_probe",
     "gptq_hip_strerror",
     "gptq_hip_abi_version",
     "gptq_hip_build_id",
@@ -82,6 +83,7 @@ PLAN_PRIVATE_ZERO_WORKSPACE = 1
 
 COPY_CHECKPOINT, COPY_SORTED, COPY_TILED = 1, 2, 4
 ROUTE_CHECKPOINT, ROUTE_SORTED, ROUTE_TILED, ROUTE_LIBRARY = 0, 1, 2, 3
+PROBE_EMPTY, PROBE_STREAM, PROBE_MIXED = 0, 1, 2
 ROUTE_NAMES = {ROUTE_CHECKPOINT: "plain", ROUTE_SORTED: "sorted", ROUTE_TILED: "tiled", ROUTE_LIBRARY: "library"}
 
 
@@ -178,6 +180,8 @@ def lib() -> ctypes.CDLL:
     l.gptq_hip_select_tiled_transposed.argtypes = [i, i, i, i, i, ctypes.POINTER(Plan)]
     l.gptq_hip_gemm_tiled_transposed.restype = i
     l.gptq_hip_gemm_tiled_transposed.argtypes = [vp, vp, vp, vp, vp, vp, sz, i, i, i, i, i, ctypes.POINTER(Plan), vp]
+    l.gptq_hip_probe.restype = i
+    l.gptq_hip_probe.argtypes = [i, vp, sz, vp, sz, i, i, i, i, vp, vp, vp]
     l.gptq_hip_dequant.restype = i
     l.gptq_hip_dequant.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
     l.gptq_hip_strerror.restype = ctypes.c_char_p

@@ -5,7 +5,7 @@ import hashlib
 import os
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
-SOURCES = ["gptq_stream.hip", "gptq_grouped.hip", "gptq_dequant.hip", "gptq_static.hip", "gptq_tiled.hip", "gptq_tiled_decode.hip", "gptq_tiled_decode16.hip", "gptq_dispatch.cpp", "gptq_capi.cpp"]
+SOURCES = ["gptq_stream.hip", "gptq_grouped.hip", "gptq_dequant.hip", "gptq_static.hip", "gptq_probe.hip", "gptq_tiled.hip", "gptq_tiled_decode.hip", "gptq_tiled_decode16.hip", "gptq_dispatch.cpp", "gptq_capi.cpp"]
 HEADERS = ["gptq_unpack.h", "gptq_internal.h", "gptq_device.h", "gptq_tiled_common.h", os.path.join("..", "..", "..", "include", "gptq_hip.h"),
            "binding.cpp"]   # (hashed with the rest: both libraries carry one build id)
 

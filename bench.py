@@ -606,6 +606,95 @@ def run_transposed(args, dev):
     }))
 
 
+def _slope_us(launch, dev, n: int, regions: int = 5) -> float:
+    """Microseconds per launch of a chain of dependent launches, as the difference of a graph of 2 n launches and
+    one of n (median over `regions` pairs), so that the fixed start-up of a replay cancels."""
+    def graph(count):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for j in range(count):
+                launch(j)
+        return g
+    launch(0)
+    torch.cuda.synchronize(dev)
+    g1, g2 = graph(n), graph(2 * n)
+    out = []
+    for _ in range(regions + 1):
+        t = []
+        for g in (g1, g2):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize(dev)
+            a.record()
+            g.replay()
+            b.record()
+            torch.cuda.synchronize(dev)
+            t.append(a.elapsed_time(b) * 1e3)
+        out.append((t[1] - t[0]) / n)
+    return float(statistics.median(out[1:]))
+
+
+def run_machine(args, dev):
+    """What this GPU gives the product kernels, measured with the library's probe kernels: the cost of a launch in a
+    chain of launches, the cost of a plain read of a layer's bytes by as many workgroups as the decode kernels use
+    (every launch a region that no cache still holds), and the rate of loads that hit L2 while the same CU also
+    streams from HBM (what the activation fragments of a matmul kernel pay next to its weight stream)."""
+    import numpy as np
+    from autogptq.tvm_amd import _lib
+    l = _lib.lib()
+    def cur():      # (inside a capture the current stream is the capturing one)
+        return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    big = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    big.view(torch.int32).random_(0, 1 << 30)
+    hot = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+    hot.view(torch.int32).random_(0, 1 << 30)
+    ticks = torch.zeros(4 * 256, dtype=torch.int64, device=dev)
+
+    def check(rc):
+        if rc != 0:
+            raise RuntimeError(f"gptq_hip_probe: {rc}")
+
+    out = {"launch_us": {}, "stream_read": [], "l2_hit_loads_per_cu": {}}
+    for wgs in (256, 432, 1024):
+        out["launch_us"][str(wgs)] = round(_slope_us(
+            lambda j: check(l.gptq_hip_probe(_lib.PROBE_EMPTY, None, 0, None, 0, wgs, 0, 0, 0, None, None, cur())),
+            dev, args.steps), 3)
+    for label, nbytes in (("int3 4096x11008", 4096 * 11008 * 3 // 8), ("int3 9216x36864", 9216 * 36864 * 3 // 8)):
+        nbytes = nbytes // 4096 * 4096
+        regions = big.numel() // nbytes
+        for wgs in (256, 432, 1024, 2048):
+            us = _slope_us(
+                lambda j: check(l.gptq_hip_probe(_lib.PROBE_STREAM, ctypes.c_void_p(big.data_ptr() + (j % regions) * nbytes),
+                                                 nbytes, None, 0, wgs, 0, 0, 0, None,
+                                                 ctypes.c_void_p(sink.data_ptr()), cur())),
+                dev, max(regions, min(args.steps, 2 * regions)))
+            out["stream_read"].append({"bytes_of": label, "bytes": nbytes, "workgroups": wgs, "us": round(us, 3),
+                                       "GBps": round(nbytes / us * 1e-3, 1)})
+    iters, wall_hz = 400, 1e8     # the wall clock of this GPU ticks at 100 MHz
+    per_cu = 2 * iters * 8 * 1024
+    for label, mode, depth in (("alone", 0, 1), ("next to two more such waves", 1, 1),
+                               ("next to an HBM stream, 1 request per round and wave", 2, 1),
+                               ("next to an HBM stream, 4 requests per round and wave", 2, 4),
+                               ("next to an HBM stream, 8 requests per round and wave", 2, 8)):
+        rates = []
+        for _ in range(3):
+            ticks.zero_()
+            check(l.gptq_hip_probe(_lib.PROBE_MIXED, ctypes.c_void_p(big.data_ptr()), big.numel(),
+                                   ctypes.c_void_p(hot.data_ptr()), hot.numel(), 256, iters, mode, depth,
+                                   ctypes.c_void_p(ticks.data_ptr()), ctypes.c_void_p(sink.data_ptr()), cur()))
+            torch.cuda.synchronize(dev)
+            tk = ticks.view(256, 4)[:, :2].double().max(dim=1).values      # the slower of a CU's two reading waves
+            rates.append(float((per_cu / (tk / wall_hz)).median()) * 1e-9)
+        out["l2_hit_loads_per_cu"][label] = {"GBps": round(float(np.median(rates)), 1)}
+    out["note"] = ("launch_us and stream_read: per launch of a chain of dependent launches, graph of 2 n minus graph of "
+                   "n; stream_read regions rotate through 1 GiB so that no cache holds them; l2_hit_loads_per_cu: two "
+                   "waves of a 256-thread workgroup (one workgroup per CU) read a 1 MiB buffer with direct loads into LDS, 16 B "
+                   "per lane, a round of eight 1 KiB requests in flight behind the round waited for; median over the "
+                   "256 workgroups")
+    print(json.dumps({"machine": out}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -621,12 +710,15 @@ def main():
     ap.add_argument("--prepared", default="auto", choices=("auto", "none", "sorted", "tiled"),
                     help="which copy of the layer to run on: the module's own choice (auto), the checkpoint's "
                          "tensors, the sorted copy or the tiled copy")
-    ap.add_argument("--kernel", type=int, default=0, help="force a kernel family (1 gather, 2 grouped, 3 blocked)")
+    ap.add_argument("--kernel", type=int, default=0, help="force a kernel family (2 grouped, 3 stream)")
     ap.add_argument("--split-k", type=int, default=0, help="force the split-K factor")
     ap.add_argument("--waves-n", type=int, default=0, help="force the waves per workgroup along N (STREAM kernel: along K)")
     ap.add_argument("--transposed", action="store_true",
                     help="time the gradient for x of the workload's layer (gy[M, N] @ W^T on the transposed tiled "
                          "copy) instead of the forward product")
+    ap.add_argument("--machine", action="store_true",
+                    help="only measure what the GPU gives the kernels (launch cost, plain streaming reads by as many "
+                         "workgroups, L2-hit loads next to an HBM stream in one CU) with the library's probe kernels")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 256 MiB device copy a few times (known traffic, for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters of a profiler run) and exit")
@@ -650,6 +742,9 @@ def main():
         torch.cuda.synchronize(dev)
         print(json.dumps({"copy_calibration": {"bytes_read": nbytes, "bytes_written": nbytes, "launches": 5,
                                                "kernel": "torch elementwise copy (int32)"}}))
+        return
+    if args.machine:
+        run_machine(args, dev)
         return
     if args.transposed:
         run_transposed(args, dev)

@@ -299,6 +299,23 @@ int gptq_hip_select_route(int M, int K, int N, int bits, int group_size, int act
 int gptq_hip_dequant(const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *g_idx,
                      void *w, int K, int N, int bits, int group_size, void *stream);
 
+/*
+ * Measurement aids, not on the product path and without a counterpart in the reference: small kernels that measure
+ * what the GPU gives the product kernels (bench.py --machine times them), so that the floors the kernels are judged
+ * against can be re-measured with committed code.  One launch on `stream`, nothing allocated.
+ *   GPTQ_HIP_PROBE_EMPTY   `workgroups` x 256 threads that do nothing (the cost of a launch in a chain of launches)
+ *   GPTQ_HIP_PROBE_STREAM  `workgroups` workgroups read `bytes` at `buf` once, 16 bytes per lane and request
+ *   GPTQ_HIP_PROBE_MIXED   per workgroup, waves 0 and 1 read the `hot_bytes` (>= 64 KiB, small enough to stay in L2)
+ *                          at `hot`, `iters` rounds of eight 1 KiB requests, while waves 2 and 3 are idle (mode 0),
+ *                          do the same (mode 1) or stream `bytes` at `buf` from HBM with `depth` (1..8) requests in
+ *                          flight (mode 2); ticks[4 * workgroup + wave] (device memory, uint64) = wall-clock ticks of
+ *                          each reading wave (hipDeviceAttributeWallClockRate gives their rate)
+ * `scratch`: 16 bytes of device memory that are never written (they keep the loads alive).
+ */
+enum { GPTQ_HIP_PROBE_EMPTY = 0, GPTQ_HIP_PROBE_STREAM = 1, GPTQ_HIP_PROBE_MIXED = 2 };
+int gptq_hip_probe(int kind, const void *buf, size_t bytes, const void *hot, size_t hot_bytes, int workgroups, int iters,
+                   int mode, int depth, unsigned long long *ticks, void *scratch, void *stream);
+
 /* Human-readable text for a gptq_hip_status. */
 const char *gptq_hip_strerror(int status);
 
