@@ -8,6 +8,12 @@ CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 SOURCES = ["gptq_stream.hip", "gptq_grouped.hip", "gptq_dequant.hip", "gptq_static.hip", "gptq_probe.hip", "gptq_tiled.hip", "gptq_tiled_decode.hip", "gptq_tiled_decode16.hip", "gptq_dispatch.cpp", "gptq_capi.cpp"]
 HEADERS = ["gptq_unpack.h", "gptq_internal.h", "gptq_device.h", "gptq_tiled_common.h", os.path.join("..", "..", "..", "include", "gptq_hip.h"),
            "binding.cpp"]   # (hashed with the rest: both libraries carry one build id)
+# Compiler options of single sources.  The decode kernels keep the four result registers of their small matrix
+# instructions in ordinary vector registers: left to itself the compiler puts them into accumulation registers
+# for the workgroups of four waves and copies them back for every epilogue.
+EXTRA_FLAGS = {
+    "gptq_tiled_decode.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
 
 
 def source_hash() -> str:
@@ -17,6 +23,7 @@ def source_hash() -> str:
     for name in sorted(SOURCES + HEADERS):
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(name.encode() + b"\0" + f.read() + b"\0")
+    h.update(repr(sorted(EXTRA_FLAGS.items())).encode())
     return h.hexdigest()[:16]
 
 

@@ -13,7 +13,7 @@ import shutil
 import subprocess
 import sys
 
-from ._sources import CSRC, HEADERS, SOURCES, source_hash  # noqa: F401
+from ._sources import CSRC, EXTRA_FLAGS, HEADERS, SOURCES, source_hash  # noqa: F401
 
 LIB = os.path.join(CSRC, "libgptq_hip.so")
 BINDING_LIB = os.path.join(CSRC, "libgptq_hip_torch.so")
@@ -69,7 +69,7 @@ def parse_resource_remarks(text: str) -> dict:
 
 
 def _compile_one(src: str, obj: str, build_id: str):
-    cmd = [hipcc()] + [f for f in flags() if f != "-shared"] + [
+    cmd = [hipcc()] + [f for f in flags() if f != "-shared"] + EXTRA_FLAGS.get(os.path.basename(src), []) + [
         f'-DGPTQ_HIP_BUILD_ID="{build_id}"', "-Rpass-analysis=kernel-resource-usage", "-c", "-o", obj, src]
     return subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
 

@@ -48,6 +48,52 @@ __device__ __forceinline__ void tile_load(const char *src, uint32_t (&wr)[BITS])
     }
 }
 
+// The same load through a buffer resource that spans one column tile: the lane's byte offset in a vector register
+// that never changes, the block's offset in a scalar register (no per-lane address arithmetic per block).  The
+// scalar offset is NOT part of the buffer's range check on this architecture: the caller keeps the block inside
+// the tile.
+typedef uint32_t u3v __attribute__((ext_vector_type(3)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_buffer(const char *tile, uint32_t bytes)
+{
+    // (a wave-uniform base; data format word of a raw buffer on this architecture)
+    const uint64_t a = (uint64_t)tile;
+    // (readfirstlane returns a signed int: through uint32_t, or the low half would sign-extend into the high one)
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32));
+    const uint64_t u = ((uint64_t)hi << 32) | (uint64_t)lo;
+    return __builtin_amdgcn_make_buffer_rsrc((void *)u, 0, bytes, 0x00020000);
+}
+
+template <int BITS>
+__device__ __forceinline__ void tile_load(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_bytes, uint32_t block_bytes,
+                                          uint32_t (&wr)[BITS])
+{
+    constexpr int NT = 2;   // the non-temporal hint the pointer loads above carry
+    if constexpr (BITS == 4) {
+        const u4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_bytes, block_bytes, NT);
+#pragma unroll
+        for (int e = 0; e < 4; e++) wr[e] = v[e];
+    } else if constexpr (BITS == 8) {
+        const u4 v0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_bytes, block_bytes, NT);
+        const u4 v1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_bytes + 1024u, block_bytes, NT);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            wr[e] = v0[e];
+            wr[4 + e] = v1[e];
+        }
+    } else if constexpr (BITS == 2) {
+        const u2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, lane_bytes, block_bytes, NT);
+        wr[0] = v[0];
+        wr[1] = v[1];
+    } else {
+        const u3v v = __builtin_amdgcn_raw_buffer_load_b96(rsrc, lane_bytes, block_bytes, 0);
+        wr[0] = v[0];
+        wr[1] = v[1];
+        wr[2] = v[2];
+    }
+}
+
 // The magic constants of the width's unpack, each held in a vector register.
 template <int BITS>
 __device__ __forceinline__ void tile_magic(uint32_t (&mg)[TileCodec<BITS>::KINDS])

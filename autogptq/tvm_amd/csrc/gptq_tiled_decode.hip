@@ -80,7 +80,6 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     const int wg_steps = ws * KW;                        // blocks of the workgroup's K range
     const int S_wg = is_half ? split * ws_first * KW : split * wg_steps;   // its first block
     const int S_begin = S_wg + wave * ws;                // this wave's first block
-    const int S_last = p.S_total - 1;
     const int span = wg_steps * 64;                      // positions the workgroup stages
     const int p0 = S_wg * 64;                            // its first position
 
@@ -112,22 +111,29 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
         for (int m = 0; m < MR; m++) xq[ps][m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
     }
     // the (scale, zero) words of the range's groups for this tile's 32 columns: SZP passes in registers
+    // (a scalar base for the range's first group and the tile's columns, a 32-bit offset per lane: the words of
+    // one tile lie within 4 N G bytes, which the format keeps below 4 GB)
     constexpr int SZP = 4;
     uint32_t szq[SZP];
+    const char *sz_wg = (const char *)(p.sz + ((size_t)g_first * (size_t)p.N + (size_t)(32 * T)));
+    auto sz_word = [&](int i) {
+        const uint32_t off = ((uint32_t)(i >> 5) * (uint32_t)p.N + (uint32_t)(i & 31)) * 4u;
+        return *(const uint32_t *)(sz_wg + off);
+    };
 #pragma unroll
-    for (int ps = 0; ps < SZP; ps++) {
-        const int i = min(tid + ps * NT, n_groups * 32 - 1);
-        szq[ps] = p.sz[(size_t)(g_first + (uint32_t)(i >> 5)) * p.N + 32 * T + (i & 31)];
-    }
+    for (int ps = 0; ps < SZP; ps++) szq[ps] = sz_word(min(tid + ps * NT, n_groups * 32 - 1));
     __builtin_amdgcn_sched_barrier(0);
     const uint32_t b_lane = tile_lane_bytes<BITS>((uint32_t)lane);
-    const uint32_t tile_off = (uint32_t)T * (uint32_t)p.S_total;
+    constexpr uint32_t BLOCK_BYTES = 256u * BITS;
+    // the tile as a buffer: the lane's offset in a vector register, the block's in a scalar one.  Blocks requested
+    // past the wave's range (ahead of the walk, never multiplied) are the next wave's; past the end of the tile:
+    // its last block again (the padding of K past the wave's range: multiplied by zeros of x)
+    const __amdgpu_buffer_rsrc_t tile = tile_buffer(p.qtile + (size_t)T * (size_t)p.S_total * BLOCK_BYTES,
+                                                    (uint32_t)p.S_total * BLOCK_BYTES);
+    const int S_last = p.S_total - 1;
     uint32_t w[2][PF][BITS];
-    const int steps = min(ws, max(p.S_total - S_begin, 0));  // blocks of this wave that lie inside K
     auto load_w = [&](int i, uint32_t (&wr)[BITS]) {
-        // block i of the wave's range; past its end: its first block again (a cache hit that is never multiplied)
-        const int Sc = min(S_begin + (i < steps ? i : 0), S_last);
-        tile_load<BITS>(p.qtile + ((size_t)(tile_off + (uint32_t)Sc) * (256u * BITS) + b_lane), wr);
+        tile_load<BITS>(tile, b_lane, (uint32_t)min(S_begin + i, S_last) * BLOCK_BYTES, wr);
     };
     // two chunks of PF blocks are in flight from here on, through the staging of x as well
 #pragma unroll
@@ -145,11 +151,22 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
 #pragma unroll
             for (int m = 0; m < MR; m++) xl[m * span + i] = (_Float16)0;
     }
+    // (a workgroup with a part of K, a half tile or one of several ranges, keeps the channels of its own range)
+    const bool ranged = is_half || gridDim.y > 1;
     auto scatter8 = [&](int k, const u4 &kv, const h8 (&xv)[MR]) {
         if (!p.kinv) {   // no activation order: the eight channels are eight consecutive positions, one store
             // (k8_lo .. k8_hi is the workgroup's own range here, a multiple of 8 away from p0)
 #pragma unroll
             for (int m = 0; m < MR; m++) *(h8 *)(xl + m * span + (k - p0)) = xv[m];
+            return;
+        }
+        if (!ranged) {   // the workgroup stages all of K: every position is its own, no test and no branch per channel
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const uint32_t pos = (kv[e >> 1] >> (16 * (e & 1))) & 0xffffu;
+#pragma unroll
+                for (int m = 0; m < MR; m++) xl[(uint32_t)(m * span) + pos] = xv[m][e];
+            }
             return;
         }
 #pragma unroll
@@ -181,9 +198,7 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
         const int i = tid + ps * NT;
         if (i < n_groups * 32) szl[i] = szq[ps];
     }
-    for (int i = tid + SZP * NT; i < n_groups * 32; i += NT) {  // more groups than the register passes hold
-        szl[i] = p.sz[(size_t)(g_first + (uint32_t)(i >> 5)) * p.N + 32 * T + (i & 31)];
-    }
+    for (int i = tid + SZP * NT; i < n_groups * 32; i += NT) szl[i] = sz_word(i);  // more groups than the passes hold
     lds_barrier();
     // ---- 3. per epilogue unit (E blocks), half and row: Xsum = sum x, Bsum = sum x * base(position) over the
     //         unit's 32 E positions of that half; every wave for the units of its own slice (LDS serves one
@@ -237,14 +252,16 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
 #pragma unroll
     for (int m = 0; m < MR; m++) ysum[m] = 0.f;
     // Per-lane byte offsets that never change; what changes per block is wave-uniform and stays in scalar
-    // registers.  A lane whose row lies past M reads the 64 zero bytes whatever the block (stride 0).
+    // registers.
     // The matrix instruction broadcasts A: with cbsz = 3 the eight 4-lane blocks of a half wave all take their A
     // operand from block `abid` of the half.  So lane block b of a half holds only positions 4 b .. 4 b + 3 of the
     // half's 32 (one 8-byte read per lane and block instead of 64 bytes), and the instruction for positions
     // 4 i .. 4 i + 3 names abid = i.
     const int lb8 = (lane >> 2) & 7;
-    const uint32_t x_base = row_i < p.M ? (uint32_t)(row_i * span + 32 * h + 4 * lb8) * 2u : zero_off;
-    const uint32_t x_stride = row_i < p.M ? 128u : 0u;
+    // (a lane whose row lies past M supplies the last row again: row i of A only reaches result register i, and
+    // the registers past M are never stored; one stride for all lanes keeps the block's offset an immediate)
+    const uint32_t x_base = (uint32_t)(min(row_i, p.M - 1) * span + 32 * h + 4 * lb8) * 2u;
+    constexpr uint32_t x_stride = 128u;
     const uint32_t xs_lane = zero_off + 64u + (uint32_t)(h * MR) * 8u;   // sums of half h of unit 0
     const uint32_t sz_lane = (uint32_t)((const unsigned char *)szl - smem) + (uint32_t)n * 4u;
 

@@ -152,7 +152,10 @@ class Layer:
         self.wbytes = K * N * bits // 8
         self.copies = max(2, -(-2 * INFINITY_CACHE_BYTES // self.wbytes), int(os.environ.get("GPTQ_BENCH_MIN_COPIES", "0")))
         self.qzeros, self.scales = self.L["qzeros"].to(dev), self.L["scales"].to(dev)
-        self.g_idx = self.L["g_idx"].to(dev) if desc_act else None
+        # a layer of one group has no order of groups to follow: its g_idx is all zeros, QuantLinear passes none
+        # to the kernels (and no channel maps of the tiled copy), and neither does this harness
+        self.mapped = bool(desc_act and 0 < gs < K)
+        self.g_idx = self.L["g_idx"].to(dev) if self.mapped else None
         self.x = self.L["x"].to(dev)
         self._fmt = {}
         self._want = None
@@ -180,7 +183,7 @@ class Layer:
             if prepared == "tiled":
                 # (every copy brings its own scale / zero words and channel maps, as every layer of a model does)
                 qtile, sz, xsrc, kinv = ops.tile_prepare(q, self.qzeros, self.scales, self.g_idx, bits, gs)
-                out["aux"].append((sz, xsrc if desc_act else None, kinv if desc_act else None))
+                out["aux"].append((sz, xsrc if self.mapped else None, kinv if self.mapped else None))
                 q = qtile
             out["qweights"].append(q)
         if prepared == "sorted":
@@ -241,7 +244,7 @@ def build_case(name: str, dev, kernel: int = 0, split_k: int = 0, waves_n: int =
         "wbytes": lay.wbytes, "flops": 2 * M * K * N, "kmap": f["kmap"], "prepared": prepared,
         "qweights": f["qweights"], "aux": f["aux"],
     }
-    act = desc_act and prepared != "sorted"   # the sorted copy is planned like contiguous groups
+    act = lay.mapped and prepared != "sorted"   # the sorted copy is planned like contiguous groups
     if prepared == "tiled":
         plan = _lib.select_tiled(M, K, N, bits, gs)
     elif prepared == "sorted" and not (kernel or split_k or waves_n):

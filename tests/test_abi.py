@@ -371,9 +371,9 @@ def table_tiled_wins(M, K, N, act_order, bits, one_group):
             return True
         if K <= 4096:
             return M <= 2 or N < 16384
-        if K > 32768:
-            return False
-        return M <= 2 or K <= 6656 or (K <= 11008 and N <= 8192)
+        if M <= 2:
+            return True
+        return K <= 6656 or (K <= 11008 and N <= 8192)
     if M <= 16:
         return (not act_order) and K <= 4096 and N > 4096 and (M >= 9 or bits == 4)
     if M <= 128:
