@@ -194,7 +194,8 @@ constexpr int kDecodeSelectRows = 4;   // rows up to which gptq_hip_select_tiled
 inline int tiled_decode_rows(int M) { return M <= 1 ? 1 : (M <= 2 ? 2 : 4); }
 inline int tiled_decode_lds_bytes(int mr, int span, int groups, int waves_k)
 {
-    return mr * span * 2 + 64 + (span / 32) * mr * 8 + groups * 128 + waves_k * mr * 128;
+    (void)groups;   // (the (scale, zero) words no longer pass through LDS)
+    return mr * span * 2 + 64 + (span / 32) * mr * 8 + waves_k * mr * 128;
 }
 // decode kernel with one workgroup per CU (16-column units, all of K staged): LDS of a workgroup that takes
 // `units_per_wg` units

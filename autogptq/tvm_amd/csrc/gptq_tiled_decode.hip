@@ -10,7 +10,7 @@ namespace gptq {
 //
 // A workgroup owns ONE column tile (32 columns) and one K range; its KW waves split that range.  With one
 // small workgroup per tile every CU gets work whatever N is (11008 columns: 344 workgroups of 4 waves,
-// 4096 columns: 128 of 16), and what a wave keeps in flight (PF blocks of 1 KB / 768 B) adds up over the
+// 4096 columns: 128 of 16), and what a wave keeps in flight (eight blocks of 1 KB / 768 B) adds up over the
 // many waves of a CU.
 // The dots run on v_mfma_f32_4x4x4_16B_f16: sixteen independent 4-lane blocks, lane 4 b + i supplies
 // row i of A and column i of B of block b, and result register v of lane 4 b + j is row v of column j.
@@ -57,7 +57,16 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     static_assert(MR <= 4 && (E == 1 || E == 2), "one matrix instruction set per lane block");
     constexpr bool EXACT = tiled_decode_exact(BITS);
     constexpr int NT = 64 * KW;
-    constexpr int PF = 2;              // blocks of weights per chunk; two chunks are in flight
+    constexpr int PF = 2;              // blocks of weights per chunk
+    // chunks in flight per wave.  A wave asks for a chunk when it has consumed one, so its walk is a chain of
+    // round trips to HBM (0.9-1 us each under load), one per NCH chunks: with two chunks in flight a wave of 16
+    // blocks makes four of them, and the walk, not the staging of x, sets the length of the kernel.  Four chunks
+    // for the workgroups of four waves (wide layers with K up to 4096: 16 or 8 blocks per wave), one or two rows:
+    // 4096 x 11008 int4 7.5 -> 7.0 us with an activation order, 7.5 -> 6.8 without (int3 6.55 either way).  The
+    // longer waves of eight and sixteen keep two: four cost them occupancy (100 registers against 60) and more
+    // than they gain (9216 x 9216 int3 9.4 -> 10.5 us, 9216 x 36864 24.9 -> 27.9), four rows and 8 bits as well.
+    constexpr int NCH = (KW == 4 && MR <= 2 && !EXACT) ? 4 : 2;
+    constexpr int RING = NCH * PF;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -84,20 +93,18 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     const int p0 = S_wg * 64;                            // its first position
 
     // LDS: x in position order [MR][span] fp16 | 64 zero bytes | block sums [span / 32][MR] (Xsum, Bsum) |
-    //      (scale, zero) words of the range's groups [groups][32] | partial results [KW][MR][32]
+    //      partial results [KW][MR][32]
     _Float16 *xl = (_Float16 *)smem;
     const uint32_t zero_off = (uint32_t)MR * (uint32_t)span * 2u;
     f2 *xs = (f2 *)(smem + zero_off + 64);
     const int lbs = span / 32;
-    const uint32_t g_first = __umulhi((uint32_t)(2 * S_wg), p.lbg_magic) + (p.lbg_add ? (uint32_t)(2 * S_wg) : 0u);
-    const uint32_t lb_end = (uint32_t)min(2 * (S_wg + wg_steps), 2 * p.S_total) - 1u;
-    const uint32_t g_lastr = min(__umulhi(lb_end, p.lbg_magic) + (p.lbg_add ? lb_end : 0u), (uint32_t)p.G - 1u);
-    const int n_groups = (int)(g_lastr - g_first) + 1;
-    uint32_t *szl = (uint32_t *)(xs + (size_t)lbs * MR);
-    float *red = (float *)(szl + (size_t)n_groups * 32);
+    float *red = (float *)(xs + (size_t)lbs * MR);
 
     // ---- 1. x and the map first (a wait for them would also wait for every older load: vector loads return
-    //         in order), then the first weights of this wave, then the (scale, zero) words ----------------
+    //         in order), then the first weights of this wave, each unit's (scale, zero) word in front of them.
+    //         (The words are cold in HBM and belong to one tile: staged through LDS they kept every wave of the
+    //         workgroup at the barrier until the last of them had arrived, 0.6-0.9 us after x; a wave now asks
+    //         for the word of a unit when it asks for the unit's weights and finds it when they are there.) -----
     // (without a map the channels of the range are the range itself)
     const int k8_lo = p.kinv ? 0 : p0 / 8, k8_hi = p.kinv ? p.K / 8 : min(p0 + span, p.K) / 8;
     constexpr int QP = 2;  // passes over x kept in registers
@@ -110,18 +117,6 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
 #pragma unroll
         for (int m = 0; m < MR; m++) xq[ps][m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
     }
-    // the (scale, zero) words of the range's groups for this tile's 32 columns: SZP passes in registers
-    // (a scalar base for the range's first group and the tile's columns, a 32-bit offset per lane: the words of
-    // one tile lie within 4 N G bytes, which the format keeps below 4 GB)
-    constexpr int SZP = 4;
-    uint32_t szq[SZP];
-    const char *sz_wg = (const char *)(p.sz + ((size_t)g_first * (size_t)p.N + (size_t)(32 * T)));
-    auto sz_word = [&](int i) {
-        const uint32_t off = ((uint32_t)(i >> 5) * (uint32_t)p.N + (uint32_t)(i & 31)) * 4u;
-        return *(const uint32_t *)(sz_wg + off);
-    };
-#pragma unroll
-    for (int ps = 0; ps < SZP; ps++) szq[ps] = sz_word(min(tid + ps * NT, n_groups * 32 - 1));
     __builtin_amdgcn_sched_barrier(0);
     const uint32_t b_lane = tile_lane_bytes<BITS>((uint32_t)lane);
     constexpr uint32_t BLOCK_BYTES = 256u * BITS;
@@ -131,15 +126,33 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     const __amdgpu_buffer_rsrc_t tile = tile_buffer(p.qtile + (size_t)T * (size_t)p.S_total * BLOCK_BYTES,
                                                     (uint32_t)p.S_total * BLOCK_BYTES);
     const int S_last = p.S_total - 1;
-    uint32_t w[2][PF][BITS];
+    // the (scale, zero) words of the tile's 32 columns as a buffer: lane n (both halves) reads column n of the
+    // group of its lane block, the group's row in a scalar register
+    const __amdgpu_buffer_rsrc_t szb = tile_buffer((const char *)(p.sz + 32 * T), (uint32_t)(((size_t)p.G * p.N - 32 * T) * 4));
+    const uint32_t sz_lane = (uint32_t)n * 4u;
+    const uint32_t row_bytes = (uint32_t)p.N * 4u;
+    auto group_of = [&](uint32_t lb) { return min(__umulhi(lb, p.lbg_magic) + (p.lbg_add ? lb : 0u), (uint32_t)p.G - 1u); };
+    constexpr int UPC = PF / E;        // units per chunk
+    uint32_t w[NCH][PF][BITS], szr[NCH][UPC];
     auto load_w = [&](int i, uint32_t (&wr)[BITS]) {
         tile_load<BITS>(tile, b_lane, (uint32_t)min(S_begin + i, S_last) * BLOCK_BYTES, wr);
     };
-    // two chunks of PF blocks are in flight from here on, through the staging of x as well
+    auto load_s = [&](int i, uint32_t &sr) {   // the unit that starts with block i of the wave's range
+        const uint32_t l0 = 2u * (uint32_t)min(S_begin + i, S_last);
+        const uint32_t g0 = group_of(l0);
+        uint32_t off = sz_lane;
+        if constexpr (E == 1) off += h ? (group_of(l0 + 1u) - g0) * row_bytes : 0u;   // the two halves of a block may differ
+        sr = __builtin_amdgcn_raw_buffer_load_b32(szb, off, g0 * row_bytes, 0);
+    };
+    auto load_chunk = [&](int i, uint32_t (&wc)[PF][BITS], uint32_t (&sc)[UPC]) {
 #pragma unroll
-    for (int u = 0; u < PF; u++) load_w(u, w[0][u]);
+        for (int u = 0; u < UPC; u++) load_s(i + u * E, sc[u]);
 #pragma unroll
-    for (int u = 0; u < PF; u++) load_w(PF + u, w[1][u]);
+        for (int u = 0; u < PF; u++) load_w(i + u, wc[u]);
+    };
+    // NCH chunks of PF blocks are in flight from here on, through the staging of x as well
+#pragma unroll
+    for (int j = 0; j < NCH; j++) load_chunk(j * PF, w[j], szr[j]);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- 2. stage x in position order ------------------------------------------------------------------
@@ -193,12 +206,6 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
         for (int m = 0; m < MR; m++) xv[m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
         scatter8(k, kv, xv);
     }
-#pragma unroll
-    for (int ps = 0; ps < SZP; ps++) {
-        const int i = tid + ps * NT;
-        if (i < n_groups * 32) szl[i] = szq[ps];
-    }
-    for (int i = tid + SZP * NT; i < n_groups * 32; i += NT) szl[i] = sz_word(i);  // more groups than the passes hold
     lds_barrier();
     // ---- 3. per epilogue unit (E blocks), half and row: Xsum = sum x, Bsum = sum x * base(position) over the
     //         unit's 32 E positions of that half; every wave for the units of its own slice (LDS serves one
@@ -263,27 +270,17 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     const uint32_t x_base = (uint32_t)(min(row_i, p.M - 1) * span + 32 * h + 4 * lb8) * 2u;
     constexpr uint32_t x_stride = 128u;
     const uint32_t xs_lane = zero_off + 64u + (uint32_t)(h * MR) * 8u;   // sums of half h of unit 0
-    const uint32_t sz_lane = (uint32_t)((const unsigned char *)szl - smem) + (uint32_t)n * 4u;
 
     // x of a block: this lane's four positions of row row_i; read one block ahead of its use
     auto load_x = [&](uint32_t sb, u2 &xv) { xv = *(const u2 *)(smem + x_base + x_stride * sb); };
     f4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};  // two chains: a matrix instruction waits for the one it adds to
     uint32_t szw = 0u;   // (scale, zero) word and sums of the unit in flight, read when the unit starts
     f2 xsv[MR];
-    auto block = [&](auto uu_c, int S, const uint32_t (&wr)[BITS], const u2 &xc, u2 &xn) {
+    auto block = [&](auto uu_c, int S, const uint32_t (&wr)[BITS], uint32_t sr, const u2 &xc, u2 &xn) {
         constexpr int uu = decltype(uu_c)::value;                 // block inside its unit
         const uint32_t sb = (uint32_t)(S - S_wg);                  // block inside the workgroup's range (wave-uniform)
         if constexpr (uu == 0) {
-            // group of the unit's lane blocks (E = 1: the two halves of the wave may differ)
-            const uint32_t l0 = 2u * (uint32_t)S;
-            const uint32_t g0 = min(__umulhi(l0, p.lbg_magic) + (p.lbg_add ? l0 : 0u), (uint32_t)p.G - 1u) - g_first;
-            uint32_t goff = g0 * 128u;
-            if constexpr (E == 1) {
-                const uint32_t l1 = l0 + 1u;
-                const uint32_t g1 = min(__umulhi(l1, p.lbg_magic) + (p.lbg_add ? l1 : 0u), (uint32_t)p.G - 1u) - g_first;
-                goff = (h ? g1 : g0) * 128u;
-            }
-            szw = *(const uint32_t *)(smem + sz_lane + goff);
+            szw = sr;   // the unit's (scale, zero) word, requested with its weights
             if constexpr (!EXACT) {
                 const f2 *xb = (const f2 *)(smem + xs_lane + (sb / E) * (uint32_t)(2 * MR * 8));
 #pragma unroll
@@ -319,35 +316,42 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
         }
     };
 
-    // Chunks of PF blocks, two in flight; x rides one block ahead in two register sets.  Blocks past the end
+    // Chunks of PF blocks, NCH in flight; x rides one block ahead in two register sets.  Blocks past the end
     // of K inside a wave's range are harmless (their x and sums are zeros), blocks past the range are skipped.
     u2 xr[2];
     load_x((uint32_t)(S_begin - S_wg), xr[0]);
-    auto chunk = [&](int c, uint32_t (&wc)[PF][BITS], auto all_c) {
+    auto chunk = [&](int c, uint32_t (&wc)[PF][BITS], const uint32_t (&sc)[UPC], auto all_c) {
         constexpr bool ALL = decltype(all_c)::value;
         [&]<int... U>(std::integer_sequence<int, U...>) {
             ((ALL || c + U < ws
-                  ? block(std::integral_constant<int, U % E>{}, S_begin + c + U, wc[U], xr[U & 1], xr[(U + 1) & 1])
+                  ? block(std::integral_constant<int, U % E>{}, S_begin + c + U, wc[U], sc[U / E], xr[U & 1], xr[(U + 1) & 1])
                   : (void)0),
              ...);
         }(std::make_integer_sequence<int, PF>{});
     };
     int c = 0;
-    for (; c + 2 * PF <= ws; c += 2 * PF) {
-        chunk(c, w[0], std::true_type{});
-        __builtin_amdgcn_sched_barrier(0);
+    // steady state: every chunk consumed is replaced by the one a ring further on, which lies inside the range
+    for (; c + 2 * RING <= ws; c += RING) {
 #pragma unroll
-        for (int u = 0; u < PF; u++) load_w(c + 2 * PF + u, w[0][u]);  // the chunk after the one in flight
-        __builtin_amdgcn_sched_barrier(0);
-        chunk(c + PF, w[1], std::true_type{});
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int u = 0; u < PF; u++) load_w(c + 3 * PF + u, w[1][u]);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int j = 0; j < NCH; j++) {
+            chunk(c + j * PF, w[j], szr[j], std::true_type{});
+            __builtin_amdgcn_sched_barrier(0);
+            load_chunk(c + RING + j * PF, w[j], szr[j]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
-    if (c < ws) {   // what is left of the range: fewer than two chunks, nothing more to request
-        chunk(c, w[0], std::false_type{});
-        chunk(c + PF, w[1], std::false_type{});
+    if (ws - c == RING) {   // exactly what is in flight is left: no more requests, no tests
+#pragma unroll
+        for (int j = 0; j < NCH; j++) chunk(c + j * PF, w[j], szr[j], std::true_type{});
+    } else {
+        // less than two rings left: the blocks in flight, then the rest, requested as registers come free
+#pragma unroll
+        for (int j = 0; j < NCH; j++) {
+            chunk(c + j * PF, w[j], szr[j], std::false_type{});
+            if (c + RING + j * PF < ws) load_chunk(c + RING + j * PF, w[j], szr[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < NCH; j++) chunk(c + RING + j * PF, w[j], szr[j], std::false_type{});
     }
 
     // ---- 5. the two halves of a column (lanes n and n + 32), then the waves along K ---------------------
@@ -419,6 +423,7 @@ int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, co
                         int group_size, const gptq_hip_plan &plan, void *stream_v)
 {
     hipStream_t stream = (hipStream_t)stream_v;
+    if ((unsigned long long)G * (unsigned long long)N >= (1ull << 30)) return GPTQ_HIP_ERR_UNSUPPORTED;   // 32-bit offsets into sz
     DecodeParams p;
     p.x = (const _Float16 *)x;
     p.kinv = kinv;
