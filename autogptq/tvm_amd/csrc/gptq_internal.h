@@ -203,8 +203,8 @@ constexpr int kNumCUs = 256;   // MI355X
 inline long long tiled_decode16_lds_bytes(int mr, int K, int groups, int units_per_wg)
 {
     const long long span = ((K + 63) / 64 + 1) / 2 * 128;
-    return mr * span * 2 + 64 + (span / 32) * mr * 8 + (long long)units_per_wg * groups * 128 +
-           (long long)units_per_wg * 16 * mr * 256;
+    (void)groups;   // (the (scale, zero) words no longer pass through LDS)
+    return mr * span * 2 + 64 + (span / 32) * mr * 8 + (long long)units_per_wg * 16 * mr * 256;
 }
 int launch_tile_prepare(const uint32_t *qweight, const uint32_t *qzeros, const void *scales, const int32_t *g_idx,
                         uint32_t *qtile, uint32_t *sz, int32_t *xsrc, uint16_t *kinv, int K, int N, int G, int bits,

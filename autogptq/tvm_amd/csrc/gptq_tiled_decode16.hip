@@ -53,14 +53,15 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     const int S_last = p.S_total - 1;
 
     // LDS: x in position order [MR][span] fp16 | 64 zero bytes | sums [span / 32][MR] (Xsum, Bsum) |
-    //      (scale, zero) as floats [n_units][G][16] | partial results [n_units][NW][MR][64]
+    //      partial results [n_units][NW][MR][64]
     _Float16 *xl = (_Float16 *)smem;
     const uint32_t zero_off = (uint32_t)MR * (uint32_t)span * 2u;
     f2 *xs = (f2 *)(smem + zero_off + 64);
-    f2 *szl = xs + (size_t)(span / 32) * MR;
-    float *red = (float *)(szl + (size_t)n_units * p.G * 16);
+    float *red = (float *)(xs + (size_t)(span / 32) * MR);
 
-    // ---- 1. requests: x and the map first (loads return in order), the (scale, zero) words, the weights ----
+    // ---- 1. requests: x and the map first (loads return in order), then the weights, each item's (scale, zero)
+    //         word in front of it (the words are cold in HBM: staged through LDS they held every wave at the
+    //         barrier until the last of them had arrived, well after x) ---------------------------------------
     const int k8_hi = p.K / 8;
     u4 kq;
     h8 xq[MR];
@@ -70,15 +71,6 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
 #pragma unroll
         for (int m = 0; m < MR; m++) xq[m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
     }
-    constexpr int SZP = 2;
-    const int sz_words = n_units * p.G * 16;
-    uint32_t szq[SZP];
-    auto sz_src = [&](int i) {   // word i of the table: unit i / (16 G), group (i / 16) % G, column i % 16
-        const int ul = i / (16 * p.G), r = i - ul * 16 * p.G;
-        return p.sz + (size_t)(r >> 4) * p.N + 16 * (u0 + ul) + (r & 15);
-    };
-#pragma unroll
-    for (int ps = 0; ps < SZP; ps++) szq[ps] = *sz_src(min(tid + ps * NT, sz_words - 1));
     __builtin_amdgcn_sched_barrier(0);
 
     // items of the workgroup: (unit, virtual block) pairs, unit after unit.
@@ -104,8 +96,23 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
                           tile_lane_bytes<BITS>(16u * (uint32_t)(unit & 1)));
     };
     const char *rq_ptr = unit_base(rq_u) + (size_t)rq_v * (512u * BITS);
-    uint32_t w[2][PF][BITS];
-    auto load_w = [&](uint32_t (&wr)[BITS]) {
+    // the (scale, zero) table as a buffer: lane (column n16, lane block lbv) reads the word of its column and of
+    // the group of its 32 positions; what is wave-uniform of that (the unit's columns, and the group where all
+    // four lane blocks share it) travels in the scalar offset
+    const __amdgpu_buffer_rsrc_t szb = tile_buffer((const char *)p.sz, (uint32_t)((size_t)p.G * p.N * 4));
+    const uint32_t row_bytes = (uint32_t)p.N * 4u;
+    auto group_of = [&](uint32_t lb) { return min(__umulhi(lb, p.lbg_magic) + (p.lbg_add ? lb : 0u), (uint32_t)p.G - 1u); };
+    uint32_t w[2][PF][BITS], szr[2][PF];
+    auto load_w = [&](uint32_t (&wr)[BITS], uint32_t &sr) {
+        {
+            const uint32_t cols = (uint32_t)(16 * (u0 + rq_u)) * 4u;
+            if constexpr (G128) {
+                sr = __builtin_amdgcn_raw_buffer_load_b32(szb, (uint32_t)n16 * 4u, group_of(4u * (uint32_t)rq_v) * row_bytes + cols, 0);
+            } else {
+                sr = __builtin_amdgcn_raw_buffer_load_b32(
+                    szb, group_of(4u * (uint32_t)rq_v + (uint32_t)lbv) * row_bytes + (uint32_t)n16 * 4u, cols, 0);
+            }
+        }
         tile_load<BITS>(rq_ptr + (2 * rq_v + 1 <= S_last ? b_lane2 : b_lane), wr);
         // past the wave's items: its last item again (a cache hit that is never multiplied)
         if (rq_left > 1) {
@@ -130,12 +137,12 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
         }
     };
 #pragma unroll
-    for (int u = 0; u < PF; u++) load_w(w[0][u]);
+    for (int u = 0; u < PF; u++) load_w(w[0][u], szr[0][u]);
 #pragma unroll
-    for (int u = 0; u < PF; u++) load_w(w[1][u]);
+    for (int u = 0; u < PF; u++) load_w(w[1][u], szr[1][u]);
     __builtin_amdgcn_sched_barrier(0);
 
-    // ---- 2. stage x in position order, and the (scale, zero) words ------------------------------------------
+    // ---- 2. stage x in position order -----------------------------------------------------------------------
     if (tid < 16) ((uint32_t *)(smem + zero_off))[tid] = 0u;
     for (int i = p.K + tid; i < span; i += NT)   // the padding of the last virtual block reads as zeros
 #pragma unroll
@@ -162,18 +169,6 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
 #pragma unroll
         for (int m = 0; m < MR; m++) xv[m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
         scatter8(k, kv, xv);
-    }
-#pragma unroll
-    for (int ps = 0; ps < SZP; ps++) {
-        const int i = tid + ps * NT;
-        if (i < sz_words) {
-            const h2 e = as_h2(szq[ps]);
-            szl[i] = (f2){(float)e[0], (float)e[1]};
-        }
-    }
-    for (int i = tid + SZP * NT; i < sz_words; i += NT) {
-        const h2 e = as_h2(*sz_src(i));
-        szl[i] = (f2){(float)e[0], (float)e[1]};
     }
     // CONTIG: a wave writes the partial results of the units it walks: the others read as zeros
     if constexpr (CONTIG)
@@ -223,7 +218,6 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     const uint32_t x_stride = row_i < p.M ? 256u : 0u;
     const uint32_t x_second = row_i < p.M ? 32u : 0u;   // bytes to positions 16 ..
     const uint32_t xs_lane = zero_off + 64u + (uint32_t)(lbv * MR) * 8u;
-    const uint32_t sz_lane = (uint32_t)((const unsigned char *)szl - smem) + (uint32_t)n16 * 8u;
     const uint32_t red_lane = (uint32_t)((const unsigned char *)red - smem) + (uint32_t)lane * 4u;
 
     auto load_x = [&](int V, u2 (&xv)[2]) {
@@ -232,18 +226,11 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
         xv[1] = *(const u2 *)(smem + xoff + x_second);
     };
     int cu = first_u, cv = first_v, c_left = n_items;   // (unit, V) of the item being computed, items still to compute
-    auto item = [&](const uint32_t (&wr)[BITS], const u2 (&xc)[2], u2 (&xn)[2]) {
+    auto item = [&](const uint32_t (&wr)[BITS], uint32_t sr, const u2 (&xc)[2], u2 (&xn)[2]) {
         const int V = cv, ul = cu;
-        // this item's scale, zero point and sums
-        uint32_t goff;
-        if constexpr (G128) {
-            const uint32_t lb = 4u * (uint32_t)V;
-            goff = min(__umulhi(lb, p.lbg_magic) + (p.lbg_add ? lb : 0u), (uint32_t)p.G - 1u) * 128u;
-        } else {
-            const uint32_t lb = 4u * (uint32_t)V + (uint32_t)lbv;
-            goff = min(__umulhi(lb, p.lbg_magic) + (p.lbg_add ? lb : 0u), (uint32_t)p.G - 1u) * 128u;
-        }
-        const f2 szf = *(const f2 *)(smem + sz_lane + (uint32_t)ul * (uint32_t)p.G * 128u + goff);
+        // this item's scale and zero point (the word that came with its weights) and sums
+        const h2 sze = as_h2(sr);
+        const f2 szf = {(float)sze[0], (float)sze[1]};
         f2 xsv[MR];
         if constexpr (!EXACT) {
             const f2 *xb = (const f2 *)(smem + xs_lane + (uint32_t)V * (uint32_t)(4 * MR * 8));
@@ -262,10 +249,7 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
         u4 q[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) TileCodec<BITS>::operand(wr, j, q[j], mg);
-        if constexpr (EXACT) {   // (both floats came from fp16 values: the conversions back are exact)
-            const h2 e = {(_Float16)szf[0], (_Float16)szf[1]};
-            tiled_dequant_exact<BITS>(q, as_u32(e));
-        }
+        if constexpr (EXACT) tiled_dequant_exact<BITS>(q, sr);
         f4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};  // two chains
         const h4 xa[2] = {__builtin_bit_cast(h4, xc[0]), __builtin_bit_cast(h4, xc[1])};
         [&]<int... V>(std::integer_sequence<int, V...>) {
@@ -291,28 +275,28 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     };
     u2 xr[2][2];
     load_x(cv, xr[0]);
-    auto chunk = [&](int c, uint32_t (&wc)[PF][BITS], auto all_c) {
+    auto chunk = [&](int c, uint32_t (&wc)[PF][BITS], const uint32_t (&sc)[PF], auto all_c) {
         constexpr bool ALL = decltype(all_c)::value;
         [&]<int... U>(std::integer_sequence<int, U...>) {
-            ((ALL || c + U < n_items ? item(wc[U], xr[U & 1], xr[(U + 1) & 1]) : (void)0), ...);
+            ((ALL || c + U < n_items ? item(wc[U], sc[U], xr[U & 1], xr[(U + 1) & 1]) : (void)0), ...);
         }(std::make_integer_sequence<int, PF>{});
     };
     int c = 0;
     for (; c + 2 * PF <= n_items; c += 2 * PF) {
-        chunk(c, w[0], std::true_type{});
+        chunk(c, w[0], szr[0], std::true_type{});
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int u = 0; u < PF; u++) load_w(w[0][u]);
+        for (int u = 0; u < PF; u++) load_w(w[0][u], szr[0][u]);
         __builtin_amdgcn_sched_barrier(0);
-        chunk(c + PF, w[1], std::true_type{});
+        chunk(c + PF, w[1], szr[1], std::true_type{});
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int u = 0; u < PF; u++) load_w(w[1][u]);
+        for (int u = 0; u < PF; u++) load_w(w[1][u], szr[1][u]);
         __builtin_amdgcn_sched_barrier(0);
     }
     if (c < n_items) {
-        chunk(c, w[0], std::false_type{});
-        chunk(c + PF, w[1], std::false_type{});
+        chunk(c, w[0], szr[0], std::false_type{});
+        chunk(c + PF, w[1], szr[1], std::false_type{});
     }
     if (!CONTIG && vpu == 0) {   // strided: a wave without virtual blocks (K shorter than sixteen of them) adds zeros
         for (int ul = 0; ul < n_units; ul++)
