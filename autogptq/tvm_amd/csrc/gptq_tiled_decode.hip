@@ -117,6 +117,53 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
 #pragma unroll
         for (int m = 0; m < MR; m++) xq[ps][m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
     }
+    // (a workgroup with a part of K, a half tile or one of several ranges, keeps the channels of its own range)
+    const bool ranged = is_half || gridDim.y > 1;
+    auto scatter8 = [&](int k, const u4 &kv, const h8 (&xv)[MR]) {
+        if (!p.kinv) {   // no activation order: the eight channels are eight consecutive positions, one store
+            // (k8_lo .. k8_hi is the workgroup's own range here, a multiple of 8 away from p0)
+#pragma unroll
+            for (int m = 0; m < MR; m++) *(h8 *)(xl + m * span + (k - p0)) = xv[m];
+            return;
+        }
+        if (!ranged) {   // the workgroup stages all of K: every position is its own, no test and no branch per channel
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const uint32_t pos = (kv[e >> 1] >> (16 * (e & 1))) & 0xffffu;
+#pragma unroll
+                for (int m = 0; m < MR; m++) xl[(uint32_t)(m * span) + pos] = xv[m][e];
+            }
+            return;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int pos = (int)((kv[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+            const int pl = pos - p0;
+            if ((unsigned)pl < (unsigned)span) {
+#pragma unroll
+                for (int m = 0; m < MR; m++) xl[m * span + pl] = xv[m][e];
+            }
+        }
+    };
+    // Long layers: the channels the register passes do not hold, a pass at a time, before the weights are asked for
+    // (a wait for a load waits for every older one).  The loads of this loop are issued and waited for inside one
+    // asm statement each: left to the compiler's own bookkeeping, a loop with loads in it made it assume their
+    // registers still pending wherever the loop may have run, and it put a wait for outstanding loads in front of
+    // the weight requests, or, with the loop behind them, a wait for all of them in front of the sums and the walk.
+    auto load16_now = [](const void *ptr) {
+        u4 v;
+        asm volatile("global_load_dwordx4 %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(ptr) : "memory");
+        return v;
+    };
+    for (int k8 = k8_lo + tid + QP * NT; k8 < k8_hi; k8 += NT) {
+        const int k = 8 * k8;
+        u4 kv = {0u, 0u, 0u, 0u};
+        if (p.kinv) kv = load16_now(p.kinv + k);
+        h8 xv[MR];
+#pragma unroll
+        for (int m = 0; m < MR; m++) xv[m] = __builtin_bit_cast(h8, load16_now(p.x + (size_t)min(m, p.M - 1) * p.K + k));
+        scatter8(k, kv, xv);
+    }
     __builtin_amdgcn_sched_barrier(0);
     const uint32_t b_lane = tile_lane_bytes<BITS>((uint32_t)lane);
     constexpr uint32_t BLOCK_BYTES = 256u * BITS;
@@ -164,47 +211,10 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
 #pragma unroll
             for (int m = 0; m < MR; m++) xl[m * span + i] = (_Float16)0;
     }
-    // (a workgroup with a part of K, a half tile or one of several ranges, keeps the channels of its own range)
-    const bool ranged = is_half || gridDim.y > 1;
-    auto scatter8 = [&](int k, const u4 &kv, const h8 (&xv)[MR]) {
-        if (!p.kinv) {   // no activation order: the eight channels are eight consecutive positions, one store
-            // (k8_lo .. k8_hi is the workgroup's own range here, a multiple of 8 away from p0)
-#pragma unroll
-            for (int m = 0; m < MR; m++) *(h8 *)(xl + m * span + (k - p0)) = xv[m];
-            return;
-        }
-        if (!ranged) {   // the workgroup stages all of K: every position is its own, no test and no branch per channel
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const uint32_t pos = (kv[e >> 1] >> (16 * (e & 1))) & 0xffffu;
-#pragma unroll
-                for (int m = 0; m < MR; m++) xl[(uint32_t)(m * span) + pos] = xv[m][e];
-            }
-            return;
-        }
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const int pos = (int)((kv[e >> 1] >> (16 * (e & 1))) & 0xffffu);
-            const int pl = pos - p0;
-            if ((unsigned)pl < (unsigned)span) {
-#pragma unroll
-                for (int m = 0; m < MR; m++) xl[m * span + pl] = xv[m][e];
-            }
-        }
-    };
 #pragma unroll
     for (int ps = 0; ps < QP; ps++) {
         const int k8 = k8_lo + tid + ps * NT;
         if (k8 < k8_hi) scatter8(8 * k8, kq[ps], xq[ps]);
-    }
-    for (int k8 = k8_lo + tid + QP * NT; k8 < k8_hi; k8 += NT) {  // long layers: the rest, a pass at a time
-        const int k = 8 * k8;
-        u4 kv = {0u, 0u, 0u, 0u};
-        if (p.kinv) kv = *(const u4 *)(p.kinv + k);
-        h8 xv[MR];
-#pragma unroll
-        for (int m = 0; m < MR; m++) xv[m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
-        scatter8(k, kv, xv);
     }
     lds_barrier();
     // ---- 3. per epilogue unit (E blocks), half and row: Xsum = sum x, Bsum = sum x * base(position) over the
