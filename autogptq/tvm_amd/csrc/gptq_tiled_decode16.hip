@@ -71,6 +71,37 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
 #pragma unroll
         for (int m = 0; m < MR; m++) xq[m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
     }
+    auto scatter8 = [&](int k, const u4 &kv, const h8 (&xv)[MR]) {
+        if (!p.kinv) {   // no activation order: the eight channels are eight consecutive positions, one store
+#pragma unroll
+            for (int m = 0; m < MR; m++) *(h8 *)(xl + m * span + k) = xv[m];
+            return;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int pos = min((int)((kv[e >> 1] >> (16 * (e & 1))) & 0xffffu), span - 1);
+#pragma unroll
+            for (int m = 0; m < MR; m++) xl[m * span + pos] = xv[m][e];
+        }
+    };
+    // Long layers: the channels past the register pass, a pass at a time, before the weights are asked for (a wait
+    // for a load waits for every older one).  Each load is issued and waited for inside one asm statement: with
+    // ordinary loads in a loop behind the weight requests the compiler put a wait for every outstanding load, the
+    // weights included, in front of the barrier, the sums and the walk of every layer.
+    auto load16_now = [](const void *ptr) {
+        u4 v;
+        asm volatile("global_load_dwordx4 %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(ptr) : "memory");
+        return v;
+    };
+    for (int k8 = tid + NT; k8 < k8_hi; k8 += NT) {
+        const int k = 8 * k8;
+        u4 kv = {0u, 0u, 0u, 0u};
+        if (p.kinv) kv = load16_now(p.kinv + k);
+        h8 xv[MR];
+#pragma unroll
+        for (int m = 0; m < MR; m++) xv[m] = __builtin_bit_cast(h8, load16_now(p.x + (size_t)min(m, p.M - 1) * p.K + k));
+        scatter8(k, kv, xv);
+    }
     __builtin_amdgcn_sched_barrier(0);
 
     // items of the workgroup: (unit, virtual block) pairs, unit after unit.
@@ -147,29 +178,7 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     for (int i = p.K + tid; i < span; i += NT)   // the padding of the last virtual block reads as zeros
 #pragma unroll
         for (int m = 0; m < MR; m++) xl[m * span + i] = (_Float16)0;
-    auto scatter8 = [&](int k, const u4 &kv, const h8 (&xv)[MR]) {
-        if (!p.kinv) {   // no activation order: the eight channels are eight consecutive positions, one store
-#pragma unroll
-            for (int m = 0; m < MR; m++) *(h8 *)(xl + m * span + k) = xv[m];
-            return;
-        }
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const int pos = min((int)((kv[e >> 1] >> (16 * (e & 1))) & 0xffffu), span - 1);
-#pragma unroll
-            for (int m = 0; m < MR; m++) xl[m * span + pos] = xv[m][e];
-        }
-    };
     if (tid < k8_hi) scatter8(8 * tid, kq, xq);
-    for (int k8 = tid + NT; k8 < k8_hi; k8 += NT) {   // long layers: the rest, a pass at a time
-        const int k = 8 * k8;
-        u4 kv = {0u, 0u, 0u, 0u};
-        if (p.kinv) kv = *(const u4 *)(p.kinv + k);
-        h8 xv[MR];
-#pragma unroll
-        for (int m = 0; m < MR; m++) xv[m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
-        scatter8(k, kv, xv);
-    }
     // CONTIG: a wave writes the partial results of the units it walks: the others read as zeros
     if constexpr (CONTIG)
         for (int i = tid; i < n_units * NW * MR * 64; i += NT) red[i] = 0.f;
