@@ -402,7 +402,7 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
         const int upw = ceil_div(units, nwg);
         const long long lds = gptq::tiled_decode16_lds_bytes(mr, K, K / gs, upw);
         // (long K: the kernel below with every tile halved, see tiled_decode_halves_all)
-        if (upw == 1 && lds <= 128 * 1024 && !gptq::tiled_decode_halves_all(N / 32, ceil_div(K, 64))) {
+        if (M <= 4 && upw == 1 && lds <= 128 * 1024 && !gptq::tiled_decode_halves_all(N / 32, ceil_div(K, 64))) {
             plan->kernel = GPTQ_HIP_KERNEL_TILED_DECODE;
             plan->row_tiles = mr;
             plan->m_blocks = 1;
@@ -439,6 +439,9 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
         // 9.9 / 12.9 with sixteen; 11008 x 4096 int3 8.4 / 11.2 and 8.5 / 11.4)
         const bool halves_all = gptq::tiled_decode_halves_all(tiles, S_total);
         if (halves_all) kw = 8;
+        // five to eight rows: at most eight waves (sixteen leave a lane 128 registers, which the two sets of rows
+        // do not fit into)
+        if (mr == 8 && kw == 16) kw = 8;
         while (kw > 4 && kw > S_total) kw >>= 1;
         // K beyond 32768 channels with more tiles than CUs: cut over workgroups of eight waves so that a wave walks
         // about eighteen blocks (36864 x 9216 int3, one group, one row: 34.6 us uncut with 72 blocks per wave, 31.4
@@ -489,10 +492,12 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
 
 extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan)
 {
-    // Up to four rows the decode kernel (one 4-row matrix instruction set per lane block); from five rows on
-    // the matmul kernel with one 32-row tile (a decode kernel with two sets took 24.6 us at eight rows of a
-    // 4096 x 11008 layer against 14.6).
-    if (M >= 1 && M <= gptq::kDecodeSelectRows) {
+    // Up to four rows the decode kernels (one 4-row matrix instruction set per lane block); five to eight rows the
+    // workgroup-per-tile decode kernel with two sets, for K up to 11008 (us at 5 / 8 rows, int4, against the matmul
+    // kernel with one 32-row tile: 4096 x 11008 9.0 / 9.4 against 9.6 / 9.7, with an activation order 12.7 / 13.2
+    // against 14.0 / 14.2; 11008 x 4096 9.9 / 10.3 against 16.7 / 17.2, with an activation order 15.1 / 15.8 against
+    // 18.9 / 19.4; 4096 x 4096 7.2 / 7.8 against 9.4 / 9.5; longer K was not measured: eight staged rows of x).
+    if (M >= 1 && (M <= gptq::kDecodeSelectRows || (M <= gptq::kDecodeMaxRows && K <= 11008))) {
         const int rc = gptq_hip_select_tiled_decode(M, K, N, bits, group_size, plan);
         if (rc != GPTQ_HIP_ERR_UNSUPPORTED || !plan) return rc;
     }
@@ -598,7 +603,12 @@ namespace {
 //     group, K cut in four ranges: 28.8 against 37.3); three and four rows: K up to 6656, and
 //     up to 11008 for layers of up to 8192 columns (beyond, the four staged rows of x cost more than they save:
 //     8192 x 28672 41.9 against 30.4);
-//   * 5 to 16 rows: only layers without an activation order, K up to 4096 and more than 4096 columns (the matmul
+//   * 5 to 8 rows, K up to 11008: the decode kernel with two sets of four rows (5 / 8 rows, int4 / int3, against the
+//     better of the other copies: 4096 x 11008 with an activation order 12.7 / 13.2 and 12.8 / 13.3 against 13.4 / 13.6
+//     and 12.5 / 12.6 on the sorted copy, without one 9.0 / 9.4 against 9.6 / 9.7 on the matmul kernel; 11008 x 4096 with
+//     an activation order 15.1 / 15.8 and 15.3 / 16.1 against 15.8 / 16.0 and 16.4 / 16.9, without one 9.9 / 10.3 against
+//     13.1; 4096 x 4096 7.2 / 7.8 against 9.9, with an activation order 9.5 / 10.2 against 10.9 (int3 12.3));
+//   * 5 to 16 rows otherwise: only layers without an activation order, K up to 4096 and more than 4096 columns (the matmul
 //     kernel then reads x itself, one launch: 4096 x 11008 int4, 5 / 8 / 16 rows: 10.6 / 10.7 / 11.5 against 11.2 /
 //     11.3 / 12.5; int3 from nine rows); with an activation order the pack pass makes it 14.6 against 13.4 at 8 rows;
 //   * 17 to 128 rows: almost everywhere (4096 x 11008 with an activation order, 32 / 64 / 128 rows: 14.8 / 19.2 /
@@ -616,6 +626,7 @@ bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
         if (K > 32768) return false;
         return K <= 6656 || (K <= 11008 && N <= 8192);
     }
+    if (M <= 8 && K <= 11008) return true;   // the decode kernel with two sets of rows (below)
     if (M <= 16) return !act_order && K <= 4096 && N > 4096 && (M >= 9 || bits == 4);
     if (M <= 128) {
         if (one_group && K > 8192 && (M > 32 || K > 16384 || N > 16384)) return false;

@@ -189,9 +189,9 @@ inline bool tiled_qualifies(int K, int N, int bits, int gs)
 }
 // decode kernel on the tiled format: rows it is built for, and the LDS of a workgroup whose waves cover
 // `span` positions of `groups` groups
-static const int kDecodeMaxRows = 4;      // rows the decode kernel of the tiled format takes
+static const int kDecodeMaxRows = 8;      // rows the decode kernel of the tiled format takes (the 16-column kernel: 4)
 constexpr int kDecodeSelectRows = 4;   // rows up to which gptq_hip_select_tiled chooses it
-inline int tiled_decode_rows(int M) { return M <= 1 ? 1 : (M <= 2 ? 2 : 4); }
+inline int tiled_decode_rows(int M) { return M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8)); }
 inline int tiled_decode_lds_bytes(int mr, int span, int groups, int waves_k)
 {
     (void)groups;   // (the (scale, zero) words no longer pass through LDS)

@@ -94,6 +94,64 @@ __device__ __forceinline__ void tile_load(__amdgpu_buffer_rsrc_t rsrc, uint32_t 
     }
 }
 
+// N 16-byte loads issued together and waited for in place, as ONE asm statement: the compiler's own bookkeeping of
+// outstanding loads does not see them (a loop of ordinary loads made it put waits for every outstanding load far
+// away from the loop, in front of code that every layer runs), and nothing can use a value before it has arrived.
+// The wait also covers every older load of the wave: such loops stand before the weight requests.
+#define GPTQ_LD(o, i) "global_load_dwordx4 %" #o ", %" #i ", off\n\t"
+template <int N>
+struct LoadNow;
+template <>
+struct LoadNow<1> {
+    static __device__ __forceinline__ void run(u4 (&v)[1], const void *const (&p)[1])
+    {
+        asm volatile(GPTQ_LD(0, 1) "s_waitcnt vmcnt(0)" : "=&v"(v[0]) : "v"(p[0]) : "memory");
+    }
+};
+template <>
+struct LoadNow<2> {
+    static __device__ __forceinline__ void run(u4 (&v)[2], const void *const (&p)[2])
+    {
+        asm volatile(GPTQ_LD(0, 2) GPTQ_LD(1, 3) "s_waitcnt vmcnt(0)" : "=&v"(v[0]), "=&v"(v[1]) : "v"(p[0]), "v"(p[1]) : "memory");
+    }
+};
+template <>
+struct LoadNow<3> {
+    static __device__ __forceinline__ void run(u4 (&v)[3], const void *const (&p)[3])
+    {
+        asm volatile(GPTQ_LD(0, 3) GPTQ_LD(1, 4) GPTQ_LD(2, 5) "s_waitcnt vmcnt(0)" : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]) : "v"(p[0]), "v"(p[1]), "v"(p[2]) : "memory");
+    }
+};
+template <>
+struct LoadNow<4> {
+    static __device__ __forceinline__ void run(u4 (&v)[4], const void *const (&p)[4])
+    {
+        asm volatile(GPTQ_LD(0, 4) GPTQ_LD(1, 5) GPTQ_LD(2, 6) GPTQ_LD(3, 7) "s_waitcnt vmcnt(0)" : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]) : "memory");
+    }
+};
+template <>
+struct LoadNow<5> {
+    static __device__ __forceinline__ void run(u4 (&v)[5], const void *const (&p)[5])
+    {
+        asm volatile(GPTQ_LD(0, 5) GPTQ_LD(1, 6) GPTQ_LD(2, 7) GPTQ_LD(3, 8) GPTQ_LD(4, 9) "s_waitcnt vmcnt(0)" : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]) : "memory");
+    }
+};
+template <>
+struct LoadNow<8> {
+    static __device__ __forceinline__ void run(u4 (&v)[8], const void *const (&p)[8])
+    {
+        asm volatile(GPTQ_LD(0, 8) GPTQ_LD(1, 9) GPTQ_LD(2, 10) GPTQ_LD(3, 11) GPTQ_LD(4, 12) GPTQ_LD(5, 13) GPTQ_LD(6, 14) GPTQ_LD(7, 15) "s_waitcnt vmcnt(0)" : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7]) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]) : "memory");
+    }
+};
+template <>
+struct LoadNow<9> {
+    static __device__ __forceinline__ void run(u4 (&v)[9], const void *const (&p)[9])
+    {
+        asm volatile(GPTQ_LD(0, 9) GPTQ_LD(1, 10) GPTQ_LD(2, 11) GPTQ_LD(3, 12) GPTQ_LD(4, 13) GPTQ_LD(5, 14) GPTQ_LD(6, 15) GPTQ_LD(7, 16) GPTQ_LD(8, 17) "s_waitcnt vmcnt(0)" : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7]), "=&v"(v[8]) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]), "v"(p[8]) : "memory");
+    }
+};
+#undef GPTQ_LD
+
 // The magic constants of the width's unpack, each held in a vector register.
 template <int BITS>
 __device__ __forceinline__ void tile_magic(uint32_t (&mg)[TileCodec<BITS>::KINDS])

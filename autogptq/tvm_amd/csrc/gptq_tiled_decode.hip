@@ -54,7 +54,8 @@ struct DecodeParams {
 template <int BITS, int MR, int KW, int E>
 __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParams p)
 {
-    static_assert(MR <= 4 && (E == 1 || E == 2), "one matrix instruction set per lane block");
+    static_assert((MR == 1 || MR == 2 || MR == 4 || MR == 8) && (E == 1 || E == 2), "one or two sets of four rows");
+    constexpr int RS = (MR + 3) / 4;   // sets of four rows: a matrix instruction takes four rows of x
     constexpr bool EXACT = tiled_decode_exact(BITS);
     constexpr int NT = 64 * KW;
     constexpr int PF = 2;              // blocks of weights per chunk
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     //         for the word of a unit when it asks for the unit's weights and finds it when they are there.) -----
     // (without a map the channels of the range are the range itself)
     const int k8_lo = p.kinv ? 0 : p0 / 8, k8_hi = p.kinv ? p.K / 8 : min(p0 + span, p.K) / 8;
-    constexpr int QP = 2;  // passes over x kept in registers
+    constexpr int QP = MR == 8 ? 1 : 2;  // passes over x kept in registers (eight rows: 32 registers a pass)
     u4 kq[QP];
     h8 xq[QP][MR];
 #pragma unroll
@@ -146,22 +147,33 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
         }
     };
     // Long layers: the channels the register passes do not hold, a pass at a time, before the weights are asked for
-    // (a wait for a load waits for every older one).  The loads of this loop are issued and waited for inside one
-    // asm statement each: left to the compiler's own bookkeeping, a loop with loads in it made it assume their
+    // (a wait for a load waits for every older one).  The loads of a pass are issued together and waited for inside one
+    // asm statement: left to the compiler's own bookkeeping, a loop with loads in it made it assume their
     // registers still pending wherever the loop may have run, and it put a wait for outstanding loads in front of
     // the weight requests, or, with the loop behind them, a wait for all of them in front of the sums and the walk.
-    auto load16_now = [](const void *ptr) {
-        u4 v;
-        asm volatile("global_load_dwordx4 %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(ptr) : "memory");
-        return v;
-    };
     for (int k8 = k8_lo + tid + QP * NT; k8 < k8_hi; k8 += NT) {
         const int k = 8 * k8;
         u4 kv = {0u, 0u, 0u, 0u};
-        if (p.kinv) kv = load16_now(p.kinv + k);
         h8 xv[MR];
+        if (p.kinv) {   // the map and the rows of x, requested together
+            const void *ptr[MR + 1];
+            u4 v[MR + 1];
+            ptr[MR] = p.kinv + k;
 #pragma unroll
-        for (int m = 0; m < MR; m++) xv[m] = __builtin_bit_cast(h8, load16_now(p.x + (size_t)min(m, p.M - 1) * p.K + k));
+            for (int m = 0; m < MR; m++) ptr[m] = p.x + (size_t)min(m, p.M - 1) * p.K + k;
+            LoadNow<MR + 1>::run(v, ptr);
+            kv = v[MR];
+#pragma unroll
+            for (int m = 0; m < MR; m++) xv[m] = __builtin_bit_cast(h8, v[m]);
+        } else {
+            const void *ptr[MR];
+            u4 v[MR];
+#pragma unroll
+            for (int m = 0; m < MR; m++) ptr[m] = p.x + (size_t)min(m, p.M - 1) * p.K + k;
+            LoadNow<MR>::run(v, ptr);
+#pragma unroll
+            for (int m = 0; m < MR; m++) xv[m] = __builtin_bit_cast(h8, v[m]);
+        }
         scatter8(k, kv, xv);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -277,16 +289,23 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     const int lb8 = (lane >> 2) & 7;
     // (a lane whose row lies past M supplies the last row again: row i of A only reaches result register i, and
     // the registers past M are never stored; one stride for all lanes keeps the block's offset an immediate)
-    const uint32_t x_base = (uint32_t)(min(row_i, p.M - 1) * span + 32 * h + 4 * lb8) * 2u;
+    uint32_t x_base[RS];
+#pragma unroll
+    for (int rs = 0; rs < RS; rs++) x_base[rs] = (uint32_t)(min(4 * rs + row_i, p.M - 1) * span + 32 * h + 4 * lb8) * 2u;
     constexpr uint32_t x_stride = 128u;
     const uint32_t xs_lane = zero_off + 64u + (uint32_t)(h * MR) * 8u;   // sums of half h of unit 0
 
     // x of a block: this lane's four positions of row row_i; read one block ahead of its use
-    auto load_x = [&](uint32_t sb, u2 &xv) { xv = *(const u2 *)(smem + x_base + x_stride * sb); };
-    f4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};  // two chains: a matrix instruction waits for the one it adds to
+    auto load_x = [&](uint32_t sb, u2 (&xv)[RS]) {
+#pragma unroll
+        for (int rs = 0; rs < RS; rs++) xv[rs] = *(const u2 *)(smem + x_base[rs] + x_stride * sb);
+    };
+    f4 c0[RS], c1[RS];  // two chains per set of rows: a matrix instruction waits for the one it adds to
+#pragma unroll
+    for (int rs = 0; rs < RS; rs++) c0[rs] = c1[rs] = (f4){0.f, 0.f, 0.f, 0.f};
     uint32_t szw = 0u;   // (scale, zero) word and sums of the unit in flight, read when the unit starts
     f2 xsv[MR];
-    auto block = [&](auto uu_c, int S, const uint32_t (&wr)[BITS], uint32_t sr, const u2 &xc, u2 &xn) {
+    auto block = [&](auto uu_c, int S, const uint32_t (&wr)[BITS], uint32_t sr, const u2 (&xc)[RS], u2 (&xn)[RS]) {
         constexpr int uu = decltype(uu_c)::value;                 // block inside its unit
         const uint32_t sb = (uint32_t)(S - S_wg);                  // block inside the workgroup's range (wave-uniform)
         if constexpr (uu == 0) {
@@ -303,32 +322,36 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
 #pragma unroll
         for (int j = 0; j < 4; j++) TileCodec<BITS>::operand(wr, j, q[j], mg);
         if constexpr (EXACT) tiled_dequant_exact<BITS>(q, szw);
-        if constexpr (uu == 0) {
-            c0 = (f4){0.f, 0.f, 0.f, 0.f};
-            c1 = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int rs = 0; rs < RS; rs++) {
+            if constexpr (uu == 0) {
+                c0[rs] = (f4){0.f, 0.f, 0.f, 0.f};
+                c1[rs] = (f4){0.f, 0.f, 0.f, 0.f};
+            }
+            const h4 xa = __builtin_bit_cast(h4, xc[rs]);
+            [&]<int... V>(std::integer_sequence<int, V...>) {
+                ((c0[rs] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa, __builtin_bit_cast(h4, (u2){q[V][0], q[V][1]}), c0[rs], 3, 2 * V, 0),
+                  c1[rs] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa, __builtin_bit_cast(h4, (u2){q[V][2], q[V][3]}), c1[rs], 3, 2 * V + 1, 0)),
+                 ...);
+            }(std::make_integer_sequence<int, 4>{});
         }
-        const h4 xa = __builtin_bit_cast(h4, xc);
-        [&]<int... V>(std::integer_sequence<int, V...>) {
-            ((c0 = __builtin_amdgcn_mfma_f32_4x4x4f16(xa, __builtin_bit_cast(h4, (u2){q[V][0], q[V][1]}), c0, 3, 2 * V, 0),
-              c1 = __builtin_amdgcn_mfma_f32_4x4x4f16(xa, __builtin_bit_cast(h4, (u2){q[V][2], q[V][3]}), c1, 3, 2 * V + 1, 0)),
-             ...);
-        }(std::make_integer_sequence<int, 4>{});
         if constexpr (uu == E - 1) {
             if constexpr (EXACT) {
 #pragma unroll
-                for (int m = 0; m < MR; m++) ysum[m] += c0[m] + c1[m];
+                for (int m = 0; m < MR; m++) ysum[m] += c0[m / 4][m % 4] + c1[m / 4][m % 4];
             } else {
                 const h2 e = as_h2(szw);
                 const float sc = (float)e[0], zp = (float)e[1];
 #pragma unroll
-                for (int m = 0; m < MR; m++) ysum[m] += sc * (((c0[m] + c1[m]) - xsv[m][1]) - zp * xsv[m][0]);
+                for (int m = 0; m < MR; m++)
+                    ysum[m] += sc * (((c0[m / 4][m % 4] + c1[m / 4][m % 4]) - xsv[m][1]) - zp * xsv[m][0]);
             }
         }
     };
 
     // Chunks of PF blocks, NCH in flight; x rides one block ahead in two register sets.  Blocks past the end
     // of K inside a wave's range are harmless (their x and sums are zeros), blocks past the range are skipped.
-    u2 xr[2];
+    u2 xr[2][RS];
     load_x((uint32_t)(S_begin - S_wg), xr[0]);
     auto chunk = [&](int c, uint32_t (&wc)[PF][BITS], const uint32_t (&sc)[UPC], auto all_c) {
         constexpr bool ALL = decltype(all_c)::value;
@@ -422,7 +445,9 @@ static int launch_decode_kw(const DecodeParams &p, const gptq_hip_plan &plan, hi
     switch (plan.waves_k) {
         case 4: return launch_decode_one<BITS, MR, 4, E>(p, plan, stream);
         case 8: return launch_decode_one<BITS, MR, 8, E>(p, plan, stream);
-        case 16: return launch_decode_one<BITS, MR, 16, E>(p, plan, stream);
+        case 16:
+            if constexpr (MR == 8) return GPTQ_HIP_ERR_UNSUPPORTED;   // (128 registers per lane do not hold two sets of rows)
+            else return launch_decode_one<BITS, MR, 16, E>(p, plan, stream);
         default: return GPTQ_HIP_ERR_UNSUPPORTED;
     }
 }
@@ -465,15 +490,19 @@ int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, co
     GPTQ_DECODE_CASE(4, 1);
     GPTQ_DECODE_CASE(4, 2);
     GPTQ_DECODE_CASE(4, 4);
+    GPTQ_DECODE_CASE(4, 8);
     GPTQ_DECODE_CASE(3, 1);
     GPTQ_DECODE_CASE(3, 2);
     GPTQ_DECODE_CASE(3, 4);
+    GPTQ_DECODE_CASE(3, 8);
     GPTQ_DECODE_CASE(2, 1);
     GPTQ_DECODE_CASE(2, 2);
     GPTQ_DECODE_CASE(2, 4);
+    GPTQ_DECODE_CASE(2, 8);
     GPTQ_DECODE_CASE(8, 1);
     GPTQ_DECODE_CASE(8, 2);
     GPTQ_DECODE_CASE(8, 4);
+    GPTQ_DECODE_CASE(8, 8);
 #undef GPTQ_DECODE_CASE
     if (rc != GPTQ_HIP_OK) return rc;
     if (plan.split_k > 1) {

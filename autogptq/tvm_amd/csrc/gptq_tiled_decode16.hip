@@ -85,21 +85,32 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
         }
     };
     // Long layers: the channels past the register pass, a pass at a time, before the weights are asked for (a wait
-    // for a load waits for every older one).  Each load is issued and waited for inside one asm statement: with
+    // for a load waits for every older one).  The loads of a pass are issued together and waited for inside one asm statement: with
     // ordinary loads in a loop behind the weight requests the compiler put a wait for every outstanding load, the
     // weights included, in front of the barrier, the sums and the walk of every layer.
-    auto load16_now = [](const void *ptr) {
-        u4 v;
-        asm volatile("global_load_dwordx4 %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(ptr) : "memory");
-        return v;
-    };
     for (int k8 = tid + NT; k8 < k8_hi; k8 += NT) {
         const int k = 8 * k8;
         u4 kv = {0u, 0u, 0u, 0u};
-        if (p.kinv) kv = load16_now(p.kinv + k);
         h8 xv[MR];
+        if (p.kinv) {   // the map and the rows of x, requested together
+            const void *ptr[MR + 1];
+            u4 v[MR + 1];
+            ptr[MR] = p.kinv + k;
 #pragma unroll
-        for (int m = 0; m < MR; m++) xv[m] = __builtin_bit_cast(h8, load16_now(p.x + (size_t)min(m, p.M - 1) * p.K + k));
+            for (int m = 0; m < MR; m++) ptr[m] = p.x + (size_t)min(m, p.M - 1) * p.K + k;
+            LoadNow<MR + 1>::run(v, ptr);
+            kv = v[MR];
+#pragma unroll
+            for (int m = 0; m < MR; m++) xv[m] = __builtin_bit_cast(h8, v[m]);
+        } else {
+            const void *ptr[MR];
+            u4 v[MR];
+#pragma unroll
+            for (int m = 0; m < MR; m++) ptr[m] = p.x + (size_t)min(m, p.M - 1) * p.K + k;
+            LoadNow<MR>::run(v, ptr);
+#pragma unroll
+            for (int m = 0; m < MR; m++) xv[m] = __builtin_bit_cast(h8, v[m]);
+        }
         scatter8(k, kv, xv);
     }
     __builtin_amdgcn_sched_barrier(0);

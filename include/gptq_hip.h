@@ -48,9 +48,9 @@ enum {
                                    tiles: chosen for several row blocks) per workgroup of waves_k = 4 waves along K
                                    (k_chunk = blocks of 64 channels per wave); x is pre-packed into the
                                    workspace; split_k > 1 adds a reduce launch */
-    GPTQ_HIP_KERNEL_TILED_DECODE = 5 /* the same layer for M <= 4 rows, x staged in LDS in the layer's sorted order,
+    GPTQ_HIP_KERNEL_TILED_DECODE = 5 /* the same layer for M <= 8 rows, x staged in LDS in the layer's sorted order,
                                    scales applied per 32 or 64 channels; row_tiles = the rows the kernel is built
-                                   for (1, 2 or 4).  waves_n = 1: a workgroup per 32 columns, waves_k (4, 8 or 16)
+                                   for (1, 2, 4 or 8; 8 with waves_n = 1 and at most 8 waves only).  waves_n = 1: a workgroup per 32 columns, waves_k (4, 8 or 16)
                                    waves along K with k_chunk blocks of 64 channels each; split_k > 1 (an x that
                                    does not fit LDS) adds a reduce launch.  waves_n = 2: units of 16 columns dealt
                                    out evenly over grid_x workgroups of 16 waves, all of K staged per workgroup
@@ -216,8 +216,8 @@ int gptq_hip_tile_prepare(const int32_t *qweight, const int32_t *qzeros, const v
  * tile table per M bucket (pycuda_warpper.py:77-127,150-189). */
 int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan);
 
-/* The plan of the family's decode kernel (GPTQ_HIP_KERNEL_TILED_DECODE), M <= 4 rows (GPTQ_HIP_ERR_UNSUPPORTED
- * above); gptq_hip_select_tiled chooses it by itself for those row counts and the matmul kernel above.  No counterpart in the reference, whose
+/* The plan of the family's decode kernel (GPTQ_HIP_KERNEL_TILED_DECODE), M <= 8 rows (GPTQ_HIP_ERR_UNSUPPORTED
+ * above); gptq_hip_select_tiled chooses it by itself up to 4 rows, and up to 8 for K <= 11008, the matmul kernel above.  No counterpart in the reference, whose
  * GEMV handler takes one row (pycuda_warpper.py:150-152).  Plans with halved tiles carry
  * GPTQ_HIP_PLAN_PRIVATE_ZERO_WORKSPACE. */
 int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan);
@@ -226,7 +226,7 @@ int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int group_size, 
  * y = x @ W (+ bias) on a layer in the tiled format, any M; replaces the same handler call as gptq_hip_gemm
  * (pycuda_warpper.py:138, qlinear_tvm.py:123,150).  x and y are in the layer's own channel order (xsrc = kinv =
  * NULL means no activation order; pass both or neither).  plan: NULL = gptq_hip_select_tiled.  workspace:
- * plan.workspace_bytes (none for most decode plans).  M <= 4: one launch (the decode kernel); above: two
+ * plan.workspace_bytes (none for most decode plans).  Decode plans: one launch; matmul plans: two
  * (pack pass, matmul); one more when the plan splits K.  A plan whose flags hold
  * GPTQ_HIP_PLAN_PRIVATE_ZERO_WORKSPACE wants ALL bytes of its workspace zero at the first call and leaves them zero
  * (the two halves of a tile that is halved along K meet in 64-bit slots behind the counters): give such plans a

@@ -291,11 +291,13 @@ def test_tiled_plans_are_consistent(bits, KN):
     K, N = KN
     gs = 128 if K % 128 == 0 else 32
     blocks = -(-K // 64)
-    for M in (1, 2, 4, 5, 16, 17, 128, 129, 1024):
+    for M in (1, 2, 4, 5, 8, 9, 16, 17, 128, 129, 1024):
         p = _lib.select_tiled(M, K, N, bits, gs)
         assert p.lds_bytes <= 160 * 1024 and p.block in (256, 512, 1024) and p.split_k == p.grid_y >= 1
-        if M <= 4:
+        if M <= 4 or (M <= 8 and K <= 11008):
             assert p.kernel == _lib.KERNEL_TILED_DECODE and p.row_tiles >= M
+            if M > 4:                # five to eight rows: the workgroup-per-tile kernel only, at most eight waves
+                assert p.row_tiles == 8 and p.waves_n == 1 and p.waves_k in (4, 8)
             if p.waves_n == 2:       # a workgroup per CU, 16-column units, sixteen waves over the 128-position blocks
                 assert p.block == 1024 and 1 <= p.grid_x <= min(N // 16, 256) and p.k_chunk * 16 >= -(-blocks // 2)
             else:                    # a workgroup per 32-column tile
@@ -334,7 +336,9 @@ def test_tiled_plans_reject_what_the_format_does_not_cover():
             _lib.select_tiled(*args)
         assert e.value.status == status, args
     with pytest.raises(_lib.GptqHipError):
-        _lib.select_tiled(5, 4096, 4096, 8, 128, decode=True)             # the decode kernels take up to four rows
+        _lib.select_tiled(9, 4096, 4096, 8, 128, decode=True)             # the decode kernels take up to eight rows
+    p8 = _lib.select_tiled(5, 4096, 4096, 8, 128, decode=True)            # five to eight: the workgroup-per-tile kernel, two row sets
+    assert p8.kernel == _lib.KERNEL_TILED_DECODE and p8.row_tiles == 8 and p8.waves_n == 1 and p8.waves_k in (4, 8)
     assert _lib.lib().gptq_hip_tiled_bytes(4096, 4096, 5) == 0
 
 
@@ -374,6 +378,8 @@ def table_tiled_wins(M, K, N, act_order, bits, one_group):
         if M <= 2:
             return True
         return K <= 6656 or (K <= 11008 and N <= 8192)
+    if M <= 8 and K <= 11008:
+        return True
     if M <= 16:
         return (not act_order) and K <= 4096 and N > 4096 and (M >= 9 or bits == 4)
     if M <= 128:

@@ -207,8 +207,8 @@ def test_tiled_integer_exact_and_guard_bands(dev):
 
 def test_tiled_rejections(dev):
     lib = _lib.lib()
-    with pytest.raises(_lib.GptqHipError):       # the decode kernel takes up to four rows
-        _lib.select_tiled(5, 4096, 352, 4, 128, decode=True)
+    with pytest.raises(_lib.GptqHipError):       # the decode kernel takes up to eight rows
+        _lib.select_tiled(9, 4096, 352, 4, 128, decode=True)
     fake, null = ctypes.c_void_p(0x1000), ctypes.c_void_p(None)
     # no workspace; groups that are not whole 32-channel lane blocks; a plan of another family
     assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, null, fake, null, 0, 40, 4096, 352, 4, 128, None, null) == _lib.ERR_WORKSPACE
@@ -466,12 +466,12 @@ def test_quantlinear_routes_prompt_sizes_to_the_tiled_copy(dev, bits, desc_act):
     q = module_of(L, dev)
     assert q._tiled is None
     x = L["x"].to(dev)
-    y8 = q(x[:8])                                  # 5..16 rows stay on the checkpoint layout (or its sorted copy)
+    y12 = q(x[:12])                                # 9..16 rows stay on the checkpoint layout (or its sorted copy)
     assert q._tiled is None
-    y40, y150, y2 = q(x[:40]), q(x), q(x[:2])      # prompt sizes, and a narrow layer's decode sizes
+    y40, y150, y2, y8 = q(x[:40]), q(x), q(x[:2]), q(x[:8])   # prompt sizes, and the decode sizes (up to eight rows)
     assert q._tiled is not None and q._tiled[1] is not None
     want = expected_output(L)
-    for y, M in ((y2, 2), (y8, 8), (y40, 40), (y150, 150)):
+    for y, M in ((y2, 2), (y8, 8), (y12, 12), (y40, 40), (y150, 150)):
         assert_close(y, want[:M], f"module, {M} rows")
         assert_tight(y, want[:M], f"module, {M} rows")
     # the same numbers (to the tight bound) from the checkpoint's own tensors
@@ -609,3 +609,23 @@ def test_quantlinear_takes_the_route_the_library_names(dev, bits, K, N, gs, desc
     q._g_state = None
     after = q(x)
     assert not torch.equal(before, after)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
+@pytest.mark.parametrize("K,N,gs", [(32, 32, 32), (160, 96, -1), (384, 64, 64), (1024, 416, 32), (2048, 1056, 256),
+                                    (4096, 352, 128), (11008, 256, 128), (4096, 11008, 128)])
+@pytest.mark.parametrize("M", [5, 6, 8])
+def test_tiled_decode_five_to_eight_rows(dev, bits, K, N, gs, M):
+    """The decode kernel with two sets of four rows (5 to 8 rows): against the oracle to the contract's bound and the
+    tight one, twice with equal results, with and without an activation order, halved tiles and long K included."""
+    for desc_act in (False, True):
+        L = layer(1700 + K + M, K, N, bits, gs, desc_act, M=M, bias=(M % 2 == 0))
+        D = to_dev(L, dev)
+        plan = _lib.select_tiled(M, K, N, bits, gs, decode=True)
+        assert plan.kernel == _lib.KERNEL_TILED_DECODE and plan.row_tiles == 8 and plan.waves_k in (4, 8)
+        prep = prepare(D)
+        want = expected_output(L)
+        y = run_tiled(D, prep, plan=plan)
+        assert_close(y, want, f"decode, two row sets: bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
+        assert_tight(y, want, f"decode, two row sets: bits={bits} K={K} N={N} gs={gs} M={M} act={desc_act}")
+        assert torch.equal(y, run_tiled(D, prep, plan=plan)), "two identical calls differ"

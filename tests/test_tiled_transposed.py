@@ -124,7 +124,7 @@ def test_transposed_integer_exact_guard_bands_and_rejections(dev):
     assert lib.gptq_hip_gemm_tiled_transposed(fake, fake, fake, null, fake, null, 0, 40, 4096, 352, 4, 128, None, null) == _lib.ERR_WORKSPACE
     assert lib.gptq_hip_gemm_tiled_transposed(fake, fake, fake, null, fake, fake, 1 << 24, 8, 4096, 352, 4, 16, None, null) == _lib.ERR_UNSUPPORTED
     assert lib.gptq_hip_gemm_tiled_transposed(fake, fake, fake, null, null, fake, 1 << 24, 8, 4096, 352, 4, 128, None, null) == _lib.ERR_BAD_ARG
-    p = _lib.select_tiled(8, 4096, 352, 4, 128)    # a plan of the forward product: its grid is not this product's
+    p = _lib.select_tiled(17, 4096, 352, 4, 128)   # a plan of the forward product (matmul kernel): its grid is not this product's
     assert lib.gptq_hip_gemm_tiled_transposed(fake, fake, fake, null, fake, fake, 1 << 24, 8, 4096, 352, 4, 128, ctypes.byref(p),
                                               null) == _lib.ERR_BAD_ARG
     assert lib.gptq_hip_tile_prepare_transposed(fake, fake, fake, null, null, fake, 4096, 352, 4, 128, null) == _lib.ERR_BAD_ARG
