@@ -10,9 +10,10 @@ HEADERS = ["gptq_unpack.h", "gptq_internal.h", "gptq_device.h", "gptq_tiled_comm
            "binding.cpp"]   # (hashed with the rest: both libraries carry one build id)
 # Compiler options of single sources.  The decode kernels keep the four result registers of their small matrix
 # instructions in ordinary vector registers: left to itself the compiler puts them into accumulation registers
-# for the workgroups of four waves and copies them back for every epilogue.
+# for the workgroups of four waves and copies them back for every epilogue.  The same kernels take their first sixteen
+# dwords of arguments preloaded into scalar registers.
 EXTRA_FLAGS = {
-    "gptq_tiled_decode.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "gptq_tiled_decode.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form", "-mllvm", "-amdgpu-kernarg-preload-count=16"],
 }
 
 

@@ -47,13 +47,38 @@ struct DecodeParams {
     int lb_per_group;       // group_size / 32
     uint32_t lbg_magic;     // lane block -> group: umulhi(lb, magic) + (add ? lb : 0)
     int lbg_add;
+    int grid_x, grid_y;     // the launch's grid (from here: the dispatch packet is one more cold line to read)
+};
+
+// Everything the kernel needs before its results are stored travels as its first fourteen dwords of arguments,
+// which the dispatcher hands over in scalar registers (this source is built with kernel-argument preloading; fourteen
+// is what the user registers leave room for): a wave otherwise begins by waiting ~0.4 us for its argument segment to
+// arrive from memory.  Hence the packing: M and the blocks per wave in one word, the group arithmetic's flag and the
+// number of K ranges in another, and what follows from these (N = 32 tiles, blocks = ceil(K / 64), the number of
+// groups) worked out in the kernel.  The pointers of the epilogue follow as a struct, read while the walk runs.
+struct DecodeTail {
+    const void *bias;
+    void *y;
+    float *partial;
+    unsigned long long *slots;
 };
 
 // E: blocks of 64 positions that share one epilogue (1, or 2 when the groups are multiples of 128 channels and
 // every wave has an even number of blocks: both lane blocks of both blocks then lie in one group).
 template <int BITS, int MR, int KW, int E>
-__global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParams p)
+__global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const _Float16 *a_x, const uint16_t *a_kinv, const char *a_qtile,
+                                                               const uint32_t *a_sz, int a_K, uint32_t a_m_steps, int a_T_total,
+                                                               int a_grid_x, uint32_t a_lbg_magic, uint32_t a_flags,
+                                                               const DecodeTail t)
 {
+    DecodeParams p;
+    p.x = a_x, p.kinv = a_kinv, p.qtile = a_qtile, p.sz = a_sz;
+    p.K = a_K, p.M = (int)(a_m_steps & 0xffu), p.wave_steps = (int)(a_m_steps >> 8);
+    p.T_total = a_T_total, p.N = 32 * a_T_total, p.S_total = (a_K + 63) >> 6, p.grid_x = a_grid_x;
+    p.lbg_magic = a_lbg_magic, p.lbg_add = (int)(a_flags & 1u), p.split_k = (int)(a_flags >> 1), p.grid_y = p.split_k;
+    // groups = (K / 32) / (lane blocks per group), by the same multiply-high that maps a lane block to its group
+    p.G = (int)(__umulhi((uint32_t)a_K >> 5, a_lbg_magic) + (p.lbg_add ? (uint32_t)a_K >> 5 : 0u));
+    p.bias = t.bias, p.y = t.y, p.partial = t.partial, p.slots = t.slots;
     static_assert((MR == 1 || MR == 2 || MR == 4 || MR == 8) && (E == 1 || E == 2), "one or two sets of four rows");
     constexpr int RS = (MR + 3) / 4;   // sets of four rows: a matrix instruction takes four rows of x
     constexpr bool EXACT = tiled_decode_exact(BITS);
@@ -77,7 +102,7 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
     // them half a tile, so that the fullest CU holds half a tile more than the others instead of a whole one
     // (two whole tiles on 88 of the 256 CUs bound both the memory and the instruction path of 11008 columns).
     // The two halves of a tile meet through one 64-bit exchange per output (see the end of the kernel).
-    const int n_halved = (int)gridDim.x - p.T_total;     // e (0: no tile is halved)
+    const int n_halved = p.grid_x - p.T_total;           // e (0: no tile is halved)
     const int n_whole = p.T_total - n_halved;
     const bool is_half = (int)blockIdx.x >= n_whole;
     const int half_i = (int)blockIdx.x - n_whole;        // (halved tile, half) = (half_i / 2, half_i % 2)
@@ -119,7 +144,7 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const DecodeParam
         for (int m = 0; m < MR; m++) xq[ps][m] = *(const h8 *)(p.x + (size_t)min(m, p.M - 1) * p.K + k);
     }
     // (a workgroup with a part of K, a half tile or one of several ranges, keeps the channels of its own range)
-    const bool ranged = is_half || gridDim.y > 1;
+    const bool ranged = is_half || p.grid_y > 1;
     auto scatter8 = [&](int k, const u4 &kv, const h8 (&xv)[MR]) {
         if (!p.kinv) {   // no activation order: the eight channels are eight consecutive positions, one store
             // (k8_lo .. k8_hi is the workgroup's own range here, a multiple of 8 away from p0)
@@ -435,7 +460,12 @@ static int launch_decode_one(const DecodeParams &p, const gptq_hip_plan &plan, h
             return GPTQ_HIP_ERR_LAUNCH;
         }
     }
-    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, 1), dim3(64 * KW), plan.lds_bytes, stream, p);
+    if (plan.split_k != plan.grid_y || p.M > 255 || p.wave_steps >= (1 << 24)) return GPTQ_HIP_ERR_BAD_ARG;
+    DecodeTail t;
+    t.bias = p.bias, t.y = p.y, t.partial = p.partial, t.slots = p.slots;
+    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, 1), dim3(64 * KW), plan.lds_bytes, stream, p.x, p.kinv, p.qtile, p.sz,
+                       p.K, (uint32_t)p.M | ((uint32_t)p.wave_steps << 8), p.T_total, plan.grid_x, p.lbg_magic,
+                       (uint32_t)p.lbg_add | ((uint32_t)p.split_k << 1), t);
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 
@@ -480,6 +510,11 @@ int launch_tiled_decode(const void *x, const void *qtile, const uint32_t *sz, co
     // lane block -> group as a multiply-high (lane blocks are below 2^16 / 32 * 2)
     p.lbg_add = p.lb_per_group == 1;
     p.lbg_magic = p.lbg_add ? 0u : (uint32_t)((1ull << 32) / (uint32_t)p.lb_per_group) + 1u;
+    {   // the kernel works the number of groups and of columns out from what it is handed: they must come out as given
+        const uint32_t lbs = (uint32_t)K >> 5;
+        const uint32_t groups = (uint32_t)(((unsigned long long)lbs * p.lbg_magic) >> 32) + (p.lbg_add ? lbs : 0u);
+        if ((int)groups != G || N % 32 != 0) return GPTQ_HIP_ERR_UNSUPPORTED;
+    }
     const int mr = tiled_decode_rows(M);
     int rc = GPTQ_HIP_ERR_UNSUPPORTED;
     // two blocks per epilogue where every unit of two blocks lies in one group
