@@ -14,6 +14,7 @@ HEADERS = ["gptq_unpack.h", "gptq_internal.h", "gptq_device.h", "gptq_tiled_comm
 # dwords of arguments preloaded into scalar registers.
 EXTRA_FLAGS = {
     "gptq_tiled_decode.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form", "-mllvm", "-amdgpu-kernarg-preload-count=16"],
+    "gptq_tiled_decode16.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
 }
 
 

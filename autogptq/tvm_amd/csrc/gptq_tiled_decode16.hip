@@ -33,11 +33,25 @@ struct Decode16Params {
     int lb_per_group;       // group_size / 32
     uint32_t lbg_magic;     // lane block (32 positions) -> group: umulhi(lb, magic) + (add ? lb : 0)
     int lbg_add;
+    int grid_x;             // workgroups of the launch
 };
 
+// The arguments arrive as fourteen dwords that the dispatcher preloads into scalar registers (this source is built
+// with kernel-argument preloading), so that a wave does not begin by waiting ~0.4 us for its argument segment: the
+// four input pointers, K, N, one word of (M, the group arithmetic's flag, the grid), the multiplier of the group
+// arithmetic, and y.  What follows from these (blocks, tiles, units, groups) is worked out here; the bias pointer,
+// needed at the very end, follows in memory.
 template <int BITS, int MR, bool G128, bool CONTIG>
-__global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Params p)
+__global__ __launch_bounds__(1024) void tiled_decode16_kernel(const _Float16 *a_x, const uint16_t *a_kinv, const char *a_qtile,
+                                                              const uint32_t *a_sz, int a_K, int a_N, uint32_t a_packed,
+                                                              uint32_t a_lbg_magic, void *a_y, const void *a_bias)
 {
+    Decode16Params p;
+    p.x = a_x, p.kinv = a_kinv, p.qtile = a_qtile, p.sz = a_sz, p.y = a_y, p.bias = a_bias;
+    p.K = a_K, p.N = a_N, p.M = (int)(a_packed & 0xffu), p.lbg_add = (int)((a_packed >> 8) & 1u), p.grid_x = (int)(a_packed >> 9);
+    p.lbg_magic = a_lbg_magic;
+    p.S_total = (a_K + 63) >> 6, p.T_total = a_N >> 5, p.V_total = (p.S_total + 1) >> 1, p.units = a_N >> 4;
+    p.G = (int)(__umulhi((uint32_t)a_K >> 5, a_lbg_magic) + (p.lbg_add ? (uint32_t)a_K >> 5 : 0u));
     static_assert(MR <= 4, "one matrix instruction set per lane block");
     constexpr bool EXACT = tiled_decode_exact(BITS);
     constexpr int NT = 1024, NW = 16;
@@ -46,8 +60,9 @@ __global__ __launch_bounds__(1024) void tiled_decode16_kernel(const Decode16Para
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n16 = lane & 15, lbv = lane >> 4;
-    const int u0 = (int)(((long long)p.units * blockIdx.x) / gridDim.x);
-    const int u1 = (int)(((long long)p.units * (blockIdx.x + 1)) / gridDim.x);
+    // (32-bit: units <= 2^16 and at most 2^15 workgroups, checked at launch; a 64-bit division is ~100 instructions)
+    const int u0 = (int)((uint32_t)p.units * blockIdx.x / (uint32_t)p.grid_x);
+    const int u1 = (int)((uint32_t)p.units * (blockIdx.x + 1u) / (uint32_t)p.grid_x);
     const int n_units = u1 - u0;
     const int span = p.V_total * 128;   // positions staged: all of K, padded to whole virtual blocks
     const int S_last = p.S_total - 1;
@@ -358,7 +373,14 @@ static int launch_decode16_one(const Decode16Params &p, const gptq_hip_plan &pla
             return GPTQ_HIP_ERR_LAUNCH;
         }
     }
-    hipLaunchKernelGGL(kern, dim3(plan.grid_x), dim3(1024), plan.lds_bytes, stream, p);
+    {   // the kernel works the number of groups out from what it is handed: it must come out as given
+        const uint32_t lbs = (uint32_t)p.K >> 5;
+        const uint32_t groups = (uint32_t)(((unsigned long long)lbs * p.lbg_magic) >> 32) + (p.lbg_add ? lbs : 0u);
+        if ((int)groups != p.G || p.M > 255 || plan.grid_x < 1 || plan.grid_x >= (1 << 15) || p.units > (1 << 16))
+            return GPTQ_HIP_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(kern, dim3(plan.grid_x), dim3(1024), plan.lds_bytes, stream, p.x, p.kinv, p.qtile, p.sz, p.K, p.N,
+                       (uint32_t)p.M | ((uint32_t)p.lbg_add << 8) | ((uint32_t)plan.grid_x << 9), p.lbg_magic, p.y, p.bias);
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 
