@@ -15,6 +15,7 @@ HEADERS = ["gptq_unpack.h", "gptq_internal.h", "gptq_device.h", "gptq_tiled_comm
 EXTRA_FLAGS = {
     "gptq_tiled_decode.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form", "-mllvm", "-amdgpu-kernarg-preload-count=16"],
     "gptq_tiled_decode16.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+    "gptq_tiled.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
 }
 
 

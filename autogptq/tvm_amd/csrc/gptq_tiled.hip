@@ -286,9 +286,31 @@ __device__ __forceinline__ h8 tiled_bop_t(const uint32_t (&w)[BITS], int j, cons
 // (4096 x 11008, us with / without the pack pass: 8 rows 14.0 / 10.7, 16 rows 14.5 / 11.5; with 32 distinct rows
 // per load 14.8 / 16.2, 64 rows 19 / 29.5: every lane then asks for a line of its own), and only when K is a whole
 // number of blocks that the waves' ranges cover exactly: there is no zero padding to read.
+// What the kernel needs before its first requests go out arrives as fourteen dwords that the dispatcher preloads
+// into scalar registers (this source is built with kernel-argument preloading), so that a wave does not begin by
+// waiting ~0.4 us for its argument segment: the source of the A operand (the packed fragments, or x itself for
+// DIRECT), the weights, the (scale, zero) words, the extents, and the group arithmetic in one word.  The pointers of
+// the epilogue and the transposed product's tables follow in memory.
+struct TiledTail {
+    const void *bias;
+    void *y;
+    float *partial;
+    const uint32_t *szt;
+    const int32_t *out_map;
+    int split_k, tiles_per_group;
+};
+
 template <int BITS, int AT, int RW, int KW, int RING, int CT, bool TRANS = false, bool DIRECT = false>
-__global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const TiledParams p)
+__global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const char *a_src, const char *a_qtile, const uint32_t *a_sz,
+                                                                  int a_wave_steps, int a_S_total, int a_T_total, int a_rt_total,
+                                                                  int a_N, int a_M, int a_K, uint32_t a_groups, const TiledTail t)
 {
+    TiledParams p;
+    p.xpack = a_src, p.x = (const _Float16 *)a_src, p.qtile = a_qtile, p.sz = a_sz;
+    p.wave_steps = a_wave_steps, p.S_total = a_S_total, p.T_total = a_T_total, p.rt_total = a_rt_total;
+    p.N = a_N, p.M = a_M, p.K = a_K, p.lb_per_group = (int)(a_groups & 0xfffu), p.G = (int)(a_groups >> 12);
+    p.bias = t.bias, p.y = t.y, p.partial = t.partial, p.szt = t.szt, p.out_map = t.out_map;
+    p.split_k = t.split_k, p.tiles_per_group = t.tiles_per_group;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -586,6 +608,20 @@ int launch_tiled_reduce(const float *partial, const void *bias, void *y, int M, 
     return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
 }
 
+// the kernel's argument list from its parameter struct
+template <typename Kern>
+static int launch_gemm_kernel(Kern kern, dim3 grid, dim3 block, int lds_bytes, hipStream_t stream, const TiledParams &p,
+                              bool direct)
+{
+    if (p.lb_per_group < 0 || p.lb_per_group > 0xfff || p.G < 0 || p.G >= (1 << 20)) return GPTQ_HIP_ERR_UNSUPPORTED;
+    TiledTail t;
+    t.bias = p.bias, t.y = p.y, t.partial = p.partial, t.szt = p.szt, t.out_map = p.out_map;
+    t.split_k = p.split_k, t.tiles_per_group = p.tiles_per_group;
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, direct ? (const char *)p.x : p.xpack, p.qtile, p.sz, p.wave_steps,
+                       p.S_total, p.T_total, p.rt_total, p.N, p.M, p.K, (uint32_t)p.lb_per_group | ((uint32_t)p.G << 12), t);
+    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+}
+
 template <int BITS, int AT, int RW, int KW, int RING, int CT, bool DIRECT = false>
 static int launch_tiled_one(const TiledParams &p, const gptq_hip_plan &plan, hipStream_t stream)
 {
@@ -598,8 +634,7 @@ static int launch_tiled_one(const TiledParams &p, const gptq_hip_plan &plan, hip
             return GPTQ_HIP_ERR_LAUNCH;
         }
     }
-    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, plan.grid_z), dim3(64 * RW * KW), lds_bytes, stream, p);
-    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+    return launch_gemm_kernel(kern, dim3(plan.grid_x, plan.grid_y, plan.grid_z), dim3(64 * RW * KW), lds_bytes, stream, p, DIRECT);
 }
 
 // x is packed into the workspace, the matmul runs, and a reduce pass follows when K is split over workgroups.
@@ -804,8 +839,7 @@ static int launch_tiled_t_one(const TiledParams &p, const gptq_hip_plan &plan, h
             return GPTQ_HIP_ERR_LAUNCH;
         }
     }
-    hipLaunchKernelGGL(kern, dim3(plan.grid_x, plan.grid_y, plan.grid_z), dim3(256), plan.lds_bytes, stream, p);
-    return hipGetLastError() == hipSuccess ? GPTQ_HIP_OK : GPTQ_HIP_ERR_LAUNCH;
+    return launch_gemm_kernel(kern, dim3(plan.grid_x, plan.grid_y, plan.grid_z), dim3(256), plan.lds_bytes, stream, p, false);
 }
 
 // gy is packed into the workspace (as x is for the forward product), the matmul runs on the transposed copy, and a
@@ -835,6 +869,8 @@ int launch_tiled_t(const void *gy, const void *qtile_t, const uint32_t *szt, con
     p.szt = szt;
     p.out_map = xsrc;
     p.tiles_per_group = group_size / 32;
+    p.x = nullptr;           // (the forward product's direct read of x: not used here)
+    p.K = K;
     const int S_pack = tiled_pack_blocks(plan.split_k, plan.waves_k, plan.k_chunk);
     hipLaunchKernelGGL(tile_pack_x_kernel, dim3(32 * p.rt_total), dim3(256), 0, stream, (const _Float16 *)gy,
                        (const int32_t *)nullptr, xpack, M, N, Np, p.rt_total, S_pack);
