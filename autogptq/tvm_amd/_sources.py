@@ -16,6 +16,7 @@ EXTRA_FLAGS = {
     "gptq_tiled_decode.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form", "-mllvm", "-amdgpu-kernarg-preload-count=16"],
     "gptq_tiled_decode16.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
     "gptq_tiled.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+    "gptq_dequant.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
 }
 
 
