@@ -627,13 +627,23 @@ bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
         return K <= 6656 || (K <= 11008 && N <= 8192);
     }
     if (M <= 8 && K <= 11008) return true;   // the decode kernel with two sets of rows (below)
-    if (M <= 16) return !act_order && K <= 4096 && N > 4096 && (M >= 9 || bits == 4);
+    if (M <= 16) {
+        if (!act_order) return K <= 4096 && N > 4096 && (M >= 9 || bits == 4);
+        // with an activation order (9 to 16 rows; pack pass + matmul against the sorted copy, whose time grows with the
+        // rows): 4096 x 11008 from twelve rows (9 / 12 / 16 rows, int4: 13.5 / 13.5 / 13.5 against 13.1 / 13.8 / 14.6; int3
+        // 13.6 / 13.5 / 13.5 against 13.5 / 13.9 / 15.2), 3-bit layers of up to 4096 columns always (4096 x 4096: 12.3 / 12.4 /
+        // 12.4 against 13.0 / 13.2 / 13.8; 4-bit there stays on the checkpoint tensors: 12.7 against 11.1); 11008 x 4096 stays
+        // on the sorted copy (18.3-18.9 against 15.9-18.7)
+        return K <= 4096 && ((N > 4096 && M >= 12) || (bits == 3 && N <= 4096));
+    }
     if (M <= 128) {
         if (one_group && K > 8192 && (M > 32 || K > 16384 || N > 16384)) return false;
         if (M <= 64 && K >= 8192 && bits == 4 && !act_order) return false;
         return true;
     }
-    return K <= 8192;
+    // (3-bit 11008 x 4096 with an activation order at 256 rows: 46.5 against 51.2 on the checkpoint tensors; 4-bit 52.4
+    // against 48.5)
+    return K <= 8192 || (bits == 3 && K <= 11008 && M <= 256);
 }
 
 // The plan gptq_hip_gemm_sorted runs for M rows of a layer whose channels were sorted by group, if that path covers
