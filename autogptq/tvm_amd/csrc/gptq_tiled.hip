@@ -376,15 +376,21 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const char *a_
         ahead = ahead + 1 == ws_n ? 0 : ahead + 1;
         return S;
     };
-    // prologue, in consumption order
+    // prologue, in consumption order.  The weights of the whole ring are asked for here (they come from HBM); the A
+    // fragments of the first slot only: those of the other slots (L2, short latency) are asked for while the first
+    // block is multiplied (FIRST in block below).  With all of them in the prologue a wave spent 2.8 us putting sixty
+    // requests into a queue that drains at the memory's pace before its first matrix instruction.
+    // (The transposed product keeps the whole ring in its prologue.)
     int S_of[RING];   // the block each ring slot holds (TRANS: its table entries are looked up by block)
 #pragma unroll
     for (int u = 0; u < RING; u++) {
         const int S = next_block();
         S_of[u] = S;
         load_b(S, w[u], szr[u]);
+        if (TRANS || u == 0) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) load_a(S, j, a[u][j]);
+            for (int j = 0; j < 4; j++) load_a(S, j, a[u][j]);
+        }
     }
     __builtin_amdgcn_sched_barrier(0);
     // TRANS: the (scale, base + zero) pairs of the workgroup's K range for the groups of its CT tiles -> LDS,
@@ -447,9 +453,10 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const char *a_
     // One block of the walk (ring slot u): the 4 CT (j, ct) operands, each multiplied with the AT row tiles
     // while the next operand of the walk is dequantised.  REFILL: the slot's registers are requested again
     // for the block a ring ahead as soon as their last reader is done.
-    auto block = [&](auto u_c, auto refill_c) {
+    auto block = [&](auto u_c, auto refill_c, auto first_c) {
         constexpr int u = decltype(u_c)::value;
         constexpr bool REFILL = decltype(refill_c)::value;
+        constexpr bool FIRST = decltype(first_c)::value;   // the first block of the walk: asks for the other slots' A fragments
         const int S_refill = REFILL ? next_block() : 0;  // the block a ring ahead of this one in the walk
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -479,6 +486,12 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const char *a_
                 for (int rt = 0; rt < AT; rt++) {
                     acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[u][j][rt], bop, acc[rt][ct], 0, 0, 0);
                 }
+                if (FIRST && ct == CT - 1) {
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int s = 1; s < RING; s++) load_a(S_of[s], j, a[s][j]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 if (REFILL && ct == CT - 1) {
                     __builtin_amdgcn_sched_barrier(0);
                     if (j == 3) {
@@ -494,16 +507,34 @@ __global__ __launch_bounds__(64 * RW * KW) void tiled_gemm_kernel(const char *a_
     // whole turns of the ring, then what is left without refills (no load sits behind a branch, and the loop
     // has no early exit: an exit into its latch would make the compiler wait at the head of every turn for
     // almost every load in flight)
-    const int full = p.wave_steps / RING * RING;
-    for (int i0 = 0; i0 < full; i0 += RING) {
-        [&]<int... U>(std::integer_sequence<int, U...>) {
-            (block(std::integral_constant<int, U>{}, std::true_type{}), ...);
-        }(std::make_integer_sequence<int, RING>{});
-    }
-    {
+    if constexpr (TRANS) {
+        const int full = p.wave_steps / RING * RING;
+        for (int i0 = 0; i0 < full; i0 += RING) {
+            [&]<int... U>(std::integer_sequence<int, U...>) {
+                (block(std::integral_constant<int, U>{}, std::true_type{}, std::false_type{}), ...);
+            }(std::make_integer_sequence<int, RING>{});
+        }
         const int rem = p.wave_steps - full;
         [&]<int... U>(std::integer_sequence<int, U...>) {
-            ((U < RING - 1 && U < rem ? block(std::integral_constant<int, U>{}, std::false_type{}) : (void)0), ...);
+            ((U < RING - 1 && U < rem ? block(std::integral_constant<int, U>{}, std::false_type{}, std::false_type{}) : (void)0), ...);
+        }(std::make_integer_sequence<int, RING>{});
+    } else {
+        // the first block by itself (every wave has one; its refill wraps around inside the wave's range when the
+        // range is shorter than the ring, like every refill near the end of the walk), then whole turns of the ring
+        // that begin at slot 1, then the rest
+        block(std::integral_constant<int, 0>{}, std::true_type{}, std::true_type{});
+        const int left = p.wave_steps - 1;
+        const int full = left / RING * RING;
+        for (int i0 = 0; i0 < full; i0 += RING) {
+            [&]<int... U>(std::integer_sequence<int, U...>) {
+                (block(std::integral_constant<int, (U + 1) % RING>{}, std::true_type{}, std::false_type{}), ...);
+            }(std::make_integer_sequence<int, RING>{});
+        }
+        const int rem = left - full;
+        [&]<int... U>(std::integer_sequence<int, U...>) {
+            ((U < RING - 1 && U < rem ? block(std::integral_constant<int, (U + 1) % RING>{}, std::false_type{}, std::false_type{})
+                                      : (void)0),
+             ...);
         }(std::make_integer_sequence<int, RING>{});
     }
 
