@@ -161,14 +161,17 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const _Float16 *a
             }
             return;
         }
+        // a part of K: a channel outside the range goes to a slot of the lane's own in the area of the partial results,
+        // which is written again before it is read (no branch per channel: the waves of a half tile are the last of
+        // the kernel to finish, and this walk over all of x is what they do first)
+        const uint32_t dump = (uint32_t)(((const unsigned char *)red - smem) >> 1) + (uint32_t)lane;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             const int pos = (int)((kv[e >> 1] >> (16 * (e & 1))) & 0xffffu);
             const int pl = pos - p0;
-            if ((unsigned)pl < (unsigned)span) {
+            const bool mine = (unsigned)pl < (unsigned)span;
 #pragma unroll
-                for (int m = 0; m < MR; m++) xl[m * span + pl] = xv[m][e];
-            }
+            for (int m = 0; m < MR; m++) xl[mine ? (uint32_t)(m * span + pl) : dump] = xv[m][e];
         }
     };
     // Long layers: the channels the register passes do not hold, a pass at a time, before the weights are asked for
