@@ -444,13 +444,15 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
         if (mr == 8 && kw == 16) kw = 8;
         while (kw > 4 && kw > S_total) kw >>= 1;
         // K beyond 32768 channels with more tiles than CUs: cut over workgroups of eight waves so that a wave walks
-        // about eighteen blocks (36864 x 9216 int3, one group, one row: 34.6 us uncut with 72 blocks per wave, 31.4
-        // in two ranges, 28.8 in four, 29.7 in eight, the pass that adds the ranges included; up to 32768 channels
-        // every cut measured lost: 9216 x 9216 9.2 -> 11.8-13.3, 28672 x 8192 25.5 -> 29.1, 11008 x 11008 13.1 -> 16.1)
+        // about twelve blocks (36864 x 9216 int3, one group, one row, the pass that adds the ranges included: 34.6 us
+        // uncut with 72 blocks per wave, 31.4 in two ranges; with the current kernel 28.4 in three, 27.6 in four,
+        // 26.7 in six, 27.9 in nine, 29.1 in twelve; six ranges of four or sixteen waves 27.6 / 28.4; an odd number
+        // of blocks per wave loses the paired epilogue: eight ranges 29.9.  Up to 32768 channels every cut measured
+        // lost: 9216 x 9216 9.2 -> 11.8-13.3, 28672 x 8192 25.5 -> 29.1, 11008 x 11008 13.1 -> 16.1)
         int first_split = 1;
         if (S_total > 512 && !halves_all) {
             kw = 8;
-            first_split = ceil_div(S_total, 8 * 18);
+            first_split = ceil_div(S_total, 8 * 12);
         }
         for (int split = first_split; split <= S_total; split++) {
             int wave_steps = ceil_div(S_total, split * kw);
@@ -600,7 +602,7 @@ namespace {
 //     8.1 / 11.0 / 11.1, int3 7.3 / 7.7 / 9.7 against 7.7 / 10.2 / 10.3; 4096 x 22016 one row 9.7 / 10.3 against
 //     11.4 / 12.8).  Longer K, one and two rows: always (8192 x 8192 9.7 / 9.9 against 14.0 / 13.3, 8192 x 28672
 //     24.6 / 26.4 against 32.3 / 30.2, 28672 x 8192 25.1 / 31.7 against 50.1 / 39.2; 36864 x 9216 int3 with one
-//     group, K cut in four ranges: 28.8 against 37.3); three and four rows: K up to 6656, and
+//     group, K cut in six ranges: 26.7 against 37.3); three and four rows: K up to 6656, and
 //     up to 11008 for layers of up to 8192 columns (beyond, the four staged rows of x cost more than they save:
 //     8192 x 28672 41.9 against 30.4);
 //   * 5 to 8 rows, K up to 11008: the decode kernel with two sets of four rows (5 / 8 rows, int4 / int3, against the
