@@ -405,11 +405,17 @@ __global__ __launch_bounds__(64 * KW) void tiled_decode_kernel(const _Float16 *a
 #pragma unroll
         for (int j = 0; j < NCH; j++) chunk(c + j * PF, w[j], szr[j], std::true_type{});
     } else {
-        // less than two rings left: the blocks in flight, then the rest, requested as registers come free
+        // less than two rings left: the blocks in flight, then the rest, requested as registers come free.  No load
+        // stands behind a test (the compiler would no longer know how many are outstanding, and wait for all of them
+        // at every chunk): a chunk past the end of the range asks for the range's last chunk again, which the
+        // cache has, and is not multiplied.
+        const int last_chunk = max((ws - 1) / PF * PF, 0);
 #pragma unroll
         for (int j = 0; j < NCH; j++) {
             chunk(c + j * PF, w[j], szr[j], std::false_type{});
-            if (c + RING + j * PF < ws) load_chunk(c + RING + j * PF, w[j], szr[j]);
+            __builtin_amdgcn_sched_barrier(0);
+            load_chunk(min(c + RING + j * PF, last_chunk), w[j], szr[j]);
+            __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int j = 0; j < NCH; j++) chunk(c + RING + j * PF, w[j], szr[j], std::false_type{});
