@@ -527,6 +527,19 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     if ((long long)M * N >= (1LL << 32)) split = 1;  // indexing of the pass that adds the partial tiles
     // every wave gets at least a ring of blocks
     while (split > 1 && S_total / (split * kwv) < gptq::tiled_ring(at)) split--;
+    // One row tile (up to 32 rows): two such workgroups share a CU, and where K is cut anyway (the pass that adds the
+    // ranges is there already) and long, finer ranges that still leave every wave two turns of its ring put up to
+    // ~480 workgroups on the chip at once instead of ~256 (us at 32 rows, int3, one group, 144 column pairs: 9216 x
+    // 9216 in 2 / 3 / 4 / 6 ranges 26.2 / 22.4 / 24.6 / 24.4; 36864 x 9216 in 2 / 3 / 4 / 6 / 8 / 12: 75.5 / 58.7 /
+    // 64.1 / 60.8 / 60.6 / 60.7: the fourth range is the 577th workgroup, which waits for a CU).  Where K is not cut,
+    // cutting it costs more than it brings (4096 x 11008, 16 rows: 13.4 -> 19.1 in two ranges).
+    if (at == 1 && m_blocks == 1 && split >= 2 && (long long)M * N < (1LL << 32)) {
+        int finer = (int)(480 / tiles);
+        const int two_turns = S_total / (kwv * 2 * gptq::tiled_ring(at));
+        if (finer > two_turns) finer = two_turns;
+        if (finer > cap) finer = cap;
+        if (finer > split) split = finer;
+    }
     const int wave_steps = ceil_div(S_total, split * kwv);
     split = ceil_div(S_total, wave_steps * kwv);
     plan->kernel = GPTQ_HIP_KERNEL_TILED;
@@ -616,8 +629,14 @@ namespace {
 //   * 17 to 128 rows: almost everywhere (4096 x 11008 with an activation order, 32 / 64 / 128 rows: 14.8 / 19.2 /
 //     26.6 against 18.1 / 22.1 / 34.1), but for K of 8192 and more where the checkpoint-layout STREAM kernel has
 //     nothing to look up per weight: 4-bit layers without an activation order up to 64 rows (8192 x 8192, 17 / 64
-//     rows: 23.4 / 28.6 against 19.7 / 25.0) and layers of one group (9216 x 36864, 32 / 128 rows: 61.9 / 134 against
-//     54.6 / 126; 36864 x 9216 86.7 / 206 against 72.8 / 173; 9216 x 9216 keeps the tiled copy up to 32 rows);
+//     rows: 23.4 / 28.6 against 19.7 / 25.0; 28672 x 8192, 17 / 32 rows: 52.5 / 53.1 against 43.3 / 43.7) and layers of
+//     one group beyond 32 rows or 16384 columns (9216 x 36864, 32 / 128 rows: 53.4 / 134 against 52.9 / 126; 36864 x
+//     9216 at 128 rows 206 against 173; up to 32 rows and 16384 columns they keep the tiled copy, whose K ranges are
+//     cut finer there: 36864 x 9216, 17 / 32 rows: 57.1 / 57.6 against 70.2 / 72.4, 18432 x 9216 33.2 / 33.8 against
+//     45.0 / 45.9, 9216 x 9216 21.6 / 22.0 against 31.4 / 32.0, 12288 x 12288 level at 28); with an activation order, up
+//     to 32 rows of layers beyond 20480 channels (28672 x 8192 at 32 rows, int4 / int3: 58.3 / 55.9 against 48.3 /
+//     49.8; 17920 x 6656 33.9 / 34.5 against 34.1 / 38.9 stays; from 64 rows the tiled copy wins there too: 60.1 / 63.0
+//     against 63.0 / 67.2);
 //   * above 128 rows: K up to 8192 (4096 x 11008, 512 rows: 75 against 95; 11008 x 4096: 127 against 81).
 bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
 {
@@ -639,8 +658,9 @@ bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
         return K <= 4096 && ((N > 4096 && M >= 12) || (bits == 3 && N <= 4096));
     }
     if (M <= 128) {
-        if (one_group && K > 8192 && (M > 32 || K > 16384 || N > 16384)) return false;
+        if (one_group && K > 8192 && (M > 32 || N > 16384)) return false;
         if (M <= 64 && K >= 8192 && bits == 4 && !act_order) return false;
+        if (M <= 32 && K > 20480 && act_order) return false;
         return true;
     }
     // (3-bit 11008 x 4096 with an activation order at 256 rows: 46.5 against 51.2 on the checkpoint tensors; 4-bit 52.4

@@ -385,14 +385,16 @@ def table_tiled_wins(M, K, N, act_order, bits, one_group):
             return K <= 4096 and N > 4096 and (M >= 9 or bits == 4)
         return K <= 4096 and ((N > 4096 and M >= 12) or (bits == 3 and N <= 4096))
     if M <= 128:
-        if one_group and K > 8192 and (M > 32 or K > 16384 or N > 16384):
+        if one_group and K > 8192 and (M > 32 or N > 16384):
+            return False
+        if M <= 32 and K > 20480 and act_order:
             return False
         return not (M <= 64 and K >= 8192 and bits == 4 and not act_order)
     return K <= 8192 or (bits == 3 and K <= 11008 and M <= 256)
 
 
-ROUTE_SHAPES = [(4096, 4096), (4096, 11008), (11008, 4096), (4096, 22016), (8192, 8192), (8192, 28672),
-                (9216, 9216), (9216, 36864), (36864, 9216), (5120, 13824), (6656, 17920)]
+ROUTE_SHAPES = [(4096, 4096), (4096, 11008), (11008, 4096), (4096, 22016), (8192, 8192), (8192, 28672), (28672, 8192),
+                (9216, 9216), (9216, 36864), (36864, 9216), (18432, 9216), (5120, 13824), (6656, 17920), (17920, 6656)]
 
 
 @pytest.mark.parametrize("bits", [3, 4])
