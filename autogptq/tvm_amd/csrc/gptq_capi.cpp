@@ -353,6 +353,9 @@ extern "C" int gptq_hip_gemm_tiled(const void *x, const void *qtile, const uint3
             return GPTQ_HIP_ERR_BAD_ARG;
         // a caller that runs halved tiles has to know what their workspace asks for
         if (halved != 0 && !(plan->flags & GPTQ_HIP_PLAN_PRIVATE_ZERO_WORKSPACE)) return GPTQ_HIP_ERR_BAD_ARG;
+        // and a plan that says so while it writes partial sums (K cut over workgroups, whole tiles) would leave them in
+        // a workspace that has to stay zero
+        if (halved == 0 && (plan->flags & GPTQ_HIP_PLAN_PRIVATE_ZERO_WORKSPACE)) return GPTQ_HIP_ERR_BAD_ARG;
         if ((kw != 4 && kw != 8 && kw != 16) || plan->block != 64 * kw || plan->split_k < 1 || plan->k_chunk < 1 ||
             plan->grid_y != plan->split_k || plan->grid_z != 1 ||
             (long long)plan->split_k * kw * plan->k_chunk < S_all ||

@@ -235,11 +235,15 @@ inline bool tiled_decode_can_halve(int wave_steps, int split_k, int waves_k, int
     return waves_k * first < S_total;                          // the second half must start inside K
 }
 // Layers of so few tiles that two workgroups per tile still find a CU each (N <= 4096), with K long enough for
-// two ranges (8192 channels): EVERY tile is halved, which gives every CU work like the 16-column kernel does, at
-// the lower cost per weight of this one (one row / four rows, us, against the 16-column kernel: 11008 x 4096 int3
-// 8.4 / 11.2 against 9.6 / 13.6, 14336 x 4096 int4 10.1 / 12.7 against 10.2 / 14.6, 8192 x 4096 7.6 / 9.1 against
-// 8.1 / 10.6; 4096 x 4096 the same 5.9, so shorter layers stay there).
-inline bool tiled_decode_halves_all(int tiles, int S_total) { return 2 * tiles <= kNumCUs && S_total >= 128; }
+// two ranges (4096 channels): EVERY tile is halved, which gives every CU work like the 16-column kernel does, at
+// the lower cost per weight of this one (one / four / eight rows, us, against the 16-column kernel, which has no
+// eight-row form: there the comparison is with whole tiles.  4096 x 4096 int4 4.11 / 5.20 / 6.42 against 4.43 / 5.86 /
+// 7.29, int3 with an activation order 4.05 / 5.96 / 9.21 against 4.40 / 6.47 / 10.0; 4096 x 2048 3.59 / 4.81 / 6.32 against
+// 4.13 / 5.58 / 7.10; 4096 x 1024 3.48 / 4.70 / 6.23 against 4.04 / 5.49 / 7.06; 6144 x 4096 4.79 / 6.04 / 7.87 against 5.45 /
+// 7.21 / 8.52; 11008 x 4096 int3 8.4 / 11.2 against 9.6 / 13.6 at one / four rows.  At 2048 channels the halves are four
+// blocks per wave: 2048 x 4096 3.93 / 5.17 / 6.31 against 3.98 / 5.33 / 5.72, 2048 x 2048 3.78 / 5.03 / 6.25 against
+// 3.79 / 5.19 / 5.66: level up to four rows, a loss at eight, so shorter layers stay with the 16-column kernel).
+inline bool tiled_decode_halves_all(int tiles, int S_total) { return 2 * tiles <= kNumCUs && S_total >= 64; }
 inline int tiled_decode_halved(int tiles, int wave_steps, int split_k, int waves_k, int S_total, int group_size)
 {
     if (!tiled_decode_can_halve(wave_steps, split_k, waves_k, S_total, group_size)) return 0;

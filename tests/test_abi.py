@@ -308,7 +308,7 @@ def test_tiled_plans_are_consistent(bits, KN):
                 halved = p.grid_x - tiles
                 assert halved in (0, tiles % 256, tiles) and p.split_k * p.waves_k * p.k_chunk >= blocks
                 if halved == tiles:
-                    assert 2 * tiles <= 256 and blocks >= 128 and p.split_k == 1 and p.waves_k == 8
+                    assert 2 * tiles <= 256 and blocks >= 64 and p.split_k == 1 and p.waves_k == 8
                 elif halved:
                     assert tiles > 256 and halved <= 128 and p.split_k == 1
                 if halved:
@@ -462,7 +462,10 @@ def test_plans_that_need_a_private_zero_workspace_say_so():
     p = _lib.select_tiled(1, 4096, 11008, 3, 128)
     assert p.kernel == _lib.KERNEL_TILED_DECODE and p.grid_x > 11008 // 32
     assert p.flags & _lib.PLAN_PRIVATE_ZERO_WORKSPACE and p.workspace_bytes > 0
-    for q in (_lib.select_tiled(1, 4096, 4096, 4, 128), _lib.select_tiled(128, 4096, 11008, 4, 128),
+    q = _lib.select_tiled(1, 4096, 4096, 4, 128)     # every tile of a narrow layer of 4096 channels and more in two halves
+    assert q.kernel == _lib.KERNEL_TILED_DECODE and q.waves_n == 1 and q.grid_x == 2 * (4096 // 32)
+    assert q.flags & _lib.PLAN_PRIVATE_ZERO_WORKSPACE and q.workspace_bytes > 0
+    for q in (_lib.select_tiled(1, 2048, 4096, 4, 128), _lib.select_tiled(128, 4096, 11008, 4, 128),
               _lib.select(1, 4096, 11008, 3, 128, True), _lib.select(64, 4096, 11008, 4, 128, True)):
         assert q.flags == 0
     assert ctypes.sizeof(_lib.Route) == 8 + ctypes.sizeof(_lib.Plan)

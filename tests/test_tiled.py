@@ -45,7 +45,7 @@ def tile_decode_plan_of(plan, M, K, N, bits, gs):
     plan.waves_n, plan.waves_k, plan.split_k, plan.k_chunk = 1, kw, 1, steps
     plan.grid_x, plan.grid_y, plan.grid_z, plan.block = tiles, 1, 1, 64 * kw
     plan.lds_bytes = mr * span * 2 + 64 + (span // 32) * mr * 8 + groups * 128 + kw * mr * 128
-    plan.workspace_bytes = 0
+    plan.workspace_bytes, plan.flags = 0, 0    # (whole tiles: no slots, whatever the family's own plan needs)
     return plan
 
 
@@ -65,6 +65,7 @@ def cu_decode_plan(M, K, N, bits, gs, grid=None):
         return None
     plan.row_tiles, plan.waves_n, plan.waves_k, plan.split_k, plan.k_chunk = mr, 2, 16, 1, -(-V // 16)
     plan.grid_x, plan.grid_y, plan.grid_z, plan.block, plan.lds_bytes, plan.workspace_bytes = grid, 1, 1, 1024, lds, 0
+    plan.flags = 0
     return plan
 
 
@@ -295,7 +296,7 @@ def test_tiled_decode_halved_tiles(dev, bits, K, N, gs, desc_act):
         plan = _lib.select_tiled(M, K, N, bits, gs)
         assert plan.kernel == _lib.KERNEL_TILED_DECODE and plan.split_k == 1
         tiles = N // 32
-        halved = tiles if (2 * tiles <= 256 and -(-K // 64) >= 128) else tiles % 256
+        halved = tiles if (2 * tiles <= 256 and -(-K // 64) >= 64) else tiles % 256
         assert plan.grid_x == tiles + halved and plan.workspace_bytes > 16384, "the plan does not halve its tiles"
         x = L["x"][:M].contiguous()
         want = expected_output(L, x=x, w16=w16)
