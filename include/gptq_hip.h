@@ -55,7 +55,7 @@ enum {
                                    does not fit LDS) adds a reduce launch.  waves_n = 2: units of 16 columns dealt
                                    out evenly over grid_x workgroups of 16 waves, all of K staged per workgroup
                                    (k_chunk = blocks of 128 channels per unit and wave); chosen for layers of up to
-                                   4096 columns */
+                                   4096 columns and fewer than 4096 channels */
 };
 
 /* What the dispatcher decided for one problem; filled by gptq_hip_select. */
