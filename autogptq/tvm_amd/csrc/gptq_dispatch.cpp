@@ -608,7 +608,7 @@ namespace {
 // Where the tiled kernels were measured faster than the ones that read the checkpoint layout or its channel-sorted
 // copy, on MI355X with the weights cold (us per call, graph replay, group size 128 unless said):
 //   * up to 4 rows, layers of up to 4096 columns (decode kernel with a workgroup per 16 columns, or every tile in two
-//     halves along K from 8192 channels): always.  4096 x 4096: 5.3-5.6 at one row, 7.4-8.0 at four, against 6.8-7.5
+//     halves along K from 4096 channels): always.  4096 x 4096: 4.1-4.2 at one row, 5.2 at four, against 6.8-7.5
 //     and 7.8-10.5; 11008 x 4096: int4 9.0-9.4 / 11.5 against 13.5 / 15.3, int3 8.7 / 11.1 against 10.9 / 15.2;
 //   * up to 4 rows, wider layers (a workgroup per 32 columns): K = 4096: one and two rows always, three and four up
 //     to 16384 columns (4096 x 11008 with an activation order, one / two / four rows: int4 7.8 / 8.1 / 9.8 against
