@@ -281,11 +281,12 @@ def test_tiled_decode_split_k(dev, bits, M):
 @pytest.mark.parametrize("bits", [2, 3, 4, 8])
 @pytest.mark.parametrize("K,N,gs", [(1024, 8224, 128), (1024, 11008, 128), (1280, 12288, 128), (2048, 9600, 64),
                                     (2048, 12288, -1), (640, 18368, 128), (1152, 9216, 32),
-                                    (8192, 1056, 128), (8256, 512, 64), (8192, 4096, 1024), (9248, 96, 32)])
+                                    (8192, 1056, 128), (8256, 512, 64), (8192, 4096, 1024), (9248, 96, 32),
+                                    (4096, 4096, 128), (4160, 352, 32), (5120, 2048, 128), (4096, 96, 64)])
 @pytest.mark.parametrize("desc_act", [False, True])
 def test_tiled_decode_halved_tiles(dev, bits, K, N, gs, desc_act):
-    # Up to 128 column tiles past a whole number per CU (256), or every tile of a long layer of up to 4096 columns
-    # (the last four shapes): the family's plan runs them as two halves along K (equal, or the first one larger:
+    # Up to 128 column tiles past a whole number per CU (256), or every tile of a layer of up to 4096 columns with 4096
+    # channels or more (the last eight shapes): the family's plan runs them as two halves along K (equal, or the first one larger:
     # 1280, 1152, 8256 and 9248 channels) that meet through the exchange slots of a workspace of their own; the
     # slots are zero again after every call, so the same workspace serves every row count in turn
     L = layer(8100 + bits, K, N, bits, gs, desc_act, M=4, bias=True)
