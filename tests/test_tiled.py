@@ -218,6 +218,18 @@ def test_tiled_rejections(dev):
     p = _lib.select(8, 4096, 352, 4, 128, False)
     assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, null, fake, fake, 1 << 24, 8, 4096, 352, 4, 128, ctypes.byref(p),
                                    null) == _lib.ERR_UNSUPPORTED
+    # halved tiles without the flag that asks for a workspace of their own, and the flag on a plan that writes partial sums
+    h = _lib.select_tiled(1, 4096, 352, 4, 128)
+    assert h.grid_x == 2 * (352 // 32) and h.flags & _lib.PLAN_PRIVATE_ZERO_WORKSPACE
+    h.flags = 0
+    assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, null, fake, fake, 1 << 24, 1, 4096, 352, 4, 128, ctypes.byref(h),
+                                   null) == _lib.ERR_BAD_ARG
+    w = tile_decode_plan(1, 4096, 352, 4, 128)
+    w.split_k = w.grid_y = 2
+    w.k_chunk = -(-(4096 // 64) // (2 * w.waves_k))
+    w.workspace_bytes, w.flags = 16384 + 2 * 352 * 4, _lib.PLAN_PRIVATE_ZERO_WORKSPACE
+    assert lib.gptq_hip_gemm_tiled(fake, fake, fake, null, null, null, fake, fake, 1 << 24, 1, 4096, 352, 4, 128, ctypes.byref(w),
+                                   null) == _lib.ERR_BAD_ARG
     other = ctypes.c_void_p(0x2000)
     assert lib.gptq_hip_tile_prepare(fake, fake, fake, null, other, fake, fake, fake, 4096, 352, 4, 16, null) == _lib.ERR_UNSUPPORTED
     assert lib.gptq_hip_tile_prepare(fake, fake, fake, null, null, fake, fake, fake, 4096, 352, 4, 128, null) == _lib.ERR_BAD_ARG
