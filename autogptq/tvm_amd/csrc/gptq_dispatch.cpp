@@ -520,6 +520,10 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     const int S_total = ceil_div(K, 64);
     const long long tiles = (long long)col_pairs * m_blocks;
     int split = (int)((256 + tiles / 2) / tiles);
+    // workgroups of four row tiles hold a CU alone: ranges that put a few workgroups past one per CU make the whole
+    // launch wait for a second turn of those few (9216 x 9216 int3 at 256 rows, 144 tiles, us in 1 / 2 / 3 ranges:
+    // 67.9 / 85.3 / 73.8; 8192 x 8192 at 256 rows, 128 tiles: 57.3 / 50.2 / 66.6)
+    if (at == 4 && tiles <= 256 && tiles * split > 256) split = (int)(256 / tiles);
     if (split < 1) split = 1;
     int cap = (int)((3LL * K * bits) / (128LL * M));
     if (cap < 1) cap = 1;
@@ -527,6 +531,10 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     if ((long long)M * N >= (1LL << 32)) split = 1;  // indexing of the pass that adds the partial tiles
     // every wave gets at least a ring of blocks
     while (split > 1 && S_total / (split * kwv) < gptq::tiled_ring(at)) split--;
+    // the partial tiles of all ranges together stay within 14 MB where fewer ranges still give two of three CUs a
+    // workgroup (11008 x 4096 at 256 rows, 128 x 128 waves, us in 2 / 3 / 4 ranges: int4 49.9 / 45.3 / 52.3, int3 50.9 /
+    // 46.5 / 53.3: the fourth range adds 4 MB of fp32 tiles to write and to read again)
+    while (split > 1 && (long long)split * M * N * 4 > (14LL << 20) && tiles * (split - 1) >= 172) split--;
     // One row tile (up to 32 rows): two such workgroups share a CU, and where K is cut anyway (the pass that adds the
     // ranges is there already) and long, finer ranges that still leave every wave two turns of its ring put up to
     // ~480 workgroups on the chip at once instead of ~256 (us at 32 rows, int3, one group, 144 column pairs: 9216 x
@@ -663,9 +671,9 @@ bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
         if (M <= 32 && K > 20480 && act_order) return false;
         return true;
     }
-    // (3-bit 11008 x 4096 with an activation order at 256 rows: 46.5 against 51.2 on the checkpoint tensors; 4-bit 52.4
-    // against 48.5)
-    return K <= 8192 || (bits == 3 && K <= 11008 && M <= 256);
+    // (11008 x 4096 with an activation order at 256 rows, K in three ranges: 3-bit 46.5 against 51.2 on the checkpoint
+    // tensors, 4-bit 45.3 against 48.5)
+    return K <= 8192 || (K <= 11008 && M <= 256);
 }
 
 // The plan gptq_hip_gemm_sorted runs for M rows of a layer whose channels were sorted by group, if that path covers

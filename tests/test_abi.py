@@ -390,7 +390,7 @@ def table_tiled_wins(M, K, N, act_order, bits, one_group):
         if M <= 32 and K > 20480 and act_order:
             return False
         return not (M <= 64 and K >= 8192 and bits == 4 and not act_order)
-    return K <= 8192 or (bits == 3 and K <= 11008 and M <= 256)
+    return K <= 8192 or (K <= 11008 and M <= 256)
 
 
 ROUTE_SHAPES = [(4096, 4096), (4096, 11008), (11008, 4096), (4096, 22016), (8192, 8192), (8192, 28672), (28672, 8192),
@@ -469,3 +469,19 @@ def test_plans_that_need_a_private_zero_workspace_say_so():
               _lib.select(1, 4096, 11008, 3, 128, True), _lib.select(64, 4096, 11008, 4, 128, True)):
         assert q.flags == 0
     assert ctypes.sizeof(_lib.Route) == 8 + ctypes.sizeof(_lib.Plan)
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_plans_of_four_row_tiles_keep_their_workgroups_within_one_per_cu(bits):
+    # a workgroup of four row tiles holds a CU alone: K ranges never put a few workgroups past one per CU
+    for K, N in ROUTE_SHAPES + [(4096, 6144), (8192, 5632), (4096, 3328), (11008, 11008)]:
+        for M in (97, 128, 192, 256, 512):
+            p = _lib.select_tiled(M, K, N, bits, 128)
+            if p.kernel != _lib.KERNEL_TILED or p.row_tiles != 4:
+                continue
+            tiles = p.grid_x * p.grid_z
+            assert p.grid_y == p.split_k
+            if tiles <= 256:
+                assert tiles * p.split_k <= 256, (M, K, N, p.as_dict())
+            else:
+                assert p.split_k == 1 or tiles * p.split_k >= 384, (M, K, N, p.as_dict())
