@@ -645,7 +645,8 @@ namespace {
 //     to 32 rows of layers beyond 20480 channels (28672 x 8192 at 32 rows, int4 / int3: 58.3 / 55.9 against 48.3 /
 //     49.8; 17920 x 6656 33.9 / 34.5 against 34.1 / 38.9 stays; from 64 rows the tiled copy wins there too: 60.1 / 63.0
 //     against 63.0 / 67.2);
-//   * above 128 rows: K up to 8192 (4096 x 11008, 512 rows: 75 against 95; 11008 x 4096: 127 against 81).
+//   * above 128 rows: K up to 8192 (4096 x 11008, 512 rows: 75 against 95; 11008 x 4096: 127 against 81), and up to
+//     256 rows the longer layers named in the function.
 bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
 {
     if (M <= 4) {
@@ -671,9 +672,13 @@ bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
         if (M <= 32 && K > 20480 && act_order) return false;
         return true;
     }
-    // (11008 x 4096 with an activation order at 256 rows, K in three ranges: 3-bit 46.5 against 51.2 on the checkpoint
-    // tensors, 4-bit 45.3 against 48.5)
-    return K <= 8192 || (K <= 11008 && M <= 256);
+    // up to 256 rows also K up to 11008, and any K with an activation order (192 / 256 rows against the checkpoint
+    // tensors: 11008 x 4096 with an activation order at 256 rows, K in three ranges, 3-bit 46.5 against 51.2, 4-bit 45.3
+    // against 48.5; 11008 x 11008 4-bit 85.9 against 109.6 at 256 rows; with an activation order 17920 x 6656 96.4 / 99.6
+    // against 112 / 116, 28672 x 8192 4-bit 169 / 172 against 178 / 192, 3-bit 165 / 166 against 169 / 192; without one
+    // the longer layers are level or behind: 28672 x 8192 167 / 169 against 164 / 169, 13824 x 5120 at 192 rows 54.7
+    // against 46.3)
+    return K <= 8192 || (M <= 256 && (K <= 11008 || act_order));
 }
 
 // The plan gptq_hip_gemm_sorted runs for M rows of a layer whose channels were sorted by group, if that path covers

@@ -390,7 +390,7 @@ def table_tiled_wins(M, K, N, act_order, bits, one_group):
         if M <= 32 and K > 20480 and act_order:
             return False
         return not (M <= 64 and K >= 8192 and bits == 4 and not act_order)
-    return K <= 8192 or (K <= 11008 and M <= 256)
+    return K <= 8192 or (M <= 256 and (K <= 11008 or act_order))
 
 
 ROUTE_SHAPES = [(4096, 4096), (4096, 11008), (11008, 4096), (4096, 22016), (8192, 8192), (8192, 28672), (28672, 8192),
