@@ -505,7 +505,26 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     }
     const int ok = tiled_args_ok(M, K, N, bits, group_size, plan);
     if (ok != GPTQ_HIP_OK) return ok;
-    const int at = gptq::tiled_row_tiles(M), rw = 1, kwv = 4;
+    int at = gptq::tiled_row_tiles(M);
+    const int rw = 1, kwv = 4;
+    // Narrow layers above 64 rows: where row blocks of 64 rows still find a CU each, they replace the 128-row blocks,
+    // whose few workgroups had to cut K (partial tiles and a pass that adds them) to fill the chip (us at 96 / 128 /
+    // 256 rows against 128-row blocks, int4 with an activation order: 4096 x 4096 16.8 / 17.1 / 21.7 against 20.1 /
+    // 21.2 / 25.1, 2048 x 4096 11.4 / 11.5 / 13.0 against 15.2 / 15.5 / 16.0, 4096 x 2048 16.0 / 16.5 / 17.4 against
+    // 17.4 / 18.6 / 24.5, 5120 x 5120 21.0 / 21.4 against 23.5 / 25.1, 6656 x 6656 27.1 / 27.5 against 29.4 / 30.8,
+    // 4096 x 8192 18.9 / 19.5 against 22.9 / 24.5, 8192 x 8192 34.3 / 35.0 against 36.7 / 38.3; with more such blocks than
+    // CUs they lose: 5120 x 5120 at 256 rows 36.6 against 31.0, 4096 x 11008 at 128 rows 31.1 against 24.8)
+    // The same one step down, 33 to 64 rows as two blocks of 32, for K up to 4096 (48 / 64 rows: 4096 x 4096 13.2 / 13.5
+    // against 14.4 / 14.9, 4096 x 8192 14.7 / 15.0 against 16.5 / 17.3, 2048 x 4096 9.6 / 9.8 against 11.4 / 11.8, 5120 x 5120
+    // and 4096 x 2048 level; 8192 x 4096 21.1 / 20.9 against 19.2 / 19.8 and 11008 x 4096 24.1 / 24.3 against 22.9 / 23.8 stay)
+    bool short_blocks = false;
+    if (at == 4 && K <= 8192 && (long long)ceil_div(N / 32, 2) * ceil_div(M, 64) <= 256) {
+        at = 2;
+        short_blocks = true;
+    } else if (at == 2 && K <= 4096 && (long long)ceil_div(N / 32, 2) * ceil_div(M, 32) <= 256) {
+        at = 1;
+        short_blocks = true;
+    }
     const int rows = 32 * at * rw;
     const int m_blocks = ceil_div(M, rows);
     // several row blocks: 128 columns per wave (waves_n = 2), which halves the x fragments a matrix instruction
@@ -514,16 +533,27 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     // then need the larger share of L2 that fewer, wider workgroups leave them.  4096 x 11008: 256 rows 49.6 ->
     // 41.9 us, 1024 rows 142 -> 123; 11008 x 4096, 512 rows: 127 -> 88; 4096 x 4096, 512 rows, 128 workgroups:
     // 33.5 -> 40.4, so not there)
-    const bool wide = m_blocks >= 2 && ((long long)ceil_div(N / 32, 4) * m_blocks >= 172 || K > 8192);
+    const bool wide = at == 4 && m_blocks >= 2 && ((long long)ceil_div(N / 32, 4) * m_blocks >= 172 || K > 8192);
     const int ct = wide ? 4 : 2;
     const int col_pairs = ceil_div(N / 32, ct);
     const int S_total = ceil_div(K, 64);
     const long long tiles = (long long)col_pairs * m_blocks;
     int split = (int)((256 + tiles / 2) / tiles);
-    // workgroups of four row tiles hold a CU alone: ranges that put a few workgroups past one per CU make the whole
-    // launch wait for a second turn of those few (9216 x 9216 int3 at 256 rows, 144 tiles, us in 1 / 2 / 3 ranges:
-    // 67.9 / 85.3 / 73.8; 8192 x 8192 at 256 rows, 128 tiles: 57.3 / 50.2 / 66.6)
-    if (at == 4 && tiles <= 256 && tiles * split > 256) split = (int)(256 / tiles);
+    // workgroups of two or four row tiles hold a CU alone: ranges that put a few workgroups past one per CU make the
+    // whole launch wait for a second turn of those few (9216 x 9216 int3 at 256 rows, 144 tiles, us in 1 / 2 / 3 ranges:
+    // 67.9 / 85.3 / 73.8; 8192 x 8192 at 256 rows, 128 tiles: 57.3 / 50.2 / 66.6; at 64 rows 8192 x 6144, 96 tiles, in
+    // 1 / 2 / 3 ranges 28.3 / 24.1 / 30.2, 11008 x 4608, 72 tiles, in 2 / 3 / 4: 28.0 / 24.8 / 32.0, 8192 x 3328, 52 tiles, in
+    // 3 / 4 / 5: 19.8 / 18.7 / 24.7)
+    if (at >= 2 && tiles <= 256 && tiles * split > 256) split = (int)(256 / tiles);
+    // the 64-row blocks of a narrow layer: at most one workgroup per CU, and K cut only while a wave keeps sixteen
+    // blocks (eight where there are at most 64 tiles): a shorter walk saves less than the partial tiles and their pass
+    // cost (4096 x 4096 at 128 rows in 1 / 2 ranges 17.1 / 17.6, 2048 x 4096 11.5 / 13.2, 8192 x 4096 29.5 / 26.5,
+    // 4096 x 2048 16.5 / 15.4)
+    if (short_blocks) {
+        split = (int)(256 / tiles);
+        const int keep = tiles <= 64 ? 8 : 16;
+        while (split > 1 && S_total / (split * kwv) < keep) split--;
+    }
     if (split < 1) split = 1;
     int cap = (int)((3LL * K * bits) / (128LL * M));
     if (cap < 1) cap = 1;
@@ -531,10 +561,10 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     if ((long long)M * N >= (1LL << 32)) split = 1;  // indexing of the pass that adds the partial tiles
     // every wave gets at least a ring of blocks
     while (split > 1 && S_total / (split * kwv) < gptq::tiled_ring(at)) split--;
-    // the partial tiles of all ranges together stay within 14 MB where fewer ranges still give two of three CUs a
+    // the partial tiles of all ranges together stay within 10 MB where fewer ranges still give two of three CUs a
     // workgroup (11008 x 4096 at 256 rows, 128 x 128 waves, us in 2 / 3 / 4 ranges: int4 49.9 / 45.3 / 52.3, int3 50.9 /
     // 46.5 / 53.3: the fourth range adds 4 MB of fp32 tiles to write and to read again)
-    while (split > 1 && (long long)split * M * N * 4 > (14LL << 20) && tiles * (split - 1) >= 172) split--;
+    while (split > 1 && (long long)split * M * N * 4 > (10LL << 20) && tiles * (split - 1) >= 172) split--;
     // One row tile (up to 32 rows): two such workgroups share a CU, and where K is cut anyway (the pass that adds the
     // ranges is there already) and long, finer ranges that still leave every wave two turns of its ring put up to
     // ~480 workgroups on the chip at once instead of ~256 (us at 32 rows, int3, one group, 144 column pairs: 9216 x
@@ -582,6 +612,8 @@ extern "C" int gptq_hip_select_tiled_transposed(int M, int K, int N, int bits, i
     const long long tiles = (long long)col_pairs * m_blocks;
     int split = (int)((256 + tiles / 2) / tiles);
     if (split < 1) split = 1;
+    // (workgroups of two or four row tiles hold a CU alone, as in the forward plan: no few workgroups past one per CU)
+    if (at >= 2 && tiles <= 256 && tiles * split > 256) split = (int)(256 / tiles);
     int cap = (int)((3LL * N * bits) / (128LL * M));   // the fp32 tiles of a split stay within 3x the packed weights
     if (cap < 1) cap = 1;
     if (split > cap) split = cap;

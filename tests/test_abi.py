@@ -472,16 +472,36 @@ def test_plans_that_need_a_private_zero_workspace_say_so():
 
 
 @pytest.mark.parametrize("bits", [3, 4])
-def test_plans_of_four_row_tiles_keep_their_workgroups_within_one_per_cu(bits):
-    # a workgroup of four row tiles holds a CU alone: K ranges never put a few workgroups past one per CU
-    for K, N in ROUTE_SHAPES + [(4096, 6144), (8192, 5632), (4096, 3328), (11008, 11008)]:
-        for M in (97, 128, 192, 256, 512):
-            p = _lib.select_tiled(M, K, N, bits, 128)
-            if p.kernel != _lib.KERNEL_TILED or p.row_tiles != 4:
-                continue
-            tiles = p.grid_x * p.grid_z
-            assert p.grid_y == p.split_k
-            if tiles <= 256:
-                assert tiles * p.split_k <= 256, (M, K, N, p.as_dict())
-            else:
-                assert p.split_k == 1 or tiles * p.split_k >= 384, (M, K, N, p.as_dict())
+def test_plans_of_two_and_four_row_tiles_keep_their_workgroups_within_one_per_cu(bits):
+    # a workgroup of two or four row tiles holds a CU alone: K ranges never put a few workgroups past one per CU
+    for K, N in ROUTE_SHAPES + [(4096, 6144), (8192, 5632), (4096, 3328), (11008, 11008), (8192, 6144), (11008, 4608)]:
+        for M in (33, 64, 97, 128, 192, 256, 512):
+            plans = [_lib.select_tiled(M, K, N, bits, 128)]
+            if N <= 11008:   # (longer reductions of the transposed product are cut so that a range's table fits LDS)
+                plans.append(_lib.select_tiled_transposed(M, K, N, bits, 128))
+            for p in plans:
+                if p.kernel != _lib.KERNEL_TILED or p.row_tiles < 2:
+                    continue
+                tiles = p.grid_x * p.grid_z
+                assert p.grid_y == p.split_k
+                if tiles <= 256:
+                    assert tiles * p.split_k <= 256, (M, K, N, p.as_dict())
+                else:
+                    assert p.split_k == 1 or tiles * p.split_k >= 384, (M, K, N, p.as_dict())
+
+
+def test_narrow_layers_run_in_shorter_row_blocks():
+    # 65 to 256 rows of a narrow layer: blocks of 64 rows while they find a CU each (K up to 8192), 33 to 64 rows as two
+    # blocks of 32 (K up to 4096); the wide and the long layers keep the taller blocks
+    for M, K, N, rt, mb in ((128, 4096, 4096, 2, 2), (256, 4096, 4096, 2, 4), (192, 5120, 5120, 2, 3), (128, 8192, 8192, 2, 2),
+                            (320, 4096, 4096, 4, 3), (256, 5120, 5120, 4, 2), (128, 4096, 11008, 4, 1), (128, 11008, 4096, 4, 1),
+                            (64, 4096, 4096, 1, 2), (48, 4096, 8192, 1, 2), (64, 8192, 4096, 2, 1), (64, 4096, 11008, 2, 1),
+                            (32, 4096, 4096, 1, 1)):
+        p = _lib.select_tiled(M, K, N, 4, 128)
+        assert (p.kernel, p.row_tiles, p.m_blocks, p.grid_z) == (_lib.KERNEL_TILED, rt, mb, mb), (M, K, N, p.as_dict())
+        assert p.waves_n == 1 or p.row_tiles == 4
+        assert p.lds_bytes == 4 * p.row_tiles * 2 * 4096 * (2 if p.waves_n == 2 else 1) or p.waves_n == 2
+    p = _lib.select_tiled(128, 4096, 4096, 4, 128)
+    assert p.split_k == 1 and p.k_chunk == 16
+    p = _lib.select_tiled(128, 8192, 4096, 4, 128)
+    assert p.split_k == 2 and p.k_chunk == 16

@@ -184,6 +184,32 @@ def test_tiled_forced_split_k(dev, bits, split, M):
     assert torch.equal(y1, y2)
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
+@pytest.mark.parametrize("M,row_tiles", [(33, 2), (64, 2), (65, 4), (127, 4), (130, 4), (257, 4), (40, 1), (130, 2), (257, 1)])
+@pytest.mark.parametrize("split", [1, 2])
+def test_tiled_every_block_height_on_a_narrow_layer(dev, bits, M, row_tiles, split):
+    # the planner gives narrow layers shorter row blocks than wide ones: every height the kernel is built for, forced on
+    # one narrow layer (the tall blocks as wide layers get them, and more, shorter blocks than the planner would choose)
+    K, N, gs = 1024, 416, 128
+    L = layer(1450 + M, K, N, bits, gs, True, M=M, bias=True)
+    D = to_dev(L, dev)
+    plan = _lib.select_tiled(M, K, N, bits, gs)
+    assert plan.kernel == _lib.KERNEL_TILED and plan.waves_n == 1
+    blocks = K // 64
+    plan.row_tiles = row_tiles
+    plan.m_blocks = plan.grid_z = -(-M // (32 * row_tiles))
+    plan.lds_bytes = plan.waves_k * row_tiles * 2 * 4096
+    plan.split_k, plan.grid_y = split, split
+    plan.k_chunk = -(-blocks // (plan.waves_k * split))
+    part = (split * M * N * 4 + 255) // 256 * 256 if split > 1 else 0
+    plan.workspace_bytes = 16384 + part + split * plan.waves_k * plan.k_chunk * 4 * plan.row_tiles * plan.m_blocks * 1024
+    prep = prepare(D)
+    y1 = run_tiled(D, prep, plan=plan)
+    assert_close(y1, expected_output(L), f"tiled M={M} row_tiles={row_tiles} split={split}")
+    assert_tight(y1, expected_output(L), f"tiled M={M} row_tiles={row_tiles} split={split}")
+    assert torch.equal(y1, run_tiled(D, prep, plan=plan)), "two identical calls differ"
+
+
 def test_tiled_integer_exact_and_guard_bands(dev):
     # x = 1, scales = 1, one group: y[n] = sum_k (q - z), an integer (8-bit sums pass 2048: one fp16 rounding)
     for bits in (2, 3, 4, 8):
