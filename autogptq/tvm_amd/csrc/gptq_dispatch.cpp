@@ -605,15 +605,35 @@ extern "C" int gptq_hip_select_tiled_transposed(int M, int K, int N, int bits, i
 {
     const int ok = tiled_args_ok(M, K, N, bits, group_size, plan);
     if (ok != GPTQ_HIP_OK) return ok;
-    const int at = gptq::tiled_row_tiles(M), kwv = 4, ct = 2;
-    const int m_blocks = ceil_div(M, 32 * at);
+    int at = gptq::tiled_row_tiles(M);
+    const int kwv = 4, ct = 2;
     const int col_pairs = ceil_div(K / 32, ct);
     const int S_total = ceil_div(N, 64);
+    // shorter row blocks where they still find a CU each, as in the forward plan (the result has K columns here and
+    // the reduction runs over N; us at 64 / 128 / 256 rows against the taller blocks, int4: 4096 x 4096 17.8 / 22.5 / 27.9
+    // against 17.7 / 25.6 / 33.0, 8192 x 4096 20.7 / 26.6 against 22.2 / 31.1, 4096 x 2048 13.1 / 16.5 / 20.1 against 14.5 /
+    // 21.7 / 24.5, 2048 x 4096 14.9 / 18.0 / 23.3 against 15.1 / 21.0 / 30.3, 5120 x 5120 at 128 rows 27.2 against 29.6; a
+    // reduction over 8192 keeps the tall blocks: 4096 x 8192 at 128 / 256 rows 30.9 / 48.4 against 29.6 / 45.8)
+    bool short_blocks = false;
+    if (at == 4 && N < 8192 && (long long)col_pairs * ceil_div(M, 64) <= 256) {
+        at = 2;
+        short_blocks = true;
+    } else if (at == 2 && N <= 4096 && (long long)col_pairs * ceil_div(M, 32) <= 256) {
+        at = 1;
+        short_blocks = true;
+    }
+    const int m_blocks = ceil_div(M, 32 * at);
     const long long tiles = (long long)col_pairs * m_blocks;
     int split = (int)((256 + tiles / 2) / tiles);
     if (split < 1) split = 1;
     // (workgroups of two or four row tiles hold a CU alone, as in the forward plan: no few workgroups past one per CU)
     if (at >= 2 && tiles <= 256 && tiles * split > 256) split = (int)(256 / tiles);
+    if (short_blocks) {
+        split = (int)(256 / tiles);
+        const int keep = tiles <= 64 ? 8 : 16;
+        while (split > 1 && S_total / (split * kwv) < keep) split--;
+        if (split < 1) split = 1;
+    }
     int cap = (int)((3LL * N * bits) / (128LL * M));   // the fp32 tiles of a split stay within 3x the packed weights
     if (cap < 1) cap = 1;
     if (split > cap) split = cap;

@@ -75,6 +75,29 @@ def test_transposed_product_shapes(dev, bits, K, N, gs, M):
         assert torch.equal(gx, run_t(D, prep, gy.to(dev))), "two identical calls differ"
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
+@pytest.mark.parametrize("M,row_tiles", [(40, 1), (40, 2), (64, 2), (65, 4), (130, 1), (130, 2), (130, 4), (257, 4)])
+def test_transposed_every_block_height_on_a_narrow_layer(dev, bits, M, row_tiles):
+    # the planner gives narrow layers shorter row blocks than wide ones: every height the kernel is built for, forced
+    K, N, gs = 416, 1024, 32
+    L = layer(3450 + M, K, N, bits, gs, True)
+    D = to_dev(L, dev)
+    plan = _lib.select_tiled_transposed(M, K, N, bits, gs)
+    plan.row_tiles = row_tiles
+    plan.m_blocks = plan.grid_z = -(-M // (32 * row_tiles))
+    plan.split_k = plan.grid_y = 1
+    plan.k_chunk = -(-(N // 64) // plan.waves_k)
+    plan.lds_bytes = max(plan.waves_k * row_tiles * 2 * 4096, 2 * plan.waves_k * plan.k_chunk * 256)
+    plan.workspace_bytes = 16384 + plan.waves_k * plan.k_chunk * 4 * row_tiles * plan.m_blocks * 1024
+    prep = prepare(D)
+    gy = grad_rows(3460 + M, M, N)
+    g1 = run_t(D, prep, gy.to(dev), plan=plan)
+    want = gy.float() @ expected_weight(L).float().t()
+    assert_close(g1, want, f"transposed M={M} row_tiles={row_tiles}")
+    assert_tight(g1, want, f"transposed M={M} row_tiles={row_tiles}")
+    assert torch.equal(g1, run_t(D, prep, gy.to(dev), plan=plan))
+
+
 @pytest.mark.parametrize("bits", [3, 4, 8])
 @pytest.mark.parametrize("split", [1, 2, 3, 5])
 @pytest.mark.parametrize("M", [20, 130])
