@@ -44,8 +44,10 @@ enum {
                                    pre-packed into matrix-instruction fragment order (needs the workspace);
                                    M <= 16: the kernel reads x itself.  split_k > 1 adds a reduce launch. */
     GPTQ_HIP_KERNEL_TILED = 4,  /* a layer re-laid by gptq_hip_tile_prepare: exact fp16 weights, 32 * row_tiles rows
-                                   (row_tiles = 1, 2 or 4) x 64 waves_n columns (waves_n = 1, or 2 with four row
-                                   tiles: chosen for several row blocks) per workgroup of waves_k = 4 waves along K
+                                   (row_tiles = 1, 2 or 4: the least that covers M up to 128 rows, one step less on
+                                   narrow layers whose shorter row blocks still find a compute unit each) x 64 waves_n
+                                   columns (waves_n = 1, or 2 with four row tiles: chosen for several row blocks) per
+                                   workgroup of waves_k = 4 waves along K, m_blocks row blocks along grid_z
                                    (k_chunk = blocks of 64 channels per wave); x is pre-packed into the
                                    workspace; split_k > 1 adds a reduce launch */
     GPTQ_HIP_KERNEL_TILED_DECODE = 5 /* the same layer for M <= 8 rows, x staged in LDS in the layer's sorted order,
