@@ -492,6 +492,42 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
     }
 }
 
+namespace {
+
+// K ranges of a matmul plan whose workgroups hold a CU alone (two or four row tiles: 264 and ~380 registers per lane).
+// The launch runs in turns of 256 workgroups, a turn lasts as long as a wave's walk, and a K that is cut costs a
+// second pass over split x M x N floats: the number of ranges is the one that makes
+//     turns x blocks per wave x (us per block) + [split > 1] (2.5 + 0.8 us per MB of partial tiles)
+// least (the fewest ranges within 3 % of it), with 0.58 / 0.94 / 1.7 us per block for 64 x 64, 128 x 64 and 128 x 128
+// waves.  Measured (us; tiles = workgroups per range): 9216 x 9216 int3, 144 tiles, 128 rows in 1 / 2 / 3 ranges 45.9 /
+// 52.0 / 43.7, 256 rows (128 x 128 waves) 64.3 / 79.6 / 68.3; 36864 x 9216, 64 / 128 rows: 109 / 115 / 80 and 208 / 187 / 129
+// (three ranges are 432 workgroups: two turns of a third of K instead of one turn of all of it, where two ranges
+// are two turns of half); 18432 x 9216 at 128 rows 83.9 / 96.0 / 68.7; 8192 x 8192 at 256 rows, 128 tiles: 57.3 / 50.2 /
+// 66.6; at 64 rows 8192 x 6144, 96 tiles: 28.3 / 24.1 / 30.2, 11008 x 4608, 72 tiles, in 2 / 3 / 4: 28.0 / 24.8 / 32.0,
+// 8192 x 3328, 52 tiles, in 3 / 4 / 5: 19.8 / 18.7 / 24.7; 64-row blocks of narrow layers at 128 rows: 4096 x 4096 in
+// 1 / 2 ranges 17.1 / 17.6, 2048 x 4096 11.5 / 13.2, 8192 x 4096 29.5 / 26.5.
+int tiled_ranges(int at, bool wide, long long tiles, int S_total, int kwv, double out_elems, int cap)
+{
+    const double us_per_block = at == 2 ? 0.58 : (wide ? 1.7 : 0.94);
+    const int ring = gptq::tiled_ring(at);
+    const int most = cap < 64 ? cap : 64;
+    double cost[65];
+    double best = 1e30;
+    for (int s = 1; s <= most; s++) {
+        cost[s] = 1e30;
+        const int steps = ceil_div(S_total, s * kwv);
+        if (s > 1 && (S_total / (s * kwv) < ring || ceil_div(S_total, steps * kwv) != s)) continue;
+        const double turns = (double)((tiles * s + 255) / 256);
+        cost[s] = turns * steps * us_per_block + (s > 1 ? 2.5 + 0.8e-6 * 4.0 * s * out_elems : 0.0);
+        if (cost[s] < best) best = cost[s];
+    }
+    for (int s = 1; s <= most; s++)
+        if (cost[s] <= 1.03 * best) return s;
+    return 1;
+}
+
+}  // namespace
+
 extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_size, gptq_hip_plan *plan)
 {
     // Up to four rows the decode kernels (one 4-row matrix instruction set per lane block); five to eight rows the
@@ -538,25 +574,19 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     const int col_pairs = ceil_div(N / 32, ct);
     const int S_total = ceil_div(K, 64);
     const long long tiles = (long long)col_pairs * m_blocks;
+    int cap = (int)((3LL * K * bits) / (128LL * M));
+    if (cap < 1) cap = 1;
     int split = (int)((256 + tiles / 2) / tiles);
-    // workgroups of two or four row tiles hold a CU alone: ranges that put a few workgroups past one per CU make the
-    // whole launch wait for a second turn of those few (9216 x 9216 int3 at 256 rows, 144 tiles, us in 1 / 2 / 3 ranges:
-    // 67.9 / 85.3 / 73.8; 8192 x 8192 at 256 rows, 128 tiles: 57.3 / 50.2 / 66.6; at 64 rows 8192 x 6144, 96 tiles, in
-    // 1 / 2 / 3 ranges 28.3 / 24.1 / 30.2, 11008 x 4608, 72 tiles, in 2 / 3 / 4: 28.0 / 24.8 / 32.0, 8192 x 3328, 52 tiles, in
-    // 3 / 4 / 5: 19.8 / 18.7 / 24.7)
-    if (at >= 2 && tiles <= 256 && tiles * split > 256) split = (int)(256 / tiles);
-    // the 64-row blocks of a narrow layer: at most one workgroup per CU, and K cut only while a wave keeps sixteen
-    // blocks (eight where there are at most 64 tiles): a shorter walk saves less than the partial tiles and their pass
-    // cost (4096 x 4096 at 128 rows in 1 / 2 ranges 17.1 / 17.6, 2048 x 4096 11.5 / 13.2, 8192 x 4096 29.5 / 26.5,
-    // 4096 x 2048 16.5 / 15.4)
-    if (short_blocks) {
+    if (at >= 2) {
+        split = tiled_ranges(at, wide, tiles, S_total, kwv, (double)M * N, cap);
+    } else if (short_blocks) {
+        // two 32-row blocks of a narrow layer: K cut only while a wave keeps sixteen blocks (eight where there are at
+        // most 64 tiles)
         split = (int)(256 / tiles);
         const int keep = tiles <= 64 ? 8 : 16;
         while (split > 1 && S_total / (split * kwv) < keep) split--;
     }
     if (split < 1) split = 1;
-    int cap = (int)((3LL * K * bits) / (128LL * M));
-    if (cap < 1) cap = 1;
     if (split > cap) split = cap;
     if ((long long)M * N >= (1LL << 32)) split = 1;  // indexing of the pass that adds the partial tiles
     // every wave gets at least a ring of blocks
@@ -564,7 +594,9 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     // the partial tiles of all ranges together stay within 10 MB where fewer ranges still give two of three CUs a
     // workgroup (11008 x 4096 at 256 rows, 128 x 128 waves, us in 2 / 3 / 4 ranges: int4 49.9 / 45.3 / 52.3, int3 50.9 /
     // 46.5 / 53.3: the fourth range adds 4 MB of fp32 tiles to write and to read again)
-    while (split > 1 && (long long)split * M * N * 4 > (10LL << 20) && tiles * (split - 1) >= 172) split--;
+    // (plans of one turn only: in a plan of two turns one range less is one and a half times the walk)
+    while (split > 1 && tiles * split <= 256 && (long long)split * M * N * 4 > (10LL << 20) && tiles * (split - 1) >= 172)
+        split--;
     // One row tile (up to 32 rows): two such workgroups share a CU, and where K is cut anyway (the pass that adds the
     // ranges is there already) and long, finer ranges that still leave every wave two turns of its ring put up to
     // ~480 workgroups on the chip at once instead of ~256 (us at 32 rows, int3, one group, 144 column pairs: 9216 x
@@ -624,18 +656,18 @@ extern "C" int gptq_hip_select_tiled_transposed(int M, int K, int N, int bits, i
     }
     const int m_blocks = ceil_div(M, 32 * at);
     const long long tiles = (long long)col_pairs * m_blocks;
+    int cap = (int)((3LL * N * bits) / (128LL * M));   // the fp32 tiles of a split stay within 3x the packed weights
+    if (cap < 1) cap = 1;
     int split = (int)((256 + tiles / 2) / tiles);
-    if (split < 1) split = 1;
-    // (workgroups of two or four row tiles hold a CU alone, as in the forward plan: no few workgroups past one per CU)
-    if (at >= 2 && tiles <= 256 && tiles * split > 256) split = (int)(256 / tiles);
-    if (short_blocks) {
+    if (at >= 2) {
+        // (workgroups of two or four row tiles hold a CU alone: ranges by the same count of turns as the forward plan)
+        split = tiled_ranges(at, false, tiles, S_total, kwv, (double)M * K, cap);
+    } else if (short_blocks) {
         split = (int)(256 / tiles);
         const int keep = tiles <= 64 ? 8 : 16;
         while (split > 1 && S_total / (split * kwv) < keep) split--;
-        if (split < 1) split = 1;
     }
-    int cap = (int)((3LL * N * bits) / (128LL * M));   // the fp32 tiles of a split stay within 3x the packed weights
-    if (cap < 1) cap = 1;
+    if (split < 1) split = 1;
     if (split > cap) split = cap;
     if ((long long)M * K >= (1LL << 32)) split = 1;
     while (split > 1 && S_total / (split * kwv) < gptq::tiled_ring(at)) split--;
@@ -690,10 +722,11 @@ namespace {
 //     26.6 against 18.1 / 22.1 / 34.1), but for K of 8192 and more where the checkpoint-layout STREAM kernel has
 //     nothing to look up per weight: 4-bit layers without an activation order up to 64 rows (8192 x 8192, 17 / 64
 //     rows: 23.4 / 28.6 against 19.7 / 25.0; 28672 x 8192, 17 / 32 rows: 52.5 / 53.1 against 43.3 / 43.7) and layers of
-//     one group beyond 32 rows or 16384 columns (9216 x 36864, 32 / 128 rows: 53.4 / 134 against 52.9 / 126; 36864 x
-//     9216 at 128 rows 206 against 173; up to 32 rows and 16384 columns they keep the tiled copy, whose K ranges are
-//     cut finer there: 36864 x 9216, 17 / 32 rows: 57.1 / 57.6 against 70.2 / 72.4, 18432 x 9216 33.2 / 33.8 against
-//     45.0 / 45.9, 9216 x 9216 21.6 / 22.0 against 31.4 / 32.0, 12288 x 12288 level at 28); with an activation order, up
+//     one group beyond 16384 columns (9216 x 36864, 32 / 128 rows: 53.4 / 134 against 52.9 / 126; up to 16384 columns
+//     they keep the tiled copy, whose K ranges are cut by turns of the chip: 36864 x 9216, 17 / 32 rows: 57.1 / 57.6
+//     against 70.2 / 72.4, 64 / 128 / 256 rows in three ranges 80.2 / 129 / 223 against 98.1 / 172 / 255; 18432 x 9216 33.2 /
+//     33.8 against 45.0 / 45.9, 64 / 128 / 256 rows 47.0 / 68.7 / 114 against 56.5 / 90.3 / 134; 9216 x 9216 21.6 / 22.0 against
+//     31.4 / 32.0, 64 / 128 / 256 rows 30.2 / 45.9 / 64.3 against 36.2 / 48.4 / 72.6; 12288 x 12288 level at 28); with an activation order, up
 //     to 32 rows of layers beyond 20480 channels (28672 x 8192 at 32 rows, int4 / int3: 58.3 / 55.9 against 48.3 /
 //     49.8; 17920 x 6656 33.9 / 34.5 against 34.1 / 38.9 stays; from 64 rows the tiled copy wins there too: 60.1 / 63.0
 //     against 63.0 / 67.2);
@@ -719,7 +752,7 @@ bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
         return K <= 4096 && ((N > 4096 && M >= 12) || (bits == 3 && N <= 4096));
     }
     if (M <= 128) {
-        if (one_group && K > 8192 && (M > 32 || N > 16384)) return false;
+        if (one_group && K > 8192 && N > 16384) return false;
         if (M <= 64 && K >= 8192 && bits == 4 && !act_order) return false;
         if (M <= 32 && K > 20480 && act_order) return false;
         return true;
@@ -730,7 +763,7 @@ bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
     // against 112 / 116, 28672 x 8192 4-bit 169 / 172 against 178 / 192, 3-bit 165 / 166 against 169 / 192; without one
     // the longer layers are level or behind: 28672 x 8192 167 / 169 against 164 / 169, 13824 x 5120 at 192 rows 54.7
     // against 46.3)
-    return K <= 8192 || (M <= 256 && (K <= 11008 || act_order));
+    return K <= 8192 || (M <= 256 && (K <= 11008 || act_order || (one_group && N <= 16384)));
 }
 
 // The plan gptq_hip_gemm_sorted runs for M rows of a layer whose channels were sorted by group, if that path covers
