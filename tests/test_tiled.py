@@ -469,7 +469,9 @@ TILED_FULL = [
     ("c4-int3-11008x4096-act", 3, 11008, 4096, 128, True, [16, 64, 128, 256]),
     ("c3-int4-4096x4096", 4, 4096, 4096, 128, False, [8, 1024]),
     ("c5-int3-9216x36864-act-g1", 3, 9216, 36864, -1, True, [32]),
-    ("c5-int3-36864x9216-act-g1", 3, 36864, 9216, -1, True, [32]),
+    ("c5-int3-36864x9216-act-g1", 3, 36864, 9216, -1, True, [32, 64, 128, 256]),   # (K in ranges over two turns of the chip)
+    ("int4-4096x4096-act", 4, 4096, 4096, 128, True, [48, 64, 100, 128, 192, 256]),    # (a narrow layer: shorter row blocks)
+    ("int3-18432x4608-act", 3, 18432, 4608, 128, True, [64, 256]),
     ("int8-4096x11008-act", 8, 4096, 11008, 128, True, [16, 128, 256]),
     ("int2-4096x11008-act", 2, 4096, 11008, 128, True, [16, 128, 256]),
     ("int8-11008x4096", 8, 11008, 4096, 128, False, [64]),
