@@ -163,6 +163,8 @@ FULL = [
     ("c4-int3-4096x11008-act", 3, 4096, 11008, 128, True, [64, 128]),
     ("c4-int4-11008x4096-act", 4, 11008, 4096, 128, True, [128]),
     ("c3-int4-4096x4096", 4, 4096, 4096, 128, False, [8, 1024]),
+    ("int4-4096x4096-act", 4, 4096, 4096, 128, True, [64, 128, 256]),       # (a narrow layer: shorter row blocks)
+    ("int3-9216x18432-act", 3, 9216, 18432, 128, True, [128]),             # (the reduction in ranges over two turns)
     ("int8-4096x11008-act", 8, 4096, 11008, 128, True, [128]),
     ("int2-11008x4096", 2, 11008, 4096, 128, False, [64]),
     ("c5-int3-9216x36864-act-g1", 3, 9216, 36864, -1, True, [32]),
