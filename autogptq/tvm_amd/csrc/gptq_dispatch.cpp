@@ -9,9 +9,6 @@
 
 namespace {
 
-const int kLdsBudget = 120 * 1024;  // of the 160 KB a gfx950 CU has
-const int kTargetWorkgroups = 512;  // two per CU keeps every XCD fed at M = 1
-
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 }  // namespace
