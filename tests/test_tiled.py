@@ -353,6 +353,37 @@ def test_tiled_decode_halved_tiles(dev, bits, K, N, gs, desc_act):
         assert torch.equal(y, run_tiled(D, prep, x=x.to(dev), plan=plan)), f"{what}: two identical calls differ"
 
 
+def _random_matmul_shapes():
+    import random
+
+    rnd = random.Random(20250)
+    shapes = []
+    for _ in range(48):
+        bits = rnd.choice([2, 3, 4, 8])
+        gs = rnd.choice([32, 64, 128, -1])
+        K = 32 * rnd.randint(1, 100) if gs == -1 else gs * rnd.randint(1, 40)
+        N = 32 * rnd.randint(1, 80)
+        M = rnd.choice([rnd.randint(9, 32), rnd.randint(33, 64), rnd.randint(65, 128), rnd.randint(129, 300)])
+        shapes.append((bits, K, N, gs, rnd.random() < 0.5, M))
+    return shapes
+
+
+@pytest.mark.parametrize("bits,K,N,gs,desc_act,M", _random_matmul_shapes())
+def test_tiled_matmul_random_shapes(dev, bits, K, N, gs, desc_act, M):
+    # the planner's own matmul plan (every block height, one to several row blocks, K whole or in ranges) on shapes
+    # drawn at random with a fixed seed
+    L = layer(9100 + K % 997 + N % 991, K, N, bits, gs, desc_act, M=M, bias=(M % 2 == 0))
+    D = to_dev(L, dev)
+    prep = prepare(D)
+    plan = _lib.select_tiled(M, K, N, bits, gs)
+    assert plan.kernel == _lib.KERNEL_TILED
+    y = run_tiled(D, prep)
+    what = (f"int{bits} {K}x{N} gs={gs} act={desc_act} M={M} ({plan.row_tiles} row tiles x {plan.m_blocks} blocks, "
+            f"{plan.split_k} ranges of {plan.k_chunk} blocks per wave)")
+    assert_close(y, expected_output(L), what)
+    assert_tight(y, expected_output(L), what)
+
+
 def _random_decode_shapes():
     import random
 
