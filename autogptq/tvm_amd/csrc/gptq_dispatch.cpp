@@ -491,12 +491,18 @@ extern "C" int gptq_hip_select_tiled_decode(int M, int K, int N, int bits, int g
 
 namespace {
 
-// K ranges of a matmul plan whose workgroups hold a CU alone (two or four row tiles: 264 and ~380 registers per lane).
-// The launch runs in turns of 256 workgroups, a turn lasts as long as a wave's walk, and a K that is cut costs a
-// second pass over split x M x N floats: the number of ranges is the one that makes
+// K ranges of a matmul plan.  Workgroups of two or four row tiles hold a CU alone (264 and ~380 registers per lane),
+// and two of one row tile on a CU share its vector ALU, which is what they wait for: either way the launch runs in
+// turns of 256 workgroups, a turn lasts as long as a wave's walk, and a K that is cut costs a second pass over
+// split x M x N floats.  The number of ranges is the one that makes
 //     turns x blocks per wave x (us per block) + [split > 1] (2.5 + 0.8 us per MB of partial tiles)
-// least (the fewest ranges within 3 % of it), with 0.58 / 0.94 / 1.7 us per block for 64 x 64, 128 x 64 and 128 x 128
-// waves.  Measured (us; tiles = workgroups per range): 9216 x 9216 int3, 144 tiles, 128 rows in 1 / 2 / 3 ranges 45.9 /
+// least (the fewest ranges within 3 % of it), with 0.4 / 0.58 / 0.94 / 1.7 us per block for 32 x 64, 64 x 64, 128 x 64
+// and 128 x 128 waves.  Measured at 17 / 32 rows (one row tile; us in the ranges named): 8192 x 5632, 88 tiles, in 1 / 2 /
+// 3 / 4: 22.0 / 17.9 / 22.4 / 20.2; 11008 x 6400, 100 tiles: 27.7 / 22.2 / 28.2 / 24.8; 8192 x 3328, 52 tiles, in 2 / 3 / 4 / 5:
+// 17.7 / 15.7 / 15.9 / 20.3; 11008 x 4608, 72 tiles, in 2 / 3 / 4: 21.7 / 19.8 / 24.3; 16384 x 6144, 96 tiles, in 1 / 2 / 3 / 5:
+// 36.7 / 27.8 / 35.2 / 31.1; 144 tiles at 32 rows in 1 / 2 / 3 / 5: 9216 x 9216 int3 22.1 / 25.9 / 21.9 / 24.1, 18432 x 9216
+// 38.7 / -- / 33.6 / 35.2, 36864 x 9216 71.9 / -- / 58.4 / 57.6; 4096 x 11008 at 16 rows, 172 tiles, in 1 / 2: 13.4 / 19.1.
+// Measured at more rows (us; tiles = workgroups per range): 9216 x 9216 int3, 144 tiles, 128 rows in 1 / 2 / 3 ranges 45.9 /
 // 52.0 / 43.7, 256 rows (128 x 128 waves) 64.3 / 79.6 / 68.3; 36864 x 9216, 64 / 128 rows: 109 / 115 / 80 and 208 / 187 / 129
 // (three ranges are 432 workgroups: two turns of a third of K instead of one turn of all of it, where two ranges
 // are two turns of half); 18432 x 9216 at 128 rows 83.9 / 96.0 / 68.7; 8192 x 8192 at 256 rows, 128 tiles: 57.3 / 50.2 /
@@ -505,7 +511,15 @@ namespace {
 // 1 / 2 ranges 17.1 / 17.6, 2048 x 4096 11.5 / 13.2, 8192 x 4096 29.5 / 26.5.
 int tiled_ranges(int at, bool wide, long long tiles, int S_total, int kwv, double out_elems, int cap)
 {
-    const double us_per_block = at == 2 ? 0.58 : (wide ? 1.7 : 0.94);
+    // One row tile: the count of turns holds for plans of one turn (above); two such workgroups on a CU also hide each
+    // other's waits, so past one turn the count is too strict: plans of up to 128 tiles take the best plan of one turn,
+    // wider ones are not cut, but for 129 to 160 tiles over a K of 9216 and more, which three ranges put on the chip
+    // at once (432 to 480 workgroups: the 144-tile figures above; five ranges at 18432 x 9216 and 9 rows 41.8 against
+    // 38.6 in three; 12288 x 12288, 192 tiles, in 1 / 4: 30.3 / 32.2; 6656 x 17920, 280 tiles, without an activation order at
+    // 9 rows in 1 / 3: 26.8 / 30.5)
+    const bool one_turn = at == 1;
+    if (one_turn && tiles > 128) return tiles * 3 <= 480 && S_total >= 144 && cap >= 3 ? 3 : 1;
+    const double us_per_block = at == 1 ? 0.4 : (at == 2 ? 0.58 : (wide ? 1.7 : 0.94));
     const int ring = gptq::tiled_ring(at);
     const int most = cap < 64 ? cap : 64;
     double cost[65];
@@ -514,6 +528,7 @@ int tiled_ranges(int at, bool wide, long long tiles, int S_total, int kwv, doubl
         cost[s] = 1e30;
         const int steps = ceil_div(S_total, s * kwv);
         if (s > 1 && (S_total / (s * kwv) < ring || ceil_div(S_total, steps * kwv) != s)) continue;
+        if (s > 1 && one_turn && tiles * s > 256) continue;
         const double turns = (double)((tiles * s + 255) / 256);
         cost[s] = turns * steps * us_per_block + (s > 1 ? 2.5 + 0.8e-6 * 4.0 * s * out_elems : 0.0);
         if (cost[s] < best) best = cost[s];
@@ -550,14 +565,10 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     // The same one step down, 33 to 64 rows as two blocks of 32, for K up to 4096 (48 / 64 rows: 4096 x 4096 13.2 / 13.5
     // against 14.4 / 14.9, 4096 x 8192 14.7 / 15.0 against 16.5 / 17.3, 2048 x 4096 9.6 / 9.8 against 11.4 / 11.8, 5120 x 5120
     // and 4096 x 2048 level; 8192 x 4096 21.1 / 20.9 against 19.2 / 19.8 and 11008 x 4096 24.1 / 24.3 against 22.9 / 23.8 stay)
-    bool short_blocks = false;
-    if (at == 4 && K <= 8192 && (long long)ceil_div(N / 32, 2) * ceil_div(M, 64) <= 256) {
+    if (at == 4 && K <= 8192 && (long long)ceil_div(N / 32, 2) * ceil_div(M, 64) <= 256)
         at = 2;
-        short_blocks = true;
-    } else if (at == 2 && K <= 4096 && (long long)ceil_div(N / 32, 2) * ceil_div(M, 32) <= 256) {
+    else if (at == 2 && K <= 4096 && (long long)ceil_div(N / 32, 2) * ceil_div(M, 32) <= 256)
         at = 1;
-        short_blocks = true;
-    }
     const int rows = 32 * at * rw;
     const int m_blocks = ceil_div(M, rows);
     // several row blocks: 128 columns per wave (waves_n = 2), which halves the x fragments a matrix instruction
@@ -573,16 +584,7 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     const long long tiles = (long long)col_pairs * m_blocks;
     int cap = (int)((3LL * K * bits) / (128LL * M));
     if (cap < 1) cap = 1;
-    int split = (int)((256 + tiles / 2) / tiles);
-    if (at >= 2) {
-        split = tiled_ranges(at, wide, tiles, S_total, kwv, (double)M * N, cap);
-    } else if (short_blocks) {
-        // two 32-row blocks of a narrow layer: K cut only while a wave keeps sixteen blocks (eight where there are at
-        // most 64 tiles)
-        split = (int)(256 / tiles);
-        const int keep = tiles <= 64 ? 8 : 16;
-        while (split > 1 && S_total / (split * kwv) < keep) split--;
-    }
+    int split = tiled_ranges(at, wide, tiles, S_total, kwv, (double)M * N, cap);
     if (split < 1) split = 1;
     if (split > cap) split = cap;
     if ((long long)M * N >= (1LL << 32)) split = 1;  // indexing of the pass that adds the partial tiles
@@ -594,19 +596,6 @@ extern "C" int gptq_hip_select_tiled(int M, int K, int N, int bits, int group_si
     // (plans of one turn only: in a plan of two turns one range less is one and a half times the walk)
     while (split > 1 && tiles * split <= 256 && (long long)split * M * N * 4 > (10LL << 20) && tiles * (split - 1) >= 172)
         split--;
-    // One row tile (up to 32 rows): two such workgroups share a CU, and where K is cut anyway (the pass that adds the
-    // ranges is there already) and long, finer ranges that still leave every wave two turns of its ring put up to
-    // ~480 workgroups on the chip at once instead of ~256 (us at 32 rows, int3, one group, 144 column pairs: 9216 x
-    // 9216 in 2 / 3 / 4 / 6 ranges 26.2 / 22.4 / 24.6 / 24.4; 36864 x 9216 in 2 / 3 / 4 / 6 / 8 / 12: 75.5 / 58.7 /
-    // 64.1 / 60.8 / 60.6 / 60.7: the fourth range is the 577th workgroup, which waits for a CU).  Where K is not cut,
-    // cutting it costs more than it brings (4096 x 11008, 16 rows: 13.4 -> 19.1 in two ranges).
-    if (at == 1 && m_blocks == 1 && split >= 2 && (long long)M * N < (1LL << 32)) {
-        int finer = (int)(480 / tiles);
-        const int two_turns = S_total / (kwv * 2 * gptq::tiled_ring(at));
-        if (finer > two_turns) finer = two_turns;
-        if (finer > cap) finer = cap;
-        if (finer > split) split = finer;
-    }
     const int wave_steps = ceil_div(S_total, split * kwv);
     split = ceil_div(S_total, wave_steps * kwv);
     plan->kernel = GPTQ_HIP_KERNEL_TILED;
@@ -643,27 +632,16 @@ extern "C" int gptq_hip_select_tiled_transposed(int M, int K, int N, int bits, i
     // against 17.7 / 25.6 / 33.0, 8192 x 4096 20.7 / 26.6 against 22.2 / 31.1, 4096 x 2048 13.1 / 16.5 / 20.1 against 14.5 /
     // 21.7 / 24.5, 2048 x 4096 14.9 / 18.0 / 23.3 against 15.1 / 21.0 / 30.3, 5120 x 5120 at 128 rows 27.2 against 29.6; a
     // reduction over 8192 keeps the tall blocks: 4096 x 8192 at 128 / 256 rows 30.9 / 48.4 against 29.6 / 45.8)
-    bool short_blocks = false;
-    if (at == 4 && N < 8192 && (long long)col_pairs * ceil_div(M, 64) <= 256) {
+    if (at == 4 && N < 8192 && (long long)col_pairs * ceil_div(M, 64) <= 256)
         at = 2;
-        short_blocks = true;
-    } else if (at == 2 && N <= 4096 && (long long)col_pairs * ceil_div(M, 32) <= 256) {
+    else if (at == 2 && N <= 4096 && (long long)col_pairs * ceil_div(M, 32) <= 256)
         at = 1;
-        short_blocks = true;
-    }
     const int m_blocks = ceil_div(M, 32 * at);
     const long long tiles = (long long)col_pairs * m_blocks;
     int cap = (int)((3LL * N * bits) / (128LL * M));   // the fp32 tiles of a split stay within 3x the packed weights
     if (cap < 1) cap = 1;
-    int split = (int)((256 + tiles / 2) / tiles);
-    if (at >= 2) {
-        // (workgroups of two or four row tiles hold a CU alone: ranges by the same count of turns as the forward plan)
-        split = tiled_ranges(at, false, tiles, S_total, kwv, (double)M * K, cap);
-    } else if (short_blocks) {
-        split = (int)(256 / tiles);
-        const int keep = tiles <= 64 ? 8 : 16;
-        while (split > 1 && S_total / (split * kwv) < keep) split--;
-    }
+    // (ranges by the same count of turns as the forward plan)
+    int split = tiled_ranges(at, false, tiles, S_total, kwv, (double)M * K, cap);
     if (split < 1) split = 1;
     if (split > cap) split = cap;
     if ((long long)M * K >= (1LL << 32)) split = 1;
