@@ -695,16 +695,19 @@ namespace {
 //     11.3 / 12.5; int3 from nine rows); with an activation order the pack pass makes it 14.6 against 13.4 at 8 rows;
 //   * 17 to 128 rows: almost everywhere (4096 x 11008 with an activation order, 32 / 64 / 128 rows: 14.8 / 19.2 /
 //     26.6 against 18.1 / 22.1 / 34.1), but for K of 8192 and more where the checkpoint-layout STREAM kernel has
-//     nothing to look up per weight: 4-bit layers without an activation order up to 64 rows (8192 x 8192, 17 / 64
-//     rows: 23.4 / 28.6 against 19.7 / 25.0; 28672 x 8192, 17 / 32 rows: 52.5 / 53.1 against 43.3 / 43.7) and layers of
+//     nothing to look up per weight: 4-bit layers without an activation order up to 64 rows, of 8192 columns and more
+//     (17 / 32 / 64 rows: 8192 x 8192 22.0 / 22.5 / 26.0 against 19.9 / 20.7 / 24.5, 8192 x 28672 43.6 / 43.2 / 54.8 against 40.9 /
+//     41.2 / 54.4, 28672 x 8192 level at 42.1 / 42.8 / 56.7 against 43.2 / 44.0 / 55.7; narrower ones keep the tiled copy, whose
+//     K ranges fill one turn of the chip: 13824 x 5120 18.7 / 19.5 / 26.7 against 22.8 / 23.1 / 26.9, 17920 x 6656 27.7 / 27.9 /
+//     38.8 against 31.1 / 31.2 / 39.3, 8192 x 6144 19.3 / 19.2 / 22.7 against 23.8 / 24.5 / 30.0, 11008 x 4608 17.4 / 17.9 / 22.8
+//     against 24.1 / 24.4 / 30.6) and layers of
 //     one group beyond 16384 columns (9216 x 36864, 32 / 128 rows: 53.4 / 134 against 52.9 / 126; up to 16384 columns
 //     they keep the tiled copy, whose K ranges are cut by turns of the chip: 36864 x 9216, 17 / 32 rows: 57.1 / 57.6
 //     against 70.2 / 72.4, 64 / 128 / 256 rows in three ranges 80.2 / 129 / 223 against 98.1 / 172 / 255; 18432 x 9216 33.2 /
 //     33.8 against 45.0 / 45.9, 64 / 128 / 256 rows 47.0 / 68.7 / 114 against 56.5 / 90.3 / 134; 9216 x 9216 21.6 / 22.0 against
-//     31.4 / 32.0, 64 / 128 / 256 rows 30.2 / 45.9 / 64.3 against 36.2 / 48.4 / 72.6; 12288 x 12288 level at 28); with an activation order, up
-//     to 32 rows of layers beyond 20480 channels (28672 x 8192 at 32 rows, int4 / int3: 58.3 / 55.9 against 48.3 /
-//     49.8; 17920 x 6656 33.9 / 34.5 against 34.1 / 38.9 stays; from 64 rows the tiled copy wins there too: 60.1 / 63.0
-//     against 63.0 / 67.2);
+//     31.4 / 32.0, 64 / 128 / 256 rows 30.2 / 45.9 / 64.3 against 36.2 / 48.4 / 72.6; 12288 x 12288 level at 28); with an activation order also
+//     beyond 20480 channels (28672 x 8192 at 17 / 32 rows, int4 48.4 / 48.4 against 47.9 / 49.0, int3 48.4 / 49.0 against
+//     49.6 / 50.7; 64 rows 61.6 / 65.5 against 64.9 / 67.9);
 //   * above 128 rows: K up to 8192 (4096 x 11008, 512 rows: 75 against 95; 11008 x 4096: 127 against 81), and up to
 //     256 rows the longer layers named in the function.
 bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
@@ -728,8 +731,7 @@ bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
     }
     if (M <= 128) {
         if (one_group && K > 8192 && N > 16384) return false;
-        if (M <= 64 && K >= 8192 && bits == 4 && !act_order) return false;
-        if (M <= 32 && K > 20480 && act_order) return false;
+        if (M <= 64 && K >= 8192 && N >= 8192 && bits == 4 && !act_order) return false;
         return true;
     }
     // up to 256 rows also K up to 11008, and any K with an activation order (192 / 256 rows against the checkpoint

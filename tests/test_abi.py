@@ -387,9 +387,7 @@ def table_tiled_wins(M, K, N, act_order, bits, one_group):
     if M <= 128:
         if one_group and K > 8192 and N > 16384:
             return False
-        if M <= 32 and K > 20480 and act_order:
-            return False
-        return not (M <= 64 and K >= 8192 and bits == 4 and not act_order)
+        return not (M <= 64 and K >= 8192 and N >= 8192 and bits == 4 and not act_order)
     return K <= 8192 or (M <= 256 and (K <= 11008 or act_order or (one_group and N <= 16384)))
 
 
