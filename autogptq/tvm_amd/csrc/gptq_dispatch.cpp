@@ -721,6 +721,13 @@ bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
     }
     if (M <= 8 && K <= 11008) return true;   // the decode kernel with two sets of rows (below)
     if (M <= 16) {
+        // (without an activation order and K beyond 4096, against the STREAM kernel that reads x itself, 9 / 16 rows:
+        // 8192 x 6144 14.5 / 16.8 against 17.4 / 19.3, 13824 x 5120 12.8 / 15.4 against 16.1 / 18.1, 28672 x 8192 33.7 / 36.2
+        // against 39.5 / 46.7, 5120 x 13824 10.0 / 14.1 against 13.0 / 15.1, 11008 x 11008 19.4 / 24.8 against 22.1 / 25.9,
+        // 6656 x 6656 11.4 / 12.7 against 13.6 / 15.2; up to 4096 columns level or behind: 11008 x 4096 15.9 / 16.1 against
+        // 13.1 / 14.0, 8192 x 4096 11.2 / 12.5 against 11.5 / 12.4; and behind at 8192 channels from 8192 columns on:
+        // 8192 x 8192 17.7 / 19.0 against 14.8 / 15.6)
+        if (!act_order && K > 4096) return N > 4096 && !(K > 6656 && K < 11008 && N >= 8192);
         if (!act_order) return K <= 4096 && N > 4096 && (M >= 9 || bits == 4);
         // with an activation order (9 to 16 rows; pack pass + matmul against the sorted copy, whose time grows with the
         // rows): 4096 x 11008 from twelve rows (9 / 12 / 16 rows, int4: 13.5 / 13.5 / 13.5 against 13.1 / 13.8 / 14.6; int3
