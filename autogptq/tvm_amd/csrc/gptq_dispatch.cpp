@@ -207,8 +207,13 @@ int plan_stream(int M, int K, int N, int bits, int gs, int G, int act_order, int
     int waves_k = force_waves > 0 ? force_waves : (rt == 4 ? 4 : (tiles * 8 <= 2048 ? 8 : 4));
     while (waves_k > 1 && waves_k * pf > steps_total) waves_k >>= 1;
     int split = (int)((256 + tiles / 2) / tiles);
+    // up to 32 rows a few workgroups past one per CU cost a second turn of the chip, as on the tiled kernels (us at 9 /
+    // 32 rows in the ranges named: 8192 x 6144, 96 tiles, in 2 / 3: 13.7 / 17.7 and 19.6 / 24.3; 8192 x 5632 with an
+    // activation order, 88 tiles: 17.6 / 25.6 and 21.5 / 30.0; 11008 x 4608, 72 tiles, in 3 / 4: 14.2 / 17.6 and 20.2 / 24.5;
+    // 9216 x 9216 int3, 144 tiles, in 1 / 2: 33.0 / 44.6 and 33.7 / 46.0; 28672 x 8192, 128 tiles, in 2 / 3: 30.3 / 39.1)
+    if (rt <= 2 && tiles <= 256 && tiles * split > 256) split = (int)(256 / tiles);
     if (split < 1) split = 1;
-    if (rt == 1 && tiles >= 128 && tiles < 256 && K / waves_k >= 2048) split = ceil_div(384, (int)tiles);
+    if (rt == 1 && tiles >= 128 && tiles < 256 && K / waves_k >= 4096) split = ceil_div(384, (int)tiles);
     int cap = (int)((3LL * K * bits) / (128LL * M));
     if (cap < 1) cap = 1;
     if (split > cap) split = cap;
@@ -722,12 +727,11 @@ bool tiled_wins(int M, int K, int N, bool act_order, int bits, bool one_group)
     if (M <= 8 && K <= 11008) return true;   // the decode kernel with two sets of rows (below)
     if (M <= 16) {
         // (without an activation order and K beyond 4096, against the STREAM kernel that reads x itself, 9 / 16 rows:
-        // 8192 x 6144 14.5 / 16.8 against 17.4 / 19.3, 13824 x 5120 12.8 / 15.4 against 16.1 / 18.1, 28672 x 8192 33.7 / 36.2
-        // against 39.5 / 46.7, 5120 x 13824 10.0 / 14.1 against 13.0 / 15.1, 11008 x 11008 19.4 / 24.8 against 22.1 / 25.9,
-        // 6656 x 6656 11.4 / 12.7 against 13.6 / 15.2; up to 4096 columns level or behind: 11008 x 4096 15.9 / 16.1 against
-        // 13.1 / 14.0, 8192 x 4096 11.2 / 12.5 against 11.5 / 12.4; and behind at 8192 channels from 8192 columns on:
-        // 8192 x 8192 17.7 / 19.0 against 14.8 / 15.6)
-        if (!act_order && K > 4096) return N > 4096 && !(K > 6656 && K < 11008 && N >= 8192);
+        // 13824 x 5120 12.4 / 15.2 against 15.9 / 18.1, 5120 x 13824 10.0 / 14.1 against 13.1 / 15.1, 11008 x 11008 19.3 / 24.9
+        // against 22.0 / 25.9, 6656 x 6656 11.2 / 12.8 against 13.7 / 15.2, 28672 x 8192 level at 31.3 / 35.5; up to 4096
+        // columns level or behind: 11008 x 4096 16.1 / 16.1 against 13.1 / 14.2, 8192 x 4096 11.1 / 12.6 against 11.5 / 12.5;
+        // and behind at 8192 channels: 8192 x 6144 14.6 / 16.8 against 13.6 / 15.2, 8192 x 8192 17.6 / 19.0 against 14.1 / 15.5)
+        if (!act_order && K > 4096) return N > 4096 && !(K > 6656 && K < 11008);
         if (!act_order) return K <= 4096 && N > 4096 && (M >= 9 || bits == 4);
         // with an activation order (9 to 16 rows; pack pass + matmul against the sorted copy, whose time grows with the
         // rows): 4096 x 11008 from twelve rows (9 / 12 / 16 rows, int4: 13.5 / 13.5 / 13.5 against 13.1 / 13.8 / 14.6; int3

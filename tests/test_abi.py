@@ -382,7 +382,7 @@ def table_tiled_wins(M, K, N, act_order, bits, one_group):
         return True
     if M <= 16:
         if not act_order and K > 4096:
-            return N > 4096 and not (6656 < K < 11008 and N >= 8192)
+            return N > 4096 and not 6656 < K < 11008
         if not act_order:
             return K <= 4096 and N > 4096 and (M >= 9 or bits == 4)
         return K <= 4096 and ((N > 4096 and M >= 12) or (bits == 3 and N <= 4096))
