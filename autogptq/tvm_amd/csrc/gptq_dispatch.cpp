@@ -92,8 +92,11 @@ bool plan_grouped(int M, int K, int N, int bits, int gs, int G, int act_order, i
     if ((size_t)col_tiles * sizeof(int) > gptq::kCounterBytes) return false;
     const int lds_cap = gptq::kGroupedLdsCap;
     // a column tile per workgroup and no split is best (nothing crosses workgroups) unless
-    // that leaves most of the 256 CUs idle
-    int want = force_split > 0 ? force_split : (col_tiles >= 128 ? 1 : ceil_div(256, col_tiles));
+    // that leaves most of the 256 CUs idle; then as many K ranges as keep the workgroups within one per CU: a few
+    // past it wait for a second turn of the chip (one row, us in the ranges named: 8192 x 5120, 80 tiles, in 2 / 3 / 4 /
+    // 5: 10.8 / 10.3 / 15.3 / 14.9; 8192 x 6144, 96 tiles, in 2 / 3 / 4: 10.8 / 16.2 / 15.5; 8192 x 7168, 112 tiles: 11.1 / 16.4 /
+    // 15.9; 13824 x 5120 int3 in 2 / 3 / 4: 12.1 / 11.0 / 13.8; 11008 x 4608, 72 tiles, in 3 / 4 / 5: 11.1 / 16.6 / 16.2)
+    int want = force_split > 0 ? force_split : (col_tiles >= 128 ? 1 : 256 / col_tiles);
     // A workgroup's time is a chain of load latencies (~0.85 us per step of a wave) rather than its share of the
     // HBM bandwidth, and the sum across workgroups costs 2-4 us: while a wave's share of an unsplit K stays within
     // 512 channels (K <= 4096) one workgroup per column tile is faster than filling the chip, however few tiles
@@ -150,8 +153,8 @@ bool plan_grouped_packed(int M, int K, int N, int bits, int gs, int force_split,
     const int waves_n = force_waves > 0 ? force_waves : 1;
     const int col_tiles = ceil_div(N, 64 * waves_n);
     if ((size_t)col_tiles * sizeof(int) > gptq::kCounterBytes) return false;
-    int want = force_split > 0 ? force_split : (col_tiles >= 128 ? 1 : ceil_div(256, col_tiles));
-    if (force_split == 0 && ceil_div(steps_total, 8 / waves_n) * kstep <= 512) want = 1;  // as in plan_grouped
+    int want = force_split > 0 ? force_split : (col_tiles >= 128 ? 1 : 256 / col_tiles);   // as in plan_grouped
+    if (force_split == 0 && ceil_div(steps_total, 8 / waves_n) * kstep <= 512) want = 1;
     if (want > steps_total) want = steps_total;
     for (int want_split = want; want_split <= steps_total && want_split <= 256; want_split++) {
         if (force_split > 0 && want_split != want) return false;
