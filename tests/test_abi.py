@@ -504,3 +504,30 @@ def test_narrow_layers_run_in_shorter_row_blocks():
     assert p.split_k == 1 and p.k_chunk == 16
     p = _lib.select_tiled(128, 8192, 4096, 4, 128)
     assert p.split_k == 2 and p.k_chunk == 16
+
+
+def test_matmul_plans_keep_the_measured_choices():
+    # (M, K, N, bits, group_size) -> (row tiles, row blocks, waves along N, K ranges): the plans that the measurements
+    # named as the best of their neighbours on MI355X (the count of turns of the chip and the shorter row blocks of
+    # narrow layers); a change of the planner that moves one of them wants a measurement
+    table = [
+        (128, 36864, 9216, 3, -1, 4, 1, 1, 3), (64, 36864, 9216, 3, -1, 2, 1, 1, 3), (128, 9216, 9216, 3, 128, 4, 1, 1, 1),
+        (64, 8192, 6144, 4, 128, 2, 1, 1, 2), (64, 11008, 4608, 4, 128, 2, 1, 1, 3), (64, 8192, 3328, 4, 128, 2, 1, 1, 4),
+        (128, 11008, 4096, 4, 128, 4, 1, 1, 4), (256, 11008, 4096, 4, 128, 4, 2, 2, 3), (192, 11008, 4096, 4, 128, 4, 2, 2, 3),
+        (128, 4096, 11008, 4, 128, 4, 1, 1, 1), (256, 4096, 11008, 4, 128, 4, 2, 2, 1), (64, 4096, 11008, 3, 128, 2, 1, 1, 1),
+        (32, 13824, 5120, 4, 128, 1, 1, 1, 3), (32, 28672, 8192, 4, 128, 1, 1, 1, 2), (32, 4096, 9216, 4, 128, 1, 1, 1, 1),
+        (32, 9216, 9216, 3, -1, 1, 1, 1, 3), (32, 36864, 9216, 3, -1, 1, 1, 1, 3), (16, 4096, 11008, 4, 128, 1, 1, 1, 1),
+        (128, 4096, 4096, 4, 128, 2, 2, 1, 1), (128, 8192, 4096, 4, 128, 2, 2, 1, 2), (64, 4096, 4096, 4, 128, 1, 2, 1, 1),
+        (256, 4096, 4096, 4, 128, 2, 4, 1, 1),
+    ]
+    for M, K, N, bits, gs, rt, mb, wn, split in table:
+        p = _lib.select_tiled(M, K, N, bits, gs)
+        assert (p.kernel, p.row_tiles, p.m_blocks, p.waves_n, p.split_k) == (_lib.KERNEL_TILED, rt, mb, wn, split), (
+            M, K, N, bits, gs, p.as_dict())
+    # the kernels on the checkpoint tensors: K ranges within one workgroup per CU
+    for M, K, N, bits, kernel, split in ((1, 8192, 5120, 4, _lib.KERNEL_GROUPED, 3), (1, 8192, 6144, 4, _lib.KERNEL_GROUPED, 2),
+                                         (1, 11008, 4096, 4, _lib.KERNEL_GROUPED, 4), (9, 8192, 6144, 4, _lib.KERNEL_STREAM, 2),
+                                         (32, 11008, 4608, 4, _lib.KERNEL_STREAM, 3), (16, 11008, 4096, 4, _lib.KERNEL_STREAM, 4)):
+        p = _lib.select(M, K, N, bits, 128, False)
+        assert (p.kernel, p.split_k) == (kernel, split), (M, K, N, bits, p.as_dict())
+        assert p.grid_x * p.grid_y * p.grid_z <= 256
