@@ -91,6 +91,8 @@ WORKLOADS = {
     "int4-4096x4096-act-m128": (4, 4096, 4096, 128, True, 128),
     "int3-4096x4096-act-m128": (3, 4096, 4096, 128, True, 128),
     "int4-4096x4096-act-m256": (4, 4096, 4096, 128, True, 256),
+    # a long, narrow layer at prompt sizes: K in three ranges, two turns of the chip
+    "int3-36864x9216-g1-m128": (3, 36864, 9216, -1, True, 128),
     # larger layers, where the fixed cost of a launch weighs less
     "int4-9216x36864-g1-m1": (4, 9216, 36864, -1, True, 1),
     "int4-8192x28672-m1": (4, 8192, 28672, 128, False, 1),
